@@ -1,0 +1,23 @@
+"""CPU oracle for the KV-cache compression hot path.
+
+TEST INFRASTRUCTURE ONLY.  Nothing in the shipped package may import this
+directory: it exists so that tests, the smoke check and the benchmark's
+CPU-baseline leg can compare the HIP kernels against an independent numpy / C
+restatement of the reference algorithms.  Every function cites the reference
+file:line it restates (paths relative to the VeloxQuant-MLX source tree).
+
+Parity pinning status (which external facts each function is checked against
+lives in tests/test_oracle_*.py):
+
+* group quantisation, packing, dequantisation, decode attention, causal
+  prefill attention, cache frontier arithmetic: pinned (hand-computed known
+  answers, closed forms, invariants, brute force, library SDPA).
+* ``quantize_vq`` on exact fp32 near-ties: PARITY UNPINNED against MLX's
+  ``mx.sum`` reduction order and ``mx.argmin`` tie order (MLX is not
+  installable here).  The oracle fixes the order the reference's Metal twin
+  uses: separately rounded squares, left-to-right fp32 sum, strict ``<``
+  (lowest index wins).
+* default random codebooks drawn from ``mx.random``: PARITY UNPINNED (MLX's
+  RNG stream is not reproducible without MLX); all parity inputs pass
+  explicit codebooks.
+"""

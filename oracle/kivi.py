@@ -1,0 +1,231 @@
+"""numpy restatement of KIVI asymmetric group quantisation and bit packing.
+
+TEST INFRASTRUCTURE ONLY (see oracle/__init__.py).
+
+All arithmetic is IEEE float32 with one rounding per operation, exactly as the
+reference's pure-MLX path performs it:
+
+* ``veloxquant_mlx/cache/kivi_cache.py:181-201``  (round trip, edge-replicated
+  padding, eps-floored scale, round-half-even, clip, ``code*scale + gmin``)
+* ``benchmark_scripts/benchmark_real_model_scalar_attend.py:115-153`` and
+  ``veloxquant_mlx/tests/metal/test_scalar_attend.py:51-82`` (split outputs:
+  codes / scale / zero)
+* ``veloxquant_mlx/quantizers/kivi.py:103-128`` (2-D research API)
+* ``veloxquant_mlx/cache/turboquant_rvq_cache.py:82-126`` (uint32 packing)
+* ``veloxquant_mlx/metal/src/bit_pack.metal:8-19`` (byte packing)
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+F32 = np.float32
+
+
+def _grouped(x32: np.ndarray, axis: int, g: int):
+    """Move ``axis`` last, pad the ragged tail by repeating the last element
+    and reshape to ``[..., n_groups, g]`` (kivi_cache.py:183-193)."""
+    xm = np.moveaxis(x32, axis, -1)
+    L = xm.shape[-1]
+    n_groups = (L + g - 1) // g
+    pad = n_groups * g - L
+    if pad:
+        tail = np.broadcast_to(xm[..., -1:], xm.shape[:-1] + (pad,))
+        xm = np.concatenate([xm, tail], axis=-1)
+    return xm.reshape(xm.shape[:-1] + (n_groups, g)), L
+
+
+def group_quant_codes(x, axis: int, group_size: int, levels: int, eps: float = 1e-8):
+    """Asymmetric min/max group quantisation along ``axis`` (-2 keys, -1 values).
+
+    Returns ``(codes uint8 like x, scale f32, zero f32)``; for ``axis=-2`` the
+    parameter arrays are ``[..., ceil(S/g), D]``, for ``axis=-1`` they are
+    ``[..., S, ceil(D/g)]`` (test_scalar_attend.py:51-82).
+    """
+    if axis not in (-1, -2):
+        raise ValueError("axis must be -1 or -2")
+    x32 = np.asarray(x).astype(F32)
+    xg, L = _grouped(x32, axis, group_size)
+    gmin = xg.min(axis=-1, keepdims=True)
+    gmax = xg.max(axis=-1, keepdims=True)
+    scale = np.maximum((gmax - gmin) / F32(levels), F32(eps)).astype(F32)
+    q = np.clip(np.round((xg - gmin) / scale), 0, levels)
+    codes = q.reshape(q.shape[:-2] + (-1,))[..., :L].astype(np.uint8)
+    codes = np.moveaxis(codes, -1, axis)
+    scale = scale[..., 0]
+    zero = gmin[..., 0]
+    if axis == -2:
+        # [..., D, GK] -> [..., GK, D]
+        scale = np.swapaxes(scale, -1, -2)
+        zero = np.swapaxes(zero, -1, -2)
+    return np.ascontiguousarray(codes), np.ascontiguousarray(scale), np.ascontiguousarray(zero)
+
+
+def group_dequant(codes, scale, zero, axis: int, group_size: int) -> np.ndarray:
+    """``code*scale + zero`` with two float32 roundings
+    (kivi_group_quant_channel.metal:83-87, scalar_affine_decode_once.metal:44)."""
+    codes = np.asarray(codes)
+    S, D = codes.shape[-2], codes.shape[-1]
+    c32 = codes.astype(F32)
+    scale = np.asarray(scale).astype(F32)
+    zero = np.asarray(zero).astype(F32)
+    if axis == -2:
+        gi = np.arange(S) // group_size
+        s = scale[..., gi, :]
+        z = zero[..., gi, :]
+    elif axis == -1:
+        gi = np.arange(D) // group_size
+        s = scale[..., :, gi]
+        z = zero[..., :, gi]
+    else:
+        raise ValueError("axis must be -1 or -2")
+    prod = (c32 * s).astype(F32)
+    return (prod + z).astype(F32)
+
+
+def quant_dequant_along(x, axis: int, group_size: int, levels: int, eps: float = 1e-8,
+                        cast=None) -> np.ndarray:
+    """The reference cache's in-place round trip (kivi_cache.py:151-201).
+
+    ``cast`` converts the float32 reconstruction to the storage dtype; the
+    default casts back to ``x.dtype`` (numpy has no bfloat16, callers pass a
+    torch-based cast for that)."""
+    x = np.asarray(x)
+    codes, scale, zero = group_quant_codes(x, axis, group_size, levels, eps)
+    recon = group_dequant(codes, scale, zero, axis, group_size)
+    if cast is not None:
+        return cast(recon)
+    return recon.astype(x.dtype)
+
+
+# ---------------------------------------------------------------------------
+# packing
+# ---------------------------------------------------------------------------
+
+def pack_indices(idx, bits: int) -> np.ndarray:
+    """Pack the trailing axis into uint32 words, ``32 // bits`` codes per word,
+    element ``i`` of a word at bits ``[i*bits, (i+1)*bits)``; a partial last
+    word is zero padded (turboquant_rvq_cache.py:82-106)."""
+    idx = np.asarray(idx)
+    d = idx.shape[-1]
+    per = 32 // bits
+    pad = (-d) % per
+    if pad:
+        idx = np.concatenate([idx, np.zeros(idx.shape[:-1] + (pad,), idx.dtype)], axis=-1)
+    w = idx.reshape(idx.shape[:-1] + ((d + pad) // per, per)).astype(np.uint64)
+    shifts = (np.arange(per, dtype=np.uint64) * np.uint64(bits))
+    return (w << shifts).sum(axis=-1).astype(np.uint32)
+
+
+def unpack_indices(packed, bits: int, d: int) -> np.ndarray:
+    """Inverse of :func:`pack_indices` (turboquant_rvq_cache.py:109-126)."""
+    packed = np.asarray(packed).astype(np.uint32)
+    per = 32 // bits
+    shifts = (np.arange(per, dtype=np.uint32) * np.uint32(bits))
+    mask = np.uint32((1 << bits) - 1)
+    ex = (packed[..., None] >> shifts) & mask
+    return ex.reshape(packed.shape[:-1] + (-1,))[..., :d].astype(np.uint8)
+
+
+def pack_bytes(indices, bits: int) -> np.ndarray:
+    """Flat byte packing, ``8 // bits`` codes per byte LSB first
+    (bit_pack.metal:8-19, _bit_packing.py:87-118).  ``len(indices)`` must be a
+    multiple of ``8 // bits``."""
+    flat = np.asarray(indices).reshape(-1).astype(np.uint32)
+    per = 8 // bits
+    if flat.size % per:
+        raise ValueError("length must be a multiple of 8 // bits")
+    w = flat.reshape(-1, per) & np.uint32((1 << bits) - 1)
+    shifts = np.arange(per, dtype=np.uint32) * np.uint32(bits)
+    return (w << shifts).sum(axis=-1).astype(np.uint8)
+
+
+def unpack_bytes(packed, n: int, bits: int) -> np.ndarray:
+    """Inverse of :func:`pack_bytes` (bit_unpack.metal:8-15)."""
+    p = np.asarray(packed).reshape(-1).astype(np.uint32)
+    per = 8 // bits
+    shifts = np.arange(per, dtype=np.uint32) * np.uint32(bits)
+    ex = (p[:, None] >> shifts) & np.uint32((1 << bits) - 1)
+    return ex.reshape(-1)[:n].astype(np.uint8)
+
+
+# ---------------------------------------------------------------------------
+# cache frontier + byte accounting (pure integer arithmetic)
+# ---------------------------------------------------------------------------
+
+def quantization_boundary(offset: int, residual_length: int, group_size: int) -> int:
+    """kivi_cache.py:206-225."""
+    aged = max(0, offset - residual_length)
+    return (aged // group_size) * group_size
+
+
+def quantized_bytes(n: int, B: int, H: int, D: int, bits: int, group_size: int):
+    """kivi_cache.py:301-306 (fp16 scale+zero)."""
+    import math
+    k = math.ceil(n * D * bits / 8) * H * B + math.ceil(n / group_size) * D * 2 * 2 * H * B
+    v = math.ceil(n * D * bits / 8) * H * B + n * math.ceil(D / group_size) * 2 * 2 * H * B
+    return k, v
+
+
+class KiviCacheModel:
+    """numpy model of ``KIVIKVCache.update_and_fetch`` / ``trim``
+    (kivi_cache.py:230-332): fp16 history, in-place round trip of the
+    group-aligned prefix that aged out of the residual window."""
+
+    def __init__(self, bits=2, group_size=32, residual_length=128):
+        self.bits, self.g, self.R = bits, group_size, residual_length
+        self.levels = (1 << bits) - 1
+        self.keys = None
+        self.values = None
+        self.offset = 0
+        self.n_quantized = 0
+        self.key_bytes_compressed = 0
+        self.value_bytes_compressed = 0
+        self.key_bytes_fp16 = 0
+        self.value_bytes_fp16 = 0
+        self.residual_fp16_bytes = 0
+        self.tokens_seen = 0
+        self.shape_bhd = (1, 1, 0)
+
+    def update_and_fetch(self, keys, values):
+        B, H, S, D = keys.shape
+        self.shape_bhd = (B, H, D)
+        if self.keys is None:
+            self.keys, self.values = keys.copy(), values.copy()
+        else:
+            self.keys = np.concatenate([self.keys[:, :, : self.offset], keys], axis=2)
+            self.values = np.concatenate([self.values[:, :, : self.offset], values], axis=2)
+        self.offset += S
+        nb = quantization_boundary(self.offset, self.R, self.g)
+        n_now = nb - self.n_quantized
+        if n_now > 0:
+            lo, hi = self.n_quantized, nb
+            self.keys[:, :, lo:hi] = quant_dequant_along(self.keys[:, :, lo:hi], -2, self.g, self.levels)
+            self.values[:, :, lo:hi] = quant_dequant_along(self.values[:, :, lo:hi], -1, self.g, self.levels)
+            self.n_quantized = nb
+            k, v = quantized_bytes(n_now, B, H, D, self.bits, self.g)
+            self.key_bytes_compressed += k
+            self.value_bytes_compressed += v
+        self.residual_fp16_bytes = (self.offset - self.n_quantized) * D * 2 * 2 * H * B
+        self.key_bytes_fp16 += H * B * S * D * 2
+        self.value_bytes_fp16 += H * B * S * D * 2
+        self.tokens_seen += S
+        return self.keys[:, :, : self.offset], self.values[:, :, : self.offset]
+
+    def trim(self, n: int) -> int:
+        n = min(self.offset, n)
+        self.offset -= n
+        if n:
+            B, H, D = self.shape_bhd
+            new_nq = min(self.n_quantized, (max(self.offset, 0) // self.g) * self.g)
+            rolled = self.n_quantized - new_nq
+            self.n_quantized = new_nq
+            if rolled > 0:
+                k, v = quantized_bytes(rolled, B, H, D, self.bits, self.g)
+                self.key_bytes_compressed = max(0, self.key_bytes_compressed - k)
+                self.value_bytes_compressed = max(0, self.value_bytes_compressed - v)
+            self.key_bytes_fp16 = max(0, self.key_bytes_fp16 - H * B * n * D * 2)
+            self.value_bytes_fp16 = max(0, self.value_bytes_fp16 - H * B * n * D * 2)
+            self.tokens_seen = max(0, self.tokens_seen - n)
+            self.residual_fp16_bytes = (self.offset - self.n_quantized) * D * 2 * 2 * H * B
+        return n
