@@ -1,0 +1,177 @@
+/* veloxquant_hip.h -- C ABI of the MI355X (gfx950) KV-cache compression library.
+ *
+ * One shared library (libveloxquant_hip.so) replaces the Metal kernel layer of
+ * VeloxQuant-MLX for the KIVI / VecInfer hot path.  Every entry point
+ *   - takes plain device pointers and sizes (no framework types),
+ *   - enqueues work on the HIP stream it is given and returns without syncing,
+ *   - never allocates or frees device memory and keeps no pointer after return,
+ *   - returns 0 on success or a negative VQ_ERR_* code; vq_last_error() holds
+ *     the message of the calling thread's last failure.
+ * Citations name the reference interface each entry point stands in for
+ * (paths relative to the VeloxQuant-MLX source tree).
+ */
+#ifndef VELOXQUANT_HIP_H
+#define VELOXQUANT_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+enum { VQ_F16 = 0, VQ_BF16 = 1, VQ_F32 = 2, VQ_U8 = 3, VQ_I32 = 4, VQ_U32 = 5 };
+
+/* status codes */
+enum {
+    VQ_OK = 0,
+    VQ_ERR_INVALID = -1,     /* bad shape / dtype / range (maps to ValueError)   */
+    VQ_ERR_UNSUPPORTED = -2, /* valid request outside what the kernels cover     */
+    VQ_ERR_WORKSPACE = -3,   /* workspace missing or too small                   */
+    VQ_ERR_HIP = -4          /* a HIP runtime call failed                        */
+};
+
+/* axis of group quantisation inside the trailing [S, D] dims */
+enum { VQ_AXIS_TOKEN = 0 /* keys: groups run along S (python axis -2)     */,
+       VQ_AXIS_CHANNEL = 1 /* values: groups run along D (python axis -1) */ };
+
+/* layout of packed VALUE codes and their scale/zero:
+ *   VQ_V_CHANNEL_PACKED  words hold consecutive channels of one token:
+ *                        codes [BH, S, ceil(D/per)], scale/zero [BH, S, GV]
+ *                        (the image _pack_indices gives for [.., S, D] codes)
+ *   VQ_V_TOKEN_PACKED    words hold consecutive tokens of one channel:
+ *                        codes [BH, ceil(S/per), D], scale/zero [BH, GV, S]
+ *                        (_pack_indices applied to the [.., D, S] transpose and
+ *                        stored with the word axis ahead of D); this is the
+ *                        layout the MFMA decode kernel streams
+ * per = 32 / pack_bits. */
+enum { VQ_V_CHANNEL_PACKED = 0, VQ_V_TOKEN_PACKED = 1 };
+
+int vq_abi_version(void);
+/* copies the calling thread's last error text; returns its length */
+int vq_last_error(char *buf, size_t n);
+/* number of HIP devices visible, or a negative VQ_ERR_HIP */
+int vq_device_count(void);
+
+/* ---- KIVI group quantisation -------------------------------------------- */
+
+/* Fused quantise -> dequantise round trip, out = cast(code*scale + min).
+ * Replaces kivi_group_quant_dequant(x, axis, group_size, levels, eps)
+ * (veloxquant_mlx/metal/_kivi_quant.py:138-207) and the pure-MLX
+ * KIVIKVCache._quant_dequant_along (veloxquant_mlx/cache/kivi_cache.py:151-201).
+ * x/out: [BH, S, D] contiguous, same dtype (VQ_F16 / VQ_BF16 / VQ_F32). */
+int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D,
+                          int axis, int group, int levels, float eps, void *stream);
+
+/* Quantise and bit-pack.  Codes follow _quant_keys/_quant_values
+ * (benchmark_scripts/benchmark_real_model_scalar_attend.py:115-153;
+ * veloxquant_mlx/quantizers/_quant_utils.py:9-46) and the word image follows
+ * _pack_indices (veloxquant_mlx/cache/turboquant_rvq_cache.py:82-106).
+ *
+ * x: [BH, S, D] with row stride D and a per-(b,h) stride of x_stride_bh
+ * elements.  Results land at token offset dst_tok0 of destination buffers that
+ * hold cap_tokens tokens per (b,h):
+ *   axis TOKEN  (keys):   packed [BH, cap_tokens, W], scale/zero
+ *                         [BH, ceil(cap_tokens/group), D]; dst_tok0 % group == 0
+ *   axis CHANNEL (values), v_layout CHANNEL_PACKED: packed [BH, cap_tokens, W],
+ *                         scale/zero [BH, cap_tokens, GV]
+ *   axis CHANNEL (values), v_layout TOKEN_PACKED: packed [BH, cap_tokens/per, D],
+ *                         scale/zero [BH, GV, cap_tokens]; dst_tok0, S and
+ *                         cap_tokens multiples of per
+ * W = ceil(D/per), per = 32/pack_bits, GV = ceil(D/group).  pack_bits == 8
+ * yields plain uint8 codes.  levels is the top code (2^b - 1 <= 2^pack_bits-1).
+ * scale/zero are written as meta_dtype (VQ_F32 exact, VQ_F16 rounded). */
+int vq_kivi_quant_pack(const void *x, int dtype, int64_t BH, int64_t S, int64_t D,
+                       int64_t x_stride_bh, int axis, int group, int levels, float eps,
+                       int pack_bits, int v_layout, void *packed, void *scale, void *zero,
+                       int meta_dtype, int64_t cap_tokens, int64_t dst_tok0, void *stream);
+
+/* Packed codes -> reconstruction, out[BH, S, D] = cast(code*scale + zero).
+ * Replaces scalar_decode_once(codes, scale, zero, group_size, mode)
+ * (veloxquant_mlx/metal/_scalar_attend.py:650-699).  Source buffers are laid
+ * out as vq_kivi_quant_pack writes them; tokens [src_tok0, src_tok0+S). */
+int vq_kivi_dequant(const void *packed, const void *scale, const void *zero, int meta_dtype,
+                    int64_t BH, int64_t S, int64_t D, int axis, int group, int pack_bits,
+                    int v_layout, int64_t cap_tokens, int64_t src_tok0, void *out, int out_dtype,
+                    void *stream);
+
+/* ---- bit packing ----------------------------------------------------------- */
+
+/* Trailing-axis word packing, idx[rows, D] uint8 <-> words[rows, ceil(D/per)].
+ * Replaces _pack_indices/_unpack_indices
+ * (veloxquant_mlx/cache/turboquant_rvq_cache.py:82-126). bits in 1..8. */
+int vq_pack_words(const uint8_t *idx, int64_t rows, int64_t D, int bits, uint32_t *words, void *stream);
+int vq_unpack_words(const uint32_t *words, int64_t rows, int64_t D, int bits, uint8_t *idx, void *stream);
+
+/* Flat byte packing, 8/bits codes per byte, LSB first; bits in {1,2,4}.
+ * Replaces turboquant_bit_pack / turboquant_bit_unpack
+ * (veloxquant_mlx/metal/_bit_packing.py:87-148). n = number of codes. */
+int vq_bit_pack(const uint8_t *idx, int64_t n, int bits, uint8_t *packed, void *stream);
+int vq_bit_unpack(const uint8_t *packed, int64_t n, int bits, uint8_t *idx, void *stream);
+
+/* ---- VecInfer product VQ -------------------------------------------------- */
+
+/* Nearest-centroid assignment with one codebook shared by all sub-vectors:
+ * x [N, sub_dim] (any float dtype), codebook [n_centroids, sub_dim]; distance
+ * sum_i (x_i - c_i)^2 in float32, dimensions added left to right, strict '<'
+ * so the lowest index wins ties.  idx_dtype VQ_I32, VQ_U32 or VQ_U8
+ * (n_centroids <= 256).  Replaces quantize_vq
+ * (veloxquant_mlx/allocators/vecinfer.py:281-318) and vecinfer_quantize_metal
+ * (veloxquant_mlx/metal/_vecinfer.py:181-222). */
+int vq_vecinfer_assign(const void *x, int x_dtype, int64_t N, const void *codebook, int cb_dtype,
+                       int n_centroids, int sub_dim, void *idx, int idx_dtype, void *stream);
+
+/* Centroid gather, out [N, sub_dim] = codebook[min(idx, n_centroids-1)].
+ * Replaces dequantize_vq (allocators/vecinfer.py:321-335) and
+ * vecinfer_dequant_metal (metal/_vecinfer.py:144-178). */
+int vq_vecinfer_dequant(const void *idx, int idx_dtype, int64_t N, const void *codebook,
+                        int cb_dtype, int n_centroids, int sub_dim, void *out, int out_dtype,
+                        void *stream);
+
+/* ---- attention over a packed KIVI cache ------------------------------------ */
+
+typedef struct vq_attend_args {
+    /* queries / output: [B, Hq, Sq, D] contiguous */
+    const void *q;
+    void *out;
+    int q_dtype;   /* VQ_F16 / VQ_BF16 / VQ_F32 */
+    int out_dtype; /* VQ_F16 / VQ_BF16 / VQ_F32 */
+    int64_t B, Hq, Hkv, Sq, D;
+    /* quantised prefix: n_packed tokens laid out as vq_kivi_quant_pack writes
+     * them (keys TOKEN axis, values CHANNEL axis in v_layout), buffers sized
+     * for cap_tokens tokens per (b, h_kv).  n_packed == 0 is allowed. */
+    const void *k_packed, *k_scale, *k_zero;
+    const void *v_packed, *v_scale, *v_zero;
+    int pack_bits, group, meta_dtype, v_layout;
+    int64_t n_packed, cap_tokens;
+    /* un-quantised tail: n_tail tokens, [B, Hkv, tail_cap, D], tail_dtype
+     * VQ_F16 / VQ_BF16 / VQ_F32.  n_tail == 0 is allowed. */
+    const void *k_tail, *v_tail;
+    int tail_dtype;
+    int64_t n_tail, tail_cap;
+    float scale; /* softmax scale applied to q.k */
+    int causal;  /* 1: query i sees slots <= n_packed + n_tail - Sq + i */
+    int num_splits; /* 0 = choose; otherwise the split count along tokens */
+    void *workspace;
+    size_t workspace_bytes;
+    void *stream;
+} vq_attend_args;
+
+/* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the
+ * shapes, pack_bits, group and num_splits are ignored). */
+size_t vq_kivi_attend_workspace(const vq_attend_args *a);
+
+/* softmax(q k^T * scale) v over [quantised prefix | tail] with GQA by
+ * repeat-interleave (query heads [h*Hq/Hkv, (h+1)*Hq/Hkv) share kv head h).
+ * Sq == 1, causal == 0 replaces scalar_fused_decode_attend
+ * (veloxquant_mlx/metal/_scalar_attend.py:370-493); a leading layer axis of
+ * scalar_fused_decode_attend_batched (:496-647) folds into B; n_packed == 0
+ * replaces scalar_predecoded_attend (:702-779) and, with causal == 1,
+ * flash_prefill_attend (veloxquant_mlx/metal/_flash_prefill.py:171-237). */
+int vq_kivi_attend(const vq_attend_args *a);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VELOXQUANT_HIP_H */

@@ -1,0 +1,205 @@
+"""HIP attention over a group-affine quantised cache against the CPU oracle.
+
+Tolerance: max-abs < 2e-3 on the fp16 / fp32 output, the bar of the reference's
+own kernel tests (veloxquant_mlx/tests/metal/test_scalar_attend.py:140-200).
+Both sides consume the same codes / scales / zeros."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attend as oa, kivi as ok
+from tests._gpu import gpu, host, outlier_kv, require_gpu, to_dev
+from veloxquant_mlx_amd import kernels as K
+
+pytestmark = gpu
+TOL = 2e-3
+
+
+def _make_inputs(B, H, S_kv, D, b, g, seed=0, H_kv=None):
+    H_kv = H_kv or H
+    rng = np.random.default_rng(seed)
+    levels = (1 << b) - 1
+    q = rng.standard_normal((B, H, 1, D)).astype(np.float16)
+    kf = rng.standard_normal((B, H_kv, S_kv, D)).astype(np.float32)
+    vf = rng.standard_normal((B, H_kv, S_kv, D)).astype(np.float32)
+    return q, ok.group_quant_codes(kf, -2, g, levels), ok.group_quant_codes(vf, -1, g, levels)
+
+
+def _run_ref_api(q, kq, vq, g, scale, nsg=None):
+    args = [to_dev(q)] + [to_dev(a) for a in kq] + [to_dev(a) for a in vq]
+    return host(K.scalar_fused_decode_attend(*args, g, scale, nsg=nsg)).astype(np.float32)
+
+
+@pytest.mark.parametrize("S_kv", [64, 512, 2048])
+@pytest.mark.parametrize("nsg", [1, 8])
+def test_scalar_attend_parity(S_kv, nsg):
+    require_gpu()
+    q, kq, vq = _make_inputs(1, 4, S_kv, 128, 2, 32)
+    scale = 1 / math.sqrt(128)
+    out = _run_ref_api(q, kq, vq, 32, scale, nsg)
+    assert np.max(np.abs(out - oa.reference_attend(q, *kq, *vq, 32, scale))) < TOL
+
+
+@pytest.mark.parametrize("b", [2, 3, 4])
+@pytest.mark.parametrize("H,H_kv", [(8, 2), (32, 4), (32, 8), (8, 8)])
+def test_scalar_attend_bits_and_gqa(b, H, H_kv):
+    require_gpu()
+    q, kq, vq = _make_inputs(2, H, 300, 128, b, 32, seed=b + H, H_kv=H_kv)
+    scale = 1 / math.sqrt(128)
+    out = _run_ref_api(q, kq, vq, 32, scale)
+    assert np.max(np.abs(out - oa.reference_attend(q, *kq, *vq, 32, scale))) < TOL
+
+
+def test_scalar_attend_d256_and_group64():
+    require_gpu()
+    q, kq, vq = _make_inputs(2, 4, 200, 256, 4, 64, seed=5, H_kv=2)
+    out = _run_ref_api(q, kq, vq, 64, 1 / 16.0)
+    assert np.max(np.abs(out - oa.reference_attend(q, *kq, *vq, 64, 1 / 16.0))) < TOL
+
+
+def test_single_slot_and_uniform_scores():
+    require_gpu()
+    q, kq, vq = _make_inputs(1, 4, 1, 128, 2, 32, seed=7, H_kv=2)
+    out = _run_ref_api(q, kq, vq, 32, 0.1)
+    v_hat = ok.group_dequant(*vq, -1, 32)
+    np.testing.assert_allclose(out[:, :, 0], np.repeat(v_hat, 2, axis=1)[:, :, 0], atol=1e-3)
+    q, kq, vq = _make_inputs(1, 4, 96, 128, 4, 32, seed=8)
+    out = _run_ref_api(np.zeros_like(q), kq, vq, 32, 0.1)
+    np.testing.assert_allclose(out[:, :, 0], ok.group_dequant(*vq, -1, 32).mean(axis=2), atol=1e-3)
+
+
+def test_batched_layers_equal_per_layer_calls_bit_for_bit():
+    require_gpu()
+    NL = 3
+    layers = [_make_inputs(2, 8, 256, 128, 2, 32, seed=10 + l, H_kv=2) for l in range(NL)]
+    stack = lambda i, j=None: to_dev(np.stack([(L[i] if j is None else L[i][j]) for L in layers]))
+    out = K.scalar_fused_decode_attend_batched(stack(0), stack(1, 0), stack(1, 1), stack(1, 2), stack(2, 0),
+                                               stack(2, 1), stack(2, 2), 32, 0.09)
+    assert out.shape == (NL, 2, 8, 1, 128)
+    for l, (q, kq, vq) in enumerate(layers):
+        one = K.scalar_fused_decode_attend(to_dev(q), *[to_dev(a) for a in kq], *[to_dev(a) for a in vq], 32, 0.09)
+        assert torch.equal(out[l], one)
+
+
+def test_predecoded_and_flash_prefill_forms():
+    require_gpu()
+    rng = np.random.default_rng(20)
+    q = rng.standard_normal((2, 8, 1, 128)).astype(np.float16)
+    k = rng.standard_normal((2, 2, 333, 128)).astype(np.float16)
+    v = rng.standard_normal((2, 2, 333, 128)).astype(np.float16)
+    out = host(K.scalar_predecoded_attend(to_dev(q), to_dev(k), to_dev(v), 0.09)).astype(np.float32)
+    assert np.max(np.abs(out - oa.sdpa(q, k, v, 0.09))) < TOL
+    for (Sq, Skv, D, H) in [(64, 64, 64, 2), (40, 100, 128, 2), (1, 77, 128, 4), (130, 130, 32, 1)]:
+        rng = np.random.default_rng(D + Sq + Skv + H)
+        q = rng.standard_normal((1, H, Sq, D)).astype(np.float16)
+        k = rng.standard_normal((1, H, Skv, D)).astype(np.float16)
+        v = rng.standard_normal((1, H, Skv, D)).astype(np.float16)
+        sc = torch.tensor([1 / math.sqrt(D)], dtype=torch.float32)
+        out = host(K.flash_prefill_attend(to_dev(q), to_dev(k), to_dev(v), sc)).astype(np.float32)
+        assert np.max(np.abs(out - oa.sdpa(q, k, v, 1 / math.sqrt(D), causal=True))) < TOL
+    with pytest.raises(ValueError, match="exceeds S_kv"):
+        K.flash_prefill_attend(to_dev(q), to_dev(k[:, :, :5]), to_dev(v[:, :, :5]), 0.1)
+
+
+def test_future_keys_do_not_leak_into_earlier_rows():
+    require_gpu()
+    rng = np.random.default_rng(31)
+    q = to_dev(rng.standard_normal((1, 2, 24, 64)).astype(np.float16))
+    k = rng.standard_normal((1, 2, 40, 64)).astype(np.float16)
+    v = rng.standard_normal((1, 2, 40, 64)).astype(np.float16)
+    a = K.flash_prefill_attend(q, to_dev(k), to_dev(v), 0.125)
+    k[:, :, 30:] += 3.0
+    v[:, :, 30:] -= 2.0
+    b = K.flash_prefill_attend(q, to_dev(k), to_dev(v), 0.125)
+    assert torch.equal(a[:, :, :14], b[:, :, :14]) and not torch.equal(a[:, :, 14:], b[:, :, 14:])
+
+
+# ------------------------------------------------------------ packed cache path
+def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, causal=False, seed=0,
+                 q_dtype=torch.float16, cap_extra=0):
+    require_gpu()
+    per = 32 // b
+    k, v = outlier_kv((B, Hkv, n_packed + n_tail, D), seed=seed)
+    rng = np.random.default_rng(seed + 1)
+    q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float32)
+    qt = to_dev(q, q_dtype)
+    kt, vt = to_dev(k), to_dev(v)
+    scale = 1 / math.sqrt(D)
+    kw = {}
+    ref_args = [None] * 6
+    if n_packed:
+        cap = n_packed + cap_extra
+        dev = "cuda:0"
+        W = -(-D // per)
+        kp = torch.zeros((B, Hkv, cap, W), dtype=torch.int32, device=dev)
+        ks = torch.zeros((B, Hkv, -(-cap // g), D), dtype=meta, device=dev)
+        kz = torch.zeros_like(ks)
+        if v_layout == "token":
+            vp = torch.zeros((B, Hkv, cap // per, D), dtype=torch.int32, device=dev)
+            vs = torch.zeros((B, Hkv, -(-D // g), cap), dtype=meta, device=dev)
+        else:
+            vp = torch.zeros((B, Hkv, cap, W), dtype=torch.int32, device=dev)
+            vs = torch.zeros((B, Hkv, cap, -(-D // g)), dtype=meta, device=dev)
+        vz = torch.zeros_like(vs)
+        K.kivi_quant_pack(kt[:, :, :n_packed], -2, g, b, meta_dtype=meta, out=(kp, ks, kz))
+        K.kivi_quant_pack(vt[:, :, :n_packed], -1, g, b, meta_dtype=meta, v_layout=v_layout, out=(vp, vs, vz))
+        kw.update(k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz)
+        levels = (1 << b) - 1
+        npm = np.float16 if meta == torch.float16 else np.float32
+        kc, ksn, kzn = ok.group_quant_codes(k[:, :, :n_packed], -2, g, levels)
+        vc, vsn, vzn = ok.group_quant_codes(v[:, :, :n_packed], -1, g, levels)
+        ref_args = [kc, ksn.astype(npm), kzn.astype(npm), vc, vsn.astype(npm), vzn.astype(npm)]
+    tail_k = kt[:, :, n_packed:].contiguous() if n_tail else None
+    tail_v = vt[:, :, n_packed:].contiguous() if n_tail else None
+    out = K.kivi_packed_attend(qt, n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k,
+                               v_tail=tail_v, n_tail=n_tail, scale=scale, causal=causal,
+                               out_dtype=torch.float32, **kw)
+    ref = oa.kivi_attend(host(qt), *ref_args, g, k[:, :, n_packed:], v[:, :, n_packed:], scale, causal=causal)
+    err = float(np.max(np.abs(host(out) - ref)))
+    assert err < TOL, err
+    return err
+
+
+@pytest.mark.parametrize("v_layout", ["channel", "token"])
+@pytest.mark.parametrize("b,g", [(2, 32), (4, 64), (4, 32), (2, 64)])
+@pytest.mark.parametrize("meta", [torch.float16, torch.float32])
+def test_packed_decode_with_tail(v_layout, b, g, meta):
+    _packed_case(2, 8, 2, 512, 37, 128, b, g, v_layout, meta, seed=b + g)
+
+
+@pytest.mark.parametrize("v_layout", ["channel", "token"])
+def test_packed_decode_config1_llama_shape(v_layout):
+    """32 query heads / 8 kv heads, 8192 tokens 2-bit group 32 + 128-token fp16 tail."""
+    _packed_case(1, 32, 8, 8192, 128, 128, 2, 32, v_layout, torch.float16, seed=1)
+
+
+def test_packed_decode_no_tail_and_spare_capacity():
+    _packed_case(1, 8, 2, 256, 0, 128, 4, 64, "token", torch.float16, seed=3, cap_extra=256)
+    _packed_case(1, 8, 8, 128, 5, 64, 4, 32, "channel", torch.float32, seed=4, cap_extra=64)
+
+
+@pytest.mark.parametrize("Sq", [2, 5, 64])
+def test_packed_causal_multi_query(Sq):
+    _packed_case(1, 8, 2, 128, 64 + Sq, 128, 4, 32, "token", torch.float16, Sq=Sq, causal=True, seed=Sq)
+
+
+def test_packed_bf16_queries():
+    _packed_case(1, 8, 2, 256, 40, 128, 4, 32, "token", torch.float16, Sq=3, causal=True, seed=9,
+                 q_dtype=torch.bfloat16)
+
+
+def test_attend_errors():
+    require_gpu()
+    q = to_dev(np.zeros((1, 6, 1, 128), np.float16))
+    kc = to_dev(np.zeros((1, 4, 8, 128), np.uint8))
+    m = to_dev(np.zeros((1, 4, 1, 128), np.float32))
+    mv = to_dev(np.zeros((1, 4, 8, 4), np.float32))
+    with pytest.raises(ValueError, match="multiple of H_kv"):
+        K.scalar_fused_decode_attend(q, kc, m, m, kc, mv, mv, 32, 0.1)
+    with pytest.raises(ValueError, match="must be 4D"):
+        K.scalar_fused_decode_attend(q[0], kc, m, m, kc, mv, mv, 32, 0.1)
+    with pytest.raises(ValueError, match="nsg=40 must be in 1..32"):
+        K.scalar_fused_decode_attend(q, kc, m, m, kc, mv, mv, 32, 0.1, nsg=40)

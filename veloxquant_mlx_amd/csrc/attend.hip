@@ -1,0 +1,88 @@
+// C entry points for attention over a packed KIVI cache: validation, the split
+// plan, workspace sizing and kernel dispatch.
+#include "attend.hpp"
+
+namespace vq {
+
+AttendPlan plan_attend(const vq_attend_args &a) {
+    AttendPlan p;
+    const int64_t n_total = a.n_packed + a.n_tail;
+    const int64_t max_splits = n_total > 0 ? cdiv(n_total, 64) : 1;
+    p.path = mfma_decode_supported(a) ? 1 : 0;
+    // units of parallel work before splitting: a wave per query row (generic)
+    // or a four-wave block per kv head (MFMA)
+    const int64_t units = p.path == 1 ? a.B * a.Hkv : a.B * a.Hq * a.Sq;
+    const int64_t target = p.path == 1 ? 1024 : 4096;
+    int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);
+    if (ns > max_splits) ns = max_splits;
+    if (ns > 512) ns = 512;
+    if (ns < 1) ns = 1;
+    int64_t len = cdiv(cdiv(n_total > 0 ? n_total : 1, ns), 64) * 64;
+    ns = n_total > 0 ? cdiv(n_total, len) : 1;
+    p.nsplit = (int)ns;
+    p.split_len = len;
+    return p;
+}
+
+static int validate(const vq_attend_args *a, const char *fn) {
+    VQ_REQUIRE(a != nullptr, VQ_ERR_INVALID, "%s: null argument block", fn);
+    VQ_REQUIRE(a->B >= 1 && a->Hq >= 1 && a->Hkv >= 1 && a->Sq >= 1 && a->D >= 1, VQ_ERR_INVALID,
+               "%s: q must be 4D with positive sizes, got B=%lld Hq=%lld Sq=%lld D=%lld", fn, (long long)a->B,
+               (long long)a->Hq, (long long)a->Sq, (long long)a->D);
+    VQ_REQUIRE(a->D <= 256, VQ_ERR_INVALID, "%s: D=%lld must be <= 256", fn, (long long)a->D);
+    VQ_REQUIRE(a->Hq % a->Hkv == 0, VQ_ERR_INVALID,
+               "%s: H_q=%lld must be a multiple of H_kv=%lld for GQA head-packing", fn, (long long)a->Hq,
+               (long long)a->Hkv);
+    VQ_REQUIRE(a->n_packed >= 0 && a->n_tail >= 0, VQ_ERR_INVALID, "%s: negative token count", fn);
+    VQ_REQUIRE(a->n_packed + a->n_tail >= 1, VQ_ERR_INVALID, "%s: no key/value slots to attend to", fn);
+    VQ_REQUIRE(a->Sq <= a->n_packed + a->n_tail || !a->causal, VQ_ERR_INVALID,
+               "%s: S_q=%lld exceeds S_kv=%lld; queries align to the tail of the KV cache", fn, (long long)a->Sq,
+               (long long)(a->n_packed + a->n_tail));
+    VQ_REQUIRE(is_float_tag(a->q_dtype) && is_float_tag(a->out_dtype), VQ_ERR_INVALID, "%s: unsupported q/out dtype", fn);
+    if (a->n_packed > 0) {
+        VQ_REQUIRE(a->pack_bits >= 1 && a->pack_bits <= 8, VQ_ERR_INVALID, "%s: pack_bits must be in 1..8", fn);
+        VQ_REQUIRE(a->group >= 1, VQ_ERR_INVALID, "%s: group_size must be >= 1", fn);
+        VQ_REQUIRE(a->meta_dtype == VQ_F32 || a->meta_dtype == VQ_F16, VQ_ERR_INVALID, "%s: meta dtype must be f32/f16", fn);
+        VQ_REQUIRE(a->v_layout == VQ_V_CHANNEL_PACKED || a->v_layout == VQ_V_TOKEN_PACKED, VQ_ERR_INVALID, "%s: bad v_layout", fn);
+        VQ_REQUIRE(a->cap_tokens >= a->n_packed, VQ_ERR_INVALID, "%s: n_packed exceeds cap_tokens", fn);
+        if (a->v_layout == VQ_V_TOKEN_PACKED)
+            VQ_REQUIRE(a->cap_tokens % (32 / a->pack_bits) == 0, VQ_ERR_INVALID, "%s: cap_tokens not word aligned", fn);
+    }
+    if (a->n_tail > 0) {
+        VQ_REQUIRE(is_float_tag(a->tail_dtype), VQ_ERR_INVALID, "%s: unsupported tail dtype", fn);
+        VQ_REQUIRE(a->tail_cap >= a->n_tail, VQ_ERR_INVALID, "%s: n_tail exceeds tail_cap", fn);
+    }
+    return VQ_OK;
+}
+
+}  // namespace vq
+
+using namespace vq;
+
+extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
+    if (!a) return 0;
+    AttendPlan p = plan_attend(*a);
+    return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nsplit * (size_t)(a->D + 2) * sizeof(float);
+}
+
+extern "C" int vq_kivi_attend(const vq_attend_args *a) {
+    const char *fn = "vq_kivi_attend";
+    int rc = validate(a, fn);
+    if (rc != VQ_OK) return rc;
+    VQ_REQUIRE(a->q && a->out, VQ_ERR_INVALID, "%s: null q/out", fn);
+    if (a->n_packed > 0)
+        VQ_REQUIRE(a->k_packed && a->v_packed && a->k_scale && a->k_zero && a->v_scale && a->v_zero, VQ_ERR_INVALID,
+                   "%s: null packed-cache pointer", fn);
+    if (a->n_tail > 0) VQ_REQUIRE(a->k_tail && a->v_tail, VQ_ERR_INVALID, "%s: null tail pointer", fn);
+    AttendPlan p = plan_attend(*a);
+    size_t need = vq_kivi_attend_workspace(a);
+    VQ_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, VQ_ERR_WORKSPACE,
+               "%s: workspace of %zu bytes required, %zu given", fn, need, a->workspace_bytes);
+    if (p.path == 1) rc = launch_attend_mfma_decode(*a, p.nsplit, p.split_len);
+    else rc = launch_attend_generic(*a, p.nsplit, p.split_len);
+    if (rc != VQ_OK) return rc;
+    VQ_HIP_CHECK_LAUNCH(fn);
+    rc = launch_attend_merge(*a, p.nsplit);
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return rc;
+}

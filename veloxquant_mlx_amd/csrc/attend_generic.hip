@@ -1,0 +1,151 @@
+// Layout-agnostic attention over [quantised prefix | tail] and the split merge.
+//
+// One wave per (query row, token split): lanes stripe the head dimension, each
+// slot's key is rebuilt as code*scale+zero in float32, the dot product is
+// reduced across the wave, and an online softmax accumulates the rebuilt value
+// row -- the scheme of veloxquant_mlx/metal/src/scalar_affine_attend.metal:57-106
+// with the split moved from SIMD groups of one threadgroup to independent
+// waves whose (max, sum, accumulator) partials are merged by a second kernel
+// (the merge of scalar_affine_attend.metal:149-174).
+//
+// This path accepts every head_dim <= 256, bit width, group size, value layout
+// and tail dtype; the MFMA kernels in attend_mfma.hip cover the shapes that
+// matter for throughput and share the partial format and the merge kernel.
+#include "attend.hpp"
+
+namespace vq {
+
+__device__ __forceinline__ float ld_tag(const void *p, int tag, int64_t i) {
+    if (tag == VQ_F16) return (float)((const f16 *)p)[i];
+    if (tag == VQ_BF16) return bf16_to_f32(((const u16 *)p)[i]);
+    return ((const float *)p)[i];
+}
+__device__ __forceinline__ void st_tag(void *p, int tag, int64_t i, float v) {
+    if (tag == VQ_F16) ((f16 *)p)[i] = (f16)v;
+    else if (tag == VQ_BF16) ((u16 *)p)[i] = f32_to_bf16(v);
+    else ((float *)p)[i] = v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void attend_generic_kernel(vq_attend_args a, int nsplit, int64_t split_len,
+                                                             float *__restrict__ ws) {
+    const int lane = threadIdx.x & 63;
+    const int64_t wid = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t rows = a.B * a.Hq * a.Sq;
+    if (wid >= rows * nsplit) return;  // whole waves leave together
+    const int64_t row = wid / nsplit;
+    const int sp = (int)(wid % nsplit);
+    const int64_t iq = row % a.Sq, h = (row / a.Sq) % a.Hq, b = row / (a.Sq * a.Hq);
+    const int64_t hpk = a.Hq / a.Hkv, bh = b * a.Hkv + h / hpk;
+    const int64_t D = a.D, n_total = a.n_packed + a.n_tail;
+    const int64_t last = a.causal ? (n_total - a.Sq + iq) : (n_total - 1);
+    int64_t t0 = (int64_t)sp * split_len, t1 = t0 + split_len;
+    if (t1 > last + 1) t1 = last + 1;
+
+    const int bits = a.pack_bits, per = 32 / bits, g = a.group;
+    const uint32_t mask = (1u << bits) - 1u;
+    const int64_t W = (D + per - 1) / per, GV = (D + g - 1) / g, GKcap = (a.cap_tokens + g - 1) / g;
+    const uint32_t *kp = (const uint32_t *)a.k_packed, *vp = (const uint32_t *)a.v_packed;
+
+    float qv[4], acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int64_t d = lane + 64 * j;
+        qv[j] = d < D ? ld_tag(a.q, a.q_dtype, row * D + d) : 0.0f;
+        acc[j] = 0.0f;
+    }
+    float m = -INFINITY, l = 0.0f;
+    for (int64_t t = t0; t < t1; ++t) {
+        float kh[4], vh[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int64_t d = lane + 64 * j;
+            kh[j] = 0.0f; vh[j] = 0.0f;
+            if (d >= D) continue;
+            if (t < a.n_packed) {
+                uint32_t kw = kp[(bh * a.cap_tokens + t) * W + d / per];
+                float kc = (float)((kw >> ((d % per) * bits)) & mask);
+                int64_t kmi = (bh * GKcap + t / g) * D + d;
+                kh[j] = __fadd_rn(__fmul_rn(kc, ld_tag(a.k_scale, a.meta_dtype, kmi)), ld_tag(a.k_zero, a.meta_dtype, kmi));
+                uint32_t vw;
+                int sh;
+                int64_t vmi;
+                if (a.v_layout == VQ_V_CHANNEL_PACKED) {
+                    vw = vp[(bh * a.cap_tokens + t) * W + d / per];
+                    sh = (int)(d % per) * bits;
+                    vmi = (bh * a.cap_tokens + t) * GV + d / g;
+                } else {
+                    vw = vp[(bh * (a.cap_tokens / per) + t / per) * D + d];
+                    sh = (int)(t % per) * bits;
+                    vmi = (bh * GV + d / g) * a.cap_tokens + t;
+                }
+                float vc = (float)((vw >> sh) & mask);
+                vh[j] = __fadd_rn(__fmul_rn(vc, ld_tag(a.v_scale, a.meta_dtype, vmi)), ld_tag(a.v_zero, a.meta_dtype, vmi));
+            } else {
+                int64_t ti = (bh * a.tail_cap + (t - a.n_packed)) * D + d;
+                kh[j] = ld_tag(a.k_tail, a.tail_dtype, ti);
+                vh[j] = ld_tag(a.v_tail, a.tail_dtype, ti);
+            }
+        }
+        float dot = qv[0] * kh[0] + qv[1] * kh[1] + qv[2] * kh[2] + qv[3] * kh[3];
+        float s = wave_sum(dot) * a.scale;
+        float mn = fmaxf(m, s);
+        float f = __expf(m - mn), w = __expf(s - mn);
+        l = l * f + w;
+        m = mn;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = acc[j] * f + w * vh[j];
+    }
+    float *o = ws + (row * nsplit + sp) * (D + 2);
+    if (lane == 0) { o[0] = m; o[1] = l; }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int64_t d = lane + 64 * j;
+        if (d < D) o[2 + d] = acc[j];
+    }
+}
+
+__global__ void attend_merge_kernel(const float *__restrict__ ws, int64_t rows, int nsplit, int64_t D,
+                                    void *__restrict__ out, int out_dtype) {
+    const int64_t n = rows * D;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t row = e / D, d = e % D;
+        const float *p = ws + row * nsplit * (D + 2);
+        float gm = -INFINITY;
+        for (int s = 0; s < nsplit; ++s) gm = fmaxf(gm, p[s * (D + 2)]);
+        float den = 0.0f, num = 0.0f;
+        for (int s = 0; s < nsplit; ++s) {
+            float ms = p[s * (D + 2)];
+            if (ms == -INFINITY) continue;
+            float f = __expf(ms - gm);
+            den += p[s * (D + 2) + 1] * f;
+            num += p[s * (D + 2) + 2 + d] * f;
+        }
+        st_tag(out, out_dtype, e, den > 0.0f ? num / den : 0.0f);
+    }
+}
+
+int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len) {
+    hipStream_t st = (hipStream_t)a.stream;
+    const int64_t rows = a.B * a.Hq * a.Sq;
+    const int64_t waves = rows * nsplit;
+    hipLaunchKernelGGL(attend_generic_kernel, dim3((unsigned)cdiv(waves, 4)), dim3(256), 0, st, a, nsplit, split_len,
+                       (float *)a.workspace);
+    return VQ_OK;
+}
+
+int launch_attend_merge(const vq_attend_args &a, int nsplit) {
+    hipStream_t st = (hipStream_t)a.stream;
+    const int64_t rows = a.B * a.Hq * a.Sq;
+    int64_t g = cdiv(rows * a.D, 256);
+    if (g > (1 << 20)) g = 1 << 20;
+    hipLaunchKernelGGL(attend_merge_kernel, dim3((unsigned)g), dim3(256), 0, st, (const float *)a.workspace, rows,
+                       nsplit, a.D, a.out, a.out_dtype);
+    return VQ_OK;
+}
+
+}  // namespace vq

@@ -1,0 +1,627 @@
+// KIVI asymmetric group quantisation, bit packing and reconstruction for gfx950.
+//
+// Math (float32, one rounding per operation, no contraction):
+//   scale = max((gmax - gmin) / levels, eps)
+//   code  = clamp(rint((x - gmin) / scale), 0, levels)      rint = half-to-even
+//   xhat  = code * scale + gmin                              (two roundings)
+// as in veloxquant_mlx/cache/kivi_cache.py:181-201 and
+// veloxquant_mlx/metal/src/kivi_group_quant_{channel,token}.metal.
+//
+// Two kinds of kernels:
+//   * tile kernels for head_dim 64/128/256 with 128-bit loads; key groups are
+//     reduced with wavefront shuffles plus one LDS exchange between the four
+//     waves of a block, value groups with shuffles only;
+//   * generic kernels (any head_dim / group / bit width) in which every thread
+//     rescans the group it needs -- slow but free of layout assumptions.
+#include "common.hpp"
+
+namespace vq {
+
+__device__ __forceinline__ float quant_code(float v, float mn, float sc, float levels) {
+    float q = rintf(__fdiv_rn(__fsub_rn(v, mn), sc));
+    return fminf(fmaxf(q, 0.0f), levels);
+}
+__device__ __forceinline__ float recon(float q, float sc, float mn) {
+    return __fadd_rn(__fmul_rn(q, sc), mn);
+}
+__device__ __forceinline__ float group_scale(float mn, float mx, float levels, float eps) {
+    return fmaxf(__fdiv_rn(__fsub_rn(mx, mn), levels), eps);
+}
+
+template <typename T> __device__ __forceinline__ void load8(const T *p, float (&v)[8]);
+template <> __device__ __forceinline__ void load8<f16>(const f16 *p, float (&v)[8]) {
+    f16x8 h = *reinterpret_cast<const f16x8 *>(p);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)h[i];
+}
+template <> __device__ __forceinline__ void load8<bf16_t>(const bf16_t *p, float (&v)[8]) {
+    uint4 u = *reinterpret_cast<const uint4 *>(p);
+    uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+template <> __device__ __forceinline__ void load8<float>(const float *p, float (&v)[8]) {
+    float4 a = *reinterpret_cast<const float4 *>(p);
+    float4 b = *reinterpret_cast<const float4 *>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <typename T> __device__ __forceinline__ void store8(T *p, const float (&v)[8]);
+template <> __device__ __forceinline__ void store8<f16>(f16 *p, const float (&v)[8]) {
+    f16x8 h;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) h[i] = (f16)v[i];
+    *reinterpret_cast<f16x8 *>(p) = h;
+}
+template <> __device__ __forceinline__ void store8<bf16_t>(bf16_t *p, const float (&v)[8]) {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)f32_to_bf16(v[2 * i]) | ((uint32_t)f32_to_bf16(v[2 * i + 1]) << 16);
+    *reinterpret_cast<uint4 *>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+}
+template <> __device__ __forceinline__ void store8<float>(float *p, const float (&v)[8]) {
+    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4 *>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+template <typename M> __device__ __forceinline__ void store_meta(M *p, float v);
+template <> __device__ __forceinline__ void store_meta<float>(float *p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_meta<f16>(f16 *p, float v) { *p = (f16)v; }
+template <typename M> __device__ __forceinline__ float load_meta(const M *p);
+template <> __device__ __forceinline__ float load_meta<float>(const float *p) { return *p; }
+template <> __device__ __forceinline__ float load_meta<f16>(const f16 *p) { return (float)*p; }
+
+// Write the eight codes one thread owns (channels 8*o .. 8*o+7 of one row) as
+// part of a channel-packed row of words.  Every lane of the wave must call it.
+template <int LPR>
+__device__ __forceinline__ void store_codes_channel_packed(uint32_t *row_words, int o, const uint32_t (&c)[8],
+                                                           int bits, bool valid) {
+    if (bits == 8) {
+        if (valid) {
+            uint32_t w0 = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+            uint32_t w1 = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+            *reinterpret_cast<uint2 *>(row_words + 2 * o) = make_uint2(w0, w1);
+        }
+    } else if (bits == 4) {
+        uint32_t w = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w |= c[i] << (4 * i);
+        if (valid) row_words[o] = w;
+    } else if (bits == 2) {
+        uint32_t f = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f |= c[i] << (2 * i);
+        uint32_t hi = __shfl_down(f, 1);
+        if (valid && (o & 1) == 0) row_words[o >> 1] = f | (hi << 16);
+    } else {  // bits == 1
+        uint32_t f = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) f |= c[i] << i;
+        uint32_t f1 = __shfl_down(f, 1), f2 = __shfl_down(f, 2), f3 = __shfl_down(f, 3);
+        if (valid && (o & 3) == 0) row_words[o >> 2] = f | (f1 << 8) | (f2 << 16) | (f3 << 24);
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Keys: groups along tokens.  One block per (group, bh); 256 threads = RPP rows
+// of LPR threads, each thread owning 8 consecutive channels of its rows.
+// MODE 0: write the reconstruction; MODE 1: write packed codes + scale/zero.
+// ---------------------------------------------------------------------------
+constexpr int KT_MAXP = 8;
+
+template <typename T, typename M, int LPR, int MODE>
+__global__ __launch_bounds__(256) void kivi_key_tile_kernel(
+    const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
+    float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
+    int64_t cap_tokens, int64_t dst_tok0, int W) {
+    constexpr int D = LPR * 8;
+    constexpr int RPP = 256 / LPR;
+    __shared__ float s_mn[4][D];
+    __shared__ float s_mx[4][D];
+    const int gk = blockIdx.x;
+    const int64_t bh = blockIdx.y;
+    const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int64_t s0 = (int64_t)gk * group;
+    const T *xb = x + bh * x_stride_bh;
+
+    float v[KT_MAXP][8];
+    float mn[8], mx[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { mn[i] = INFINITY; mx[i] = -INFINITY; }
+#pragma unroll
+    for (int p = 0; p < KT_MAXP; ++p) {
+        int rl = p * RPP + r;
+        int64_t s = s0 + rl;
+        if (rl < group && s < S) {
+            load8<T>(xb + s * D + 8 * o, v[p]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { mn[i] = fminf(mn[i], v[p][i]); mx[i] = fmaxf(mx[i], v[p][i]); }
+        }
+    }
+#pragma unroll
+    for (int off = LPR; off < 64; off <<= 1) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            mn[i] = fminf(mn[i], __shfl_xor(mn[i], off));
+            mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], off));
+        }
+    }
+    if (lane < LPR) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { s_mn[wave][8 * o + i] = mn[i]; s_mx[wave][8 * o + i] = mx[i]; }
+    }
+    __syncthreads();
+    float sc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        float a = fminf(fminf(s_mn[0][8 * o + i], s_mn[1][8 * o + i]), fminf(s_mn[2][8 * o + i], s_mn[3][8 * o + i]));
+        float b = fmaxf(fmaxf(s_mx[0][8 * o + i], s_mx[1][8 * o + i]), fmaxf(s_mx[2][8 * o + i], s_mx[3][8 * o + i]));
+        mn[i] = a;
+        sc[i] = group_scale(a, b, levels, eps);
+    }
+    if (MODE == 1 && r == 0) {
+        int64_t gdst = dst_tok0 / group + gk;
+        int64_t gcap = (cap_tokens + group - 1) / group;
+        M *sp = scale + (bh * gcap + gdst) * D + 8 * o;
+        M *zp = zero + (bh * gcap + gdst) * D + 8 * o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { store_meta<M>(sp + i, sc[i]); store_meta<M>(zp + i, mn[i]); }
+    }
+#pragma unroll
+    for (int p = 0; p < KT_MAXP; ++p) {
+        int rl = p * RPP + r;
+        int64_t s = s0 + rl;
+        bool valid = rl < group && s < S;
+        if (p * RPP >= group) break;  // uniform across the block
+        if (MODE == 0) {
+            if (valid) {
+                float y[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) y[i] = recon(quant_code(v[p][i], mn[i], sc[i], levels), sc[i], mn[i]);
+                store8<T>(out + (bh * S + s) * D + 8 * o, y);
+            }
+        } else {
+            uint32_t c[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) c[i] = valid ? (uint32_t)quant_code(v[p][i], mn[i], sc[i], levels) : 0u;
+            uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;
+            store_codes_channel_packed<LPR>(row, o, c, bits, valid);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Values: groups along channels.  One block per (row tile, bh); a group is
+// reduced across g/8 neighbouring lanes.  MODE 0 reconstruction, MODE 1
+// channel-packed codes, MODE 2 token-packed codes (transposed through LDS).
+// ---------------------------------------------------------------------------
+template <typename T, typename M, int LPR, int MODE>
+__global__ __launch_bounds__(256) void kivi_value_tile_kernel(
+    const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
+    float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
+    int64_t cap_tokens, int64_t dst_tok0, int W) {
+    constexpr int D = LPR * 8;
+    constexpr int RPP = 256 / LPR;
+    constexpr int LDS_STRIDE = D + 8;
+    __shared__ __align__(8) unsigned char s_codes[MODE == 2 ? RPP * LDS_STRIDE : 4];
+    const int64_t bh = blockIdx.y;
+    const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
+    const int64_t s = (int64_t)blockIdx.x * RPP + r;
+    const bool valid = s < S;
+    const int GL = group / 8;  // lanes per group (power of two <= LPR)
+    const int GV = D / group;
+
+    float v[8];
+    float mn = INFINITY, mx = -INFINITY;
+    if (valid) {
+        load8<T>(x + bh * x_stride_bh + s * D + 8 * o, v);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { mn = fminf(mn, v[i]); mx = fmaxf(mx, v[i]); }
+    }
+    for (int off = 1; off < GL; off <<= 1) {
+        mn = fminf(mn, __shfl_xor(mn, off));
+        mx = fmaxf(mx, __shfl_xor(mx, off));
+    }
+    const float sc = group_scale(mn, mx, levels, eps);
+    if (MODE != 0 && valid && (o % GL) == 0) {
+        int gv = o / GL;
+        int64_t mi = (MODE == 1) ? ((bh * cap_tokens + dst_tok0 + s) * GV + gv)
+                                 : ((bh * GV + gv) * cap_tokens + dst_tok0 + s);
+        store_meta<M>(scale + mi, sc);
+        store_meta<M>(zero + mi, mn);
+    }
+    if (MODE == 0) {
+        if (valid) {
+            float y[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) y[i] = recon(quant_code(v[i], mn, sc, levels), sc, mn);
+            store8<T>(out + (bh * S + s) * D + 8 * o, y);
+        }
+        return;
+    }
+    uint32_t c[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) c[i] = valid ? (uint32_t)quant_code(v[i], mn, sc, levels) : 0u;
+    if (MODE == 1) {
+        uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;
+        store_codes_channel_packed<LPR>(row, o, c, bits, valid);
+    } else {
+        uint32_t w0 = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+        uint32_t w1 = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+        *reinterpret_cast<uint2 *>(&s_codes[r * LDS_STRIDE + 8 * o]) = make_uint2(w0, w1);
+        __syncthreads();
+        const int per = 32 / bits;
+        const int nwords = (RPP / per) * D;
+        const int64_t tile_tok0 = (int64_t)blockIdx.x * RPP;
+        for (int idx = tid; idx < nwords; idx += 256) {
+            int wl = idx / D, d = idx % D;
+            if (tile_tok0 + (int64_t)wl * per >= S) continue;
+            uint32_t w = 0;
+            for (int i = 0; i < per; ++i) w |= (uint32_t)s_codes[(wl * per + i) * LDS_STRIDE + d] << (i * bits);
+            int64_t wrow = (dst_tok0 + tile_tok0) / per + wl;
+            packed[(bh * (cap_tokens / per) + wrow) * D + d] = w;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+// Generic kernels: every thread rescans the group(s) it needs.
+// ---------------------------------------------------------------------------
+template <typename T>
+__device__ __forceinline__ void scan_group(const T *xb, int64_t S, int64_t D, int axis, int group, int64_t s,
+                                           int64_t d, float &mn, float &mx) {
+    mn = INFINITY; mx = -INFINITY;
+    if (axis == VQ_AXIS_TOKEN) {
+        int64_t a = (s / group) * group, b = a + group < S ? a + group : S;
+        for (int64_t t = a; t < b; ++t) { float v = Elem<T>::ld(xb + t * D + d); mn = fminf(mn, v); mx = fmaxf(mx, v); }
+    } else {
+        int64_t a = (d / group) * group, b = a + group < D ? a + group : D;
+        for (int64_t t = a; t < b; ++t) { float v = Elem<T>::ld(xb + s * D + t); mn = fminf(mn, v); mx = fmaxf(mx, v); }
+    }
+}
+
+template <typename T>
+__global__ void kivi_roundtrip_generic_kernel(const T *__restrict__ x, T *__restrict__ out, int64_t BH, int64_t S,
+                                              int64_t D, int axis, int group, float levels, float eps) {
+    int64_t n = BH * S * D;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t d = e % D, s = (e / D) % S, bh = e / (D * S);
+        const T *xb = x + bh * S * D;
+        float mn, mx;
+        scan_group<T>(xb, S, D, axis, group, s, d, mn, mx);
+        float sc = group_scale(mn, mx, levels, eps);
+        float v = Elem<T>::ld(xb + s * D + d);
+        Elem<T>::st(out + e, recon(quant_code(v, mn, sc, levels), sc, mn));
+    }
+}
+
+// One thread per output word.  layout 0: word = `per` channels of one token
+// (keys, or channel-packed values); layout 1: word = `per` tokens of one channel.
+template <typename T, typename M>
+__global__ void kivi_pack_generic_kernel(const T *__restrict__ x, int64_t BH, int64_t S, int64_t D,
+                                         int64_t x_stride_bh, int axis, int group, float levels, float eps,
+                                         int bits, int layout, uint32_t *__restrict__ packed,
+                                         M *__restrict__ scale, M *__restrict__ zero, int64_t cap_tokens,
+                                         int64_t dst_tok0) {
+    const int per = 32 / bits;
+    const int64_t W = (D + per - 1) / per;
+    const int64_t GV = (D + group - 1) / group;
+    const int64_t GKcap = (cap_tokens + group - 1) / group;
+    const int64_t rows = layout == 0 ? S : (S + per - 1) / per;
+    const int64_t cols = layout == 0 ? W : D;
+    const int64_t n = BH * rows * cols;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t c = e % cols, rr = (e / cols) % rows, bh = e / (cols * rows);
+        const T *xb = x + bh * x_stride_bh;
+        uint32_t word = 0;
+        for (int i = 0; i < per; ++i) {
+            int64_t s = layout == 0 ? rr : rr * per + i;
+            int64_t d = layout == 0 ? c * per + i : c;
+            if (s >= S || d >= D) continue;
+            float mn, mx;
+            scan_group<T>(xb, S, D, axis, group, s, d, mn, mx);
+            float sc = group_scale(mn, mx, levels, eps);
+            float v = Elem<T>::ld(xb + s * D + d);
+            word |= (uint32_t)quant_code(v, mn, sc, levels) << (i * bits);
+            // the thread that meets the first element of a group records its parameters
+            if (axis == VQ_AXIS_TOKEN) {
+                if (s % group == 0) {
+                    int64_t mi = (bh * GKcap + (dst_tok0 + s) / group) * D + d;
+                    store_meta<M>(scale + mi, sc);
+                    store_meta<M>(zero + mi, mn);
+                }
+            } else if (d % group == 0) {
+                int64_t mi = layout == 0 ? ((bh * cap_tokens + dst_tok0 + s) * GV + d / group)
+                                         : ((bh * GV + d / group) * cap_tokens + dst_tok0 + s);
+                store_meta<M>(scale + mi, sc);
+                store_meta<M>(zero + mi, mn);
+            }
+        }
+        if (layout == 0)
+            packed[(bh * cap_tokens + dst_tok0 + rr) * W + c] = word;
+        else
+            packed[(bh * (cap_tokens / per) + dst_tok0 / per + rr) * D + c] = word;
+    }
+}
+
+// Reconstruction from packed codes: one thread per output element.
+template <typename O, typename M>
+__global__ void kivi_dequant_kernel(const uint32_t *__restrict__ packed, const M *__restrict__ scale,
+                                    const M *__restrict__ zero, int64_t BH, int64_t S, int64_t D, int axis,
+                                    int group, int bits, int layout, int64_t cap_tokens, int64_t src_tok0,
+                                    O *__restrict__ out) {
+    const int per = 32 / bits;
+    const int64_t W = (D + per - 1) / per;
+    const int64_t GV = (D + group - 1) / group;
+    const int64_t GKcap = (cap_tokens + group - 1) / group;
+    const uint32_t mask = bits == 32 ? 0xffffffffu : ((1u << bits) - 1u);
+    const int64_t n = BH * S * D;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t d = e % D, s = (e / D) % S, bh = e / (D * S);
+        int64_t t = src_tok0 + s;
+        uint32_t word;
+        int sh;
+        if (layout == 0) {
+            word = packed[(bh * cap_tokens + t) * W + d / per];
+            sh = (int)(d % per) * bits;
+        } else {
+            word = packed[(bh * (cap_tokens / per) + t / per) * D + d];
+            sh = (int)(t % per) * bits;
+        }
+        float c = (float)((word >> sh) & mask);
+        int64_t mi;
+        if (axis == VQ_AXIS_TOKEN) mi = (bh * GKcap + t / group) * D + d;
+        else mi = layout == 0 ? ((bh * cap_tokens + t) * GV + d / group) : ((bh * GV + d / group) * cap_tokens + t);
+        Elem<O>::st(out + e, recon(c, load_meta<M>(scale + mi), load_meta<M>(zero + mi)));
+    }
+}
+
+__global__ void pack_words_kernel(const uint8_t *__restrict__ idx, int64_t rows, int64_t D, int bits,
+                                  uint32_t *__restrict__ words) {
+    const int per = 32 / bits;
+    const int64_t W = (D + per - 1) / per, n = rows * W;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t w = e % W, r = e / W;
+        uint32_t acc = 0;
+        for (int i = 0; i < per; ++i) {
+            int64_t d = w * per + i;
+            if (d < D) acc |= ((uint32_t)idx[r * D + d]) << (i * bits);
+        }
+        words[e] = acc;
+    }
+}
+__global__ void unpack_words_kernel(const uint32_t *__restrict__ words, int64_t rows, int64_t D, int bits,
+                                    uint8_t *__restrict__ idx) {
+    const int per = 32 / bits;
+    const int64_t W = (D + per - 1) / per, n = rows * D;
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        int64_t d = e % D, r = e / D;
+        idx[e] = (uint8_t)((words[r * W + d / per] >> ((d % per) * bits)) & mask);
+    }
+}
+__global__ void bit_pack_kernel(const uint8_t *__restrict__ idx, int64_t nbytes, int bits, uint8_t *__restrict__ packed) {
+    const int per = 8 / bits;
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < nbytes; e += (int64_t)gridDim.x * blockDim.x) {
+        uint32_t acc = 0;
+        for (int i = 0; i < per; ++i) acc |= ((uint32_t)idx[e * per + i] & mask) << (i * bits);
+        packed[e] = (uint8_t)acc;
+    }
+}
+__global__ void bit_unpack_kernel(const uint8_t *__restrict__ packed, int64_t n, int bits, uint8_t *__restrict__ idx) {
+    const int per = 8 / bits;
+    const uint32_t mask = (1u << bits) - 1u;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x)
+        idx[e] = (uint8_t)((packed[e / per] >> ((e % per) * bits)) & mask);
+}
+
+static inline int grid_for(int64_t n, int block) {
+    int64_t g = (n + block - 1) / block;
+    if (g < 1) g = 1;
+    if (g > 65536 * 16) g = 65536 * 16;
+    return (int)g;
+}
+static inline bool pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
+static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace vq
+
+using namespace vq;
+
+// ---- launchers ----------------------------------------------------------------
+
+template <typename T, typename M, int LPR>
+static void launch_key_tile(int mode, const void *x, void *out, int64_t BH, int64_t S, int64_t xs, int group,
+                            int levels, float eps, int bits, void *packed, void *scale, void *zero, int64_t cap,
+                            int64_t tok0, hipStream_t st) {
+    dim3 grid((unsigned)cdiv(S, group), (unsigned)BH);
+    int W = (int)cdiv(LPR * 8, 32 / (bits > 0 ? bits : 8));
+    if (mode == 0)
+        hipLaunchKernelGGL((kivi_key_tile_kernel<T, M, LPR, 0>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, xs,
+                           group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W);
+    else
+        hipLaunchKernelGGL((kivi_key_tile_kernel<T, M, LPR, 1>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, xs,
+                           group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W);
+}
+template <typename T, typename M, int LPR>
+static void launch_value_tile(int mode, const void *x, void *out, int64_t BH, int64_t S, int64_t xs, int group,
+                              int levels, float eps, int bits, void *packed, void *scale, void *zero, int64_t cap,
+                              int64_t tok0, hipStream_t st) {
+    constexpr int RPP = 256 / LPR;
+    dim3 grid((unsigned)cdiv(S, RPP), (unsigned)BH);
+    int W = (int)cdiv(LPR * 8, 32 / (bits > 0 ? bits : 8));
+#define VQ_LV(MODE)                                                                                                  \
+    hipLaunchKernelGGL((kivi_value_tile_kernel<T, M, LPR, MODE>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, \
+                       xs, group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W)
+    if (mode == 0) VQ_LV(0);
+    else if (mode == 1) VQ_LV(1);
+    else VQ_LV(2);
+#undef VQ_LV
+}
+
+// mode: 0 round trip, 1 channel-packed codes, 2 token-packed codes (values only)
+template <typename T, typename M>
+static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t BH, int64_t S, int64_t D, int64_t xs,
+                          int group, int levels, float eps, int bits, void *packed, void *scale, void *zero,
+                          int64_t cap, int64_t tok0, hipStream_t st) {
+    if (!(D == 64 || D == 128 || D == 256)) return false;
+    if (!aligned16(x) || (xs % 8) != 0 || BH > 65535) return false;
+    if (mode == 0 && !aligned16(out)) return false;
+    if (mode != 0 && !(bits == 1 || bits == 2 || bits == 4 || bits == 8)) return false;
+    if (mode != 0 && !aligned16(packed)) return false;
+    const int LPR = (int)(D / 8), RPP = 256 / LPR;
+    if (axis == VQ_AXIS_TOKEN) {
+        if (group > KT_MAXP * RPP) return false;
+#define VQ_K(L) launch_key_tile<T, M, L>(mode, x, out, BH, S, xs, group, levels, eps, bits, packed, scale, zero, cap, tok0, st)
+        if (LPR == 8) VQ_K(8); else if (LPR == 16) VQ_K(16); else VQ_K(32);
+#undef VQ_K
+        return true;
+    }
+    if (group % 8 != 0 || !pow2(group / 8) || group > D || D % group != 0) return false;
+    if (mode == 2 && (RPP % (32 / bits)) != 0) return false;
+#define VQ_V(L) launch_value_tile<T, M, L>(mode, x, out, BH, S, xs, group, levels, eps, bits, packed, scale, zero, cap, tok0, st)
+    if (LPR == 8) VQ_V(8); else if (LPR == 16) VQ_V(16); else VQ_V(32);
+#undef VQ_V
+    return true;
+}
+
+extern "C" int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int axis,
+                                     int group, int levels, float eps, void *stream) {
+    VQ_REQUIRE(axis == VQ_AXIS_TOKEN || axis == VQ_AXIS_CHANNEL, VQ_ERR_INVALID,
+               "vq_kivi_quant_dequant: axis must be -1 or -2 (VQ_AXIS_CHANNEL / VQ_AXIS_TOKEN), got %d", axis);
+    VQ_REQUIRE(group >= 1, VQ_ERR_INVALID, "vq_kivi_quant_dequant: group_size must be >= 1, got %d", group);
+    VQ_REQUIRE(levels >= 1, VQ_ERR_INVALID, "vq_kivi_quant_dequant: levels must be >= 1, got %d", levels);
+    VQ_REQUIRE(BH >= 0 && S >= 0 && D >= 0, VQ_ERR_INVALID, "vq_kivi_quant_dequant: negative dimension");
+    VQ_REQUIRE(is_float_tag(dtype), VQ_ERR_INVALID, "vq_kivi_quant_dequant: unsupported dtype tag %d", dtype);
+    if (BH * S * D == 0) return VQ_OK;
+    VQ_REQUIRE(x && out, VQ_ERR_INVALID, "vq_kivi_quant_dequant: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    VQ_DISPATCH_FLOAT(dtype, T, {
+        if (!try_tile_path<T, float>(0, axis, x, out, BH, S, D, S * D, group, levels, eps, 0, nullptr, nullptr, nullptr,
+                                     0, 0, st))
+            hipLaunchKernelGGL((kivi_roundtrip_generic_kernel<T>), dim3(grid_for(BH * S * D, 256)), dim3(256), 0, st,
+                               (const T *)x, (T *)out, BH, S, D, axis, group, (float)levels, eps);
+    });
+    VQ_HIP_CHECK_LAUNCH("vq_kivi_quant_dequant");
+    return VQ_OK;
+}
+
+extern "C" int vq_kivi_quant_pack(const void *x, int dtype, int64_t BH, int64_t S, int64_t D, int64_t x_stride_bh,
+                                  int axis, int group, int levels, float eps, int pack_bits, int v_layout,
+                                  void *packed, void *scale, void *zero, int meta_dtype, int64_t cap_tokens,
+                                  int64_t dst_tok0, void *stream) {
+    const char *fn = "vq_kivi_quant_pack";
+    VQ_REQUIRE(axis == VQ_AXIS_TOKEN || axis == VQ_AXIS_CHANNEL, VQ_ERR_INVALID, "%s: bad axis %d", fn, axis);
+    VQ_REQUIRE(group >= 1, VQ_ERR_INVALID, "%s: group_size must be >= 1, got %d", fn, group);
+    VQ_REQUIRE(pack_bits >= 1 && pack_bits <= 8, VQ_ERR_INVALID, "%s: pack_bits must be in 1..8, got %d", fn, pack_bits);
+    VQ_REQUIRE(levels >= 1 && levels <= (1 << pack_bits) - 1, VQ_ERR_INVALID,
+               "%s: levels=%d does not fit pack_bits=%d", fn, levels, pack_bits);
+    VQ_REQUIRE(is_float_tag(dtype), VQ_ERR_INVALID, "%s: unsupported dtype tag %d", fn, dtype);
+    VQ_REQUIRE(meta_dtype == VQ_F32 || meta_dtype == VQ_F16, VQ_ERR_INVALID, "%s: meta dtype must be f32 or f16", fn);
+    VQ_REQUIRE(BH >= 0 && S >= 0 && D >= 1, VQ_ERR_INVALID, "%s: bad dimensions", fn);
+    VQ_REQUIRE(dst_tok0 >= 0 && dst_tok0 + S <= cap_tokens, VQ_ERR_INVALID,
+               "%s: tokens [%lld, %lld) exceed capacity %lld", fn, (long long)dst_tok0, (long long)(dst_tok0 + S),
+               (long long)cap_tokens);
+    VQ_REQUIRE(x_stride_bh >= S * D, VQ_ERR_INVALID, "%s: x_stride_bh too small", fn);
+    const bool tokpacked = axis == VQ_AXIS_CHANNEL && v_layout == VQ_V_TOKEN_PACKED;
+    VQ_REQUIRE(v_layout == VQ_V_CHANNEL_PACKED || v_layout == VQ_V_TOKEN_PACKED, VQ_ERR_INVALID, "%s: bad v_layout", fn);
+    const int per = 32 / pack_bits;
+    if (axis == VQ_AXIS_TOKEN)
+        VQ_REQUIRE(dst_tok0 % group == 0, VQ_ERR_INVALID, "%s: key blocks must start on a group boundary", fn);
+    if (tokpacked)
+        VQ_REQUIRE(dst_tok0 % per == 0 && S % per == 0 && cap_tokens % per == 0, VQ_ERR_INVALID,
+                   "%s: token-packed values need dst_tok0, S and cap_tokens to be multiples of %d", fn, per);
+    if (BH * S == 0) return VQ_OK;
+    VQ_REQUIRE(x && packed && scale && zero, VQ_ERR_INVALID, "%s: null pointer", fn);
+    hipStream_t st = (hipStream_t)stream;
+    const int mode = tokpacked ? 2 : 1;
+    const int64_t n_words = tokpacked ? BH * (S / per) * D : BH * S * cdiv(D, per);
+#define VQ_PACK(T, M)                                                                                              \
+    if (!try_tile_path<T, M>(mode, axis, x, nullptr, BH, S, D, x_stride_bh, group, levels, eps, pack_bits, packed,  \
+                             scale, zero, cap_tokens, dst_tok0, st))                                              \
+        hipLaunchKernelGGL((kivi_pack_generic_kernel<T, M>), dim3(grid_for(n_words, 128)), dim3(128), 0, st,      \
+                           (const T *)x, BH, S, D, x_stride_bh, axis, group, (float)levels, eps, pack_bits,       \
+                           tokpacked ? 1 : 0, (uint32_t *)packed, (M *)scale, (M *)zero, cap_tokens, dst_tok0)
+    VQ_DISPATCH_FLOAT(dtype, T, {
+        if (meta_dtype == VQ_F32) { VQ_PACK(T, float); } else { VQ_PACK(T, f16); }
+    });
+#undef VQ_PACK
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_kivi_dequant(const void *packed, const void *scale, const void *zero, int meta_dtype, int64_t BH,
+                               int64_t S, int64_t D, int axis, int group, int pack_bits, int v_layout,
+                               int64_t cap_tokens, int64_t src_tok0, void *out, int out_dtype, void *stream) {
+    const char *fn = "vq_kivi_dequant";
+    VQ_REQUIRE(axis == VQ_AXIS_TOKEN || axis == VQ_AXIS_CHANNEL, VQ_ERR_INVALID, "%s: bad axis %d", fn, axis);
+    VQ_REQUIRE(group >= 1, VQ_ERR_INVALID, "%s: group_size must be >= 1", fn);
+    VQ_REQUIRE(pack_bits >= 1 && pack_bits <= 8, VQ_ERR_INVALID, "%s: pack_bits must be in 1..8", fn);
+    VQ_REQUIRE(meta_dtype == VQ_F32 || meta_dtype == VQ_F16, VQ_ERR_INVALID, "%s: meta dtype must be f32 or f16", fn);
+    VQ_REQUIRE(is_float_tag(out_dtype), VQ_ERR_INVALID, "%s: unsupported out dtype", fn);
+    VQ_REQUIRE(src_tok0 >= 0 && src_tok0 + S <= cap_tokens, VQ_ERR_INVALID, "%s: token range exceeds capacity", fn);
+    const bool tokpacked = axis == VQ_AXIS_CHANNEL && v_layout == VQ_V_TOKEN_PACKED;
+    if (tokpacked) VQ_REQUIRE(cap_tokens % (32 / pack_bits) == 0, VQ_ERR_INVALID, "%s: capacity not word aligned", fn);
+    if (BH * S * D == 0) return VQ_OK;
+    VQ_REQUIRE(packed && scale && zero && out, VQ_ERR_INVALID, "%s: null pointer", fn);
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(grid_for(BH * S * D, 256));
+    VQ_DISPATCH_FLOAT(out_dtype, O, {
+        if (meta_dtype == VQ_F32)
+            hipLaunchKernelGGL((kivi_dequant_kernel<O, float>), grid, dim3(256), 0, st, (const uint32_t *)packed,
+                               (const float *)scale, (const float *)zero, BH, S, D, axis, group, pack_bits,
+                               tokpacked ? 1 : 0, cap_tokens, src_tok0, (O *)out);
+        else
+            hipLaunchKernelGGL((kivi_dequant_kernel<O, f16>), grid, dim3(256), 0, st, (const uint32_t *)packed,
+                               (const f16 *)scale, (const f16 *)zero, BH, S, D, axis, group, pack_bits,
+                               tokpacked ? 1 : 0, cap_tokens, src_tok0, (O *)out);
+    });
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_pack_words(const uint8_t *idx, int64_t rows, int64_t D, int bits, uint32_t *words, void *stream) {
+    VQ_REQUIRE(bits >= 1 && bits <= 8, VQ_ERR_INVALID, "vq_pack_words: bits must be in 1..8, got %d", bits);
+    VQ_REQUIRE(rows >= 0 && D >= 0, VQ_ERR_INVALID, "vq_pack_words: negative dimension");
+    if (rows * D == 0) return VQ_OK;
+    VQ_REQUIRE(idx && words, VQ_ERR_INVALID, "vq_pack_words: null pointer");
+    hipLaunchKernelGGL(pack_words_kernel, dim3(grid_for(rows * cdiv(D, 32 / bits), 256)), dim3(256), 0,
+                       (hipStream_t)stream, idx, rows, D, bits, words);
+    VQ_HIP_CHECK_LAUNCH("vq_pack_words");
+    return VQ_OK;
+}
+extern "C" int vq_unpack_words(const uint32_t *words, int64_t rows, int64_t D, int bits, uint8_t *idx, void *stream) {
+    VQ_REQUIRE(bits >= 1 && bits <= 8, VQ_ERR_INVALID, "vq_unpack_words: bits must be in 1..8, got %d", bits);
+    VQ_REQUIRE(rows >= 0 && D >= 0, VQ_ERR_INVALID, "vq_unpack_words: negative dimension");
+    if (rows * D == 0) return VQ_OK;
+    VQ_REQUIRE(idx && words, VQ_ERR_INVALID, "vq_unpack_words: null pointer");
+    hipLaunchKernelGGL(unpack_words_kernel, dim3(grid_for(rows * D, 256)), dim3(256), 0, (hipStream_t)stream, words,
+                       rows, D, bits, idx);
+    VQ_HIP_CHECK_LAUNCH("vq_unpack_words");
+    return VQ_OK;
+}
+extern "C" int vq_bit_pack(const uint8_t *idx, int64_t n, int bits, uint8_t *packed, void *stream) {
+    VQ_REQUIRE(bits == 1 || bits == 2 || bits == 4, VQ_ERR_INVALID, "vq_bit_pack: bits must be 1, 2 or 4, got %d", bits);
+    VQ_REQUIRE(n >= 0 && n % (8 / bits) == 0, VQ_ERR_INVALID,
+               "vq_bit_pack: length %lld is not a multiple of %d", (long long)n, 8 / bits);
+    if (n == 0) return VQ_OK;
+    VQ_REQUIRE(idx && packed, VQ_ERR_INVALID, "vq_bit_pack: null pointer");
+    hipLaunchKernelGGL(bit_pack_kernel, dim3(grid_for(n / (8 / bits), 256)), dim3(256), 0, (hipStream_t)stream, idx,
+                       n / (8 / bits), bits, packed);
+    VQ_HIP_CHECK_LAUNCH("vq_bit_pack");
+    return VQ_OK;
+}
+extern "C" int vq_bit_unpack(const uint8_t *packed, int64_t n, int bits, uint8_t *idx, void *stream) {
+    VQ_REQUIRE(bits == 1 || bits == 2 || bits == 4, VQ_ERR_INVALID, "vq_bit_unpack: bits must be 1, 2 or 4, got %d", bits);
+    VQ_REQUIRE(n >= 0, VQ_ERR_INVALID, "vq_bit_unpack: negative length");
+    if (n == 0) return VQ_OK;
+    VQ_REQUIRE(idx && packed, VQ_ERR_INVALID, "vq_bit_unpack: null pointer");
+    hipLaunchKernelGGL(bit_unpack_kernel, dim3(grid_for(n, 256)), dim3(256), 0, (hipStream_t)stream, packed, n, bits, idx);
+    VQ_HIP_CHECK_LAUNCH("vq_bit_unpack");
+    return VQ_OK;
+}

@@ -1,0 +1,552 @@
+"""Kernel entry points on ``torch`` ROCm tensors.
+
+Same names, argument meaning and error behaviour as the functions the reference
+re-exports from ``veloxquant_mlx/metal/kernels.py:111-146`` for the KIVI /
+VecInfer hot path; each forwards to the C ABI in ``libveloxquant_hip.so`` on the
+current torch stream.  Inputs must live on a ROCm device; nothing here computes
+on the CPU.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+from ._lib import (VQ_AXIS_CHANNEL, VQ_AXIS_TOKEN, VQ_BF16, VQ_F16, VQ_F32, VQ_I32, VQ_U8,
+                   VQ_V_CHANNEL_PACKED, VQ_V_TOKEN_PACKED, AttendArgs)
+
+_FLOAT_TAG = {torch.float16: VQ_F16, torch.bfloat16: VQ_BF16, torch.float32: VQ_F32}
+_V_LAYOUT = {"channel": VQ_V_CHANNEL_PACKED, "token": VQ_V_TOKEN_PACKED}
+
+# Largest GQA ratio the reference's fused decode accepts (_scalar_attend.py:326).
+_MAX_HEADS_PER_KV = 16
+
+
+def hip_available() -> bool:
+    """True when the kernel library loads and a ROCm device is visible (the
+    counterpart of ``metal_available``, veloxquant_mlx/metal/__init__.py:26-31)."""
+    return _lib.library_present() and torch.cuda.is_available()
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _need_gpu(name: str, *tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise RuntimeError(f"{name}: tensors must live on a ROCm device (got {t.device}); "
+                               "there is no CPU path")
+
+
+def _ftag(name: str, t: torch.Tensor) -> int:
+    if t.dtype not in _FLOAT_TAG:
+        raise ValueError(f"{name}: unsupported dtype {t.dtype}; expected one of "
+                         f"{sorted(str(d) for d in _FLOAT_TAG)}")
+    return _FLOAT_TAG[t.dtype]
+
+
+def _axis_tag(name: str, axis: int) -> int:
+    if axis not in (-1, -2):
+        raise ValueError(f"{name}: axis must be -1 or -2, got {axis}")
+    return VQ_AXIS_TOKEN if axis == -2 else VQ_AXIS_CHANNEL
+
+
+# ---------------------------------------------------------------------------
+# KIVI group quantisation
+# ---------------------------------------------------------------------------
+
+def kivi_group_quant_dequant(x: torch.Tensor, axis: int, group_size: int, levels: int,
+                             eps: float = 1e-8) -> torch.Tensor:
+    """Round-trip ``x [..., S, D]`` through KIVI asymmetric group quantisation.
+
+    Drop-in for ``kivi_group_quant_dequant`` (veloxquant_mlx/metal/_kivi_quant.py:138-207):
+    ``axis=-2`` per-channel (keys), ``axis=-1`` per-token (values); bit-identical
+    to ``KIVIKVCache._quant_dequant_along`` (veloxquant_mlx/cache/kivi_cache.py:151-201).
+    """
+    name = "kivi_group_quant_dequant"
+    ax = _axis_tag(name, axis)
+    if x.ndim < 2:
+        raise ValueError(f"{name}: x must be at least 2D, got {tuple(x.shape)}")
+    if group_size < 1:
+        raise ValueError(f"{name}: group_size must be >= 1, got {group_size}")
+    if levels < 1:
+        raise ValueError(f"{name}: levels must be >= 1, got {levels}")
+    tag = _ftag(name, x)
+    if x.numel() == 0:
+        return x
+    _need_gpu(name, x)
+    S, D = x.shape[-2], x.shape[-1]
+    flat = x.contiguous()
+    out = torch.empty_like(flat)
+    rc = _lib.load().vq_kivi_quant_dequant(flat.data_ptr(), out.data_ptr(), tag, flat.numel() // (S * D), S, D,
+                                           ax, int(group_size), int(levels), float(eps), _stream(x))
+    _lib.check(rc)
+    return out.view(x.shape)
+
+
+def kivi_quant_pack(x: torch.Tensor, axis: int, group_size: int, bits: int, *, levels: int | None = None,
+                    eps: float = 1e-8, meta_dtype: torch.dtype = torch.float16, v_layout: str = "channel",
+                    out: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
+                    dst_tok0: int = 0):
+    """Quantise ``x [B, H, S, D]`` and bit-pack the codes.
+
+    Codes are those of ``_quant_keys`` / ``_quant_values``
+    (benchmark_scripts/benchmark_real_model_scalar_attend.py:115-153); words are
+    the ``_pack_indices`` image (veloxquant_mlx/cache/turboquant_rvq_cache.py:82-106).
+    Returns ``(packed uint32-as-int32, scale, zero)``:
+
+    * ``axis=-2``: packed ``[B,H,S,W]``, scale/zero ``[B,H,ceil(S/g),D]``
+    * ``axis=-1``, ``v_layout="channel"``: packed ``[B,H,S,W]``, scale/zero ``[B,H,S,GV]``
+    * ``axis=-1``, ``v_layout="token"``: packed ``[B,H,S/per,D]``, scale/zero ``[B,H,GV,S]``
+
+    With ``out=(packed, scale, zero)`` the results are written at token offset
+    ``dst_tok0`` of pre-allocated cache buffers whose token capacity is read
+    from ``packed`` (``x`` may then be a slice with a larger head stride).
+    """
+    name = "kivi_quant_pack"
+    ax = _axis_tag(name, axis)
+    if x.ndim != 4:
+        raise ValueError(f"{name}: x must be 4D [B,H,S,D], got {tuple(x.shape)}")
+    if v_layout not in _V_LAYOUT:
+        raise ValueError(f"{name}: v_layout must be 'channel' or 'token', got {v_layout!r}")
+    if not (1 <= bits <= 8):
+        raise ValueError(f"{name}: bits must be in 1..8, got {bits}")
+    if meta_dtype not in (torch.float16, torch.float32):
+        raise ValueError(f"{name}: meta_dtype must be float16 or float32, got {meta_dtype}")
+    tag = _ftag(name, x)
+    _need_gpu(name, x)
+    B, H, S, D = x.shape
+    per = 32 // bits
+    levels = (1 << bits) - 1 if levels is None else int(levels)
+    tokpacked = ax == VQ_AXIS_CHANNEL and v_layout == "token"
+    # accept a [B,H,S,D] view whose rows are dense but whose head stride is larger
+    xs = x.stride(1) if H > 1 else (x.stride(0) if B > 1 else S * D)
+    if x.stride(-1) != 1 or x.stride(-2) != D or xs < S * D or (B > 1 and H > 1 and x.stride(0) != H * xs):
+        x = x.contiguous()
+        xs = S * D
+    W = -(-D // per)
+    GV = -(-D // group_size)
+    if out is None:
+        cap = S
+        if tokpacked:
+            packed = torch.empty((B, H, -(-S // per), D), dtype=torch.int32, device=x.device)
+            mshape = (B, H, GV, S)
+        else:
+            packed = torch.empty((B, H, S, W), dtype=torch.int32, device=x.device)
+            mshape = (B, H, -(-S // group_size), D) if ax == VQ_AXIS_TOKEN else (B, H, S, GV)
+        scale = torch.empty(mshape, dtype=meta_dtype, device=x.device)
+        zero = torch.empty(mshape, dtype=meta_dtype, device=x.device)
+    else:
+        packed, scale, zero = out
+        cap = packed.shape[2] * per if tokpacked else packed.shape[2]
+        if scale.dtype != meta_dtype or zero.dtype != meta_dtype:
+            raise ValueError(f"{name}: out scale/zero dtype must equal meta_dtype")
+        for t in (packed, scale, zero):
+            if not t.is_contiguous():
+                raise ValueError(f"{name}: out buffers must be contiguous")
+    rc = _lib.load().vq_kivi_quant_pack(
+        x.data_ptr(), tag, B * H, S, D, xs, ax, int(group_size), levels, float(eps), int(bits),
+        _V_LAYOUT[v_layout], packed.data_ptr(), scale.data_ptr(), zero.data_ptr(),
+        VQ_F16 if meta_dtype == torch.float16 else VQ_F32, cap, int(dst_tok0), _stream(x))
+    _lib.check(rc)
+    return packed, scale, zero
+
+
+def kivi_quant_codes(x: torch.Tensor, axis: int, group_size: int, levels: int, eps: float = 1e-8):
+    """``(codes uint8, scale f32, zero f32)`` exactly as the reference's split
+    form returns them (test_scalar_attend.py:51-82)."""
+    packed, scale, zero = kivi_quant_pack(x, axis, group_size, 8, levels=levels, eps=eps,
+                                          meta_dtype=torch.float32)
+    B, H, S, D = x.shape
+    codes = packed.view(torch.uint8).view(B, H, S, -1)[..., :D]
+    return codes, scale, zero
+
+
+def kivi_dequant(packed: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, axis: int, group_size: int,
+                 bits: int, S: int, D: int, *, v_layout: str = "channel", out_dtype: torch.dtype = torch.float16,
+                 src_tok0: int = 0) -> torch.Tensor:
+    """Rebuild ``[B,H,S,D]`` from packed codes (``code*scale+zero``, two roundings)."""
+    name = "kivi_dequant"
+    ax = _axis_tag(name, axis)
+    _need_gpu(name, packed, scale, zero)
+    if out_dtype not in _FLOAT_TAG:
+        raise ValueError(f"{name}: unsupported out dtype {out_dtype}")
+    B, H = packed.shape[0], packed.shape[1]
+    per = 32 // bits
+    tokpacked = ax == VQ_AXIS_CHANNEL and v_layout == "token"
+    cap = packed.shape[2] * per if tokpacked else packed.shape[2]
+    out = torch.empty((B, H, S, D), dtype=out_dtype, device=packed.device)
+    rc = _lib.load().vq_kivi_dequant(
+        packed.data_ptr(), scale.data_ptr(), zero.data_ptr(),
+        VQ_F16 if scale.dtype == torch.float16 else VQ_F32, B * H, S, D, ax, int(group_size), int(bits),
+        _V_LAYOUT[v_layout], cap, int(src_tok0), out.data_ptr(), _FLOAT_TAG[out_dtype], _stream(packed))
+    _lib.check(rc)
+    return out
+
+
+def scalar_decode_once(codes: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, group_size: int,
+                       mode: str) -> torch.Tensor:
+    """uint8 codes + fp32 scale/zero -> fp16 (veloxquant_mlx/metal/_scalar_attend.py:650-699)."""
+    if mode not in ("K", "V"):
+        raise ValueError(f"scalar_decode_once: mode must be 'K' or 'V', got {mode!r}")
+    if codes.ndim != 4:
+        raise ValueError(f"scalar_decode_once: codes must be 4D, got {tuple(codes.shape)}")
+    B, H, S, D = codes.shape
+    if D % 4:
+        raise ValueError("scalar_decode_once: D must be a multiple of 4")
+    words = codes.to(torch.uint8).contiguous().view(torch.int32)
+    return kivi_dequant(words, scale.float().contiguous(), zero.float().contiguous(),
+                        -2 if mode == "K" else -1, group_size, 8, S, D, out_dtype=torch.float16)
+
+
+# ---------------------------------------------------------------------------
+# bit packing
+# ---------------------------------------------------------------------------
+
+def pack_indices(idx: torch.Tensor, bits: int) -> torch.Tensor:
+    """``_pack_indices`` (veloxquant_mlx/cache/turboquant_rvq_cache.py:82-106): trailing
+    axis -> uint32 words (returned as int32 storage), LSB first, zero padded."""
+    if not (1 <= bits <= 8):
+        raise ValueError(f"pack_indices: bits must be in 1..8, got {bits}")
+    _need_gpu("pack_indices", idx)
+    d = idx.shape[-1]
+    per = 32 // bits
+    flat = idx.to(torch.uint8).contiguous()
+    out = torch.empty(idx.shape[:-1] + (-(-d // per),), dtype=torch.int32, device=idx.device)
+    rows = flat.numel() // d if d else 0
+    _lib.check(_lib.load().vq_pack_words(flat.data_ptr(), rows, d, bits, out.data_ptr(), _stream(idx)))
+    return out
+
+
+def unpack_indices(packed: torch.Tensor, bits: int, d: int) -> torch.Tensor:
+    """``_unpack_indices`` (turboquant_rvq_cache.py:109-126)."""
+    if not (1 <= bits <= 8):
+        raise ValueError(f"unpack_indices: bits must be in 1..8, got {bits}")
+    _need_gpu("unpack_indices", packed)
+    per = 32 // bits
+    if packed.shape[-1] != -(-d // per):
+        raise ValueError(f"unpack_indices: {packed.shape[-1]} words cannot hold d={d} at bits={bits}")
+    flat = packed.contiguous()
+    out = torch.empty(packed.shape[:-1] + (d,), dtype=torch.uint8, device=packed.device)
+    rows = out.numel() // d if d else 0
+    _lib.check(_lib.load().vq_unpack_words(flat.data_ptr(), rows, d, bits, out.data_ptr(), _stream(packed)))
+    return out
+
+
+def turboquant_bit_pack(indices: torch.Tensor, b: int) -> torch.Tensor:
+    """``turboquant_bit_pack`` (veloxquant_mlx/metal/_bit_packing.py:87-118)."""
+    if b not in (1, 2, 4):
+        raise ValueError(f"turboquant_bit_pack: b must be 1, 2, or 4, got {b}")
+    N = indices.numel()
+    if N % (8 // b) != 0:
+        raise ValueError(f"turboquant_bit_pack: N={N} not divisible by {8 // b} (= 8/b)")
+    _need_gpu("turboquant_bit_pack", indices)
+    flat = indices.reshape(-1).to(torch.uint8).contiguous()
+    out = torch.empty(N * b // 8, dtype=torch.uint8, device=indices.device)
+    _lib.check(_lib.load().vq_bit_pack(flat.data_ptr(), N, b, out.data_ptr(), _stream(indices)))
+    return out
+
+
+def turboquant_bit_unpack(packed: torch.Tensor, N: int, b: int) -> torch.Tensor:
+    """``turboquant_bit_unpack`` (veloxquant_mlx/metal/_bit_packing.py:121-148)."""
+    if b not in (1, 2, 4):
+        raise ValueError(f"turboquant_bit_unpack: b must be 1, 2, or 4, got {b}")
+    if N < 0:
+        raise ValueError(f"turboquant_bit_unpack: N must be >= 0, got {N}")
+    need = -(-N * b // 8)
+    if packed.numel() < need:
+        raise ValueError(f"turboquant_bit_unpack: packed has {packed.numel()} byte(s) but N={N} "
+                         f"at b={b} needs {need}")
+    _need_gpu("turboquant_bit_unpack", packed)
+    flat = packed.reshape(-1).to(torch.uint8).contiguous()
+    out = torch.empty(N, dtype=torch.uint8, device=packed.device)
+    _lib.check(_lib.load().vq_bit_unpack(flat.data_ptr(), N, b, out.data_ptr(), _stream(packed)))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# VecInfer product VQ
+# ---------------------------------------------------------------------------
+
+def vecinfer_quantize_metal(x: torch.Tensor, codebook: torch.Tensor, sub_dim: int, *,
+                            index_dtype: torch.dtype = torch.int32) -> torch.Tensor:
+    """Nearest-centroid indices ``[..., D // sub_dim]``; drop-in for ``quantize_vq``
+    (veloxquant_mlx/allocators/vecinfer.py:281-318) and ``vecinfer_quantize_metal``
+    (veloxquant_mlx/metal/_vecinfer.py:181-222).  ``index_dtype=torch.uint8`` stores
+    one byte per index (codebooks of at most 256 centroids)."""
+    name = "vecinfer_quantize_metal"
+    D = x.shape[-1]
+    if D % sub_dim != 0:
+        raise ValueError(f"{name}: D={D} not divisible by sub_dim={sub_dim}")
+    if codebook.ndim != 2 or codebook.shape[1] != sub_dim:
+        raise ValueError(f"{name}: codebook must be [n_centroids, {sub_dim}], got {tuple(codebook.shape)}")
+    if index_dtype not in (torch.int32, torch.uint8):
+        raise ValueError(f"{name}: index_dtype must be int32 or uint8")
+    _need_gpu(name, x, codebook)
+    if x.dtype not in _FLOAT_TAG:
+        x = x.float()
+    if codebook.dtype not in _FLOAT_TAG:
+        codebook = codebook.float()
+    xf, cb = x.contiguous(), codebook.contiguous()
+    n_sub = D // sub_dim
+    out = torch.empty(x.shape[:-1] + (n_sub,), dtype=index_dtype, device=x.device)
+    rc = _lib.load().vq_vecinfer_assign(xf.data_ptr(), _FLOAT_TAG[xf.dtype], out.numel(), cb.data_ptr(),
+                                        _FLOAT_TAG[cb.dtype], cb.shape[0], sub_dim, out.data_ptr(),
+                                        VQ_U8 if index_dtype == torch.uint8 else VQ_I32, _stream(x))
+    _lib.check(rc)
+    return out
+
+
+def vecinfer_dequant_metal(indices: torch.Tensor, codebook: torch.Tensor,
+                           out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Centroid gather ``[..., n_sub] -> [..., n_sub*sub_dim]``; drop-in for
+    ``dequantize_vq`` (allocators/vecinfer.py:321-335) / ``vecinfer_dequant_metal``
+    (metal/_vecinfer.py:144-178)."""
+    name = "vecinfer_dequant_metal"
+    if codebook.ndim != 2:
+        raise ValueError(f"{name}: codebook must be 2D, got {tuple(codebook.shape)}")
+    _need_gpu(name, indices, codebook)
+    if out_dtype is None:
+        out_dtype = codebook.dtype
+    if out_dtype not in _FLOAT_TAG:
+        raise ValueError(f"{name}: unsupported out dtype {out_dtype}")
+    if codebook.dtype not in _FLOAT_TAG:
+        codebook = codebook.float()
+    if indices.dtype not in (torch.int32, torch.uint8):
+        indices = indices.to(torch.int32)
+    idx, cb = indices.contiguous(), codebook.contiguous()
+    sub = cb.shape[1]
+    out = torch.empty(indices.shape[:-1] + (indices.shape[-1] * sub,), dtype=out_dtype, device=indices.device)
+    rc = _lib.load().vq_vecinfer_dequant(idx.data_ptr(), VQ_U8 if idx.dtype == torch.uint8 else VQ_I32,
+                                         idx.numel(), cb.data_ptr(), _FLOAT_TAG[cb.dtype], cb.shape[0], sub,
+                                         out.data_ptr(), _FLOAT_TAG[out_dtype], _stream(indices))
+    _lib.check(rc)
+    return out
+
+
+vecinfer_quantize_hip = vecinfer_quantize_metal
+vecinfer_dequant_hip = vecinfer_dequant_metal
+
+
+# ---------------------------------------------------------------------------
+# attention over a packed cache
+# ---------------------------------------------------------------------------
+
+_workspaces: dict[tuple, torch.Tensor] = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=None, v_packed=None,
+                       v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
+                       v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
+                       scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
+                       num_splits: int = 0) -> torch.Tensor:
+    """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
+
+    q ``[B,Hq,Sq,D]``; packed buffers as :func:`kivi_quant_pack` lays them out
+    with capacity read from their shapes, of which the first ``n_packed`` tokens
+    are live; tails ``[B,Hkv,tail_cap,D]`` with ``n_tail`` live tokens.  GQA by
+    repeat-interleave.  ``causal`` aligns queries to the end of the slots."""
+    name = "kivi_packed_attend"
+    if q.ndim != 4:
+        raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
+    _need_gpu(name, q)
+    B, Hq, Sq, D = q.shape
+    q = q.contiguous()
+    if out_dtype is None:
+        out_dtype = q.dtype
+    a = AttendArgs()
+    out = torch.empty((B, Hq, Sq, D), dtype=out_dtype, device=q.device)
+    a.q, a.out = q.data_ptr(), out.data_ptr()
+    a.q_dtype, a.out_dtype = _ftag(name, q), _FLOAT_TAG[out_dtype]
+    Hkv = None
+    keep = [q, out]
+    if n_packed > 0:
+        for t in (k_packed, k_scale, k_zero, v_packed, v_scale, v_zero):
+            if t is None or not t.is_contiguous():
+                raise ValueError(f"{name}: packed-cache tensors must be given and contiguous")
+        _need_gpu(name, k_packed, v_packed, k_scale, k_zero, v_scale, v_zero)
+        Hkv = k_packed.shape[1]
+        per = 32 // bits
+        a.k_packed, a.k_scale, a.k_zero = k_packed.data_ptr(), k_scale.data_ptr(), k_zero.data_ptr()
+        a.v_packed, a.v_scale, a.v_zero = v_packed.data_ptr(), v_scale.data_ptr(), v_zero.data_ptr()
+        a.pack_bits, a.group = int(bits), int(group_size)
+        if k_scale.dtype not in (torch.float16, torch.float32) or any(
+                t.dtype != k_scale.dtype for t in (k_zero, v_scale, v_zero)):
+            raise ValueError(f"{name}: scale/zero must share one dtype, float16 or float32")
+        a.meta_dtype = VQ_F16 if k_scale.dtype == torch.float16 else VQ_F32
+        a.v_layout = _V_LAYOUT[v_layout]
+        a.cap_tokens = k_packed.shape[2]
+        vcap = v_packed.shape[2] * per if v_layout == "token" else v_packed.shape[2]
+        if vcap != a.cap_tokens:
+            raise ValueError(f"{name}: key capacity {a.cap_tokens} != value capacity {vcap}")
+        keep += [k_packed, k_scale, k_zero, v_packed, v_scale, v_zero]
+    if n_tail > 0:
+        if k_tail is None or v_tail is None:
+            raise ValueError(f"{name}: n_tail > 0 needs k_tail and v_tail")
+        _need_gpu(name, k_tail, v_tail)
+        if k_tail.dtype != v_tail.dtype:
+            raise ValueError(f"{name}: k_tail and v_tail dtypes differ")
+        if not (k_tail.is_contiguous() and v_tail.is_contiguous()):
+            raise ValueError(f"{name}: tail tensors must be contiguous")
+        if Hkv is not None and k_tail.shape[1] != Hkv:
+            raise ValueError(f"{name}: tail has {k_tail.shape[1]} kv heads, packed cache has {Hkv}")
+        Hkv = k_tail.shape[1]
+        a.k_tail, a.v_tail = k_tail.data_ptr(), v_tail.data_ptr()
+        a.tail_dtype = _ftag(name, k_tail)
+        a.tail_cap = k_tail.shape[2]
+        keep += [k_tail, v_tail]
+    if Hkv is None:
+        raise ValueError(f"{name}: no key/value slots to attend to")
+    a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
+    a.n_packed, a.n_tail = int(n_packed), int(n_tail)
+    a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
+    lib = _lib.load()
+    need = lib.vq_kivi_attend_workspace(a)
+    ws = _workspace(q.device, need)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.stream = _stream(q)
+    _lib.check(lib.vq_kivi_attend(a))
+    return out
+
+
+def _check_fused_args(name, q, k_codes, v_codes, ndim):
+    if q.ndim != ndim:
+        raise ValueError(f"{name}: q must be {ndim}D, got {tuple(q.shape)}")
+    if k_codes.ndim != ndim or v_codes.ndim != ndim:
+        raise ValueError(f"{name}: k_codes and v_codes must be {ndim}D, "
+                         f"got k_codes={tuple(k_codes.shape)}, v_codes={tuple(v_codes.shape)}")
+
+
+def scalar_fused_decode_attend(q, k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, group_size: int,
+                               scale: float, nsg: int | None = None) -> torch.Tensor:
+    """Fused group-affine decode + attention over uint8 codes and fp32 scale/zero;
+    drop-in for ``scalar_fused_decode_attend``
+    (veloxquant_mlx/metal/_scalar_attend.py:370-493).  ``nsg`` (SIMD groups per
+    threadgroup on Apple GPUs) is validated for range and otherwise unused: the
+    token axis is split across workgroups instead."""
+    name = "scalar_fused_decode_attend"
+    _check_fused_args(name, q, k_codes, v_codes, 4)
+    B, H, S_q, D = q.shape
+    if D > 256:
+        raise ValueError(f"{name}: D={D} must be <= 256")
+    if nsg is not None and not (1 <= nsg <= 32):
+        raise ValueError(f"{name}: nsg={nsg} must be in 1..32")
+    Bk, H_kv, S_kv, Dk = k_codes.shape
+    if Bk != B:
+        raise ValueError(f"{name}: batch mismatch: q B={B} vs k_codes B={Bk}")
+    if Dk != D:
+        raise ValueError(f"{name}: head_dim mismatch: q D={D} vs k_codes D={Dk}")
+    if v_codes.shape[1] != H_kv:
+        raise ValueError(f"{name}: k_codes H_kv={H_kv} vs v_codes H_kv={v_codes.shape[1]} mismatch")
+    if H % H_kv != 0:
+        raise ValueError(f"{name}: H_q={H} must be a multiple of H_kv={H_kv} (k_codes.shape[1]) "
+                         "for GQA head-packing")
+    if H // H_kv > _MAX_HEADS_PER_KV:
+        raise ValueError(f"{name}: heads_per_kv={H // H_kv} exceeds the supported maximum of {_MAX_HEADS_PER_KV}")
+    if D % 4:
+        raise ValueError(f"{name}: D={D} must be a multiple of 4")
+    _need_gpu(name, q, k_codes, v_codes)
+    kw = k_codes.to(torch.uint8).contiguous().view(torch.int32)
+    vw = v_codes.to(torch.uint8).contiguous().view(torch.int32)
+    return kivi_packed_attend(
+        q.to(torch.float16), k_packed=kw, k_scale=k_scale.float().contiguous(), k_zero=k_zero.float().contiguous(),
+        v_packed=vw, v_scale=v_scale.float().contiguous(), v_zero=v_zero.float().contiguous(),
+        n_packed=S_kv, bits=8, group_size=group_size, scale=scale, causal=False, out_dtype=torch.float16)
+
+
+def scalar_fused_decode_attend_batched(q, k_codes, k_scale, k_zero, v_codes, v_scale, v_zero, group_size: int,
+                                       scale: float, nsg: int | None = None) -> torch.Tensor:
+    """Layer-batched form: every tensor carries a leading ``NL`` axis, which folds
+    into the batch axis (veloxquant_mlx/metal/_scalar_attend.py:496-647)."""
+    name = "scalar_fused_decode_attend_batched"
+    if q.ndim != 5:
+        raise ValueError(f"{name}: q must be 5D [NL,B,H,S_q,D], got {tuple(q.shape)}")
+    _check_fused_args(name, q, k_codes, v_codes, 5)
+    NL, B = q.shape[0], q.shape[1]
+    if NL < 1:
+        raise ValueError(f"{name}: NL={NL} must be >= 1")
+    if k_codes.shape[0] != NL:
+        raise ValueError(f"{name}: NL mismatch: q NL={NL} vs k_codes NL={k_codes.shape[0]}")
+    if k_codes.shape[1] != B:
+        raise ValueError(f"{name}: batch mismatch: q B={B} vs k_codes B={k_codes.shape[1]}")
+    if v_codes.shape != k_codes.shape:
+        raise ValueError(f"{name}: k_codes shape={tuple(k_codes.shape)} vs v_codes shape={tuple(v_codes.shape)} mismatch")
+    H_kv = k_codes.shape[2]
+    for nm, arr in (("k_scale", k_scale), ("k_zero", k_zero), ("v_scale", v_scale), ("v_zero", v_zero)):
+        if arr.ndim != 5 or arr.shape[0] != NL or arr.shape[1] != B or arr.shape[2] != H_kv:
+            raise ValueError(f"{name}: {nm} shape={tuple(arr.shape)} must be 5D with leading "
+                             f"[NL={NL}, B={B}, H_kv={H_kv}, ...]")
+    fold = lambda t: t.reshape((NL * B,) + tuple(t.shape[2:]))
+    out = scalar_fused_decode_attend(fold(q), fold(k_codes), fold(k_scale), fold(k_zero), fold(v_codes),
+                                     fold(v_scale), fold(v_zero), group_size, scale, nsg)
+    return out.view((NL, B) + tuple(out.shape[1:]))
+
+
+def scalar_predecoded_attend(q, k_hat, v_hat, scale: float, nsg: int | None = None) -> torch.Tensor:
+    """Decode attention over already reconstructed fp16 K/V
+    (veloxquant_mlx/metal/_scalar_attend.py:702-779)."""
+    name = "scalar_predecoded_attend"
+    if q.ndim != 4:
+        raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
+    if k_hat.ndim != 4 or v_hat.ndim != 4:
+        raise ValueError(f"{name}: k_hat and v_hat must be 4D, got k_hat={tuple(k_hat.shape)}, v_hat={tuple(v_hat.shape)}")
+    B, H, S_q, D = q.shape
+    if D > 256:
+        raise ValueError(f"{name}: D={D} must be <= 256")
+    if nsg is not None and not (1 <= nsg <= 32):
+        raise ValueError(f"{name}: nsg={nsg} must be in 1..32")
+    if k_hat.shape[0] != B:
+        raise ValueError(f"{name}: batch mismatch: q B={B} vs k_hat B={k_hat.shape[0]}")
+    if k_hat.shape[3] != D:
+        raise ValueError(f"{name}: head_dim mismatch: q D={D} vs k_hat D={k_hat.shape[3]}")
+    if v_hat.shape != k_hat.shape:
+        raise ValueError(f"{name}: k_hat shape={tuple(k_hat.shape)} vs v_hat shape={tuple(v_hat.shape)} mismatch")
+    if H % k_hat.shape[1] != 0:
+        raise ValueError(f"{name}: H_q={H} must be a multiple of H_kv={k_hat.shape[1]} (k_hat.shape[1])")
+    return kivi_packed_attend(q.to(torch.float16), k_tail=k_hat.to(torch.float16).contiguous(),
+                              v_tail=v_hat.to(torch.float16).contiguous(), n_tail=k_hat.shape[2], scale=scale,
+                              causal=False, out_dtype=torch.float16)
+
+
+def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
+    """Causal, tail-aligned attention over plain fp16 K/V
+    (veloxquant_mlx/metal/_flash_prefill.py:171-237); GQA is accepted as well."""
+    name = "flash_prefill_attend"
+    if q.ndim != 4:
+        raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
+    B, H, S_q, D = q.shape
+    if D % 8 != 0:
+        raise ValueError(f"{name}: D={D} must be divisible by 8")
+    if k.ndim != 4 or k.shape[0] != B or k.shape[3] != D or H % k.shape[1] != 0:
+        raise ValueError(f"{name}: k must be [B, H, S_kv, {D}], got {tuple(k.shape)}")
+    S_kv = k.shape[2]
+    if tuple(v.shape) != tuple(k.shape):
+        raise ValueError(f"{name}: v must be {tuple(k.shape)}, got {tuple(v.shape)}")
+    if S_q > S_kv:
+        raise ValueError(f"{name}: S_q={S_q} exceeds S_kv={S_kv}; queries align to the tail of the KV cache, "
+                         "so every query needs a slot to attend to")
+    s = float(scale.reshape(-1)[0].item()) if isinstance(scale, torch.Tensor) else float(scale)
+    return kivi_packed_attend(q.to(torch.float16), k_tail=k.to(torch.float16).contiguous(),
+                              v_tail=v.to(torch.float16).contiguous(), n_tail=S_kv, scale=s, causal=True,
+                              out_dtype=torch.float16)
+
+
+__all__ = [
+    "hip_available", "kivi_group_quant_dequant", "kivi_quant_pack", "kivi_quant_codes", "kivi_dequant",
+    "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
+    "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
+    "kivi_packed_attend", "scalar_fused_decode_attend", "scalar_fused_decode_attend_batched",
+    "scalar_predecoded_attend", "flash_prefill_attend",
+]
