@@ -48,6 +48,12 @@ def _ftag(name: str, t: torch.Tensor) -> int:
     return _FLOAT_TAG[t.dtype]
 
 
+def _bytes_as_words(codes: torch.Tensor) -> torch.Tensor:
+    """uint8 ``[..., D]`` (D % 4 == 0) reinterpreted as int32 words ``[..., D/4]``."""
+    c = codes.to(torch.uint8).contiguous()
+    return c.reshape(-1).view(torch.int32).view(c.shape[:-1] + (c.shape[-1] // 4,))
+
+
 def _axis_tag(name: str, axis: int) -> int:
     if axis not in (-1, -2):
         raise ValueError(f"{name}: axis must be -1 or -2, got {axis}")
@@ -161,7 +167,7 @@ def kivi_quant_codes(x: torch.Tensor, axis: int, group_size: int, levels: int, e
     packed, scale, zero = kivi_quant_pack(x, axis, group_size, 8, levels=levels, eps=eps,
                                           meta_dtype=torch.float32)
     B, H, S, D = x.shape
-    codes = packed.view(torch.uint8).view(B, H, S, -1)[..., :D]
+    codes = packed.reshape(-1).view(torch.uint8).view(B, H, S, -1)[..., :D]
     return codes, scale, zero
 
 
@@ -197,7 +203,7 @@ def scalar_decode_once(codes: torch.Tensor, scale: torch.Tensor, zero: torch.Ten
     B, H, S, D = codes.shape
     if D % 4:
         raise ValueError("scalar_decode_once: D must be a multiple of 4")
-    words = codes.to(torch.uint8).contiguous().view(torch.int32)
+    words = _bytes_as_words(codes)
     return kivi_dequant(words, scale.float().contiguous(), zero.float().contiguous(),
                         -2 if mode == "K" else -1, group_size, 8, S, D, out_dtype=torch.float16)
 
@@ -458,8 +464,8 @@ def scalar_fused_decode_attend(q, k_codes, k_scale, k_zero, v_codes, v_scale, v_
     if D % 4:
         raise ValueError(f"{name}: D={D} must be a multiple of 4")
     _need_gpu(name, q, k_codes, v_codes)
-    kw = k_codes.to(torch.uint8).contiguous().view(torch.int32)
-    vw = v_codes.to(torch.uint8).contiguous().view(torch.int32)
+    kw = _bytes_as_words(k_codes)
+    vw = _bytes_as_words(v_codes)
     return kivi_packed_attend(
         q.to(torch.float16), k_packed=kw, k_scale=k_scale.float().contiguous(), k_zero=k_zero.float().contiguous(),
         v_packed=vw, v_scale=v_scale.float().contiguous(), v_zero=v_zero.float().contiguous(),
