@@ -1,0 +1,256 @@
+"""Cache classes on the GPU against the oracle's cache model.
+
+KIVI cases restate veloxquant_mlx/tests/cache/test_kivi_cache.py:60-221 and
+veloxquant_mlx/tests/metal/test_kivi_quant.py:200-235; VecInfer cases restate
+veloxquant_mlx/tests/cache/test_vecinfer_memory_bound_state.py:72-146."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import attend as oa, kivi as ok, vecinfer as ov
+from tests._gpu import gpu, host, outlier_kv, require_gpu, to_dev
+from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+from veloxquant_mlx_amd.quantizers import KIVIQuantizer
+
+pytestmark = gpu
+
+
+def _kv(B, H, S, D, seed):
+    rng = np.random.default_rng(seed)
+    return (rng.standard_normal((B, H, S, D)).astype(np.float16),
+            rng.standard_normal((B, H, S, D)).astype(np.float16))
+
+
+def _make(**kw):
+    cfg = dict(method="kivi", head_dim=128, bit_width_inlier=2, kivi_group_size=32, residual_length=128)
+    cfg.update(kw)
+    return KVCacheFactory.create(KVCacheConfig(**cfg))
+
+
+def test_residual_window_passthrough():
+    require_gpu()
+    c = _make(residual_length=64)
+    k, v = _kv(1, 2, 32, 128, 1)
+    ko, vo = c.update_and_fetch(to_dev(k), to_dev(v))
+    assert np.array_equal(host(ko), k) and np.array_equal(host(vo), v) and c.compressed_key_bytes == 0
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_prefill_plus_decode_matches_cache_model_bit_for_bit(fused):
+    require_gpu()
+    c = _make(residual_length=32, fused_sdpa=fused)
+    m = ok.KiviCacheModel(2, 32, 32)
+    rng = np.random.default_rng(3)
+    k = rng.standard_normal((1, 8, 200, 128)).astype(np.float16)
+    v = rng.standard_normal((1, 8, 200, 128)).astype(np.float16)
+    ko, vo = c.update_and_fetch(to_dev(k), to_dev(v))
+    mk, mv = m.update_and_fetch(k, v)
+    for _ in range(40):
+        k1 = rng.standard_normal((1, 8, 1, 128)).astype(np.float16)
+        v1 = rng.standard_normal((1, 8, 1, 128)).astype(np.float16)
+        ko, vo = c.update_and_fetch(to_dev(k1), to_dev(v1))
+        mk, mv = m.update_and_fetch(k1, v1)
+    assert np.array_equal(host(ko), mk) and np.array_equal(host(vo), mv)
+    assert c.offset == 240 and c._n_quantized == m.n_quantized == 192
+    assert c.compressed_key_bytes == m.key_bytes_compressed
+    assert c.compressed_value_bytes == m.value_bytes_compressed
+    assert c.residual_fp16_bytes == m.residual_fp16_bytes and c.fp16_key_bytes == m.key_bytes_fp16
+    total_fp16 = m.key_bytes_fp16 + m.value_bytes_fp16
+    assert c.effective_compression_ratio == total_fp16 / (m.key_bytes_compressed + m.value_bytes_compressed
+                                                          + m.residual_fp16_bytes)
+
+
+def test_one_shot_equals_token_by_token():
+    require_gpu()
+    k, v = _kv(1, 2, 48, 128, 13)
+    a = _make(residual_length=8, kivi_group_size=8)
+    ka, va = a.update_and_fetch(to_dev(k), to_dev(v))
+    b = _make(residual_length=8, kivi_group_size=8)
+    for t in range(48):
+        kb, vb = b.update_and_fetch(to_dev(k[:, :, t:t + 1]), to_dev(v[:, :, t:t + 1]))
+        assert b._n_quantized % 8 == 0 and b.offset - b._n_quantized <= 8 + 8 - 1
+    assert torch.equal(ka, kb) and torch.equal(va, vb) and a._n_quantized == b._n_quantized == 40
+
+
+def test_trim_equals_model_and_requantises():
+    require_gpu()
+    k, v = _kv(1, 2, 100, 64, 5)
+    c = _make(head_dim=64, residual_length=8, kivi_group_size=8)
+    m = ok.KiviCacheModel(2, 8, 8)
+    c.update_and_fetch(to_dev(k), to_dev(v)); m.update_and_fetch(k, v)
+    assert c.trim(36) == m.trim(36) == 36
+    assert (c.offset, c._n_quantized) == (m.offset, m.n_quantized) == (64, 64)
+    assert c.compressed_key_bytes == m.key_bytes_compressed and c.fp16_key_bytes == m.key_bytes_fp16
+    k2, v2 = _kv(1, 2, 30, 64, 6)
+    ko, vo = c.update_and_fetch(to_dev(k2), to_dev(v2)); mk, mv = m.update_and_fetch(k2, v2)
+    assert np.array_equal(host(ko), mk) and np.array_equal(host(vo), mv)
+
+
+@pytest.mark.parametrize("memory_bound", [False, True])
+@pytest.mark.parametrize("bits,g,meta", [(2, 32, "float16"), (4, 64, "float16"), (4, 32, "float32")])
+def test_fused_sdpa_over_packed_prefix(memory_bound, bits, g, meta):
+    """Decode through the packed store: the same positions are quantised with the
+    same groups as the cache model, and attention matches the oracle."""
+    require_gpu()
+    R = 64
+    c = _make(bit_width_inlier=bits, kivi_group_size=g, residual_length=R, fused_sdpa=True,
+              fused_sdpa_memory_bound=memory_bound, kivi_meta_dtype=meta)
+    k, v = outlier_kv((2, 2, 300, 128), seed=bits + g)
+    rng = np.random.default_rng(9)
+    c.update_and_fetch(to_dev(k[:, :, :257]), to_dev(v[:, :, :257]))
+    for t in range(257, 300):
+        ko, vo = c.update_and_fetch(to_dev(k[:, :, t:t + 1]), to_dev(v[:, :, t:t + 1]))
+    nq = ok.quantization_boundary(300, R, g)
+    assert c._n_quantized == nq and ko.shape == (2, 2, 300, 128)
+    q = rng.standard_normal((2, 8, 1, 128)).astype(np.float16)
+    out = c.fused_sdpa(to_dev(q), 1 / math.sqrt(128))
+    assert out.dtype == torch.float16
+    levels = (1 << bits) - 1
+    npm = np.float16 if meta == "float16" else np.float32
+    kq = ok.group_quant_codes(k[:, :, :nq], -2, g, levels)
+    vq = ok.group_quant_codes(v[:, :, :nq], -1, g, levels)
+    ref = oa.kivi_attend(q, kq[0], kq[1].astype(npm), kq[2].astype(npm), vq[0], vq[1].astype(npm),
+                         vq[2].astype(npm), g, k[:, :, nq:], v[:, :, nq:], 1 / math.sqrt(128))
+    assert np.max(np.abs(host(out).astype(np.float32) - ref)) < 2e-3
+    if memory_bound:
+        assert c.nbytes < 0.6 * (2 * 2 * 2 * 300 * 128 * 2) + 4 * c._tail_k.numel()
+        assert float(ko.abs().sum()) == 0.0 and not c.empty()
+    else:
+        # stash mode still returns the reference's fp16 history
+        mk, _ = ok.KiviCacheModel(bits, g, R).update_and_fetch(k, v)
+        assert np.array_equal(host(ko), mk)
+
+
+def test_memory_bound_trim_restores_reconstruction():
+    require_gpu()
+    c = _make(bit_width_inlier=4, kivi_group_size=32, residual_length=32, fused_sdpa=True,
+              fused_sdpa_memory_bound=True, kivi_meta_dtype="float32")
+    m = ok.KiviCacheModel(4, 32, 32)
+    k, v = outlier_kv((1, 2, 200, 128), seed=2)
+    c.update_and_fetch(to_dev(k), to_dev(v)); mk, mv = m.update_and_fetch(k, v)
+    assert c.trim(90) == m.trim(90) == 90 and c._n_quantized == m.n_quantized == 96
+    live = c.offset - c._n_quantized
+    assert np.array_equal(host(c._tail_k[:, :, :live]), mk[:, :, 96:110])
+    assert np.array_equal(host(c._tail_v[:, :, :live]), mv[:, :, 96:110])
+    q = np.random.default_rng(0).standard_normal((1, 4, 1, 128)).astype(np.float16)
+    out = c.fused_sdpa(to_dev(q), 0.09)
+    ref = oa.sdpa(q, mk[:, :, :110], mv[:, :, :110], 0.09)
+    assert np.max(np.abs(host(out).astype(np.float32) - ref)) < 2e-3
+
+
+def test_chunked_prefill_through_the_cache_matches_oracle():
+    """Quantise-on-write prefill: chunks of 64 through a cache with R=32, g=32."""
+    require_gpu()
+    B, Hq, Hkv, S, D = 1, 8, 2, 256, 128
+    k, v = outlier_kv((B, Hkv, S, D), seed=12)
+    q = np.random.default_rng(5).standard_normal((B, Hq, S, D)).astype(np.float16)
+    c = _make(bit_width_inlier=4, kivi_group_size=32, residual_length=32, fused_sdpa=True,
+              fused_sdpa_memory_bound=True, kivi_meta_dtype="float32")
+    outs = []
+    for s0 in range(0, S, 64):
+        c.update_and_fetch(to_dev(k[:, :, s0:s0 + 64]), to_dev(v[:, :, s0:s0 + 64]))
+        outs.append(host(c.fused_sdpa(to_dev(q[:, :, s0:s0 + 64]), 1 / math.sqrt(D), causal=True)))
+    got = np.concatenate(outs, axis=2).astype(np.float32)
+    ref = oa.chunked_prefill(q, k, v, 64, 4, 32, 32, 1 / math.sqrt(D))
+    assert np.max(np.abs(got - ref)) < 2e-3
+
+
+def test_kivi_quantizer_encode_decode():
+    require_gpu()
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((96, 128)).astype(np.float16)
+    for axis, ax in (("channel", -2), ("token", -1)):
+        qz = KIVIQuantizer(d=128, b=2, group_size=32, axis=axis)
+        ev = qz.encode(to_dev(x))
+        codes, scale, zero = ok.group_quant_codes(x[None, None], ax, 32, 3)
+        assert np.array_equal(host(ev.indices), codes[0, 0]) and np.array_equal(host(ev.norm), scale[0, 0])
+        assert ev.memory_bytes() == codes.nbytes + scale.nbytes + zero.nbytes
+        dec = qz.decode(ev)
+        assert np.array_equal(host(dec), ok.group_dequant(codes, scale, zero, ax, 32)[0, 0].astype(np.float16))
+        qv = rng.standard_normal(128).astype(np.float16)
+        ip = qz.estimate_inner_product(to_dev(qv), ev)
+        np.testing.assert_allclose(host(ip).astype(np.float32), host(dec).astype(np.float32) @ qv.astype(np.float32),
+                                   rtol=2e-3, atol=2e-2)
+    from veloxquant_mlx_amd.core import QuantizerConfigError
+    bad = x.copy(); bad[0, 0] = np.inf
+    with pytest.raises(QuantizerConfigError, match="NaN or Inf"):
+        KIVIQuantizer(d=128).encode(to_dev(bad))
+
+
+# ------------------------------------------------------------------ VecInfer
+def _vi_cfg(**kw):
+    rng = np.random.default_rng(7)
+    base = dict(method="vecinfer", head_dim=128, key_sub_dim=8, value_sub_dim=8, key_codebook_bits=8,
+                value_codebook_bits=8, key_codebook=rng.standard_normal((256, 8)).astype(np.float32),
+                value_codebook=rng.standard_normal((256, 8)).astype(np.float32))
+    base.update(kw)
+    return KVCacheConfig(**base)
+
+
+def test_vecinfer_standard_mode_matches_oracle_pipeline():
+    require_gpu()
+    rng = np.random.default_rng(1)
+    smooth = (np.abs(rng.standard_normal((2, 128))) + 0.5).astype(np.float32)
+    cfg = _vi_cfg(smooth_factors=smooth)
+    c = KVCacheFactory.create(cfg)
+    k, v = _kv(1, 2, 40, 128, 2)
+    ko, vo = c.update_and_fetch(to_dev(k), to_dev(v))
+    # values: plain VQ round trip, exact
+    v_idx = ov.quantize_vq(v, cfg.value_codebook, 8)
+    assert np.array_equal(host(vo), ov.dequantize_vq(v_idx, cfg.value_codebook).astype(np.float16))
+    # keys: transform (BLAS) then VQ; compare the reconstruction within fp16 rounding
+    H = ov.walsh_hadamard_matrix(128)
+    kt = ov.apply_dual_transform_keys(k, smooth, H)
+    k_hat = (ov.dequantize_vq(ov.quantize_vq(kt, cfg.key_codebook, 8), cfg.key_codebook) @ H.T) * smooth[:, None, :]
+    close = np.isclose(host(ko).astype(np.float32), k_hat, atol=2e-2, rtol=2e-3)
+    assert close.mean() > 0.995   # a near-tie may flip one sub-vector's centroid
+    assert c.compressed_key_bytes == 16 * 2 * 40 and c.fp16_key_bytes == 2 * 40 * 128 * 2
+
+
+@pytest.mark.parametrize("memory_bound", [False, True])
+def test_vecinfer_fused_modes_and_state_round_trip(memory_bound):
+    require_gpu()
+    cfg = _vi_cfg(fused_sdpa=True, fused_sdpa_memory_bound=memory_bound)
+    c = KVCacheFactory.create(cfg)
+    k, v = _kv(2, 2, 70, 128, 3)
+    c.update_and_fetch(to_dev(k[:, :, :64]), to_dev(v[:, :, :64]))
+    for t in range(64, 70):
+        ko, vo = c.update_and_fetch(to_dev(k[:, :, t:t + 1]), to_dev(v[:, :, t:t + 1]))
+    assert c.offset == 70 and c._stored_S_kv == 70 and c._stored_k_indices.shape[2] == 256
+    H = ov.walsh_hadamard_matrix(128)
+    k_idx = host(c._stored_k_indices[:, :, :70])
+    v_idx = host(c._stored_v_indices[:, :, :70])
+    assert np.array_equal(v_idx, ov.quantize_vq(v, cfg.value_codebook, 8))
+    kt_gpu = host(to_dev(k).float() @ to_dev(H))
+    assert np.array_equal(k_idx, ov.quantize_vq(kt_gpu, cfg.key_codebook, 8))
+    q = np.random.default_rng(4).standard_normal((2, 8, 1, 128)).astype(np.float16)
+    out = c.fused_sdpa(to_dev(q), 0.09, causal=True)
+    k_t_hat = ov.dequantize_vq(k_idx, cfg.key_codebook)
+    v_hat = ov.dequantize_vq(v_idx, cfg.value_codebook)
+    ref = oa.sdpa(q.astype(np.float32) @ H, k_t_hat, v_hat, 0.09)
+    assert np.max(np.abs(host(out).astype(np.float32) - ref)) < 2e-3
+    st = c.state
+    if memory_bound:
+        assert len(st) == 2 and st[0].shape == (2, 2, 70, 16) and float(ko.abs().sum()) == 0
+        c2 = KVCacheFactory.create(cfg)
+        c2.state = st
+        assert c2.offset == 70 and c2._stored_S_kv == 70
+        assert torch.equal(c2.fused_sdpa(to_dev(q), 0.09), out)
+    else:
+        assert len(st) == 4 and st[0].shape == (2, 2, 70, 128)
+    assert c.trim(6) == 6 and c._stored_S_kv == 64 and c.offset == 64
+    assert c.compressed_key_bytes == int(16 * 2 * 2 * 70 * (64 / 70))
+    with pytest.raises(ValueError, match="sliding_window"):
+        c.fused_sdpa(to_dev(q), 0.09, sliding_window=16)
+
+
+def test_vecinfer_max_ctx_cap():
+    require_gpu()
+    c = KVCacheFactory.create(_vi_cfg(fused_sdpa=True, fused_sdpa_max_ctx=100))
+    k, v = _kv(1, 1, 90, 128, 1)
+    c.update_and_fetch(to_dev(k), to_dev(v))
+    with pytest.raises(RuntimeError, match="exceeded fused_sdpa_max_ctx=100"):
+        c.update_and_fetch(to_dev(k[:, :, :20]), to_dev(v[:, :, :20]))

@@ -1,0 +1,162 @@
+"""Host-side configuration surface (no GPU work): option read-through, explicit
+field priority, factory dispatch and rejections, builder validation.  Restates
+veloxquant_mlx/tests/cache/test_kvcache_config_options.py:21-107 and
+veloxquant_mlx/tests/cache/test_cache_factory.py:28-99 for the two methods built."""
+
+import dataclasses
+import warnings
+from types import SimpleNamespace
+
+import pytest
+
+import veloxquant_mlx_amd.cache.options as opts
+from veloxquant_mlx_amd.cache import KIVIOptions, KVCacheBuilder, KVCacheConfig, KVCacheFactory, VecInferOptions
+from veloxquant_mlx_amd.cache.base import _CACHE_CLASS_BY_METHOD, _FIELD_TO_OPTIONS_CLASS
+from veloxquant_mlx_amd.cache.kivi_cache import KIVIKVCache
+from veloxquant_mlx_amd.cache.vecinfer_cache import VecInferKVCache
+from veloxquant_mlx_amd.core import EncodedVector, QuantizerConfigError, QuantizerRegistry
+
+
+def test_defaults_match_reference_values():
+    c = KVCacheConfig()
+    assert (c.head_dim, c.bit_width_inlier, c.kivi_group_size, c.residual_length) == (128, 2, 32, 128)
+    assert (c.key_sub_dim, c.value_sub_dim, c.key_codebook_bits, c.value_codebook_bits) == (4, 8, 12, 8)
+    assert c.use_metal_kernels is None and c.fused_sdpa is False and c.fused_sdpa_memory_bound is False
+    assert c.fused_sdpa_max_ctx is None and c.seed == 42
+
+
+def test_flat_field_construction_no_warning():
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        config = KVCacheConfig(method="kivi", kivi_group_size=64)
+    assert config.kivi_group_size == 64
+    assert not any(issubclass(w.category, DeprecationWarning) for w in caught)
+
+
+def test_options_populate_flat_fields_and_explicit_wins():
+    c = KVCacheConfig(method="vecinfer", options=VecInferOptions(key_sub_dim=8, key_codebook_bits=8))
+    assert c.key_sub_dim == 8 and c.key_codebook_bits == 8 and c.value_sub_dim == 8
+    c = KVCacheConfig(method="kivi", kivi_group_size=16, options=KIVIOptions(kivi_group_size=64))
+    assert c.kivi_group_size == 16
+    # an explicit value equal to the default still beats options
+    c = KVCacheConfig(method="kivi", kivi_group_size=32, options=KIVIOptions(kivi_group_size=64))
+    assert c.kivi_group_size == 32
+
+
+def test_post_construction_set_warns_only_for_option_fields():
+    c = KVCacheConfig(method="kivi")
+    with warnings.catch_warnings(record=True) as caught:
+        warnings.simplefilter("always")
+        c.kivi_group_size = 64
+        c.seed = 7
+    dep = [w for w in caught if issubclass(w.category, DeprecationWarning)]
+    assert len(dep) == 1 and "KIVIOptions" in str(dep[0].message)
+    assert c.kivi_group_size == 64 and c.seed == 7
+
+
+def test_every_options_default_matches_config_default():
+    flat = {f.name: f.default for f in dataclasses.fields(KVCacheConfig)}
+    for cls_name in set(_FIELD_TO_OPTIONS_CLASS.values()):
+        for f in dataclasses.fields(getattr(opts, cls_name)):
+            assert f.default == flat[f.name], f"{cls_name}.{f.name}"
+
+
+def test_inlier_bits_warning_for_methods_that_ignore_it():
+    with pytest.warns(UserWarning, match="ignores bit_width_inlier"):
+        KVCacheConfig(method="vecinfer", bit_width_inlier=3)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        KVCacheConfig(method="kivi", bit_width_inlier=3)
+        dataclasses.replace(KVCacheConfig(method="vecinfer"), head_dim=64)
+
+
+def test_factory_dispatch_and_rejections():
+    assert set(_CACHE_CLASS_BY_METHOD) == {"kivi", "vecinfer"}
+    assert isinstance(KVCacheFactory.create(KVCacheConfig(method="kivi")), KIVIKVCache)
+    with pytest.warns(UserWarning, match="random N"):
+        assert isinstance(KVCacheFactory.create(KVCacheConfig(method="vecinfer")), VecInferKVCache)
+    with pytest.raises(QuantizerConfigError, match="unknown method 'nope'. Choices: vecinfer, kivi"):
+        KVCacheFactory.create(KVCacheConfig(method="nope"))
+    with pytest.raises(QuantizerConfigError, match="observers"):
+        KVCacheFactory.create(KVCacheConfig(method="kivi", observers=[object()]))
+    with pytest.raises(QuantizerConfigError, match="bit_width_outlier"):
+        KVCacheFactory.create(KVCacheConfig(method="kivi", bit_width_outlier=3))
+    with pytest.raises(QuantizerConfigError, match="single int"):
+        KVCacheFactory.create(KVCacheConfig(method="kivi", bit_width_inlier=[2, 4]))
+    with pytest.raises(QuantizerConfigError, match="sliding_window"):
+        KVCacheFactory.create(KVCacheConfig(method="kivi", sliding_window=64))
+
+
+def test_kivi_cache_surface():
+    c = KVCacheFactory.create(KVCacheConfig(method="kivi", bit_width_inlier=4))
+    assert not hasattr(c, "bits") and c.assigned_avg_bits == 4.0
+    assert c.offset == 0 and c.empty() and c.size() == 0 and c.nbytes == 0
+    assert c.effective_compression_ratio == 1.0 and c.trim(3) == 0
+    with pytest.raises(RuntimeError, match="fused_sdpa was not enabled"):
+        c.fused_sdpa(None, 1.0)
+    with pytest.raises(RuntimeError, match="requires fused_sdpa=True"):
+        KIVIKVCache(KVCacheConfig(method="kivi", fused_sdpa_memory_bound=True))
+    with pytest.raises(QuantizerConfigError, match="kivi_meta_dtype"):
+        KIVIKVCache(KVCacheConfig(method="kivi", kivi_meta_dtype="int8"))
+    # duck-typed configs work, as in the reference's tests
+    c = KIVIKVCache(SimpleNamespace(head_dim=64, bit_width_inlier=2, kivi_group_size=8, residual_length=4))
+    assert c._group_size == 8 and c._residual_length == 4 and c._v_layout == "channel"
+    assert KIVIKVCache(KVCacheConfig(method="kivi"))._v_layout == "token"
+
+
+def test_vecinfer_cache_validation():
+    import numpy as np
+    kw = dict(method="vecinfer", key_codebook=np.zeros((256, 8), np.float32), key_sub_dim=8, key_codebook_bits=8,
+              value_codebook=np.zeros((256, 8), np.float32))
+    with pytest.raises(QuantizerConfigError, match="power-of-2 head_dim"):
+        KVCacheFactory.create(KVCacheConfig(head_dim=96, **kw))
+    with pytest.raises(QuantizerConfigError, match="not divisible by key_sub_dim"):
+        KVCacheFactory.create(KVCacheConfig(head_dim=128, **{**kw, "key_sub_dim": 3}))
+    with pytest.raises(QuantizerConfigError, match="smooth_factors must be finite"):
+        KVCacheFactory.create(KVCacheConfig(head_dim=128, smooth_factors=np.zeros(128, np.float32), **kw))
+    with pytest.raises(RuntimeError, match="requires fused_sdpa=True"):
+        KVCacheFactory.create(KVCacheConfig(head_dim=128, fused_sdpa_memory_bound=True, **kw))
+    c = KVCacheFactory.create(KVCacheConfig(head_dim=128, fused_sdpa=True, fused_sdpa_memory_bound=True, **kw))
+    assert c._memory_bound and c.empty() and c.state[0].shape == (1, 1, 0, 16)
+    assert c.assigned_avg_bits == 1.0 and c.codebook_bytes == 2 * 256 * 8 * 2
+    with pytest.raises(AttributeError):
+        c.merge
+    with pytest.raises(RuntimeError, match="before any tokens"):
+        c.fused_sdpa(None, 1.0)
+    c._smooth = __import__("torch").ones(3, 128)
+    with pytest.raises(QuantizerConfigError, match="has 3 rows"):
+        c._resolve_smooth_heads(2)
+
+
+def test_builder_validation_and_for_model():
+    with pytest.raises(QuantizerConfigError, match="power of 2"):
+        KVCacheBuilder().with_method("kivi").with_head_dim(96).build()
+    with pytest.raises(QuantizerConfigError, match="must be >= 1"):
+        KVCacheBuilder().with_method("kivi").with_bit_width(0).build()
+    with pytest.raises(QuantizerConfigError, match="must not be empty"):
+        KVCacheBuilder().with_method("kivi").with_bit_width([]).build()
+    assert isinstance(KVCacheBuilder().with_method("kivi").with_head_dim(64).with_bit_width(4).build(), KIVIKVCache)
+
+    attn = SimpleNamespace(head_dim=64)
+    layers = [SimpleNamespace(self_attn=attn), SimpleNamespace(mlp=1), SimpleNamespace(self_attn=SimpleNamespace(head_dim=None))]
+    model = SimpleNamespace(layers=layers, args=SimpleNamespace(hidden_size=512, num_attention_heads=4, head_dim=None))
+    caches = KVCacheBuilder.for_model(model, KVCacheConfig(method="kivi", bit_width_inlier=[2, 4], seed=5))
+    assert [type(c).__name__ for c in caches] == ["KIVIKVCache", "FP16KVCache", "KIVIKVCache"]
+    assert caches[0]._head_dim == 64 and caches[2]._head_dim == 128
+    assert caches[0]._b == 2 and caches[2]._b == 4
+    with pytest.raises(QuantizerConfigError, match="one entry per attention layer"):
+        KVCacheBuilder.for_model(model, KVCacheConfig(method="kivi", bit_width_inlier=[2, 4, 8]))
+
+
+def test_core_types():
+    ev = EncodedVector("kivi", 2, 4)
+    assert ev.memory_bytes() == 0 and "kivi" in repr(ev)
+    import veloxquant_mlx_amd.quantizers  # registers
+    assert "kivi" in QuantizerRegistry.names()
+    q = QuantizerRegistry.create("kivi", d=16, b=4)
+    assert "b=4" in repr(q)
+    with pytest.raises(QuantizerConfigError, match=r"must be in \[1, 8\]"):
+        QuantizerRegistry.create("kivi", d=16, b=9)
+    with pytest.raises(QuantizerConfigError, match="'channel' or 'token'"):
+        QuantizerRegistry.create("kivi", d=16, axis="rows")
+    assert issubclass(QuantizerConfigError, ValueError)

@@ -1,0 +1,397 @@
+"""KIVI KV cache on torch ROCm tensors.
+
+Behaviour follows ``KIVIKVCache`` (veloxquant_mlx/cache/kivi_cache.py:83-410):
+keys are quantised per channel (groups along tokens), values per token (groups
+along channels), the newest ``residual_length`` tokens stay fp16, and tokens are
+flushed only in whole ``kivi_group_size`` blocks.
+
+Three storage modes, selected with the same two flags the reference's VecInfer
+cache uses (veloxquant_mlx/cache/vecinfer_cache.py:384-411):
+
+* ``fused_sdpa=False`` (default) -- the reference's behaviour: an fp16 history
+  whose aged-out prefix is round-tripped in place; ``update_and_fetch`` returns
+  fp16 ``[B,H,offset,D]``.
+* ``fused_sdpa=True`` -- the same, plus bit-packed codes and scale/zero kept
+  beside it so :meth:`fused_sdpa` can attend over the packed prefix.
+* ``fused_sdpa=True, fused_sdpa_memory_bound=True`` -- packed prefix and a short
+  fp16 tail only; ``update_and_fetch`` returns zero-stride placeholders and
+  attention must go through :meth:`fused_sdpa`.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Any
+
+import torch
+
+from .. import kernels as K
+from ..core.exceptions import QuantizerConfigError
+from ._fp16_cache import FP16KVCache
+
+_META = {"float16": torch.float16, "float32": torch.float32}
+
+
+class KIVIKVCache(FP16KVCache):
+    """KV cache with KIVI asymmetric group quantisation.
+
+    Never exposes ``.bits`` (a host attention dispatcher would take it for a
+    natively quantised cache, kivi_cache.py:93-95); see ``assigned_avg_bits``.
+    """
+
+    def __init__(self, config: Any) -> None:
+        super().__init__()
+        self._head_dim = int(config.head_dim)
+        b = config.bit_width_inlier
+        if isinstance(b, list):
+            raise QuantizerConfigError(
+                "KIVIKVCache: bit_width_inlier must be a single int; "
+                "per-layer lists are dispatched by KVCacheBuilder.for_model().")
+        self._b = int(b)
+        if not (1 <= self._b <= 8):
+            raise QuantizerConfigError(f"KIVIKVCache: bit_width_inlier={self._b} must be in [1, 8].")
+        self._group_size = int(getattr(config, "kivi_group_size", 32))
+        self._residual_length = int(getattr(config, "residual_length", 128))
+        if self._group_size < 1:
+            raise QuantizerConfigError(f"KIVIKVCache: kivi_group_size={self._group_size} must be >= 1.")
+        self._levels = (1 << self._b) - 1
+        self._eps = 1e-8
+
+        # use_metal_kernels keeps its three states (kivi_cache.py:113-130).  The
+        # HIP library is the only implementation, so True and None both require
+        # it and False selects the same kernels (the reference's two paths are
+        # bit-identical by contract).
+        requested = getattr(config, "use_metal_kernels", None)
+        available = K._lib.library_present()
+        if not available:
+            raise RuntimeError(
+                "KIVIKVCache: the HIP kernel library is not available on this build "
+                f"(use_metal_kernels={requested!r}); there is no fallback path.")
+        self._use_metal = True
+
+        fused = bool(getattr(config, "fused_sdpa", False))
+        self._memory_bound = bool(getattr(config, "fused_sdpa_memory_bound", False))
+        if self._memory_bound and not fused:
+            raise RuntimeError("KIVIKVCache: fused_sdpa_memory_bound=True requires fused_sdpa=True.")
+        self._fused_enabled = fused
+        cap = getattr(config, "fused_sdpa_max_ctx", None)
+        self._max_ctx = None if cap is None else int(cap)
+        meta = getattr(config, "kivi_meta_dtype", "float16")
+        if meta not in _META:
+            raise QuantizerConfigError(f"KIVIKVCache: kivi_meta_dtype={meta!r} must be 'float16' or 'float32'.")
+        self._meta_dtype = _META[meta]
+        per = 32 // self._b
+        layout = getattr(config, "kivi_value_layout", "auto")
+        if layout == "auto":
+            layout = "token" if self._group_size % per == 0 else "channel"
+        if layout not in ("token", "channel"):
+            raise QuantizerConfigError(f"KIVIKVCache: kivi_value_layout={layout!r} must be token/channel/auto.")
+        if layout == "token" and self._group_size % per != 0:
+            raise QuantizerConfigError(
+                f"KIVIKVCache: token-packed values need kivi_group_size % {per} == 0 at {self._b} bits.")
+        self._v_layout = layout
+        self._per = per
+
+        # byte accounting (kivi_cache.py:132-146)
+        self._key_bytes_compressed = 0
+        self._key_bytes_fp16 = 0
+        self._value_bytes_compressed = 0
+        self._value_bytes_fp16 = 0
+        self._residual_fp16_bytes = 0
+        self._tokens_seen = 0
+        self._n_quantized = 0
+        self._shape_bhd: tuple[int, int, int] = (1, 1, int(config.head_dim))
+
+        # packed store (fused modes)
+        self._kp = self._ks = self._kz = None
+        self._vp = self._vs = self._vz = None
+        self._packed_cap = 0
+        # fp16 tail (memory-bound mode): tokens [_n_quantized, offset)
+        self._tail_k = self._tail_v = None
+
+    # ------------------------------------------------------------------
+    def _quant_dequant_along(self, x: torch.Tensor, axis: int) -> torch.Tensor:
+        """Round-trip ``x`` through group quantisation (kivi_cache.py:151-201)."""
+        return K.kivi_group_quant_dequant(x, axis=axis, group_size=self._group_size, levels=self._levels,
+                                          eps=self._eps)
+
+    def _quantization_boundary(self) -> int:
+        """Absolute position up to which tokens may be quantised now (kivi_cache.py:206-225)."""
+        aged = max(0, self.offset - self._residual_length)
+        return (aged // self._group_size) * self._group_size
+
+    # ------------------------------------------------------------------ packed store
+    def _ensure_packed_capacity(self, B: int, H: int, D: int, needed: int, device) -> None:
+        if self._max_ctx is not None and needed > self._max_ctx:
+            raise RuntimeError(f"KIVIKVCache: context length {needed} exceeded fused_sdpa_max_ctx={self._max_ctx}. "
+                               "Raise or unset KVCacheConfig.fused_sdpa_max_ctx.")
+        if needed <= self._packed_cap:
+            return
+        g, per = self._group_size, self._per
+        unit = g * per // math.gcd(g, per)
+        cap = max(needed, 2 * self._packed_cap, 1024)
+        if self._max_ctx is not None:
+            cap = min(cap, self._max_ctx)
+        cap = -(-cap // unit) * unit
+        W = -(-D // per)
+        GV = -(-D // g)
+        z = lambda shape, dt: torch.zeros(shape, dtype=dt, device=device)
+        kp = z((B, H, cap, W), torch.int32)
+        ks = z((B, H, cap // g, D), self._meta_dtype)
+        kz = z((B, H, cap // g, D), self._meta_dtype)
+        if self._v_layout == "token":
+            vp = z((B, H, cap // per, D), torch.int32)
+            vs = z((B, H, GV, cap), self._meta_dtype)
+            vz = z((B, H, GV, cap), self._meta_dtype)
+        else:
+            vp = z((B, H, cap, W), torch.int32)
+            vs = z((B, H, cap, GV), self._meta_dtype)
+            vz = z((B, H, cap, GV), self._meta_dtype)
+        n = self._n_quantized
+        if self._kp is not None and n > 0:
+            kp[:, :, :n] = self._kp[:, :, :n]
+            ks[:, :, : n // g] = self._ks[:, :, : n // g]
+            kz[:, :, : n // g] = self._kz[:, :, : n // g]
+            if self._v_layout == "token":
+                vp[:, :, : n // per] = self._vp[:, :, : n // per]
+                vs[..., :n] = self._vs[..., :n]
+                vz[..., :n] = self._vz[..., :n]
+            else:
+                vp[:, :, :n] = self._vp[:, :, :n]
+                vs[:, :, :n] = self._vs[:, :, :n]
+                vz[:, :, :n] = self._vz[:, :, :n]
+        self._kp, self._ks, self._kz, self._vp, self._vs, self._vz = kp, ks, kz, vp, vs, vz
+        self._packed_cap = cap
+
+    def _pack_block(self, k_blk: torch.Tensor, v_blk: torch.Tensor, lo: int) -> None:
+        """Quantise + pack fp16 tokens (a group-aligned block) at packed position ``lo``."""
+        B, H, n, D = k_blk.shape
+        self._ensure_packed_capacity(B, H, D, lo + n, k_blk.device)
+        K.kivi_quant_pack(k_blk, -2, self._group_size, self._b, eps=self._eps, meta_dtype=self._meta_dtype,
+                          out=(self._kp, self._ks, self._kz), dst_tok0=lo)
+        K.kivi_quant_pack(v_blk, -1, self._group_size, self._b, eps=self._eps, meta_dtype=self._meta_dtype,
+                          v_layout=self._v_layout, out=(self._vp, self._vs, self._vz), dst_tok0=lo)
+
+    # ------------------------------------------------------------------ protocol
+    def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
+        """Append ``[B,H,S,D]`` keys/values and quantise whatever aged out of the
+        fp16 residual window, in ``kivi_group_size``-aligned blocks
+        (kivi_cache.py:230-262)."""
+        B, H, S, D = keys.shape
+        self._shape_bhd = (B, H, D)
+        if self._memory_bound:
+            return self._update_memory_bound(keys, values)
+        k_all, v_all = super().update_and_fetch(keys, values)
+        new_boundary = self._quantization_boundary()
+        n_quant_now = new_boundary - self._n_quantized
+        if n_quant_now > 0:
+            lo, hi = self._n_quantized, new_boundary
+            if self._fused_enabled:
+                # pack from the still-exact fp16 rows before they are overwritten
+                self._pack_block(self.keys[:, :, lo:hi], self.values[:, :, lo:hi], lo)
+            self.keys[:, :, lo:hi] = self._quant_dequant_along(self.keys[:, :, lo:hi], axis=-2)
+            self.values[:, :, lo:hi] = self._quant_dequant_along(self.values[:, :, lo:hi], axis=-1)
+            self._n_quantized = new_boundary
+            k_all, v_all = self.keys[:, :, : self.offset], self.values[:, :, : self.offset]
+        self._account_bytes(B, H, S, D, n_quant_now)
+        return k_all, v_all
+
+    def _update_memory_bound(self, keys: torch.Tensor, values: torch.Tensor):
+        B, H, S, D = keys.shape
+        n_tail = self.offset - self._n_quantized
+        need = n_tail + S
+        if self._tail_k is None or need > self._tail_k.shape[2]:
+            cap = max(need, self._residual_length + 2 * self._group_size)
+            cap = -(-cap // 64) * 64
+            tk = torch.zeros((B, H, cap, D), dtype=keys.dtype, device=keys.device)
+            tv = torch.zeros((B, H, cap, D), dtype=values.dtype, device=values.device)
+            if self._tail_k is not None and n_tail:
+                tk[:, :, :n_tail] = self._tail_k[:, :, :n_tail]
+                tv[:, :, :n_tail] = self._tail_v[:, :, :n_tail]
+            self._tail_k, self._tail_v = tk, tv
+        self._tail_k[:, :, n_tail:need] = keys
+        self._tail_v[:, :, n_tail:need] = values
+        self.offset += S
+        new_boundary = self._quantization_boundary()
+        n_quant_now = new_boundary - self._n_quantized
+        if n_quant_now > 0:
+            self._pack_block(self._tail_k[:, :, :n_quant_now], self._tail_v[:, :, :n_quant_now], self._n_quantized)
+            keep = need - n_quant_now
+            if keep:
+                self._tail_k[:, :, :keep] = self._tail_k[:, :, n_quant_now:need].clone()
+                self._tail_v[:, :, :keep] = self._tail_v[:, :, n_quant_now:need].clone()
+            self._n_quantized = new_boundary
+        self._account_bytes(B, H, S, D, n_quant_now)
+        z = torch.zeros((), dtype=keys.dtype, device=keys.device)
+        return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
+
+    def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0):
+        """Attention of ``q [B,H_q,S_q,D]`` over the packed prefix and the fp16 tail,
+        queries aligned to the end of the cache (the contract of
+        ``VecInferKVCache.fused_sdpa``, veloxquant_mlx/cache/vecinfer_cache.py:670-731)."""
+        if not self._fused_enabled:
+            raise RuntimeError("KIVIKVCache.fused_sdpa called but fused_sdpa was not enabled via "
+                               "KVCacheConfig.fused_sdpa=True.")
+        if self.offset == 0:
+            raise RuntimeError("KIVIKVCache.fused_sdpa called before any tokens were cached via update_and_fetch.")
+        if sliding_window:
+            raise ValueError("KIVIKVCache.fused_sdpa: sliding_window attention is not supported")
+        nq = self._n_quantized
+        n_tail = self.offset - nq
+        if self._memory_bound:
+            tk, tv = self._tail_k, self._tail_v
+        else:
+            tk, tv = self.keys[:, :, nq:], self.values[:, :, nq:]
+        return K.kivi_packed_attend(
+            q, k_packed=self._kp, k_scale=self._ks, k_zero=self._kz, v_packed=self._vp, v_scale=self._vs,
+            v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
+            k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
+            causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype)
+
+    # ------------------------------------------------------------------ trim / state
+    def _rollback_frontier(self, new_offset: int) -> int:
+        """kivi_cache.py:264-278: the frontier snaps down to a group multiple."""
+        gs = self._group_size
+        new_nq = min(self._n_quantized, (max(new_offset, 0) // gs) * gs)
+        n_rolled = self._n_quantized - new_nq
+        self._n_quantized = new_nq
+        return n_rolled
+
+    def _rollback_bytes(self, n_tokens: int, n_rolled: int) -> None:
+        B, H, D = self._shape_bhd
+        if n_rolled > 0:
+            k, v = self._quantized_bytes(n_rolled, B, H, D)
+            self._key_bytes_compressed = max(0, self._key_bytes_compressed - k)
+            self._value_bytes_compressed = max(0, self._value_bytes_compressed - v)
+        self._key_bytes_fp16 = max(0, self._key_bytes_fp16 - H * B * n_tokens * D * 2)
+        self._value_bytes_fp16 = max(0, self._value_bytes_fp16 - H * B * n_tokens * D * 2)
+        self._tokens_seen = max(0, self._tokens_seen - n_tokens)
+        self._residual_fp16_bytes = (self.offset - self._n_quantized) * D * 2 * 2 * H * B
+
+    def trim(self, n: int) -> int:
+        """Drop the last ``n`` tokens and roll frontier and accounting back (kivi_cache.py:293-299)."""
+        old_nq = self._n_quantized
+        trimmed = super().trim(n)
+        if trimmed:
+            n_rolled = self._rollback_frontier(self.offset)
+            if self._memory_bound and self._tail_k is not None:
+                # rows [new frontier, offset) that had been packed come back as their
+                # reconstruction, which is what the fp16 history of the other modes holds
+                live = self.offset - self._n_quantized
+                if n_rolled > 0 and live > 0:
+                    B, H, D = self._shape_bhd
+                    if live > self._tail_k.shape[2]:
+                        self._tail_k = torch.zeros((B, H, -(-live // 64) * 64, D), dtype=self._tail_k.dtype,
+                                                   device=self._tail_k.device)
+                        self._tail_v = torch.zeros_like(self._tail_k)
+                    lo = self._n_quantized
+                    self._tail_k[:, :, :live] = K.kivi_dequant(
+                        self._kp, self._ks, self._kz, -2, self._group_size, self._b, live, D,
+                        out_dtype=self._tail_k.dtype, src_tok0=lo)
+                    self._tail_v[:, :, :live] = K.kivi_dequant(
+                        self._vp, self._vs, self._vz, -1, self._group_size, self._b, live, D,
+                        v_layout=self._v_layout, out_dtype=self._tail_v.dtype, src_tok0=lo)
+            self._rollback_bytes(trimmed, n_rolled)
+        del old_nq
+        return trimmed
+
+    def empty(self) -> bool:
+        if self._memory_bound:
+            return self.offset == 0
+        return super().empty()
+
+    @property
+    def state(self):
+        """Standard / stash mode: the fp16 history (stash mode appends the live packed
+        rows).  Memory-bound mode: live packed rows followed by the live fp16 tail."""
+        if not self._fused_enabled:
+            return FP16KVCache.state.fget(self)
+        packed = self._packed_state()
+        if not self._memory_bound:
+            return (*FP16KVCache.state.fget(self), *packed)
+        n_tail = self.offset - self._n_quantized
+        if self._tail_k is None:
+            return packed
+        return (*packed, self._tail_k[:, :, :n_tail], self._tail_v[:, :, :n_tail])
+
+    def _packed_state(self):
+        n, g, per = self._n_quantized, self._group_size, self._per
+        if self._kp is None or n == 0:
+            return ()
+        if self._v_layout == "token":
+            v = (self._vp[:, :, : n // per], self._vs[..., :n], self._vz[..., :n])
+        else:
+            v = (self._vp[:, :, :n], self._vs[:, :, :n], self._vz[:, :, :n])
+        return (self._kp[:, :, :n], self._ks[:, :, : n // g], self._kz[:, :, : n // g], *v)
+
+    @state.setter
+    def state(self, v) -> None:
+        if self._fused_enabled:
+            raise NotImplementedError("KIVIKVCache: restoring a packed state is not supported yet")
+        FP16KVCache.state.fset(self, v)
+
+    @property
+    def nbytes(self) -> int:
+        total = 0 if self._memory_bound else FP16KVCache.nbytes.fget(self)
+        for t in (self._kp, self._ks, self._kz, self._vp, self._vs, self._vz, self._tail_k, self._tail_v):
+            if t is not None:
+                total += t.numel() * t.element_size()
+        return total
+
+    # ------------------------------------------------------------------ accounting
+    def _quantized_bytes(self, n: int, B: int, H: int, D: int) -> tuple[int, int]:
+        """(key, value) packed-byte cost of ``n`` group-aligned tokens (kivi_cache.py:301-306)."""
+        gs = self._group_size
+        k = math.ceil(n * D * self._b / 8) * H * B + math.ceil(n / gs) * D * 2 * 2 * H * B
+        v = math.ceil(n * D * self._b / 8) * H * B + n * math.ceil(D / gs) * 2 * 2 * H * B
+        return k, v
+
+    def _account_bytes(self, B: int, H: int, S: int, D: int, n_quant_now: int) -> None:
+        """kivi_cache.py:308-332."""
+        if n_quant_now > 0:
+            k, v = self._quantized_bytes(n_quant_now, B, H, D)
+            self._key_bytes_compressed += k
+            self._value_bytes_compressed += v
+        n_res = self.offset - self._n_quantized
+        self._residual_fp16_bytes = n_res * D * 2 * 2 * H * B
+        self._key_bytes_fp16 += H * B * S * D * 2
+        self._value_bytes_fp16 += H * B * S * D * 2
+        self._tokens_seen += S
+
+    @property
+    def compressed_key_bytes(self) -> int:
+        """Packed-storage byte cost of quantised key codes + fp16 (scale, zero)."""
+        return self._key_bytes_compressed
+
+    @property
+    def fp16_key_bytes(self) -> int:
+        return self._key_bytes_fp16
+
+    @property
+    def compressed_value_bytes(self) -> int:
+        return self._value_bytes_compressed
+
+    @property
+    def fp16_value_bytes(self) -> int:
+        return self._value_bytes_fp16
+
+    @property
+    def residual_fp16_bytes(self) -> int:
+        """Bytes held in fp16 and not yet quantised (keys + values)."""
+        return self._residual_fp16_bytes
+
+    @property
+    def assigned_avg_bits(self) -> float:
+        return float(self._b)
+
+    @property
+    def effective_compression_ratio(self) -> float:
+        """End-to-end KV byte ratio vs fp16, residual window included (kivi_cache.py:387-410)."""
+        total_fp16 = self._key_bytes_fp16 + self._value_bytes_fp16
+        if total_fp16 == 0:
+            return 1.0
+        total = self._key_bytes_compressed + self._value_bytes_compressed + self._residual_fp16_bytes
+        return total_fp16 / total if total else 1.0
+
+
+__all__ = ["KIVIKVCache"]

@@ -1,0 +1,27 @@
+"""Per-method option dataclasses read through by ``KVCacheConfig``
+(veloxquant_mlx/cache/options.py:36-50 in the reference)."""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+
+@dataclass
+class VecInferOptions:
+    """VecInfer-specific configuration."""
+
+    key_sub_dim: int = 4
+    value_sub_dim: int = 8
+    key_codebook_bits: int = 12
+    value_codebook_bits: int = 8
+    residual_length: int = 128
+
+
+@dataclass
+class KIVIOptions:
+    """KIVI configuration (asymmetric group quantization)."""
+
+    kivi_group_size: int = 32  # min/max group size (KIVI default 32)
+
+
+__all__ = ["VecInferOptions", "KIVIOptions"]

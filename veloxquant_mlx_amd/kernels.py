@@ -353,6 +353,19 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+def _tail_layout(t: torch.Tensor):
+    """Return ``(tensor, capacity)`` for a ``[B,H,n,D]`` tail that is either dense or
+    a token slice of a dense ``[B,H,capacity,D]`` buffer (rows dense, uniform head
+    stride); anything else is copied."""
+    B, H, n, D = t.shape
+    if t.stride(3) == 1 and t.stride(2) == D:
+        hs = t.stride(1) if H > 1 else (t.stride(0) if B > 1 else n * D)
+        if hs % D == 0 and hs >= n * D and (B == 1 or H == 1 or t.stride(0) == H * hs):
+            return t, hs // D
+    t = t.contiguous()
+    return t, n
+
+
 def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=None, v_packed=None,
                        v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
                        v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
@@ -404,14 +417,17 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         _need_gpu(name, k_tail, v_tail)
         if k_tail.dtype != v_tail.dtype:
             raise ValueError(f"{name}: k_tail and v_tail dtypes differ")
-        if not (k_tail.is_contiguous() and v_tail.is_contiguous()):
-            raise ValueError(f"{name}: tail tensors must be contiguous")
         if Hkv is not None and k_tail.shape[1] != Hkv:
             raise ValueError(f"{name}: tail has {k_tail.shape[1]} kv heads, packed cache has {Hkv}")
         Hkv = k_tail.shape[1]
+        k_tail, kcap = _tail_layout(k_tail)
+        v_tail, vcap = _tail_layout(v_tail)
+        if kcap != vcap:
+            k_tail, v_tail = k_tail.contiguous(), v_tail.contiguous()
+            kcap = vcap = k_tail.shape[2]
         a.k_tail, a.v_tail = k_tail.data_ptr(), v_tail.data_ptr()
         a.tail_dtype = _ftag(name, k_tail)
-        a.tail_cap = k_tail.shape[2]
+        a.tail_cap = kcap
         keep += [k_tail, v_tail]
     if Hkv is None:
         raise ValueError(f"{name}: no key/value slots to attend to")
