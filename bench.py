@@ -1,0 +1,258 @@
+#!/usr/bin/env python3
+"""Benchmark of the KV-cache compression hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[3], the "@32k ctx" decode the metric is
+quoted on): Qwen3-8B shape, 36 layers, 32 query / 8 kv heads, D=128, batch 16,
+32768 tokens of context per sequence stored as 4-bit packed KIVI codes (keys per
+channel, values per token, group 64) plus an fp16 tail.  One step = one decode
+token for every sequence through all 36 layers: append K/V to the fp16 tail,
+flush a 64-token block into the packed store when one is due, attend.
+
+Prints ONE JSON line.  ``value`` is algorithmic HBM bytes per step divided by
+the step time, inputs resident in HBM.  ``roofline`` prices the attention
+kernel alone (HIP events on the launch stream); ``cpu_baseline`` times the
+scalar C oracle on a bounded sample of the same workload on the host.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def _parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--warmup", type=int, default=3)
+    p.add_argument("--layers", type=int, default=36)
+    p.add_argument("--batch", type=int, default=16)
+    p.add_argument("--ctx", type=int, default=32768)
+    p.add_argument("--bits", type=int, default=4)
+    p.add_argument("--group", type=int, default=64)
+    p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    p.add_argument("--no-extras", action="store_true", help="skip the per-kernel side measurements")
+    p.add_argument("--only-kernel", action="store_true", help="time the attention kernel loop only (profiling)")
+    return p.parse_args()
+
+
+def _event_ms(fn, iters, torch):
+    """Average milliseconds per call, HIP events on the current stream."""
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    s.record()
+    for _ in range(iters):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) / iters
+
+
+def _algorithmic_bytes_per_layer(B, Hkv, ctx, D, bits, g):
+    codes = 2 * B * Hkv * ctx * D * bits // 8
+    meta = B * Hkv * (ctx // g) * D * 2 * 2 + B * Hkv * ctx * (D // g) * 2 * 2  # fp16 scale+zero, K and V
+    return codes + meta
+
+
+def _synthetic_layer(torch, B, Hkv, S, D, seed, dev):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    f = torch.exp(torch.randn(D, generator=g, device=dev))
+    k = (torch.randn((B, Hkv, S, D), generator=g, device=dev) * f).to(torch.float16)
+    v = torch.randn((B, Hkv, S, D), generator=g, device=dev).to(torch.float16)
+    return k, v
+
+
+def main() -> int:
+    a = _parse()
+    if a.gpus != 1:
+        print(f"bench.py: this build runs on ONE GPU (every kernel is independent per (sequence, kv head); "
+              f"--gpus {a.gpus} is not supported)", file=sys.stderr)
+        return 2
+    import numpy as np
+    import torch
+
+    from veloxquant_mlx_amd import kernels as K
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+
+    if not K.hip_available():
+        print("bench.py: no ROCm device / kernel library", file=sys.stderr)
+        return 1
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    NL, B, Hq, Hkv, D, ctx, bits, g = a.layers, a.batch, 32, 8, 128, a.ctx, a.bits, a.group
+    R = 128
+    scale = 1.0 / math.sqrt(D)
+
+    # ---- build the resident caches: prefill ctx + R tokens per layer in chunks
+    cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=bits, kivi_group_size=g, residual_length=R,
+                        fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=ctx + 4096)
+    caches = []
+    chunk = 4096
+    # stop ten tokens short of the next 64-token flush so that one falls inside the timed steps
+    prefill = ctx + R + g - 10
+    for l in range(NL):
+        c = KVCacheFactory.create(cfg)
+        for s0 in range(0, prefill, chunk):
+            n = min(chunk, prefill - s0)
+            k, v = _synthetic_layer(torch, B, Hkv, n, D, 1000 * l + s0, dev)
+            c.update_and_fetch(k, v)
+        caches.append(c)
+    del k, v
+    torch.cuda.synchronize()
+    assert caches[0]._n_quantized == ctx, caches[0]._n_quantized
+
+    gen = torch.Generator(device=dev).manual_seed(7)
+    q = torch.randn((NL, B, Hq, 1, D), generator=gen, device=dev).to(torch.float16)
+    k_new = torch.randn((NL, B, Hkv, 1, D), generator=gen, device=dev).to(torch.float16)
+    v_new = torch.randn((NL, B, Hkv, 1, D), generator=gen, device=dev).to(torch.float16)
+
+    def step():
+        for l, c in enumerate(caches):
+            c.update_and_fetch(k_new[l], v_new[l])
+            c.fused_sdpa(q[l], scale)
+
+    def attend_only():
+        for l, c in enumerate(caches):
+            c.fused_sdpa(q[l], scale)
+
+    layer_bytes = _algorithmic_bytes_per_layer(B, Hkv, ctx, D, bits, g)
+    if a.only_kernel:
+        for _ in range(a.warmup):
+            attend_only()
+        ms = _event_ms(attend_only, a.steps, torch) / NL
+        print(json.dumps({"attend_ms_per_layer": ms, "GBps": layer_bytes / ms / 1e6}))
+        return 0
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    step_bytes = layer_bytes * NL
+    value = step_bytes / dt / 1e9
+
+    # ---- roofline of the dominant kernel (attention), events on the launch stream
+    kern_ms = _event_ms(attend_only, max(3, a.steps // 2), torch) / NL
+    achieved = layer_bytes / (kern_ms * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                "kernel": "attention over packed cache (one layer: attend + split merge)",
+                "bytes_per_launch": layer_bytes, "ms_per_launch": round(kern_ms, 5)}
+
+    out = {
+        "metric": "dequant-SDPA decode HBM GB/s @32k ctx", "value": round(value, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8/f16 (f32 accumulate)",
+        "data": "synthetic",
+        "config": {"workload": f"configs[3]: batched decode, {NL} layers, 32q/8kv heads, D=128, batch {B}, "
+                               f"context {ctx}, {bits}-bit packed KV group {g}, append+flush+attend per step",
+                   "layers": NL, "batch": B, "context": ctx, "bits": bits, "group": g,
+                   "algorithmic_bytes_per_step": step_bytes},
+        "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+        "roofline": roofline,
+    }
+
+    if not a.no_extras:
+        out["extras"] = _extras(torch, K, dev)
+    if not a.no_cpu:
+        out["cpu_baseline"] = _cpu_baseline(np, torch, caches[0], q[0], ctx, Hkv, D, bits, g, scale)
+    print(json.dumps(out))
+    return 0
+
+
+def _extras(torch, K, dev):
+    """Side measurements the metric string also names: 2-bit 32k decode, quantise GB/s,
+    VQ assignment MFMA utilisation.  Each is an event-timed loop of one kernel."""
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+    ex = {}
+    D, Hq, Hkv = 128, 32, 8
+    for B in (1, 16):
+        cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=2, kivi_group_size=32, residual_length=128,
+                            fused_sdpa=True, fused_sdpa_memory_bound=True)
+        c = KVCacheFactory.create(cfg)
+        for s0 in range(0, 32768 + 128, 8192):
+            n = min(8192, 32768 + 128 - s0)
+            k, v = _synthetic_layer(torch, B, Hkv, n, D, 5 + s0, dev)
+            c.update_and_fetch(k, v)
+        q = torch.randn((B, Hq, 1, D), device=dev).to(torch.float16)
+        fn = lambda: c.fused_sdpa(q, 1 / math.sqrt(D))
+        for _ in range(3):
+            fn()
+        ms = _event_ms(fn, 30, torch)
+        nbytes = _algorithmic_bytes_per_layer(B, Hkv, 32768, D, 2, 32)
+        ex[f"decode_2bit_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
+                                        "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}
+        del c
+    # config 0: quantise + pack of one layer's K and V [1,8,2048,128], 4-bit, group 32; and a large flush
+    for name, shape in (("cfg0_[1,8,2048,128]", (1, 8, 2048, 128)), ("large_[16,8,8192,128]", (16, 8, 8192, 128))):
+        k, v = _synthetic_layer(torch, shape[0], shape[1], shape[2], shape[3], 11, dev)
+        def qp():
+            K.kivi_quant_pack(k, -2, 32, 4)
+            K.kivi_quant_pack(v, -1, 32, 4, v_layout="token")
+        def rt():
+            K.kivi_group_quant_dequant(k, -2, 32, 15)
+            K.kivi_group_quant_dequant(v, -1, 32, 15)
+        for _ in range(3):
+            qp(); rt()
+        n = k.numel()
+        b_qp = 2 * (n * 2 + n // 2 + (n // 32) * 4)
+        b_rt = 2 * (n * 2 + n * 2)
+        ms_qp, ms_rt = _event_ms(qp, 30, torch), _event_ms(rt, 30, torch)
+        ex[f"quant_pack_{name}"] = {"ms": round(ms_qp, 5), "GBps": round(b_qp / ms_qp / 1e6, 1), "bytes": b_qp}
+        ex[f"quant_dequant_{name}"] = {"ms": round(ms_rt, 5), "GBps": round(b_rt / ms_rt / 1e6, 1), "bytes": b_rt}
+    # config 2: VQ assignment, keys [4,4096,256], 256 centroids x 8 dims
+    x = (torch.randn((4, 4096, 256), device=dev) * torch.exp(torch.randn(256, device=dev))).to(torch.float16)
+    cb = torch.randn((256, 8), device=dev).to(torch.float16)
+    fn = lambda: K.vecinfer_quantize_metal(x, cb, 8, index_dtype=torch.uint8)
+    for _ in range(3):
+        fn()
+    ms = _event_ms(fn, 20, torch)
+    flops = 2 * 524288 * 256 * 8
+    ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
+                            "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
+    return ex
+
+
+def _cpu_baseline(np, torch, cache, q_layer, ctx, Hkv, D, bits, g, scale):
+    """Scalar C oracle (one thread) on one sequence of one layer: dequantise each
+    slot and attend, the same arithmetic the GPU step does for that slice."""
+    from oracle import cref, kivi as ok
+    n = ctx
+    kp = cache._kp[:1, :, :n].cpu().numpy().view(np.uint32)
+    codes_k = ok.unpack_indices(kp, bits, D)
+    ks = cache._ks[:1, :, : n // g].float().cpu().numpy()
+    kz = cache._kz[:1, :, : n // g].float().cpu().numpy()
+    per = 32 // bits
+    vp = cache._vp[:1, :, : n // per].cpu().numpy().view(np.uint32)       # [1,H,n/per,D]
+    codes_v = ok.unpack_indices(np.ascontiguousarray(vp.swapaxes(-1, -2)), bits, n).swapaxes(-1, -2)
+    vs = np.ascontiguousarray(cache._vs[:1, :, :, :n].float().cpu().numpy().swapaxes(-1, -2))
+    vz = np.ascontiguousarray(cache._vz[:1, :, :, :n].float().cpu().numpy().swapaxes(-1, -2))
+    qn = q_layer[:1].float().cpu().numpy()
+    cref.lib()
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 10.0:
+        cref.attend(qn, codes_k, ks, kz, np.ascontiguousarray(codes_v), vs, vz, g, scale)
+        reps += 1
+    dt = (time.perf_counter() - t0) / reps
+    nbytes = _algorithmic_bytes_per_layer(1, Hkv, ctx, D, bits, g)
+    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"one sequence of one layer ({Hkv} kv heads x {ctx} tokens, 32 query heads), scalar C oracle "
+                      f"oracle/c/kv_oracle.c:kvo_attend, {reps} repetitions, {dt:.3f} s each"}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -221,6 +221,12 @@ class KIVIKVCache(FP16KVCache):
                 self._tail_k[:, :, :keep] = self._tail_k[:, :, n_quant_now:need].clone()
                 self._tail_v[:, :, :keep] = self._tail_v[:, :, n_quant_now:need].clone()
             self._n_quantized = new_boundary
+            # a large prefill chunk leaves an oversized tail buffer behind: give it back
+            floor_cap = -(-(self._residual_length + 2 * self._group_size) // 64) * 64
+            if self._tail_k.shape[2] > max(floor_cap, 4 * keep):
+                cap = max(floor_cap, -(-2 * keep // 64) * 64)
+                self._tail_k = self._tail_k[:, :, :cap].clone()
+                self._tail_v = self._tail_v[:, :, :cap].clone()
         self._account_bytes(B, H, S, D, n_quant_now)
         z = torch.zeros((), dtype=keys.dtype, device=keys.device)
         return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
