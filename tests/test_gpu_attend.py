@@ -119,7 +119,7 @@ def test_future_keys_do_not_leak_into_earlier_rows():
 
 # ------------------------------------------------------------ packed cache path
 def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, causal=False, seed=0,
-                 q_dtype=torch.float16, cap_extra=0):
+                 q_dtype=torch.float16, cap_extra=0, expect_path=None):
     require_gpu()
     per = 32 // b
     k, v = outlier_kv((B, Hkv, n_packed + n_tail, D), seed=seed)
@@ -154,11 +154,15 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
         ref_args = [kc, ksn.astype(npm), kzn.astype(npm), vc, vsn.astype(npm), vzn.astype(npm)]
     tail_k = kt[:, :, n_packed:].contiguous() if n_tail else None
     tail_v = vt[:, :, n_packed:].contiguous() if n_tail else None
+    plan = {}
     out = K.kivi_packed_attend(qt, n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k,
                                v_tail=tail_v, n_tail=n_tail, scale=scale, causal=causal,
-                               out_dtype=torch.float32, **kw)
+                               out_dtype=torch.float32, _plan_out=plan, **kw)
+    if expect_path is not None:
+        assert plan["path"] == expect_path, plan
     ref = oa.kivi_attend(host(qt), *ref_args, g, k[:, :, n_packed:], v[:, :, n_packed:], scale, causal=causal)
     err = float(np.max(np.abs(host(out) - ref)))
+    print(f"max-abs err {err:.2e} (path {plan['path']}, {plan['nparts']} partials)")
     assert err < TOL, err
     return err
 
@@ -167,13 +171,15 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
 @pytest.mark.parametrize("b,g", [(2, 32), (4, 64), (4, 32), (2, 64)])
 @pytest.mark.parametrize("meta", [torch.float16, torch.float32])
 def test_packed_decode_with_tail(v_layout, b, g, meta):
-    _packed_case(2, 8, 2, 512, 37, 128, b, g, v_layout, meta, seed=b + g)
+    _packed_case(2, 8, 2, 512, 37, 128, b, g, v_layout, meta, seed=b + g,
+                 expect_path=1 if v_layout == "token" else 0)
 
 
 @pytest.mark.parametrize("v_layout", ["channel", "token"])
 def test_packed_decode_config1_llama_shape(v_layout):
     """32 query heads / 8 kv heads, 8192 tokens 2-bit group 32 + 128-token fp16 tail."""
-    _packed_case(1, 32, 8, 8192, 128, 128, 2, 32, v_layout, torch.float16, seed=1)
+    _packed_case(1, 32, 8, 8192, 128, 128, 2, 32, v_layout, torch.float16, seed=1,
+                 expect_path=1 if v_layout == "token" else 0)
 
 
 def test_packed_decode_no_tail_and_spare_capacity():
@@ -203,3 +209,40 @@ def test_attend_errors():
         K.scalar_fused_decode_attend(q[0], kc, m, m, kc, mv, mv, 32, 0.1)
     with pytest.raises(ValueError, match="nsg=40 must be in 1..32"):
         K.scalar_fused_decode_attend(q, kc, m, m, kc, mv, mv, 32, 0.1, nsg=40)
+
+
+@pytest.mark.parametrize("b,g", [(2, 32), (4, 64), (4, 128), (2, 128)])
+@pytest.mark.parametrize("Hq,Hkv", [(8, 8), (16, 2), (32, 8), (12, 4)])
+def test_mfma_decode_head_ratios_and_groups(b, g, Hq, Hkv):
+    """GQA ratios 1, 8, 4, 3 through the MFMA kernel (ratios above 8 take the vector kernel)."""
+    _packed_case(2, Hq, Hkv, 1024, 0, 128, b, g, "token", torch.float16, seed=Hq + g + b, expect_path=1)
+
+
+def test_mfma_decode_many_splits_and_single_unit():
+    _packed_case(1, 4, 1, 32, 3, 128, 4, 32, "token", torch.float16, seed=2, expect_path=1)
+    _packed_case(1, 4, 1, 4096, 200, 128, 2, 64, "token", torch.float32, seed=3, expect_path=1)
+    _packed_case(1, 32, 2, 256, 0, 128, 4, 64, "token", torch.float16, seed=4, expect_path=0)   # ratio 16
+
+
+def test_mfma_decode_peaked_attention():
+    """One key aligned with the query dominates the softmax: rounding of the
+    reconstruction is not averaged away."""
+    require_gpu()
+    rng = np.random.default_rng(5)
+    B, Hq, Hkv, S, D, b, g = 1, 8, 2, 512, 128, 4, 32
+    k, v = outlier_kv((B, Hkv, S, D), seed=6)
+    q = np.repeat(k[:, :, 100:101].astype(np.float32), 4, axis=1) * 0.5
+    q = q.astype(np.float16)
+    kp, ks, kz = K.kivi_quant_pack(to_dev(k), -2, g, b)
+    vp, vs, vz = K.kivi_quant_pack(to_dev(v), -1, g, b, v_layout="token")
+    plan = {}
+    out = K.kivi_packed_attend(to_dev(q), k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz,
+                               n_packed=S, bits=b, group_size=g, v_layout="token", scale=1 / math.sqrt(D),
+                               out_dtype=torch.float32, _plan_out=plan)
+    kq = ok.group_quant_codes(k, -2, g, 15)
+    vq = ok.group_quant_codes(v, -1, g, 15)
+    h = lambda a: a.astype(np.float16)
+    ref = oa.kivi_attend(q, kq[0], h(kq[1]), h(kq[2]), vq[0], h(vq[1]), h(vq[2]), g, None, None, 1 / math.sqrt(D))
+    err = float(np.max(np.abs(host(out) - ref)))
+    print(f"peaked: max-abs err {err:.2e}, max |out| {np.abs(ref).max():.2f}")
+    assert plan["path"] == 1 and err < TOL

@@ -6,21 +6,23 @@ namespace vq {
 
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
-    const int64_t n_total = a.n_packed + a.n_tail;
-    const int64_t max_splits = n_total > 0 ? cdiv(n_total, 64) : 1;
     p.path = mfma_decode_supported(a) ? 1 : 0;
+    // tokens the main kernel splits: the MFMA path gives the tail its own block
+    const int64_t n_split = p.path == 1 ? a.n_packed : a.n_packed + a.n_tail;
+    const int64_t max_splits = n_split > 0 ? cdiv(n_split, 64) : 1;
     // units of parallel work before splitting: a wave per query row (generic)
     // or a four-wave block per kv head (MFMA)
     const int64_t units = p.path == 1 ? a.B * a.Hkv : a.B * a.Hq * a.Sq;
-    const int64_t target = p.path == 1 ? 1024 : 4096;
+    const int64_t target = p.path == 1 ? 512 : 4096;
     int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);
     if (ns > max_splits) ns = max_splits;
     if (ns > 512) ns = 512;
     if (ns < 1) ns = 1;
-    int64_t len = cdiv(cdiv(n_total > 0 ? n_total : 1, ns), 64) * 64;
-    ns = n_total > 0 ? cdiv(n_total, len) : 1;
+    int64_t len = cdiv(cdiv(n_split > 0 ? n_split : 1, ns), 64) * 64;
+    ns = n_split > 0 ? cdiv(n_split, len) : 1;
     p.nsplit = (int)ns;
     p.split_len = len;
+    p.nparts = p.nsplit + ((p.path == 1 && a.n_tail > 0) ? 1 : 0);
     return p;
 }
 
@@ -62,7 +64,16 @@ using namespace vq;
 extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
     if (!a) return 0;
     AttendPlan p = plan_attend(*a);
-    return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nsplit * (size_t)(a->D + 2) * sizeof(float);
+    return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nparts * (size_t)(a->D + 2) * sizeof(float);
+}
+
+extern "C" int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts) {
+    int rc = validate(a, "vq_kivi_attend_plan");
+    if (rc != VQ_OK) return rc;
+    AttendPlan p = plan_attend(*a);
+    if (path) *path = p.path;
+    if (nparts) *nparts = p.nparts;
+    return VQ_OK;
 }
 
 extern "C" int vq_kivi_attend(const vq_attend_args *a) {
@@ -82,7 +93,7 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a) {
     else rc = launch_attend_generic(*a, p.nsplit, p.split_len);
     if (rc != VQ_OK) return rc;
     VQ_HIP_CHECK_LAUNCH(fn);
-    rc = launch_attend_merge(*a, p.nsplit);
+    rc = launch_attend_merge(*a, p.nparts);
     VQ_HIP_CHECK_LAUNCH(fn);
     return rc;
 }

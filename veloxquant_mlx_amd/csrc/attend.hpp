@@ -6,7 +6,8 @@ namespace vq {
 
 struct AttendPlan {
     int path;           // 0 generic waves, 1 MFMA decode
-    int nsplit;         // partials per query row
+    int nsplit;         // splits along the tokens the main kernel covers
+    int nparts;         // partials per query row handed to the merge kernel
     int64_t split_len;  // tokens per split (multiple of 64)
 };
 
@@ -15,7 +16,7 @@ struct AttendPlan {
 AttendPlan plan_attend(const vq_attend_args &a);
 
 int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len);
-int launch_attend_merge(const vq_attend_args &a, int nsplit);
+int launch_attend_merge(const vq_attend_args &a, int nparts);
 
 // MFMA decode path (attend_mfma.hip)
 bool mfma_decode_supported(const vq_attend_args &a);

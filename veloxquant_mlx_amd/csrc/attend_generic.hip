@@ -138,13 +138,13 @@ int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len
     return VQ_OK;
 }
 
-int launch_attend_merge(const vq_attend_args &a, int nsplit) {
+int launch_attend_merge(const vq_attend_args &a, int nparts) {
     hipStream_t st = (hipStream_t)a.stream;
     const int64_t rows = a.B * a.Hq * a.Sq;
     int64_t g = cdiv(rows * a.D, 256);
     if (g > (1 << 20)) g = 1 << 20;
     hipLaunchKernelGGL(attend_merge_kernel, dim3((unsigned)g), dim3(256), 0, st, (const float *)a.workspace, rows,
-                       nsplit, a.D, a.out, a.out_dtype);
+                       nparts, a.D, a.out, a.out_dtype);
     return VQ_OK;
 }
 

@@ -370,7 +370,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
                        v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
                        scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
-                       num_splits: int = 0) -> torch.Tensor:
+                       num_splits: int = 0, _plan_out: dict | None = None) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
     q ``[B,Hq,Sq,D]``; packed buffers as :func:`kivi_quant_pack` lays them out
@@ -435,6 +435,11 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
     lib = _lib.load()
+    if _plan_out is not None:
+        import ctypes
+        pth, npt = ctypes.c_int(0), ctypes.c_int(0)
+        _lib.check(lib.vq_kivi_attend_plan(a, ctypes.byref(pth), ctypes.byref(npt)))
+        _plan_out["path"], _plan_out["nparts"] = pth.value, npt.value
     need = lib.vq_kivi_attend_workspace(a)
     ws = _workspace(q.device, need)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
