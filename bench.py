@@ -43,6 +43,8 @@ def _parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extras", action="store_true", help="skip the per-kernel side measurements")
     p.add_argument("--only-kernel", action="store_true", help="time the attention kernel loop only (profiling)")
+    p.add_argument("--copy-calib", action="store_true",
+                   help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
 
 
@@ -89,6 +91,13 @@ def main() -> int:
         return 1
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if a.copy_calib:
+        src = torch.arange(1 << 29, device=dev, dtype=torch.int32).view(torch.float16)  # 2 GiB, read half
+        dst = torch.empty(1 << 29, device=dev, dtype=torch.float16)                     # 1 GiB written
+        ms = _event_ms(lambda: dst.copy_(src[: 1 << 29]), 5, torch)
+        print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "ms": ms,
+                          "GBps": (2 << 30) / ms / 1e6}))
+        return 0
     NL, B, Hq, Hkv, D, ctx, bits, g = a.layers, a.batch, 32, 8, 128, a.ctx, a.bits, a.group
     R = 128
     scale = 1.0 / math.sqrt(D)
@@ -147,9 +156,14 @@ def main() -> int:
     # ---- roofline of the dominant kernel (attention), events on the launch stream
     kern_ms = _event_ms(attend_only, max(3, a.steps // 2), torch) / NL
     achieved = layer_bytes / (kern_ms * 1e-3) / 1e9
+    # HBM bytes one attention call moved under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated against
+    # a 1 GiB device copy: x2.000 and x1.000), summed over its three kernels; measured at the default
+    # workload only (profiles/attend_mfma_decode_4bit_cfg3_hbm_traffic.md)
+    default_workload = (B, ctx, bits, g) == (16, 32768, 4, 64)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "attention over packed cache (one layer: attend + split merge)",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 620066816 if default_workload else None,
+                "kernel": "vq_kivi_attend, one layer = 3 launches (fp16 tail, packed prefix "
+                          "attend_mfma_decode_kernel, split merge); the prefix kernel is ~90% of it",
                 "bytes_per_launch": layer_bytes, "ms_per_launch": round(kern_ms, 5)}
 
     out = {
