@@ -1,0 +1,484 @@
+// MFMA decode attention over the packed prefix of a KIVI cache (gfx950, wave64).
+//
+// One block of four waves per (kv head, token split).  Every wave streams units of
+// 32 tokens and never reconstructs a key or a value: both products run on the raw
+// codes, which are dropped from the packed word into the mantissa of an fp16
+// constant by one and-or per two codes (value = offset + code, exact), and every
+// affine term is pushed onto the matrix unit:
+//
+//   scores   S^T[token, row] = sum_d (off + c_td) (q s)_d          A = codes, B = folded query
+//                            + sum_d z_d q_d - off * sum_d (q s)_d   the accumulator the product starts from
+//   output   O[row, chan]    = sum_t (P s_g)[row, t] (off + c_t,chan)     A = P scaled per channel group
+//                            - off * sum_t (P s_g)[row, t]           extra tile against ones, same A
+//                            + sum_t P[row, t] z_g[t]                extra tile, B = value zeros
+//   denominator               sum_t P[row, t]                        extra tile against ones
+//
+// Keys (per-channel scale s_d, zero z_d per token group): the scale is folded into
+// the query, carried as an fp16 high part in columns [0, R) of the 16-wide tile and
+// the exact fp16 remainder in columns [R, 2R), so the product is as accurate as a
+// float32 one although keys carry outlier channels; the two columns are added with
+// one DPP add per score.  The per-group row bias is itself a small MFMA chain
+// (A = the group's zeros / a constant -off, B = the query) whose result seeds the
+// score accumulators, so opening a token group costs no reductions.
+//
+// Values (per-token scale s_g[t], zero z_g[t] per channel group g): the scale is
+// folded into the probabilities, one fp16 multiply per two tokens per group.  A
+// value tile covers 16 consecutive channels, which lie in one group.
+//
+// Query rows (the H_q/H_kv heads sharing the kv head) sit in the 16-wide M/N
+// dimension.  Keys are packed along channels, so a lane's eight k-slots of the
+// first product are eight channels of one token; values are packed along tokens
+// (VQ_V_TOKEN_PACKED), so a lane's eight k-slots of the second product are eight
+// tokens of one channel; token rows of the two score tiles interleave so that the
+// accumulator layout of S^T is the A-operand layout of P.
+//
+// Loads run one unit ahead in registers (two unit buffers used alternately); the
+// softmax keeps a lazily updated reference maximum, so the common path has no
+// cross-lane traffic at all.
+#pragma once
+#include "attend_mfma.hpp"
+
+namespace vq {
+
+#define VQ_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16((A), (B), (C), 0, 0, 0)
+
+// ---- value scale / zero of a lane's eight tokens (tA..tA+3, tB..tB+3)
+template <typename M> struct TokMeta;
+template <> struct TokMeta<f16> {
+    uint2 a, b;
+    __device__ __forceinline__ void load(const char *base, u32 off, u32 gap_bytes) {
+        a = ldg<uint2>(base, off);
+        b = ldg<uint2>(base + gap_bytes, off);
+    }
+    // k-slot pair p = (token tA + p, token tB + p)
+    __device__ __forceinline__ u32 pair(int p) const {
+        const u32 x = p < 2 ? a.x : a.y, y = p < 2 ? b.x : b.y;
+        return (p & 1) ? pair_hi(x, y) : pair_lo(x, y);
+    }
+};
+template <> struct TokMeta<float> {
+    float4 a, b;
+    __device__ __forceinline__ void load(const char *base, u32 off, u32 gap_bytes) {
+        a = ldg<float4>(base, off);
+        b = ldg<float4>(base + gap_bytes, off);
+    }
+    __device__ __forceinline__ float lo(int p) const { return p == 0 ? a.x : p == 1 ? a.y : p == 2 ? a.z : a.w; }
+    __device__ __forceinline__ float hi(int p) const { return p == 0 ? b.x : p == 1 ? b.y : p == 2 ? b.z : b.w; }
+};
+
+// ---- key scale / zero of a lane's 32 channels for one token group, memory order
+template <typename M> struct ChanMeta;
+template <> struct ChanMeta<f16> {
+    uint4 s[4], z[4];
+    __device__ __forceinline__ void load(const char *sb, const char *zb, u32 off) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            s[j] = ldg<uint4>(sb + 16 * j, off);
+            z[j] = ldg<uint4>(zb + 16 * j, off);
+        }
+    }
+    __device__ __forceinline__ u32 sword(int w) const {   // channels 2w, 2w+1
+        const uint4 &q = s[w / 4];
+        return w % 4 == 0 ? q.x : w % 4 == 1 ? q.y : w % 4 == 2 ? q.z : q.w;
+    }
+    // {scale[lo], scale[hi]} for two channels of equal parity
+    __device__ __forceinline__ u32 spair(int lo, int hi) const {
+        return (lo & 1) ? pair_hi(sword(lo / 2), sword(hi / 2)) : pair_lo(sword(lo / 2), sword(hi / 2));
+    }
+};
+template <> struct ChanMeta<float> {
+    float4 s[8], z[8];
+    __device__ __forceinline__ void load(const char *sb, const char *zb, u32 off) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            s[j] = ldg<float4>(sb + 16 * j, off);
+            z[j] = ldg<float4>(zb + 16 * j, off);
+        }
+    }
+    static __device__ __forceinline__ float pick(const float4 &q, int e) { return e == 0 ? q.x : e == 1 ? q.y : e == 2 ? q.z : q.w; }
+    __device__ __forceinline__ float sval(int ch) const { return pick(s[ch / 4], ch % 4); }
+    __device__ __forceinline__ float zval(int ch) const { return pick(z[ch / 4], ch % 4); }
+};
+
+// Per-wave state of the packed kernel.  GV = channel groups per value row.
+template <int GV> struct PackedAcc {
+    f32x4 O[8];     // tile nt: channels 16*nt + n, still carrying off * Off[group]
+    f32x4 Off[GV];  // sum_t (P s_g)[row, t], every column alike
+    f32x4 Z;        // column g < GV: sum_t P[row, t] z_g[t]
+    f32x4 L;        // sum_t P[row, t], every column alike
+    float m_run;    // softmax reference, log2 domain, per lane column (query row)
+};
+
+template <int BITS, typename M, int GV> struct PackedUnit {
+    u32 kw[2][(MF_D * BITS / 32) / 4];   // key words of the lane's 32 channels, two token rows
+    u32 vw[8];                           // value words, one per 16-channel tile
+    TokMeta<M> s[GV];                    // value scales of the lane's eight tokens, every group
+    TokMeta<M> z;                        // value zeros of the lane's eight tokens, group n % GV
+};
+
+// LDS image of the query, three operand forms of 4 k-steps x 64 lanes each:
+//   [0..3]  memory order, rows < R only            (B operand of the zero-point product)
+//   [4..7]  k-slot pair order, +q in columns [0,R), -q in columns [R,2R)
+//   [8..11] k-slot pair order, q in columns [R,2R) only
+// so that  t = [4..7] * s  and  fma([8..11], s, t)  give the rounded product in the
+// high columns and its exact remainder in the low columns without a select.
+constexpr int MF_QIMG = 12 * 64;
+
+template <int BITS>
+__device__ __forceinline__ void build_query_image(const vq_attend_args &a, int64_t row0, int R, int tid, f16 *s_qraw,
+                                                  uint4 *s_q) {
+    for (int e = tid; e < MF_ROWS * MF_D; e += 256) {
+        const int row = e / MF_D, d = e % MF_D;
+        s_qraw[e] = row < R ? (f16)ldq(a.q, a.q_dtype, (row0 + row) * MF_D + d) : (f16)0.f;
+    }
+    __syncthreads();
+    for (int e = tid; e < MF_QIMG; e += 256) {
+        const int form = e / 256, ks = (e / 64) % 4, l = e % 64;
+        const int n = l & 15, blk = l >> 4;
+        const int rq = n < R ? n : n - R;
+        const bool hi_col = n < R, lo_col = n >= R && n < 2 * R;
+        f16 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            int ch;
+            if (form == 0) ch = 8 * ks + j;
+            else ch = (j & 1) ? kchan_hi<BITS>(ks, j >> 1) : kchan_lo<BITS>(ks, j >> 1);
+            const f16 q = (hi_col || lo_col) ? s_qraw[rq * MF_D + 32 * blk + ch] : (f16)0.f;
+            f16 x;
+            if (form == 0) x = hi_col ? q : (f16)0.f;
+            else if (form == 1) x = hi_col ? q : -q;
+            else x = lo_col ? q : (f16)0.f;
+            v[j] = x;
+        }
+        f16x8 o = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]};
+        s_q[e] = __builtin_bit_cast(uint4, o);
+    }
+    __syncthreads();
+}
+
+template <int BITS, typename M, int GV>
+__device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, int R, float c, int64_t t_begin,
+                                             int n_units, int lane, int wave, PackedAcc<GV> &acc, const uint4 *s_q) {
+    constexpr int PER = 32 / BITS;           // codes per word
+    constexpr int KW = MF_D / PER;           // key words per token row
+    constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
+    constexpr int GAP = vtok_gap<BITS>();
+    constexpr int G = MF_D / GV;             // tokens per key group = channels per value group
+    constexpr int TPG = 8 / GV;              // value tiles per channel group
+    constexpr u32 MSZ = sizeof(M);
+    const int n = lane & 15, blk = lane >> 4;
+    const u32 magic = vreg_const(Magic<BITS>::bits);
+    const int64_t cap = a.cap_tokens;
+
+    const int per_wave = (n_units + 3) / 4;
+    const int u0 = wave * per_wave;
+    const int u1 = u0 + per_wave < n_units ? u0 + per_wave : n_units;
+    if (u0 >= u1) return;
+
+    // block-uniform bases, 32-bit per-lane byte offsets
+    const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
+    const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
+    const char *ksb = (const char *)a.k_scale + bh * (cap / G) * MF_D * MSZ;
+    const char *kzb = (const char *)a.k_zero + bh * (cap / G) * MF_D * MSZ;
+    const char *vsb = (const char *)a.v_scale + bh * GV * cap * MSZ;
+    const char *vzb = (const char *)a.v_zero + bh * GV * cap * MSZ;
+    // token of S^T row n in tile T: vtok_lo(n / 4, n % 4) + T * GAP
+    const u32 koff = (u32)((vtok_lo<BITS>(n >> 2, n & 3) * KW + KWL * blk) * 4);
+    const u32 voff = (u32)(((BITS == 4 ? blk : blk / 2) * MF_D + n) * 4);
+    const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
+    const u32 vsoff = (u32)vtok_lo<BITS>(blk, 0) * MSZ;
+    const u32 vzoff = (u32)(((int64_t)(n % GV) * cap + vtok_lo<BITS>(blk, 0)) * MSZ);
+    const u32 kmoff = 32u * blk * MSZ;
+
+    using Unit = PackedUnit<BITS, M, GV>;
+    auto load_unit = [&](int u, Unit &d) {
+        const int64_t base = t_begin + (int64_t)u * 32;
+        const char *kp = kb + base * KW * 4;
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            if (BITS == 4) {
+                uint4 x = ldg<uint4>(kp + T * GAP * KW * 4, koff);
+                d.kw[T][0] = x.x; d.kw[T][1] = x.y; d.kw[T][KWL - 2] = x.z; d.kw[T][KWL - 1] = x.w;
+            } else {
+                uint2 x = ldg<uint2>(kp + T * GAP * KW * 4, koff);
+                d.kw[T][0] = x.x; d.kw[T][KWL - 1] = x.y;
+            }
+        }
+        const char *vp = vb + (base / PER) * MF_D * 4;
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) d.vw[nt] = ldg<u32>(vp + 64 * nt, voff);
+#pragma unroll
+        for (int g = 0; g < GV; ++g) d.s[g].load(vsb + ((int64_t)g * cap + base) * MSZ, vsoff, GAP * MSZ);
+        d.z.load(vzb + base * MSZ, vzoff, GAP * MSZ);
+    };
+
+    f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
+    f32x4 bias;    // what the score accumulators start from; every register alike
+    const f16x8 ones = ones8();
+    const f16x8 negoff = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair,
+                               Magic<BITS>::neg_off_pair);
+
+    auto open_group = [&](const ChanMeta<M> &km) {
+        f32x4 bt = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (sizeof(M) == 2) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) bt = VQ_MFMA(as_h8(km.z[ks]), as_h8(s_q[ks * 64 + lane]), bt);
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const uint4 qs = s_q[(4 + ks) * 64 + lane], ql = s_q[(8 + ks) * 64 + lane];
+                const u32 qsw[4] = {qs.x, qs.y, qs.z, qs.w}, qlw[4] = {ql.x, ql.y, ql.z, ql.w};
+                u32 o[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const f16x2 sp = as_h2(km.spair(kchan_lo<BITS>(ks, p), kchan_hi<BITS>(ks, p)));
+                    const f16x2 t = as_h2(qsw[p]) * sp;   // +round(q s) | -round(q s)
+                    // q*s has at most 22 significant bits: the remainder after the fp16
+                    // high part is itself an fp16 number, so this fma is exact
+                    o[p] = as_u(__builtin_elementwise_fma(as_h2(qlw[p]), sp, t));
+                }
+                qB[ks] = as_h8(o[0], o[1], o[2], o[3]);
+            }
+        } else {
+            // float32 scale / zero: zeros split into an fp16 pair, the folded query formed
+            // in float32 and split the same way
+            f16x8 zh[4], zl[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float z = km.zval(8 * ks + j);
+                    zh[ks][j] = (f16)z;
+                    zl[ks][j] = (f16)(z - (float)zh[ks][j]);
+                }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const f16x8 qz = as_h8(s_q[ks * 64 + lane]);
+                bt = VQ_MFMA(zh[ks], qz, bt);
+                bt = VQ_MFMA(zl[ks], qz, bt);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const f16x8 qs = as_h8(s_q[(4 + ks) * 64 + lane]);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int ch = (j & 1) ? kchan_hi<BITS>(ks, j >> 1) : kchan_lo<BITS>(ks, j >> 1);
+                    const float qv = n < R ? (float)qs[j] : -(float)qs[j];   // columns >= R hold -q
+                    const float t = qv * km.sval(ch);
+                    const f16 hi = (f16)t;
+                    const f16 lo = (f16)(t - (float)hi);
+                    qB[ks][j] = n < R ? hi : lo;
+                }
+            }
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) bt = VQ_MFMA(negoff, qB[ks], bt);
+        bias = bt;
+    };
+
+    // ---- one unit: scores, softmax, output
+    auto compute = [&](const Unit &cur) {
+        f32x4 S[2];
+#pragma unroll
+        for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const u32 w = BITS == 4 ? cur.kw[T][ks] : (cur.kw[T][ks / 2] >> (8 * (ks % 2)));
+                const f16x8 A = unpack8<BITS>(w, magic);
+                S[T] = VQ_MFMA(A, qB[ks], ks == 0 ? bias : S[T]);
+            }
+        // column n < R: add the remainder column n + R; other columns idle
+#define VQ_ADD_SHL(N)                                                                         \
+    _Pragma("unroll") for (int T = 0; T < 2; ++T) _Pragma("unroll") for (int r = 0; r < 4; ++r) \
+        S[T][r] += row_shl<N>(S[T][r]);
+        switch (R) {   // block-uniform
+            case 1: VQ_ADD_SHL(1) break;
+            case 2: VQ_ADD_SHL(2) break;
+            case 4: VQ_ADD_SHL(4) break;
+            case 8: VQ_ADD_SHL(8) break;
+            default:
+#pragma unroll
+                for (int T = 0; T < 2; ++T)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) S[T][r] += __shfl(S[T][r], (lane & ~15) | ((n + R) & 15));
+        }
+#undef VQ_ADD_SHL
+
+        // softmax against a lazily updated reference: the fast path touches no other lane
+        const float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
+                               fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
+        if (__any(mx * c > acc.m_run + RESCALE_SLACK)) {
+            float m_seen = mx * c;
+            m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 16));
+            m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 32));
+            const float m_new = fmaxf(acc.m_run, m_seen);   // finite: scores are finite
+            const float alpha = exp2f(acc.m_run - m_new);   // 0 on the first unit
+            float al[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) acc.O[nt][r] *= al[r];
+#pragma unroll
+                for (int g = 0; g < GV; ++g) acc.Off[g][r] *= al[r];
+                acc.Z[r] *= al[r];
+                acc.L[r] *= al[r];
+            }
+            acc.m_run = m_new;
+        }
+        const float nm = -acc.m_run;
+        float Pf[2][4];
+        u32 P[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            Pf[0][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], c, nm));
+            Pf[1][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], c, nm));
+            P[r] = as_u(f16x2{(f16)Pf[0][r], (f16)Pf[1][r]});
+        }
+        const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
+
+        // output: per channel group, A = P * s_g
+#pragma unroll
+        for (int g = 0; g < GV; ++g) {
+            u32 ag[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                if constexpr (sizeof(M) == 2) ag[p] = as_u(as_h2(P[p]) * as_h2(cur.s[g].pair(p)));
+                else ag[p] = as_u(f16x2{(f16)(Pf[0][p] * cur.s[g].lo(p)), (f16)(Pf[1][p] * cur.s[g].hi(p))});
+            }
+            const f16x8 A = as_h8(ag[0], ag[1], ag[2], ag[3]);
+#pragma unroll
+            for (int j = 0; j < TPG; ++j) {
+                const int nt = g * TPG + j;
+                acc.O[nt] = VQ_MFMA(A, unpack8<BITS>(cur.vw[nt] >> vshift, magic), acc.O[nt]);
+            }
+            acc.Off[g] = VQ_MFMA(A, ones, acc.Off[g]);
+        }
+        if constexpr (sizeof(M) == 2) {
+            acc.Z = VQ_MFMA(P8, as_h8(cur.z.pair(0), cur.z.pair(1), cur.z.pair(2), cur.z.pair(3)), acc.Z);
+        } else {
+            u32 zh[4], zl[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const f16x2 h = {(f16)cur.z.lo(p), (f16)cur.z.hi(p)};
+                zh[p] = as_u(h);
+                zl[p] = as_u(f16x2{(f16)(cur.z.lo(p) - (float)h[0]), (f16)(cur.z.hi(p) - (float)h[1])});
+            }
+            acc.Z = VQ_MFMA(P8, as_h8(zh[0], zh[1], zh[2], zh[3]), acc.Z);
+            acc.Z = VQ_MFMA(P8, as_h8(zl[0], zl[1], zl[2], zl[3]), acc.Z);
+        }
+        acc.L = VQ_MFMA(P8, ones, acc.L);
+    };
+
+    Unit ua, ub;
+    ChanMeta<M> km;
+    int64_t cur_group = (t_begin + (int64_t)u0 * 32) / G;
+    load_unit(u0, ua);
+    km.load(ksb + cur_group * MF_D * MSZ, kzb + cur_group * MF_D * MSZ, kmoff);
+    open_group(km);
+
+    // loads of unit u+1 (and of the next group's key scale / zero when u+1 opens one) are
+    // issued before unit u is computed; past the end the last unit is simply loaded again
+    auto step = [&](const Unit &cur, Unit &nxt, int u) {
+        const int un = u + 1 < u1 ? u + 1 : u;
+        load_unit(un, nxt);
+        const int64_t next_group = (t_begin + (int64_t)un * 32) / G;
+        const bool new_group = next_group != cur_group;
+        if (new_group) km.load(ksb + next_group * MF_D * MSZ, kzb + next_group * MF_D * MSZ, kmoff);
+        compute(cur);
+        if (new_group) {
+            open_group(km);
+            cur_group = next_group;
+        }
+    };
+    for (int u = u0; u < u1; u += 2) {
+        step(ua, ub, u);
+        if (u + 1 < u1) step(ub, ua, u + 1);
+    }
+}
+
+// grid (nsplit, B*Hkv): block x covers tokens [x*split_len, (x+1)*split_len) of the packed prefix
+template <int BITS, typename M, int GV>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int nparts,
+                                                                 float *__restrict__ ws) {
+    __shared__ float s_m[4][MF_ROWS];
+    __shared__ float s_l[4][MF_ROWS];
+    __shared__ float s_z[4][MF_ROWS][4];
+    __shared__ float s_o[4][MF_ROWS][MF_D];
+    __shared__ uint4 s_q[MF_QIMG];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: loops below stay scalar
+    const int n = lane & 15, blk = lane >> 4;
+    const int64_t bh = blockIdx.y;
+    const int sp = (int)blockIdx.x;
+    const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    const int R = (int)(a.Hq / a.Hkv);
+    const int64_t row0 = b * a.Hq + hkv * R;   // first query row of this kv head (Sq == 1)
+    const float c = a.scale * LOG2E;
+
+    // the raw query is staged in the (not yet used) output exchange buffer
+    build_query_image<BITS>(a, row0, R, tid, reinterpret_cast<f16 *>(&s_o[0][0][0]), s_q);
+
+    PackedAcc<GV> acc;
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) acc.O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < GV; ++g) acc.Off[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc.Z = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc.L = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc.m_run = -INFINITY;
+
+    const int64_t t_begin = (int64_t)sp * split_len;
+    int64_t t_end = t_begin + split_len;
+    if (t_end > a.n_packed) t_end = a.n_packed;
+    packed_units<BITS, M, GV>(a, bh, R, c, t_begin, (int)((t_end - t_begin) / 32), lane, wave, acc, s_q);
+
+    // ---- merge the four waves: accumulator register r of lane (n, blk) is row 4*blk + r,
+    // tile nt column n is channel 16*nt + n
+    if (blk == 0) s_m[wave][n] = acc.m_run;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * blk + r;
+        if (row < R) {
+            if (n == 0) s_l[wave][row] = acc.L[r];
+            if (n < GV) s_z[wave][row][n] = acc.Z[r];
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt)
+                s_o[wave][row][16 * nt + n] = acc.O[nt][r] - Magic<BITS>::off * acc.Off[nt / (8 / GV)][r];
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < R * MF_D; e += 256) {
+        const int row = e / MF_D, d = e % MF_D;
+        const float gm = fmaxf(fmaxf(s_m[0][row], s_m[1][row]), fmaxf(s_m[2][row], s_m[3][row]));
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit
+            const float f = exp2f(s_m[w][row] - gm);
+            num += (s_o[w][row][d] + s_z[w][row][d / (MF_D / GV)]) * f;
+            den += s_l[w][row] * f;
+        }
+        float *o = ws + ((row0 + row) * nparts + sp) * MF_PART;
+        o[2 + d] = num;
+        if (d == 0) { o[0] = gm * LN2; o[1] = den; }
+    }
+}
+
+template <typename M>
+static void launch_mfma_packed(const vq_attend_args &a, int nsplit, int64_t split_len, int nparts, float *ws,
+                               hipStream_t st) {
+    const dim3 grid((unsigned)nsplit, (unsigned)(a.B * a.Hkv)), block(256);
+    const int gv = (int)(MF_D / a.group);
+#define VQ_LAUNCH(BITS, GV) \
+    hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, 0, st, a, split_len, nparts, ws)
+    if (a.pack_bits == 4) {
+        if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);
+    } else {
+        if (gv == 1) VQ_LAUNCH(2, 1); else if (gv == 2) VQ_LAUNCH(2, 2); else VQ_LAUNCH(2, 4);
+    }
+#undef VQ_LAUNCH
+}
+
+}  // namespace vq
