@@ -156,6 +156,11 @@ typedef struct vq_attend_args {
     void *workspace;
     size_t workspace_bytes;
     void *stream;
+    /* Optional: B*Hkv int32 counters, all zero when the call is enqueued; the call leaves
+     * them zero.  With them the MFMA decode path finishes in a single launch (the last
+     * block of every kv head merges the split partials); without them (NULL) a separate
+     * merge kernel follows.  Calls sharing counters must not overlap. */
+    int32_t *sync_counters;
 } vq_attend_args;
 
 /* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the

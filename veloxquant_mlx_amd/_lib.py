@@ -35,6 +35,7 @@ class AttendArgs(C.Structure):
         ("n_tail", i64), ("tail_cap", i64),
         ("scale", f32), ("causal", i32), ("num_splits", i32),
         ("workspace", vp), ("workspace_bytes", sz), ("stream", vp),
+        ("sync_counters", vp),
     ]
 
 

@@ -7,8 +7,14 @@ namespace vq {
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
     p.path = mfma_decode_supported(a) ? 1 : 0;
-    // tokens the main kernel splits: the MFMA path gives the tail its own block
-    const int64_t n_split = p.path == 1 ? a.n_packed : a.n_packed + a.n_tail;
+    p.tail_equiv = 0;
+    // tokens the kernel splits: the MFMA path hands the tail to the block of split 0 and
+    // prices a tail token at two packed tokens when it balances the splits
+    int64_t n_split = a.n_packed + a.n_tail;
+    if (p.path == 1) {
+        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 2, 64) * 64 : 0;
+        n_split = a.n_packed + p.tail_equiv;
+    }
     const int64_t max_splits = n_split > 0 ? cdiv(n_split, 64) : 1;
     // units of parallel work before splitting: a wave per query row (generic)
     // or a four-wave block per kv head (MFMA)
@@ -19,7 +25,9 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     if (ns > 512) ns = 512;
     if (ns < 1) ns = 1;
     int64_t len = cdiv(cdiv(n_split > 0 ? n_split : 1, ns), 64) * 64;
-    ns = n_split > 0 ? cdiv(n_split, len) : 1;
+    if (p.tail_equiv > len) p.tail_equiv = len;   // split 0 may end up with the tail only
+    ns = cdiv(a.n_packed + p.tail_equiv > 0 ? a.n_packed + p.tail_equiv : 1, len);
+    if (p.path == 0) ns = n_split > 0 ? cdiv(n_split, len) : 1;
     p.nsplit = (int)ns;
     p.split_len = len;
     p.nparts = p.nsplit + ((p.path == 1 && a.n_tail > 0) ? 1 : 0);
@@ -89,10 +97,15 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a) {
     size_t need = vq_kivi_attend_workspace(a);
     VQ_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, VQ_ERR_WORKSPACE,
                "%s: workspace of %zu bytes required, %zu given", fn, need, a->workspace_bytes);
-    if (p.path == 1) rc = launch_attend_mfma_decode(*a, p.nsplit, p.split_len);
-    else rc = launch_attend_generic(*a, p.nsplit, p.split_len);
-    if (rc != VQ_OK) return rc;
-    VQ_HIP_CHECK_LAUNCH(fn);
+    if (p.path == 1) {
+        const bool merged = launch_attend_mfma_decode(*a, p);
+        VQ_HIP_CHECK_LAUNCH(fn);
+        if (merged) return VQ_OK;
+    } else {
+        rc = launch_attend_generic(*a, p.nsplit, p.split_len);
+        if (rc != VQ_OK) return rc;
+        VQ_HIP_CHECK_LAUNCH(fn);
+    }
     rc = launch_attend_merge(*a, p.nparts);
     VQ_HIP_CHECK_LAUNCH(fn);
     return rc;

@@ -9,7 +9,51 @@ struct AttendPlan {
     int nsplit;         // splits along the tokens the main kernel covers
     int nparts;         // partials per query row handed to the merge kernel
     int64_t split_len;  // tokens per split (multiple of 64)
+    // MFMA path: the block of split 0 also runs the fp16 tail and takes this many fewer
+    // packed tokens (multiple of 64); split s covers packed tokens
+    // [max(0, s*split_len - tail_equiv), min(n_packed, (s+1)*split_len - tail_equiv))
+    int64_t tail_equiv;
 };
+
+// One output element from the split partials of its query row: p points at nparts records
+// of `stride` floats (max in natural-log units, sum, accumulator[D]).  Eight records are
+// fetched at a time with independent loads; DEVICE_SCOPE reads partials that other blocks
+// of the same launch wrote.
+template <bool DEVICE_SCOPE> __device__ __forceinline__ float ld_part(const float *p) {
+    if (DEVICE_SCOPE) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return *p;
+}
+template <bool DEVICE_SCOPE>
+__device__ __forceinline__ float merge_partials(const float *p, int nparts, int64_t stride, int64_t d) {
+    float gm = -INFINITY, num = 0.f, den = 0.f;
+    for (int s0 = 0; s0 < nparts; s0 += 8) {
+        float m[8], l[8], o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float *q = p + (int64_t)(s0 + j < nparts ? s0 + j : s0) * stride;
+            m[j] = ld_part<DEVICE_SCOPE>(q);
+            l[j] = ld_part<DEVICE_SCOPE>(q + 1);
+            o[j] = ld_part<DEVICE_SCOPE>(q + 2 + d);
+        }
+        float cm = gm;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (s0 + j < nparts) cm = fmaxf(cm, m[j]);
+        if (cm == -INFINITY) continue;   // nothing visible so far
+        const float f0 = __expf(gm - cm);   // 0 on the first chunk
+        num *= f0;
+        den *= f0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            if (s0 + j < nparts && m[j] != -INFINITY) {
+                const float f = __expf(m[j] - cm);
+                den += l[j] * f;
+                num += o[j] * f;
+            }
+        gm = cm;
+    }
+    return den > 0.f ? num / den : 0.f;
+}
 
 // Decides kernel and split count from shapes only, so that the workspace query
 // and the launch agree.
@@ -20,6 +64,7 @@ int launch_attend_merge(const vq_attend_args &a, int nparts);
 
 // MFMA decode path (attend_mfma.hip)
 bool mfma_decode_supported(const vq_attend_args &a);
-int launch_attend_mfma_decode(const vq_attend_args &a, int nsplit, int64_t split_len);
+// returns true when the kernel also merged the partials (sync counters were given)
+bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p);
 
 }  // namespace vq

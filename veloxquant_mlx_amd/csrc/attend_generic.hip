@@ -113,19 +113,8 @@ __global__ void attend_merge_kernel(const float *__restrict__ ws, int64_t rows, 
                                     void *__restrict__ out, int out_dtype) {
     const int64_t n = rows * D;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
-        int64_t row = e / D, d = e % D;
-        const float *p = ws + row * nsplit * (D + 2);
-        float gm = -INFINITY;
-        for (int s = 0; s < nsplit; ++s) gm = fmaxf(gm, p[s * (D + 2)]);
-        float den = 0.0f, num = 0.0f;
-        for (int s = 0; s < nsplit; ++s) {
-            float ms = p[s * (D + 2)];
-            if (ms == -INFINITY) continue;
-            float f = __expf(ms - gm);
-            den += p[s * (D + 2) + 1] * f;
-            num += p[s * (D + 2) + 2 + d] * f;
-        }
-        st_tag(out, out_dtype, e, den > 0.0f ? num / den : 0.0f);
+        const int64_t row = e / D, d = e % D;
+        st_tag(out, out_dtype, e, merge_partials<false>(ws + row * nsplit * (D + 2), nsplit, D + 2, d));
     }
 }
 

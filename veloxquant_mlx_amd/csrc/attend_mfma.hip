@@ -1,0 +1,32 @@
+// Shape gate and dispatch of the MFMA decode path (the kernels live in
+// attend_mfma_packed.hpp, instantiated per scale/zero dtype in attend_mfma_packed_*.hip).
+#include "attend_mfma.hpp"
+
+namespace vq {
+
+bool mfma_decode_supported(const vq_attend_args &a) {
+    if (a.D != MF_D || a.Sq != 1 || a.n_packed <= 0) return false;
+    if (a.Hq % a.Hkv != 0 || 2 * (a.Hq / a.Hkv) > MF_ROWS) return false;  // high + remainder columns
+    if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
+    if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
+    if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
+    if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
+    if (a.cap_tokens > (1 << 24)) return false;   // per-lane byte offsets are 32-bit
+    if (!(a.scale > 0.f)) return false;
+    if (a.n_tail > 0 && (a.tail_dtype != VQ_F16 || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
+    if (a.B * a.Hkv > 65535) return false;
+    const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
+                         (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
+    if (al & 15u) return false;
+    return true;
+}
+
+bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p) {
+    hipStream_t st = (hipStream_t)a.stream;
+    float *ws = (float *)a.workspace;
+    if (a.meta_dtype == VQ_F16) launch_mfma_packed_f16meta(a, p, ws, st);
+    else launch_mfma_packed_f32meta(a, p, ws, st);
+    return a.sync_counters != nullptr;
+}
+
+}  // namespace vq

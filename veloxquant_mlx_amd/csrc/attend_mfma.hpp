@@ -104,10 +104,183 @@ template <typename T> __device__ __forceinline__ T ldg(const char *base, u32 off
     return *reinterpret_cast<const T *>(base + off);
 }
 
-// launchers of the two kernels (packed prefix, fp16 tail); each writes (max, sum, accumulator)
-// partials [rows][nparts][MF_PART] that the shared merge kernel combines
-void launch_mfma_tail(const vq_attend_args &a, int nsplit, int nparts, float *ws, hipStream_t st);
-void launch_mfma_packed_f16meta(const vq_attend_args &a, int nsplit, int64_t split_len, int nparts, float *ws, hipStream_t st);
-void launch_mfma_packed_f32meta(const vq_attend_args &a, int nsplit, int64_t split_len, int nparts, float *ws, hipStream_t st);
+
+// ---------------------------------------------------------------------------
+// Un-quantised fp16 tail, run by the four waves of one block in units of 32 tokens:
+//   S^T[token, row] = K[token, :] . q[row, :]          A = K as stored, B = q
+//   O[row, chan]   += P[row, token] * V[token, chan]   A = P, B = V
+// Values are loaded as eight rows of eight channels per lane and transposed in
+// registers into the token-major k-slots.  The softmax denominator is a ninth
+// output tile against a ones operand.  Writes one (max, sum, accumulator) partial
+// per query row into slot `slot` of the partials.
+// ---------------------------------------------------------------------------
+struct TailAcc {
+    f32x4 O[9];
+    float m_run;   // log2 domain, row = lane % 16, replicated over the four lane groups
+};
+
+// token (0..31 inside a unit) of S^T row 4*blk + r of tile T: rows of the two tiles interleave
+// so that accumulator register r of tile T is k-slot pair r of the P.V product
+__device__ __forceinline__ int tail_tok(int blk, int r, int T) { return 8 * blk + r + 4 * T; }
+
+__device__ __forceinline__ f16x8 tail_softmax_unit(const f32x4 (&S)[2], float c, TailAcc &acc, int blk) {
+    float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
+                     fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
+    mx = fmaxf(mx, __shfl_xor(mx, 16));
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_seen = mx * c;
+    if (__any(m_seen > acc.m_run + RESCALE_SLACK)) {
+        const float m_new = fmaxf(acc.m_run, m_seen);
+        const float alpha = m_new == -INFINITY ? 1.f : exp2f(acc.m_run - m_new);   // 0 on the first unit
+        float al[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
+#pragma unroll
+        for (int n = 0; n < 9; ++n)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc.O[n][r] *= al[r];
+        acc.m_run = m_new;
+    }
+    const float mm = acc.m_run == -INFINITY ? 0.f : acc.m_run;   // a row with no visible token yet
+    f16x8 P;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        P[2 * r] = (f16)__builtin_amdgcn_exp2f(S[0][r] * c - mm);
+        P[2 * r + 1] = (f16)__builtin_amdgcn_exp2f(S[1][r] * c - mm);
+    }
+    return P;
+}
+
+// Partials another block will read in this launch go out as device-scope stores (written
+// through to where every compute die sees them); otherwise plain stores.
+__device__ __forceinline__ void st_partial(float *p, float v, bool device_scope) {
+    if (device_scope) __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else *p = v;
+}
+
+// s_m, s_l: [4][MF_ROWS] floats; s_o: [4][MF_ROWS][MF_D] floats of block-shared memory.
+// s_qraw: the query rows of this kv head as fp16 [MF_ROWS][MF_D] (rows >= R zero); it may
+// alias s_o: it is read into registers before s_o is written.
+__device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, int64_t row0, int R, float c, int slot,
+                                           int nparts, float *__restrict__ ws, float *s_m, float *s_l, float *s_o,
+                                           const f16 *s_qraw, int tid, int wave, bool device_scope) {
+    const int lane = tid & 63, i = lane & 15, blk = lane >> 4;
+    TailAcc acc;
+#pragma unroll
+    for (int n = 0; n < 9; ++n) acc.O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+    acc.m_run = -INFINITY;
+
+    const f16 *kt = (const f16 *)a.k_tail + bh * a.tail_cap * MF_D;
+    const f16 *vt = (const f16 *)a.v_tail + bh * a.tail_cap * MF_D;
+    f16x8 qT[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * MF_D + 32 * blk + 8 * ks);
+    __syncthreads();   // s_qraw may alias s_o
+    const f16x8 ones = ones8();
+    const int n_tu = (int)((a.n_tail + 31) / 32);
+
+    struct TUnit { f16x8 kr[2][4], vr[8]; };
+    // every load of a unit is issued before its first product; clamped rows are masked below
+    auto load = [&](int u, TUnit &d) {
+        const int64_t base = (int64_t)u * 32;
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            const int64_t tok = base + tail_tok(i >> 2, i & 3, T);
+            const f16 *p = kt + (tok < a.n_tail ? tok : 0) * MF_D + 32 * blk;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) d.kr[T][ks] = *reinterpret_cast<const f16x8 *>(p + 8 * ks);
+        }
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int64_t tA = base + tail_tok(blk, p, 0), tB = base + tail_tok(blk, p, 1);
+            d.vr[2 * p] = *reinterpret_cast<const f16x8 *>(vt + (tA < a.n_tail ? tA : 0) * MF_D + 8 * i);
+            d.vr[2 * p + 1] = *reinterpret_cast<const f16x8 *>(vt + (tB < a.n_tail ? tB : 0) * MF_D + 8 * i);
+        }
+    };
+    auto compute = [&](int u, const TUnit &d) {
+        const int64_t base = (int64_t)u * 32;
+        f32x4 S[2];
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            S[T] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) S[T] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.kr[T][ks], qT[ks], S[T], 0, 0, 0);
+        }
+#pragma unroll
+        for (int T = 0; T < 2; ++T)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (i < R && base + tail_tok(blk, r, T) >= a.n_tail) S[T][r] = -INFINITY;
+        const f16x8 P = tail_softmax_unit(S, c, acc, blk);
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) {   // lane column i is channel 8*i + nt
+            f16x8 Bv;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) Bv[j] = d.vr[j][nt];
+            acc.O[nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(P, Bv, acc.O[nt], 0, 0, 0);
+        }
+        acc.O[8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(P, ones, acc.O[8], 0, 0, 0);
+    };
+    // two units of a wave in flight at a time
+    for (int u = wave; u < n_tu; u += 8) {
+        TUnit d0, d1;
+        load(u, d0);
+        if (u + 4 < n_tu) load(u + 4, d1);
+        compute(u, d0);
+        if (u + 4 < n_tu) compute(u + 4, d1);
+    }
+
+    // merge the four waves: accumulator register r of lane (i, blk) is row 4*blk + r, channel 8*i + nt
+    if (blk == 0) s_m[wave * MF_ROWS + i] = acc.m_run;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int row = 4 * blk + r;
+        if (row < R) {
+            if (i == 0) s_l[wave * MF_ROWS + row] = acc.O[8][r];
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) s_o[(wave * MF_ROWS + row) * MF_D + 8 * i + nt] = acc.O[nt][r];
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < R * MF_D; e += 256) {
+        const int row = e / MF_D, d = e % MF_D;
+        float gm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) gm = fmaxf(gm, s_m[w * MF_ROWS + row]);
+        float num = 0.f, den = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float mw = s_m[w * MF_ROWS + row];
+            if (mw == -INFINITY) continue;
+            const float f = exp2f(mw - gm);
+            num += s_o[(w * MF_ROWS + row) * MF_D + d] * f;
+            den += s_l[w * MF_ROWS + row] * f;
+        }
+        float *o = ws + ((row0 + row) * nparts + slot) * MF_PART;
+        st_partial(o + 2 + d, num, device_scope);
+        if (d == 0) { st_partial(o, gm * LN2, device_scope); st_partial(o + 1, den, device_scope); }
+    }
+    __syncthreads();   // the exchange buffers are free again
+}
+
+// Combine the nparts partials of query rows [row0, row0 + R) into the output (the
+// arithmetic of attend_merge_kernel, which shares merge_partials).  Partials written by
+// other blocks of this launch are read with device-scope loads.
+__device__ __forceinline__ void merge_rows(const vq_attend_args &a, int64_t row0, int R, int nparts,
+                                           const float *ws, int tid) {
+    for (int e = tid; e < R * MF_D; e += 256) {
+        const int row = e / MF_D, d = e % MF_D;
+        const float v = merge_partials<true>(ws + (row0 + row) * nparts * MF_PART, nparts, MF_PART, d);
+        const int64_t oi = (row0 + row) * MF_D + d;
+        if (a.out_dtype == VQ_F16) ((f16 *)a.out)[oi] = (f16)v;
+        else if (a.out_dtype == VQ_BF16) ((u16 *)a.out)[oi] = f32_to_bf16(v);
+        else ((float *)a.out)[oi] = v;
+    }
+}
+
+// launchers of the packed-prefix kernel (it also runs the fp16 tail and, given sync counters,
+// the final merge); partials are [rows][nparts][MF_PART] floats of (max, sum, accumulator)
+void launch_mfma_packed_f16meta(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_f32meta(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
 
 }  // namespace vq

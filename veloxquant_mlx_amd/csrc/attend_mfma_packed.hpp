@@ -277,6 +277,17 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 
     // ---- one unit: scores, softmax, output
     auto compute = [&](const Unit &cur) {
+#ifdef VQ_EXPERIMENT_LOADS_ONLY
+        if constexpr (sizeof(M) == 2) {
+            u32 x = 0;
+            for (int T = 0; T < 2; ++T) for (int k = 0; k < KWL; ++k) x ^= cur.kw[T][k];
+            for (int nt = 0; nt < 8; ++nt) x ^= cur.vw[nt];
+            for (int g = 0; g < GV; ++g) x ^= cur.s[g].a.x ^ cur.s[g].a.y ^ cur.s[g].b.x ^ cur.s[g].b.y;
+            x ^= cur.z.a.x ^ cur.z.a.y ^ cur.z.b.x ^ cur.z.b.y;
+            acc.L[0] += __builtin_bit_cast(float, x & 0x3fffffffu);
+            return;
+        }
+#endif
         f32x4 S[2];
 #pragma unroll
         for (int T = 0; T < 2; ++T)
@@ -397,28 +408,38 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     }
 }
 
-// grid (nsplit, B*Hkv): block x covers tokens [x*split_len, (x+1)*split_len) of the packed prefix
+// grid (nsplit, B*Hkv).  Block x covers packed tokens
+// [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)); block 0 first
+// runs the fp16 tail, whose partial goes to slot nsplit.  With sync counters the block that
+// finishes last for its kv head merges the nparts partials into the output.
 template <int BITS, typename M, int GV>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int nparts,
-                                                                 float *__restrict__ ws) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts,
+                               float *__restrict__ ws) {
     __shared__ float s_m[4][MF_ROWS];
     __shared__ float s_l[4][MF_ROWS];
     __shared__ float s_z[4][MF_ROWS][4];
     __shared__ float s_o[4][MF_ROWS][MF_D];
     __shared__ uint4 s_q[MF_QIMG];
+    __shared__ int s_ticket;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: loops below stay scalar
     const int n = lane & 15, blk = lane >> 4;
     const int64_t bh = blockIdx.y;
-    const int sp = (int)blockIdx.x;
+    const int sp = (int)blockIdx.x, nsplit = (int)gridDim.x;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
     const int R = (int)(a.Hq / a.Hkv);
     const int64_t row0 = b * a.Hq + hkv * R;   // first query row of this kv head (Sq == 1)
     const float c = a.scale * LOG2E;
 
+    const bool single_launch = a.sync_counters != nullptr;
     // the raw query is staged in the (not yet used) output exchange buffer
-    build_query_image<BITS>(a, row0, R, tid, reinterpret_cast<f16 *>(&s_o[0][0][0]), s_q);
+    f16 *s_qraw = reinterpret_cast<f16 *>(&s_o[0][0][0]);
+    build_query_image<BITS>(a, row0, R, tid, s_qraw, s_q);
+    if (sp == 0 && a.n_tail > 0)
+        tail_block(a, bh, row0, R, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid, wave,
+                   single_launch);
 
     PackedAcc<GV> acc;
 #pragma unroll
@@ -429,10 +450,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     acc.L = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
 
-    const int64_t t_begin = (int64_t)sp * split_len;
+    int64_t t_begin = (int64_t)sp * split_len - tail_equiv;
     int64_t t_end = t_begin + split_len;
+    if (t_begin < 0) t_begin = 0;
     if (t_end > a.n_packed) t_end = a.n_packed;
-    packed_units<BITS, M, GV>(a, bh, R, c, t_begin, (int)((t_end - t_begin) / 32), lane, wave, acc, s_q);
+    const int n_units = t_end > t_begin ? (int)((t_end - t_begin) / 32) : 0;
+    packed_units<BITS, M, GV>(a, bh, R, c, t_begin, n_units, lane, wave, acc, s_q);
 
     // ---- merge the four waves: accumulator register r of lane (n, blk) is row 4*blk + r,
     // tile nt column n is channel 16*nt + n
@@ -461,18 +484,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             den += s_l[w][row] * f;
         }
         float *o = ws + ((row0 + row) * nparts + sp) * MF_PART;
-        o[2 + d] = num;
-        if (d == 0) { o[0] = gm * LN2; o[1] = den; }
+        st_partial(o + 2 + d, num, single_launch);
+        if (d == 0) { st_partial(o, gm * LN2, single_launch); st_partial(o + 1, den, single_launch); }
     }
+
+    // ---- last block of this kv head merges the splits (no block ever waits for another).
+    // Partials travel as device-scope stores and loads, so no cache-wide write-back or
+    // invalidate is needed: the barrier below waits until this block's stores are
+    // acknowledged, then one thread takes a ticket.
+    if (!single_launch) return;
+    __syncthreads();
+    if (tid == 0) s_ticket = __hip_atomic_fetch_add(a.sync_counters + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __syncthreads();
+    if (s_ticket != nsplit - 1) return;
+    merge_rows(a, row0, R, nparts, ws, tid);
+    if (tid == 0) __hip_atomic_store(a.sync_counters + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <typename M>
-static void launch_mfma_packed(const vq_attend_args &a, int nsplit, int64_t split_len, int nparts, float *ws,
-                               hipStream_t st) {
-    const dim3 grid((unsigned)nsplit, (unsigned)(a.B * a.Hkv)), block(256);
+static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
+    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv)), block(256);
     const int gv = (int)(MF_D / a.group);
 #define VQ_LAUNCH(BITS, GV) \
-    hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, 0, st, a, split_len, nparts, ws)
+    hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, 0, st, a, p.split_len, p.tail_equiv, \
+                       p.nparts, ws)
     if (a.pack_bits == 4) {
         if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);
     } else {

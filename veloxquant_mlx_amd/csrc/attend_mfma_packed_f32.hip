@@ -3,9 +3,8 @@
 
 namespace vq {
 
-void launch_mfma_packed_f32meta(const vq_attend_args &a, int nsplit, int64_t split_len, int nparts, float *ws,
-                                hipStream_t st) {
-    launch_mfma_packed<float>(a, nsplit, split_len, nparts, ws, st);
+void launch_mfma_packed_f32meta(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
+    launch_mfma_packed<float>(a, p, ws, st);
 }
 
 }  // namespace vq

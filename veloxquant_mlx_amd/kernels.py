@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import math
 
+import os
 import torch
 
 from . import _lib
@@ -353,6 +354,20 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+_sync_counters: dict[tuple, torch.Tensor] = {}
+
+
+def _counters(device: torch.device) -> torch.Tensor:
+    """Per-(device, stream) int32 counters the single-launch decode path needs: zero when a
+    call is enqueued, left zero by it (65536 = the largest B*H_kv the MFMA path takes)."""
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    c = _sync_counters.get(key)
+    if c is None:
+        c = torch.zeros(65536, dtype=torch.int32, device=device)
+        _sync_counters[key] = c
+    return c
+
+
 def _tail_layout(t: torch.Tensor):
     """Return ``(tensor, capacity)`` for a ``[B,H,n,D]`` tail that is either dense or
     a token slice of a dense ``[B,H,capacity,D]`` buffer (rows dense, uniform head
@@ -370,7 +385,8 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
                        v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
                        scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
-                       num_splits: int = 0, _plan_out: dict | None = None) -> torch.Tensor:
+                       num_splits: int = 0, _plan_out: dict | None = None,
+                       _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
     q ``[B,Hq,Sq,D]``; packed buffers as :func:`kivi_quant_pack` lays them out
@@ -443,6 +459,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     need = lib.vq_kivi_attend_workspace(a)
     ws = _workspace(q.device, need)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.sync_counters = _counters(q.device).data_ptr() if (_single_launch and not os.environ.get('VQ_TWO_LAUNCH')) else None
     a.stream = _stream(q)
     _lib.check(lib.vq_kivi_attend(a))
     return out
