@@ -254,3 +254,30 @@ def test_mfma_decode_peaked_attention():
     err = float(np.max(np.abs(host(out) - ref)))
     print(f"peaked: max-abs err {err:.2e}, max |out| {np.abs(ref).max():.2f}")
     assert plan["path"] == 1 and err < TOL
+
+
+# ------------------------------------------------- multi-query (prefill) on the MFMA path
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (8, 8), (4, 2), (8, 1)])
+@pytest.mark.parametrize("Sq,n_packed,n_tail", [(64, 256, 20), (37, 128, 0), (96, 160, 33)])
+def test_mfma_prefill_causal_edge_inside_packed_prefix(Hq, Hkv, Sq, n_packed, n_tail):
+    """Queries align to the end of the slots, so with a short tail the causal edge of most
+    rows lies inside the packed prefix (the chunked quantise-on-write situation)."""
+    _packed_case(1, Hq, Hkv, n_packed, n_tail, 128, 4, 32, "token", torch.float16, Sq=Sq, causal=True,
+                 seed=Hq + Sq, expect_path=1)
+
+
+@pytest.mark.parametrize("b,g,meta", [(2, 32, torch.float16), (4, 64, torch.float32), (2, 128, torch.float16)])
+def test_mfma_prefill_bits_groups_and_bf16_queries(b, g, meta):
+    _packed_case(2, 8, 2, 512, 70, 128, b, g, "token", meta, Sq=50, causal=True, seed=b + g,
+                 q_dtype=torch.bfloat16, expect_path=1)
+
+
+def test_mfma_prefill_not_causal_and_split_tokens():
+    # every row sees every slot; few row tiles, so the token range is split across blocks
+    _packed_case(1, 8, 2, 2048, 100, 128, 4, 64, "token", torch.float16, Sq=4, causal=False, seed=21, expect_path=1)
+    _packed_case(1, 8, 2, 2048, 100, 128, 4, 64, "token", torch.float16, Sq=6, causal=True, seed=22, expect_path=1)
+
+
+def test_mfma_prefill_odd_head_ratio_takes_vector_kernel():
+    _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=4, causal=True, seed=23, expect_path=0)
+    _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=1, seed=24, expect_path=1)

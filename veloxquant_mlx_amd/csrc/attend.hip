@@ -8,17 +8,21 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
     p.path = mfma_decode_supported(a) ? 1 : 0;
     p.tail_equiv = 0;
+    p.pq = 1;
+    p.tiles = 1;
     // tokens the kernel splits: the MFMA path hands the tail to the block of split 0 and
     // prices a tail token at two packed tokens when it balances the splits
     int64_t n_split = a.n_packed + a.n_tail;
     if (p.path == 1) {
+        p.pq = mfma_positions_per_tile(a);
+        p.tiles = (int)cdiv(a.Sq, p.pq);
         p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 2, 64) * 64 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
     const int64_t max_splits = n_split > 0 ? cdiv(n_split, 64) : 1;
     // units of parallel work before splitting: a wave per query row (generic)
     // or a four-wave block per kv head (MFMA)
-    const int64_t units = p.path == 1 ? a.B * a.Hkv : a.B * a.Hq * a.Sq;
+    const int64_t units = p.path == 1 ? a.B * a.Hkv * p.tiles : a.B * a.Hq * a.Sq;
     const int64_t target = p.path == 1 ? 512 : 4096;
     int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);
     if (ns > max_splits) ns = max_splits;

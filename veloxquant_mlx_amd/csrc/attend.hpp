@@ -13,6 +13,9 @@ struct AttendPlan {
     // packed tokens (multiple of 64); split s covers packed tokens
     // [max(0, s*split_len - tail_equiv), min(n_packed, (s+1)*split_len - tail_equiv))
     int64_t tail_equiv;
+    // MFMA path: a block works on the GQA group of one kv head at pq consecutive query
+    // positions; tiles = ceil(Sq / pq) such blocks per (batch, kv head)
+    int pq, tiles;
 };
 
 // One output element from the split partials of its query row: p points at nparts records
@@ -64,6 +67,7 @@ int launch_attend_merge(const vq_attend_args &a, int nparts);
 
 // MFMA decode path (attend_mfma.hip)
 bool mfma_decode_supported(const vq_attend_args &a);
+int mfma_positions_per_tile(const vq_attend_args &a);
 // returns true when the kernel also merged the partials (sync counters were given)
 bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p);
 

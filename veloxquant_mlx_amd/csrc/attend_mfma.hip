@@ -4,9 +4,20 @@
 
 namespace vq {
 
+// Query positions one block takes: rows = (heads of the GQA group) x positions, at most eight
+// (a high and a remainder column each in the 16-wide tile).
+int mfma_positions_per_tile(const vq_attend_args &a) {
+    const int64_t R = a.Hq / a.Hkv;
+    if (a.Sq == 1) return 1;
+    return (int)(8 / R);
+}
+
 bool mfma_decode_supported(const vq_attend_args &a) {
-    if (a.D != MF_D || a.Sq != 1 || a.n_packed <= 0) return false;
+    if (a.D != MF_D || a.n_packed <= 0) return false;
     if (a.Hq % a.Hkv != 0 || 2 * (a.Hq / a.Hkv) > MF_ROWS) return false;  // high + remainder columns
+    const int64_t R = a.Hq / a.Hkv;
+    if (a.Sq > 1 && !(R == 1 || R == 2 || R == 4 || R == 8)) return false;
+    if (a.B * a.Hkv * cdiv(a.Sq, mfma_positions_per_tile(a)) > 65535) return false;   // grid y, sync counters
     if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
     if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
     if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
@@ -14,7 +25,6 @@ bool mfma_decode_supported(const vq_attend_args &a) {
     if (a.cap_tokens > (1 << 24)) return false;   // per-lane byte offsets are 32-bit
     if (!(a.scale > 0.f)) return false;
     if (a.n_tail > 0 && (a.tail_dtype != VQ_F16 || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
-    if (a.B * a.Hkv > 65535) return false;
     const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
                          (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
     if (al & 15u) return false;

@@ -104,6 +104,22 @@ template <typename T> __device__ __forceinline__ T ldg(const char *base, u32 off
     return *reinterpret_cast<const T *>(base + off);
 }
 
+// The query rows one block works on: RT = R * PQ rows that share a kv head, namely the R
+// heads of the GQA group at PQ consecutive query positions starting at pos0.  Tile row
+// j is head j % R at position pos0 + j / R.  Decode (Sq == 1) is the case PQ == 1.
+struct RowTile {
+    int64_t base_row;   // flattened [B, Hq, Sq] row of (b, first head of the group, position 0)
+    int64_t Sq, n_total;
+    int R, RT, pos0, causal;
+    __device__ __forceinline__ bool valid(int j) const { return j < RT && pos0 + j / R < Sq; }
+    __device__ __forceinline__ int64_t row(int j) const { return base_row + (int64_t)(j % R) * Sq + pos0 + j / R; }
+    // number of visible slots of tile row j (queries align to the end of the slots)
+    __device__ __forceinline__ int64_t visible(int j) const {
+        int64_t pos = pos0 + j / R;
+        if (pos > Sq - 1) pos = Sq - 1;
+        return causal ? n_total - Sq + pos + 1 : n_total;
+    }
+};
 
 // ---------------------------------------------------------------------------
 // Un-quantised fp16 tail, run by the four waves of one block in units of 32 tokens:
@@ -161,10 +177,14 @@ __device__ __forceinline__ void st_partial(float *p, float v, bool device_scope)
 // s_m, s_l: [4][MF_ROWS] floats; s_o: [4][MF_ROWS][MF_D] floats of block-shared memory.
 // s_qraw: the query rows of this kv head as fp16 [MF_ROWS][MF_D] (rows >= R zero); it may
 // alias s_o: it is read into registers before s_o is written.
-__device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, int64_t row0, int R, float c, int slot,
+__device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, const RowTile &tile, float c, int slot,
                                            int nparts, float *__restrict__ ws, float *s_m, float *s_l, float *s_o,
                                            const f16 *s_qraw, int tid, int wave, bool device_scope) {
     const int lane = tid & 63, i = lane & 15, blk = lane >> 4;
+    const int R = tile.RT;
+    // tail tokens this lane's query row sees
+    int64_t n_vis = tile.visible(i < R ? i : 0) - a.n_packed;
+    if (n_vis > a.n_tail) n_vis = a.n_tail;
     TailAcc acc;
 #pragma unroll
     for (int n = 0; n < 9; ++n) acc.O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -210,7 +230,7 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
         for (int T = 0; T < 2; ++T)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                if (i < R && base + tail_tok(blk, r, T) >= a.n_tail) S[T][r] = -INFINITY;
+                if (i < R && base + tail_tok(blk, r, T) >= n_vis) S[T][r] = -INFINITY;
         const f16x8 P = tail_softmax_unit(S, c, acc, blk);
 #pragma unroll
         for (int nt = 0; nt < 8; ++nt) {   // lane column i is channel 8*i + nt
@@ -256,22 +276,25 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
             num += s_o[(w * MF_ROWS + row) * MF_D + d] * f;
             den += s_l[w * MF_ROWS + row] * f;
         }
-        float *o = ws + ((row0 + row) * nparts + slot) * MF_PART;
+        if (!tile.valid(row)) continue;
+        float *o = ws + (tile.row(row) * nparts + slot) * MF_PART;
         st_partial(o + 2 + d, num, device_scope);
         if (d == 0) { st_partial(o, gm * LN2, device_scope); st_partial(o + 1, den, device_scope); }
     }
     __syncthreads();   // the exchange buffers are free again
 }
 
-// Combine the nparts partials of query rows [row0, row0 + R) into the output (the
+// Combine the nparts partials of the tile's query rows into the output (the
 // arithmetic of attend_merge_kernel, which shares merge_partials).  Partials written by
 // other blocks of this launch are read with device-scope loads.
-__device__ __forceinline__ void merge_rows(const vq_attend_args &a, int64_t row0, int R, int nparts,
-                                           const float *ws, int tid) {
-    for (int e = tid; e < R * MF_D; e += 256) {
-        const int row = e / MF_D, d = e % MF_D;
-        const float v = merge_partials<true>(ws + (row0 + row) * nparts * MF_PART, nparts, MF_PART, d);
-        const int64_t oi = (row0 + row) * MF_D + d;
+__device__ __forceinline__ void merge_rows(const vq_attend_args &a, const RowTile &tile, int nparts, const float *ws,
+                                           int tid) {
+    for (int e = tid; e < tile.RT * MF_D; e += 256) {
+        const int j = e / MF_D, d = e % MF_D;
+        if (!tile.valid(j)) continue;
+        const int64_t row = tile.row(j);
+        const float v = merge_partials<true>(ws + row * nparts * MF_PART, nparts, MF_PART, d);
+        const int64_t oi = row * MF_D + d;
         if (a.out_dtype == VQ_F16) ((f16 *)a.out)[oi] = (f16)v;
         else if (a.out_dtype == VQ_BF16) ((u16 *)a.out)[oi] = f32_to_bf16(v);
         else ((float *)a.out)[oi] = v;

@@ -8,7 +8,7 @@
 //
 //   scores   S^T[token, row] = sum_d (off + c_td) (q s)_d          A = codes, B = folded query
 //                            + sum_d z_d q_d - off * sum_d (q s)_d   the accumulator the product starts from
-//   output   O[row, chan]    = sum_t (P s_g)[row, t] (off + c_t,chan)     A = P scaled per channel group
+//   output   O[row, chan]    = sum_t (P s_g)[row, t] (off + c_t,chan)     A = P scaled per channel group (hi + remainder)
 //                            - off * sum_t (P s_g)[row, t]           extra tile against ones, same A
 //                            + sum_t P[row, t] z_g[t]                extra tile, B = value zeros
 //   denominator               sum_t P[row, t]                        extra tile against ones
@@ -22,8 +22,9 @@
 // score accumulators, so opening a token group costs no reductions.
 //
 // Values (per-token scale s_g[t], zero z_g[t] per channel group g): the scale is
-// folded into the probabilities, one fp16 multiply per two tokens per group.  A
-// value tile covers 16 consecutive channels, which lie in one group.
+// folded into the probabilities (fp16 product plus its exact fp16 remainder, so that a
+// sharply peaked softmax still returns code*scale+zero to float32 accuracy).  A value
+// tile covers 16 consecutive channels, which lie in one group.
 //
 // Query rows (the H_q/H_kv heads sharing the kv head) sit in the 16-wide M/N
 // dimension.  Keys are packed along channels, so a lane's eight k-slots of the
@@ -125,11 +126,12 @@ template <int BITS, typename M, int GV> struct PackedUnit {
 constexpr int MF_QIMG = 12 * 64;
 
 template <int BITS>
-__device__ __forceinline__ void build_query_image(const vq_attend_args &a, int64_t row0, int R, int tid, f16 *s_qraw,
+__device__ __forceinline__ void build_query_image(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw,
                                                   uint4 *s_q) {
+    const int R = tile.RT;
     for (int e = tid; e < MF_ROWS * MF_D; e += 256) {
         const int row = e / MF_D, d = e % MF_D;
-        s_qraw[e] = row < R ? (f16)ldq(a.q, a.q_dtype, (row0 + row) * MF_D + d) : (f16)0.f;
+        s_qraw[e] = tile.valid(row) ? (f16)ldq(a.q, a.q_dtype, tile.row(row) * MF_D + d) : (f16)0.f;
     }
     __syncthreads();
     for (int e = tid; e < MF_QIMG; e += 256) {
@@ -158,7 +160,8 @@ __device__ __forceinline__ void build_query_image(const vq_attend_args &a, int64
 
 template <int BITS, typename M, int GV>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, int R, float c, int64_t t_begin,
-                                             int n_units, int lane, int wave, PackedAcc<GV> &acc, const uint4 *s_q) {
+                                             int n_units, int64_t lane_vis, int64_t full_vis, int lane, int wave,
+                                             PackedAcc<GV> &acc, const uint4 *s_q) {
     constexpr int PER = 32 / BITS;           // codes per word
     constexpr int KW = MF_D / PER;           // key words per token row
     constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
@@ -276,7 +279,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     };
 
     // ---- one unit: scores, softmax, output
-    auto compute = [&](const Unit &cur) {
+    auto compute = [&](const Unit &cur, int64_t base) {
 #ifdef VQ_EXPERIMENT_LOADS_ONLY
         if constexpr (sizeof(M) == 2) {
             u32 x = 0;
@@ -313,6 +316,15 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                     for (int r = 0; r < 4; ++r) S[T][r] += __shfl(S[T][r], (lane & ~15) | ((n + R) & 15));
         }
 #undef VQ_ADD_SHL
+        // causal edge: tokens this lane's query row does not see (units below full_vis are
+        // visible to every row of the tile)
+        if (base + 32 > full_vis) {
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (base + vtok_lo<BITS>(blk, r) + T * GAP >= lane_vis) S[T][r] = -INFINITY;
+        }
 
         // softmax against a lazily updated reference: the fast path touches no other lane
         const float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
@@ -321,8 +333,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             float m_seen = mx * c;
             m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 16));
             m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 32));
-            const float m_new = fmaxf(acc.m_run, m_seen);   // finite: scores are finite
-            const float alpha = exp2f(acc.m_run - m_new);   // 0 on the first unit
+            const float m_new = fmaxf(acc.m_run, m_seen);
+            const float alpha = m_new == -INFINITY ? 1.f : exp2f(acc.m_run - m_new);   // 0 on the first unit
             float al[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
@@ -337,7 +349,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             }
             acc.m_run = m_new;
         }
-        const float nm = -acc.m_run;
+        const float nm = acc.m_run == -INFINITY ? 0.f : -acc.m_run;   // a row with no visible token yet
         float Pf[2][4];
         u32 P[4];
 #pragma unroll
@@ -348,22 +360,35 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         }
         const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
 
-        // output: per channel group, A = P * s_g
+        // output: per channel group, A = P * s_g as an fp16 high part plus its exact fp16
+        // remainder (P and s have 11 significant bits each), both multiplied into the codes
 #pragma unroll
         for (int g = 0; g < GV; ++g) {
-            u32 ag[4];
+            u32 ah[4], al[4];
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                if constexpr (sizeof(M) == 2) ag[p] = as_u(as_h2(P[p]) * as_h2(cur.s[g].pair(p)));
-                else ag[p] = as_u(f16x2{(f16)(Pf[0][p] * cur.s[g].lo(p)), (f16)(Pf[1][p] * cur.s[g].hi(p))});
+                if constexpr (sizeof(M) == 2) {
+                    const f16x2 sp = as_h2(cur.s[g].pair(p));
+                    const f16x2 hi = as_h2(P[p]) * sp;
+                    ah[p] = as_u(hi);
+                    al[p] = as_u(__builtin_elementwise_fma(as_h2(P[p]), sp, -hi));
+                } else {
+                    const float t0 = (float)as_h2(P[p])[0] * cur.s[g].lo(p), t1 = (float)as_h2(P[p])[1] * cur.s[g].hi(p);
+                    const f16x2 hi = {(f16)t0, (f16)t1};
+                    ah[p] = as_u(hi);
+                    al[p] = as_u(f16x2{(f16)(t0 - (float)hi[0]), (f16)(t1 - (float)hi[1])});
+                }
             }
-            const f16x8 A = as_h8(ag[0], ag[1], ag[2], ag[3]);
+            const f16x8 Ah = as_h8(ah[0], ah[1], ah[2], ah[3]), Al = as_h8(al[0], al[1], al[2], al[3]);
 #pragma unroll
             for (int j = 0; j < TPG; ++j) {
                 const int nt = g * TPG + j;
-                acc.O[nt] = VQ_MFMA(A, unpack8<BITS>(cur.vw[nt] >> vshift, magic), acc.O[nt]);
+                const f16x8 Bv = unpack8<BITS>(cur.vw[nt] >> vshift, magic);
+                acc.O[nt] = VQ_MFMA(Ah, Bv, acc.O[nt]);
+                acc.O[nt] = VQ_MFMA(Al, Bv, acc.O[nt]);
             }
-            acc.Off[g] = VQ_MFMA(A, ones, acc.Off[g]);
+            acc.Off[g] = VQ_MFMA(Ah, ones, acc.Off[g]);
+            acc.Off[g] = VQ_MFMA(Al, ones, acc.Off[g]);
         }
         if constexpr (sizeof(M) == 2) {
             acc.Z = VQ_MFMA(P8, as_h8(cur.z.pair(0), cur.z.pair(1), cur.z.pair(2), cur.z.pair(3)), acc.Z);
@@ -396,7 +421,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         const int64_t next_group = (t_begin + (int64_t)un * 32) / G;
         const bool new_group = next_group != cur_group;
         if (new_group) km.load(ksb + next_group * MF_D * MSZ, kzb + next_group * MF_D * MSZ, kmoff);
-        compute(cur);
+        compute(cur, t_begin + (int64_t)u * 32);
         if (new_group) {
             open_group(km);
             cur_group = next_group;
@@ -408,13 +433,14 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     }
 }
 
-// grid (nsplit, B*Hkv).  Block x covers packed tokens
-// [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)); block 0 first
-// runs the fp16 tail, whose partial goes to slot nsplit.  With sync counters the block that
-// finishes last for its kv head merges the nparts partials into the output.
+// grid (nsplit, B*Hkv*tiles).  A block works on one tile of query rows (the GQA group at pq
+// consecutive positions) and on packed tokens
+// [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)), cut to what the
+// tile sees; block 0 first runs the fp16 tail, whose partial goes to slot nsplit.  With sync
+// counters the block that finishes last for its tile merges the nparts partials into the output.
 template <int BITS, typename M, int GV>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts,
+void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
                                float *__restrict__ ws) {
     __shared__ float s_m[4][MF_ROWS];
     __shared__ float s_l[4][MF_ROWS];
@@ -426,19 +452,27 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: loops below stay scalar
     const int n = lane & 15, blk = lane >> 4;
-    const int64_t bh = blockIdx.y;
+    const int64_t bh = blockIdx.y / tiles;
     const int sp = (int)blockIdx.x, nsplit = (int)gridDim.x;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
-    const int R = (int)(a.Hq / a.Hkv);
-    const int64_t row0 = b * a.Hq + hkv * R;   // first query row of this kv head (Sq == 1)
     const float c = a.scale * LOG2E;
+
+    RowTile tile;
+    tile.R = (int)(a.Hq / a.Hkv);
+    tile.RT = tile.R * pq;
+    tile.pos0 = (int)(blockIdx.y % tiles) * pq;
+    tile.Sq = a.Sq;
+    tile.n_total = a.n_packed + a.n_tail;
+    tile.causal = a.causal;
+    tile.base_row = (b * a.Hq + hkv * tile.R) * a.Sq;
+    const int RT = tile.RT;
 
     const bool single_launch = a.sync_counters != nullptr;
     // the raw query is staged in the (not yet used) output exchange buffer
     f16 *s_qraw = reinterpret_cast<f16 *>(&s_o[0][0][0]);
-    build_query_image<BITS>(a, row0, R, tid, s_qraw, s_q);
+    build_query_image<BITS>(a, tile, tid, s_qraw, s_q);
     if (sp == 0 && a.n_tail > 0)
-        tail_block(a, bh, row0, R, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid, wave,
+        tail_block(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid, wave,
                    single_launch);
 
     PackedAcc<GV> acc;
@@ -450,12 +484,19 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     acc.L = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
 
+    // packed tokens the rows of the tile see: all of them up to full_vis, none from max_vis on
+    int64_t full_vis = tile.visible(0), max_vis = tile.visible(RT - 1);
+    if (full_vis > a.n_packed) full_vis = a.n_packed;
+    if (max_vis > a.n_packed) max_vis = a.n_packed;
+    int64_t lane_vis = tile.visible(n < RT ? n : (n < 2 * RT ? n - RT : 0));
+    if (lane_vis > a.n_packed) lane_vis = a.n_packed;
+
     int64_t t_begin = (int64_t)sp * split_len - tail_equiv;
     int64_t t_end = t_begin + split_len;
     if (t_begin < 0) t_begin = 0;
-    if (t_end > a.n_packed) t_end = a.n_packed;
+    if (t_end > (max_vis + 31) / 32 * 32) t_end = (max_vis + 31) / 32 * 32;
     const int n_units = t_end > t_begin ? (int)((t_end - t_begin) / 32) : 0;
-    packed_units<BITS, M, GV>(a, bh, R, c, t_begin, n_units, lane, wave, acc, s_q);
+    packed_units<BITS, M, GV>(a, bh, RT, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_q);
 
     // ---- merge the four waves: accumulator register r of lane (n, blk) is row 4*blk + r,
     // tile nt column n is channel 16*nt + n
@@ -463,7 +504,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * blk + r;
-        if (row < R) {
+        if (row < RT) {
             if (n == 0) s_l[wave][row] = acc.L[r];
             if (n < GV) s_z[wave][row][n] = acc.Z[r];
 #pragma unroll
@@ -472,42 +513,44 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         }
     }
     __syncthreads();
-    for (int e = tid; e < R * MF_D; e += 256) {
+    for (int e = tid; e < RT * MF_D; e += 256) {
         const int row = e / MF_D, d = e % MF_D;
+        if (!tile.valid(row)) continue;
         const float gm = fmaxf(fmaxf(s_m[0][row], s_m[1][row]), fmaxf(s_m[2][row], s_m[3][row]));
         float num = 0.f, den = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit
+            if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit, or saw nothing
             const float f = exp2f(s_m[w][row] - gm);
             num += (s_o[w][row][d] + s_z[w][row][d / (MF_D / GV)]) * f;
             den += s_l[w][row] * f;
         }
-        float *o = ws + ((row0 + row) * nparts + sp) * MF_PART;
+        float *o = ws + (tile.row(row) * nparts + sp) * MF_PART;
         st_partial(o + 2 + d, num, single_launch);
         if (d == 0) { st_partial(o, gm * LN2, single_launch); st_partial(o + 1, den, single_launch); }
     }
 
-    // ---- last block of this kv head merges the splits (no block ever waits for another).
+    // ---- last block of this tile merges the splits (no block ever waits for another).
     // Partials travel as device-scope stores and loads, so no cache-wide write-back or
     // invalidate is needed: the barrier below waits until this block's stores are
     // acknowledged, then one thread takes a ticket.
     if (!single_launch) return;
     __syncthreads();
-    if (tid == 0) s_ticket = __hip_atomic_fetch_add(a.sync_counters + bh, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0)
+        s_ticket = __hip_atomic_fetch_add(a.sync_counters + blockIdx.y, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != nsplit - 1) return;
-    merge_rows(a, row0, R, nparts, ws, tid);
-    if (tid == 0) __hip_atomic_store(a.sync_counters + bh, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    merge_rows(a, tile, nparts, ws, tid);
+    if (tid == 0) __hip_atomic_store(a.sync_counters + blockIdx.y, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <typename M>
 static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
-    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv)), block(256);
+    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles)), block(256);
     const int gv = (int)(MF_D / a.group);
 #define VQ_LAUNCH(BITS, GV) \
     hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, 0, st, a, p.split_len, p.tail_equiv, \
-                       p.nparts, ws)
+                       p.nparts, p.pq, p.tiles, ws)
     if (a.pack_bits == 4) {
         if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);
     } else {
