@@ -227,6 +227,34 @@ def _extras(torch, K, dev):
         ms_qp, ms_rt = _event_ms(qp, 30, torch), _event_ms(rt, 30, torch)
         ex[f"quant_pack_{name}"] = {"ms": round(ms_qp, 5), "GBps": round(b_qp / ms_qp / 1e6, 1), "bytes": b_qp}
         ex[f"quant_dequant_{name}"] = {"ms": round(ms_rt, 5), "GBps": round(b_rt / ms_rt / 1e6, 1), "bytes": b_rt}
+    # config 4: causal prefill of 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
+    # tokens plus their own tokens, quantise-on-write (group 32, residual 128)
+    def prefill_pass(timed):
+        cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=4, kivi_group_size=32, residual_length=128,
+                            fused_sdpa=True, fused_sdpa_memory_bound=True)
+        c = KVCacheFactory.create(cfg)
+        k, v = _synthetic_layer(torch, 1, Hkv, 4096, D, 77, dev)
+        c.update_and_fetch(k.to(torch.bfloat16), v.to(torch.bfloat16))
+        chunks = []
+        for ci in range(8):
+            k, v = _synthetic_layer(torch, 1, Hkv, 512, D, 78 + ci, dev)
+            chunks.append((k.to(torch.bfloat16), v.to(torch.bfloat16),
+                           torch.randn((1, Hq, 512, D), device=dev).to(torch.bfloat16)))
+        torch.cuda.synchronize()
+        s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s_.record()
+        for k, v, q in chunks:
+            c.update_and_fetch(k, v)
+            c.fused_sdpa(q, 1 / math.sqrt(D), causal=True)
+        e_.record()
+        torch.cuda.synchronize()
+        return s_.elapsed_time(e_)
+    prefill_pass(False)
+    ms = min(prefill_pass(True) for _ in range(3))
+    flops = 412350414848
+    ex["prefill_cfg4"] = {"ms": round(ms, 4), "TFLOPs": round(flops / ms / 1e9, 1),
+                          "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
+                          "note": "8 chunks of 512 queries: quantise-on-write append + attention per chunk"}
     # config 2: VQ assignment, keys [4,4096,256], 256 centroids x 8 dims
     x = (torch.randn((4, 4096, 256), device=dev) * torch.exp(torch.randn(256, device=dev))).to(torch.float16)
     cb = torch.randn((256, 8), device=dev).to(torch.float16)

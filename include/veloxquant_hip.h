@@ -152,7 +152,9 @@ typedef struct vq_attend_args {
     int64_t n_tail, tail_cap;
     float scale; /* softmax scale applied to q.k */
     int causal;  /* 1: query i sees slots <= n_packed + n_tail - Sq + i */
-    int num_splits; /* 0 = choose; otherwise the split count along tokens */
+    int num_splits; /* 0 = choose; > 0 the split count along tokens; < 0 choose, but take the
+                     * layout-agnostic vector kernel even where the MFMA kernel applies
+                     * (cross-checks of the two implementations) */
     void *workspace;
     size_t workspace_bytes;
     void *stream;

@@ -119,7 +119,7 @@ def test_future_keys_do_not_leak_into_earlier_rows():
 
 # ------------------------------------------------------------ packed cache path
 def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, causal=False, seed=0,
-                 q_dtype=torch.float16, cap_extra=0, expect_path=None):
+                 q_dtype=torch.float16, cap_extra=0, expect_path=None, tail_dtype=torch.float16):
     require_gpu()
     per = 32 // b
     k, v = outlier_kv((B, Hkv, n_packed + n_tail, D), seed=seed)
@@ -152,8 +152,12 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
         kc, ksn, kzn = ok.group_quant_codes(k[:, :, :n_packed], -2, g, levels)
         vc, vsn, vzn = ok.group_quant_codes(v[:, :, :n_packed], -1, g, levels)
         ref_args = [kc, ksn.astype(npm), kzn.astype(npm), vc, vsn.astype(npm), vzn.astype(npm)]
-    tail_k = kt[:, :, n_packed:].contiguous() if n_tail else None
-    tail_v = vt[:, :, n_packed:].contiguous() if n_tail else None
+    tail_k = kt[:, :, n_packed:].to(tail_dtype).contiguous() if n_tail else None
+    tail_v = vt[:, :, n_packed:].to(tail_dtype).contiguous() if n_tail else None
+    if n_tail and tail_dtype != torch.float16:   # the reference sees the tail as stored
+        k, v = k.astype(np.float32), v.astype(np.float32)
+        k[:, :, n_packed:] = tail_k.float().cpu().numpy()
+        v[:, :, n_packed:] = tail_v.float().cpu().numpy()
     plan = {}
     out = K.kivi_packed_attend(qt, n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k,
                                v_tail=tail_v, n_tail=n_tail, scale=scale, causal=causal,
@@ -281,3 +285,12 @@ def test_mfma_prefill_not_causal_and_split_tokens():
 def test_mfma_prefill_odd_head_ratio_takes_vector_kernel():
     _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=4, causal=True, seed=23, expect_path=0)
     _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=1, seed=24, expect_path=1)
+
+
+def test_mfma_path_takes_bf16_tails():
+    _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=1, seed=31, q_dtype=torch.bfloat16,
+                 tail_dtype=torch.bfloat16, expect_path=1)
+    _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=40, causal=True, seed=32,
+                 q_dtype=torch.bfloat16, tail_dtype=torch.bfloat16, expect_path=1)
+    _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=1, seed=33, tail_dtype=torch.float32,
+                 expect_path=0)

@@ -12,6 +12,7 @@ import torch
 
 from oracle import attend as oa, kivi as ok, vecinfer as ov
 from tests._gpu import gpu, host, outlier_kv, require_gpu, to_dev
+from veloxquant_mlx_amd import kernels as K
 from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
 from veloxquant_mlx_amd.quantizers import KIVIQuantizer
 
@@ -156,6 +157,44 @@ def test_chunked_prefill_through_the_cache_matches_oracle():
     got = np.concatenate(outs, axis=2).astype(np.float32)
     ref = oa.chunked_prefill(q, k, v, 64, 4, 32, 32, 1 / math.sqrt(D))
     assert np.max(np.abs(got - ref)) < 2e-3
+
+
+def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
+    """BASELINE configs[4]: 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
+    tokens plus their own tokens (32 query / 8 kv heads, D=128, group 32, residual 128).  The
+    oracle is too slow at this size, so the two independent GPU implementations (each checked
+    against the oracle at small sizes) are compared on the chunks with the shortest and the
+    longest visible history; chunks in between only advance the cache."""
+    require_gpu()
+    B, Hq, Hkv, D, P, C = 1, 32, 8, 128, 4096, 512
+    dev = "cuda:0"
+    g = torch.Generator(device=dev).manual_seed(4)
+    f = torch.exp(torch.randn(D, generator=g, device=dev))
+    c = _make(bit_width_inlier=4, kivi_group_size=32, residual_length=128, fused_sdpa=True,
+              fused_sdpa_memory_bound=True)
+    mk = lambda n: ((torch.randn((B, Hkv, n, D), generator=g, device=dev) * f).to(torch.bfloat16),
+                    torch.randn((B, Hkv, n, D), generator=g, device=dev).to(torch.bfloat16))
+    c.update_and_fetch(*mk(P))
+    scale = 1 / math.sqrt(D)
+    for ci in range(8):
+        c.update_and_fetch(*mk(C))
+        q = torch.randn((B, Hq, C, D), generator=g, device=dev).to(torch.bfloat16)
+        if ci not in (0, 7):
+            continue
+        nq, n_tail = c._n_quantized, c.offset - c._n_quantized
+        assert nq == (P + C * (ci + 1) - 128) // 32 * 32
+        kw = dict(k_packed=c._kp, k_scale=c._ks, k_zero=c._kz, v_packed=c._vp, v_scale=c._vs, v_zero=c._vz,
+                  n_packed=nq, bits=4, group_size=32, v_layout="token", k_tail=c._tail_k, v_tail=c._tail_v,
+                  n_tail=n_tail, scale=scale, causal=True, out_dtype=torch.float32)
+        p1, p0 = {}, {}
+        o1 = K.kivi_packed_attend(q, _plan_out=p1, **kw)
+        o0 = K.kivi_packed_attend(q, num_splits=-1, _plan_out=p0, **kw)
+        assert p1["path"] == 1 and p0["path"] == 0
+        err = float((o1 - o0).abs().max())
+        print(f"chunk {ci}: {nq} packed + {n_tail} tail slots, max |mfma - vector| = {err:.2e}")
+        assert err < 2e-3
+        # the cache's own entry point returns the same numbers in the query dtype
+        assert torch.equal(c.fused_sdpa(q, scale, causal=True), o1.to(torch.bfloat16))
 
 
 def test_kivi_quantizer_encode_decode():

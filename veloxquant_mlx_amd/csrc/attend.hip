@@ -6,7 +6,7 @@ namespace vq {
 
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
-    p.path = mfma_decode_supported(a) ? 1 : 0;
+    p.path = (a.num_splits >= 0 && mfma_decode_supported(a)) ? 1 : 0;
     p.tail_equiv = 0;
     p.pq = 1;
     p.tiles = 1;
@@ -24,7 +24,7 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     // or a four-wave block per kv head (MFMA)
     const int64_t units = p.path == 1 ? a.B * a.Hkv * p.tiles : a.B * a.Hq * a.Sq;
     const int64_t target = p.path == 1 ? 512 : 4096;
-    int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);
+    int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);   // < 0: choose as well
     if (ns > max_splits) ns = max_splits;
     if (ns > 512) ns = 512;
     if (ns < 1) ns = 1;

@@ -24,7 +24,7 @@ bool mfma_decode_supported(const vq_attend_args &a) {
     if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
     if (a.cap_tokens > (1 << 24)) return false;   // per-lane byte offsets are 32-bit
     if (!(a.scale > 0.f)) return false;
-    if (a.n_tail > 0 && (a.tail_dtype != VQ_F16 || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
+    if (a.n_tail > 0 && (!(a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
     const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
                          (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
     if (al & 15u) return false;

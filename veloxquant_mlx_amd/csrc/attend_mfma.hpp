@@ -122,7 +122,7 @@ struct RowTile {
 };
 
 // ---------------------------------------------------------------------------
-// Un-quantised fp16 tail, run by the four waves of one block in units of 32 tokens:
+// Un-quantised fp16 / bf16 tail, run by the four waves of one block in units of 32 tokens:
 //   S^T[token, row] = K[token, :] . q[row, :]          A = K as stored, B = q
 //   O[row, chan]   += P[row, token] * V[token, chan]   A = P, B = V
 // Values are loaded as eight rows of eight channels per lane and transposed in
@@ -174,6 +174,22 @@ __device__ __forceinline__ void st_partial(float *p, float v, bool device_scope)
     else *p = v;
 }
 
+// Eight consecutive tail elements as fp16.  A bf16 tail is converted: exact for magnitudes in
+// fp16's normal range, an absolute error below 2^-25 for smaller ones, saturating at 65504.
+__device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool bf16) {
+    if (!bf16) return *reinterpret_cast<const f16x8 *>((const f16 *)base + elem);
+    const uint4 u = *reinterpret_cast<const uint4 *>((const u16 *)base + elem);
+    const u32 w[4] = {u.x, u.y, u.z, u.w};
+    f16x8 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float lo = __uint_as_float(w[j] << 16), hi = __uint_as_float(w[j] & 0xffff0000u);
+        o[2 * j] = (f16)fminf(fmaxf(lo, -65504.f), 65504.f);
+        o[2 * j + 1] = (f16)fminf(fmaxf(hi, -65504.f), 65504.f);
+    }
+    return o;
+}
+
 // s_m, s_l: [4][MF_ROWS] floats; s_o: [4][MF_ROWS][MF_D] floats of block-shared memory.
 // s_qraw: the query rows of this kv head as fp16 [MF_ROWS][MF_D] (rows >= R zero); it may
 // alias s_o: it is read into registers before s_o is written.
@@ -190,8 +206,8 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
     for (int n = 0; n < 9; ++n) acc.O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
 
-    const f16 *kt = (const f16 *)a.k_tail + bh * a.tail_cap * MF_D;
-    const f16 *vt = (const f16 *)a.v_tail + bh * a.tail_cap * MF_D;
+    const bool bf16 = a.tail_dtype == VQ_BF16;
+    const int64_t tbase = bh * a.tail_cap * MF_D;
     f16x8 qT[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * MF_D + 32 * blk + 8 * ks);
@@ -206,15 +222,15 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             const int64_t tok = base + tail_tok(i >> 2, i & 3, T);
-            const f16 *p = kt + (tok < a.n_tail ? tok : 0) * MF_D + 32 * blk;
+            const int64_t e = tbase + (tok < a.n_tail ? tok : 0) * MF_D + 32 * blk;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) d.kr[T][ks] = *reinterpret_cast<const f16x8 *>(p + 8 * ks);
+            for (int ks = 0; ks < 4; ++ks) d.kr[T][ks] = ld_tail8(a.k_tail, e + 8 * ks, bf16);
         }
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const int64_t tA = base + tail_tok(blk, p, 0), tB = base + tail_tok(blk, p, 1);
-            d.vr[2 * p] = *reinterpret_cast<const f16x8 *>(vt + (tA < a.n_tail ? tA : 0) * MF_D + 8 * i);
-            d.vr[2 * p + 1] = *reinterpret_cast<const f16x8 *>(vt + (tB < a.n_tail ? tB : 0) * MF_D + 8 * i);
+            d.vr[2 * p] = ld_tail8(a.v_tail, tbase + (tA < a.n_tail ? tA : 0) * MF_D + 8 * i, bf16);
+            d.vr[2 * p + 1] = ld_tail8(a.v_tail, tbase + (tB < a.n_tail ? tB : 0) * MF_D + 8 * i, bf16);
         }
     };
     auto compute = [&](int u, const TUnit &d) {
