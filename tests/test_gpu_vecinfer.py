@@ -105,3 +105,42 @@ def test_wrapper_errors():
         K.vecinfer_quantize_metal(x, cb, 5)
     with pytest.raises(ValueError, match="codebook must be 2D"):
         K.vecinfer_dequant_metal(to_dev(np.zeros((2, 2), np.int32)), cb.reshape(-1))
+
+
+# ------------------------------------------------ the MFMA filter's undecided cases
+@pytest.mark.parametrize("sub,nc", [(8, 256), (8, 200), (4, 256), (8, 5), (4, 17)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32, torch.bfloat16])
+def test_mfma_filter_near_ties_follow_the_exact_rule(sub, nc, dtype):
+    """Sub-vectors placed (almost) on the bisector of two or more centroids, where only the
+    float32 rounding of the sequential rule decides: one ulp nudges either way, clusters of
+    near-identical centroids, exact duplicates in several tracker positions."""
+    require_gpu()
+    rng = np.random.default_rng(sub * 7 + nc)
+    cb = rng.standard_normal((nc, sub)).astype(np.float16).astype(np.float32)
+    if nc >= 17:
+        cb[3] = cb[16]; cb[nc - 1] = cb[16]            # triple duplicate across tiles and rows
+        cb[5] = cb[4] + np.float32(2.0 ** -10)           # a cluster of near-identical centroids
+        cb[6] = cb[4] - np.float32(2.0 ** -10)
+        cb[7] = cb[4]
+    cbt = to_dev(cb, torch.float32 if dtype == torch.float32 else torch.float16)
+    cbh = host(cbt).astype(np.float32)
+    n = 4096 + 37
+    a = rng.integers(0, nc, n)
+    b = rng.integers(0, nc, n)
+    mid = 0.5 * (cbh[a] + cbh[b])
+    x = mid + rng.standard_normal((n, sub)).astype(np.float32) * np.float32(1e-4) * (rng.integers(0, 3, (n, 1)) > 0)
+    x[::5] = cbh[a[::5]]                                 # exactly on a centroid (duplicates tie)
+    xt = to_dev(x.astype(np.float32), dtype)
+    got = host(K.vecinfer_quantize_metal(xt, cbt, sub)).reshape(-1)
+    ref = ov.quantize_vq(host(xt).astype(np.float32), cbh, sub).reshape(-1)
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_mfma_filter_large_magnitudes_and_ragged_count():
+    require_gpu()
+    rng = np.random.default_rng(11)
+    cb = (rng.standard_normal((256, 8)) * 30).astype(np.float16)
+    for n in (1, 63, 64, 65, 1000):
+        x = (rng.standard_normal((n, 8)) * np.exp(2 * rng.standard_normal(8))).astype(np.float16)
+        got = host(K.vecinfer_quantize_metal(to_dev(x), to_dev(cb), 8)).reshape(-1)
+        np.testing.assert_array_equal(got, ov.quantize_vq(x, cb, 8).reshape(-1))

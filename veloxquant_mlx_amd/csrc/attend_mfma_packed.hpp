@@ -280,17 +280,6 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 
     // ---- one unit: scores, softmax, output
     auto compute = [&](const Unit &cur, int64_t base) {
-#ifdef VQ_EXPERIMENT_LOADS_ONLY
-        if constexpr (sizeof(M) == 2) {
-            u32 x = 0;
-            for (int T = 0; T < 2; ++T) for (int k = 0; k < KWL; ++k) x ^= cur.kw[T][k];
-            for (int nt = 0; nt < 8; ++nt) x ^= cur.vw[nt];
-            for (int g = 0; g < GV; ++g) x ^= cur.s[g].a.x ^ cur.s[g].a.y ^ cur.s[g].b.x ^ cur.s[g].b.y;
-            x ^= cur.z.a.x ^ cur.z.a.y ^ cur.z.b.x ^ cur.z.b.y;
-            acc.L[0] += __builtin_bit_cast(float, x & 0x3fffffffu);
-            return;
-        }
-#endif
         f32x4 S[2];
 #pragma unroll
         for (int T = 0; T < 2; ++T)

@@ -7,35 +7,13 @@
 //
 // The codebook is staged once per block in LDS as float32; all lanes read the
 // same centroid at the same time, which the LDS serves as a broadcast.
-#include "common.hpp"
+#include "vecinfer.hpp"
 
 namespace vq {
 
-// Element loads/stores typed at run time: they sit outside the distance loop,
-// so one kernel per (SUB, codebook placement) serves every dtype combination.
-__device__ __forceinline__ float ld_any(const void *p, int tag, int64_t i) {
-    if (tag == VQ_F16) return (float)((const f16 *)p)[i];
-    if (tag == VQ_BF16) return bf16_to_f32(((const u16 *)p)[i]);
-    return ((const float *)p)[i];
-}
-__device__ __forceinline__ void st_any(void *p, int tag, int64_t i, float v) {
-    if (tag == VQ_F16) ((f16 *)p)[i] = (f16)v;
-    else if (tag == VQ_BF16) ((u16 *)p)[i] = f32_to_bf16(v);
-    else ((float *)p)[i] = v;
-}
-__device__ __forceinline__ void st_idx(void *p, int tag, int64_t i, int v) {
-    if (tag == VQ_U8) ((uint8_t *)p)[i] = (uint8_t)v;
-    else ((int32_t *)p)[i] = v;
-}
-__device__ __forceinline__ uint32_t ld_idx(const void *p, int tag, int64_t i) {
-    if (tag == VQ_U8) return ((const uint8_t *)p)[i];
-    return (uint32_t)((const int32_t *)p)[i];
-}
-
 constexpr int VQ_VPT = 4;  // sub-vectors per thread
 
-// X: input element type, C: codebook element type, SUB: sub-vector length
-// (0 = runtime), LDS_CB: codebook staged in LDS (else read from global memory).
+// SUB: sub-vector length (0 = runtime), LDS_CB: codebook staged in LDS (else read from global memory).
 template <int SUB, bool LDS_CB>
 __global__ __launch_bounds__(256) void vq_assign_kernel(const void *__restrict__ x, int xt, int64_t N,
                                                         const void *__restrict__ cb, int ct, int nc, int sub_rt,
@@ -153,7 +131,8 @@ extern "C" int vq_vecinfer_assign(const void *x, int x_dtype, int64_t N, const v
     if (N == 0) return VQ_OK;
     VQ_REQUIRE(x && codebook && idx, VQ_ERR_INVALID, "%s: null pointer", fn);
     hipStream_t st = (hipStream_t)stream;
-    launch_assign(x, x_dtype, N, codebook, cb_dtype, n_centroids, sub_dim, idx, idx_dtype, st);
+    if (!launch_assign_mfma(x, x_dtype, N, codebook, cb_dtype, n_centroids, sub_dim, idx, idx_dtype, st))
+        launch_assign(x, x_dtype, N, codebook, cb_dtype, n_centroids, sub_dim, idx, idx_dtype, st);
     VQ_HIP_CHECK_LAUNCH(fn);
     return VQ_OK;
 }

@@ -459,7 +459,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     need = lib.vq_kivi_attend_workspace(a)
     ws = _workspace(q.device, need)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
-    a.sync_counters = _counters(q.device).data_ptr() if (_single_launch and not os.environ.get('VQ_TWO_LAUNCH')) else None
+    a.sync_counters = _counters(q.device).data_ptr() if _single_launch else None
     a.stream = _stream(q)
     _lib.check(lib.vq_kivi_attend(a))
     return out
