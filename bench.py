@@ -156,14 +156,14 @@ def main() -> int:
     # ---- roofline of the dominant kernel (attention), events on the launch stream
     kern_ms = _event_ms(attend_only, max(3, a.steps // 2), torch) / NL
     achieved = layer_bytes / (kern_ms * 1e-3) / 1e9
-    # HBM bytes one attention call moved under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated against
-    # a 1 GiB device copy: x2.000 and x1.000), summed over its three kernels; measured at the default
-    # workload only (profiles/attend_mfma_decode_4bit_cfg3_hbm_traffic.md)
+    # HBM bytes one attention launch moved under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated
+    # against a 1 GiB device copy); measured at the default workload only
+    # (profiles/attend_mfma_packed_4bit_cfg3_hbm_traffic.md)
     default_workload = (B, ctx, bits, g) == (16, 32768, 4, 64)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 620066816 if default_workload else None,
-                "kernel": "vq_kivi_attend, one layer = 3 launches (fp16 tail, packed prefix "
-                          "attend_mfma_decode_kernel, split merge); the prefix kernel is ~90% of it",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 620451430 if default_workload else None,
+                "kernel": "attend_mfma_packed_kernel<4, f16, 2>: one launch per layer does the fp16 tail, "
+                          "the packed prefix and the split merge (vq_kivi_attend with sync counters)",
                 "bytes_per_launch": layer_bytes, "ms_per_launch": round(kern_ms, 5)}
 
     out = {
