@@ -9,8 +9,9 @@
 //   scores   S^T[token, row] = sum_d (off + c_td) (q s)_d          A = codes, B = folded query
 //                            + sum_d z_d q_d - off * sum_d (q s)_d   the accumulator the product starts from
 //   output   O[row, chan]    = sum_t (P s_g)[row, t] (off + c_t,chan)     A = P scaled per channel group (hi + remainder)
-//                            - off * sum_t (P s_g)[row, t]           extra tile against ones, same A
-//                            + sum_t P[row, t] z_g[t]                extra tile, B = value zeros
+//                            - off * sum_t P[row, t] s_g[t]          extra tile, A = P, B = value scales
+//                                                                    (float32 scale / zero: against ones, same A)
+//                            + sum_t P[row, t] z_g[t]                same tile, B = value zeros
 //   denominator               sum_t P[row, t]                        extra tile against ones
 //
 // Keys (per-channel scale s_d, zero z_d per token group): the scale is folded into
@@ -102,10 +103,10 @@ template <> struct ChanMeta<float> {
 };
 
 // Per-wave state of the packed kernel.  GV = channel groups per value row.
-template <int GV> struct PackedAcc {
-    f32x4 O[8];     // tile nt: channels 16*nt + n, still carrying off * Off[group]
-    f32x4 Off[GV];  // sum_t (P s_g)[row, t], every column alike
-    f32x4 Z;        // column g < GV: sum_t P[row, t] z_g[t]
+template <int GV, bool OFF_TILES> struct PackedAcc {
+    f32x4 O[8];     // tile nt: channels 16*nt + n, still carrying off * sum_t (P s_g)[row, t]
+    f32x4 Z;        // column g < GV: sum_t P[row, t] z_g[t]; column GV + g: sum_t P[row, t] s_g[t]
+    f32x4 Off[OFF_TILES ? GV : 1];  // float32 scale / zero only: sum_t (P s_g)[row, t] from the same A operands, every column alike
     f32x4 L;        // sum_t P[row, t], every column alike
     float m_run;    // softmax reference, log2 domain, per lane column (query row)
 };
@@ -114,7 +115,8 @@ template <int BITS, typename M, int GV> struct PackedUnit {
     u32 kw[2][(MF_D * BITS / 32) / 4];   // key words of the lane's 32 channels, two token rows
     u32 vw[8];                           // value words, one per 16-channel tile
     TokMeta<M> s[GV];                    // value scales of the lane's eight tokens, every group
-    TokMeta<M> z;                        // value zeros of the lane's eight tokens, group n % GV
+    TokMeta<M> z;                        // lane column n < GV: value zeros of group n, else value scales of
+                                         // group n % GV, of the lane's eight tokens
 };
 
 // LDS image of the query, three operand forms of 4 k-steps x 64 lanes each:
@@ -161,7 +163,7 @@ __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const
 template <int BITS, typename M, int GV>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, int R, float c, int64_t t_begin,
                                              int n_units, int64_t lane_vis, int64_t full_vis, int lane, int wave,
-                                             PackedAcc<GV> &acc, const uint4 *s_q) {
+                                             PackedAcc<GV, sizeof(M) != 2> &acc, const uint4 *s_q) {
     constexpr int PER = 32 / BITS;           // codes per word
     constexpr int KW = MF_D / PER;           // key words per token row
     constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
@@ -191,6 +193,9 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
     const u32 vsoff = (u32)vtok_lo<BITS>(blk, 0) * MSZ;
     const u32 vzoff = (u32)(((int64_t)(n % GV) * cap + vtok_lo<BITS>(blk, 0)) * MSZ);
+    // B operand of the zero-point tile: zeros in columns [0, GV), scales in [GV, 2 GV) (and,
+    // unused, in the columns beyond)
+    const char *vzs = n < GV ? vzb : vsb;
     const u32 kmoff = 32u * blk * MSZ;
 
     using Unit = PackedUnit<BITS, M, GV>;
@@ -212,7 +217,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         for (int nt = 0; nt < 8; ++nt) d.vw[nt] = ldg<u32>(vp + 64 * nt, voff);
 #pragma unroll
         for (int g = 0; g < GV; ++g) d.s[g].load(vsb + ((int64_t)g * cap + base) * MSZ, vsoff, GAP * MSZ);
-        d.z.load(vzb + base * MSZ, vzoff, GAP * MSZ);
+        d.z.load(vzs + base * MSZ, vzoff, GAP * MSZ);
     };
 
     f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
@@ -331,10 +336,12 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             for (int r = 0; r < 4; ++r) {
 #pragma unroll
                 for (int nt = 0; nt < 8; ++nt) acc.O[nt][r] *= al[r];
-#pragma unroll
-                for (int g = 0; g < GV; ++g) acc.Off[g][r] *= al[r];
                 acc.Z[r] *= al[r];
                 acc.L[r] *= al[r];
+                if constexpr (sizeof(M) != 2) {
+#pragma unroll
+                    for (int g = 0; g < GV; ++g) acc.Off[g][r] *= al[r];
+                }
             }
             acc.m_run = m_new;
         }
@@ -376,8 +383,10 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                 acc.O[nt] = VQ_MFMA(Ah, Bv, acc.O[nt]);
                 acc.O[nt] = VQ_MFMA(Al, Bv, acc.O[nt]);
             }
-            acc.Off[g] = VQ_MFMA(Ah, ones, acc.Off[g]);
-            acc.Off[g] = VQ_MFMA(Al, ones, acc.Off[g]);
+            if constexpr (sizeof(M) != 2) {
+                acc.Off[g] = VQ_MFMA(Ah, ones, acc.Off[g]);
+                acc.Off[g] = VQ_MFMA(Al, ones, acc.Off[g]);
+            }
         }
         if constexpr (sizeof(M) == 2) {
             acc.Z = VQ_MFMA(P8, as_h8(cur.z.pair(0), cur.z.pair(1), cur.z.pair(2), cur.z.pair(3)), acc.Z);
@@ -433,7 +442,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
                                float *__restrict__ ws) {
     __shared__ float s_m[4][MF_ROWS];
     __shared__ float s_l[4][MF_ROWS];
-    __shared__ float s_z[4][MF_ROWS][4];
+    __shared__ float s_z[4][MF_ROWS][8];
     __shared__ float s_o[4][MF_ROWS][MF_D];
     __shared__ uint4 s_q[MF_QIMG];
     __shared__ int s_ticket;
@@ -464,14 +473,16 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         tail_block(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid, wave,
                    single_launch);
 
-    PackedAcc<GV> acc;
+    PackedAcc<GV, sizeof(M) != 2> acc;
 #pragma unroll
     for (int nt = 0; nt < 8; ++nt) acc.O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int g = 0; g < GV; ++g) acc.Off[g] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.Z = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.L = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
+    if constexpr (sizeof(M) != 2) {
+#pragma unroll
+        for (int g = 0; g < GV; ++g) acc.Off[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
 
     // packed tokens the rows of the tile see: all of them up to full_vis, none from max_vis on
     int64_t full_vis = tile.visible(0), max_vis = tile.visible(RT - 1);
@@ -495,10 +506,11 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         const int row = 4 * blk + r;
         if (row < RT) {
             if (n == 0) s_l[wave][row] = acc.L[r];
-            if (n < GV) s_z[wave][row][n] = acc.Z[r];
+            if (n < 2 * GV) s_z[wave][row][n] = acc.Z[r];
 #pragma unroll
             for (int nt = 0; nt < 8; ++nt)
-                s_o[wave][row][16 * nt + n] = acc.O[nt][r] - Magic<BITS>::off * acc.Off[nt / (8 / GV)][r];
+                if constexpr (sizeof(M) == 2) s_o[wave][row][16 * nt + n] = acc.O[nt][r];
+                else s_o[wave][row][16 * nt + n] = acc.O[nt][r] - Magic<BITS>::off * acc.Off[nt / (8 / GV)][r];
         }
     }
     __syncthreads();
@@ -511,7 +523,9 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         for (int w = 0; w < 4; ++w) {
             if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit, or saw nothing
             const float f = exp2f(s_m[w][row] - gm);
-            num += (s_o[w][row][d] + s_z[w][row][d / (MF_D / GV)]) * f;
+            const int g = d / (MF_D / GV);
+            const float off_sum = sizeof(M) == 2 ? Magic<BITS>::off * s_z[w][row][GV + g] : 0.f;
+            num += ((s_o[w][row][d] - off_sum) + s_z[w][row][g]) * f;
             den += s_l[w][row] * f;
         }
         float *o = ws + (tile.row(row) * nparts + sp) * MF_PART;
