@@ -170,8 +170,9 @@ typedef struct vq_attend_args {
 size_t vq_kivi_attend_workspace(const vq_attend_args *a);
 
 /* Reports what vq_kivi_attend would do for these arguments: *path = 0 for the
- * layout-agnostic vector kernel, 1 for the MFMA decode kernel; *nparts = number
- * of partial results per query row.  No counterpart in the reference (its
+ * layout-agnostic vector kernel, 1 for the MFMA decode kernel, 2 for the MFMA
+ * prefill kernel (16 or more queries per sequence); *nparts = number of partial
+ * results per query row.  No counterpart in the reference (its
  * _auto_nsg heuristic, veloxquant_mlx/metal/_scalar_attend.py:337-362, is the
  * nearest thing); used by tests and benchmarks to name the kernel measured. */
 int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts);

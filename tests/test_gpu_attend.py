@@ -267,12 +267,17 @@ def test_mfma_prefill_causal_edge_inside_packed_prefix(Hq, Hkv, Sq, n_packed, n_
     """Queries align to the end of the slots, so with a short tail the causal edge of most
     rows lies inside the packed prefix (the chunked quantise-on-write situation)."""
     _packed_case(1, Hq, Hkv, n_packed, n_tail, 128, 4, 32, "token", torch.float16, Sq=Sq, causal=True,
-                 seed=Hq + Sq, expect_path=1)
+                 seed=Hq + Sq, expect_path=2)
+    # the same rows through the 8-row decode-style tiles (what calls with fewer than 16 queries take)
+    _packed_case(1, Hq, Hkv, n_packed, n_tail, 128, 4, 32, "token", torch.float16, Sq=min(Sq, 15), causal=True,
+                 seed=Hq + Sq + 1, expect_path=1)
 
 
 @pytest.mark.parametrize("b,g,meta", [(2, 32, torch.float16), (4, 64, torch.float32), (2, 128, torch.float16)])
 def test_mfma_prefill_bits_groups_and_bf16_queries(b, g, meta):
     _packed_case(2, 8, 2, 512, 70, 128, b, g, "token", meta, Sq=50, causal=True, seed=b + g,
+                 q_dtype=torch.bfloat16, expect_path=2 if meta == torch.float16 else 1)
+    _packed_case(2, 8, 2, 512, 70, 128, b, g, "token", meta, Sq=9, causal=True, seed=b + g + 1,
                  q_dtype=torch.bfloat16, expect_path=1)
 
 
@@ -291,6 +296,18 @@ def test_mfma_path_takes_bf16_tails():
     _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=1, seed=31, q_dtype=torch.bfloat16,
                  tail_dtype=torch.bfloat16, expect_path=1)
     _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=40, causal=True, seed=32,
+                 q_dtype=torch.bfloat16, tail_dtype=torch.bfloat16, expect_path=2)
+    _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=12, causal=True, seed=34,
                  q_dtype=torch.bfloat16, tail_dtype=torch.bfloat16, expect_path=1)
     _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=1, seed=33, tail_dtype=torch.float32,
                  expect_path=0)
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 2)])
+@pytest.mark.parametrize("b,g,meta", [(4, 32, torch.float16), (2, 64, torch.float16), (4, 128, torch.float32),
+                                      (2, 32, torch.float32)])
+def test_mfma_prefill_lds_kernel_shapes(Hq, Hkv, b, g, meta):
+    """64-row blocks over several units and token groups, ragged last tile, not-causal and causal."""
+    path = 2 if meta == torch.float16 else 1   # float32 scale / zero stays on the 8-row tiles
+    _packed_case(1, Hq, Hkv, 384, 45, 128, b, g, "token", meta, Sq=100, causal=True, seed=Hq + b + g, expect_path=path)
+    _packed_case(1, Hq, Hkv, 384, 0, 128, b, g, "token", meta, Sq=16, causal=False, seed=Hq + b + g + 1, expect_path=path)

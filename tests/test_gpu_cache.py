@@ -189,7 +189,7 @@ def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
         p1, p0 = {}, {}
         o1 = K.kivi_packed_attend(q, _plan_out=p1, **kw)
         o0 = K.kivi_packed_attend(q, num_splits=-1, _plan_out=p0, **kw)
-        assert p1["path"] == 1 and p0["path"] == 0
+        assert p1["path"] == 2 and p0["path"] == 0
         err = float((o1 - o0).abs().max())
         print(f"chunk {ci}: {nq} packed + {n_tail} tail slots, max |mfma - vector| = {err:.2e}")
         assert err < 2e-3

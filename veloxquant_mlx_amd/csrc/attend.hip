@@ -10,6 +10,20 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     p.tail_equiv = 0;
     p.pq = 1;
     p.tiles = 1;
+    if (a.num_splits >= 0 && mfma_prefill_supported(a)) {
+        // 64-row blocks; split their work until the grid holds two blocks per compute unit
+        p.path = 2;
+        const int64_t blocks = a.B * a.Hkv * cdiv(a.Sq, 64 / (a.Hq / a.Hkv));
+        const int64_t work = cdiv(a.n_packed + a.n_tail, 32);
+        int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(512, blocks);
+        if (ns > 8) ns = 8;
+        if (ns > work) ns = work;
+        if (ns < 1) ns = 1;
+        p.nsplit = (int)ns;
+        p.split_len = a.n_packed;
+        p.nparts = p.nsplit;
+        return p;
+    }
     // tokens the kernel splits: the MFMA path hands the tail to the block of split 0 and
     // prices a tail token at two packed tokens when it balances the splits
     int64_t n_split = a.n_packed + a.n_tail;
@@ -105,6 +119,9 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a) {
         const bool merged = launch_attend_mfma_decode(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
         if (merged) return VQ_OK;
+    } else if (p.path == 2) {
+        launch_attend_mfma_prefill(*a, p);
+        VQ_HIP_CHECK_LAUNCH(fn);
     } else {
         rc = launch_attend_generic(*a, p.nsplit, p.split_len);
         if (rc != VQ_OK) return rc;

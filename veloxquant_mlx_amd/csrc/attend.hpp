@@ -5,7 +5,7 @@
 namespace vq {
 
 struct AttendPlan {
-    int path;           // 0 generic waves, 1 MFMA decode
+    int path;           // 0 generic waves, 1 MFMA decode (row tiles of <= 8), 2 MFMA prefill (LDS-staged, 64-row blocks)
     int nsplit;         // splits along the tokens the main kernel covers
     int nparts;         // partials per query row handed to the merge kernel
     int64_t split_len;  // tokens per split (multiple of 64)
@@ -68,6 +68,10 @@ int launch_attend_merge(const vq_attend_args &a, int nparts);
 // MFMA decode path (attend_mfma.hip)
 bool mfma_decode_supported(const vq_attend_args &a);
 int mfma_positions_per_tile(const vq_attend_args &a);
+
+// MFMA prefill path (attend_prefill.hip): packed prefix into partial slot 0, tail into slot 1
+bool mfma_prefill_supported(const vq_attend_args &a);
+void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p);
 // returns true when the kernel also merged the partials (sync counters were given)
 bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p);
 

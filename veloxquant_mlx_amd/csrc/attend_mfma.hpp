@@ -40,14 +40,16 @@ constexpr float LN2 = 0.6931471805599453f;
 // row's maximum creeps up.
 constexpr float RESCALE_SLACK = 8.0f;
 
-// Magic constants: an fp16 whose mantissa field receives the code.  A 4-bit code
-// in mantissa bits 4..7 of 64.0 reads 64 + code; a 2-bit code in bits 6..7 of 16.0
-// reads 16 + code.
+// Magic constants: an fp16 whose TOP mantissa bits receive the code, so that the constant is
+// as small as it can be next to the codes (the products carry offset + code, and float32
+// accumulation of the offset part costs accuracy in proportion to offset / code).  A 4-bit
+// code in mantissa bits 6..9 of 16.0 reads 16 + code; a 2-bit code in bits 8..9 of 4.0 reads
+// 4 + code.
 template <int BITS> struct Magic {
-    static constexpr u32 bits = BITS == 4 ? 0x54005400u : 0x4C004C00u;
-    static constexpr u32 mask = BITS == 4 ? 0x00F000F0u : 0x00C000C0u;
-    static constexpr float off = BITS == 4 ? 64.f : 16.f;
-    static constexpr u32 neg_off_pair = BITS == 4 ? 0xD400D400u : 0xCC00CC00u;   // {-off, -off}
+    static constexpr u32 bits = BITS == 4 ? 0x4C004C00u : 0x44004400u;
+    static constexpr u32 mask = BITS == 4 ? 0x03C003C0u : 0x03000300u;
+    static constexpr float off = BITS == 4 ? 16.f : 4.f;
+    static constexpr u32 neg_off_pair = BITS == 4 ? 0xCC00CC00u : 0xC400C400u;   // {-off, -off}
 };
 
 // Eight codes of one packed word as fp16 values (offset + code), in k-slot pair order.
@@ -60,15 +62,15 @@ template <int BITS> __device__ __forceinline__ f16x8 unpack8(u32 w, u32 magic) {
     constexpr u32 mask = Magic<BITS>::mask;
     u32 r0, r1, r2, r3;
     if (BITS == 4) {
-        r0 = ((w << 4) & mask) | magic;
-        r1 = (w & mask) | magic;
-        r2 = ((w >> 4) & mask) | magic;
-        r3 = ((w >> 8) & mask) | magic;
-    } else {
         r0 = ((w << 6) & mask) | magic;
-        r1 = ((w << 4) & mask) | magic;
-        r2 = ((w << 2) & mask) | magic;
-        r3 = (w & mask) | magic;
+        r1 = ((w << 2) & mask) | magic;
+        r2 = ((w >> 2) & mask) | magic;
+        r3 = ((w >> 6) & mask) | magic;
+    } else {
+        r0 = ((w << 8) & mask) | magic;
+        r1 = ((w << 6) & mask) | magic;
+        r2 = ((w << 4) & mask) | magic;
+        r3 = ((w << 2) & mask) | magic;
     }
     return as_h8(r0, r1, r2, r3);
 }

@@ -1,0 +1,421 @@
+// Multi-query (prefill) attention over the packed prefix of a KIVI cache on MFMA, with the
+// packed tokens staged through LDS once per block of 64 query rows (gfx950, wave64).
+//
+// A block owns 64 query rows that share a kv head -- the GQA group at 64 / R consecutive
+// query positions -- as four waves of 16 rows, and walks the packed prefix in units of 32
+// tokens.  All 256 threads unpack the next unit into a double-buffered LDS tile while the
+// matrix unit works on the current one:
+//
+//   keys     the 4-/2-bit codes become fp16 "offset + code" values (one and-or per two codes,
+//            exact), channel order, [32 tokens][128 channels];
+//   values   the same, transposed to [128 channels][32 tokens].
+//
+// Both products run on the raw codes exactly as in the decode kernel, so no reconstructed
+// key or value is ever rounded to fp16.  Scores: the per-channel key scale of the open token
+// group is folded into the wave's 16 query rows (fp16 high part plus exact fp16 remainder,
+// two MFMAs into one accumulator), and the zero-point and offset terms seed the score
+// accumulator through a short MFMA chain.  Output: the per-token value scale of each
+// channel group is folded into the probabilities (high part plus exact remainder), the
+// offset and zero-point terms are extra MFMA tiles.  S^T[token, row] accumulators are
+// already the A operand of P.V; the softmax keeps a lazily updated reference maximum per
+// row; the denominator is an extra MFMA tile against ones.  Each wave owns its rows for the
+// whole run, so it writes its (max, sum, accumulator) partial straight to the workspace.
+// The un-quantised tail follows the packed units through the same pipeline (plain keys
+// against the plain query, plain values transposed into the value tile).  When there are
+// fewer blocks than the chip holds twice over, the work of a block is split into runs
+// handled by separate blocks; attend_merge_kernel combines the partials.
+#include "attend_mfma.hpp"
+
+namespace vq {
+
+#define VQ_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16((A), (B), (C), 0, 0, 0)
+
+constexpr int PF_KSTRIDE = MF_D + 8;   // fp16 per token row of the key-code tile (272 B: conflict-free b128 reads)
+constexpr int PF_VSTRIDE = 32 + 8;     // fp16 per channel row of the value tile (80 B)
+
+// four k-slot pair registers of one unpacked word -> the same eight values in code order
+__device__ __forceinline__ uint4 pairs_to_order(u32 r0, u32 r1, u32 r2, u32 r3) {
+    return make_uint4(pair_lo(r0, r1), pair_lo(r2, r3), pair_hi(r0, r1), pair_hi(r2, r3));
+}
+template <int BITS> __device__ __forceinline__ void unpack_pairs(u32 w, u32 magic, u32 (&r)[4]) {
+    const f16x8 h = unpack8<BITS>(w, magic);
+    const u32x4 v = __builtin_bit_cast(u32x4, h);
+    r[0] = v[0]; r[1] = v[1]; r[2] = v[2]; r[3] = v[3];
+}
+// One 4-bit word (8 codes) or one half of a 2-bit word -> values in code order.
+// 4-bit: codes 0..7 of the word.  2-bit: lo = codes 0..7, hi = codes 8..15 of the word.
+__device__ __forceinline__ uint4 word4_in_order(u32 w, u32 magic) {
+    u32 r[4];
+    unpack_pairs<4>(w, magic, r);   // pairs (0,4) (1,5) (2,6) (3,7)
+    return pairs_to_order(r[0], r[1], r[2], r[3]);
+}
+__device__ __forceinline__ void word2_in_order(u32 w, u32 magic, uint4 &lo, uint4 &hi) {
+    u32 a[4], b[4];
+    unpack_pairs<2>(w, magic, a);        // pairs (0,8) (1,9) (2,10) (3,11)
+    unpack_pairs<2>(w >> 8, magic, b);   // pairs (4,12) (5,13) (6,14) (7,15)
+    lo = make_uint4(pair_lo(a[0], a[1]), pair_lo(a[2], a[3]), pair_lo(b[0], b[1]), pair_lo(b[2], b[3]));
+    hi = make_uint4(pair_hi(a[0], a[1]), pair_hi(a[2], a[3]), pair_hi(b[0], b[1]), pair_hi(b[2], b[3]));
+}
+
+// packed words a thread fetches for one prefix unit before it unpacks them into LDS
+template <int BITS> struct PfStage {
+    u32 kw[BITS == 4 ? 2 : 1];   // key words: 16 channels of one token
+    u32 vw[BITS == 4 ? 2 : 1];   // value words: 16 tokens of one channel
+};
+
+// fp16 value scale / zero of a lane's eight consecutive tokens
+template <int GV> struct PfMeta {
+    uint4 s[GV];   // scales, every channel group (pair p = tokens 2p, 2p+1)
+    uint4 z;       // lane column n < GV: zeros of group n; otherwise scales of group n % GV
+};
+__device__ __forceinline__ u32 u4_at(const uint4 &v, int p) { return p == 0 ? v.x : p == 1 ? v.y : p == 2 ? v.z : v.w; }
+
+// token (0..31 of the unit) of S^T row i of tile T: accumulator register r of lane group blk is
+// token 8 blk + 2 r + T, so a lane's P pairs are eight consecutive tokens
+__device__ __forceinline__ int pf_tok(int blk, int r, int T) { return 8 * blk + 2 * r + T; }
+
+// grid (tiles, B*Hkv, nsplit).  The work of a block -- the packed units its rows see, then the
+// tail units -- is cut into nsplit equal runs; block z takes run z and writes partial slot z.
+// Scale / zero are fp16 (GV = channel groups per value row).
+template <int BITS, int GV>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restrict__ ws) {
+    __shared__ __align__(16) f16 s_k[2][32 * PF_KSTRIDE];
+    __shared__ __align__(16) f16 s_v[2][MF_D * PF_VSTRIDE];
+    __shared__ uint4 s_q[4][4][64];   // per wave: the query as B operand of k-step ks, lane-major
+
+    constexpr int PER = 32 / BITS;
+    constexpr int KW = MF_D / PER;
+    constexpr int gshift = GV == 4 ? 5 : GV == 2 ? 6 : 7;   // log2 of the group size
+    constexpr int TPG = 8 / GV;                             // value tiles per channel group
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, blk = lane >> 4;
+    const int64_t bh = blockIdx.y;
+    const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    const int R = (int)(a.Hq / a.Hkv);
+    const int64_t cap = a.cap_tokens;
+    const float c = a.scale * LOG2E;
+    const u32 magic = vreg_const(Magic<BITS>::bits);
+    const int pos0 = (int)blockIdx.x * qp;
+    const int64_t n_total = a.n_packed + a.n_tail;
+
+    // ---- this lane's query row (as a score column): row j = 16 wave + n of the block
+    const int j = 16 * wave + n;
+    const int64_t pos = pos0 + j % qp;
+    const bool row_ok = pos < a.Sq;
+    const int64_t qrow = (b * a.Hq + hkv * R + j / qp) * a.Sq + (row_ok ? pos : a.Sq - 1);
+    auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
+    const int64_t last_pos = pos0 + qp - 1 < a.Sq - 1 ? pos0 + qp - 1 : a.Sq - 1;
+    const int64_t vis_lane = visible(row_ok ? pos : a.Sq - 1), vis_min = visible(pos0), vis_max = visible(last_pos);
+    // packed tokens / tail tokens seen by this lane's row, by every row, by some row of the block
+    const int lane_vis = (int)(vis_lane < a.n_packed ? vis_lane : a.n_packed);
+    const int full_vis = (int)(vis_min < a.n_packed ? vis_min : a.n_packed);
+    const int max_vis = (int)(vis_max < a.n_packed ? vis_max : a.n_packed);
+    const int64_t tv_lane = vis_lane - a.n_packed, tv_min = vis_min - a.n_packed, tv_max = vis_max - a.n_packed;
+    const int lane_tvis = (int)(tv_lane < 0 ? 0 : tv_lane < a.n_tail ? tv_lane : a.n_tail);
+    const int full_tvis = (int)(tv_min < 0 ? 0 : tv_min < a.n_tail ? tv_min : a.n_tail);
+    const int max_tvis = (int)(tv_max < 0 ? 0 : tv_max < a.n_tail ? tv_max : a.n_tail);
+    const int n_punits = (max_vis + 31) / 32;
+    const int n_tunits = (max_tvis + 31) / 32;
+    const int n_work = n_punits + n_tunits;
+    const int nsplit = (int)gridDim.z, sp = (int)blockIdx.z;
+    const int w0 = (int)((int64_t)n_work * sp / nsplit), w1 = (int)((int64_t)n_work * (sp + 1) / nsplit);
+
+    // query as the B operand, parked in LDS: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of row n
+    {
+        f16x8 q8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) q8[e] = (f16)ldq(a.q, a.q_dtype, qrow * MF_D + 32 * ks + 8 * blk + e);
+            s_q[wave][ks][lane] = __builtin_bit_cast(uint4, q8);
+        }
+    }
+
+    // ---- producer side: block-uniform bases, per-thread offsets
+    const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
+    const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
+    const f16 *vsb = (const f16 *)a.v_scale + bh * GV * cap;
+    const f16 *vzb = (const f16 *)a.v_zero + bh * GV * cap;
+    const int kt = tid >> 3, kc = tid & 7;        // key tile: token, 16-channel chunk
+    const int vc = tid & 127, vh = tid >> 7;      // value tile: channel, 16-token half
+    const bool tail_bf16 = a.tail_dtype == VQ_BF16;
+    const int64_t tbase = bh * a.tail_cap * MF_D;
+    using Stage = PfStage<BITS>;
+    auto fetch = [&](int w, Stage &st) {   // packed work units only
+        if (w >= n_punits) return;
+        const int64_t base = (int64_t)w * 32;
+        if (BITS == 4) {
+            const uint2 x = *reinterpret_cast<const uint2 *>(kb + ((base + kt) * KW + 2 * kc) * 4);
+            st.kw[0] = x.x; st.kw[BITS == 4 ? 1 : 0] = x.y;
+            const char *p = vb + ((base / 8 + 2 * vh) * MF_D + vc) * 4;
+            st.vw[0] = *reinterpret_cast<const u32 *>(p);
+            st.vw[BITS == 4 ? 1 : 0] = *reinterpret_cast<const u32 *>(p + MF_D * 4);
+        } else {
+            st.kw[0] = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + kc) * 4);
+            st.vw[0] = *reinterpret_cast<const u32 *>(vb + ((base / 16 + vh) * MF_D + vc) * 4);
+        }
+    };
+    auto unpack_to_lds = [&](int w, const Stage &st, int buf) {
+        if (w < n_punits) {
+            // keys: 16 channels of token kt
+            uint4 k0, k1;
+            if (BITS == 4) { k0 = word4_in_order(st.kw[0], magic); k1 = word4_in_order(st.kw[BITS == 4 ? 1 : 0], magic); }
+            else word2_in_order(st.kw[0], magic, k0, k1);
+            uint4 *kd = reinterpret_cast<uint4 *>(&s_k[buf][kt * PF_KSTRIDE + 16 * kc]);
+            kd[0] = k0; kd[1] = k1;
+            // values: 16 tokens of channel vc, still codes
+            uint4 c0, c1;
+            if (BITS == 4) { c0 = word4_in_order(st.vw[0], magic); c1 = word4_in_order(st.vw[BITS == 4 ? 1 : 0], magic); }
+            else word2_in_order(st.vw[0], magic, c0, c1);
+            uint4 *vd = reinterpret_cast<uint4 *>(&s_v[buf][vc * PF_VSTRIDE + 16 * vh]);
+            vd[0] = c0; vd[1] = c1;
+        } else {
+            // tail unit (few per block, fetched here): plain key row chunk; value row chunk transposed
+            int64_t tok = (int64_t)(w - n_punits) * 32 + kt;
+            if (tok >= a.n_tail) tok = 0;   // masked in the softmax
+            const int64_t e0 = tbase + tok * MF_D + 16 * kc;
+            f16x8 *kd = reinterpret_cast<f16x8 *>(&s_k[buf][kt * PF_KSTRIDE + 16 * kc]);
+            kd[0] = ld_tail8(a.k_tail, e0, tail_bf16);
+            kd[1] = ld_tail8(a.k_tail, e0 + 8, tail_bf16);
+            const f16x8 v0 = ld_tail8(a.v_tail, e0, tail_bf16), v1 = ld_tail8(a.v_tail, e0 + 8, tail_bf16);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                s_v[buf][(16 * kc + e) * PF_VSTRIDE + kt] = v0[e];
+                s_v[buf][(16 * kc + 8 + e) * PF_VSTRIDE + kt] = v1[e];
+            }
+        }
+    };
+    // scale / zero of the lane's eight tokens of packed unit u
+    using Meta = PfMeta<GV>;
+    const f16 *vzs = (n < GV ? vzb : vsb) + (int64_t)(n % GV) * cap + 8 * blk;
+    auto fetch_meta = [&](int u, Meta &m) {
+        const int64_t t0 = (int64_t)u * 32;
+#pragma unroll
+        for (int g = 0; g < GV; ++g) m.s[g] = *reinterpret_cast<const uint4 *>(vsb + (int64_t)g * cap + t0 + 8 * blk);
+        m.z = *reinterpret_cast<const uint4 *>(vzs + t0);
+    };
+
+    // ---- consumer state
+    // O[nt]: channels 16 nt + n, still carrying off * sum_t P s_g; Z column g < GV = sum_t P[row, t] z_g[t],
+    // column GV + g = sum_t P[row, t] s_g[t]; L = sum_t P[row, t]
+    f32x4 O[8], Z = {0.f, 0.f, 0.f, 0.f}, L = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY;
+    f16x8 qh[4], ql[4];
+    f32x4 bias = {0.f, 0.f, 0.f, 0.f};
+    const f16x8 ones = ones8();
+    const f16x8 negoff = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair,
+                               Magic<BITS>::neg_off_pair);
+    const f16 *ksb = (const f16 *)a.k_scale + bh * (cap >> gshift) * MF_D + 8 * blk;
+    const f16 *kzb = (const f16 *)a.k_zero + bh * (cap >> gshift) * MF_D + 8 * blk;
+
+    // fold the key scales of a token group into the query rows; seed the scores with
+    // sum_d z_d q_d - off * sum_d (q s)_d
+    auto open_group = [&](int64_t grp) {
+        f32x4 bt = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const f16x8 s = as_h8(*reinterpret_cast<const uint4 *>(ksb + grp * MF_D + 32 * ks));
+            const f16x8 z = as_h8(*reinterpret_cast<const uint4 *>(kzb + grp * MF_D + 32 * ks));
+            const f16x8 q8 = as_h8(s_q[wave][ks][lane]);
+            bt = VQ_MFMA(z, q8, bt);
+            const f16x8 hi = q8 * s;
+            // q*s has at most 22 significant bits: its remainder after the fp16 high part is
+            // itself an fp16 number, so this fma is exact
+            qh[ks] = hi;
+            ql[ks] = __builtin_elementwise_fma(q8, s, -hi);
+            bt = VQ_MFMA(negoff, qh[ks], bt);
+            bt = VQ_MFMA(negoff, ql[ks], bt);
+        }
+        bias = bt;
+    };
+
+    // softmax of one unit against the lazily updated reference; returns P as the A operand
+    // (pair r = tokens 8 blk + 2 r, 8 blk + 2 r + 1).  Tokens at or past `lim` are masked when
+    // the unit reaches past `full`.
+    auto softmax = [&](f32x4 (&S)[2], int base, int lim, int full, u32 (&P)[4]) {
+        if (base + 32 > full) {
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (base + pf_tok(blk, r, T) >= lim) S[T][r] = -INFINITY;
+        }
+        const float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
+                               fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
+        if (__any(mx * c > m_run + RESCALE_SLACK)) {
+            float m_seen = mx * c;
+            m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 16));
+            m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 32));
+            const float m_new = fmaxf(m_run, m_seen);
+            const float alpha = m_new == -INFINITY ? 1.f : exp2f(m_run - m_new);
+            float al[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) O[nt][r] *= al[r];
+                Z[r] *= al[r];
+                L[r] *= al[r];
+            }
+            m_run = m_new;
+        }
+        const float nm = m_run == -INFINITY ? 0.f : -m_run;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            P[r] = as_u(f16x2{(f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], c, nm)),
+                              (f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], c, nm))});
+    };
+
+    auto compute_packed = [&](int buf, int base, const Meta &vm) {
+        // two accumulator chains per score tile (high and remainder part of the folded query)
+        f32x4 S[2], Sl[2];
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            const f16 *kr = &s_k[buf][pf_tok(n >> 2, n & 3, T) * PF_KSTRIDE + 8 * blk];
+            Sl[T] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const f16x8 A = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
+                S[T] = VQ_MFMA(A, qh[ks], ks == 0 ? bias : S[T]);
+                Sl[T] = VQ_MFMA(A, ql[ks], Sl[T]);
+            }
+            S[T] += Sl[T];
+        }
+        u32 P[4];
+        softmax(S, base, lane_vis, full_vis, P);
+        const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
+        // per channel group: A = P * s_g as fp16 high part plus exact fp16 remainder
+#pragma unroll
+        for (int g = 0; g < GV; ++g) {
+            u32 ah[4], al[4];
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const f16x2 sp2 = as_h2(u4_at(vm.s[g], p));
+                const f16x2 hi = as_h2(P[p]) * sp2;
+                ah[p] = as_u(hi);
+                al[p] = as_u(__builtin_elementwise_fma(as_h2(P[p]), sp2, -hi));
+            }
+            const f16x8 Ah = as_h8(ah[0], ah[1], ah[2], ah[3]), Al = as_h8(al[0], al[1], al[2], al[3]);
+#pragma unroll
+            for (int jt = 0; jt < TPG; ++jt) {
+                const int nt = g * TPG + jt;
+                const f16x8 Bv = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+                O[nt] = VQ_MFMA(Ah, Bv, O[nt]);
+                O[nt] = VQ_MFMA(Al, Bv, O[nt]);
+            }
+        }
+        Z = VQ_MFMA(P8, as_h8(vm.z), Z);
+        L = VQ_MFMA(P8, ones, L);
+    };
+    // tail unit: plain keys against the plain query, plain values
+    auto compute_tail = [&](int buf, int tok0) {
+        f32x4 S[2];
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            const f16 *kr = &s_k[buf][pf_tok(n >> 2, n & 3, T) * PF_KSTRIDE + 8 * blk];
+            S[T] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+                S[T] = VQ_MFMA(*reinterpret_cast<const f16x8 *>(kr + 32 * ks), as_h8(s_q[wave][ks][lane]), S[T]);
+        }
+        u32 P[4];
+        softmax(S, tok0, lane_tvis, full_tvis, P);
+        const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt)
+            O[nt] = VQ_MFMA(P8, *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]), O[nt]);
+        L = VQ_MFMA(P8, ones, L);
+    };
+
+    // ---- pipeline over the work units [w0, w1): registers hold the packed words of unit w+1
+    // while unit w is computed from LDS
+    Stage st;
+    if (w1 > w0) {
+        fetch(w0, st);
+        unpack_to_lds(w0, st, 0);
+        __syncthreads();
+        if (w0 + 1 < w1) fetch(w0 + 1, st);
+    }
+    int cur_group = -1;
+    for (int w = w0; w < w1; ++w) {
+        const int buf = (w - w0) & 1;
+        if (w < n_punits) {
+            const int base = w * 32;
+            Meta vm;
+            fetch_meta(w, vm);   // used after the score products
+            if ((base >> gshift) != cur_group) {
+                cur_group = base >> gshift;
+                open_group(cur_group);
+            }
+            compute_packed(buf, base, vm);
+        } else {
+            compute_tail(buf, (w - n_punits) * 32);
+        }
+        if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
+        __syncthreads();
+        if (w + 2 < w1) fetch(w + 2, st);
+    }
+
+    // ---- every wave owns its 16 rows: accumulator register r of lane (n, blk) is row 4 blk + r,
+    // tile nt column n is channel 16 nt + n; the row's reference maximum sits in lane 4 blk + r
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int jr = 16 * wave + 4 * blk + r;
+        const int64_t pr = pos0 + jr % qp;
+        const float mr = __shfl(m_run, 4 * blk + r);
+        float zs[GV], ss[GV];   // zero-point and scale sums of this row: columns g and GV + g of the Z tile
+#pragma unroll
+        for (int g = 0; g < GV; ++g) {
+            zs[g] = __shfl(Z[r], 16 * blk + g);
+            ss[g] = __shfl(Z[r], 16 * blk + GV + g);
+        }
+        if (pr < a.Sq) {
+            const int64_t row = (b * a.Hq + hkv * R + jr / qp) * a.Sq + pr;
+            float *o = ws + (row * nparts + sp) * MF_PART;
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) o[2 + 16 * nt + n] = (O[nt][r] - Magic<BITS>::off * ss[nt / TPG]) + zs[nt / TPG];
+            if (n == 0) { o[0] = mr * LN2; o[1] = L[r]; }
+        }
+    }
+}
+
+bool mfma_prefill_supported(const vq_attend_args &a) {
+    if (a.D != MF_D || a.n_packed <= 0 || a.Sq < 16) return false;
+    if (a.Hq % a.Hkv != 0) return false;
+    const int64_t R = a.Hq / a.Hkv;
+    if (!(R == 1 || R == 2 || R == 4 || R == 8)) return false;
+    if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
+    if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
+    if (a.meta_dtype != VQ_F16) return false;   // float32 scale / zero stays on the 8-row tiles of the decode kernel
+    if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
+    if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
+    if (!(a.scale > 0.f)) return false;
+    if (a.n_tail > 0 && (!(a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
+    if (a.B * a.Hkv > 65535) return false;
+    if (a.n_tail > 0 && a.tail_cap * MF_D % 8 != 0) return false;
+    const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
+                         (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
+    if (al & 15u) return false;
+    return true;
+}
+
+void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
+    hipStream_t st = (hipStream_t)a.stream;
+    float *ws = (float *)a.workspace;
+    const int R = (int)(a.Hq / a.Hkv);
+    const int qp = 64 / R, tiles = (int)cdiv(a.Sq, qp);
+    const int gv = (int)(MF_D / a.group);
+    const dim3 grid((unsigned)tiles, (unsigned)(a.B * a.Hkv), (unsigned)p.nsplit), block(256);
+#define VQ_LAUNCH(BITS, GV) \
+    hipLaunchKernelGGL((attend_prefill_kernel<BITS, GV>), grid, block, 0, st, a, qp, p.nparts, ws)
+    if (a.pack_bits == 4) { if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4); }
+    else { if (gv == 1) VQ_LAUNCH(2, 1); else if (gv == 2) VQ_LAUNCH(2, 2); else VQ_LAUNCH(2, 4); }
+#undef VQ_LAUNCH
+}
+
+}  // namespace vq
