@@ -20,8 +20,9 @@
 // already the A operand of P.V; the softmax keeps a lazily updated reference maximum per
 // row; the denominator is an extra MFMA tile against ones.  Each wave owns its rows for the
 // whole run, so it writes its (max, sum, accumulator) partial straight to the workspace.
-// The un-quantised tail follows the packed units through the same pipeline (plain keys
-// against the plain query, plain values transposed into the value tile).  When there are
+// The un-quantised tail follows the packed units through the same pipeline and the same
+// code: its tiles hold plain keys and (transposed) plain values, and the scale / zero / offset
+// staged with them are 1 / 0 / 0.  When there are
 // fewer blocks than the chip holds twice over, the work of a block is split into runs
 // handled by separate blocks; attend_merge_kernel combines the partials.
 #include "attend_mfma.hpp"
@@ -61,6 +62,7 @@ __device__ __forceinline__ void word2_in_order(u32 w, u32 magic, uint4 &lo, uint
 template <int BITS> struct PfStage {
     u32 kw[BITS == 4 ? 2 : 1];   // key words: 16 channels of one token
     u32 vw[BITS == 4 ? 2 : 1];   // value words: 16 tokens of one channel
+    uint4 meta;                  // threads 0..63: one 16-byte piece of the unit's scale / zero
 };
 
 // fp16 value scale / zero of a lane's eight consecutive tokens
@@ -73,6 +75,9 @@ __device__ __forceinline__ u32 u4_at(const uint4 &v, int p) { return p == 0 ? v.
 // token (0..31 of the unit) of S^T row i of tile T: accumulator register r of lane group blk is
 // token 8 blk + 2 r + T, so a lane's P pairs are eight consecutive tokens
 __device__ __forceinline__ int pf_tok(int blk, int r, int T) { return 8 * blk + 2 * r + T; }
+// LDS row of token t in the key tile: even tokens first, so that the sixteen rows one score
+// tile reads (tokens of equal parity) are consecutive and the b128 reads are conflict-free
+__device__ __forceinline__ int pf_krow(int t) { return (t >> 1) + 16 * (t & 1); }
 
 // grid (tiles, B*Hkv, nsplit).  The work of a block -- the packed units its rows see, then the
 // tail units -- is cut into nsplit equal runs; block z takes run z and writes partial slot z.
@@ -82,7 +87,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restrict__ ws) {
     __shared__ __align__(16) f16 s_k[2][32 * PF_KSTRIDE];
     __shared__ __align__(16) f16 s_v[2][MF_D * PF_VSTRIDE];
-    __shared__ uint4 s_q[4][4][64];   // per wave: the query as B operand of k-step ks, lane-major
+    // What turns the unit's tile into keys and values, staged with it: keys [scale | zero |
+    // minus the code offset][128 channels] of its token group, values [scale | zero | scale as
+    // the offset correction sees it][GV][32 tokens].  A tail unit holds plain values: scale 1,
+    // zero 0, no offset.
+    __shared__ __align__(16) f16 s_km[2][3][MF_D];
+    __shared__ __align__(16) f16 s_vm[2][3][GV][32];
 
     constexpr int PER = 32 / BITS;
     constexpr int KW = MF_D / PER;
@@ -122,20 +132,18 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     const int nsplit = (int)gridDim.z, sp = (int)blockIdx.z;
     const int w0 = (int)((int64_t)n_work * sp / nsplit), w1 = (int)((int64_t)n_work * (sp + 1) / nsplit);
 
-    // query as the B operand, parked in LDS: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of row n
-    {
-        f16x8 q8;
+    // query as the B operand: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of row n
+    f16x8 qn[4];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+    for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) q8[e] = (f16)ldq(a.q, a.q_dtype, qrow * MF_D + 32 * ks + 8 * blk + e);
-            s_q[wave][ks][lane] = __builtin_bit_cast(uint4, q8);
-        }
-    }
+        for (int e = 0; e < 8; ++e) qn[ks][e] = (f16)ldq(a.q, a.q_dtype, qrow * MF_D + 32 * ks + 8 * blk + e);
 
     // ---- producer side: block-uniform bases, per-thread offsets
     const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
     const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
+    const f16 *ksb = (const f16 *)a.k_scale + bh * (cap >> gshift) * MF_D;
+    const f16 *kzb = (const f16 *)a.k_zero + bh * (cap >> gshift) * MF_D;
     const f16 *vsb = (const f16 *)a.v_scale + bh * GV * cap;
     const f16 *vzb = (const f16 *)a.v_zero + bh * GV * cap;
     const int kt = tid >> 3, kc = tid & 7;        // key tile: token, 16-channel chunk
@@ -156,6 +164,13 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
             st.kw[0] = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + kc) * 4);
             st.vw[0] = *reinterpret_cast<const u32 *>(vb + ((base / 16 + vh) * MF_D + vc) * 4);
         }
+        if (tid < 32) {          // key scale (pieces 0..15) and zero (16..31) of the unit's token group
+            const f16 *src = (tid < 16 ? ksb : kzb) + (base >> gshift) * MF_D + 8 * (tid & 15);
+            st.meta = *reinterpret_cast<const uint4 *>(src);
+        } else if (tid < 32 + 12 * GV) {   // value scale | zero | scale again: piece = (which, group, 8-token chunk)
+            const int pc = tid - 32, which = pc / (4 * GV), g = (pc / 4) % GV, ch = pc % 4;
+            st.meta = *reinterpret_cast<const uint4 *>((which == 1 ? vzb : vsb) + (int64_t)g * cap + base + 8 * ch);
+        }
     };
     auto unpack_to_lds = [&](int w, const Stage &st, int buf) {
         if (w < n_punits) {
@@ -163,7 +178,7 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
             uint4 k0, k1;
             if (BITS == 4) { k0 = word4_in_order(st.kw[0], magic); k1 = word4_in_order(st.kw[BITS == 4 ? 1 : 0], magic); }
             else word2_in_order(st.kw[0], magic, k0, k1);
-            uint4 *kd = reinterpret_cast<uint4 *>(&s_k[buf][kt * PF_KSTRIDE + 16 * kc]);
+            uint4 *kd = reinterpret_cast<uint4 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 16 * kc]);
             kd[0] = k0; kd[1] = k1;
             // values: 16 tokens of channel vc, still codes
             uint4 c0, c1;
@@ -171,12 +186,20 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
             else word2_in_order(st.vw[0], magic, c0, c1);
             uint4 *vd = reinterpret_cast<uint4 *>(&s_v[buf][vc * PF_VSTRIDE + 16 * vh]);
             vd[0] = c0; vd[1] = c1;
+            if (tid < 32) *reinterpret_cast<uint4 *>(&s_km[buf][tid >> 4][8 * (tid & 15)]) = st.meta;
+            else if (tid < 32 + 12 * GV) {
+                const int pc = tid - 32;
+                *reinterpret_cast<uint4 *>(&s_vm[buf][pc / (4 * GV)][(pc / 4) % GV][8 * (pc % 4)]) = st.meta;
+            } else if (tid == 255) {
+                const u32 no = Magic<BITS>::neg_off_pair;
+                *reinterpret_cast<uint4 *>(&s_km[buf][2][0]) = make_uint4(no, no, no, no);
+            }
         } else {
             // tail unit (few per block, fetched here): plain key row chunk; value row chunk transposed
             int64_t tok = (int64_t)(w - n_punits) * 32 + kt;
             if (tok >= a.n_tail) tok = 0;   // masked in the softmax
             const int64_t e0 = tbase + tok * MF_D + 16 * kc;
-            f16x8 *kd = reinterpret_cast<f16x8 *>(&s_k[buf][kt * PF_KSTRIDE + 16 * kc]);
+            f16x8 *kd = reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 16 * kc]);
             kd[0] = ld_tail8(a.k_tail, e0, tail_bf16);
             kd[1] = ld_tail8(a.k_tail, e0 + 8, tail_bf16);
             const f16x8 v0 = ld_tail8(a.v_tail, e0, tail_bf16), v1 = ld_tail8(a.v_tail, e0 + 8, tail_bf16);
@@ -185,16 +208,22 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
                 s_v[buf][(16 * kc + e) * PF_VSTRIDE + kt] = v0[e];
                 s_v[buf][(16 * kc + 8 + e) * PF_VSTRIDE + kt] = v1[e];
             }
+            const uint4 one8 = make_uint4(0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u), zero8 = make_uint4(0, 0, 0, 0);
+            if (tid < 32) *reinterpret_cast<uint4 *>(&s_km[buf][tid >> 4][8 * (tid & 15)]) = tid < 16 ? one8 : zero8;
+            else if (tid < 32 + 12 * GV) {
+                const int pc = tid - 32, which = pc / (4 * GV);
+                *reinterpret_cast<uint4 *>(&s_vm[buf][which][(pc / 4) % GV][8 * (pc % 4)]) = which == 0 ? one8 : zero8;
+            } else if (tid == 255) {
+                *reinterpret_cast<uint4 *>(&s_km[buf][2][0]) = zero8;
+            }
         }
     };
-    // scale / zero of the lane's eight tokens of packed unit u
+    // scale / zero of the lane's eight tokens of the unit staged in buffer buf
     using Meta = PfMeta<GV>;
-    const f16 *vzs = (n < GV ? vzb : vsb) + (int64_t)(n % GV) * cap + 8 * blk;
-    auto fetch_meta = [&](int u, Meta &m) {
-        const int64_t t0 = (int64_t)u * 32;
+    auto fetch_meta = [&](int buf, Meta &m) {
 #pragma unroll
-        for (int g = 0; g < GV; ++g) m.s[g] = *reinterpret_cast<const uint4 *>(vsb + (int64_t)g * cap + t0 + 8 * blk);
-        m.z = *reinterpret_cast<const uint4 *>(vzs + t0);
+        for (int g = 0; g < GV; ++g) m.s[g] = *reinterpret_cast<const uint4 *>(&s_vm[buf][0][g][8 * blk]);
+        m.z = *reinterpret_cast<const uint4 *>(&s_vm[buf][n < GV ? 1 : 2][n % GV][8 * blk]);
     };
 
     // ---- consumer state
@@ -207,36 +236,37 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     f16x8 qh[4], ql[4];
     f32x4 bias = {0.f, 0.f, 0.f, 0.f};
     const f16x8 ones = ones8();
-    const f16x8 negoff = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair,
-                               Magic<BITS>::neg_off_pair);
-    const f16 *ksb = (const f16 *)a.k_scale + bh * (cap >> gshift) * MF_D + 8 * blk;
-    const f16 *kzb = (const f16 *)a.k_zero + bh * (cap >> gshift) * MF_D + 8 * blk;
 
     // fold the key scales of a token group into the query rows; seed the scores with
     // sum_d z_d q_d - off * sum_d (q s)_d
-    auto open_group = [&](int64_t grp) {
-        f32x4 bt = {0.f, 0.f, 0.f, 0.f};
+    auto open_group = [&](int buf) {
+        // three short MFMA chains (zeros, high part, remainder) instead of one long one
+        f32x4 bz = {0.f, 0.f, 0.f, 0.f}, bh_ = {0.f, 0.f, 0.f, 0.f}, bl = {0.f, 0.f, 0.f, 0.f};
+        const f16x8 negoff = as_h8(*reinterpret_cast<const uint4 *>(&s_km[buf][2][0]));   // all lanes alike
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            const f16x8 s = as_h8(*reinterpret_cast<const uint4 *>(ksb + grp * MF_D + 32 * ks));
-            const f16x8 z = as_h8(*reinterpret_cast<const uint4 *>(kzb + grp * MF_D + 32 * ks));
-            const f16x8 q8 = as_h8(s_q[wave][ks][lane]);
-            bt = VQ_MFMA(z, q8, bt);
+            const f16x8 s = as_h8(*reinterpret_cast<const uint4 *>(&s_km[buf][0][32 * ks + 8 * blk]));
+            const f16x8 z = as_h8(*reinterpret_cast<const uint4 *>(&s_km[buf][1][32 * ks + 8 * blk]));
+            const f16x8 q8 = qn[ks];
+            bz = VQ_MFMA(z, q8, bz);
             const f16x8 hi = q8 * s;
             // q*s has at most 22 significant bits: its remainder after the fp16 high part is
             // itself an fp16 number, so this fma is exact
             qh[ks] = hi;
             ql[ks] = __builtin_elementwise_fma(q8, s, -hi);
-            bt = VQ_MFMA(negoff, qh[ks], bt);
-            bt = VQ_MFMA(negoff, ql[ks], bt);
+            bh_ = VQ_MFMA(negoff, qh[ks], bh_);
+            bl = VQ_MFMA(negoff, ql[ks], bl);
         }
-        bias = bt;
+        bias = (bz + bh_) + bl;
     };
 
-    // softmax of one unit against the lazily updated reference; returns P as the A operand
-    // (pair r = tokens 8 blk + 2 r, 8 blk + 2 r + 1).  Tokens at or past `lim` are masked when
-    // the unit reaches past `full`.
-    auto softmax = [&](f32x4 (&S)[2], int base, int lim, int full, u32 (&P)[4]) {
+    // Softmax of one unit against the lazily updated reference.  Tokens at or past `lim` are
+    // masked when the unit reaches past `full`.  Returns false, having done nothing but note the
+    // new maxima in m_seen, when some row's scores outgrow the reference: the caller rescales
+    // and repeats the unit.  Otherwise P is the A operand of the second product (pair r =
+    // tokens 8 blk + 2 r, 8 blk + 2 r + 1).
+    float m_seen = -INFINITY;
+    auto softmax = [&](f32x4 (&S)[2], int base, int lim, int full, u32 (&P)[4]) -> bool {
         if (base + 32 > full) {
 #pragma unroll
             for (int T = 0; T < 2; ++T)
@@ -247,36 +277,42 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
         const float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
                                fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
         if (__any(mx * c > m_run + RESCALE_SLACK)) {
-            float m_seen = mx * c;
-            m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 16));
-            m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 32));
-            const float m_new = fmaxf(m_run, m_seen);
-            const float alpha = m_new == -INFINITY ? 1.f : exp2f(m_run - m_new);
-            float al[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-#pragma unroll
-                for (int nt = 0; nt < 8; ++nt) O[nt][r] *= al[r];
-                Z[r] *= al[r];
-                L[r] *= al[r];
-            }
-            m_run = m_new;
+            m_seen = mx * c;
+            return false;
         }
         const float nm = m_run == -INFINITY ? 0.f : -m_run;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
             P[r] = as_u(f16x2{(f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], c, nm)),
                               (f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], c, nm))});
+        return true;
+    };
+    // move the reference of every row up to what it has seen and rescale the accumulators
+    auto rescale = [&]() {
+        float ms = m_seen;
+        ms = fmaxf(ms, __shfl_xor(ms, 16));
+        ms = fmaxf(ms, __shfl_xor(ms, 32));
+        const float m_new = fmaxf(m_run, ms);
+        const float alpha = m_new == -INFINITY ? 1.f : exp2f(m_run - m_new);
+        float al[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) O[nt][r] *= al[r];
+            Z[r] *= al[r];
+            L[r] *= al[r];
+        }
+        m_run = m_new;
     };
 
-    auto compute_packed = [&](int buf, int base, const Meta &vm) {
+    auto compute = [&](int buf, int base, int lim, int full, const Meta &vm) -> bool {
         // two accumulator chains per score tile (high and remainder part of the folded query)
         f32x4 S[2], Sl[2];
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
-            const f16 *kr = &s_k[buf][pf_tok(n >> 2, n & 3, T) * PF_KSTRIDE + 8 * blk];
+            const f16 *kr = &s_k[buf][pf_krow(pf_tok(n >> 2, n & 3, T)) * PF_KSTRIDE + 8 * blk];
             Sl[T] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
@@ -287,7 +323,7 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
             S[T] += Sl[T];
         }
         u32 P[4];
-        softmax(S, base, lane_vis, full_vis, P);
+        if (!softmax(S, base, lim, full, P)) return false;
         const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
         // per channel group: A = P * s_g as fp16 high part plus exact fp16 remainder
 #pragma unroll
@@ -311,29 +347,14 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
         }
         Z = VQ_MFMA(P8, as_h8(vm.z), Z);
         L = VQ_MFMA(P8, ones, L);
+        return true;
     };
-    // tail unit: plain keys against the plain query, plain values
-    auto compute_tail = [&](int buf, int tok0) {
-        f32x4 S[2];
-#pragma unroll
-        for (int T = 0; T < 2; ++T) {
-            const f16 *kr = &s_k[buf][pf_tok(n >> 2, n & 3, T) * PF_KSTRIDE + 8 * blk];
-            S[T] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-                S[T] = VQ_MFMA(*reinterpret_cast<const f16x8 *>(kr + 32 * ks), as_h8(s_q[wave][ks][lane]), S[T]);
-        }
-        u32 P[4];
-        softmax(S, tok0, lane_tvis, full_tvis, P);
-        const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
-#pragma unroll
-        for (int nt = 0; nt < 8; ++nt)
-            O[nt] = VQ_MFMA(P8, *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]), O[nt]);
-        L = VQ_MFMA(P8, ones, L);
-    };
-
     // ---- pipeline over the work units [w0, w1): registers hold the packed words of unit w+1
     // while unit w is computed from LDS
+    // Iteration w: unpack unit w+1 (fetched during iteration w-1) into the other buffer, start
+    // the fetch of unit w+2, then compute unit w; the barrier at the end makes unit w+1 visible
+    // and frees the buffer of unit w.  A unit whose scores outgrow the softmax reference is
+    // repeated after a rescale (a handful of times per wave) without touching the pipeline.
     Stage st;
     if (w1 > w0) {
         fetch(w0, st);
@@ -342,23 +363,32 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
         if (w0 + 1 < w1) fetch(w0 + 1, st);
     }
     int cur_group = -1;
-    for (int w = w0; w < w1; ++w) {
+    bool staged = false;   // unit w+1 already unpacked (set while a unit is being repeated)
+    for (int w = w0; w < w1;) {
         const int buf = (w - w0) & 1;
-        if (w < n_punits) {
-            const int base = w * 32;
-            Meta vm;
-            fetch_meta(w, vm);   // used after the score products
-            if ((base >> gshift) != cur_group) {
-                cur_group = base >> gshift;
-                open_group(cur_group);
-            }
-            compute_packed(buf, base, vm);
-        } else {
-            compute_tail(buf, (w - n_punits) * 32);
+        if (!staged) {
+            if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
+            if (w + 2 < w1) fetch(w + 2, st);
+            staged = true;
         }
-        if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
+        // a tail unit runs through the same code: its staged scale / zero / offset make the
+        // products plain ones
+        const bool packed = w < n_punits;
+        const int base = packed ? w * 32 : (w - n_punits) * 32;
+        const int grp = packed ? (base >> gshift) : -2;
+        Meta vm;
+        fetch_meta(buf, vm);
+        if (grp != cur_group) {
+            cur_group = grp;
+            open_group(buf);
+        }
+        if (!compute(buf, base, packed ? lane_vis : lane_tvis, packed ? full_vis : full_tvis, vm)) {
+            rescale();
+            continue;
+        }
         __syncthreads();
-        if (w + 2 < w1) fetch(w + 2, st);
+        staged = false;
+        ++w;
     }
 
     // ---- every wave owns its 16 rows: accumulator register r of lane (n, blk) is row 4 blk + r,
