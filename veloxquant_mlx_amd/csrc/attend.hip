@@ -35,9 +35,9 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     }
     const int64_t max_splits = n_split > 0 ? cdiv(n_split, 64) : 1;
     // units of parallel work before splitting: a wave per query row (generic)
-    // or a four-wave block per kv head (MFMA)
+    // or an eight-wave block per kv head (MFMA)
     const int64_t units = p.path == 1 ? a.B * a.Hkv * p.tiles : a.B * a.Hq * a.Sq;
-    const int64_t target = p.path == 1 ? 512 : 4096;
+        const int64_t target = p.path == 1 ? 256 : 4096;   // MFMA path: one eight-wave block per CU
     int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);   // < 0: choose as well
     if (ns > max_splits) ns = max_splits;
     if (ns > 512) ns = 512;

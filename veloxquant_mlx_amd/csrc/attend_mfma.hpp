@@ -106,6 +106,40 @@ template <typename T> __device__ __forceinline__ T ldg(const char *base, u32 off
     return *reinterpret_cast<const T *>(base + off);
 }
 
+// ---- asynchronous copies from global memory straight into LDS (no register in between).
+// Lane l's BYTES bytes land at LDS address  lds + OFF + BYTES * l  and come from global address
+// base + voff + OFF (base wave-uniform, voff a 32-bit per-lane byte offset); the instruction
+// offset OFF applies to both sides.  The optimiser sees neither the LDS write nor the
+// outstanding-load counter of these copies: a caller orders them against its LDS reads with
+// wait_copies<N>(), which returns once at most N of the wave's copies are still in flight
+// (they complete in issue order) and is a compiler barrier for memory.  m0 carries the LDS
+// address; the compiler itself does not use m0 in these kernels.
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+// a wave-uniform value the register allocator must keep in scalar registers
+__device__ __forceinline__ u32 uniform(u32 x) { return (u32)__builtin_amdgcn_readfirstlane((int)x); }
+__device__ __forceinline__ const void *uniform(const void *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    return (const void *)(uintptr_t)(((uint64_t)uniform((u32)(v >> 32)) << 32) | uniform((u32)v));
+}
+template <int OFF> __device__ __forceinline__ void lds_copy16(const void *base, u32 voff, u32 lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :: "v"(voff), "s"(uniform(base)), "s"(uniform(lds)), "n"(OFF) : "memory", "m0");
+}
+template <int OFF> __device__ __forceinline__ void lds_copy4(const void *base, u32 voff, u32 lds) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1 offset:%3"
+                 :: "v"(voff), "s"(uniform(base)), "s"(uniform(lds)), "n"(OFF) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+template <int N> __device__ __forceinline__ void wait_copies() {
+    static_assert(N >= 0 && N < 64, "the counter has six bits");
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory");
+}
+// LDS byte address of a pointer into block-shared memory
+__device__ __forceinline__ u32 lds_addr(const void *p) {
+    return (u32)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
 // The query rows one block works on: RT = R * PQ rows that share a kv head, namely the R
 // heads of the GQA group at PQ consecutive query positions starting at pos0.  Tile row
 // j is head j % R at position pos0 + j / R.  Decode (Sq == 1) is the case PQ == 1.
@@ -192,9 +226,10 @@ __device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool b
     return o;
 }
 
-// s_m, s_l: [4][MF_ROWS] floats; s_o: [4][MF_ROWS][MF_D] floats of block-shared memory.
-// s_qraw: the query rows of this kv head as fp16 [MF_ROWS][MF_D] (rows >= R zero); it may
-// alias s_o: it is read into registers before s_o is written.
+// NW waves per block.  s_m, s_l: [NW][MF_ROWS] floats; s_o: [NW][MF_ROWS][MF_D] floats of
+// block-shared memory.  s_qraw: the query rows of this kv head as fp16 [MF_ROWS][MF_D] (rows >= R
+// zero); it may alias s_o: it is read into registers before s_o is written.
+template <int NW>
 __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, const RowTile &tile, float c, int slot,
                                            int nparts, float *__restrict__ ws, float *s_m, float *s_l, float *s_o,
                                            const f16 *s_qraw, int tid, int wave, bool device_scope) {
@@ -260,15 +295,15 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
         acc.O[8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(P, ones, acc.O[8], 0, 0, 0);
     };
     // two units of a wave in flight at a time
-    for (int u = wave; u < n_tu; u += 8) {
+    for (int u = wave; u < n_tu; u += 2 * NW) {
         TUnit d0, d1;
         load(u, d0);
-        if (u + 4 < n_tu) load(u + 4, d1);
+        if (u + NW < n_tu) load(u + NW, d1);
         compute(u, d0);
-        if (u + 4 < n_tu) compute(u + 4, d1);
+        if (u + NW < n_tu) compute(u + NW, d1);
     }
 
-    // merge the four waves: accumulator register r of lane (i, blk) is row 4*blk + r, channel 8*i + nt
+    // merge the waves: accumulator register r of lane (i, blk) is row 4*blk + r, channel 8*i + nt
     if (blk == 0) s_m[wave * MF_ROWS + i] = acc.m_run;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -280,14 +315,14 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
         }
     }
     __syncthreads();
-    for (int e = tid; e < R * MF_D; e += 256) {
+    for (int e = tid; e < R * MF_D; e += 64 * NW) {
         const int row = e / MF_D, d = e % MF_D;
         float gm = -INFINITY;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) gm = fmaxf(gm, s_m[w * MF_ROWS + row]);
+        for (int w = 0; w < NW; ++w) gm = fmaxf(gm, s_m[w * MF_ROWS + row]);
         float num = 0.f, den = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < NW; ++w) {
             const float mw = s_m[w * MF_ROWS + row];
             if (mw == -INFINITY) continue;
             const float f = exp2f(mw - gm);
@@ -306,8 +341,8 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
 // arithmetic of attend_merge_kernel, which shares merge_partials).  Partials written by
 // other blocks of this launch are read with device-scope loads.
 __device__ __forceinline__ void merge_rows(const vq_attend_args &a, const RowTile &tile, int nparts, const float *ws,
-                                           int tid) {
-    for (int e = tid; e < tile.RT * MF_D; e += 256) {
+                                           int tid, int nthreads) {
+    for (int e = tid; e < tile.RT * MF_D; e += nthreads) {
         const int j = e / MF_D, d = e % MF_D;
         if (!tile.valid(j)) continue;
         const int64_t row = tile.row(j);

@@ -1,7 +1,7 @@
 // MFMA decode attention over the packed prefix of a KIVI cache (gfx950, wave64).
 //
-// One block of four waves per (kv head, token split).  Every wave streams units of
-// 32 tokens and never reconstructs a key or a value: both products run on the raw
+// One block of eight waves per (kv head, token split), one block per CU.  Every wave streams
+// units of 32 tokens and never reconstructs a key or a value: both products run on the raw
 // codes, which are dropped from the packed word into the mantissa of an fp16
 // constant by one and-or per two codes (value = offset + code, exact), and every
 // affine term is pushed onto the matrix unit:
@@ -34,23 +34,29 @@
 // tokens of one channel; token rows of the two score tiles interleave so that the
 // accumulator layout of S^T is the A-operand layout of P.
 //
-// Loads run one unit ahead in registers (two unit buffers used alternately); the
-// softmax keeps a lazily updated reference maximum, so the common path has no
-// cross-lane traffic at all.
+// Every wave streams its units through its own ring of LDS slots, filled by copies
+// that go from global memory straight into LDS and run DEPTH - 1 units ahead of the
+// arithmetic: the bytes in flight per wave are set by the ring, not by the register
+// file, and a unit is read into registers only when its turn comes.  The softmax
+// keeps a lazily updated reference maximum, so the common path has no cross-lane
+// traffic at all.
 #pragma once
 #include "attend_mfma.hpp"
 
 namespace vq {
 
+// One block of PK_WAVES waves per CU (two waves per SIMD, the register file split in two).
+constexpr int PK_WAVES = 8;
+constexpr int PK_THREADS = 64 * PK_WAVES;
 #define VQ_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16((A), (B), (C), 0, 0, 0)
 
 // ---- value scale / zero of a lane's eight tokens (tA..tA+3, tB..tB+3)
 template <typename M> struct TokMeta;
 template <> struct TokMeta<f16> {
     uint2 a, b;
-    __device__ __forceinline__ void load(const char *base, u32 off, u32 gap_bytes) {
-        a = ldg<uint2>(base, off);
-        b = ldg<uint2>(base + gap_bytes, off);
+    __device__ __forceinline__ void read(const char *p, int gap_bytes) {
+        a = *reinterpret_cast<const uint2 *>(p);
+        b = *reinterpret_cast<const uint2 *>(p + gap_bytes);
     }
     // k-slot pair p = (token tA + p, token tB + p)
     __device__ __forceinline__ u32 pair(int p) const {
@@ -60,9 +66,9 @@ template <> struct TokMeta<f16> {
 };
 template <> struct TokMeta<float> {
     float4 a, b;
-    __device__ __forceinline__ void load(const char *base, u32 off, u32 gap_bytes) {
-        a = ldg<float4>(base, off);
-        b = ldg<float4>(base + gap_bytes, off);
+    __device__ __forceinline__ void read(const char *p, int gap_bytes) {
+        a = *reinterpret_cast<const float4 *>(p);
+        b = *reinterpret_cast<const float4 *>(p + gap_bytes);
     }
     __device__ __forceinline__ float lo(int p) const { return p == 0 ? a.x : p == 1 ? a.y : p == 2 ? a.z : a.w; }
     __device__ __forceinline__ float hi(int p) const { return p == 0 ? b.x : p == 1 ? b.y : p == 2 ? b.z : b.w; }
@@ -72,11 +78,11 @@ template <> struct TokMeta<float> {
 template <typename M> struct ChanMeta;
 template <> struct ChanMeta<f16> {
     uint4 s[4], z[4];
-    __device__ __forceinline__ void load(const char *sb, const char *zb, u32 off) {
+    __device__ __forceinline__ void read(const char *sp, const char *zp) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            s[j] = ldg<uint4>(sb + 16 * j, off);
-            z[j] = ldg<uint4>(zb + 16 * j, off);
+            s[j] = *reinterpret_cast<const uint4 *>(sp + 16 * j);
+            z[j] = *reinterpret_cast<const uint4 *>(zp + 16 * j);
         }
     }
     __device__ __forceinline__ u32 sword(int w) const {   // channels 2w, 2w+1
@@ -90,11 +96,11 @@ template <> struct ChanMeta<f16> {
 };
 template <> struct ChanMeta<float> {
     float4 s[8], z[8];
-    __device__ __forceinline__ void load(const char *sb, const char *zb, u32 off) {
+    __device__ __forceinline__ void read(const char *sp, const char *zp) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            s[j] = ldg<float4>(sb + 16 * j, off);
-            z[j] = ldg<float4>(zb + 16 * j, off);
+            s[j] = *reinterpret_cast<const float4 *>(sp + 16 * j);
+            z[j] = *reinterpret_cast<const float4 *>(zp + 16 * j);
         }
     }
     static __device__ __forceinline__ float pick(const float4 &q, int e) { return e == 0 ? q.x : e == 1 ? q.y : e == 2 ? q.z : q.w; }
@@ -119,24 +125,74 @@ template <int BITS, typename M, int GV> struct PackedUnit {
                                          // group n % GV, of the lane's eight tokens
 };
 
+constexpr int MF_QIMG = 12 * 64;              // uint4 entries of the query image (below)
+constexpr int MF_QIMG_BYTES = MF_QIMG * 16;
+
+// One ring slot holds everything a unit needs, as it lies in memory:
+//   key codes    32 tokens x 16*BITS bytes (4-bit: lane l's two 16-byte pieces at 16 l and 1024 + 16 l;
+//                2-bit: the 16-byte piece lane l asked for at 16 l)
+//   value codes  the unit's word rows, 512 bytes each
+//   value scale rows (one per channel group, 32 tokens), then value zero rows
+//   key scale, key zero of the token group the unit opens (128 channels each); filled only for
+//   a unit that opens a group
+// exchange arrays of the waves (tail, cross-wave merge), which share the ring's bytes:
+// accumulators [PK_WAVES][MF_ROWS][MF_D], zero-point sums [PK_WAVES][MF_ROWS][8], maxima and
+// sums [PK_WAVES][MF_ROWS]
+constexpr int EX_O = PK_WAVES * MF_ROWS * MF_D * 4, EX_Z = PK_WAVES * MF_ROWS * 8 * 4, EX_M = PK_WAVES * MF_ROWS * 4;
+constexpr int EX_BYTES = EX_O + EX_Z + 2 * EX_M;
+
+template <int BITS, typename M, int GV> struct Ring {
+    static constexpr int MSZ = sizeof(M);
+    static constexpr int KB = 512 * BITS, VB = 512 * BITS;
+    static constexpr int VMR = GV * 32 * MSZ;      // bytes of the scale rows (and of the zero rows)
+    static constexpr int KMR = MF_D * MSZ;         // bytes of a key scale (zero) row
+    static constexpr int K_OFF = 0, V_OFF = KB, VS_OFF = KB + VB, VZ_OFF = VS_OFF + VMR, KS_OFF = VZ_OFF + VMR,
+                         KZ_OFF = KS_OFF + KMR;
+    static constexpr int SLOT = KZ_OFF + KMR;
+    // copies per unit, and per unit that opens a token group
+    static constexpr int VM_COPIES = VMR > 256 ? VMR / 256 : 1, KM_COPIES = KMR / 256;
+    static constexpr int UNIT_COPIES = (BITS == 4 ? 4 : 2) + 2 * VM_COPIES, GROUP_COPIES = 2 * KM_COPIES;
+    static constexpr int UPG = 4 / GV;             // units per token group
+    // the block has the CU's 160 KB to itself: the waves' rings next to the query image
+    static constexpr int BUDGET = (160 * 1024 - MF_QIMG_BYTES - 1024) / PK_WAVES;
+    static constexpr int DEPTH = BUDGET / SLOT > 5 ? 5 : BUDGET / SLOT < 2 ? 2 : BUDGET / SLOT;   // one slot in use, at least one in flight
+    // copies issued after those of the unit about to be read: DEPTH - 1 later units, of which at
+    // least (DEPTH - 1) / UPG open a group
+    static constexpr int LATER = (DEPTH - 1) * UNIT_COPIES + ((DEPTH - 1) / UPG) * GROUP_COPIES;
+    static constexpr int WAVE_BYTES = DEPTH * SLOT;
+    static constexpr int BYTES = PK_WAVES * WAVE_BYTES > EX_BYTES ? PK_WAVES * WAVE_BYTES : EX_BYTES;
+    // Units are handed out to the waves in chunks of CHUNK consecutive units: whole token groups,
+    // and at least DEPTH - 1 units, so that the copies never run more than one chunk ahead of
+    // the arithmetic.
+    static constexpr int CHUNK = ((DEPTH - 1 + UPG - 1) / UPG) * UPG;
+};
+
 // LDS image of the query, three operand forms of 4 k-steps x 64 lanes each:
 //   [0..3]  memory order, rows < R only            (B operand of the zero-point product)
 //   [4..7]  k-slot pair order, +q in columns [0,R), -q in columns [R,2R)
 //   [8..11] k-slot pair order, q in columns [R,2R) only
 // so that  t = [4..7] * s  and  fma([8..11], s, t)  give the rounded product in the
 // high columns and its exact remainder in the low columns without a select.
-constexpr int MF_QIMG = 12 * 64;
-
 template <int BITS>
 __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw,
                                                   uint4 *s_q) {
     const int R = tile.RT;
-    for (int e = tid; e < MF_ROWS * MF_D; e += 256) {
-        const int row = e / MF_D, d = e % MF_D;
-        s_qraw[e] = tile.valid(row) ? (f16)ldq(a.q, a.q_dtype, tile.row(row) * MF_D + d) : (f16)0.f;
+    // raw rows: eight consecutive channels per thread, one load each
+    for (int e = tid; e < MF_ROWS * MF_D / 8; e += PK_THREADS) {
+        const int row = e / (MF_D / 8), d = 8 * (e % (MF_D / 8));
+        f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (tile.valid(row)) {
+            const int64_t i = tile.row(row) * MF_D + d;
+            if (a.q_dtype == VQ_F16) v = *reinterpret_cast<const f16x8 *>((const f16 *)a.q + i);
+            else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) v[j] = (f16)ldq(a.q, a.q_dtype, i + j);
+            }
+        }
+        *reinterpret_cast<f16x8 *>(s_qraw + 8 * e) = v;
     }
     __syncthreads();
-    for (int e = tid; e < MF_QIMG; e += 256) {
+    for (int e = tid; e < MF_QIMG; e += PK_THREADS) {
         const int form = e / 256, ks = (e / 64) % 4, l = e % 64;
         const int n = l & 15, blk = l >> 4;
         const int rq = n < R ? n : n - R;
@@ -163,7 +219,8 @@ __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const
 template <int BITS, typename M, int GV>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, int R, float c, int64_t t_begin,
                                              int n_units, int64_t lane_vis, int64_t full_vis, int lane, int wave,
-                                             PackedAcc<GV, sizeof(M) != 2> &acc, const uint4 *s_q) {
+                                             PackedAcc<GV, sizeof(M) != 2> &acc, const uint4 *s_q, char *ring,
+                                             int *s_next) {
     constexpr int PER = 32 / BITS;           // codes per word
     constexpr int KW = MF_D / PER;           // key words per token row
     constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
@@ -175,11 +232,6 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const u32 magic = vreg_const(Magic<BITS>::bits);
     const int64_t cap = a.cap_tokens;
 
-    const int per_wave = (n_units + 3) / 4;
-    const int u0 = wave * per_wave;
-    const int u1 = u0 + per_wave < n_units ? u0 + per_wave : n_units;
-    if (u0 >= u1) return;
-
     // block-uniform bases, 32-bit per-lane byte offsets
     const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
     const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
@@ -187,37 +239,91 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const char *kzb = (const char *)a.k_zero + bh * (cap / G) * MF_D * MSZ;
     const char *vsb = (const char *)a.v_scale + bh * GV * cap * MSZ;
     const char *vzb = (const char *)a.v_zero + bh * GV * cap * MSZ;
-    // token of S^T row n in tile T: vtok_lo(n / 4, n % 4) + T * GAP
-    const u32 koff = (u32)((vtok_lo<BITS>(n >> 2, n & 3) * KW + KWL * blk) * 4);
-    const u32 voff = (u32)(((BITS == 4 ? blk : blk / 2) * MF_D + n) * 4);
-    const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
-    const u32 vsoff = (u32)vtok_lo<BITS>(blk, 0) * MSZ;
-    const u32 vzoff = (u32)(((int64_t)(n % GV) * cap + vtok_lo<BITS>(blk, 0)) * MSZ);
-    // B operand of the zero-point tile: zeros in columns [0, GV), scales in [GV, 2 GV) (and,
-    // unused, in the columns beyond)
-    const char *vzs = n < GV ? vzb : vsb;
-    const u32 kmoff = 32u * blk * MSZ;
 
+    using RG = Ring<BITS, M, GV>;
     using Unit = PackedUnit<BITS, M, GV>;
-    auto load_unit = [&](int u, Unit &d) {
+    char *wring = ring + wave * RG::WAVE_BYTES;
+    const u32 wring_lds = lds_addr(wring);
+    // ---- what a lane copies.  Key codes: token of S^T row n in tile T is vtok_lo(n / 4, n % 4) + T * GAP.
+    //   4-bit: the lane's own 16 bytes (its 32 channels) of both token rows, two copies
+    //   2-bit: one copy; lane (n, blk) fetches the 16-byte half blk / 2 of token row T = blk % 2
+    const u32 koff = BITS == 4 ? (u32)((vtok_lo<BITS>(n >> 2, n & 3) * KW + KWL * blk) * 4)
+                               : (u32)(((vtok_lo<BITS>(n >> 2, n & 3) + (blk & 1) * GAP) * KW + 4 * (blk >> 1)) * 4);
+    // value codes, every scale / zero row: memory order, 16 (4) bytes per lane
+    const u32 l16 = 16u * lane, l4 = 4u * lane;
+    // value scale (zero) rows: byte 4*lane (+256 for a second copy) of the [GV][32] image, row g at g*cap
+    constexpr int VROW = 32 * (int)MSZ;
+    const u32 vmoff0 = (u32)((int64_t)(l4 / VROW) * cap * MSZ + l4 % VROW);
+    const u32 vmoff1 = (u32)((int64_t)((256 + l4) / VROW) * cap * MSZ + (256 + l4) % VROW);
+    constexpr u32 VM_ACTIVE = RG::VMR / 4 < 64 ? RG::VMR / 4 : 64;
+
+    const int64_t unit0 = t_begin / 32;   // absolute unit number of unit 0 of this block
+    // a unit brings the key scale / zero of its token group along when it opens the group or
+    // is the first of a chunk
+    auto issue_unit = [&](int u, int slot, bool opener) {
         const int64_t base = t_begin + (int64_t)u * 32;
+        const u32 sl = wring_lds + (u32)slot * RG::SLOT;
         const char *kp = kb + base * KW * 4;
-#pragma unroll
-        for (int T = 0; T < 2; ++T) {
-            if (BITS == 4) {
-                uint4 x = ldg<uint4>(kp + T * GAP * KW * 4, koff);
-                d.kw[T][0] = x.x; d.kw[T][1] = x.y; d.kw[T][KWL - 2] = x.z; d.kw[T][KWL - 1] = x.w;
-            } else {
-                uint2 x = ldg<uint2>(kp + T * GAP * KW * 4, koff);
-                d.kw[T][0] = x.x; d.kw[T][KWL - 1] = x.y;
-            }
+        if constexpr (BITS == 4) {
+            lds_copy16<0>(kp, koff, sl + RG::K_OFF);
+            lds_copy16<GAP * KW * 4>(kp, koff, sl + RG::K_OFF + 1024 - GAP * KW * 4);
+        } else {
+            lds_copy16<0>(kp, koff, sl + RG::K_OFF);
         }
         const char *vp = vb + (base / PER) * MF_D * 4;
+        lds_copy16<0>(vp, l16, sl + RG::V_OFF);
+        if constexpr (BITS == 4) lds_copy16<1024>(vp, l16, sl + RG::V_OFF);
+        const char *vsp = vsb + base * MSZ, *vzp = vzb + base * MSZ;
+        if (VM_ACTIVE == 64 || lane < (int)VM_ACTIVE) {
+            lds_copy4<0>(vsp, vmoff0, sl + RG::VS_OFF);
+            lds_copy4<0>(vzp, vmoff0, sl + RG::VZ_OFF);
+            if constexpr (RG::VM_COPIES == 2) {
+                lds_copy4<0>(vsp, vmoff1, sl + RG::VS_OFF + 256);
+                lds_copy4<0>(vzp, vmoff1, sl + RG::VZ_OFF + 256);
+            }
+        }
+        if (opener) {
+            const int64_t grp = base / G;
+            const char *ksp = ksb + grp * MF_D * MSZ, *kzp = kzb + grp * MF_D * MSZ;
+            lds_copy4<0>(ksp, l4, sl + RG::KS_OFF);
+            lds_copy4<0>(kzp, l4, sl + RG::KZ_OFF);
+            if constexpr (RG::KM_COPIES == 2) {
+                lds_copy4<256>(ksp, l4, sl + RG::KS_OFF);
+                lds_copy4<256>(kzp, l4, sl + RG::KZ_OFF);
+            }
+        }
+    };
+
+    // ---- what a lane reads back (ordinary LDS loads)
+    const int vrow = BITS == 4 ? blk : blk >> 1;          // word row of the lane's eight tokens
+    const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
+    const int tok_a = vtok_lo<BITS>(blk, 0);
+    const int zrow = n < GV ? GV + n : n % GV;            // row of the [scale rows | zero rows] image
+    auto read_unit = [&](int slot, Unit &d) {
+        const char *sl = wring + slot * RG::SLOT;
+        if constexpr (BITS == 4) {
 #pragma unroll
-        for (int nt = 0; nt < 8; ++nt) d.vw[nt] = ldg<u32>(vp + 64 * nt, voff);
+            for (int T = 0; T < 2; ++T) {
+                const uint4 x = *reinterpret_cast<const uint4 *>(sl + RG::K_OFF + 1024 * T + 16 * lane);
+                d.kw[T][0] = x.x; d.kw[T][1] = x.y; d.kw[T][2] = x.z; d.kw[T][3] = x.w;
+            }
+        } else {
 #pragma unroll
-        for (int g = 0; g < GV; ++g) d.s[g].load(vsb + ((int64_t)g * cap + base) * MSZ, vsoff, GAP * MSZ);
-        d.z.load(vzs + base * MSZ, vzoff, GAP * MSZ);
+            for (int T = 0; T < 2; ++T) {
+                const uint2 x = *reinterpret_cast<const uint2 *>(sl + RG::K_OFF + (16 * (2 * (blk >> 1) + T) + n) * 16 + 8 * (blk & 1));
+                d.kw[T][0] = x.x; d.kw[T][1] = x.y;
+            }
+        }
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt)
+            d.vw[nt] = *reinterpret_cast<const u32 *>(sl + RG::V_OFF + vrow * 512 + (16 * nt + n) * 4);
+#pragma unroll
+        for (int g = 0; g < GV; ++g) d.s[g].read(sl + RG::VS_OFF + g * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
+        d.z.read(sl + RG::VS_OFF + zrow * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
+    };
+    auto read_group = [&](int slot, ChanMeta<M> &km) {
+        const char *sl = wring + slot * RG::SLOT;
+        km.read(sl + RG::KS_OFF + 32 * blk * (int)MSZ, sl + RG::KZ_OFF + 32 * blk * (int)MSZ);
     };
 
     f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
@@ -404,61 +510,101 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         acc.L = VQ_MFMA(P8, ones, acc.L);
     };
 
-    Unit ua, ub;
-    ChanMeta<M> km;
-    int64_t cur_group = (t_begin + (int64_t)u0 * 32) / G;
-    load_unit(u0, ua);
-    km.load(ksb + cur_group * MF_D * MSZ, kzb + cur_group * MF_D * MSZ, kmoff);
-    open_group(km);
-
-    // loads of unit u+1 (and of the next group's key scale / zero when u+1 opens one) are
-    // issued before unit u is computed; past the end the last unit is simply loaded again
-    auto step = [&](const Unit &cur, Unit &nxt, int u) {
-        const int un = u + 1 < u1 ? u + 1 : u;
-        load_unit(un, nxt);
-        const int64_t next_group = (t_begin + (int64_t)un * 32) / G;
-        const bool new_group = next_group != cur_group;
-        if (new_group) km.load(ksb + next_group * MF_D * MSZ, kzb + next_group * MF_D * MSZ, kmoff);
-        compute(cur, t_begin + (int64_t)u * 32);
-        if (new_group) {
-            open_group(km);
-            cur_group = next_group;
+    // ---- the waves of a block draw chunks of CHUNK units from a shared counter (a wave that
+    // is ahead simply draws more), so no wave waits for a slower one until the block's units are
+    // used up.  Copies run DEPTH - 1 units ahead of the arithmetic: `i_*` is where the copies are,
+    // `c_*` where the arithmetic is.  Chunks being at least DEPTH - 1 units long (but for the
+    // block's last), the copies have entered at most two chunks beyond the one being computed:
+    // `c_next`, `c_after` queue them (NONE = nothing queued, END = the block has no more).
+    constexpr int CH = RG::CHUNK;
+    const int n_chunks = (n_units + CH - 1) / CH;
+    auto draw = [&]() {   // the next chunk of the block; the value is used a chunk later
+        int id = 0;
+        if (lane == 0) id = __hip_atomic_fetch_add(s_next, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return id;
+    };
+    auto chunk_len = [&](int chunk) { return n_units - chunk * CH < CH ? n_units - chunk * CH : CH; };
+    if (wave >= n_chunks) return;   // the first PK_WAVES chunks are dealt out, the counter starts behind them
+    constexpr int END = -1, NONE = -2;
+    int i_chunk = wave, i_pos = 0, i_slot = 0;
+    int c_chunk = wave, c_pos = 0, c_next = NONE, c_after = NONE, c_slot = 0;
+    int in_flight = 0;
+    int drawn = draw();
+    auto issue_next = [&]() {
+        const int u = i_chunk * CH + i_pos;
+        issue_unit(u, i_slot, i_pos == 0 || (unit0 + u) % RG::UPG == 0);
+        i_slot = i_slot + 1 == RG::DEPTH ? 0 : i_slot + 1;
+        ++in_flight;
+        if (++i_pos == chunk_len(i_chunk)) {
+            const int got = __builtin_amdgcn_readfirstlane(drawn);
+            i_chunk = got < n_chunks ? got : END;
+            i_pos = 0;
+            if (c_next == NONE) c_next = i_chunk;
+            else c_after = i_chunk;
+            if (i_chunk >= 0) drawn = draw();
         }
     };
-    for (int u = u0; u < u1; u += 2) {
-        step(ua, ub, u);
-        if (u + 1 < u1) step(ub, ua, u + 1);
+#pragma unroll
+    for (int j = 0; j < RG::DEPTH - 1; ++j)
+        if (i_chunk >= 0) issue_next();
+    while (c_chunk >= 0) {
+        if (i_chunk >= 0) issue_next();
+        // with a full ring exactly DEPTH - 1 units were issued behind the one awaited
+        if (in_flight == RG::DEPTH) wait_copies<RG::LATER>();
+        else wait_copies<0>();
+        const int u = c_chunk * CH + c_pos;
+        Unit cur;
+        read_unit(c_slot, cur);
+        if (c_pos == 0 || (unit0 + u) % RG::UPG == 0) {
+            ChanMeta<M> km;
+            read_group(c_slot, km);
+            open_group(km);
+        }
+        compute(cur, t_begin + (int64_t)u * 32);
+        c_slot = c_slot + 1 == RG::DEPTH ? 0 : c_slot + 1;
+        --in_flight;
+        if (++c_pos == chunk_len(c_chunk)) {
+            c_chunk = c_next;   // queued by then: the copies are ahead
+            c_next = c_after;
+            c_after = NONE;
+            c_pos = 0;
+        }
     }
 }
 
-// grid (nsplit, B*Hkv*tiles).  A block works on one tile of query rows (the GQA group at pq
-// consecutive positions) and on packed tokens
+// grid (nsplit, B*Hkv*tiles), PK_THREADS threads.  A block works on one tile of query rows (the GQA
+// group at pq consecutive positions) and on packed tokens
 // [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)), cut to what the
 // tile sees; block 0 first runs the fp16 tail, whose partial goes to slot nsplit.  With sync
 // counters the block that finishes last for its tile merges the nparts partials into the output.
 template <int BITS, typename M, int GV>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(PK_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
                                float *__restrict__ ws) {
-    __shared__ float s_m[4][MF_ROWS];
-    __shared__ float s_l[4][MF_ROWS];
-    __shared__ float s_z[4][MF_ROWS][8];
-    __shared__ float s_o[4][MF_ROWS][MF_D];
     __shared__ uint4 s_q[MF_QIMG];
-    __shared__ int s_ticket;
+    // the waves' rings; before and after the units the same bytes are the exchange buffer
+    // s_o[PK_WAVES][MF_ROWS][MF_D] of the tail and of the cross-wave merge
+    extern __shared__ __align__(16) char s_ring[];
+    float (*s_o)[MF_ROWS][MF_D] = reinterpret_cast<float (*)[MF_ROWS][MF_D]>(s_ring);
+    float (*s_z)[MF_ROWS][8] = reinterpret_cast<float (*)[MF_ROWS][8]>(s_ring + EX_O);
+    float (*s_m)[MF_ROWS] = reinterpret_cast<float (*)[MF_ROWS]>(s_ring + EX_O + EX_Z);
+    float (*s_l)[MF_ROWS] = reinterpret_cast<float (*)[MF_ROWS]>(s_ring + EX_O + EX_Z + EX_M);
+    __shared__ int s_ticket, s_next;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: loops below stay scalar
+    if (tid == 0) s_next = PK_WAVES;   // chunks 0 .. PK_WAVES - 1 are dealt to the waves up front
     const int n = lane & 15, blk = lane >> 4;
-    const int64_t bh = blockIdx.y / tiles;
+    const int by = blockIdx.y;
     const int sp = (int)blockIdx.x, nsplit = (int)gridDim.x;
+    const int64_t bh = by / tiles;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
     const float c = a.scale * LOG2E;
 
     RowTile tile;
     tile.R = (int)(a.Hq / a.Hkv);
     tile.RT = tile.R * pq;
-    tile.pos0 = (int)(blockIdx.y % tiles) * pq;
+    tile.pos0 = (int)(by % tiles) * pq;
     tile.Sq = a.Sq;
     tile.n_total = a.n_packed + a.n_tail;
     tile.causal = a.causal;
@@ -470,8 +616,8 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     f16 *s_qraw = reinterpret_cast<f16 *>(&s_o[0][0][0]);
     build_query_image<BITS>(a, tile, tid, s_qraw, s_q);
     if (sp == 0 && a.n_tail > 0)
-        tail_block(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid, wave,
-                   single_launch);
+        tail_block<PK_WAVES>(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid,
+                             wave, single_launch);
 
     PackedAcc<GV, sizeof(M) != 2> acc;
 #pragma unroll
@@ -496,9 +642,12 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (t_begin < 0) t_begin = 0;
     if (t_end > (max_vis + 31) / 32 * 32) t_end = (max_vis + 31) / 32 * 32;
     const int n_units = t_end > t_begin ? (int)((t_end - t_begin) / 32) : 0;
-    packed_units<BITS, M, GV>(a, bh, RT, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_q);
+    __syncthreads();   // the query staging and the tail are done with the ring's bytes
+    packed_units<BITS, M, GV>(a, bh, RT, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_q, s_ring,
+                              &s_next);
+    __syncthreads();   // every wave has read its last slot
 
-    // ---- merge the four waves: accumulator register r of lane (n, blk) is row 4*blk + r,
+    // ---- merge the waves: accumulator register r of lane (n, blk) is row 4*blk + r,
     // tile nt column n is channel 16*nt + n
     if (blk == 0) s_m[wave][n] = acc.m_run;
 #pragma unroll
@@ -514,13 +663,15 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         }
     }
     __syncthreads();
-    for (int e = tid; e < RT * MF_D; e += 256) {
+    for (int e = tid; e < RT * MF_D; e += PK_THREADS) {
         const int row = e / MF_D, d = e % MF_D;
         if (!tile.valid(row)) continue;
-        const float gm = fmaxf(fmaxf(s_m[0][row], s_m[1][row]), fmaxf(s_m[2][row], s_m[3][row]));
+        float gm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < PK_WAVES; ++w) gm = fmaxf(gm, s_m[w][row]);
         float num = 0.f, den = 0.f;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) {
+        for (int w = 0; w < PK_WAVES; ++w) {
             if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit, or saw nothing
             const float f = exp2f(s_m[w][row] - gm);
             const int g = d / (MF_D / GV);
@@ -540,20 +691,32 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (!single_launch) return;
     __syncthreads();
     if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(a.sync_counters + blockIdx.y, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != nsplit - 1) return;
-    merge_rows(a, tile, nparts, ws, tid);
-    if (tid == 0) __hip_atomic_store(a.sync_counters + blockIdx.y, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    merge_rows(a, tile, nparts, ws, tid, PK_THREADS);
+    if (tid == 0) __hip_atomic_store(a.sync_counters + by, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <typename M>
 static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
-    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles)), block(256);
+    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles)), block(PK_THREADS);
     const int gv = (int)(MF_D / a.group);
-#define VQ_LAUNCH(BITS, GV) \
-    hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, 0, st, a, p.split_len, p.tail_equiv, \
-                       p.nparts, p.pq, p.tiles, ws)
+    // more than 64 KB of block-shared memory has to be allowed per kernel and device, once
+#define VQ_LAUNCH(BITS, GV)                                                                                       \
+    do {                                                                                                          \
+        constexpr int ring_bytes = Ring<BITS, M, GV>::BYTES;                                                      \
+        static bool allowed[64] = {};                                                                             \
+        int dev = 0;                                                                                              \
+        (void)hipGetDevice(&dev);                                                                                 \
+        if (dev < 0 || dev >= 64 || !allowed[dev]) {                                                              \
+            (void)hipFuncSetAttribute((const void *)attend_mfma_packed_kernel<BITS, M, GV>,                       \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);                    \
+            if (dev >= 0 && dev < 64) allowed[dev] = true;                                                        \
+        }                                                                                                         \
+        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, ring_bytes, st, a, p.split_len, \
+                           p.tail_equiv, p.nparts, p.pq, p.tiles, ws);                                            \
+    } while (0)
     if (a.pack_bits == 4) {
         if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);
     } else {
