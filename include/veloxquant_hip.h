@@ -96,6 +96,17 @@ int vq_kivi_dequant(const void *packed, const void *scale, const void *zero, int
                     int v_layout, int64_t cap_tokens, int64_t src_tok0, void *out, int out_dtype,
                     void *stream);
 
+/* Appends S new tokens of keys and values, [B, H, S, D] each with element strides
+ * k_strides / v_strides = {batch, head, token} and contiguous channels, to the
+ * un-quantised tails [B, H, tail_cap, D] (contiguous) at token `pos`, both in one
+ * launch.  elem_bytes is 2 (fp16, bf16) or 4; D * elem_bytes and every stride in
+ * bytes must be multiples of 16 and every pointer 16-byte aligned.  This is the
+ * concatenation step of KIVIKVCache.update_and_fetch
+ * (veloxquant_mlx/cache/kivi_cache.py:206-260) into a buffer that already has room. */
+int vq_kv_tail_append(const void *k_new, const void *v_new, const int64_t k_strides[3], const int64_t v_strides[3],
+                      void *k_tail, void *v_tail, int elem_bytes, int64_t B, int64_t H, int64_t S, int64_t D,
+                      int64_t tail_cap, int64_t pos, void *stream);
+
 /* ---- bit packing ----------------------------------------------------------- */
 
 /* Trailing-axis word packing, idx[rows, D] uint8 <-> words[rows, ceil(D/per)].

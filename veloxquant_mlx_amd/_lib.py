@@ -46,6 +46,7 @@ _SIGNATURES = {
     "vq_kivi_quant_dequant": (i32, [vp, vp, i32, i64, i64, i64, i32, i32, i32, f32, vp]),
     "vq_kivi_quant_pack": (i32, [vp, i32, i64, i64, i64, i64, i32, i32, i32, f32, i32, i32, vp, vp, vp, i32, i64, i64, vp]),
     "vq_kivi_dequant": (i32, [vp, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, i64, i64, vp, i32, vp]),
+    "vq_kv_tail_append": (i32, [vp, vp, C.POINTER(i64), C.POINTER(i64), vp, vp, i32, i64, i64, i64, i64, i64, i64, vp]),
     "vq_pack_words": (i32, [vp, i64, i64, i32, vp, vp]),
     "vq_unpack_words": (i32, [vp, i64, i64, i32, vp, vp]),
     "vq_bit_pack": (i32, [vp, i64, i32, vp, vp]),

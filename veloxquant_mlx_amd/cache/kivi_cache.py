@@ -108,6 +108,7 @@ class KIVIKVCache(FP16KVCache):
         self._packed_cap = 0
         # fp16 tail (memory-bound mode): tokens [_n_quantized, offset)
         self._tail_k = self._tail_v = None
+        self._zero_scalar = None
 
     # ------------------------------------------------------------------
     def _quant_dequant_along(self, x: torch.Tensor, axis: int) -> torch.Tensor:
@@ -209,8 +210,11 @@ class KIVIKVCache(FP16KVCache):
                 tk[:, :, :n_tail] = self._tail_k[:, :, :n_tail]
                 tv[:, :, :n_tail] = self._tail_v[:, :, :n_tail]
             self._tail_k, self._tail_v = tk, tv
-        self._tail_k[:, :, n_tail:need] = keys
-        self._tail_v[:, :, n_tail:need] = values
+        if keys.dtype == self._tail_k.dtype and values.dtype == keys.dtype and (D * keys.element_size()) % 16 == 0:
+            K.kv_tail_append(keys, values, self._tail_k, self._tail_v, n_tail)
+        else:
+            self._tail_k[:, :, n_tail:need] = keys
+            self._tail_v[:, :, n_tail:need] = values
         self.offset += S
         new_boundary = self._quantization_boundary()
         n_quant_now = new_boundary - self._n_quantized
@@ -228,7 +232,9 @@ class KIVIKVCache(FP16KVCache):
                 self._tail_k = self._tail_k[:, :, :cap].clone()
                 self._tail_v = self._tail_v[:, :, :cap].clone()
         self._account_bytes(B, H, S, D, n_quant_now)
-        z = torch.zeros((), dtype=keys.dtype, device=keys.device)
+        z = self._zero_scalar
+        if z is None or z.dtype != keys.dtype or z.device != keys.device:
+            z = self._zero_scalar = torch.zeros((), dtype=keys.dtype, device=keys.device)
         return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
 
     def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0):

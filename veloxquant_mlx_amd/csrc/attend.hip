@@ -30,7 +30,10 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
         p.tiles = (int)cdiv(a.Sq, p.pq);
-        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 2, 64) * 64 : 0;
+        #ifndef VQ_X_TAILEQ
+#define VQ_X_TAILEQ 2
+#endif
+        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * VQ_X_TAILEQ, 64) * 64 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
     const int64_t max_splits = n_split > 0 ? cdiv(n_split, 64) : 1;

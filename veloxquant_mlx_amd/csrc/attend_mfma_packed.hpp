@@ -155,7 +155,11 @@ template <int BITS, typename M, int GV> struct Ring {
     static constexpr int UPG = 4 / GV;             // units per token group
     // the block has the CU's 160 KB to itself: the waves' rings next to the query image
     static constexpr int BUDGET = (160 * 1024 - MF_QIMG_BYTES - 1024) / PK_WAVES;
+#ifdef VQ_X_DEPTH
+    static constexpr int DEPTH = VQ_X_DEPTH;
+#else
     static constexpr int DEPTH = BUDGET / SLOT > 5 ? 5 : BUDGET / SLOT < 2 ? 2 : BUDGET / SLOT;   // one slot in use, at least one in flight
+#endif
     // copies issued after those of the unit about to be read: DEPTH - 1 later units, of which at
     // least (DEPTH - 1) / UPG open a group
     static constexpr int LATER = (DEPTH - 1) * UNIT_COPIES + ((DEPTH - 1) / UPG) * GROUP_COPIES;
@@ -164,7 +168,11 @@ template <int BITS, typename M, int GV> struct Ring {
     // Units are handed out to the waves in chunks of CHUNK consecutive units: whole token groups,
     // and at least DEPTH - 1 units, so that the copies never run more than one chunk ahead of
     // the arithmetic.
+#ifdef VQ_X_CHUNK
+    static constexpr int CHUNK = VQ_X_CHUNK;
+#else
     static constexpr int CHUNK = ((DEPTH - 1 + UPG - 1) / UPG) * UPG;
+#endif
 };
 
 // LDS image of the query, three operand forms of 4 k-steps x 64 lanes each:

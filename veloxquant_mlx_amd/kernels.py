@@ -9,9 +9,9 @@ on the CPU.
 
 from __future__ import annotations
 
+import ctypes as C
 import math
 
-import os
 import torch
 
 from . import _lib
@@ -170,6 +170,38 @@ def kivi_quant_codes(x: torch.Tensor, axis: int, group_size: int, levels: int, e
     B, H, S, D = x.shape
     codes = packed.reshape(-1).view(torch.uint8).view(B, H, S, -1)[..., :D]
     return codes, scale, zero
+
+
+def kv_tail_append(k_new: torch.Tensor, v_new: torch.Tensor, k_tail: torch.Tensor, v_tail: torch.Tensor,
+                   pos: int) -> None:
+    """Write ``k_new, v_new [B,H,S,D]`` into rows ``[pos, pos+S)`` of the tails ``[B,H,cap,D]``
+    (one launch for both): the concatenation step of ``KIVIKVCache.update_and_fetch``
+    (veloxquant_mlx/cache/kivi_cache.py:206-260) into buffers that already have room."""
+    name = "kv_tail_append"
+    _need_gpu(name, k_new, v_new, k_tail, v_tail)
+    if k_new.shape != v_new.shape or k_tail.shape != v_tail.shape or k_new.ndim != 4 or k_tail.ndim != 4:
+        raise ValueError(f"{name}: keys/values must be [B,H,S,D] and the tails [B,H,cap,D]")
+    B, H, S, D = k_new.shape
+    if k_tail.shape[0] != B or k_tail.shape[1] != H or k_tail.shape[3] != D:
+        raise ValueError(f"{name}: tail shape {tuple(k_tail.shape)} does not match new tokens {tuple(k_new.shape)}")
+    if not (k_new.dtype == v_new.dtype == k_tail.dtype == v_tail.dtype):
+        raise ValueError(f"{name}: new tokens and tails must share one dtype")
+    if not (k_tail.is_contiguous() and v_tail.is_contiguous()):
+        raise ValueError(f"{name}: the tails must be contiguous")
+    cap = k_tail.shape[2]
+    if pos < 0 or pos + S > cap:
+        raise ValueError(f"{name}: tokens [{pos}, {pos + S}) exceed the tail capacity {cap}")
+
+    es = k_new.element_size()
+
+    def strides(t):   # channels contiguous, every other stride a multiple of 16 bytes; else a packed copy
+        if B * H * S * D and (t.stride(3) != 1 or any((t.stride(i) * es) % 16 for i in range(3)) or t.data_ptr() % 16):
+            t = t.contiguous()
+        return t, (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+    k_new, ks = strides(k_new)
+    v_new, vs = strides(v_new)
+    _lib.check(_lib.load().vq_kv_tail_append(k_new.data_ptr(), v_new.data_ptr(), ks, vs, k_tail.data_ptr(),
+                                             v_tail.data_ptr(), es, B, H, S, D, cap, pos, _stream(k_new)))
 
 
 def kivi_dequant(packed: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, axis: int, group_size: int,
