@@ -30,22 +30,21 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
         p.tiles = (int)cdiv(a.Sq, p.pq);
-        #ifndef VQ_X_TAILEQ
-#define VQ_X_TAILEQ 2
-#endif
-        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * VQ_X_TAILEQ, 64) * 64 : 0;
+                p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 2, 128) * 128 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
-    const int64_t max_splits = n_split > 0 ? cdiv(n_split, 64) : 1;
+    // the MFMA kernel wants every block to start on a boundary of the largest token group (128)
+    const int64_t gran = p.path == 1 ? 128 : 64;
+    const int64_t max_splits = n_split > 0 ? cdiv(n_split, gran) : 1;
     // units of parallel work before splitting: a wave per query row (generic)
     // or an eight-wave block per kv head (MFMA)
     const int64_t units = p.path == 1 ? a.B * a.Hkv * p.tiles : a.B * a.Hq * a.Sq;
-        const int64_t target = p.path == 1 ? 256 : 4096;   // MFMA path: one eight-wave block per CU
+    const int64_t target = p.path == 1 ? 256 : 4096;   // MFMA path: one eight-wave block per CU
     int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(target, units > 0 ? units : 1);   // < 0: choose as well
     if (ns > max_splits) ns = max_splits;
     if (ns > 512) ns = 512;
     if (ns < 1) ns = 1;
-    int64_t len = cdiv(cdiv(n_split > 0 ? n_split : 1, ns), 64) * 64;
+    int64_t len = cdiv(cdiv(n_split > 0 ? n_split : 1, ns), gran) * gran;
     if (p.tail_equiv > len) p.tail_equiv = len;   // split 0 may end up with the tail only
     ns = cdiv(a.n_packed + p.tail_equiv > 0 ? a.n_packed + p.tail_equiv : 1, len);
     if (p.path == 0) ns = n_split > 0 ? cdiv(n_split, len) : 1;

@@ -75,6 +75,34 @@ template <int BITS> __device__ __forceinline__ f16x8 unpack8(u32 w, u32 magic) {
     return as_h8(r0, r1, r2, r3);
 }
 
+// Two packed words at a time: a 64-bit shift (full rate on this part) moves both, and what
+// crosses from one word into the other lands outside the mask.  SH > 0 shifts left.
+typedef unsigned long long u64;
+template <int SH> __device__ __forceinline__ u64 shift64(u64 x) {
+    u64 r = x;
+    if constexpr (SH > 0) asm("v_lshlrev_b64 %0, %2, %1" : "=v"(r) : "v"(x), "n"(SH));
+    else if constexpr (SH < 0) asm("v_lshrrev_b64 %0, %2, %1" : "=v"(r) : "v"(x), "n"(-SH));
+    return r;
+}
+template <int BITS, int S0, int S1, int S2, int S3>
+__device__ __forceinline__ void unpack8_pair_at(u64 x, u32 magic, f16x8 &lo, f16x8 &hi) {
+    constexpr u32 mask = Magic<BITS>::mask;
+    const u64 t0 = shift64<S0>(x), t1 = shift64<S1>(x), t2 = shift64<S2>(x), t3 = shift64<S3>(x);
+    lo = as_h8(((u32)t0 & mask) | magic, ((u32)t1 & mask) | magic, ((u32)t2 & mask) | magic, ((u32)t3 & mask) | magic);
+    hi = as_h8(((u32)(t0 >> 32) & mask) | magic, ((u32)(t1 >> 32) & mask) | magic, ((u32)(t2 >> 32) & mask) | magic,
+               ((u32)(t3 >> 32) & mask) | magic);
+}
+__device__ __forceinline__ u64 pack64(u32 lo, u32 hi) { return (u64)lo | ((u64)hi << 32); }
+// unpack8 of the words w0 and w1
+template <int BITS> __device__ __forceinline__ void unpack8_pair(u32 w0, u32 w1, u32 magic, f16x8 &a0, f16x8 &a1) {
+    if constexpr (BITS == 4) unpack8_pair_at<4, 6, 2, -2, -6>(pack64(w0, w1), magic, a0, a1);
+    else unpack8_pair_at<2, 8, 6, 4, 2>(pack64(w0, w1), magic, a0, a1);
+}
+// 2-bit only: unpack8 of w0 >> 8 and w1 >> 8
+__device__ __forceinline__ void unpack8_pair_upper2(u32 w0, u32 w1, u32 magic, f16x8 &a0, f16x8 &a1) {
+    unpack8_pair_at<2, 0, -2, -4, -6>(pack64(w0, w1), magic, a0, a1);
+}
+
 // channel (0..31 inside a lane's 32-channel slice) of k-slot pair p of k-step ks
 template <int BITS> __device__ __forceinline__ constexpr int kchan_lo(int ks, int p) {
     return BITS == 4 ? 8 * ks + p : 16 * (ks / 2) + 4 * (ks % 2) + p;

@@ -48,6 +48,9 @@ namespace vq {
 // One block of PK_WAVES waves per CU (two waves per SIMD, the register file split in two).
 constexpr int PK_WAVES = 8;
 constexpr int PK_THREADS = 64 * PK_WAVES;
+// Every lambda below must be inlined at every call: a closure left in memory would be read back
+// with vector loads, whose completion the ring's copy counter cannot tell from its own.
+#define VQ_INLINE_LAMBDA __attribute__((always_inline))
 #define VQ_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16((A), (B), (C), 0, 0, 0)
 
 // ---- value scale / zero of a lane's eight tokens (tA..tA+3, tB..tB+3)
@@ -125,62 +128,63 @@ template <int BITS, typename M, int GV> struct PackedUnit {
                                          // group n % GV, of the lane's eight tokens
 };
 
-constexpr int MF_QIMG = 12 * 64;              // uint4 entries of the query image (below)
+constexpr int MF_QIMG = 8 * 64;               // uint4 entries of the query image (below)
 constexpr int MF_QIMG_BYTES = MF_QIMG * 16;
 
-// One ring slot holds everything a unit needs, as it lies in memory:
+// A wave's ring: DEPTH unit slots, then GROUP_SLOTS group slots.  A unit slot holds what every
+// unit needs, as it lies in memory:
 //   key codes    32 tokens x 16*BITS bytes (4-bit: lane l's two 16-byte pieces at 16 l and 1024 + 16 l;
 //                2-bit: the 16-byte piece lane l asked for at 16 l)
 //   value codes  the unit's word rows, 512 bytes each
 //   value scale rows (one per channel group, 32 tokens), then value zero rows
-//   key scale, key zero of the token group the unit opens (128 channels each); filled only for
-//   a unit that opens a group
-// exchange arrays of the waves (tail, cross-wave merge), which share the ring's bytes:
+// A group slot holds the key scale and key zero (128 channels each) of a token group; the unit
+// that opens a group brings them along.  Blocks start on a group boundary, so units open a
+// group every UPG units and at most ceil(DEPTH / UPG) group slots are live at a time.
+// The exchange arrays of the waves (tail, cross-wave merge) share the rings' bytes:
 // accumulators [PK_WAVES][MF_ROWS][MF_D], zero-point sums [PK_WAVES][MF_ROWS][8], maxima and
 // sums [PK_WAVES][MF_ROWS]
 constexpr int EX_O = PK_WAVES * MF_ROWS * MF_D * 4, EX_Z = PK_WAVES * MF_ROWS * 8 * 4, EX_M = PK_WAVES * MF_ROWS * 4;
 constexpr int EX_BYTES = EX_O + EX_Z + 2 * EX_M;
+constexpr int PK_ALIGN = 128;                 // tokens: blocks start on a multiple of the largest token group
 
 template <int BITS, typename M, int GV> struct Ring {
     static constexpr int MSZ = sizeof(M);
     static constexpr int KB = 512 * BITS, VB = 512 * BITS;
     static constexpr int VMR = GV * 32 * MSZ;      // bytes of the scale rows (and of the zero rows)
     static constexpr int KMR = MF_D * MSZ;         // bytes of a key scale (zero) row
-    static constexpr int K_OFF = 0, V_OFF = KB, VS_OFF = KB + VB, VZ_OFF = VS_OFF + VMR, KS_OFF = VZ_OFF + VMR,
-                         KZ_OFF = KS_OFF + KMR;
-    static constexpr int SLOT = KZ_OFF + KMR;
+    static constexpr int K_OFF = 0, V_OFF = KB, VS_OFF = KB + VB, VZ_OFF = VS_OFF + VMR;
+    static constexpr int SLOT = VZ_OFF + VMR, GROUP_SLOT = 2 * KMR;
     // copies per unit, and per unit that opens a token group
     static constexpr int VM_COPIES = VMR > 256 ? VMR / 256 : 1, KM_COPIES = KMR / 256;
     static constexpr int UNIT_COPIES = (BITS == 4 ? 4 : 2) + 2 * VM_COPIES, GROUP_COPIES = 2 * KM_COPIES;
     static constexpr int UPG = 4 / GV;             // units per token group
     // the block has the CU's 160 KB to itself: the waves' rings next to the query image
-    static constexpr int BUDGET = (160 * 1024 - MF_QIMG_BYTES - 1024) / PK_WAVES;
+    static constexpr int BUDGET = (160 * 1024 - MF_QIMG_BYTES - 256) / PK_WAVES;
+    static constexpr int bytes_at(int depth) { return depth * SLOT + ((depth + UPG - 1) / UPG) * GROUP_SLOT; }
 #ifdef VQ_X_DEPTH
     static constexpr int DEPTH = VQ_X_DEPTH;
 #else
-    static constexpr int DEPTH = BUDGET / SLOT > 5 ? 5 : BUDGET / SLOT < 2 ? 2 : BUDGET / SLOT;   // one slot in use, at least one in flight
+    // one slot in use, at least one in flight
+    static constexpr int DEPTH = bytes_at(5) <= BUDGET ? 5 : bytes_at(4) <= BUDGET ? 4 : bytes_at(3) <= BUDGET ? 3 : 2;
 #endif
+    static constexpr int GROUP_SLOTS = (DEPTH + UPG - 1) / UPG;
+    static constexpr int GROUP_OFF = DEPTH * SLOT;
     // copies issued after those of the unit about to be read: DEPTH - 1 later units, of which at
     // least (DEPTH - 1) / UPG open a group
     static constexpr int LATER = (DEPTH - 1) * UNIT_COPIES + ((DEPTH - 1) / UPG) * GROUP_COPIES;
-    static constexpr int WAVE_BYTES = DEPTH * SLOT;
+    static constexpr int WAVE_BYTES = bytes_at(DEPTH);
     static constexpr int BYTES = PK_WAVES * WAVE_BYTES > EX_BYTES ? PK_WAVES * WAVE_BYTES : EX_BYTES;
     // Units are handed out to the waves in chunks of CHUNK consecutive units: whole token groups,
     // and at least DEPTH - 1 units, so that the copies never run more than one chunk ahead of
     // the arithmetic.
-#ifdef VQ_X_CHUNK
-    static constexpr int CHUNK = VQ_X_CHUNK;
-#else
     static constexpr int CHUNK = ((DEPTH - 1 + UPG - 1) / UPG) * UPG;
-#endif
 };
 
-// LDS image of the query, three operand forms of 4 k-steps x 64 lanes each:
-//   [0..3]  memory order, rows < R only            (B operand of the zero-point product)
-//   [4..7]  k-slot pair order, +q in columns [0,R), -q in columns [R,2R)
-//   [8..11] k-slot pair order, q in columns [R,2R) only
-// so that  t = [4..7] * s  and  fma([8..11], s, t)  give the rounded product in the
-// high columns and its exact remainder in the low columns without a select.
+// LDS image of the query, two operand forms of 4 k-steps x 64 lanes each:
+//   [0..3]  memory order, rows in columns [0, R) only       (B operand of the zero-point product)
+//   [4..7]  k-slot pair order, q in columns [0, R) and again in columns [R, 2R)
+// so that  t = [4..7] * s  is the rounded product and  fma([4..7], s, -t)  its exact remainder;
+// columns [0, R) keep the first, columns [R, 2R) the second.
 template <int BITS>
 __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw,
                                                   uint4 *s_q) {
@@ -201,7 +205,7 @@ __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const
     }
     __syncthreads();
     for (int e = tid; e < MF_QIMG; e += PK_THREADS) {
-        const int form = e / 256, ks = (e / 64) % 4, l = e % 64;
+        const int form = e / 256, ks = (e / 64) % 4, l = e % 64;   // 256 entries per form
         const int n = l & 15, blk = l >> 4;
         const int rq = n < R ? n : n - R;
         const bool hi_col = n < R, lo_col = n >= R && n < 2 * R;
@@ -212,11 +216,7 @@ __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const
             if (form == 0) ch = 8 * ks + j;
             else ch = (j & 1) ? kchan_hi<BITS>(ks, j >> 1) : kchan_lo<BITS>(ks, j >> 1);
             const f16 q = (hi_col || lo_col) ? s_qraw[rq * MF_D + 32 * blk + ch] : (f16)0.f;
-            f16 x;
-            if (form == 0) x = hi_col ? q : (f16)0.f;
-            else if (form == 1) x = hi_col ? q : -q;
-            else x = lo_col ? q : (f16)0.f;
-            v[j] = x;
+            v[j] = (form == 0 && !hi_col) ? (f16)0.f : q;
         }
         f16x8 o = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]};
         s_q[e] = __builtin_bit_cast(uint4, o);
@@ -265,10 +265,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const u32 vmoff1 = (u32)((int64_t)((256 + l4) / VROW) * cap * MSZ + (256 + l4) % VROW);
     constexpr u32 VM_ACTIVE = RG::VMR / 4 < 64 ? RG::VMR / 4 : 64;
 
-    const int64_t unit0 = t_begin / 32;   // absolute unit number of unit 0 of this block
-    // a unit brings the key scale / zero of its token group along when it opens the group or
-    // is the first of a chunk
-    auto issue_unit = [&](int u, int slot, bool opener) {
+    // a unit that opens a token group brings the group's key scale / zero along, into group slot `gslot`
+    auto issue_unit = [&](int u, int slot, bool opener, int gslot) VQ_INLINE_LAMBDA {
         const int64_t base = t_begin + (int64_t)u * 32;
         const u32 sl = wring_lds + (u32)slot * RG::SLOT;
         const char *kp = kb + base * KW * 4;
@@ -293,11 +291,12 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         if (opener) {
             const int64_t grp = base / G;
             const char *ksp = ksb + grp * MF_D * MSZ, *kzp = kzb + grp * MF_D * MSZ;
-            lds_copy4<0>(ksp, l4, sl + RG::KS_OFF);
-            lds_copy4<0>(kzp, l4, sl + RG::KZ_OFF);
+            const u32 gs = wring_lds + RG::GROUP_OFF + (u32)gslot * RG::GROUP_SLOT;
+            lds_copy4<0>(ksp, l4, gs);
+            lds_copy4<0>(kzp, l4, gs + RG::KMR);
             if constexpr (RG::KM_COPIES == 2) {
-                lds_copy4<256>(ksp, l4, sl + RG::KS_OFF);
-                lds_copy4<256>(kzp, l4, sl + RG::KZ_OFF);
+                lds_copy4<256>(ksp, l4, gs);
+                lds_copy4<256>(kzp, l4, gs + RG::KMR);
             }
         }
     };
@@ -307,7 +306,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
     const int tok_a = vtok_lo<BITS>(blk, 0);
     const int zrow = n < GV ? GV + n : n % GV;            // row of the [scale rows | zero rows] image
-    auto read_unit = [&](int slot, Unit &d) {
+    auto read_unit = [&](int slot, Unit &d) VQ_INLINE_LAMBDA {
         const char *sl = wring + slot * RG::SLOT;
         if constexpr (BITS == 4) {
 #pragma unroll
@@ -329,9 +328,9 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         for (int g = 0; g < GV; ++g) d.s[g].read(sl + RG::VS_OFF + g * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
         d.z.read(sl + RG::VS_OFF + zrow * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
     };
-    auto read_group = [&](int slot, ChanMeta<M> &km) {
-        const char *sl = wring + slot * RG::SLOT;
-        km.read(sl + RG::KS_OFF + 32 * blk * (int)MSZ, sl + RG::KZ_OFF + 32 * blk * (int)MSZ);
+    auto read_group = [&](int gslot, ChanMeta<M> &km) VQ_INLINE_LAMBDA {
+        const char *gs = wring + RG::GROUP_OFF + gslot * RG::GROUP_SLOT;
+        km.read(gs + 32 * blk * (int)MSZ, gs + RG::KMR + 32 * blk * (int)MSZ);
     };
 
     f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
@@ -340,23 +339,24 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const f16x8 negoff = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair,
                                Magic<BITS>::neg_off_pair);
 
-    auto open_group = [&](const ChanMeta<M> &km) {
+    auto open_group = [&](const ChanMeta<M> &km) VQ_INLINE_LAMBDA {
         f32x4 bt = {0.f, 0.f, 0.f, 0.f};
         if constexpr (sizeof(M) == 2) {
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) bt = VQ_MFMA(as_h8(km.z[ks]), as_h8(s_q[ks * 64 + lane]), bt);
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
-                const uint4 qs = s_q[(4 + ks) * 64 + lane], ql = s_q[(8 + ks) * 64 + lane];
-                const u32 qsw[4] = {qs.x, qs.y, qs.z, qs.w}, qlw[4] = {ql.x, ql.y, ql.z, ql.w};
+                const uint4 qs = s_q[(4 + ks) * 64 + lane];
+                const u32 qsw[4] = {qs.x, qs.y, qs.z, qs.w};
                 u32 o[4];
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
                     const f16x2 sp = as_h2(km.spair(kchan_lo<BITS>(ks, p), kchan_hi<BITS>(ks, p)));
-                    const f16x2 t = as_h2(qsw[p]) * sp;   // +round(q s) | -round(q s)
+                    const f16x2 t = as_h2(qsw[p]) * sp;   // round(q s)
                     // q*s has at most 22 significant bits: the remainder after the fp16
                     // high part is itself an fp16 number, so this fma is exact
-                    o[p] = as_u(__builtin_elementwise_fma(as_h2(qlw[p]), sp, t));
+                    const f16x2 rem = __builtin_elementwise_fma(as_h2(qsw[p]), sp, -t);
+                    o[p] = n < R ? as_u(t) : as_u(rem);
                 }
                 qB[ks] = as_h8(o[0], o[1], o[2], o[3]);
             }
@@ -384,8 +384,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const int ch = (j & 1) ? kchan_hi<BITS>(ks, j >> 1) : kchan_lo<BITS>(ks, j >> 1);
-                    const float qv = n < R ? (float)qs[j] : -(float)qs[j];   // columns >= R hold -q
-                    const float t = qv * km.sval(ch);
+                    const float t = (float)qs[j] * km.sval(ch);
                     const f16 hi = (f16)t;
                     const f16 lo = (f16)(t - (float)hi);
                     qB[ks][j] = n < R ? hi : lo;
@@ -398,16 +397,21 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     };
 
     // ---- one unit: scores, softmax, output
-    auto compute = [&](const Unit &cur, int64_t base) {
+    auto compute = [&](const Unit &cur, int64_t base) VQ_INLINE_LAMBDA {
         f32x4 S[2];
 #pragma unroll
-        for (int T = 0; T < 2; ++T)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const u32 w = BITS == 4 ? cur.kw[T][ks] : (cur.kw[T][ks / 2] >> (8 * (ks % 2)));
-                const f16x8 A = unpack8<BITS>(w, magic);
-                S[T] = VQ_MFMA(A, qB[ks], ks == 0 ? bias : S[T]);
+        for (int T = 0; T < 2; ++T) {
+            f16x8 A[4];   // per k-step
+            if constexpr (BITS == 4) {
+                unpack8_pair<4>(cur.kw[T][0], cur.kw[T][1], magic, A[0], A[1]);
+                unpack8_pair<4>(cur.kw[T][2], cur.kw[T][3], magic, A[2], A[3]);
+            } else {   // word j holds k-steps 2j (low bytes) and 2j + 1 (high bytes)
+                unpack8_pair<2>(cur.kw[T][0], cur.kw[T][1], magic, A[0], A[2]);
+                unpack8_pair_upper2(cur.kw[T][0], cur.kw[T][1], magic, A[1], A[3]);
             }
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) S[T] = VQ_MFMA(A[ks], qB[ks], ks == 0 ? bias : S[T]);
+        }
         // column n < R: add the remainder column n + R; other columns idle
 #define VQ_ADD_SHL(N)                                                                         \
     _Pragma("unroll") for (int T = 0; T < 2; ++T) _Pragma("unroll") for (int r = 0; r < 4; ++r) \
@@ -491,11 +495,18 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             }
             const f16x8 Ah = as_h8(ah[0], ah[1], ah[2], ah[3]), Al = as_h8(al[0], al[1], al[2], al[3]);
 #pragma unroll
-            for (int j = 0; j < TPG; ++j) {
+            for (int j = 0; j < TPG; j += 2) {
                 const int nt = g * TPG + j;
-                const f16x8 Bv = unpack8<BITS>(cur.vw[nt] >> vshift, magic);
-                acc.O[nt] = VQ_MFMA(Ah, Bv, acc.O[nt]);
-                acc.O[nt] = VQ_MFMA(Al, Bv, acc.O[nt]);
+                f16x8 Bv0, Bv1;
+                if constexpr (BITS == 4) unpack8_pair<4>(cur.vw[nt], cur.vw[nt + 1], magic, Bv0, Bv1);
+                else {
+                    const u64 x = pack64(cur.vw[nt], cur.vw[nt + 1]) >> vshift;   // the lane's byte of each 16-token word
+                    unpack8_pair<2>((u32)x, (u32)(x >> 32), magic, Bv0, Bv1);
+                }
+                acc.O[nt] = VQ_MFMA(Ah, Bv0, acc.O[nt]);
+                acc.O[nt] = VQ_MFMA(Al, Bv0, acc.O[nt]);
+                acc.O[nt + 1] = VQ_MFMA(Ah, Bv1, acc.O[nt + 1]);
+                acc.O[nt + 1] = VQ_MFMA(Al, Bv1, acc.O[nt + 1]);
             }
             if constexpr (sizeof(M) != 2) {
                 acc.Off[g] = VQ_MFMA(Ah, ones, acc.Off[g]);
@@ -526,22 +537,24 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     // `c_next`, `c_after` queue them (NONE = nothing queued, END = the block has no more).
     constexpr int CH = RG::CHUNK;
     const int n_chunks = (n_units + CH - 1) / CH;
-    auto draw = [&]() {   // the next chunk of the block; the value is used a chunk later
+    auto draw = [&]() VQ_INLINE_LAMBDA {   // the next chunk of the block; the value is used a chunk later
         int id = 0;
         if (lane == 0) id = __hip_atomic_fetch_add(s_next, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         return id;
     };
-    auto chunk_len = [&](int chunk) { return n_units - chunk * CH < CH ? n_units - chunk * CH : CH; };
+    auto chunk_len = [&](int chunk) VQ_INLINE_LAMBDA { return n_units - chunk * CH < CH ? n_units - chunk * CH : CH; };
     if (wave >= n_chunks) return;   // the first PK_WAVES chunks are dealt out, the counter starts behind them
     constexpr int END = -1, NONE = -2;
-    int i_chunk = wave, i_pos = 0, i_slot = 0;
-    int c_chunk = wave, c_pos = 0, c_next = NONE, c_after = NONE, c_slot = 0;
+    int i_chunk = wave, i_pos = 0, i_slot = 0, i_gslot = 0;
+    int c_chunk = wave, c_pos = 0, c_next = NONE, c_after = NONE, c_slot = 0, c_gslot = 0;
     int in_flight = 0;
     int drawn = draw();
-    auto issue_next = [&]() {
-        const int u = i_chunk * CH + i_pos;
-        issue_unit(u, i_slot, i_pos == 0 || (unit0 + u) % RG::UPG == 0);
+    auto issue_next = [&]() VQ_INLINE_LAMBDA {
+        const bool opener = i_pos % RG::UPG == 0;   // chunks start on group boundaries
+        issue_unit(i_chunk * CH + i_pos, i_slot, opener, i_gslot);
         i_slot = i_slot + 1 == RG::DEPTH ? 0 : i_slot + 1;
+        const int g_next = i_gslot + 1 == RG::GROUP_SLOTS ? 0 : i_gslot + 1;
+        i_gslot = opener ? g_next : i_gslot;
         ++in_flight;
         if (++i_pos == chunk_len(i_chunk)) {
             const int got = __builtin_amdgcn_readfirstlane(drawn);
@@ -552,22 +565,24 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             if (i_chunk >= 0) drawn = draw();
         }
     };
-#pragma unroll
-    for (int j = 0; j < RG::DEPTH - 1; ++j)
+    // the first DEPTH - 1 passes only issue copies
+    for (int pass = 1 - RG::DEPTH; c_chunk >= 0; ++pass) {
         if (i_chunk >= 0) issue_next();
-    while (c_chunk >= 0) {
-        if (i_chunk >= 0) issue_next();
+        if (pass < 0) continue;
         // with a full ring exactly DEPTH - 1 units were issued behind the one awaited
         if (in_flight == RG::DEPTH) wait_copies<RG::LATER>();
         else wait_copies<0>();
         const int u = c_chunk * CH + c_pos;
         Unit cur;
         read_unit(c_slot, cur);
-        if (c_pos == 0 || (unit0 + u) % RG::UPG == 0) {
+        const bool opens = c_pos % RG::UPG == 0;
+        if (opens) {
             ChanMeta<M> km;
-            read_group(c_slot, km);
+            read_group(c_gslot, km);
             open_group(km);
         }
+        const int cg_next = c_gslot + 1 == RG::GROUP_SLOTS ? 0 : c_gslot + 1;
+        c_gslot = opens ? cg_next : c_gslot;
         compute(cur, t_begin + (int64_t)u * 32);
         c_slot = c_slot + 1 == RG::DEPTH ? 0 : c_slot + 1;
         --in_flight;
