@@ -266,20 +266,23 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     constexpr u32 VM_ACTIVE = RG::VMR / 4 < 64 ? RG::VMR / 4 : 64;
 
     // a unit that opens a token group brings the group's key scale / zero along, into group slot `gslot`
+    // blocks start on a token-group boundary; every byte offset of a unit fits 32 bits
+    // (cap_tokens <= 2^24)
+    const u32 unit0 = (u32)(t_begin / 32);
     auto issue_unit = [&](int u, int slot, bool opener, int gslot) VQ_INLINE_LAMBDA {
-        const int64_t base = t_begin + (int64_t)u * 32;
+        const u32 ug = unit0 + (u32)u;   // unit number counted from token 0
         const u32 sl = wring_lds + (u32)slot * RG::SLOT;
-        const char *kp = kb + base * KW * 4;
+        const char *kp = kb + ug * (u32)RG::KB;
         if constexpr (BITS == 4) {
             lds_copy16<0>(kp, koff, sl + RG::K_OFF);
             lds_copy16<GAP * KW * 4>(kp, koff, sl + RG::K_OFF + 1024 - GAP * KW * 4);
         } else {
             lds_copy16<0>(kp, koff, sl + RG::K_OFF);
         }
-        const char *vp = vb + (base / PER) * MF_D * 4;
+        const char *vp = vb + ug * (u32)RG::VB;
         lds_copy16<0>(vp, l16, sl + RG::V_OFF);
         if constexpr (BITS == 4) lds_copy16<1024>(vp, l16, sl + RG::V_OFF);
-        const char *vsp = vsb + base * MSZ, *vzp = vzb + base * MSZ;
+        const char *vsp = vsb + ug * (32 * MSZ), *vzp = vzb + ug * (32 * MSZ);
         if (VM_ACTIVE == 64 || lane < (int)VM_ACTIVE) {
             lds_copy4<0>(vsp, vmoff0, sl + RG::VS_OFF);
             lds_copy4<0>(vzp, vmoff0, sl + RG::VZ_OFF);
@@ -289,8 +292,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             }
         }
         if (opener) {
-            const int64_t grp = base / G;
-            const char *ksp = ksb + grp * MF_D * MSZ, *kzp = kzb + grp * MF_D * MSZ;
+            const u32 goff = (ug / (u32)RG::UPG) * (u32)RG::KMR;
+            const char *ksp = ksb + goff, *kzp = kzb + goff;
             const u32 gs = wring_lds + RG::GROUP_OFF + (u32)gslot * RG::GROUP_SLOT;
             lds_copy4<0>(ksp, l4, gs);
             lds_copy4<0>(kzp, l4, gs + RG::KMR);
