@@ -21,6 +21,32 @@ __device__ __forceinline__ float quant_code(float v, float mn, float sc, float l
     float q = rintf(__fdiv_rn(__fsub_rn(v, mn), sc));
     return fminf(fmaxf(q, 0.0f), levels);
 }
+// Eight codes at once without eight IEEE divisions.  q0 = (v - mn) * rcp(sc) lies within
+// 2.4e-7 * q of the correctly rounded quotient q = (v - mn) / sc, so rint(q0) == rint(q)
+// unless q0 is that close to a tie k + 0.5; `tie_eps` = 5e-7 * (levels + 1) bounds that
+// distance for every quotient in range.  A wave in which any lane meets such a case (or a
+// quotient out of range, or `redo`: a scale too small for rcp) redoes its eight codes with
+// the true division.  `rs` = approximate 1 / sc per element.  Bit-identical to quant_code.
+__device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
+                                             const float (&rs)[8], float levels, float tie_eps, bool redo,
+                                             float (&q)[8]) {
+    bool close = redo;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float q0 = __fmul_rn(__fsub_rn(v[i], mn[i]), rs[i]);
+        const float r = rintf(q0);
+        close |= fabsf(fabsf(q0 - r) - 0.5f) <= tie_eps;
+        close |= q0 > levels + 1.0f;
+        q[i] = fminf(fmaxf(r, 0.0f), levels);
+    }
+    if (__any(close)) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
+    }
+}
+__device__ __forceinline__ float tie_distance(float levels) { return 5e-7f * (levels + 1.0f); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+
 __device__ __forceinline__ float recon(float q, float sc, float mn) {
     return __fadd_rn(__fmul_rn(q, sc), mn);
 }
@@ -70,6 +96,10 @@ template <> __device__ __forceinline__ void store8<float>(float *p, const float 
 template <typename M> __device__ __forceinline__ void store_meta(M *p, float v);
 template <> __device__ __forceinline__ void store_meta<float>(float *p, float v) { *p = v; }
 template <> __device__ __forceinline__ void store_meta<f16>(f16 *p, float v) { *p = (f16)v; }
+// eight consecutive scale / zero values, 16-byte aligned destination
+template <typename M> __device__ __forceinline__ void store_meta8(M *p, const float (&v)[8]);
+template <> __device__ __forceinline__ void store_meta8<float>(float *p, const float (&v)[8]) { store8<float>(p, v); }
+template <> __device__ __forceinline__ void store_meta8<f16>(f16 *p, const float (&v)[8]) { store8<f16>(p, v); }
 template <typename M> __device__ __forceinline__ float load_meta(const M *p);
 template <> __device__ __forceinline__ float load_meta<float>(const float *p) { return *p; }
 template <> __device__ __forceinline__ float load_meta<f16>(const f16 *p) { return (float)*p; }
@@ -112,28 +142,29 @@ __device__ __forceinline__ void store_codes_channel_packed(uint32_t *row_words, 
 // ---------------------------------------------------------------------------
 constexpr int KT_MAXP = 8;
 
-template <typename T, typename M, int LPR, int MODE>
+template <typename T, typename M, int LPR, int MODE, int NP>
 __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
     const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
     float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
     int64_t cap_tokens, int64_t dst_tok0, int W) {
     constexpr int D = LPR * 8;
     constexpr int RPP = 256 / LPR;
-    __shared__ float s_mn[4][D];
-    __shared__ float s_mx[4][D];
+    // per-row-slot minima / maxima, then the group's (zero, scale, 1 / scale) per channel
+    __shared__ __align__(16) float s_mn[RPP][D];
+    __shared__ __align__(16) float s_mx[RPP][D];
+    __shared__ __align__(16) float s_par[3][D];
     const int gk = blockIdx.x;
     const int64_t bh = blockIdx.y;
     const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
-    const int lane = tid & 63, wave = tid >> 6;
     const int64_t s0 = (int64_t)gk * group;
     const T *xb = x + bh * x_stride_bh;
 
-    float v[KT_MAXP][8];
+    float v[NP][8];   // NP passes of RPP rows cover the group
     float mn[8], mx[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) { mn[i] = INFINITY; mx[i] = -INFINITY; }
 #pragma unroll
-    for (int p = 0; p < KT_MAXP; ++p) {
+    for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
         if (rl < group && s < S) {
@@ -142,52 +173,66 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
             for (int i = 0; i < 8; ++i) { mn[i] = fminf(mn[i], v[p][i]); mx[i] = fmaxf(mx[i], v[p][i]); }
         }
     }
+    *reinterpret_cast<float4 *>(&s_mn[r][8 * o]) = make_float4(mn[0], mn[1], mn[2], mn[3]);
+    *reinterpret_cast<float4 *>(&s_mn[r][8 * o + 4]) = make_float4(mn[4], mn[5], mn[6], mn[7]);
+    *reinterpret_cast<float4 *>(&s_mx[r][8 * o]) = make_float4(mx[0], mx[1], mx[2], mx[3]);
+    *reinterpret_cast<float4 *>(&s_mx[r][8 * o + 4]) = make_float4(mx[4], mx[5], mx[6], mx[7]);
+    __syncthreads();
+    // one thread per channel folds the row slots and does the one division of the group
+    for (int ch = tid; ch < D; ch += 256) {
+        float a = INFINITY, b = -INFINITY;
 #pragma unroll
-    for (int off = LPR; off < 64; off <<= 1) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            mn[i] = fminf(mn[i], __shfl_xor(mn[i], off));
-            mx[i] = fmaxf(mx[i], __shfl_xor(mx[i], off));
-        }
-    }
-    if (lane < LPR) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { s_mn[wave][8 * o + i] = mn[i]; s_mx[wave][8 * o + i] = mx[i]; }
+        for (int j = 0; j < RPP; ++j) { a = fminf(a, s_mn[j][ch]); b = fmaxf(b, s_mx[j][ch]); }
+        const float scv = group_scale(a, b, levels, eps);
+        s_par[0][ch] = a;
+        s_par[1][ch] = scv;
+        s_par[2][ch] = fast_rcp(scv);
     }
     __syncthreads();
-    float sc[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        float a = fminf(fminf(s_mn[0][8 * o + i], s_mn[1][8 * o + i]), fminf(s_mn[2][8 * o + i], s_mn[3][8 * o + i]));
-        float b = fmaxf(fmaxf(s_mx[0][8 * o + i], s_mx[1][8 * o + i]), fmaxf(s_mx[2][8 * o + i], s_mx[3][8 * o + i]));
-        mn[i] = a;
-        sc[i] = group_scale(a, b, levels, eps);
+    float sc[8], rs[8];
+    {
+        const float4 a0 = *reinterpret_cast<const float4 *>(&s_par[0][8 * o]), a1 = *reinterpret_cast<const float4 *>(&s_par[0][8 * o + 4]);
+        const float4 b0 = *reinterpret_cast<const float4 *>(&s_par[1][8 * o]), b1 = *reinterpret_cast<const float4 *>(&s_par[1][8 * o + 4]);
+        const float4 c0 = *reinterpret_cast<const float4 *>(&s_par[2][8 * o]), c1 = *reinterpret_cast<const float4 *>(&s_par[2][8 * o + 4]);
+        mn[0] = a0.x; mn[1] = a0.y; mn[2] = a0.z; mn[3] = a0.w; mn[4] = a1.x; mn[5] = a1.y; mn[6] = a1.z; mn[7] = a1.w;
+        sc[0] = b0.x; sc[1] = b0.y; sc[2] = b0.z; sc[3] = b0.w; sc[4] = b1.x; sc[5] = b1.y; sc[6] = b1.z; sc[7] = b1.w;
+        rs[0] = c0.x; rs[1] = c0.y; rs[2] = c0.z; rs[3] = c0.w; rs[4] = c1.x; rs[5] = c1.y; rs[6] = c1.z; rs[7] = c1.w;
     }
     if (MODE == 1 && r == 0) {
         int64_t gdst = dst_tok0 / group + gk;
         int64_t gcap = (cap_tokens + group - 1) / group;
         M *sp = scale + (bh * gcap + gdst) * D + 8 * o;
         M *zp = zero + (bh * gcap + gdst) * D + 8 * o;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { store_meta<M>(sp + i, sc[i]); store_meta<M>(zp + i, mn[i]); }
+        store_meta8<M>(sp, sc);
+        store_meta8<M>(zp, mn);
     }
+    const float tie_eps = tie_distance(levels);
+    bool redo = false;
 #pragma unroll
-    for (int p = 0; p < KT_MAXP; ++p) {
+    for (int i = 0; i < 8; ++i) redo |= !(rs[i] < 1e30f);
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
         bool valid = rl < group && s < S;
         if (p * RPP >= group) break;  // uniform across the block
+        float q[8];
+        if (!valid) {   // keep the arithmetic defined; the lane's results are not stored
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[p][i] = mn[i];
+        }
+        quant_codes8(v[p], mn, sc, rs, levels, tie_eps, redo, q);
         if (MODE == 0) {
             if (valid) {
                 float y[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) y[i] = recon(quant_code(v[p][i], mn[i], sc[i], levels), sc[i], mn[i]);
+                for (int i = 0; i < 8; ++i) y[i] = recon(q[i], sc[i], mn[i]);
                 store8<T>(out + (bh * S + s) * D + 8 * o, y);
             }
         } else {
             uint32_t c[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) c[i] = valid ? (uint32_t)quant_code(v[p][i], mn[i], sc[i], levels) : 0u;
+            for (int i = 0; i < 8; ++i) c[i] = valid ? (uint32_t)q[i] : 0u;
             uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;
             store_codes_channel_packed<LPR>(row, o, c, bits, valid);
         }
@@ -199,6 +244,8 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
 // reduced across g/8 neighbouring lanes.  MODE 0 reconstruction, MODE 1
 // channel-packed codes, MODE 2 token-packed codes (transposed through LDS).
 // ---------------------------------------------------------------------------
+constexpr int VT_TILES = 4;   // row tiles of 256 / LPR rows one block of the value kernel takes
+
 template <typename T, typename M, int LPR, int MODE>
 __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
     const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
@@ -206,57 +253,102 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
     int64_t cap_tokens, int64_t dst_tok0, int W) {
     constexpr int D = LPR * 8;
     constexpr int RPP = 256 / LPR;
+    constexpr int ROWS = RPP * VT_TILES;
     constexpr int LDS_STRIDE = D + 8;
-    __shared__ __align__(8) unsigned char s_codes[MODE == 2 ? RPP * LDS_STRIDE : 4];
+    __shared__ __align__(8) unsigned char s_codes[MODE == 2 ? ROWS * LDS_STRIDE : 4];
+    // token-packed scale / zero rows of the tile, staged so that they leave as whole vectors
+    constexpr int MAXGV = 4;
+    __shared__ __align__(16) M s_meta[MODE == 2 ? 2 * MAXGV * ROWS : 1];
     const int64_t bh = blockIdx.y;
     const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
-    const int64_t s = (int64_t)blockIdx.x * RPP + r;
-    const bool valid = s < S;
+    const int64_t tile_tok0 = (int64_t)blockIdx.x * ROWS;
     const int GL = group / 8;  // lanes per group (power of two <= LPR)
     const int GV = D / group;
 
-    float v[8];
-    float mn = INFINITY, mx = -INFINITY;
-    if (valid) {
-        load8<T>(x + bh * x_stride_bh + s * D + 8 * o, v);
+    // every load of the thread's VT_TILES rows goes out before the first is used
+    float v[VT_TILES][8];
+    bool valid[VT_TILES];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) { mn = fminf(mn, v[i]); mx = fmaxf(mx, v[i]); }
+    for (int j = 0; j < VT_TILES; ++j) {
+        const int64_t s = tile_tok0 + j * RPP + r;
+        valid[j] = s < S;
+        if (valid[j]) load8<T>(x + bh * x_stride_bh + s * D + 8 * o, v[j]);
     }
-    for (int off = 1; off < GL; off <<= 1) {
-        mn = fminf(mn, __shfl_xor(mn, off));
-        mx = fmaxf(mx, __shfl_xor(mx, off));
-    }
-    const float sc = group_scale(mn, mx, levels, eps);
-    if (MODE != 0 && valid && (o % GL) == 0) {
-        int gv = o / GL;
-        int64_t mi = (MODE == 1) ? ((bh * cap_tokens + dst_tok0 + s) * GV + gv)
-                                 : ((bh * GV + gv) * cap_tokens + dst_tok0 + s);
-        store_meta<M>(scale + mi, sc);
-        store_meta<M>(zero + mi, mn);
-    }
-    if (MODE == 0) {
-        if (valid) {
-            float y[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) y[i] = recon(quant_code(v[i], mn, sc, levels), sc, mn);
-            store8<T>(out + (bh * S + s) * D + 8 * o, y);
+    for (int j = 0; j < VT_TILES; ++j) {
+        const int rl = j * RPP + r;
+        const int64_t s = tile_tok0 + rl;
+        float mn = INFINITY, mx = -INFINITY;
+        if (valid[j]) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { mn = fminf(mn, v[j][i]); mx = fmaxf(mx, v[j][i]); }
         }
-        return;
-    }
-    uint32_t c[8];
+        for (int off = 1; off < GL; off <<= 1) {
+            mn = fminf(mn, __shfl_xor(mn, off));
+            mx = fmaxf(mx, __shfl_xor(mx, off));
+        }
+        const float sc = group_scale(mn, mx, levels, eps);
+        if (MODE != 0 && valid[j] && (o % GL) == 0) {
+            int gv = o / GL;
+            if (MODE == 2 && GV <= MAXGV) {
+                store_meta<M>(&s_meta[gv * ROWS + rl], sc);
+                store_meta<M>(&s_meta[(MAXGV + gv) * ROWS + rl], mn);
+            } else {
+                int64_t mi = (MODE == 1) ? ((bh * cap_tokens + dst_tok0 + s) * GV + gv)
+                                         : ((bh * GV + gv) * cap_tokens + dst_tok0 + s);
+                store_meta<M>(scale + mi, sc);
+                store_meta<M>(zero + mi, mn);
+            }
+        }
+        float q[8];
+        {
+            const float rs = fast_rcp(sc);
+            float mn8[8], sc8[8], rs8[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) c[i] = valid ? (uint32_t)quant_code(v[i], mn, sc, levels) : 0u;
-    if (MODE == 1) {
-        uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;
-        store_codes_channel_packed<LPR>(row, o, c, bits, valid);
-    } else {
-        uint32_t w0 = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-        uint32_t w1 = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
-        *reinterpret_cast<uint2 *>(&s_codes[r * LDS_STRIDE + 8 * o]) = make_uint2(w0, w1);
+            for (int i = 0; i < 8; ++i) { mn8[i] = mn; sc8[i] = sc; rs8[i] = rs; if (!valid[j]) v[j][i] = mn; }
+            quant_codes8(v[j], mn8, sc8, rs8, levels, tie_distance(levels), !(rs < 1e30f), q);
+        }
+        if (MODE == 0) {
+            if (valid[j]) {
+                float y[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) y[i] = recon(q[i], sc, mn);
+                store8<T>(out + (bh * S + s) * D + 8 * o, y);
+            }
+            continue;
+        }
+        uint32_t c[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c[i] = valid[j] ? (uint32_t)q[i] : 0u;
+        if (MODE == 1) {
+            uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid[j] ? s : 0)) * W;
+            store_codes_channel_packed<LPR>(row, o, c, bits, valid[j]);
+        } else {
+            uint32_t w0 = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
+            uint32_t w1 = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
+            *reinterpret_cast<uint2 *>(&s_codes[rl * LDS_STRIDE + 8 * o]) = make_uint2(w0, w1);
+        }
+    }
+    if (MODE == 2) {
         __syncthreads();
+        if (GV <= MAXGV) {
+            constexpr int VEC = 16 / (int)sizeof(M);          // elements per 16-byte store
+            const int nvec = 2 * GV * (ROWS / VEC);
+            const int64_t tok = dst_tok0 + tile_tok0;
+            const bool whole = tile_tok0 + ROWS <= S && (tok % VEC) == 0 && (cap_tokens % VEC) == 0;
+            for (int idx = tid; idx < nvec; idx += 256) {
+                const int which = idx / (GV * (ROWS / VEC)), rem = idx % (GV * (ROWS / VEC));
+                const int gv = rem / (ROWS / VEC), t0 = (rem % (ROWS / VEC)) * VEC;
+                M *dst = (which ? zero : scale) + (bh * GV + gv) * cap_tokens + tok + t0;
+                const M *src = &s_meta[(which * MAXGV + gv) * ROWS + t0];
+                if (whole) *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
+                else
+                    for (int i = 0; i < VEC; ++i)
+                        if (tile_tok0 + t0 + i < S) dst[i] = src[i];
+            }
+        }
         const int per = 32 / bits;
-        const int nwords = (RPP / per) * D;
-        const int64_t tile_tok0 = (int64_t)blockIdx.x * RPP;
+        const int nwords = (ROWS / per) * D;
         for (int idx = tid; idx < nwords; idx += 256) {
             int wl = idx / D, d = idx % D;
             if (tile_tok0 + (int64_t)wl * per >= S) continue;
@@ -441,19 +533,22 @@ static void launch_key_tile(int mode, const void *x, void *out, int64_t BH, int6
                             int64_t tok0, hipStream_t st) {
     dim3 grid((unsigned)cdiv(S, group), (unsigned)BH);
     int W = (int)cdiv(LPR * 8, 32 / (bits > 0 ? bits : 8));
-    if (mode == 0)
-        hipLaunchKernelGGL((kivi_key_tile_kernel<T, M, LPR, 0>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, xs,
-                           group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W);
-    else
-        hipLaunchKernelGGL((kivi_key_tile_kernel<T, M, LPR, 1>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, xs,
-                           group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W);
+    // fewer passes held in registers let more blocks share a CU
+    constexpr int RPP = 256 / LPR;
+    const bool small = group <= (KT_MAXP / 2) * RPP;
+#define VQ_LK(MODE, NP)                                                                                               \
+    hipLaunchKernelGGL((kivi_key_tile_kernel<T, M, LPR, MODE, NP>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, \
+                       xs, group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W)
+    if (mode == 0) { if (small) VQ_LK(0, KT_MAXP / 2); else VQ_LK(0, KT_MAXP); }
+    else { if (small) VQ_LK(1, KT_MAXP / 2); else VQ_LK(1, KT_MAXP); }
+#undef VQ_LK
 }
 template <typename T, typename M, int LPR>
 static void launch_value_tile(int mode, const void *x, void *out, int64_t BH, int64_t S, int64_t xs, int group,
                               int levels, float eps, int bits, void *packed, void *scale, void *zero, int64_t cap,
                               int64_t tok0, hipStream_t st) {
-    constexpr int RPP = 256 / LPR;
-    dim3 grid((unsigned)cdiv(S, RPP), (unsigned)BH);
+    constexpr int ROWS = (256 / LPR) * VT_TILES;
+    dim3 grid((unsigned)cdiv(S, ROWS), (unsigned)BH);
     int W = (int)cdiv(LPR * 8, 32 / (bits > 0 ? bits : 8));
 #define VQ_LV(MODE)                                                                                                  \
     hipLaunchKernelGGL((kivi_value_tile_kernel<T, M, LPR, MODE>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, \
@@ -473,7 +568,7 @@ static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t 
     if (!aligned16(x) || (xs % 8) != 0 || BH > 65535) return false;
     if (mode == 0 && !aligned16(out)) return false;
     if (mode != 0 && !(bits == 1 || bits == 2 || bits == 4 || bits == 8)) return false;
-    if (mode != 0 && !aligned16(packed)) return false;
+    if (mode != 0 && !(aligned16(packed) && aligned16(scale) && aligned16(zero))) return false;
     const int LPR = (int)(D / 8), RPP = 256 / LPR;
     if (axis == VQ_AXIS_TOKEN) {
         if (group > KT_MAXP * RPP) return false;
