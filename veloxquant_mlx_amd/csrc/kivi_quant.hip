@@ -21,30 +21,55 @@ __device__ __forceinline__ float quant_code(float v, float mn, float sc, float l
     float q = rintf(__fdiv_rn(__fsub_rn(v, mn), sc));
     return fminf(fmaxf(q, 0.0f), levels);
 }
-// Eight codes at once without eight IEEE divisions.  q0 = (v - mn) * rcp(sc) lies within
-// 2.4e-7 * q of the correctly rounded quotient q = (v - mn) / sc, so rint(q0) == rint(q)
-// unless q0 is that close to a tie k + 0.5; `tie_eps` = 5e-7 * (levels + 1) bounds that
-// distance for every quotient in range.  A wave in which any lane meets such a case (or a
-// quotient out of range, or `redo`: a scale too small for rcp) redoes its eight codes with
-// the true division.  `rs` = approximate 1 / sc per element.  Bit-identical to quant_code.
+// Eight codes at once without eight IEEE divisions.  With rs ~ 1 / sc and nb = -mn * rs,
+// q0 = fma(v, rs, nb) lies within 3e-7 * q + 6e-8 * |nb| of the correctly rounded quotient
+// q = (v - mn) / sc, so rint(q0) == rint(q) unless q0 is that close to a tie k + 0.5:
+// `tie_lo` = 0.5 - (5e-7 * (levels + 1) + 2e-7 * |nb|) is the distance from rint(q0) beyond
+// which a lane counts as undecided.  A wave in which any lane is undecided (or `redo`: a scale
+// too small for rcp) redoes its eight codes with the true division.  Bit-identical to quant_code;
+// the codes come back as floats.
 __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
-                                             const float (&rs)[8], float levels, float tie_eps, bool redo,
-                                             float (&q)[8]) {
+                                             const float (&rs)[8], const float (&nb)[8], const float (&tie_lo)[8],
+                                             float levels, bool redo, float (&q)[8]) {
     bool close = redo;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-        const float q0 = __fmul_rn(__fsub_rn(v[i], mn[i]), rs[i]);
+        const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
         const float r = rintf(q0);
-        close |= fabsf(fabsf(q0 - r) - 0.5f) <= tie_eps;
-        close |= q0 > levels + 1.0f;
-        q[i] = fminf(fmaxf(r, 0.0f), levels);
+        close |= fabsf(q0 - r) >= tie_lo[i];
+        q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels);   // clamp; a NaN becomes 0 as with fmaxf / fminf
     }
     if (__any(close)) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
-__device__ __forceinline__ float tie_distance(float levels) { return 5e-7f * (levels + 1.0f); }
+__device__ __forceinline__ float tie_limit(float levels, float nb) {
+    return 0.5f - (5e-7f * (levels + 1.0f) + 2e-7f * fabsf(nb));
+}
+// Eight codes (exact small integers held as floats) as one bit field, code i at bit i * bits;
+// bits * 8 <= 32.  Sums stay below 2^16 per half, so float arithmetic is exact.
+__device__ __forceinline__ uint32_t field8(const float (&q)[8], int bits) {
+    const float b = (float)(1 << bits);
+    if (bits <= 2) {
+        float f = q[7];
+#pragma unroll
+        for (int i = 6; i >= 0; --i) f = __builtin_fmaf(f, b, q[i]);
+        return (uint32_t)f;
+    }
+    if (bits == 4) {
+        const float lo = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(q[3], b, q[2]), b, q[1]), b, q[0]);
+        const float hi = __builtin_fmaf(__builtin_fmaf(__builtin_fmaf(q[7], b, q[6]), b, q[5]), b, q[4]);
+        return (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+    return 0;   // 8 bits: two words, see bytes8
+}
+// eight codes as eight bytes
+__device__ __forceinline__ uint2 bytes8(const float (&q)[8]) {
+    const uint32_t a = (uint32_t)__builtin_fmaf(q[1], 256.0f, q[0]), b = (uint32_t)__builtin_fmaf(q[3], 256.0f, q[2]);
+    const uint32_t c = (uint32_t)__builtin_fmaf(q[5], 256.0f, q[4]), d = (uint32_t)__builtin_fmaf(q[7], 256.0f, q[6]);
+    return make_uint2(a | (b << 16), c | (d << 16));
+}
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 
 __device__ __forceinline__ float recon(float q, float sc, float mn) {
@@ -107,33 +132,81 @@ template <> __device__ __forceinline__ float load_meta<f16>(const f16 *p) { retu
 // Write the eight codes one thread owns (channels 8*o .. 8*o+7 of one row) as
 // part of a channel-packed row of words.  Every lane of the wave must call it.
 template <int LPR>
-__device__ __forceinline__ void store_codes_channel_packed(uint32_t *row_words, int o, const uint32_t (&c)[8],
+__device__ __forceinline__ void store_codes_channel_packed(uint32_t *row_words, int o, const float (&q)[8],
                                                            int bits, bool valid) {
     if (bits == 8) {
-        if (valid) {
-            uint32_t w0 = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-            uint32_t w1 = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
-            *reinterpret_cast<uint2 *>(row_words + 2 * o) = make_uint2(w0, w1);
-        }
+        if (valid) *reinterpret_cast<uint2 *>(row_words + 2 * o) = bytes8(q);
     } else if (bits == 4) {
-        uint32_t w = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) w |= c[i] << (4 * i);
+        const uint32_t w = field8(q, 4);
         if (valid) row_words[o] = w;
     } else if (bits == 2) {
-        uint32_t f = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f |= c[i] << (2 * i);
+        const uint32_t f = field8(q, 2);
         uint32_t hi = __shfl_down(f, 1);
         if (valid && (o & 1) == 0) row_words[o >> 1] = f | (hi << 16);
     } else {  // bits == 1
-        uint32_t f = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) f |= c[i] << i;
+        const uint32_t f = field8(q, 1);
         uint32_t f1 = __shfl_down(f, 1), f2 = __shfl_down(f, 2), f3 = __shfl_down(f, 3);
         if (valid && (o & 3) == 0) row_words[o >> 2] = f | (f1 << 8) | (f2 << 16) | (f3 << 24);
     }
 }
+
+// Eight consecutive elements as loaded, with running per-element minima / maxima kept in the
+// storage type where that is exact and cheaper (fp16: packed min / max, two elements per
+// instruction).
+template <typename T> struct Raw8 {
+    float v[8];
+    struct Acc { float mn[8], mx[8]; };
+    __device__ __forceinline__ void load(const T *p) { load8<T>(p, v); }
+    __device__ __forceinline__ void floats(float (&o)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = v[i];
+    }
+    static __device__ __forceinline__ void init(Acc &a) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { a.mn[i] = INFINITY; a.mx[i] = -INFINITY; }
+    }
+    __device__ __forceinline__ void fold(Acc &a) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { a.mn[i] = fminf(a.mn[i], v[i]); a.mx[i] = fmaxf(a.mx[i], v[i]); }
+    }
+    static __device__ __forceinline__ void result(const Acc &a, float (&mn)[8], float (&mx)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { mn[i] = a.mn[i]; mx[i] = a.mx[i]; }
+    }
+    // minimum / maximum over the eight elements
+    __device__ __forceinline__ void span(float &mn, float &mx) const {
+        mn = INFINITY; mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { mn = fminf(mn, v[i]); mx = fmaxf(mx, v[i]); }
+    }
+};
+template <> struct Raw8<f16> {
+    f16x8 h;
+    struct Acc { f16x8 mn, mx; };
+    __device__ __forceinline__ void load(const f16 *p) { h = *reinterpret_cast<const f16x8 *>(p); }
+    __device__ __forceinline__ void floats(float (&o)[8]) const {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o[i] = (float)h[i];
+    }
+    static __device__ __forceinline__ void init(Acc &a) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { a.mn[i] = (f16)INFINITY; a.mx[i] = (f16)-INFINITY; }
+    }
+    __device__ __forceinline__ void fold(Acc &a) const {
+        a.mn = __builtin_elementwise_min(a.mn, h);
+        a.mx = __builtin_elementwise_max(a.mx, h);
+    }
+    static __device__ __forceinline__ void result(const Acc &a, float (&mn)[8], float (&mx)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { mn[i] = (float)a.mn[i]; mx[i] = (float)a.mx[i]; }
+    }
+    __device__ __forceinline__ void span(float &mn, float &mx) const {
+        const f16x4 a = __builtin_elementwise_min(h.lo, h.hi), b = __builtin_elementwise_max(h.lo, h.hi);
+        const f16x2 a2 = __builtin_elementwise_min(a.lo, a.hi), b2 = __builtin_elementwise_max(b.lo, b.hi);
+        mn = fminf((float)a2[0], (float)a2[1]);
+        mx = fmaxf((float)b2[0], (float)b2[1]);
+    }
+};
 
 // ---------------------------------------------------------------------------
 // Keys: groups along tokens.  One block per (group, bh); 256 threads = RPP rows
@@ -152,27 +225,27 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
     // per-row-slot minima / maxima, then the group's (zero, scale, 1 / scale) per channel
     __shared__ __align__(16) float s_mn[RPP][D];
     __shared__ __align__(16) float s_mx[RPP][D];
-    __shared__ __align__(16) float s_par[3][D];
+    __shared__ __align__(16) float s_par[4][D];
     const int gk = blockIdx.x;
     const int64_t bh = blockIdx.y;
     const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
     const int64_t s0 = (int64_t)gk * group;
     const T *xb = x + bh * x_stride_bh;
 
-    float v[NP][8];   // NP passes of RPP rows cover the group
-    float mn[8], mx[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { mn[i] = INFINITY; mx[i] = -INFINITY; }
+    Raw8<T> v[NP];   // NP passes of RPP rows cover the group
+    typename Raw8<T>::Acc acc;
+    Raw8<T>::init(acc);
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
         if (rl < group && s < S) {
-            load8<T>(xb + s * D + 8 * o, v[p]);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) { mn[i] = fminf(mn[i], v[p][i]); mx[i] = fmaxf(mx[i], v[p][i]); }
+            v[p].load(xb + s * D + 8 * o);
+            v[p].fold(acc);
         }
     }
+    float mn[8], mx[8];
+    Raw8<T>::result(acc, mn, mx);
     *reinterpret_cast<float4 *>(&s_mn[r][8 * o]) = make_float4(mn[0], mn[1], mn[2], mn[3]);
     *reinterpret_cast<float4 *>(&s_mn[r][8 * o + 4]) = make_float4(mn[4], mn[5], mn[6], mn[7]);
     *reinterpret_cast<float4 *>(&s_mx[r][8 * o]) = make_float4(mx[0], mx[1], mx[2], mx[3]);
@@ -184,20 +257,22 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
 #pragma unroll
         for (int j = 0; j < RPP; ++j) { a = fminf(a, s_mn[j][ch]); b = fmaxf(b, s_mx[j][ch]); }
         const float scv = group_scale(a, b, levels, eps);
+        const float rsv = fast_rcp(scv);
         s_par[0][ch] = a;
         s_par[1][ch] = scv;
-        s_par[2][ch] = fast_rcp(scv);
+        s_par[2][ch] = rsv;
+        s_par[3][ch] = -a * rsv;
     }
     __syncthreads();
-    float sc[8], rs[8];
-    {
-        const float4 a0 = *reinterpret_cast<const float4 *>(&s_par[0][8 * o]), a1 = *reinterpret_cast<const float4 *>(&s_par[0][8 * o + 4]);
-        const float4 b0 = *reinterpret_cast<const float4 *>(&s_par[1][8 * o]), b1 = *reinterpret_cast<const float4 *>(&s_par[1][8 * o + 4]);
-        const float4 c0 = *reinterpret_cast<const float4 *>(&s_par[2][8 * o]), c1 = *reinterpret_cast<const float4 *>(&s_par[2][8 * o + 4]);
-        mn[0] = a0.x; mn[1] = a0.y; mn[2] = a0.z; mn[3] = a0.w; mn[4] = a1.x; mn[5] = a1.y; mn[6] = a1.z; mn[7] = a1.w;
-        sc[0] = b0.x; sc[1] = b0.y; sc[2] = b0.z; sc[3] = b0.w; sc[4] = b1.x; sc[5] = b1.y; sc[6] = b1.z; sc[7] = b1.w;
-        rs[0] = c0.x; rs[1] = c0.y; rs[2] = c0.z; rs[3] = c0.w; rs[4] = c1.x; rs[5] = c1.y; rs[6] = c1.z; rs[7] = c1.w;
-    }
+    float sc[8], rs[8], nb[8], tie_lo[8];
+    auto row8 = [&](int k, float (&d)[8]) {
+        const float4 lo = *reinterpret_cast<const float4 *>(&s_par[k][8 * o]), hi = *reinterpret_cast<const float4 *>(&s_par[k][8 * o + 4]);
+        d[0] = lo.x; d[1] = lo.y; d[2] = lo.z; d[3] = lo.w; d[4] = hi.x; d[5] = hi.y; d[6] = hi.z; d[7] = hi.w;
+    };
+    row8(0, mn); row8(1, sc); row8(2, rs); row8(3, nb);
+    bool redo = false;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { tie_lo[i] = tie_limit(levels, nb[i]); redo |= !(rs[i] < 1e30f); }
     if (MODE == 1 && r == 0) {
         int64_t gdst = dst_tok0 / group + gk;
         int64_t gcap = (cap_tokens + group - 1) / group;
@@ -206,22 +281,19 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
         store_meta8<M>(sp, sc);
         store_meta8<M>(zp, mn);
     }
-    const float tie_eps = tie_distance(levels);
-    bool redo = false;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) redo |= !(rs[i] < 1e30f);
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
         bool valid = rl < group && s < S;
         if (p * RPP >= group) break;  // uniform across the block
-        float q[8];
-        if (!valid) {   // keep the arithmetic defined; the lane's results are not stored
+        float x8[8], q[8];
+        if (valid) v[p].floats(x8);
+        else {   // keep the arithmetic defined; the lane's results are not stored
 #pragma unroll
-            for (int i = 0; i < 8; ++i) v[p][i] = mn[i];
+            for (int i = 0; i < 8; ++i) x8[i] = mn[i];
         }
-        quant_codes8(v[p], mn, sc, rs, levels, tie_eps, redo, q);
+        quant_codes8(x8, mn, sc, rs, nb, tie_lo, levels, redo, q);
         if (MODE == 0) {
             if (valid) {
                 float y[8];
@@ -230,11 +302,8 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
                 store8<T>(out + (bh * S + s) * D + 8 * o, y);
             }
         } else {
-            uint32_t c[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) c[i] = valid ? (uint32_t)q[i] : 0u;
             uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;
-            store_codes_channel_packed<LPR>(row, o, c, bits, valid);
+            store_codes_channel_packed<LPR>(row, o, q, bits, valid);
         }
     }
 }
@@ -266,23 +335,20 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
     const int GV = D / group;
 
     // every load of the thread's VT_TILES rows goes out before the first is used
-    float v[VT_TILES][8];
+    Raw8<T> v[VT_TILES];
     bool valid[VT_TILES];
 #pragma unroll
     for (int j = 0; j < VT_TILES; ++j) {
         const int64_t s = tile_tok0 + j * RPP + r;
         valid[j] = s < S;
-        if (valid[j]) load8<T>(x + bh * x_stride_bh + s * D + 8 * o, v[j]);
+        if (valid[j]) v[j].load(x + bh * x_stride_bh + s * D + 8 * o);
     }
 #pragma unroll
     for (int j = 0; j < VT_TILES; ++j) {
         const int rl = j * RPP + r;
         const int64_t s = tile_tok0 + rl;
         float mn = INFINITY, mx = -INFINITY;
-        if (valid[j]) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) { mn = fminf(mn, v[j][i]); mx = fmaxf(mx, v[j][i]); }
-        }
+        if (valid[j]) v[j].span(mn, mx);
         for (int off = 1; off < GL; off <<= 1) {
             mn = fminf(mn, __shfl_xor(mn, off));
             mx = fmaxf(mx, __shfl_xor(mx, off));
@@ -302,11 +368,20 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
         }
         float q[8];
         {
-            const float rs = fast_rcp(sc);
-            float mn8[8], sc8[8], rs8[8];
+            const float rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
+            float x8[8], mn8[8], sc8[8], rs8[8], nb8[8], tl8[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { mn8[i] = mn; sc8[i] = sc; rs8[i] = rs; if (!valid[j]) v[j][i] = mn; }
-            quant_codes8(v[j], mn8, sc8, rs8, levels, tie_distance(levels), !(rs < 1e30f), q);
+            for (int i = 0; i < 8; ++i) { mn8[i] = mn; sc8[i] = sc; rs8[i] = rs; nb8[i] = nb; tl8[i] = tl; }
+            if (valid[j]) v[j].floats(x8);
+            else {   // keep the arithmetic defined; the lane's results are not stored
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x8[i] = 0.0f;
+            }
+            quant_codes8(x8, mn8, sc8, rs8, nb8, tl8, levels, !(rs < 1e30f), q);
+            if (!valid[j]) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) q[i] = 0.0f;
+            }
         }
         if (MODE == 0) {
             if (valid[j]) {
@@ -317,16 +392,11 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
             }
             continue;
         }
-        uint32_t c[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) c[i] = valid[j] ? (uint32_t)q[i] : 0u;
         if (MODE == 1) {
             uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid[j] ? s : 0)) * W;
-            store_codes_channel_packed<LPR>(row, o, c, bits, valid[j]);
+            store_codes_channel_packed<LPR>(row, o, q, bits, valid[j]);
         } else {
-            uint32_t w0 = c[0] | (c[1] << 8) | (c[2] << 16) | (c[3] << 24);
-            uint32_t w1 = c[4] | (c[5] << 8) | (c[6] << 16) | (c[7] << 24);
-            *reinterpret_cast<uint2 *>(&s_codes[rl * LDS_STRIDE + 8 * o]) = make_uint2(w0, w1);
+            *reinterpret_cast<uint2 *>(&s_codes[rl * LDS_STRIDE + 8 * o]) = bytes8(q);
         }
     }
     if (MODE == 2) {
