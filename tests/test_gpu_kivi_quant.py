@@ -70,6 +70,39 @@ def test_exact_half_codes_round_half_to_even(axis):
 
 
 @pytest.mark.parametrize("axis", [-2, -1])
+@pytest.mark.parametrize("b", [2, 4, 8])
+def test_quotients_on_and_next_to_ties(axis, b):
+    """Every group spans [lo, lo + levels * step] for steps with and without an exact reciprocal
+    and holds, next to random values, the values whose quotient is k + 1/2 exactly and one fp16
+    step either side of it: the kernels decide codes from a reciprocal product and must fall
+    back to the true division wherever that product cannot tell the side of the tie."""
+    rng = np.random.default_rng(100 + b)
+    levels = (1 << b) - 1
+    g, D, S = 32, 128, 64
+    x = np.zeros((1, 4, S, D), np.float32)
+    steps = [1.0, 0.5, 3.0, 0.75, 1.5, 0.375, 6.0, 0.046875]
+    for h in range(4):
+        for blk in range((S // g) if axis == -2 else (D // g)):
+            for line in range(D if axis == -2 else S):
+                step = steps[(h + blk + line) % len(steps)] * (2.0 if b == 2 else 1.0) * (1 / 16 if b == 8 else 1.0)
+                lo = float(np.float16(rng.integers(-8, 8) * step))
+                vals = lo + step * rng.uniform(0, levels, g)
+                ks = rng.integers(0, levels, g // 2)
+                vals[: g // 2] = lo + step * (ks + 0.5)
+                vals[0], vals[1] = lo, lo + step * levels
+                v16 = vals.astype(np.float16)
+                v16[2:g // 2:3] = np.nextafter(v16[2:g // 2:3], np.float16(np.inf))
+                v16[3:g // 2:3] = np.nextafter(v16[3:g // 2:3], np.float16(-np.inf))
+                if axis == -2:
+                    x[0, h, blk * g:(blk + 1) * g, line] = v16
+                else:
+                    x[0, h, line, blk * g:(blk + 1) * g] = v16
+    x16 = x.astype(np.float16)
+    _roundtrip_exact(x16, axis, b=b, g=g)
+    _pack_exact(x16, axis, b, g, torch.float16)
+
+
+@pytest.mark.parametrize("axis", [-2, -1])
 def test_no_fma_contraction_in_reconstruction(axis):
     rng = np.random.default_rng(7)
     _roundtrip_exact(rng.standard_normal((1, 4, 128, 128)).astype(np.float16), axis, b=8, g=32)
