@@ -176,6 +176,14 @@ typedef struct vq_attend_args {
     int32_t *sync_counters;
 } vq_attend_args;
 
+/* The decode kernel balances its waves by handing out token chunks on demand, so the order in
+ * which partial sums are formed, and with it the last bits of the output, can differ from one
+ * run to the next (well inside the 2e-3 bar).  enable != 0 makes every later vq_kivi_attend
+ * of the process deal the chunks in a fixed order instead: identical bits from run to run, a
+ * few percent slower.  Returns the previous setting.  No counterpart in the reference (its
+ * kernels use a fixed split order); for callers that compare runs bit for bit. */
+int vq_kivi_attend_fixed_order(int enable);
+
 /* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the
  * shapes, pack_bits, group and num_splits are ignored). */
 size_t vq_kivi_attend_workspace(const vq_attend_args *a);

@@ -197,6 +197,62 @@ def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
         assert torch.equal(c.fused_sdpa(q, scale, causal=True), o1.to(torch.bfloat16))
 
 
+def test_config3_decode_at_full_size_against_the_oracle_and_the_vector_kernel():
+    """BASELINE configs[3], one layer: batch 16, 32 query / 8 kv heads, D=128, 32768 tokens of
+    context in a 4-bit group-64 packed cache plus the fp16 residual, one query token.  The last
+    sequence is checked against the scalar C oracle (about a second of CPU), every sequence
+    against the independent vector kernel."""
+    require_gpu()
+    from oracle import cref
+    B, Hq, Hkv, D, ctx, g, bits = 16, 32, 8, 128, 32768, 64, 4
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(33)
+    f = torch.exp(torch.randn(D, generator=gen, device=dev))
+    c = _make(bit_width_inlier=bits, kivi_group_size=g, residual_length=128, fused_sdpa=True,
+              fused_sdpa_memory_bound=True)
+    n_total = ctx + 128 + 37                      # packed prefix of ctx tokens, 165 in the residual
+    for s0 in range(0, n_total, 4096):
+        n = min(4096, n_total - s0)
+        c.update_and_fetch((torch.randn((B, Hkv, n, D), generator=gen, device=dev) * f).half(),
+                           torch.randn((B, Hkv, n, D), generator=gen, device=dev).half())
+    nq, n_tail = c._n_quantized, c.offset - c._n_quantized
+    assert nq == ctx and n_tail == 165
+    q = torch.randn((B, Hq, 1, D), generator=gen, device=dev).half()
+    scale = 1 / math.sqrt(D)
+    kw = dict(k_packed=c._kp, k_scale=c._ks, k_zero=c._kz, v_packed=c._vp, v_scale=c._vs, v_zero=c._vz,
+              n_packed=nq, bits=bits, group_size=g, v_layout="token", k_tail=c._tail_k, v_tail=c._tail_v,
+              n_tail=n_tail, scale=scale, out_dtype=torch.float32)
+    p1, p0 = {}, {}
+    o1 = K.kivi_packed_attend(q, _plan_out=p1, **kw)
+    o0 = K.kivi_packed_attend(q, num_splits=-1, _plan_out=p0, **kw)
+    assert p1["path"] == 1 and p0["path"] == 0
+    err = float((o1 - o0).abs().max())
+    print(f"max |mfma - vector| over 16 sequences = {err:.2e}")
+    assert err < 2e-3
+    # chunks handed out on demand: repeated runs agree to rounding; dealt in a fixed order: bit for bit
+    assert float((c.fused_sdpa(q, scale).float() - o1).abs().max()) < 2e-3   # fp16 output
+    prev = K.attend_fixed_order(True)
+    try:
+        f1, f2 = K.kivi_packed_attend(q, **kw), K.kivi_packed_attend(q, **kw)
+    finally:
+        K.attend_fixed_order(prev)
+    assert torch.equal(f1, f2) and float((f1 - o1).abs().max()) < 2e-3
+
+    b, per = B - 1, 32 // bits
+    kp = c._kp[b:b + 1, :, :nq].cpu().numpy().view(np.uint32)
+    codes_k = ok.unpack_indices(kp, bits, D)
+    vp = c._vp[b:b + 1, :, : nq // per].cpu().numpy().view(np.uint32)
+    codes_v = np.ascontiguousarray(ok.unpack_indices(np.ascontiguousarray(vp.swapaxes(-1, -2)), bits, nq).swapaxes(-1, -2))
+    ks, kz = (t[b:b + 1, :, : nq // g].float().cpu().numpy() for t in (c._ks, c._kz))
+    vs, vz = (np.ascontiguousarray(t[b:b + 1, :, :, :nq].float().cpu().numpy().swapaxes(-1, -2)) for t in (c._vs, c._vz))
+    ref = cref.attend(q[b:b + 1].float().cpu().numpy(), codes_k, ks, kz, codes_v, vs, vz, g, scale,
+                      k_tail=c._tail_k[b:b + 1, :, :n_tail].float().cpu().numpy(),
+                      v_tail=c._tail_v[b:b + 1, :, :n_tail].float().cpu().numpy())
+    err = float(np.max(np.abs(o1[b:b + 1].cpu().numpy() - ref)))
+    print(f"max |mfma - oracle| on the last sequence = {err:.2e}")
+    assert err < 2e-3
+
+
 def test_kivi_quantizer_encode_decode():
     require_gpu()
     rng = np.random.default_rng(0)

@@ -2,10 +2,15 @@
 // plan, workspace sizing and kernel dispatch.
 #include "attend.hpp"
 
+#include <atomic>
+
 namespace vq {
+
+static std::atomic<int> g_fixed_order{0};
 
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
+    p.fixed_order = g_fixed_order.load(std::memory_order_relaxed);
     p.path = (a.num_splits >= 0 && mfma_decode_supported(a)) ? 1 : 0;
     p.tail_equiv = 0;
     p.pq = 1;
@@ -88,6 +93,10 @@ static int validate(const vq_attend_args *a, const char *fn) {
 }  // namespace vq
 
 using namespace vq;
+
+extern "C" int vq_kivi_attend_fixed_order(int enable) {
+    return g_fixed_order.exchange(enable ? 1 : 0, std::memory_order_relaxed);
+}
 
 extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
     if (!a) return 0;

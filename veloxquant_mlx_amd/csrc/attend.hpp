@@ -16,6 +16,9 @@ struct AttendPlan {
     // MFMA path: a block works on the GQA group of one kv head at pq consecutive query
     // positions; tiles = ceil(Sq / pq) such blocks per (batch, kv head)
     int pq, tiles;
+    // MFMA decode path: deal token chunks to the waves round robin instead of on demand, so that
+    // results are identical from run to run
+    int fixed_order;
 };
 
 // One output element from the split partials of its query row: p points at nparts records

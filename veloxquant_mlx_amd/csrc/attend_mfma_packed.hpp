@@ -228,7 +228,7 @@ template <int BITS, typename M, int GV>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, int R, float c, int64_t t_begin,
                                              int n_units, int64_t lane_vis, int64_t full_vis, int lane, int wave,
                                              PackedAcc<GV, sizeof(M) != 2> &acc, const uint4 *s_q, char *ring,
-                                             int *s_next) {
+                                             int *s_next, bool fixed_order) {
     constexpr int PER = 32 / BITS;           // codes per word
     constexpr int KW = MF_D / PER;           // key words per token row
     constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
@@ -534,15 +534,18 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 
     // ---- the waves of a block draw chunks of CHUNK units from a shared counter (a wave that
     // is ahead simply draws more), so no wave waits for a slower one until the block's units are
-    // used up.  Copies run DEPTH - 1 units ahead of the arithmetic: `i_*` is where the copies are,
+    // used up.  Which wave meets which tokens then depends on timing, and with it the last bits
+    // of the result; `fixed_order` deals the chunks round robin instead.  Copies run DEPTH - 1 units ahead of the arithmetic: `i_*` is where the copies are,
     // `c_*` where the arithmetic is.  Chunks being at least DEPTH - 1 units long (but for the
     // block's last), the copies have entered at most two chunks beyond the one being computed:
     // `c_next`, `c_after` queue them (NONE = nothing queued, END = the block has no more).
     constexpr int CH = RG::CHUNK;
     const int n_chunks = (n_units + CH - 1) / CH;
+    int dealt = wave;   // fixed order: wave w takes chunks w, w + PK_WAVES, ...
     auto draw = [&]() VQ_INLINE_LAMBDA {   // the next chunk of the block; the value is used a chunk later
         int id = 0;
-        if (lane == 0) id = __hip_atomic_fetch_add(s_next, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (fixed_order) id = (dealt += PK_WAVES);
+        else if (lane == 0) id = __hip_atomic_fetch_add(s_next, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         return id;
     };
     auto chunk_len = [&](int chunk) VQ_INLINE_LAMBDA { return n_units - chunk * CH < CH ? n_units - chunk * CH : CH; };
@@ -606,7 +609,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 template <int BITS, typename M, int GV>
 __global__ __launch_bounds__(PK_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
-                               float *__restrict__ ws) {
+                               int fixed_order, float *__restrict__ ws) {
     __shared__ uint4 s_q[MF_QIMG];
     // the waves' rings; before and after the units the same bytes are the exchange buffer
     // s_o[PK_WAVES][MF_ROWS][MF_D] of the tail and of the cross-wave merge
@@ -670,7 +673,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int n_units = t_end > t_begin ? (int)((t_end - t_begin) / 32) : 0;
     __syncthreads();   // the query staging and the tail are done with the ring's bytes
     packed_units<BITS, M, GV>(a, bh, RT, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_q, s_ring,
-                              &s_next);
+                              &s_next, fixed_order != 0);
     __syncthreads();   // every wave has read its last slot
 
     // ---- merge the waves: accumulator register r of lane (n, blk) is row 4*blk + r,
@@ -741,7 +744,7 @@ static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, flo
             if (dev >= 0 && dev < 64) allowed[dev] = true;                                                        \
         }                                                                                                         \
         hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, ring_bytes, st, a, p.split_len, \
-                           p.tail_equiv, p.nparts, p.pq, p.tiles, ws);                                            \
+                           p.tail_equiv, p.nparts, p.pq, p.tiles, p.fixed_order, ws);                             \
     } while (0)
     if (a.pack_bits == 4) {
         if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);

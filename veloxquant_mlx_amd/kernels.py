@@ -413,6 +413,12 @@ def _tail_layout(t: torch.Tensor):
     return t, n
 
 
+def attend_fixed_order(enable: bool) -> bool:
+    """Deal the decode kernel's token chunks to its waves in a fixed order (bit-identical results
+    from run to run, a few percent slower) instead of on demand.  Returns the previous setting."""
+    return bool(_lib.load().vq_kivi_attend_fixed_order(1 if enable else 0))
+
+
 def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=None, v_packed=None,
                        v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
                        v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
