@@ -205,6 +205,43 @@ int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts);
  * flash_prefill_attend (veloxquant_mlx/metal/_flash_prefill.py:171-237). */
 int vq_kivi_attend(const vq_attend_args *a);
 
+/* ---- attention over VecInfer indices ----------------------------------------- */
+
+typedef struct vq_lut_attend_args {
+    /* transformed queries (apply_dual_transform_queries already applied) / output:
+     * [B, Hq, Sq, D] contiguous */
+    const void *q;
+    void *out;
+    int32_t q_dtype, out_dtype;
+    int64_t B, Hq, Hkv, Sq, D;
+    /* codebook indices [B, Hkv, cap_tokens, D / sub_dim], VQ_U8, VQ_I32 or VQ_U32; the first
+     * n_tokens tokens are live */
+    const void *k_idx, *v_idx;
+    int32_t idx_dtype;
+    int64_t n_tokens, cap_tokens;
+    /* codebooks [n_centroids, sub_dim] shared by every sub-vector position */
+    const void *k_codebook, *v_codebook;
+    int32_t cb_dtype;
+    int32_t n_centroids, k_sub_dim, v_sub_dim;
+    float scale;
+    int32_t causal;          /* queries align to the end of the tokens */
+    int64_t sliding_window;  /* > 0: a query sees only that many last tokens before its position */
+    int32_t num_splits;      /* 0 = choose */
+    void *workspace;         /* at least vq_vecinfer_attend_workspace(args) bytes */
+    size_t workspace_bytes;
+    void *stream;
+} vq_lut_attend_args;
+
+/* softmax((q~ k~^T) * scale) v^ computed from the indices with a per-query look-up table
+ * (scores) and a per-query histogram over centroids (values); neither k~^ nor v^ is
+ * materialised.  Covers n_centroids <= 256, D / sub_dim <= 32 and
+ * (D / k_sub_dim + D / v_sub_dim) * n_centroids * 4 <= 64 KB; other shapes return
+ * VQ_ERR_UNSUPPORTED.  Replaces metal_fused_sdpa
+ * (veloxquant_mlx/metal/fused_sdpa.py:200-299, fused_sdpa.metal) under
+ * VecInferKVCache.fused_sdpa (veloxquant_mlx/cache/vecinfer_cache.py:670-731). */
+size_t vq_vecinfer_attend_workspace(const vq_lut_attend_args *a);
+int vq_vecinfer_attend(const vq_lut_attend_args *a);
+
 #ifdef __cplusplus
 }
 #endif

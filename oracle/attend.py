@@ -23,12 +23,14 @@ from .kivi import KiviCacheModel, group_dequant
 F32 = np.float32
 
 
-def sdpa(q, k, v, scale: float, causal: bool = False, acc=np.float32) -> np.ndarray:
+def sdpa(q, k, v, scale: float, causal: bool = False, acc=np.float32, sliding_window: int = 0) -> np.ndarray:
     """softmax(q k^T * scale) v with GQA by repeat-interleave.
 
     q ``[B,H_q,S_q,D]``, k/v ``[B,H_kv,S_kv,D]``.  With ``causal`` the queries
     are aligned to the tail of the keys and slot ``j`` is masked when
-    ``j > S_kv - S_q + q_pos``."""
+    ``j > S_kv - S_q + q_pos``; with ``sliding_window > 0`` slot ``j`` is also
+    masked when ``j < q_abs - sliding_window + 1``
+    (veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:105-113)."""
     q = np.asarray(q).astype(acc)
     k = np.asarray(k).astype(acc)
     v = np.asarray(v).astype(acc)
@@ -42,6 +44,10 @@ def sdpa(q, k, v, scale: float, causal: bool = False, acc=np.float32) -> np.ndar
     if causal:
         q_abs = (S_kv - S_q) + np.arange(S_q)
         mask = np.arange(S_kv)[None, :] > q_abs[:, None]
+        scores = np.where(mask, -np.inf, scores)
+    if sliding_window and sliding_window > 0:
+        q_abs = (S_kv - S_q) + np.arange(S_q)
+        mask = np.arange(S_kv)[None, :] < (q_abs[:, None] - sliding_window + 1)
         scores = np.where(mask, -np.inf, scores)
     scores = scores - scores.max(axis=-1, keepdims=True)
     w = np.exp(scores)

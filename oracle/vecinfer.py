@@ -152,3 +152,16 @@ def calibrate_smooth_factors(keys_calib, eps: float = 1e-4) -> np.ndarray:
     if k.ndim not in (2, 3):
         raise ValueError("calibrate_smooth_factors: keys_calib must be 2D or 3D")
     return np.sqrt(np.maximum(np.abs(k).max(axis=0), eps))
+
+
+def fused_sdpa(q_tilde, k_indices, k_codebook, v_indices, v_codebook, scale: float, causal: bool = True,
+               sliding_window: int = 0, acc=np.float64) -> np.ndarray:
+    """``softmax((q_tilde @ K_tilde^T) * scale) @ V_hat`` with both operands gathered from
+    their codebooks: the reference's own oracle for its table kernel
+    (veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:80-115, for
+    veloxquant_mlx/metal/fused_sdpa.py:200-299), queries aligned to the tail."""
+    from .attend import sdpa
+    k_tilde = dequantize_vq(k_indices, k_codebook)
+    v_hat = dequantize_vq(v_indices, v_codebook)
+    return sdpa(np.asarray(q_tilde, np.float32), k_tilde, v_hat, scale, causal=causal, acc=acc,
+                sliding_window=sliding_window)

@@ -333,13 +333,15 @@ def test_vecinfer_fused_modes_and_state_round_trip(memory_bound):
         c2 = KVCacheFactory.create(cfg)
         c2.state = st
         assert c2.offset == 70 and c2._stored_S_kv == 70
-        assert torch.equal(c2.fused_sdpa(to_dev(q), 0.09), out)
+        # the value histogram is summed in LDS in arrival order: equal up to float reassociation
+        assert float((c2.fused_sdpa(to_dev(q), 0.09).float() - out.float()).abs().max()) < 2e-3
     else:
         assert len(st) == 4 and st[0].shape == (2, 2, 70, 128)
     assert c.trim(6) == 6 and c._stored_S_kv == 64 and c.offset == 64
     assert c.compressed_key_bytes == int(16 * 2 * 2 * 70 * (64 / 70))
-    with pytest.raises(ValueError, match="sliding_window"):
-        c.fused_sdpa(to_dev(q), 0.09, sliding_window=16)
+    out_w = c.fused_sdpa(to_dev(q), 0.09, sliding_window=16)
+    ref_w = oa.sdpa(q.astype(np.float32) @ H, k_t_hat[:, :, :64], v_hat[:, :, :64], 0.09, sliding_window=16)
+    assert np.max(np.abs(host(out_w).astype(np.float32) - ref_w)) < 2e-3
 
 
 def test_vecinfer_max_ctx_cap():

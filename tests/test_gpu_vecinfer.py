@@ -144,3 +144,136 @@ def test_mfma_filter_large_magnitudes_and_ragged_count():
         x = (rng.standard_normal((n, 8)) * np.exp(2 * rng.standard_normal(8))).astype(np.float16)
         got = host(K.vecinfer_quantize_metal(to_dev(x), to_dev(cb), 8)).reshape(-1)
         np.testing.assert_array_equal(got, ov.quantize_vq(x, cb, 8).reshape(-1))
+
+
+# ---------------------------------------------------------------------------
+# attention straight from the indices (look-up table + centroid histogram)
+# ---------------------------------------------------------------------------
+
+LUT_TOL = 2e-3   # max-abs against the float64 oracle; the reference's own bar is 1e-2
+                 # (veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:20)
+
+
+def _lut_case(B, Hq, Hkv, Sq, S, D, sub_k, sub_v, C, seed, idx_dtype=np.uint8, cap=None, q_scale=1.0):
+    rng = np.random.default_rng(seed)
+    cap = cap or S
+    q = (rng.standard_normal((B, Hq, Sq, D)) * q_scale).astype(np.float32)
+    kcb = rng.standard_normal((C, sub_k)).astype(np.float32)
+    vcb = rng.standard_normal((C, sub_v)).astype(np.float32)
+    ki = rng.integers(0, C, (B, Hkv, cap, D // sub_k)).astype(idx_dtype)
+    vi = rng.integers(0, C, (B, Hkv, cap, D // sub_v)).astype(idx_dtype)
+    return q, ki, kcb, vi, vcb
+
+
+def _lut_run(q, ki, kcb, vi, vcb, scale, q_dtype=torch.float32, cb_dtype=torch.float32, **kw):
+    return host(K.metal_fused_sdpa(to_dev(q, q_dtype), to_dev(ki), to_dev(kcb, cb_dtype), to_dev(vi),
+                                   to_dev(vcb, cb_dtype), scale, **kw)).astype(np.float32)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,S,D,sub,C", [
+    (1, 4, 4, 1, 128, 64, 4, 256),       # the reference's default case (test_vecinfer_fused_sdpa.py:120-131)
+    (1, 32, 8, 1, 256, 128, 8, 256),     # GQA 32/8 (ibid. 172-184)
+    (1, 4, 4, 8, 128, 64, 4, 256),       # S_q = 8 (ibid. 218-228)
+    (1, 4, 4, 1, 4096, 64, 4, 256),      # long context (ibid. 206-216)
+    (2, 8, 2, 5, 777, 128, 8, 256),      # ragged length, several query rows per kv head
+    (1, 8, 8, 1, 1500, 256, 16, 200),    # D = 256, fewer centroids
+    (1, 2, 1, 3, 300, 96, 8, 17),        # n_sub = 12
+])
+def test_lut_attention_matches_the_gather_oracle(B, Hq, Hkv, Sq, S, D, sub, C, causal):
+    require_gpu()
+    q, ki, kcb, vi, vcb = _lut_case(B, Hq, Hkv, Sq, S, D, sub, sub, C, seed=S + D + Sq)
+    scale = 1.0 / np.sqrt(D)
+    ref = ov.fused_sdpa(q, ki, kcb, vi, vcb, scale, causal=causal)
+    got = _lut_run(q, ki, kcb, vi, vcb, scale, causal=causal)
+    assert got.shape == ref.shape
+    assert np.max(np.abs(got - ref)) < LUT_TOL
+    # 32-bit indices take the word path; same answer
+    got32 = _lut_run(q, ki.astype(np.int32), kcb, vi.astype(np.int32), vcb, scale, causal=causal)
+    assert np.max(np.abs(got32 - ref)) < LUT_TOL
+
+
+@pytest.mark.parametrize("S", [1, 2])
+def test_lut_attention_one_and_two_tokens(S):
+    """veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:186-204"""
+    require_gpu()
+    q, ki, kcb, vi, vcb = _lut_case(1, 4, 4, 1, S, 64, 4, 4, 256, seed=S)
+    ref = ov.fused_sdpa(q, ki, kcb, vi, vcb, 0.125)
+    assert np.max(np.abs(_lut_run(q, ki, kcb, vi, vcb, 0.125) - ref)) < LUT_TOL
+    if S == 1:   # one token: the output is that token's value, whatever the query
+        np.testing.assert_allclose(_lut_run(q, ki, kcb, vi, vcb, 0.125), ov.dequantize_vq(vi, vcb)[:, :, :1], atol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Sq,S,window", [(1, 256, 64), (8, 256, 64), (4, 1300, 100), (3, 40, 64), (2, 600, 1)])
+def test_lut_attention_sliding_window(Sq, S, window, causal):
+    """window mask of veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:105-113, 155-170"""
+    require_gpu()
+    q, ki, kcb, vi, vcb = _lut_case(1, 4, 2, Sq, S, 64, 4, 4, 256, seed=window + Sq)
+    ref = ov.fused_sdpa(q, ki, kcb, vi, vcb, 0.125, causal=causal, sliding_window=window)
+    got = _lut_run(q, ki, kcb, vi, vcb, 0.125, causal=causal, sliding_window=window)
+    assert np.max(np.abs(got - ref)) < LUT_TOL
+    if window == 1 and causal:   # each query sees only its own position
+        vh = ov.dequantize_vq(vi, vcb)
+        np.testing.assert_allclose(got[0, 0], vh[0, 0, S - Sq:], atol=1e-6)
+
+
+def test_lut_attention_mixed_sub_dims_dtypes_and_a_prefix_of_the_buffer():
+    require_gpu()
+    # keys in 8-wide, values in 4-wide sub-vectors; only the first 333 of 512 rows are tokens
+    q, ki, kcb, vi, vcb = _lut_case(2, 8, 4, 2, 333, 128, 8, 4, 64, seed=5, cap=512)
+    scale = 0.1
+    ref = ov.fused_sdpa(q, ki[:, :, :333], kcb, vi[:, :, :333], vcb, scale)
+    assert np.max(np.abs(_lut_run(q, ki, kcb, vi, vcb, scale, n_tokens=333) - ref)) < LUT_TOL
+    # fp16 queries, codebooks and output: compare on the rounded operands
+    q16, kcb16, vcb16 = (x.astype(np.float16).astype(np.float32) for x in (q, kcb, vcb))
+    ref16 = ov.fused_sdpa(q16, ki[:, :, :333], kcb16, vi[:, :, :333], vcb16, scale)
+    got16 = _lut_run(q, ki, kcb, vi, vcb, scale, q_dtype=torch.float16, cb_dtype=torch.float16, n_tokens=333)
+    assert np.max(np.abs(got16 - ref16)) < LUT_TOL
+    gotbf = host(K.metal_fused_sdpa(to_dev(q16), to_dev(ki), to_dev(kcb16), to_dev(vi), to_dev(vcb16), scale,
+                                    n_tokens=333, out_dtype=torch.bfloat16).float())
+    assert np.max(np.abs(gotbf - ref16)) < 2e-2   # bf16 output rounding
+
+
+def test_lut_attention_properties():
+    require_gpu()
+    q, ki, kcb, vi, vcb = _lut_case(1, 8, 2, 4, 2000, 128, 8, 8, 256, seed=9)
+    scale = 1.0 / np.sqrt(128)
+    base = _lut_run(q, ki, kcb, vi, vcb, scale)
+    # the token split must not matter
+    for ns in (1, 2, 3, 4):
+        assert np.max(np.abs(_lut_run(q, ki, kcb, vi, vcb, scale, num_splits=ns) - base)) < 1e-4
+    # causal: the first query position cannot see the last three tokens
+    ki2, vi2 = ki.copy(), vi.copy()
+    ki2[:, :, -3:] += 7      # uint8 wraps inside the 256 centroids
+    vi2[:, :, -3:] += 11
+    pert = _lut_run(q, ki2, kcb, vi2, vcb, scale)
+    assert np.max(np.abs(pert[:, :, 0] - base[:, :, 0])) < 1e-5
+    assert np.max(np.abs(pert[:, :, 3] - base[:, :, 3])) > 1e-4
+    # zero query: uniform weights, so the mean of the decoded values
+    z = _lut_run(np.zeros_like(q[:, :, :1]), ki, kcb, vi, vcb, scale)
+    np.testing.assert_allclose(z[0, 0, 0], ov.dequantize_vq(vi, vcb)[0, 0].mean(0), atol=1e-5)
+    # large logits: a softmax that does not overflow
+    big = _lut_run(q * 40, ki, kcb, vi, vcb, 1.0)
+    ref = ov.fused_sdpa(q * 40, ki, kcb, vi, vcb, 1.0)
+    assert np.isfinite(big).all() and np.max(np.abs(big - ref)) < LUT_TOL
+
+
+def test_lut_attention_errors():
+    """messages of veloxquant_mlx/metal/fused_sdpa.py:229-248 plus this kernel's own limits"""
+    require_gpu()
+    q, ki, kcb, vi, vcb = _lut_case(1, 4, 4, 1, 32, 64, 4, 4, 256, seed=1)
+    t = lambda *xs: [to_dev(x) for x in xs]
+    with pytest.raises(ValueError, match="must equal n_sub"):
+        K.metal_fused_sdpa(*t(q[..., :60], ki, kcb, vi, vcb), 0.1)
+    with pytest.raises(ValueError, match="same n_centroids"):
+        K.metal_fused_sdpa(*t(q, ki, kcb, vi, vcb[:128]), 0.1)
+    with pytest.raises(ValueError, match="multiple of H_kv"):
+        K.metal_fused_sdpa(*t(np.concatenate([q, q[:, :1]], 1), ki, kcb, vi, vcb), 0.1)
+    big = np.random.default_rng(0).standard_normal((512, 4)).astype(np.float32)
+    with pytest.raises(ValueError, match="exceeds 256"):
+        K.metal_fused_sdpa(*t(q, ki.astype(np.int32), big, vi.astype(np.int32), big), 0.1)
+    with pytest.raises(ValueError, match="S_q"):
+        K.metal_fused_sdpa(*t(np.repeat(q, 40, 2), ki, kcb, vi, vcb), 0.1, causal=True)
+    with pytest.raises(RuntimeError, match="ROCm device"):
+        K.metal_fused_sdpa(torch.from_numpy(q), *t(ki, kcb, vi, vcb), 0.1)

@@ -101,3 +101,28 @@ def test_chunked_prefill_sees_quantised_prefix_and_fp16_window():
     # with a residual window longer than the sequence nothing is quantised
     out_fp = attend.chunked_prefill(q, k, v, chunk=32, bits=2, group_size=8, residual_length=512, scale=0.2)
     np.testing.assert_allclose(out_fp, attend.sdpa(q, k, v, 0.2, causal=True, acc=np.float64), atol=1e-6)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("window", [1, 5, 64])
+def test_sliding_window_and_index_attention_match_library_sdpa(causal, window):
+    """The window keeps slots q_abs-window+1 .. (veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:105-113);
+    the index form is plain attention over the gathered centroids (ibid. 80-115)."""
+    from oracle import vecinfer
+    rng = np.random.default_rng(window)
+    B, Hq, Hkv, Sq, Skv, D, sub, C = 1, 4, 2, 6, 33, 16, 4, 32
+    q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float32)
+    kcb = rng.standard_normal((C, sub)).astype(np.float32)
+    vcb = rng.standard_normal((C, sub)).astype(np.float32)
+    ki = rng.integers(0, C, (B, Hkv, Skv, D // sub))
+    vi = rng.integers(0, C, (B, Hkv, Skv, D // sub))
+    out = vecinfer.fused_sdpa(q, ki, kcb, vi, vcb, 0.3, causal=causal, sliding_window=window)
+    k = torch.from_numpy(kcb)[torch.from_numpy(ki)].reshape(B, Hkv, Skv, D).repeat_interleave(Hq // Hkv, 1)
+    v = torch.from_numpy(vcb)[torch.from_numpy(vi)].reshape(B, Hkv, Skv, D).repeat_interleave(Hq // Hkv, 1)
+    mask = torch.zeros(Sq, Skv, dtype=torch.bool)
+    for i in range(Sq):
+        qa = Skv - Sq + i
+        for j in range(Skv):
+            mask[i, j] = (j <= qa or not causal) and j >= qa - window + 1
+    ref = torch.nn.functional.scaled_dot_product_attention(torch.from_numpy(q), k, v, attn_mask=mask, scale=0.3)
+    np.testing.assert_allclose(out, ref.numpy(), atol=2e-5)

@@ -39,6 +39,21 @@ class AttendArgs(C.Structure):
     ]
 
 
+class LutAttendArgs(C.Structure):
+    """Mirror of ``vq_lut_attend_args``."""
+
+    _fields_ = [
+        ("q", vp), ("out", vp), ("q_dtype", i32), ("out_dtype", i32),
+        ("B", i64), ("Hq", i64), ("Hkv", i64), ("Sq", i64), ("D", i64),
+        ("k_idx", vp), ("v_idx", vp), ("idx_dtype", i32),
+        ("n_tokens", i64), ("cap_tokens", i64),
+        ("k_codebook", vp), ("v_codebook", vp), ("cb_dtype", i32),
+        ("n_centroids", i32), ("k_sub_dim", i32), ("v_sub_dim", i32),
+        ("scale", f32), ("causal", i32), ("sliding_window", i64), ("num_splits", i32),
+        ("workspace", vp), ("workspace_bytes", sz), ("stream", vp),
+    ]
+
+
 _SIGNATURES = {
     "vq_abi_version": (i32, []),
     "vq_last_error": (i32, [C.c_char_p, sz]),
@@ -57,6 +72,8 @@ _SIGNATURES = {
     "vq_kivi_attend_workspace": (sz, [C.POINTER(AttendArgs)]),
     "vq_kivi_attend_plan": (i32, [C.POINTER(AttendArgs), C.POINTER(i32), C.POINTER(i32)]),
     "vq_kivi_attend": (i32, [C.POINTER(AttendArgs)]),
+    "vq_vecinfer_attend_workspace": (sz, [C.POINTER(LutAttendArgs)]),
+    "vq_vecinfer_attend": (i32, [C.POINTER(LutAttendArgs)]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)

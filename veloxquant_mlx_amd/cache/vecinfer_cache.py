@@ -345,13 +345,24 @@ class VecInferKVCache(FP16KVCache):
                                "KVCacheConfig.fused_sdpa=True.")
         if self._stored_k_indices is None or self._stored_S_kv == 0:
             raise RuntimeError("VecInferKVCache.fused_sdpa called before any tokens were cached via update_and_fetch.")
-        if sliding_window:
-            raise ValueError("VecInferKVCache.fused_sdpa: sliding_window attention is not supported")
         self._to_device(q)
         n = self._stored_S_kv
         smooth = self._smooth.float() if self._smooth is not None else torch.ones(
             (self._head_dim,), dtype=torch.float32, device=q.device)
         q_tilde = apply_dual_transform_queries(q.float(), smooth, self._H)
+        kcb, vcb = self._key_codebook, self._value_codebook
+        n_sub_k, n_sub_v = self._head_dim // kcb.shape[1], self._head_dim // vcb.shape[1]
+        table_kernel = (kcb.shape[0] == vcb.shape[0] <= 256 and max(n_sub_k, n_sub_v) <= 32
+                        and (n_sub_k + n_sub_v) * kcb.shape[0] * 4 <= 65536
+                        and (self._stored_k_indices.dtype != torch.uint8 or (n_sub_k % 4 == 0 and n_sub_v % 4 == 0)))
+        if table_kernel:
+            # look-up table + centroid histogram straight from the indices
+            return K.metal_fused_sdpa(q_tilde, self._stored_k_indices, kcb, self._stored_v_indices, vcb, float(scale),
+                                      causal=bool(causal) and q.shape[2] > 1, sliding_window=int(sliding_window or 0),
+                                      out_dtype=q.dtype, n_tokens=n)
+        if sliding_window:
+            raise ValueError("VecInferKVCache.fused_sdpa: sliding_window attention needs the table kernel "
+                             "(n_centroids <= 256, at most 32 sub-vectors per head)")
         k_tilde_hat = K.vecinfer_dequant_metal(self._stored_k_indices[:, :, :n].contiguous(), self._key_codebook,
                                                out_dtype=torch.float32)
         v_hat = K.vecinfer_dequant_metal(self._stored_v_indices[:, :, :n].contiguous(), self._value_codebook,

@@ -127,6 +127,12 @@ int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len
     return VQ_OK;
 }
 
+void launch_merge_rows(const float *ws, int64_t rows, int nparts, int64_t D, void *out, int out_dtype, hipStream_t st) {
+    int64_t g = cdiv(rows * D, 256);
+    if (g > (1 << 20)) g = 1 << 20;
+    hipLaunchKernelGGL(attend_merge_kernel, dim3((unsigned)g), dim3(256), 0, st, ws, rows, nparts, D, out, out_dtype);
+}
+
 int launch_attend_merge(const vq_attend_args &a, int nparts) {
     hipStream_t st = (hipStream_t)a.stream;
     const int64_t rows = a.B * a.Hq * a.Sq;

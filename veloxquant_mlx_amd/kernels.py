@@ -16,7 +16,7 @@ import torch
 
 from . import _lib
 from ._lib import (VQ_AXIS_CHANNEL, VQ_AXIS_TOKEN, VQ_BF16, VQ_F16, VQ_F32, VQ_I32, VQ_U8,
-                   VQ_V_CHANNEL_PACKED, VQ_V_TOKEN_PACKED, AttendArgs)
+                   VQ_V_CHANNEL_PACKED, VQ_V_TOKEN_PACKED, AttendArgs, LutAttendArgs)
 
 _FLOAT_TAG = {torch.float16: VQ_F16, torch.bfloat16: VQ_BF16, torch.float32: VQ_F32}
 _V_LAYOUT = {"channel": VQ_V_CHANNEL_PACKED, "token": VQ_V_TOKEN_PACKED}
@@ -632,3 +632,81 @@ __all__ = [
     "kivi_packed_attend", "scalar_fused_decode_attend", "scalar_fused_decode_attend_batched",
     "scalar_predecoded_attend", "flash_prefill_attend",
 ]
+
+
+# ---------------------------------------------------------------------------
+# attention over VecInfer indices
+# ---------------------------------------------------------------------------
+
+def metal_fused_sdpa(q_tilde: torch.Tensor, k_indices: torch.Tensor, k_codebook: torch.Tensor,
+                     v_indices: torch.Tensor, v_codebook: torch.Tensor, scale: float, *, causal: bool = True,
+                     sliding_window: int = 0, out_dtype: torch.dtype | None = None,
+                     n_tokens: int | None = None, num_splits: int = 0) -> torch.Tensor:
+    """``softmax((q_tilde @ K_tilde^T) * scale) @ V_hat`` from codebook indices, without
+    materialising ``K_tilde`` or ``V_hat``.  Same contract as ``metal_fused_sdpa``
+    (veloxquant_mlx/metal/fused_sdpa.py:200-299): ``q_tilde [B,H_q,S_q,D]`` already passed through
+    ``apply_dual_transform_queries``; ``k_indices, v_indices [B,H_kv,S_kv,n_sub]`` (uint8 or
+    32-bit); codebooks ``[n_centroids, sub_dim]``; queries align to the tail of ``S_kv``;
+    ``sliding_window > 0`` keeps only that many last keys before each query position.
+    ``n_tokens`` (this build) attends over the first ``n_tokens`` rows of longer index buffers."""
+    name = "fused_sdpa"
+    if q_tilde.ndim != 4 or k_indices.ndim != 4 or v_indices.ndim != 4:
+        raise ValueError(f"{name}: q_tilde and the index tensors must be 4D")
+    if k_codebook.ndim != 2 or v_codebook.ndim != 2:
+        raise ValueError(f"{name}: codebooks must be 2D [n_centroids, sub_dim]")
+    _need_gpu(name, q_tilde, k_indices, v_indices, k_codebook, v_codebook)
+    B, H_q, S_q, D = q_tilde.shape
+    _, H_kv, cap, n_sub = k_indices.shape
+    n_centroids, sub_dim = k_codebook.shape
+    n_sub_v = v_indices.shape[3]
+    n_centroids_v, sub_dim_v = v_codebook.shape
+    if n_sub * sub_dim != D:
+        raise ValueError(f"{name}: D={D} must equal n_sub*sub_dim={n_sub * sub_dim}.")
+    if n_sub_v * sub_dim_v != D:
+        raise ValueError(f"{name}: D={D} must equal n_sub_v*sub_dim_v={n_sub_v * sub_dim_v}.")
+    if n_centroids != n_centroids_v:
+        raise ValueError(f"{name}: key and value codebooks must currently have the same n_centroids "
+                         f"(got {n_centroids} vs {n_centroids_v}).")
+    if H_q % H_kv != 0:
+        raise ValueError(f"{name}: H_q={H_q} must be a multiple of H_kv={H_kv}.")
+    if v_indices.shape[:3] != k_indices.shape[:3] or k_indices.shape[0] != B:
+        raise ValueError(f"{name}: key and value indices must share [B,H_kv,S_kv]")
+    S_kv = cap if n_tokens is None else int(n_tokens)
+    if not 1 <= S_kv <= cap:
+        raise ValueError(f"{name}: n_tokens={S_kv} outside 1..{cap}")
+    if out_dtype is None:
+        out_dtype = q_tilde.dtype
+    if q_tilde.dtype not in _FLOAT_TAG:
+        q_tilde = q_tilde.float()
+    if out_dtype not in _FLOAT_TAG:
+        raise ValueError(f"{name}: unsupported out dtype {out_dtype}")
+
+    def idx(t):
+        if t.dtype not in (torch.uint8, torch.int32):
+            t = t.to(torch.int32)
+        return t.contiguous()
+    ki, vi = idx(k_indices), idx(v_indices)
+    if ki.dtype != vi.dtype:
+        ki, vi = ki.to(torch.int32), vi.to(torch.int32)
+    cb_dtype = k_codebook.dtype if k_codebook.dtype in _FLOAT_TAG and k_codebook.dtype == v_codebook.dtype else torch.float32
+    kcb, vcb = k_codebook.to(cb_dtype).contiguous(), v_codebook.to(cb_dtype).contiguous()
+    q = q_tilde.contiguous()
+    out = torch.empty((B, H_q, S_q, D), dtype=out_dtype, device=q.device)
+    a = LutAttendArgs(q=q.data_ptr(), out=out.data_ptr(), q_dtype=_FLOAT_TAG[q.dtype], out_dtype=_FLOAT_TAG[out_dtype],
+                      B=B, Hq=H_q, Hkv=H_kv, Sq=S_q, D=D, k_idx=ki.data_ptr(), v_idx=vi.data_ptr(),
+                      idx_dtype=VQ_U8 if ki.dtype == torch.uint8 else VQ_I32, n_tokens=S_kv, cap_tokens=cap,
+                      k_codebook=kcb.data_ptr(), v_codebook=vcb.data_ptr(), cb_dtype=_FLOAT_TAG[cb_dtype],
+                      n_centroids=n_centroids, k_sub_dim=sub_dim, v_sub_dim=sub_dim_v, scale=float(scale),
+                      causal=1 if causal else 0, sliding_window=int(sliding_window or 0), num_splits=int(num_splits))
+    lib = _lib.load()
+    need = lib.vq_vecinfer_attend_workspace(C.byref(a))
+    if need == 0:
+        _lib.check(lib.vq_vecinfer_attend(C.byref(a)))   # raises with the validation message
+    ws = _workspace(q.device, need)
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.stream = _stream(q)
+    _lib.check(lib.vq_vecinfer_attend(C.byref(a)))
+    return out
+
+
+vecinfer_fused_sdpa = metal_fused_sdpa
