@@ -277,3 +277,28 @@ def test_lut_attention_errors():
         K.metal_fused_sdpa(*t(np.repeat(q, 40, 2), ki, kcb, vi, vcb), 0.1, causal=True)
     with pytest.raises(RuntimeError, match="ROCm device"):
         K.metal_fused_sdpa(torch.from_numpy(q), *t(ki, kcb, vi, vcb), 0.1)
+
+
+def test_lut_attention_many_weights_below_one_unit_still_count():
+    """One dominant token and thousands whose weights are each below the resolution of the
+    integer histogram (2^-18 of the largest weight in blocks of 8192 tokens): their total is a
+    few percent of the sum and must not be rounded away."""
+    require_gpu()
+    rng = np.random.default_rng(3)
+    B, H, S, D, sub, C = 16, 8, 8192, 64, 4, 256
+    kcb = (rng.standard_normal((C, sub)) * 0.05).astype(np.float32)
+    kcb[7] = [3.0, -3.0, 3.0, -3.0]
+    vcb = rng.standard_normal((C, sub)).astype(np.float32)
+    ki = rng.integers(8, C, (B, H, S, D // sub)).astype(np.uint8)
+    vi = rng.integers(0, C, (B, H, S, D // sub)).astype(np.uint8)
+    ki[:, :, 100] = 7
+    q = np.tile(kcb[7], D // sub)[None, None, None, :].repeat(B, 0).repeat(H, 1).astype(np.float32)
+    # the dominant score is 16 * 36 * scale, the others are near zero: a gap of about 13.5 nats
+    scale = 13.5 / (16 * 36)
+    ref = ov.fused_sdpa(q, ki, kcb, vi, vcb, scale)
+    w_small = np.exp(-13.5) * (S - 1)
+    assert 0.005 < w_small < 0.05 and np.exp(-13.5) * 2 ** 18 < 0.5
+    got = _lut_run(q, ki, kcb, vi, vcb, scale)
+    dom = ov.dequantize_vq(vi, vcb)[:, :, 100:101]
+    assert np.max(np.abs(ref - dom)) > 5e-3          # the small weights matter at the tolerance below
+    assert np.max(np.abs(got - ref)) < 2e-4

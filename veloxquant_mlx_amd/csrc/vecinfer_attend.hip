@@ -10,13 +10,16 @@
 // tables live in LDS, and LDS traffic, not HBM, bounds the kernel.
 //
 // The histogram is an integer one.  A weight is exp2(score - reference) <= 1 with the reference
-// at or above every score the block has seen, and it is added as round(weight * 2^20) with an
-// integer LDS atomic: on this chip a random-address ds_add_u32 costs what a ds_read_b32 does,
-// a ds_add_f32 about 27 times that.  A block takes at most 2048 tokens, so a cell cannot exceed
-// 2^31; the sum of the weights is read back from the histogram itself, which makes the output
-// an exact convex combination of centroids, and integer addition makes it independent of the
-// order in which the waves arrive.  When a later tile of tokens raises the reference the
-// histogram is rescaled in place.
+// at or above every score the block has seen, and it is added in units of 2^-F with an integer
+// LDS atomic: on this chip a random-address ds_add_u32 costs what a ds_read_b32 does, a
+// ds_add_f32 about 27 times that.  F is 20 for blocks of up to 2048 tokens, 19 up to 4096 and
+// 18 up to 8192, so a cell cannot exceed 2^31.  The weight is rounded down after adding a
+// per-token offset in [0, 1) from a low-discrepancy sequence (token number times the golden
+// ratio), so that many weights below one unit still add up to their true total.  The sum of
+// the weights is read back from the histogram itself, which makes the output an exact convex
+// combination of centroids, and integer addition makes it independent of the order in which
+// the waves arrive.  When a later tile of tokens raises the reference the histogram is rescaled
+// in place.
 //
 // One block of four waves per (kv head, tile of RB query rows, token split); a lane is a token.
 // Every block writes one (max, sum, accumulator) partial per row; the merge kernel of the
@@ -29,11 +32,10 @@
 namespace vq {
 
 constexpr int LA_THREADS = 256, LA_WAVES = 4;
-constexpr int LA_TILES = 2;                           // 64-token tiles a wave holds scores of between the two phases
+constexpr int LA_TILES = 4;                           // 64-token tiles a wave holds scores of between the two phases
 constexpr int LA_SUPER = LA_WAVES * LA_TILES * 64;    // tokens a block takes per step
-constexpr int LA_FBITS = 20;                          // weights are integers in units of 2^-20
-constexpr int LA_MAX_SPLIT = 2048;                    // tokens per block: 2048 * 2^20 = 2^31 fits a cell
-constexpr float LA_UNIT = (float)(1 << LA_FBITS), LA_INV_UNIT = 1.0f / (float)(1 << LA_FBITS);
+constexpr int LA_MAX_SPLIT = 8192;                    // tokens per block
+constexpr float LA_GOLDEN = 0.6180339887498949f;
 constexpr float LA_HEADROOM = 1.0f;                   // a raised reference goes this far (log2) above the new maximum
 constexpr float LA_LOG2E = 1.4426950408889634f, LA_LN2 = 0.6931471805599453f;
 constexpr int LA_MAX_SUB = 32;                        // sub-vectors per head
@@ -46,6 +48,7 @@ struct LutPlan {
     int tiles;     // row tiles per (batch, kv head)
     int nsplit;    // token splits
     int64_t split_len;   // tokens per split, a multiple of LA_SUPER, at most LA_MAX_SPLIT
+    int fbits;     // weights are integers in units of 2^-fbits: split_len * 2^fbits <= 2^31
     size_t lds;    // bytes of dynamic LDS
 };
 
@@ -81,6 +84,7 @@ static LutPlan plan_lut(const vq_lut_attend_args &a) {
     if (ns < min_splits) ns = min_splits;
     p.split_len = cdiv(cdiv(n, ns), LA_SUPER) * LA_SUPER;
     p.nsplit = (int)cdiv(n, p.split_len);
+    p.fbits = p.split_len <= 2048 ? 20 : p.split_len <= 4096 ? 19 : 18;
     return p;
 }
 
@@ -104,10 +108,19 @@ struct RowGeom {
     }
 };
 
+// maximum over the wave, in every lane: four cross-lane moves inside the rows of 16, then one
+// lane of each row
+template <int CTRL> __device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off));
-    return v;
+    v = fmaxf(v, dpp_move<0xB1>(v));    // quad_perm [1,0,3,2]
+    v = fmaxf(v, dpp_move<0x4E>(v));    // quad_perm [2,3,0,1]
+    v = fmaxf(v, dpp_move<0x124>(v));   // row_ror 4
+    v = fmaxf(v, dpp_move<0x128>(v));   // row_ror 8
+    const int b = __builtin_bit_cast(int, v);
+    return fmaxf(fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16))),
+                 fmaxf(__builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48))));
 }
 
 // After the waves have published their tiles' maxima: raise the references that a maximum
@@ -140,8 +153,12 @@ __device__ __forceinline__ void raise_references(const float (*s_max)[4], float 
     }
 }
 
-__device__ __forceinline__ uint32_t weight_units(float s, float m) {
-    return s == -INFINITY ? 0u : __float2uint_rn(__builtin_amdgcn_exp2f(s - m) * LA_UNIT);
+// weight exp2(s - m) <= 1 in units of 1 / unit, rounded down after the token's offset
+__device__ __forceinline__ uint32_t weight_units(float s, float m, float unit, float dither) {
+    return s == -INFINITY ? 0u : __float2uint_rd(__builtin_amdgcn_exp2f(s - m) * unit + dither);
+}
+__device__ __forceinline__ float token_dither(int64_t t) {
+    return __builtin_amdgcn_fractf((float)((uint32_t)t & 0xffffu) * LA_GOLDEN);
 }
 
 __device__ __forceinline__ void lds_add(uint32_t *p, uint32_t v) {
@@ -183,7 +200,7 @@ template <int NW> struct ByteIdx {   // a token's NS = 4 * NW indices
 // histogram [RB][NS][256] integers (first the staged query rows).
 template <int RB, int NS>
 __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend_args a, int tiles, int64_t split_len, int nparts,
-                                                                   int tab_rows, float *__restrict__ ws) {
+                                                                   int tab_rows, int fbits, float *__restrict__ ws) {
     extern __shared__ __align__(16) float s_tab[];
     __shared__ float s_max[LA_WAVES][4], s_ref[4];
     __shared__ uint32_t s_sum[4];
@@ -191,6 +208,7 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int C = a.n_centroids, SUB = a.k_sub_dim, D = (int)a.D;
+    const float unit = (float)(1u << fbits), inv_unit = 1.0f / unit;
     float *lut = s_tab;
     uint32_t *hist = reinterpret_cast<uint32_t *>(s_tab + tab_rows * LA_ROW);
 
@@ -252,30 +270,42 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
 #pragma unroll
     for (int r = 0; r < RB; ++r) m_row[r] = -INFINITY;
 
+    // the indices of a step are loaded one step ahead
+    ByteIdx<NW> kn[LA_TILES], vn[LA_TILES];
+    auto fetch = [&](int64_t base) {
+#pragma unroll
+        for (int T = 0; T < LA_TILES; ++T) {
+            const int64_t t = base + (wave * LA_TILES + T) * 64 + lane;
+            kn[T].load(kib + t * NS, t < t_end);
+            vn[T].load(vib + t * NS, t < t_end);
+        }
+    };
+    fetch(t_begin);
     for (int64_t base = t_begin; base < t_end; base += LA_SUPER) {
         // ---- phase 1: scores of the wave's tiles, and their maxima per row
         float s[LA_TILES][RB], wmax[RB];
-        ByteIdx<NW> vi[LA_TILES];
+        ByteIdx<NW> ki[LA_TILES], vi[LA_TILES];
+#pragma unroll
+        for (int T = 0; T < LA_TILES; ++T) { ki[T] = kn[T]; vi[T] = vn[T]; }
+        fetch(base + LA_SUPER);
 #pragma unroll
         for (int r = 0; r < RB; ++r) wmax[r] = -INFINITY;
 #pragma unroll
         for (int T = 0; T < LA_TILES; ++T) {
             const int64_t t = base + (wave * LA_TILES + T) * 64 + lane;
             const bool valid = t < t_end;
-            ByteIdx<NW> ki;
-            ki.load(kib + t * NS, valid);
-            vi[T].load(vib + t * NS, valid);
 #pragma unroll
             for (int r = 0; r < RB; ++r) s[T][r] = 0.f;
 #pragma unroll
             for (int j = 0; j < NS; ++j) {
-                const float *e = lut + (j * LA_ROW + ki.get(j)) * RB;
+                const float *e = lut + (j * LA_ROW + ki[T].get(j)) * RB;
                 if constexpr (RB == 4) { const float4 x = *reinterpret_cast<const float4 *>(e); s[T][0] += x.x; s[T][1] += x.y; s[T][2] += x.z; s[T][3] += x.w; }
                 else if constexpr (RB == 2) { const float2 x = *reinterpret_cast<const float2 *>(e); s[T][0] += x.x; s[T][1] += x.y; }
                 else s[T][0] += *e;
             }
 #pragma unroll
             for (int r = 0; r < RB; ++r) {
+                asm volatile("" : "+v"(s[T][r]));   // the look-ups stay whole reads, outside the masks' branches
                 if (!(valid && t < vis_hi[r] && t >= vis_lo[r])) s[T][r] = -INFINITY;
                 wmax[r] = fmaxf(wmax[r], s[T][r]);
             }
@@ -291,9 +321,10 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
         // ---- phase 2: weights into the histogram
 #pragma unroll
         for (int T = 0; T < LA_TILES; ++T) {
+            const float dither = token_dither(base + (wave * LA_TILES + T) * 64 + lane);
             uint32_t w[RB], any = 0;
 #pragma unroll
-            for (int r = 0; r < RB; ++r) { w[r] = weight_units(s[T][r], m_row[r]); any |= w[r]; }
+            for (int r = 0; r < RB; ++r) { w[r] = weight_units(s[T][r], m_row[r], unit, dither); any |= w[r]; }
             if (__any(any != 0)) {
 #pragma unroll
                 for (int j = 0; j < NS; ++j) {
@@ -337,10 +368,10 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
             acc += (float)hh.x * vv.x + (float)hh.y * vv.y + (float)hh.z * vv.z + (float)hh.w * vv.w;
         }
         float *o = ws + (g.qrow(a, r) * nparts + blockIdx.x) * (a.D + 2);
-        o[2 + d] = acc * LA_INV_UNIT;
+        o[2 + d] = acc * inv_unit;
         if (d == 0) {
             o[0] = s_ref[r] == -INFINITY ? -INFINITY : s_ref[r] * LA_LN2;
-            o[1] = (float)s_sum[r] * LA_INV_UNIT;
+            o[1] = (float)s_sum[r] * inv_unit;
         }
     }
 }
@@ -351,13 +382,14 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
 // memory where they are used; a stray index is held to the last centroid.
 template <int RB>
 __global__ __launch_bounds__(LA_THREADS) void lut_attend_any_kernel(vq_lut_attend_args a, int tiles, int64_t split_len, int nparts,
-                                                                    float *__restrict__ ws) {
+                                                                    int fbits, float *__restrict__ ws) {
     extern __shared__ __align__(16) float s_tab[];
     __shared__ float s_max[LA_WAVES][4], s_ref[4];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int C = a.n_centroids, D = (int)a.D;
     const int nsk = D / a.k_sub_dim, nsv = D / a.v_sub_dim;
+    const float unit = (float)(1u << fbits), inv_unit = 1.0f / unit;
     float *lut = s_tab;
     uint32_t *hist = reinterpret_cast<uint32_t *>(s_tab + RB * nsk * C);
 
@@ -435,9 +467,10 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_any_kernel(vq_lut_atten
 #pragma unroll
         for (int T = 0; T < LA_TILES; ++T) {
             const int64_t t = base + (wave * LA_TILES + T) * 64 + lane;
+            const float dither = token_dither(t);
             uint32_t w[RB], any = 0;
 #pragma unroll
-            for (int r = 0; r < RB; ++r) { w[r] = weight_units(s[T][r], m_row[r]); any |= w[r]; }
+            for (int r = 0; r < RB; ++r) { w[r] = weight_units(s[T][r], m_row[r], unit, dither); any |= w[r]; }
             if (any != 0) {
                 for (int j = 0; j < nsv; ++j) {
                     uint32_t c = ld_idx(vib, a.idx_dtype, t * nsv + j);
@@ -462,12 +495,12 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_any_kernel(vq_lut_atten
         float acc = 0.f;
         for (int c = 0; c < C; ++c) acc += (float)h[c] * ld_any(a.v_codebook, a.cb_dtype, (int64_t)c * a.v_sub_dim + i);
         float *o = ws + (g.qrow(a, r) * nparts + blockIdx.x) * (a.D + 2);
-        o[2 + d] = acc * LA_INV_UNIT;
+        o[2 + d] = acc * inv_unit;
         if (d == 0) {
             uint32_t sum = 0;   // the weights of sub-vector 0 add up to the sum over the tokens
             for (int c = 0; c < C; ++c) sum += hist[r * nsv * C + c];
             o[0] = s_ref[r] == -INFINITY ? -INFINITY : s_ref[r] * LA_LN2;
-            o[1] = (float)sum * LA_INV_UNIT;
+            o[1] = (float)sum * inv_unit;
         }
     }
 }
@@ -539,16 +572,16 @@ extern "C" int vq_vecinfer_attend(const vq_lut_attend_args *a) {
     if (p.bytes) {
         const int ns = (int)(a->D / a->k_sub_dim);
         const int tab_rows = p.rb * ns > a->k_sub_dim ? p.rb * ns : a->k_sub_dim;
-#define VQ_LUT_U8(RB, NS) VQ_LUT_LAUNCH((lut_attend_u8_kernel<RB, NS>), tab_rows, ws)
+#define VQ_LUT_U8(RB, NS) VQ_LUT_LAUNCH((lut_attend_u8_kernel<RB, NS>), tab_rows, p.fbits, ws)
         if (ns == 4) { if (p.rb == 4) VQ_LUT_U8(4, 4); else if (p.rb == 2) VQ_LUT_U8(2, 4); else VQ_LUT_U8(1, 4); }
         else if (ns == 8) { if (p.rb == 4) VQ_LUT_U8(4, 8); else if (p.rb == 2) VQ_LUT_U8(2, 8); else VQ_LUT_U8(1, 8); }
         else if (ns == 16) { if (p.rb == 2) VQ_LUT_U8(2, 16); else VQ_LUT_U8(1, 16); }
         else VQ_LUT_U8(1, 32);
 #undef VQ_LUT_U8
     } else {
-        if (p.rb == 4) VQ_LUT_LAUNCH((lut_attend_any_kernel<4>), ws);
-        else if (p.rb == 2) VQ_LUT_LAUNCH((lut_attend_any_kernel<2>), ws);
-        else VQ_LUT_LAUNCH((lut_attend_any_kernel<1>), ws);
+        if (p.rb == 4) VQ_LUT_LAUNCH((lut_attend_any_kernel<4>), p.fbits, ws);
+        else if (p.rb == 2) VQ_LUT_LAUNCH((lut_attend_any_kernel<2>), p.fbits, ws);
+        else VQ_LUT_LAUNCH((lut_attend_any_kernel<1>), p.fbits, ws);
     }
 #undef VQ_LUT_LAUNCH
     VQ_HIP_CHECK_LAUNCH(fn);
