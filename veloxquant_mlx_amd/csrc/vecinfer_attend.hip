@@ -44,6 +44,7 @@ constexpr size_t LA_MAX_LDS = 96 * 1024;
 
 struct LutPlan {
     bool bytes;    // lut_attend_u8_kernel
+    bool vt_apart; // lut_attend_u8_kernel: the transposed value codebook has LDS of its own
     int rb;        // query rows per block (1, 2 or 4)
     int tiles;     // row tiles per (batch, kv head)
     int nsplit;    // token splits
@@ -57,7 +58,8 @@ static LutPlan plan_lut(const vq_lut_attend_args &a) {
     const int64_t nsk = a.D / a.k_sub_dim, nsv = a.D / a.v_sub_dim;
     const int64_t rows = (a.Hq / a.Hkv) * a.Sq;
     p.bytes = a.idx_dtype == VQ_U8 && nsk == nsv && (nsk == 4 || nsk == 8 || nsk == 16 || nsk == 32) &&
-              a.k_sub_dim % 4 == 0 && a.k_sub_dim <= 256 && a.n_centroids <= LA_ROW;
+              a.k_sub_dim % 4 == 0 && a.k_sub_dim <= 256 && a.n_centroids <= LA_ROW &&
+              (((uintptr_t)a.q | (uintptr_t)a.k_codebook | (uintptr_t)a.v_codebook) & 15u) == 0;
     int rb;
     if (p.bytes) {
         rb = (int)(32 / nsk);   // table and histogram of a block: 2 * rb * nsk KB <= 64 KB, two blocks a CU
@@ -70,9 +72,11 @@ static LutPlan plan_lut(const vq_lut_attend_args &a) {
     while (rb > 1 && rb / 2 >= rows) rb /= 2;
     p.rb = rb;
     p.tiles = (int)cdiv(rows, rb);
+    p.vt_apart = false;
     if (p.bytes) {
-        const int64_t tab = rb * nsk > a.k_sub_dim ? rb * nsk : a.k_sub_dim;   // the table's rows later hold the transposed value codebook
-        p.lds = (size_t)(tab + rb * nsk) * LA_ROW * 4;
+        p.vt_apart = 2 * rb * nsk + a.k_sub_dim <= 78;   // 1 KB rows; two blocks of 78 fit the 160 KB of a CU
+        const int64_t tab = p.vt_apart || rb * nsk > a.k_sub_dim ? rb * nsk : a.k_sub_dim;
+        p.lds = (size_t)(tab + rb * nsk + (p.vt_apart ? a.k_sub_dim : 0)) * LA_ROW * 4;
     } else {
         p.lds = (size_t)(rb * (nsk + nsv) * a.n_centroids * 4);
     }
@@ -165,6 +169,18 @@ __device__ __forceinline__ void lds_add(uint32_t *p, uint32_t v) {
     (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
 
+// four consecutive elements from index i (a multiple of four) of a buffer whose base is 16-byte aligned
+__device__ __forceinline__ float4 ld4_any(const void *p, int tag, int64_t i) {
+    if (tag == VQ_F32) return *reinterpret_cast<const float4 *>((const float *)p + i);
+    const uint2 raw = *reinterpret_cast<const uint2 *>((const u16 *)p + i);
+    if (tag == VQ_F16) {
+        const f16x2 lo = __builtin_bit_cast(f16x2, raw.x), hi = __builtin_bit_cast(f16x2, raw.y);
+        return make_float4((float)lo[0], (float)lo[1], (float)hi[0], (float)hi[1]);
+    }
+    return make_float4(__builtin_bit_cast(float, raw.x << 16), __builtin_bit_cast(float, raw.x & 0xffff0000u),
+                       __builtin_bit_cast(float, raw.y << 16), __builtin_bit_cast(float, raw.y & 0xffff0000u));
+}
+
 // a block none of whose rows sees a token of its split: empty partials
 template <int RB>
 __device__ __forceinline__ void write_empty(const vq_lut_attend_args &a, const RowGeom &g, int nparts, float *ws, int tid) {
@@ -200,7 +216,7 @@ template <int NW> struct ByteIdx {   // a token's NS = 4 * NW indices
 // histogram [RB][NS][256] integers (first the staged query rows).
 template <int RB, int NS>
 __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend_args a, int tiles, int64_t split_len, int nparts,
-                                                                   int tab_rows, int fbits, float *__restrict__ ws) {
+                                                                   int vt_apart, int fbits, float *__restrict__ ws) {
     extern __shared__ __align__(16) float s_tab[];
     __shared__ float s_max[LA_WAVES][4], s_ref[4];
     __shared__ uint32_t s_sum[4];
@@ -210,7 +226,11 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
     const int C = a.n_centroids, SUB = a.k_sub_dim, D = (int)a.D;
     const float unit = (float)(1u << fbits), inv_unit = 1.0f / unit;
     float *lut = s_tab;
+    // the transposed value codebook has rows of its own behind the histogram when two blocks
+    // still fit a CU that way (vt_apart); otherwise it overwrites the table at the end
+    const int tab_rows = vt_apart || RB * NS > SUB ? RB * NS : SUB;
     uint32_t *hist = reinterpret_cast<uint32_t *>(s_tab + tab_rows * LA_ROW);
+    float *vt = vt_apart ? s_tab + (tab_rows + RB * NS) * LA_ROW : lut;
 
     RowGeom g;
     const int64_t bh = blockIdx.y / tiles;
@@ -232,9 +252,33 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
     }
     if (t_begin >= t_end) { write_empty<RB>(a, g, nparts, ws, tid); return; }
 
-    // ---- query rows into LDS, then the table: thread c holds centroid c
+    // ---- everything the block reads before its token loop is requested first: the first
+    // step's indices, the query rows, the codebook rows of thread c = centroid c
+    const uint8_t *kib = (const uint8_t *)a.k_idx + bh * a.cap_tokens * NS;
+    const uint8_t *vib = (const uint8_t *)a.v_idx + bh * a.cap_tokens * NS;
+    ByteIdx<NW> kn[LA_TILES], vn[LA_TILES];
+    auto fetch = [&](int64_t base) {
+#pragma unroll
+        for (int T = 0; T < LA_TILES; ++T) {
+            const int64_t t = base + (wave * LA_TILES + T) * 64 + lane;
+            kn[T].load(kib + t * NS, t < t_end);
+            vn[T].load(vib + t * NS, t < t_end);
+        }
+    };
+    fetch(t_begin);
     float *sq = reinterpret_cast<float *>(hist);
-    for (int e = tid; e < RB * D; e += LA_THREADS) sq[e] = ld_any(a.q, a.q_dtype, g.qrow(a, e / D) * a.D + e % D);
+    for (int e = tid; e < RB * D / 4; e += LA_THREADS) {
+        const int r = 4 * e / D, d = 4 * e % D;
+        *reinterpret_cast<float4 *>(sq + 4 * e) = ld4_any(a.q, a.q_dtype, g.qrow(a, r) * a.D + d);
+    }
+    if (vt_apart) {
+        for (int i0 = 0; i0 < SUB; i0 += 4) {
+            const float4 v = tid < C ? ld4_any(a.v_codebook, a.cb_dtype, (int64_t)tid * SUB + i0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            vt[(i0 + 0) * LA_ROW + tid] = v.x; vt[(i0 + 1) * LA_ROW + tid] = v.y;
+            vt[(i0 + 2) * LA_ROW + tid] = v.z; vt[(i0 + 3) * LA_ROW + tid] = v.w;
+        }
+    }
+    float4 kc_next = tid < C ? ld4_any(a.k_codebook, a.cb_dtype, (int64_t)tid * SUB) : make_float4(0.f, 0.f, 0.f, 0.f);
     __syncthreads();
     {
         const float c2 = a.scale * LA_LOG2E;   // scores are kept in log2 units
@@ -244,15 +288,14 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
 #pragma unroll
             for (int j = 0; j < NS; ++j) acc[r][j] = 0.f;
         for (int i0 = 0; i0 < SUB; i0 += 4) {
-            float kc[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) kc[e] = tid < C ? ld_any(a.k_codebook, a.cb_dtype, (int64_t)tid * SUB + i0 + e) : 0.f;
+            const float4 kc = kc_next;
+            if (i0 + 4 < SUB && tid < C) kc_next = ld4_any(a.k_codebook, a.cb_dtype, (int64_t)tid * SUB + i0 + 4);
 #pragma unroll
             for (int r = 0; r < RB; ++r)
 #pragma unroll
                 for (int j = 0; j < NS; ++j) {
                     const float4 qv = *reinterpret_cast<const float4 *>(sq + r * D + j * SUB + i0);
-                    acc[r][j] += qv.x * kc[0] + qv.y * kc[1] + qv.z * kc[2] + qv.w * kc[3];
+                    acc[r][j] += qv.x * kc.x + qv.y * kc.y + qv.z * kc.z + qv.w * kc.w;
                 }
         }
 #pragma unroll
@@ -264,23 +307,11 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
     for (int e = tid; e < RB * NS * LA_ROW / 4; e += LA_THREADS) reinterpret_cast<uint4 *>(hist)[e] = make_uint4(0, 0, 0, 0);
     __syncthreads();
 
-    const uint8_t *kib = (const uint8_t *)a.k_idx + bh * a.cap_tokens * NS;
-    const uint8_t *vib = (const uint8_t *)a.v_idx + bh * a.cap_tokens * NS;
     float m_row[RB];   // the block's softmax reference per row, log2 units
 #pragma unroll
     for (int r = 0; r < RB; ++r) m_row[r] = -INFINITY;
 
     // the indices of a step are loaded one step ahead
-    ByteIdx<NW> kn[LA_TILES], vn[LA_TILES];
-    auto fetch = [&](int64_t base) {
-#pragma unroll
-        for (int T = 0; T < LA_TILES; ++T) {
-            const int64_t t = base + (wave * LA_TILES + T) * 64 + lane;
-            kn[T].load(kib + t * NS, t < t_end);
-            vn[T].load(vib + t * NS, t < t_end);
-        }
-    };
-    fetch(t_begin);
     for (int64_t base = t_begin; base < t_end; base += LA_SUPER) {
         // ---- phase 1: scores of the wave's tiles, and their maxima per row
         float s[LA_TILES][RB], wmax[RB];
@@ -338,9 +369,9 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
     __syncthreads();   // every weight has landed; the table is dead
 
     // ---- value codebook transposed over the table, the sums of the weights from sub-vector 0
-    float *vt = lut;
-    for (int e = tid; e < SUB * LA_ROW; e += LA_THREADS)   // e % 256 == tid
-        vt[e] = tid < C ? ld_any(a.v_codebook, a.cb_dtype, (int64_t)tid * SUB + e / LA_ROW) : 0.f;
+    if (!vt_apart)
+        for (int e = tid; e < SUB * LA_ROW; e += LA_THREADS)   // e % 256 == tid
+            vt[e] = tid < C ? ld_any(a.v_codebook, a.cb_dtype, (int64_t)tid * SUB + e / LA_ROW) : 0.f;
     if (wave < RB) {
         const uint4 h = reinterpret_cast<const uint4 *>(hist + wave * NS * LA_ROW)[lane];
         uint32_t t = h.x + h.y + h.z + h.w;
@@ -571,8 +602,7 @@ extern "C" int vq_vecinfer_attend(const vq_lut_attend_args *a) {
     float *ws = (float *)a->workspace;
     if (p.bytes) {
         const int ns = (int)(a->D / a->k_sub_dim);
-        const int tab_rows = p.rb * ns > a->k_sub_dim ? p.rb * ns : a->k_sub_dim;
-#define VQ_LUT_U8(RB, NS) VQ_LUT_LAUNCH((lut_attend_u8_kernel<RB, NS>), tab_rows, p.fbits, ws)
+#define VQ_LUT_U8(RB, NS) VQ_LUT_LAUNCH((lut_attend_u8_kernel<RB, NS>), (int)p.vt_apart, p.fbits, ws)
         if (ns == 4) { if (p.rb == 4) VQ_LUT_U8(4, 4); else if (p.rb == 2) VQ_LUT_U8(2, 4); else VQ_LUT_U8(1, 4); }
         else if (ns == 8) { if (p.rb == 4) VQ_LUT_U8(4, 8); else if (p.rb == 2) VQ_LUT_U8(2, 8); else VQ_LUT_U8(1, 8); }
         else if (ns == 16) { if (p.rb == 2) VQ_LUT_U8(2, 16); else VQ_LUT_U8(1, 16); }
