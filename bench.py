@@ -265,6 +265,21 @@ def _extras(torch, K, dev):
     flops = 2 * 524288 * 256 * 8
     ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
                             "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
+    # attention straight from VecInfer indices: 32768 tokens, 8 kv heads x 4 query heads, D 128 in 16
+    # sub-vectors of 256 centroids (uint8 indices, 32 B per token and kv head); LDS-bound by design
+    for B in (1, 16):
+        ki = torch.randint(0, 256, (B, Hkv, 32768, 16), device=dev).to(torch.uint8)
+        vi = torch.randint(0, 256, (B, Hkv, 32768, 16), device=dev).to(torch.uint8)
+        kcb, vcb = cb, torch.randn((256, 8), device=dev).to(torch.float16)
+        q = torch.randn((B, Hq, 1, D), device=dev).to(torch.float16)
+        fn = lambda: K.metal_fused_sdpa(q, ki, kcb, vi, vcb, 1 / math.sqrt(D))
+        for _ in range(3):
+            fn()
+        ms = _event_ms(fn, 30, torch)
+        nbytes = 2 * ki.numel()
+        lds_ops = B * Hq * 32768 * 16 * 2 / 64    # one look-up and one histogram addition per row, token and sub-vector, 64 lanes an instruction
+        ex[f"index_attend_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1), "bytes": nbytes,
+                                        "lds_cycles_per_wave_op_per_cu": round(ms * 1e-3 * 2.1e9 * 256 / lds_ops, 2)}
     return ex
 
 

@@ -10,8 +10,9 @@ Parity pinning status (which external facts each function is checked against
 lives in tests/test_oracle_*.py):
 
 * group quantisation, packing, dequantisation, decode attention, causal
-  prefill attention, cache frontier arithmetic: pinned (hand-computed known
-  answers, closed forms, invariants, brute force, library SDPA).
+  prefill attention, attention from codebook indices with its sliding-window
+  mask, cache frontier arithmetic: pinned (hand-computed known answers,
+  closed forms, invariants, brute force, library SDPA).
 * ``quantize_vq`` on exact fp32 near-ties: PARITY UNPINNED against MLX's
   ``mx.sum`` reduction order and ``mx.argmin`` tie order (MLX is not
   installable here).  The oracle fixes the order the reference's Metal twin
