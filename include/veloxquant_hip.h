@@ -133,6 +133,23 @@ int vq_bit_unpack(const uint8_t *packed, int64_t n, int bits, uint8_t *idx, void
 int vq_vecinfer_assign(const void *x, int x_dtype, int64_t N, const void *codebook, int cb_dtype,
                        int n_centroids, int sub_dim, void *idx, int idx_dtype, void *stream);
 
+/* Fused key encode (+ optional decode) in one launch: keys [B, H, S, D] (any float dtype,
+ * contiguous) -> k~ = (keys / smooth) @ Hd with Hd the orthonormal Sylvester-Hadamard matrix
+ * of size D (entries +-hadamard_scale, natural order; done as a fast Walsh-Hadamard
+ * transform) -> idx [B, H, S, D / sub_dim] by the rule of vq_vecinfer_assign.  smooth is
+ * float32 [smooth_rows, D] with smooth_rows 1 or H, or NULL.  k_hat, when not NULL, receives
+ * the reconstruction (codebook[idx] @ Hd^T) * smooth in the dtype of keys; k_tilde, when not
+ * NULL, receives k~ as float32.  Covers sub_dim 4 or 8, D / sub_dim in {8, 16, 32, 64},
+ * n_centroids <= 256, 16-byte aligned buffers; VQ_ERR_UNSUPPORTED otherwise (callers then
+ * transform with a matrix product and call vq_vecinfer_assign).  Replaces
+ * vecinfer_encode_decode_metal (veloxquant_mlx/metal/_vecinfer.py:225-293,
+ * metal/src/vecinfer_encode_decode_full.metal) and the encode half of
+ * VecInferKVCache._encode_decode_keys (cache/vecinfer_cache.py:313-356). */
+int vq_vecinfer_encode_keys(const void *keys, int k_dtype, int64_t B, int64_t H, int64_t S, int64_t D,
+                            const float *smooth, int smooth_rows, float hadamard_scale, const void *codebook,
+                            int cb_dtype, int n_centroids, int sub_dim, void *idx, int idx_dtype, void *k_hat,
+                            float *k_tilde, void *stream);
+
 /* Centroid gather, out [N, sub_dim] = codebook[min(idx, n_centroids-1)].
  * Replaces dequantize_vq (allocators/vecinfer.py:321-335) and
  * vecinfer_dequant_metal (metal/_vecinfer.py:144-178). */

@@ -154,6 +154,28 @@ def calibrate_smooth_factors(keys_calib, eps: float = 1e-4) -> np.ndarray:
     return np.sqrt(np.maximum(np.abs(k).max(axis=0), eps))
 
 
+def encode_decode_keys(keys, smooth, H, codebook, sub_dim: int):
+    """Key encode+decode of the fused kernel (metal/_vecinfer.py:225-293; the cache's
+    composition, cache/vecinfer_cache.py:313-356): ``k_tilde = (K / smooth) @ H`` -> indices ->
+    ``k_hat = (codebook[idx] @ H^T) * smooth``.  The two matrix products are accumulated in
+    float64 and rounded to float32 once, i.e. the mathematical value rather than one particular
+    summation order.  ``smooth``: ``None``, ``[D]`` or ``[H_kv, D]``.  Returns
+    ``(k_tilde, idx, k_hat)``, all float32 / int32."""
+    K = np.asarray(keys).astype(F32)
+    Hm = np.asarray(H).astype(np.float64)
+    sm = None
+    if smooth is not None:
+        sm = np.asarray(smooth).astype(F32)
+        sm = sm[:, None, :] if sm.ndim == 2 and sm.shape[0] == K.shape[-3] else (sm.mean(axis=0) if sm.ndim == 2 else sm)
+    x = K / sm if sm is not None else K
+    k_tilde = (x.astype(np.float64) @ Hm).astype(F32)
+    idx = quantize_vq(k_tilde, codebook, sub_dim)
+    k_hat = (dequantize_vq(idx, np.asarray(codebook).astype(F32)).astype(np.float64) @ Hm.T).astype(F32)
+    if sm is not None:
+        k_hat = k_hat * sm
+    return k_tilde, idx, k_hat.astype(F32)
+
+
 def fused_sdpa(q_tilde, k_indices, k_codebook, v_indices, v_codebook, scale: float, causal: bool = True,
                sliding_window: int = 0, acc=np.float64) -> np.ndarray:
     """``softmax((q_tilde @ K_tilde^T) * scale) @ V_hat`` with both operands gathered from

@@ -302,3 +302,98 @@ def test_lut_attention_many_weights_below_one_unit_still_count():
     dom = ov.dequantize_vq(vi, vcb)[:, :, 100:101]
     assert np.max(np.abs(ref - dom)) > 5e-3          # the small weights matter at the tolerance below
     assert np.max(np.abs(got - ref)) < 2e-4
+
+
+# ---------------------------------------------------------------------------
+# fused key encode (+ decode): smooth, Walsh-Hadamard transform, assignment, way back
+# ---------------------------------------------------------------------------
+
+def _gap_to_second(k_tilde, cb, sub):
+    """relative gap between the two smallest squared distances of every sub-vector"""
+    x = k_tilde.reshape(-1, sub).astype(np.float64)
+    d = ((x[:, None, :] - cb[None].astype(np.float64)) ** 2).sum(-1)
+    d.sort(axis=1)
+    return ((d[:, 1] - d[:, 0]) / np.maximum(d[:, 1], 1e-30)).reshape(k_tilde.shape[:-1] + (-1,))
+
+
+@pytest.mark.parametrize("D,sub", [(64, 8), (128, 8), (256, 8), (512, 8), (32, 4), (64, 4), (128, 4), (256, 4)])
+def test_encode_keys_on_integer_keys_is_exact(D, sub):
+    """Integer keys and power-of-two smoothing factors: every partial sum of the transform is
+    exact in float32 whatever its order, so the transformed keys, hence the indices, must equal
+    the oracle's bit for bit."""
+    require_gpu()
+    rng = np.random.default_rng(D + sub)
+    B, Hh, S, C = 2, 3, 21, 200
+    keys = rng.integers(-8, 9, (B, Hh, S, D)).astype(np.float16)
+    smooth = (2.0 ** rng.integers(-2, 3, (Hh, D))).astype(np.float32)
+    Hm = ov.walsh_hadamard_matrix(D)
+    cb = rng.standard_normal((C, sub)).astype(np.float32)
+    kt_ref, idx_ref, khat_ref = ov.encode_decode_keys(keys, smooth, Hm, cb, sub)
+    k_hat, idx, k_tilde = K.vecinfer_encode_decode_metal(to_dev(keys), to_dev(cb), sub, to_dev(Hm), to_dev(smooth),
+                                                          want_k_tilde=True)
+    np.testing.assert_array_equal(host(k_tilde), kt_ref)
+    np.testing.assert_array_equal(host(idx), idx_ref)
+    assert k_hat.dtype == torch.float16 and k_hat.shape == keys.shape
+    np.testing.assert_allclose(host(k_hat).astype(np.float32), khat_ref, rtol=1.5e-3, atol=1e-3)
+    # indices only, one byte each
+    none, idx8 = K.vecinfer_encode_decode_metal(to_dev(keys), to_dev(cb), sub, to_dev(Hm), to_dev(smooth),
+                                                index_dtype=torch.uint8, want_k_hat=False)
+    assert none is None
+    np.testing.assert_array_equal(host(idx8), idx_ref.astype(np.uint8))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("smooth_rows", [None, 1, "heads", "vector"])
+def test_encode_keys_random_keys(dtype, smooth_rows):
+    require_gpu()
+    rng = np.random.default_rng(11)
+    B, Hh, S, D, sub, C = 2, 4, 333, 128, 8, 256
+    keys_t = to_dev((rng.standard_normal((B, Hh, S, D)) * np.exp(rng.standard_normal(D))).astype(np.float32), dtype)
+    keys = host(keys_t).astype(np.float32)
+    smooth = {None: None, 1: np.exp(rng.standard_normal((1, D)) * 0.5), "heads": np.exp(rng.standard_normal((Hh, D)) * 0.5),
+              "vector": np.exp(rng.standard_normal(D) * 0.5)}[smooth_rows]
+    smooth = None if smooth is None else smooth.astype(np.float32)
+    Hm = ov.walsh_hadamard_matrix(D)
+    cb = rng.standard_normal((C, sub)).astype(np.float32)
+    kt_ref, idx_ref, _ = ov.encode_decode_keys(keys, smooth, Hm, cb, sub)
+    k_hat, idx, k_tilde = K.vecinfer_encode_decode_metal(keys_t, to_dev(cb), sub, to_dev(Hm),
+                                                          None if smooth is None else to_dev(smooth), want_k_tilde=True)
+    kt, idx = host(k_tilde), host(idx)
+    # the transform: float32 butterflies against the float64 product
+    assert np.max(np.abs(kt - kt_ref)) <= 2e-6 * np.max(np.abs(kt_ref))
+    # the assignment is exact on the kernel's own transformed keys
+    np.testing.assert_array_equal(idx, ov.quantize_vq(kt, cb, sub))
+    # against the oracle's transformed keys only near ties may differ
+    diff = idx != idx_ref
+    assert diff.mean() < 1e-3
+    if diff.any():
+        assert _gap_to_second(kt_ref, cb, sub)[diff].max() < 1e-4
+    # the way back, from the kernel's own indices
+    sm = 1.0 if smooth is None else (smooth[:, None, :] if smooth.ndim == 2 and smooth.shape[0] == Hh else smooth.reshape(-1, D)[0])
+    back = (ov.dequantize_vq(idx, cb).astype(np.float64) @ Hm.T.astype(np.float64)) * sm
+    tol = {torch.float16: 1.5e-3, torch.bfloat16: 1e-2, torch.float32: 1e-5}[dtype]
+    assert k_hat.dtype == dtype
+    np.testing.assert_allclose(host(k_hat).astype(np.float64), back, rtol=tol, atol=tol)
+
+
+def test_encode_keys_other_shapes_take_the_composition():
+    """sub_dim 16, a non-Hadamard matrix, more than 256 centroids: same contract through the
+    matrix product and the assignment / gather kernels."""
+    require_gpu()
+    rng = np.random.default_rng(2)
+    keys = rng.standard_normal((1, 2, 40, 64)).astype(np.float16)
+    Hm = ov.walsh_hadamard_matrix(64)
+    for sub, C, Hmat in ((16, 64, Hm), (8, 300, Hm), (8, 64, np.linalg.qr(rng.standard_normal((64, 64)))[0].astype(np.float32))):
+        cb = rng.standard_normal((C, sub)).astype(np.float32)
+        k_hat, idx, k_tilde = K.vecinfer_encode_decode_metal(to_dev(keys), to_dev(cb), sub, to_dev(Hmat), want_k_tilde=True)
+        np.testing.assert_array_equal(host(idx), ov.quantize_vq(host(k_tilde), cb, sub))
+        np.testing.assert_allclose(host(k_tilde), keys.astype(np.float32) @ Hmat, rtol=1e-4, atol=1e-4)
+        back = ov.dequantize_vq(host(idx), cb) @ Hmat.T
+        np.testing.assert_allclose(host(k_hat).astype(np.float32), back, rtol=2e-3, atol=2e-3)
+    v_hat, v_idx = K.vecinfer_encode_decode_simple_metal(to_dev(keys), to_dev(cb), 8)
+    np.testing.assert_array_equal(host(v_idx), ov.quantize_vq(keys, cb, 8))
+    np.testing.assert_allclose(host(v_hat).astype(np.float32), ov.dequantize_vq(host(v_idx), cb), rtol=1e-3, atol=1e-3)
+    with pytest.raises(ValueError, match="must be 4D"):
+        K.vecinfer_encode_decode_metal(to_dev(keys[0]), to_dev(cb), 8, to_dev(Hm))
+    with pytest.raises(ValueError, match="not divisible"):
+        K.vecinfer_encode_decode_metal(to_dev(keys), to_dev(cb), 7, to_dev(Hm))

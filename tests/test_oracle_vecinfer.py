@@ -111,3 +111,31 @@ def test_calibrate_smooth_factors():
     k = np.array([[1.0, -4.0], [0.25, 9.0]], np.float32)
     np.testing.assert_allclose(vi.calibrate_smooth_factors(k), [1.0, 3.0])
     np.testing.assert_allclose(vi.calibrate_smooth_factors(np.zeros((3, 2), np.float32)), [0.01, 0.01], rtol=1e-6)
+
+
+def test_encode_decode_keys_is_the_composition_and_inverts_on_centroid_points():
+    """encode_decode_keys = transform, assignment, gather, inverse transform
+    (veloxquant_mlx/cache/vecinfer_cache.py:313-356).  Pins: the Hadamard entries follow
+    (-1)^popcount(a & b); keys built as (c @ H^T) * smooth from centroids come back as those
+    centroids' indices with k_hat == keys; the transform agrees with a plain float32 loop."""
+    rng = np.random.default_rng(0)
+    D, sub, C = 32, 4, 16
+    H = vi.walsh_hadamard_matrix(D)
+    a = np.arange(D)
+    par = np.array([[bin(x & y).count("1") & 1 for y in a] for x in a])
+    np.testing.assert_array_equal(np.sign(H), 1 - 2 * par)
+    assert len(set(np.abs(H).reshape(-1).tolist())) == 1
+    cb = rng.standard_normal((C, sub)).astype(np.float32) * 3
+    want = rng.integers(0, C, (1, 2, 5, D // sub))
+    smooth = np.exp(rng.standard_normal((2, D))).astype(np.float32)
+    keys = (vi.dequantize_vq(want, cb).astype(np.float64) @ H.T.astype(np.float64)) * smooth[:, None, :]
+    k_tilde, idx, k_hat = vi.encode_decode_keys(keys.astype(np.float32), smooth, H, cb, sub)
+    np.testing.assert_array_equal(idx, want)
+    np.testing.assert_allclose(k_hat, keys, rtol=2e-6, atol=2e-6)
+    loop = np.zeros_like(k_tilde)
+    x = keys.astype(np.float32) / smooth[:, None, :]
+    for b in range(D):
+        for aa in range(D):
+            loop[..., b] += x[..., aa] * H[aa, b]
+    np.testing.assert_allclose(k_tilde, loop, rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(k_tilde, vi.apply_dual_transform_keys(keys.astype(np.float32), smooth, H), rtol=1e-5, atol=1e-5)

@@ -68,6 +68,7 @@ _SIGNATURES = {
     "vq_bit_unpack": (i32, [vp, i64, i32, vp, vp]),
     "vq_vecinfer_assign": (i32, [vp, i32, i64, vp, i32, i32, i32, vp, i32, vp]),
     "vq_vecinfer_dequant": (i32, [vp, i32, i64, vp, i32, i32, i32, vp, i32, vp]),
+    "vq_vecinfer_encode_keys": (i32, [vp, i32, i64, i64, i64, i64, vp, i32, f32, vp, i32, i32, i32, vp, i32, vp, vp, vp]),
     "vq_kivi_attend_fixed_order": (i32, [i32]),
     "vq_kivi_attend_workspace": (sz, [C.POINTER(AttendArgs)]),
     "vq_kivi_attend_plan": (i32, [C.POINTER(AttendArgs), C.POINTER(i32), C.POINTER(i32)]),

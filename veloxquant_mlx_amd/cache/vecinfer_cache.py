@@ -157,7 +157,11 @@ class VecInferKVCache(FP16KVCache):
         return k32 @ self._H
 
     def _encode_decode_keys(self, keys: torch.Tensor):
-        """smooth -> WHT -> VQ -> gather -> inverse WHT -> un-smooth (vecinfer_cache.py:313-356)."""
+        """smooth -> WHT -> VQ -> gather -> inverse WHT -> un-smooth (vecinfer_cache.py:313-356):
+        one launch for 4D keys, the composition below otherwise."""
+        if keys.ndim == 4:
+            return K.vecinfer_encode_decode_metal(keys, self._key_codebook, self._key_sub_dim, self._H, self._smooth,
+                                                  index_dtype=self._k_idx_dtype)
         k_tilde = self._transform_keys(keys)
         k_idx = K.vecinfer_quantize_metal(k_tilde, self._key_codebook, self._key_sub_dim,
                                           index_dtype=self._k_idx_dtype)
@@ -238,8 +242,8 @@ class VecInferKVCache(FP16KVCache):
     def _update_and_fetch_fused(self, keys, values):
         """Indices only; returns zero-stride placeholders (vecinfer_cache.py:491-532)."""
         B, H, S, D = keys.shape
-        k_idx = K.vecinfer_quantize_metal(self._transform_keys(keys), self._key_codebook, self._key_sub_dim,
-                                          index_dtype=self._k_idx_dtype)
+        _, k_idx = K.vecinfer_encode_decode_metal(keys, self._key_codebook, self._key_sub_dim, self._H, self._smooth,
+                                                  index_dtype=self._k_idx_dtype, want_k_hat=False)
         v_idx = K.vecinfer_quantize_metal(values, self._value_codebook, self._value_sub_dim,
                                           index_dtype=self._v_idx_dtype)
         self._stash(k_idx, v_idx)

@@ -137,6 +137,32 @@ extern "C" int vq_vecinfer_assign(const void *x, int x_dtype, int64_t N, const v
     return VQ_OK;
 }
 
+extern "C" int vq_vecinfer_encode_keys(const void *keys, int k_dtype, int64_t B, int64_t H, int64_t S, int64_t D,
+                                       const float *smooth, int smooth_rows, float hadamard_scale, const void *codebook,
+                                       int cb_dtype, int n_centroids, int sub_dim, void *idx, int idx_dtype, void *k_hat,
+                                       float *k_tilde, void *stream) {
+    const char *fn = "vq_vecinfer_encode_keys";
+    VQ_REQUIRE(is_float_tag(k_dtype) && is_float_tag(cb_dtype), VQ_ERR_INVALID, "%s: unsupported float dtype", fn);
+    VQ_REQUIRE(idx_dtype == VQ_I32 || idx_dtype == VQ_U32 || idx_dtype == VQ_U8, VQ_ERR_INVALID,
+               "%s: idx dtype must be int32, uint32 or uint8", fn);
+    VQ_REQUIRE(B >= 0 && H >= 1 && S >= 0 && D >= 1, VQ_ERR_INVALID, "%s: keys must be 4D [B, H, S, D]", fn);
+    VQ_REQUIRE(n_centroids >= 1 && sub_dim >= 1 && D % sub_dim == 0, VQ_ERR_INVALID,
+               "%s: D=%lld not divisible by sub_dim=%d", fn, (long long)D, sub_dim);
+    VQ_REQUIRE((D & (D - 1)) == 0, VQ_ERR_INVALID, "%s: D=%lld must be a power of 2 (Walsh-Hadamard transform)", fn, (long long)D);
+    VQ_REQUIRE(idx_dtype != VQ_U8 || n_centroids <= 256, VQ_ERR_INVALID, "%s: uint8 indices need n_centroids <= 256, got %d", fn,
+               n_centroids);
+    VQ_REQUIRE(smooth == nullptr || smooth_rows == 1 || smooth_rows == H, VQ_ERR_INVALID,
+               "%s: smooth must have 1 or H=%lld rows, got %d", fn, (long long)H, smooth_rows);
+    if (B * S == 0) return VQ_OK;
+    VQ_REQUIRE(keys && codebook && idx, VQ_ERR_INVALID, "%s: null pointer", fn);
+    VQ_REQUIRE(launch_encode_keys_mfma(keys, k_dtype, B, H, S, D, smooth, smooth_rows, hadamard_scale, codebook, cb_dtype,
+                                       n_centroids, sub_dim, idx, idx_dtype, k_hat, k_tilde, (hipStream_t)stream),
+               VQ_ERR_UNSUPPORTED,
+               "%s: needs sub_dim 4 or 8, D / sub_dim in {8, 16, 32, 64}, n_centroids <= 256 and 16-byte aligned buffers", fn);
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
 extern "C" int vq_vecinfer_dequant(const void *idx, int idx_dtype, int64_t N, const void *codebook, int cb_dtype,
                                    int n_centroids, int sub_dim, void *out, int out_dtype, void *stream) {
     const char *fn = "vq_vecinfer_dequant";

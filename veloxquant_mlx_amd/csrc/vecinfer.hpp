@@ -30,4 +30,12 @@ __device__ __forceinline__ uint32_t ld_idx(const void *p, int tag, int64_t i) {
 bool launch_assign_mfma(const void *x, int xt, int64_t N, const void *cb, int ct, int nc, int sub, void *idx, int it,
                         hipStream_t st);
 
+// Fused key encode (and optional decode) around the MFMA assignment: keys [B, heads, S, D] ->
+// (keys / smooth) @ H -> indices [B * heads * S, D / sub], optionally k_hat (dtype of keys) and
+// k_tilde (float32).  Returns false, launching nothing, for shapes it does not cover
+// (sub_dim 4 or 8, D / sub_dim in {8, 16, 32, 64}, at most 256 centroids, 16-byte aligned buffers).
+bool launch_encode_keys_mfma(const void *keys, int kt, int64_t B, int64_t heads, int64_t S, int64_t D, const float *smooth,
+                             int smooth_rows, float h, const void *cb, int ct, int nc, int sub, void *idx, int it, void *k_hat,
+                             float *k_tilde, hipStream_t st);
+
 }  // namespace vq

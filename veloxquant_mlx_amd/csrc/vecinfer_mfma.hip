@@ -67,10 +67,70 @@ __device__ __forceinline__ void merge_top2(float &a1, float &a2, int &ia1, int &
     ia2 = c2 ? sia : sib;
 }
 
-template <int SUB>
+// ---- the key transform in front of the assignment, and the reconstruction behind it --------
+//
+// With LT > 0 the sub-vectors are not taken as they are: 64 consecutive sub-vectors are 64 / LT
+// whole tokens of D = LT * SUB channels (lane j of a group of LT lanes holds channels
+// [SUB j, SUB (j + 1))), and each token first goes through  k~ = (k / smooth) @ H  with H the
+// orthonormal Sylvester-Hadamard matrix (entries +-h in natural order), done as a fast
+// Walsh-Hadamard transform across the LT lanes: in-lane butterflies over the SUB registers, then
+// one butterfly per lane bit (cross-lane moves inside the row of 16, LDS permutes beyond it), then
+// the scale h.  Optionally the chosen centroids go back the same way, k^ = (c @ H^T) * smooth
+// (H is symmetric), and k~ itself can be written out.  This is the reference's fused key
+// encode+decode (veloxquant_mlx/metal/_vecinfer.py:225-293) as a front and back end of the
+// MFMA assignment.
+struct KeyXform {
+    const float *smooth;   // [smooth_rows, D] float32 or null
+    int smooth_rows;       // 1 or the number of heads
+    int64_t heads, S;      // keys are [B, heads, S, D]
+    float h;               // |H[0][0]|
+    void *k_hat;           // [N * SUB] reconstruction in dtype hat_dtype, or null
+    int hat_dtype;
+    float *k_tilde;        // [N * SUB] transformed keys, or null
+};
+
+template <int CTRL> __device__ __forceinline__ float xform_dpp(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, x), __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+// value of lane (lane ^ M)
+template <int M> __device__ __forceinline__ float lane_xor(float x) {
+    if constexpr (M == 1) return xform_dpp<0xB1>(x);        // quad_perm [1,0,3,2]
+    else if constexpr (M == 2) return xform_dpp<0x4E>(x);   // quad_perm [2,3,0,1]
+    else if constexpr (M == 8) return xform_dpp<0x128>(x);  // row_ror 8
+    else return __shfl_xor(x, M);
+}
+template <int SUB, int M> __device__ __forceinline__ void lane_butterfly(float (&x)[8], int lane) {
+    const bool upper = (lane & M) != 0;
+#pragma unroll
+    for (int e = 0; e < SUB; ++e) {
+        const float p = lane_xor<M>(x[e]);
+        x[e] = upper ? p - x[e] : x[e] + p;
+    }
+}
+// unnormalised Walsh-Hadamard transform of the LT * SUB values a group of LT lanes holds
+template <int SUB, int LT> __device__ __forceinline__ void wht_lanes(float (&x)[8], int lane) {
+#pragma unroll
+    for (int hlf = 1; hlf < SUB; hlf <<= 1)
+#pragma unroll
+        for (int i = 0; i < SUB; i += 2 * hlf)
+#pragma unroll
+            for (int k = i; k < i + hlf; ++k) {
+                const float a = x[k], b = x[k + hlf];
+                x[k] = a + b;
+                x[k + hlf] = a - b;
+            }
+    if constexpr (LT > 1) lane_butterfly<SUB, 1>(x, lane);
+    if constexpr (LT > 2) lane_butterfly<SUB, 2>(x, lane);
+    if constexpr (LT > 4) lane_butterfly<SUB, 4>(x, lane);
+    if constexpr (LT > 8) lane_butterfly<SUB, 8>(x, lane);
+    if constexpr (LT > 16) lane_butterfly<SUB, 16>(x, lane);
+    if constexpr (LT > 32) lane_butterfly<SUB, 32>(x, lane);
+}
+
+template <int SUB, int LT>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void vq_assign_mfma_kernel(const void *__restrict__ x, int xt, int64_t N,
                                                              const void *__restrict__ cb, int ct, int nc,
-                                                             void *__restrict__ idx, int it) {
+                                                             void *__restrict__ idx, int it, KeyXform kx) {
     __shared__ float s_cb[VM_MAXC * 8];          // codebook as float32, row stride SUB
     __shared__ float s_c2[VM_MAXC];              // |c|^2, huge past the end
     __shared__ uint4 s_A[VM_TILES][64];          // MFMA A operands of every centroid tile
@@ -159,6 +219,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
         } else {
 #pragma unroll
             for (int e = 0; e < 8; ++e) xf[e] = (e < SUB && sv < N) ? ld_any(x, xt, sv * SUB + e) : 0.f;
+        }
+        float sm[8];
+        if constexpr (LT > 0) {
+            // the lane's channels of its token: divide by the smoothing factors, transform, scale
+            const int64_t token = sv / LT;
+            const int64_t srow = kx.smooth_rows > 1 ? (token / kx.S) % kx.heads : 0;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sm[e] = 1.f;
+            if (kx.smooth != nullptr && sv < N) {
+                const float *sp = kx.smooth + (srow * LT + (lane & (LT - 1))) * SUB;
+#pragma unroll
+                for (int e = 0; e < SUB; ++e) { sm[e] = sp[e]; xf[e] = xf[e] / sm[e]; }
+            }
+            wht_lanes<SUB, LT>(xf, lane);
+#pragma unroll
+            for (int e = 0; e < SUB; ++e) xf[e] *= kx.h;
+            if (kx.k_tilde != nullptr && sv < N) {
+#pragma unroll
+                for (int e = 0; e < SUB; e += 4)
+                    *reinterpret_cast<float4 *>(kx.k_tilde + sv * SUB + e) = make_float4(xf[e], xf[e + 1], xf[e + 2], xf[e + 3]);
+            }
         }
         f16x8 xh, xl;
         float x2 = 0.f;
@@ -267,6 +348,33 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             if (blk == t) my_idx = res;
         }
         if (sv < N) st_idx(idx, it, sv, my_idx);
+        if constexpr (LT > 0) {
+            if (kx.k_hat != nullptr) {   // block-uniform
+                float c[8];
+                const int ci = my_idx < nc ? my_idx : nc - 1;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) c[e] = e < SUB ? s_cb[ci * SUB + e] : 0.f;
+                wht_lanes<SUB, LT>(c, lane);
+#pragma unroll
+                for (int e = 0; e < SUB; ++e) c[e] = c[e] * kx.h * sm[e];
+                if (sv < N) {
+                    if (kx.hat_dtype == VQ_F32) {
+#pragma unroll
+                        for (int e = 0; e < SUB; e += 4)
+                            *reinterpret_cast<float4 *>((float *)kx.k_hat + sv * SUB + e) = make_float4(c[e], c[e + 1], c[e + 2], c[e + 3]);
+                    } else {
+                        u32 w[4];
+#pragma unroll
+                        for (int e = 0; e < SUB; e += 2) {
+                            if (kx.hat_dtype == VQ_F16) w[e / 2] = __builtin_bit_cast(u32, f16x2{(f16)c[e], (f16)c[e + 1]});
+                            else w[e / 2] = (u32)f32_to_bf16(c[e]) | ((u32)f32_to_bf16(c[e + 1]) << 16);
+                        }
+                        if constexpr (SUB == 8) *reinterpret_cast<uint4 *>((u16 *)kx.k_hat + sv * 8) = make_uint4(w[0], w[1], w[2], w[3]);
+                        else *reinterpret_cast<uint2 *>((u16 *)kx.k_hat + sv * 4) = make_uint2(w[0], w[1]);
+                    }
+                }
+            }
+        }
         raw = raw_next;
         __builtin_amdgcn_wave_barrier();   // the next step overwrites this wave's LDS slots
     }
@@ -279,10 +387,30 @@ bool launch_assign_mfma(const void *x, int xt, int64_t N, const void *cb, int ct
     int64_t blocks = cdiv(cdiv(N, 64), 4);
     if (blocks > 512) blocks = 512;   // two resident blocks per compute unit
     if (blocks < 1) blocks = 1;
+    const KeyXform none = {};
     if (sub == 8)
-        hipLaunchKernelGGL((vq_assign_mfma_kernel<8>), dim3((unsigned)blocks), dim3(256), 0, st, x, xt, N, cb, ct, nc, idx, it);
+        hipLaunchKernelGGL((vq_assign_mfma_kernel<8, 0>), dim3((unsigned)blocks), dim3(256), 0, st, x, xt, N, cb, ct, nc, idx, it, none);
     else
-        hipLaunchKernelGGL((vq_assign_mfma_kernel<4>), dim3((unsigned)blocks), dim3(256), 0, st, x, xt, N, cb, ct, nc, idx, it);
+        hipLaunchKernelGGL((vq_assign_mfma_kernel<4, 0>), dim3((unsigned)blocks), dim3(256), 0, st, x, xt, N, cb, ct, nc, idx, it, none);
+    return true;
+}
+
+bool launch_encode_keys_mfma(const void *keys, int kt, int64_t B, int64_t heads, int64_t S, int64_t D, const float *smooth,
+                             int smooth_rows, float h, const void *cb, int ct, int nc, int sub, void *idx, int it, void *k_hat,
+                             float *k_tilde, hipStream_t st) {
+    if (nc > VM_MAXC || !(sub == 4 || sub == 8) || D % sub != 0) return false;
+    const int64_t lt = D / sub;
+    if (!(lt == 8 || lt == 16 || lt == 32 || lt == 64)) return false;
+    if (((uintptr_t)keys | (uintptr_t)k_hat | (uintptr_t)k_tilde | (uintptr_t)smooth) & 15u) return false;
+    const int64_t N = B * heads * S * lt;
+    int64_t blocks = cdiv(cdiv(N, 64), 4);
+    if (blocks > 512) blocks = 512;
+    if (blocks < 1) blocks = 1;
+    const KeyXform kx = {smooth, smooth_rows, heads, S, h, k_hat, kt, k_tilde};
+#define VQ_ENC(SUB, LT) hipLaunchKernelGGL((vq_assign_mfma_kernel<SUB, LT>), dim3((unsigned)blocks), dim3(256), 0, st, keys, kt, N, cb, ct, nc, idx, it, kx)
+    if (sub == 8) { if (lt == 8) VQ_ENC(8, 8); else if (lt == 16) VQ_ENC(8, 16); else if (lt == 32) VQ_ENC(8, 32); else VQ_ENC(8, 64); }
+    else { if (lt == 8) VQ_ENC(4, 8); else if (lt == 16) VQ_ENC(4, 16); else if (lt == 32) VQ_ENC(4, 32); else VQ_ENC(4, 64); }
+#undef VQ_ENC
     return true;
 }
 

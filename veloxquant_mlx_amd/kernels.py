@@ -370,6 +370,116 @@ vecinfer_quantize_hip = vecinfer_quantize_metal
 vecinfer_dequant_hip = vecinfer_dequant_metal
 
 
+def _sylvester_scale(H_mat: torch.Tensor) -> float:
+    """``|H[0, 0]|`` if ``H_mat`` is the orthonormal Sylvester-Hadamard matrix in natural order
+    (every entry ``(-1)^popcount(a & b)`` times one magnitude), else 0.  Checked once per tensor
+    object and version (the verdict rides on the tensor itself)."""
+    memo = getattr(H_mat, "_vq_sylvester", None)
+    if memo is None or memo[0] != H_mat._version:
+        D = H_mat.shape[0]
+        ok = H_mat.ndim == 2 and H_mat.shape[1] == D and D >= 1 and (D & (D - 1)) == 0
+        h = 0.0
+        if ok:
+            Hf = H_mat.float()
+            h = float(Hf[0, 0].abs())
+            a = torch.arange(D, device=H_mat.device)
+            par = a[:, None] & a[None, :]
+            sign = torch.ones_like(Hf)
+            for b in range(max(D.bit_length() - 1, 0)):
+                sign = sign * (1 - 2 * ((par >> b) & 1)).to(Hf.dtype)
+            ok = h > 0 and bool(torch.equal(Hf, sign * h))
+        memo = (H_mat._version, h if ok else 0.0)
+        H_mat._vq_sylvester = memo
+    return memo[1]
+
+
+def vecinfer_encode_decode_metal(keys: torch.Tensor, k_codebook: torch.Tensor, sub_dim: int, H_mat: torch.Tensor,
+                                 smooth: torch.Tensor | None = None, *, index_dtype: torch.dtype = torch.int32,
+                                 want_k_hat: bool = True, want_k_tilde: bool = False):
+    """Fused key encode+decode, smooth -> WHT -> VQ -> dequant -> inverse WHT -> smooth, in one
+    launch; drop-in for ``vecinfer_encode_decode_metal`` (veloxquant_mlx/metal/_vecinfer.py:225-293).
+    Returns ``(k_hat [B,H,S,D] in the dtype of keys, k_indices [B,H,S,n_sub])``; with
+    ``want_k_hat=False`` the first element is ``None`` (indices only, what the memory-bound
+    cache needs), with ``want_k_tilde=True`` a third element holds the transformed keys (float32).
+    ``H_mat`` must be the orthonormal Sylvester-Hadamard matrix (``walsh_hadamard_matrix(D)``),
+    which is applied as a fast transform; any other matrix, or a shape the fused kernel does not
+    cover, takes the matrix product followed by the assignment and gather kernels."""
+    name = "vecinfer_encode_decode_metal"
+    if keys.ndim != 4:
+        raise ValueError(f"{name}: keys must be 4D, got {tuple(keys.shape)}")
+    B, Hh, S, D = keys.shape
+    if D % sub_dim != 0:
+        raise ValueError(f"{name}: D={D} not divisible by sub_dim={sub_dim}")
+    if D > 512:
+        raise ValueError(f"{name}: D={D} > 512 (threadgroup limit)")
+    if k_codebook.ndim != 2 or k_codebook.shape[1] != sub_dim or k_codebook.shape[0] == 0:
+        raise ValueError(f"{name}: codebook must be non-empty [n_centroids, {sub_dim}], got {tuple(k_codebook.shape)}")
+    if index_dtype not in (torch.int32, torch.uint8):
+        raise ValueError(f"{name}: index_dtype must be int32 or uint8")
+    _need_gpu(name, keys, k_codebook, H_mat)
+    if keys.dtype not in _FLOAT_TAG:
+        keys = keys.float()
+    kk = keys.contiguous()
+    cb = (k_codebook if k_codebook.dtype in _FLOAT_TAG else k_codebook.float()).contiguous()
+    sm = None
+    if smooth is not None:
+        sm = smooth.reshape(1, D) if smooth.ndim == 1 else smooth
+        sm = sm.to(device=keys.device, dtype=torch.float32)
+        if sm.shape[0] not in (1, Hh):   # e.g. factors calibrated on query heads under GQA: one averaged row
+            sm = sm.mean(dim=0, keepdim=True)
+        sm = sm.contiguous()
+    n_sub = D // sub_dim
+    h = _sylvester_scale(H_mat)
+    fused = h > 0 and sub_dim in (4, 8) and n_sub in (8, 16, 32, 64) and cb.shape[0] <= 256
+    if fused:
+        idx = torch.empty((B, Hh, S, n_sub), dtype=index_dtype, device=keys.device)
+        k_hat = torch.empty_like(kk) if want_k_hat else None
+        k_tilde = torch.empty((B, Hh, S, D), dtype=torch.float32, device=keys.device) if want_k_tilde else None
+        rc = _lib.load().vq_vecinfer_encode_keys(
+            kk.data_ptr(), _FLOAT_TAG[kk.dtype], B, Hh, S, D, sm.data_ptr() if sm is not None else None,
+            sm.shape[0] if sm is not None else 1, h, cb.data_ptr(), _FLOAT_TAG[cb.dtype], cb.shape[0], sub_dim,
+            idx.data_ptr(), VQ_U8 if index_dtype == torch.uint8 else VQ_I32,
+            k_hat.data_ptr() if k_hat is not None else None, k_tilde.data_ptr() if k_tilde is not None else None,
+            _stream(keys))
+        _lib.check(rc)
+    else:
+        Hf = H_mat.float()
+        x = kk.float()
+        if sm is not None:
+            x = x / (sm[:, None, :] if sm.shape[0] == Hh and Hh > 1 else sm[0])
+        k_tilde = x @ Hf
+        idx = vecinfer_quantize_metal(k_tilde, cb, sub_dim, index_dtype=index_dtype)
+        k_hat = None
+        if want_k_hat:
+            k_hat = vecinfer_dequant_metal(idx, cb, out_dtype=torch.float32) @ Hf.T
+            if sm is not None:
+                k_hat = k_hat * (sm[:, None, :] if sm.shape[0] == Hh and Hh > 1 else sm[0])
+            k_hat = k_hat.to(keys.dtype)
+        if not want_k_tilde:
+            k_tilde = None
+    return (k_hat, idx, k_tilde) if want_k_tilde else (k_hat, idx)
+
+
+def vecinfer_encode_decode_simple_metal(values: torch.Tensor, v_codebook: torch.Tensor, sub_dim: int, *,
+                                        index_dtype: torch.dtype = torch.int32):
+    """Value encode+decode: nearest centroid and its gather; drop-in for
+    ``vecinfer_encode_decode_simple_metal`` (veloxquant_mlx/metal/_vecinfer.py:296-345).
+    Returns ``(v_hat [B,H,S,D] in the dtype of values, v_indices [B,H,S,n_sub])``."""
+    name = "vecinfer_encode_decode_simple_metal"
+    if values.ndim != 4:
+        raise ValueError(f"{name}: values must be 4D, got {tuple(values.shape)}")
+    D = values.shape[-1]
+    if D % sub_dim != 0:
+        raise ValueError(f"{name}: D={D} not divisible by sub_dim={sub_dim}")
+    if D > 512:
+        raise ValueError(f"{name}: D={D} > 512 (threadgroup limit)")
+    if v_codebook.ndim != 2 or v_codebook.shape[1] != sub_dim or v_codebook.shape[0] == 0:
+        raise ValueError(f"{name}: codebook must be non-empty [n_centroids, {sub_dim}], got {tuple(v_codebook.shape)}")
+    idx = vecinfer_quantize_metal(values, v_codebook, sub_dim, index_dtype=index_dtype)
+    out_dtype = values.dtype if values.dtype in _FLOAT_TAG else torch.float32
+    return vecinfer_dequant_metal(idx, v_codebook, out_dtype=out_dtype), idx
+
+
 # ---------------------------------------------------------------------------
 # attention over a packed cache
 # ---------------------------------------------------------------------------
@@ -629,6 +739,8 @@ __all__ = [
     "hip_available", "kivi_group_quant_dequant", "kivi_quant_pack", "kivi_quant_codes", "kivi_dequant",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
+    "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",
+    "kv_tail_append", "attend_fixed_order",
     "kivi_packed_attend", "scalar_fused_decode_attend", "scalar_fused_decode_attend_batched",
     "scalar_predecoded_attend", "flash_prefill_attend",
 ]
