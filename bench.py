@@ -265,6 +265,19 @@ def _extras(torch, K, dev):
     flops = 2 * 524288 * 256 * 8
     ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
                             "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
+    # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,
+    # and with the reconstruction written as well
+    from veloxquant_mlx_amd.allocators.vecinfer import walsh_hadamard_matrix
+    x4 = x.reshape(1, 4, 4096, 256)
+    Hm = walsh_hadamard_matrix(256).to(dev)
+    sm = torch.exp(torch.randn((4, 256), device=dev) * 0.3)
+    for name, hat in (("indices", False), ("indices+k_hat", True)):
+        fn = lambda: K.vecinfer_encode_decode_metal(x4, cb, 8, Hm, sm, index_dtype=torch.uint8, want_k_hat=hat)
+        for _ in range(3):
+            fn()
+        ms = _event_ms(fn, 20, torch)
+        nbytes = x4.numel() * 2 + x4.numel() // 8 + (x4.numel() * 2 if hat else 0)
+        ex[f"vq_encode_keys_cfg2_{name}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1), "bytes": nbytes}
     # attention straight from VecInfer indices: 32768 tokens, 8 kv heads x 4 query heads, D 128 in 16
     # sub-vectors of 256 centroids (uint8 indices, 32 B per token and kv head); LDS-bound by design
     for B in (1, 16):
