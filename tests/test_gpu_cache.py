@@ -142,6 +142,59 @@ def test_memory_bound_trim_restores_reconstruction():
     assert np.max(np.abs(host(out).astype(np.float32) - ref)) < 2e-3
 
 
+@pytest.mark.parametrize("mode", ["memory_bound", "stash", "standard"])
+@pytest.mark.parametrize("bits,g,layout", [(4, 32, "auto"), (2, 32, "auto"), (4, 64, "channel")])
+def test_packed_state_round_trip_and_prompt_cache_file(mode, bits, g, layout, tmp_path):
+    """A cache rebuilt from (state, meta_state), directly and through a prompt-cache file,
+    is the cache it came from: same frontier, same bytes, same attention now and after
+    further tokens."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import load_prompt_cache, save_prompt_cache
+    kw = dict(bit_width_inlier=bits, kivi_group_size=g, residual_length=128, kivi_value_layout=layout,
+              fused_sdpa=mode != "standard", fused_sdpa_memory_bound=mode == "memory_bound")
+    K.attend_fixed_order(True)
+    try:
+        c = _make(**kw)
+        k, v = outlier_kv((2, 2, 333, 128), seed=bits + g)
+        c.update_and_fetch(to_dev(k[:, :, :300]), to_dev(v[:, :, :300]))
+        st, meta = c.state, c.meta_state
+        assert meta[0] == "300" and int(meta[1]) == c._n_quantized == ((300 - 128) // g) * g
+        c2 = type(c).from_state(KVCacheConfig(method="kivi", head_dim=128, **kw), st, meta)
+        f = str(tmp_path / "prompt.safetensors")
+        save_prompt_cache(f, [c], metadata={"model": "synthetic"})
+        (c3,), user = load_prompt_cache(f, lambda i, name: _make(**kw), return_metadata=True)
+        assert user == {"model": "synthetic"}
+        q = to_dev(np.random.default_rng(1).standard_normal((2, 8, 1, 128)).astype(np.float16))
+        for step in range(2):
+            for other in (c2, c3):
+                assert other.offset == c.offset and other._n_quantized == c._n_quantized
+                assert other.meta_state == c.meta_state
+                for name in ("compressed_key_bytes", "compressed_value_bytes", "fp16_key_bytes", "residual_fp16_bytes"):
+                    assert getattr(other, name) == getattr(c, name), name
+                assert len(other.state) == len(c.state)
+                for a, b in zip(other.state, c.state):
+                    assert a.shape == b.shape and torch.equal(a, b)
+                if mode != "standard":
+                    assert torch.equal(other.fused_sdpa(q, 0.09), c.fused_sdpa(q, 0.09))
+            if step == 0:   # 33 more tokens: at least one group ages out of the residual window in all three
+                for cc in (c, c2, c3):
+                    cc.update_and_fetch(to_dev(k[:, :, 300:]), to_dev(v[:, :, 300:]))
+        assert c._n_quantized > int(meta[1])
+        # what must be refused
+        with pytest.raises(ValueError, match="configured as"):
+            _make(**{**kw, "bit_width_inlier": 8 if bits != 8 else 4}).meta_state = meta
+        if mode != "standard":
+            with pytest.raises(ValueError, match="arrays"):
+                _make(**kw).state = st[:3]
+            with pytest.raises(ValueError, match="do not fit|must be"):
+                _make(**{**kw, "kivi_group_size": 2 * g}).state = st
+        empty = _make(**kw)
+        empty.state = ()
+        assert empty.offset == 0 and empty.empty()
+    finally:
+        K.attend_fixed_order(False)
+
+
 def test_chunked_prefill_through_the_cache_matches_oracle():
     """Quantise-on-write prefill: chunks of 64 through a cache with R=32, g=32."""
     require_gpu()

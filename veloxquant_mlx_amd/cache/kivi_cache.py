@@ -338,9 +338,126 @@ class KIVIKVCache(FP16KVCache):
 
     @state.setter
     def state(self, v) -> None:
+        """Inverse of the getter, mode by mode.  The frontier comes from the packed rows' own
+        length; byte accounting is rebuilt for the restored token count."""
+        v = tuple(v)
+        if not self._fused_enabled:
+            FP16KVCache.state.fset(self, v)
+            if v:
+                self._shape_bhd = (int(v[0].shape[0]), int(v[0].shape[1]), self._head_dim)
+            return
+        if self._memory_bound:
+            if len(v) not in (0, 2, 6, 8):
+                raise ValueError(f"KIVIKVCache.state: a memory-bound packed state has 0, 2, 6 or 8 arrays, got {len(v)}")
+            packed, tail = (v[:6] if len(v) >= 6 else ()), (v[-2:] if len(v) in (2, 8) else ())
+            self.keys = self.values = None
+        else:
+            if len(v) not in (0, 2, 8):
+                raise ValueError(f"KIVIKVCache.state: a stashed packed state has 0, 2 or 8 arrays, got {len(v)}")
+            FP16KVCache.state.fset(self, v[:2])
+            packed, tail = v[2:], ()
+        ref = packed[0] if packed else (tail[0] if tail else (v[0] if v else None))
+        if ref is not None:
+            self._shape_bhd = (int(ref.shape[0]), int(ref.shape[1]), self._head_dim)
+        self._restore_packed(packed)
+        if self._memory_bound:
+            n_tail = int(tail[0].shape[2]) if tail else 0
+            self._tail_k = self._tail_v = None
+            if tail:
+                tk, tv = tail
+                B, H, D = self._shape_bhd
+                if tuple(tk.shape) != (B, H, n_tail, D) or tuple(tv.shape) != (B, H, n_tail, D):
+                    raise ValueError(f"KIVIKVCache.state: residual rows must be [{B}, {H}, n, {D}], got "
+                                     f"{tuple(tk.shape)} and {tuple(tv.shape)}")
+                cap = -(-max(n_tail, self._residual_length + 2 * self._group_size) // 64) * 64
+                self._tail_k = torch.zeros((B, H, cap, D), dtype=tk.dtype, device=tk.device)
+                self._tail_v = torch.zeros((B, H, cap, D), dtype=tv.dtype, device=tv.device)
+                self._tail_k[:, :, :n_tail] = tk
+                self._tail_v[:, :, :n_tail] = tv
+            self.offset = self._n_quantized + n_tail
+        self._rebuild_accounting()
+
+    def _restore_packed(self, packed) -> None:
+        """Install live packed rows (the six arrays of ``_packed_state``) as the packed store."""
+        self._kp = self._ks = self._kz = self._vp = self._vs = self._vz = None
+        self._packed_cap = 0
+        self._n_quantized = 0
+        if not packed:
+            return
+        kp, ks, kz, vp, vs, vz = packed
+        B, H, D = self._shape_bhd
+        g, per = self._group_size, self._per
+        n = int(kp.shape[2])
+        W, GV = -(-D // per), -(-D // g)
+        if self._v_layout == "token":
+            want_v = ((B, H, n // per, D), (B, H, GV, n), (B, H, GV, n))
+        else:
+            want_v = ((B, H, n, W), (B, H, n, GV), (B, H, n, GV))
+        want = ((B, H, n, W), (B, H, n // g, D), (B, H, n // g, D), *want_v)
+        got = tuple(tuple(t.shape) for t in packed)
+        if n % g or (self._v_layout == "token" and n % per) or got != want:
+            raise ValueError(f"KIVIKVCache.state: packed rows {got} do not fit bits={self._b}, group={g}, "
+                             f"value layout {self._v_layout!r}, head_dim={D} (expected {want})")
+        if any(t.dtype != self._meta_dtype for t in (ks, kz, vs, vz)):
+            raise ValueError(f"KIVIKVCache.state: scale/zero must be {self._meta_dtype}")
+        self._ensure_packed_capacity(B, H, D, n, kp.device)
+        self._kp[:, :, :n] = kp.to(torch.int32) if kp.dtype != torch.int32 else kp
+        self._ks[:, :, : n // g] = ks
+        self._kz[:, :, : n // g] = kz
+        vp32 = vp.to(torch.int32) if vp.dtype != torch.int32 else vp
+        if self._v_layout == "token":
+            self._vp[:, :, : n // per] = vp32
+            self._vs[..., :n] = vs
+            self._vz[..., :n] = vz
+        else:
+            self._vp[:, :, :n] = vp32
+            self._vs[:, :, :n] = vs
+            self._vz[:, :, :n] = vz
+        self._n_quantized = n
+
+    def _rebuild_accounting(self) -> None:
+        B, H, D = self._shape_bhd
+        k, v = self._quantized_bytes(self._n_quantized, B, H, D) if self._n_quantized else (0, 0)
+        self._key_bytes_compressed, self._value_bytes_compressed = k, v
+        self._key_bytes_fp16 = self._value_bytes_fp16 = H * B * self.offset * D * 2
+        self._residual_fp16_bytes = (self.offset - self._n_quantized) * D * 2 * 2 * H * B
+        self._tokens_seen = self.offset
+
+    @property
+    def meta_state(self):
+        """Strings, as prompt-cache files store them: what a restored cache must agree with
+        (offset, frontier, bit width, group, value layout, scale/zero dtype, mode)."""
+        mode = "memory_bound" if self._memory_bound else ("stash" if self._fused_enabled else "standard")
+        return tuple(map(str, (self.offset, self._n_quantized, self._b, self._group_size, self._v_layout,
+                               str(self._meta_dtype).replace("torch.", ""), mode)))
+
+    @meta_state.setter
+    def meta_state(self, v) -> None:
+        v = tuple(v)
+        if len(v) != 7:
+            raise ValueError(f"KIVIKVCache.meta_state: expected 7 fields, got {len(v)}")
+        mine = self.meta_state
+        if tuple(v[2:]) != mine[2:]:
+            raise ValueError(f"KIVIKVCache.meta_state: saved with (bits, group, value layout, meta dtype, mode) = {tuple(v[2:])}, "
+                             f"this cache is configured as {mine[2:]}")
+        offset, n_q = int(v[0]), int(v[1])
         if self._fused_enabled:
-            raise NotImplementedError("KIVIKVCache: restoring a packed state is not supported yet")
-        FP16KVCache.state.fset(self, v)
+            if (offset, n_q) != (self.offset, self._n_quantized):
+                raise ValueError(f"KIVIKVCache.meta_state: offset/frontier {offset}/{n_q} do not match the restored state "
+                                 f"({self.offset}/{self._n_quantized}); assign state first")
+        else:
+            if offset != self.offset:
+                raise ValueError(f"KIVIKVCache.meta_state: offset {offset} does not match the restored state ({self.offset})")
+            self._n_quantized = n_q   # rows below the frontier of the fp16 history are already reconstructions
+            self._rebuild_accounting()
+
+    @classmethod
+    def from_state(cls, config: Any, state, meta_state=None) -> "KIVIKVCache":
+        c = cls(config)
+        c.state = state
+        if meta_state is not None:
+            c.meta_state = meta_state
+        return c
 
     @property
     def nbytes(self) -> int:
