@@ -193,6 +193,21 @@ def _extras(torch, K, dev):
     from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
     ex = {}
     D, Hq, Hkv = 128, 32, 8
+    # ceilings measured in this run, beside the published peaks: a 1 GiB device copy (read + write),
+    # a 2 GiB read (library reduction) and a large fp16 matrix product (library GEMM)
+    src = torch.empty(1 << 29, dtype=torch.float16, device=dev).normal_()
+    dst = torch.empty_like(src)
+    big = torch.empty(1 << 30, dtype=torch.float16, device=dev).fill_(0.25)
+    ga = torch.randn((8192, 8192), device=dev).to(torch.float16)
+    gb = torch.randn((8192, 8192), device=dev).to(torch.float16)
+    for f in (lambda: dst.copy_(src), lambda: big.view(torch.int32).max(), lambda: ga @ gb):
+        for _ in range(3):
+            f()
+    ms_c, ms_r, ms_g = (_event_ms(lambda: dst.copy_(src), 20, torch), _event_ms(lambda: big.view(torch.int32).max(), 20, torch),
+                        _event_ms(lambda: ga @ gb, 10, torch))
+    ex["measured_ceilings"] = {"copy_GBps": round((2 << 30) / ms_c / 1e6, 1), "read_GBps_library_reduction": round((2 << 30) / ms_r / 1e6, 1),
+                               "gemm_f16_TFLOPs": round(2 * 8192 ** 3 / ms_g / 1e9, 1)}
+    del src, dst, big, ga, gb
     for B in (1, 16):
         cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=2, kivi_group_size=32, residual_length=128,
                             fused_sdpa=True, fused_sdpa_memory_bound=True)
