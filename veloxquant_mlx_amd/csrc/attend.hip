@@ -30,12 +30,13 @@ AttendPlan plan_attend(const vq_attend_args &a) {
         return p;
     }
     // tokens the kernel splits: the MFMA path hands the tail to the block of split 0 and
-    // prices a tail token at two packed tokens when it balances the splits
+    // prices a tail token at five packed tokens when it balances the splits (the tail pass
+    // is short but latency-bound: about 5 us, the time a block streams 500-800 packed tokens)
     int64_t n_split = a.n_packed + a.n_tail;
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
         p.tiles = (int)cdiv(a.Sq, p.pq);
-                p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 2, 128) * 128 : 0;
+                p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 5, 128) * 128 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
     // the MFMA kernel wants every block to start on a boundary of the largest token group (128)

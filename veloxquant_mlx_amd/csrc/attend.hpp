@@ -22,35 +22,39 @@ struct AttendPlan {
 };
 
 // One output element from the split partials of its query row: p points at nparts records
-// of `stride` floats (max in natural-log units, sum, accumulator[D]).  Eight records are
-// fetched at a time with independent loads; DEVICE_SCOPE reads partials that other blocks
+// of `stride` floats (max in natural-log units, sum, accumulator[D]).  CH records are
+// fetched at a time with independent loads (a round costs one memory latency, so callers with
+// many records pick a large CH); DEVICE_SCOPE reads partials that other blocks
 // of the same launch wrote.
 template <bool DEVICE_SCOPE> __device__ __forceinline__ float ld_part(const float *p) {
     if (DEVICE_SCOPE) return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return *p;
 }
-template <bool DEVICE_SCOPE>
+template <bool DEVICE_SCOPE, int CH = 8>
 __device__ __forceinline__ float merge_partials(const float *p, int nparts, int64_t stride, int64_t d) {
     float gm = -INFINITY, num = 0.f, den = 0.f;
-    for (int s0 = 0; s0 < nparts; s0 += 8) {
-        float m[8], l[8], o[8];
+    for (int s0 = 0; s0 < nparts; s0 += CH) {
+        float m[CH], l[CH], o[CH];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
+        for (int j = 0; j < CH; ++j) {
             const float *q = p + (int64_t)(s0 + j < nparts ? s0 + j : s0) * stride;
             m[j] = ld_part<DEVICE_SCOPE>(q);
             l[j] = ld_part<DEVICE_SCOPE>(q + 1);
             o[j] = ld_part<DEVICE_SCOPE>(q + 2 + d);
         }
+        // every load of the round is issued before the first use: left to itself the scheduler
+        // weaves the maxima between the loads and waits for each record in turn
+        __builtin_amdgcn_sched_barrier(0);
         float cm = gm;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < CH; ++j)
             if (s0 + j < nparts) cm = fmaxf(cm, m[j]);
         if (cm == -INFINITY) continue;   // nothing visible so far
         const float f0 = __expf(gm - cm);   // 0 on the first chunk
         num *= f0;
         den *= f0;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)
+        for (int j = 0; j < CH; ++j)
             if (s0 + j < nparts && m[j] != -INFINITY) {
                 const float f = __expf(m[j] - cm);
                 den += l[j] * f;
@@ -60,6 +64,15 @@ __device__ __forceinline__ float merge_partials(const float *p, int nparts, int6
     }
     return den > 0.f ? num / den : 0.f;
 }
+// the round size by the number of records: one round of loads when they fit (every caller goes
+// through here, so the in-kernel merge and the merge kernel add in the same order)
+template <bool DEVICE_SCOPE>
+__device__ __forceinline__ float merge_records(const float *p, int nparts, int64_t stride, int64_t d) {
+    return nparts <= 8 ? merge_partials<DEVICE_SCOPE, 8>(p, nparts, stride, d)
+           : nparts <= 16 ? merge_partials<DEVICE_SCOPE, 16>(p, nparts, stride, d)
+                          : merge_partials<DEVICE_SCOPE, 36>(p, nparts, stride, d);
+}
+
 
 // Decides kernel and split count from shapes only, so that the workspace query
 // and the launch agree.

@@ -114,7 +114,7 @@ __global__ void attend_merge_kernel(const float *__restrict__ ws, int64_t rows, 
     const int64_t n = rows * D;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
         const int64_t row = e / D, d = e % D;
-        st_tag(out, out_dtype, e, merge_partials<false>(ws + row * nsplit * (D + 2), nsplit, D + 2, d));
+        st_tag(out, out_dtype, e, merge_records<false>(ws + row * nsplit * (D + 2), nsplit, D + 2, d));
     }
 }
 

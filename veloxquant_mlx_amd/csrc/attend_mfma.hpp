@@ -374,7 +374,8 @@ __device__ __forceinline__ void merge_rows(const vq_attend_args &a, const RowTil
         const int j = e / MF_D, d = e % MF_D;
         if (!tile.valid(j)) continue;
         const int64_t row = tile.row(j);
-        const float v = merge_partials<true>(ws + row * nparts * MF_PART, nparts, MF_PART, d);
+        // partials of other blocks come from beyond this XCD's L2: as few rounds of loads as possible
+        const float v = merge_records<true>(ws + row * nparts * MF_PART, nparts, MF_PART, d);
         const int64_t oi = row * MF_D + d;
         if (a.out_dtype == VQ_F16) ((f16 *)a.out)[oi] = (f16)v;
         else if (a.out_dtype == VQ_BF16) ((u16 *)a.out)[oi] = f32_to_bf16(v);
