@@ -182,7 +182,10 @@ typedef struct vq_attend_args {
     int causal;  /* 1: query i sees slots <= n_packed + n_tail - Sq + i */
     int num_splits; /* 0 = choose; > 0 the split count along tokens; < 0 choose, but take the
                      * layout-agnostic vector kernel even where the MFMA kernel applies
-                     * (cross-checks of the two implementations) */
+                     * (cross-checks of the two implementations); -2: that kernel with every
+                     * reconstructed key and value rounded to fp16 first, the form in which the
+                     * reference's cache holds them (cache/kivi_cache.py:198-201) and the
+                     * 256-row prefill blocks attend over them */
     void *workspace;
     size_t workspace_bytes;
     void *stream;

@@ -64,15 +64,22 @@ def reference_attend(q, kc, ks, kz, vc, vs, vz, g: int, scale: float) -> np.ndar
 
 
 def kivi_attend(q, kc, ks, kz, vc, vs, vz, g: int, k_tail, v_tail, scale: float,
-                causal: bool = False, acc=np.float64) -> np.ndarray:
+                causal: bool = False, acc=np.float64, recon_dtype=None) -> np.ndarray:
     """Attention over a quantised prefix followed by an fp16 tail.
 
     The tail is what ``KIVIKVCache`` keeps un-quantised (residual window plus
-    the partial group); either part may be empty."""
+    the partial group); either part may be empty.  ``recon_dtype`` (e.g.
+    ``np.float16``) rounds the reconstruction to the dtype the cache stores it in
+    before it is attended over (kivi_cache.py:198-201: ``x_hat.astype(x.dtype)``);
+    ``None`` keeps the float32 reconstruction of the fused decode kernel
+    (metal/src/scalar_affine_attend.metal)."""
     parts_k, parts_v = [], []
     if kc is not None and kc.shape[-2] > 0:
-        parts_k.append(group_dequant(kc, ks, kz, -2, g))
-        parts_v.append(group_dequant(vc, vs, vz, -1, g))
+        kh, vh = group_dequant(kc, ks, kz, -2, g), group_dequant(vc, vs, vz, -1, g)
+        if recon_dtype is not None:
+            kh, vh = kh.astype(recon_dtype).astype(F32), vh.astype(recon_dtype).astype(F32)
+        parts_k.append(kh)
+        parts_v.append(vh)
     if k_tail is not None and k_tail.shape[-2] > 0:
         parts_k.append(np.asarray(k_tail).astype(F32))
         parts_v.append(np.asarray(v_tail).astype(F32))

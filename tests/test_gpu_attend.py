@@ -183,6 +183,16 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
     ref = oa.kivi_attend(host(qt), *ref_args, g, k[:, :, n_packed:], v[:, :, n_packed:], scale, causal=causal)
     err = float(np.max(np.abs(host(out) - ref)))
     print(f"max-abs err {err:.2e} (path {plan['path']}, {plan['nparts']} partials)")
+    if plan["path"] == 2 and (Hq // Hkv) * Sq >= 256:
+        # The 256-row prefill blocks attend over the reconstruction rounded to fp16, which is
+        # what the reference's cache holds (kivi_cache.py:198-201): that is the oracle at the
+        # usual tolerance; against the float32 reconstruction the rounding of keys and values
+        # shows (2^-11 relative each).
+        assert err < 1e-2, err   # the bar of the reference's own fused attention tests
+        ref16 = oa.kivi_attend(host(qt), *ref_args, g, k[:, :, n_packed:], v[:, :, n_packed:], scale, causal=causal,
+                               recon_dtype=np.float16)
+        err = float(np.max(np.abs(host(out) - ref16)))
+        print(f"max-abs err {err:.2e} against the fp16 reconstruction")
     assert err < TOL, err
     return err
 

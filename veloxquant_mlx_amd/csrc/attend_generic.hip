@@ -85,6 +85,10 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(vq_attend_args a, i
                 }
                 float vc = (float)((vw >> sh) & mask);
                 vh[j] = __fadd_rn(__fmul_rn(vc, ld_tag(a.v_scale, a.meta_dtype, vmi)), ld_tag(a.v_zero, a.meta_dtype, vmi));
+                if (a.num_splits == -2) {   // the reconstruction as a cache that stores it in fp16 holds it
+                    kh[j] = (float)(f16)kh[j];
+                    vh[j] = (float)(f16)vh[j];
+                }
             } else {
                 int64_t ti = (bh * a.tail_cap + (t - a.n_packed)) * D + d;
                 kh[j] = ld_tag(a.k_tail, a.tail_dtype, ti);

@@ -414,6 +414,291 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     }
 }
 
+// ---- 256-row blocks: keys and values reconstructed in the producer --------------------------
+//
+// With many query rows per kv head (a prefill chunk) the cost that matters is MFMA issue, and
+// the raw-code formulation above spends 46 MFMAs per 16 rows and 32 tokens where 16 are useful.
+// Here the producer turns the codes into the reconstruction itself, k^ = c s + z and
+// v^ = c s + z as packed fp16 fused multiply-adds on exact fp16 codes (c s + z is formed
+// exactly and rounded once to fp16, which is what the reference's cache holds: it stores the
+// reconstruction cast to the input dtype, veloxquant_mlx/cache/kivi_cache.py:181-201), and the
+// consumer is plain attention: 8 + 8 MFMAs per 16 rows and unit plus one for the row sums.  A
+// wave owns two 16-row blocks so that every LDS read of a key or value tile feeds two MFMAs and
+// everything still fits the 256 registers of two waves per SIMD (with four row blocks the
+// accumulators spill into the accumulation registers and the compiler moves them back and
+// forth around every product); a block is eight waves = 256 rows = the GQA group at 256 / R
+// consecutive positions, one block per CU, so a unit is unpacked once for 256 rows.  Tiles,
+// token order, lazily rescaled softmax and partials are those of the kernel above.
+constexpr int PR_RB = 2;          // 16-row blocks per wave
+constexpr int PR_THREADS = 512;
+
+template <int BITS> struct PrStage {
+    u32 kw;          // key word: the thread's 8 channels of one token (2-bit: the word holding them)
+    u32 vw;          // value word: the thread's 8 tokens of one channel (2-bit: the word holding them)
+    uint4 vs, vz;    // value scale / zero of those 8 tokens (the thread's channel group)
+};
+
+template <int BITS, int GV>
+__global__ __launch_bounds__(PR_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__restrict__ ws) {
+    __shared__ __align__(16) f16 s_k[2][32 * PF_KSTRIDE];
+    __shared__ __align__(16) f16 s_v[2][MF_D * PF_VSTRIDE];
+
+    constexpr int PER = 32 / BITS;
+    constexpr int KW = MF_D / PER;
+    constexpr int gshift = GV == 4 ? 5 : GV == 2 ? 6 : 7;   // log2 of the group size
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, blk = lane >> 4;
+    const int64_t bh = blockIdx.y;
+    const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    const int R = (int)(a.Hq / a.Hkv);
+    const int64_t cap = a.cap_tokens;
+    const float c = a.scale * LOG2E;
+    const u32 magic = vreg_const(Magic<BITS>::bits);
+    const int pos0 = (int)blockIdx.x * qp;
+    const int64_t n_total = a.n_packed + a.n_tail;
+    auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
+
+    // ---- this lane's query rows (score columns): row j = 32 wave + 16 rb + n of the block
+    int lane_vis[PR_RB], lane_tvis[PR_RB];
+    f16x8 qn[PR_RB][4];   // B operands: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of its row
+#pragma unroll
+    for (int rb = 0; rb < PR_RB; ++rb) {
+        const int j = 16 * PR_RB * wave + 16 * rb + n;
+        const int64_t pos = pos0 + j % qp;
+        const bool row_ok = pos < a.Sq && j / qp < R;
+        const int64_t qrow = (b * a.Hq + hkv * R + (j / qp < R ? j / qp : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
+        const int64_t vis = visible(row_ok ? pos : a.Sq - 1);
+        lane_vis[rb] = (int)(vis < a.n_packed ? vis : a.n_packed);
+        const int64_t tv = vis - a.n_packed;
+        lane_tvis[rb] = (int)(tv < 0 ? 0 : tv < a.n_tail ? tv : a.n_tail);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int64_t e0 = qrow * MF_D + 32 * ks + 8 * blk;
+            if (a.q_dtype == VQ_F32) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qn[rb][ks][e] = (f16)((const float *)a.q)[e0 + e];
+            } else {
+                qn[rb][ks] = ld_tail8(a.q, e0, a.q_dtype == VQ_BF16);
+            }
+        }
+    }
+    const int64_t last_pos = pos0 + qp - 1 < a.Sq - 1 ? pos0 + qp - 1 : a.Sq - 1;
+    const int64_t vis_min = visible(pos0), vis_max = visible(last_pos);
+    const int full_vis = (int)(vis_min < a.n_packed ? vis_min : a.n_packed);
+    const int max_vis = (int)(vis_max < a.n_packed ? vis_max : a.n_packed);
+    const int64_t tv_min = vis_min - a.n_packed, tv_max = vis_max - a.n_packed;
+    const int full_tvis = (int)(tv_min < 0 ? 0 : tv_min < a.n_tail ? tv_min : a.n_tail);
+    const int max_tvis = (int)(tv_max < 0 ? 0 : tv_max < a.n_tail ? tv_max : a.n_tail);
+    const int n_punits = (max_vis + 31) / 32;
+    const int n_tunits = (max_tvis + 31) / 32;
+    const int n_work = n_punits + n_tunits;
+    const int nsplit = (int)gridDim.z, sp = (int)blockIdx.z;
+    const int w0 = (int)((int64_t)n_work * sp / nsplit), w1 = (int)((int64_t)n_work * (sp + 1) / nsplit);
+
+    // ---- producer side
+    const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
+    const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
+    const f16 *ksb = (const f16 *)a.k_scale + bh * (cap >> gshift) * MF_D;
+    const f16 *kzb = (const f16 *)a.k_zero + bh * (cap >> gshift) * MF_D;
+    const f16 *vsb = (const f16 *)a.v_scale + bh * GV * cap;
+    const f16 *vzb = (const f16 *)a.v_zero + bh * GV * cap;
+    const int kt = tid >> 4, kc = tid & 15;       // key tile: token, 8-channel chunk
+    const int vc = tid & 127, vq = tid >> 7;      // value tile: channel, 8-token quarter
+    const int vg = vc >> gshift;                  // channel group of the thread's value channel
+    const bool tail_bf16 = a.tail_dtype == VQ_BF16;
+    const int64_t tbase = bh * a.tail_cap * MF_D;
+    const f16x8 off8 = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair);
+    using Stage = PrStage<BITS>;
+    f16x8 ksr, kzr;   // key scale / zero of the thread's 8 channels in the token group last fetched
+    int meta_group = -1;
+    auto fetch = [&](int w, Stage &st) {   // packed work units only
+        if (w >= n_punits) return;
+        const int64_t base = (int64_t)w * 32;
+        if (BITS == 4) {
+            st.kw = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + kc) * 4);
+            st.vw = *reinterpret_cast<const u32 *>(vb + ((base / 8 + vq) * MF_D + vc) * 4);
+        } else {
+            st.kw = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + (kc >> 1)) * 4);
+            st.vw = *reinterpret_cast<const u32 *>(vb + ((base / 16 + (vq >> 1)) * MF_D + vc) * 4);
+        }
+        st.vs = *reinterpret_cast<const uint4 *>(vsb + (int64_t)vg * cap + base + 8 * vq);
+        st.vz = *reinterpret_cast<const uint4 *>(vzb + (int64_t)vg * cap + base + 8 * vq);
+        const int grp = (int)(base >> gshift);
+        if (grp != meta_group) {   // block-uniform
+            meta_group = grp;
+            ksr = *reinterpret_cast<const f16x8 *>(ksb + (int64_t)grp * MF_D + 8 * kc);
+            kzr = *reinterpret_cast<const f16x8 *>(kzb + (int64_t)grp * MF_D + 8 * kc);
+        }
+    };
+    // the thread's eight codes of a word, in order, as exact fp16 numbers
+    auto codes8 = [&](u32 w, int half) -> f16x8 {
+        uint4 lo;
+        if (BITS == 4) lo = word4_in_order(w, magic);
+        else {
+            uint4 hi;
+            word2_in_order(w, magic, lo, hi);
+            if (half) lo = hi;
+        }
+        return as_h8(lo) + off8;
+    };
+    auto unpack_to_lds = [&](int w, const Stage &st, int buf) {
+        if (w < n_punits) {
+            // keys: 8 channels of token kt; c s + z is formed exactly and rounded once
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) =
+                __builtin_elementwise_fma(codes8(st.kw, kc & 1), ksr, kzr);
+            // values: 8 tokens of channel vc
+            *reinterpret_cast<f16x8 *>(&s_v[buf][vc * PF_VSTRIDE + 8 * vq]) =
+                __builtin_elementwise_fma(codes8(st.vw, vq & 1), as_h8(st.vs), as_h8(st.vz));
+        } else {
+            // tail unit (few per block, fetched here): plain key row chunk; value row chunk transposed
+            int64_t tok = (int64_t)(w - n_punits) * 32 + kt;
+            if (tok >= a.n_tail) tok = 0;   // masked in the softmax
+            const int64_t e0 = tbase + tok * MF_D + 8 * kc;
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = ld_tail8(a.k_tail, e0, tail_bf16);
+            const f16x8 v0 = ld_tail8(a.v_tail, e0, tail_bf16);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s_v[buf][(8 * kc + e) * PF_VSTRIDE + kt] = v0[e];
+        }
+    };
+
+    // ---- consumer state: O[rb][nt] rows 16 rb + 4 blk + r of the wave, channels 16 nt + n; L the row sums
+    f32x4 O[PR_RB][8], L[PR_RB];
+    float m_run[PR_RB], m_seen[PR_RB];
+#pragma unroll
+    for (int rb = 0; rb < PR_RB; ++rb) {
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) O[rb][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        L[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m_run[rb] = -INFINITY;
+        m_seen[rb] = -INFINITY;
+    }
+    const f16x8 ones = ones8();
+
+    // move the reference of every row up to what it has seen and rescale the accumulators
+    auto rescale = [&]() {
+#pragma unroll
+        for (int rb = 0; rb < PR_RB; ++rb) {
+            float ms = m_seen[rb];
+            ms = fmaxf(ms, __shfl_xor(ms, 16));
+            ms = fmaxf(ms, __shfl_xor(ms, 32));
+            const float m_new = fmaxf(m_run[rb], ms);
+            const float alpha = m_new == -INFINITY ? 1.f : exp2f(m_run[rb] - m_new);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float al = __shfl(alpha, 4 * blk + r);
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) O[rb][nt][r] *= al;
+                L[rb][r] *= al;
+            }
+            m_run[rb] = m_new;
+        }
+    };
+
+    // One unit: scores of the wave's row blocks, softmax against the lazily updated
+    // references, second product.  Returns false, having only noted the maxima, when some row's
+    // scores outgrow its reference: the caller rescales and repeats the unit.
+    auto compute = [&](int buf, int base, bool packed, int full) -> bool {
+        f32x4 S[PR_RB][2];
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            const f16 *kr = &s_k[buf][pf_krow(pf_tok(n >> 2, n & 3, T)) * PF_KSTRIDE + 8 * blk];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                const f16x8 A = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
+#pragma unroll
+                for (int rb = 0; rb < PR_RB; ++rb)
+                    S[rb][T] = VQ_MFMA(A, qn[rb][ks], ks == 0 ? (f32x4{0.f, 0.f, 0.f, 0.f}) : S[rb][T]);
+            }
+        }
+        bool grow = false;
+#pragma unroll
+        for (int rb = 0; rb < PR_RB; ++rb) {
+            if (base + 32 > full) {
+                const int lim = packed ? lane_vis[rb] : lane_tvis[rb];
+#pragma unroll
+                for (int T = 0; T < 2; ++T)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (base + pf_tok(blk, r, T) >= lim) S[rb][T][r] = -INFINITY;
+            }
+            const float mx = fmaxf(fmaxf(fmaxf(S[rb][0][0], S[rb][0][1]), fmaxf(S[rb][0][2], S[rb][0][3])),
+                                   fmaxf(fmaxf(S[rb][1][0], S[rb][1][1]), fmaxf(S[rb][1][2], S[rb][1][3])));
+            m_seen[rb] = mx * c;
+            grow |= mx * c > m_run[rb] + RESCALE_SLACK;
+        }
+        if (__any(grow)) return false;
+        f16x8 P8[PR_RB];
+#pragma unroll
+        for (int rb = 0; rb < PR_RB; ++rb) {
+            const float nm = m_run[rb] == -INFINITY ? 0.f : -m_run[rb];
+            u32 P[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                P[r] = as_u(f16x2{(f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[rb][0][r], c, nm)),
+                                  (f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[rb][1][r], c, nm))});
+            P8[rb] = as_h8(P[0], P[1], P[2], P[3]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) {
+            const f16x8 Bv = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+#pragma unroll
+            for (int rb = 0; rb < PR_RB; ++rb) O[rb][nt] = VQ_MFMA(P8[rb], Bv, O[rb][nt]);
+        }
+#pragma unroll
+        for (int rb = 0; rb < PR_RB; ++rb) L[rb] = VQ_MFMA(P8[rb], ones, L[rb]);
+        return true;
+    };
+
+    // ---- pipeline over the work units [w0, w1), as in the kernel above
+    Stage st;
+    if (w1 > w0) {
+        fetch(w0, st);
+        unpack_to_lds(w0, st, 0);
+        __syncthreads();
+        if (w0 + 1 < w1) fetch(w0 + 1, st);
+    }
+    bool staged = false;   // unit w+1 already unpacked (set while a unit is being repeated)
+    for (int w = w0; w < w1;) {
+        const int buf = (w - w0) & 1;
+        if (!staged) {
+            if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
+            if (w + 2 < w1) fetch(w + 2, st);
+            staged = true;
+        }
+        const bool packed = w < n_punits;
+        const int base = packed ? w * 32 : (w - n_punits) * 32;
+        if (!compute(buf, base, packed, packed ? full_vis : full_tvis)) {
+            rescale();
+            continue;
+        }
+        __syncthreads();
+        staged = false;
+        ++w;
+    }
+
+    // ---- every wave owns its rows: accumulator register r of lane (n, blk) is row 4 blk + r of the
+    // row block, tile nt column n is channel 16 nt + n; the row's reference sits in lane 4 blk + r
+#pragma unroll
+    for (int rb = 0; rb < PR_RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int jr = 16 * PR_RB * wave + 16 * rb + 4 * blk + r;
+            const int64_t pr = pos0 + jr % qp;
+            const float mr = __shfl(m_run[rb], 4 * blk + r);
+            if (pr < a.Sq && jr / qp < R) {
+                const int64_t row = (b * a.Hq + hkv * R + jr / qp) * a.Sq + pr;
+                float *o = ws + (row * nparts + sp) * MF_PART;
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) o[2 + 16 * nt + n] = O[rb][nt][r];
+                if (n == 0) { o[0] = mr * LN2; o[1] = L[rb][r]; }
+            }
+        }
+}
+
+int mfma_prefill_block_rows(const vq_attend_args &a);
+
 bool mfma_prefill_supported(const vq_attend_args &a) {
     if (a.D != MF_D || a.n_packed <= 0 || a.Sq < 16) return false;
     if (a.Hq % a.Hkv != 0) return false;
@@ -431,18 +716,29 @@ bool mfma_prefill_supported(const vq_attend_args &a) {
     const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
                          (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
     if (al & 15u) return false;
+    if (mfma_prefill_block_rows(a) == 256 && a.q_dtype != VQ_F32 && ((uintptr_t)a.q & 15u)) return false;
     return true;
+}
+
+int mfma_prefill_block_rows(const vq_attend_args &a) {
+    return (a.Hq / a.Hkv) * a.Sq >= 256 ? 256 : 64;
 }
 
 void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     hipStream_t st = (hipStream_t)a.stream;
     float *ws = (float *)a.workspace;
     const int R = (int)(a.Hq / a.Hkv);
-    const int qp = 64 / R, tiles = (int)cdiv(a.Sq, qp);
+    const int rows = mfma_prefill_block_rows(a);
+    const int qp = rows / R, tiles = (int)cdiv(a.Sq, qp);
     const int gv = (int)(MF_D / a.group);
     const dim3 grid((unsigned)tiles, (unsigned)(a.B * a.Hkv), (unsigned)p.nsplit), block(256);
-#define VQ_LAUNCH(BITS, GV) \
-    hipLaunchKernelGGL((attend_prefill_kernel<BITS, GV>), grid, block, 0, st, a, qp, p.nparts, ws)
+#define VQ_LAUNCH(BITS, GV)                                                                                          \
+    do {                                                                                                             \
+        if (rows == 256)                                                                                             \
+            hipLaunchKernelGGL((attend_prefill_rows_kernel<BITS, GV>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \
+        else                                                                                                         \
+            hipLaunchKernelGGL((attend_prefill_kernel<BITS, GV>), grid, block, 0, st, a, qp, p.nparts, ws);           \
+    } while (0)
     if (a.pack_bits == 4) { if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4); }
     else { if (gv == 1) VQ_LAUNCH(2, 1); else if (gv == 2) VQ_LAUNCH(2, 2); else VQ_LAUNCH(2, 4); }
 #undef VQ_LAUNCH
