@@ -117,7 +117,8 @@ def test_fused_sdpa_over_packed_prefix(memory_bound, bits, g, meta):
                          vq[2].astype(npm), g, k[:, :, nq:], v[:, :, nq:], 1 / math.sqrt(128))
     assert np.max(np.abs(host(out).astype(np.float32) - ref)) < 2e-3
     if memory_bound:
-        assert c.nbytes < 0.6 * (2 * 2 * 2 * c._packed_cap * 128 * 2) + 4 * c._tail_k.numel()
+        # packed store plus the two pairs of fp16 tail buffers (the kept rows move between them at a flush)
+        assert c.nbytes < 0.6 * (2 * 2 * 2 * c._packed_cap * 128 * 2) + 8 * c._tail_k.numel()
         assert float(ko.abs().sum()) == 0.0 and not c.empty()
     else:
         # stash mode still returns the reference's fp16 history

@@ -108,6 +108,7 @@ class KIVIKVCache(FP16KVCache):
         self._packed_cap = 0
         # fp16 tail (memory-bound mode): tokens [_n_quantized, offset)
         self._tail_k = self._tail_v = None
+        self._tail_spare = None   # second pair of tail buffers the kept rows move into at a flush
         self._zero_scalar = None
 
     # ------------------------------------------------------------------
@@ -221,16 +222,24 @@ class KIVIKVCache(FP16KVCache):
         if n_quant_now > 0:
             self._pack_block(self._tail_k[:, :, :n_quant_now], self._tail_v[:, :, :n_quant_now], self._n_quantized)
             keep = need - n_quant_now
-            if keep:
-                self._tail_k[:, :, :keep] = self._tail_k[:, :, n_quant_now:need].clone()
-                self._tail_v[:, :, :keep] = self._tail_v[:, :, n_quant_now:need].clone()
-            self._n_quantized = new_boundary
-            # a large prefill chunk leaves an oversized tail buffer behind: give it back
+            # the rows that stay move to the front of a second buffer (one copy each, no
+            # temporaries); a very large prefill chunk leaves an oversized buffer behind, which is
+            # given back here, while chunked prefill keeps its buffers from chunk to chunk
             floor_cap = -(-(self._residual_length + 2 * self._group_size) // 64) * 64
-            if self._tail_k.shape[2] > max(floor_cap, 4 * keep):
+            cap = self._tail_k.shape[2]
+            if cap > max(4 * floor_cap, 16 * keep):
                 cap = max(floor_cap, -(-2 * keep // 64) * 64)
-                self._tail_k = self._tail_k[:, :, :cap].clone()
-                self._tail_v = self._tail_v[:, :, :cap].clone()
+            spare = self._tail_spare
+            if spare is None or spare[0].shape != (B, H, cap, D) or spare[0].dtype != self._tail_k.dtype:
+                spare = (torch.zeros((B, H, cap, D), dtype=self._tail_k.dtype, device=keys.device),
+                         torch.zeros((B, H, cap, D), dtype=self._tail_v.dtype, device=keys.device))
+            if keep:
+                spare[0][:, :, :keep] = self._tail_k[:, :, n_quant_now:need]
+                spare[1][:, :, :keep] = self._tail_v[:, :, n_quant_now:need]
+            old = (self._tail_k, self._tail_v)
+            self._tail_k, self._tail_v = spare
+            self._tail_spare = old if old[0].shape[2] == cap else None
+            self._n_quantized = new_boundary
         self._account_bytes(B, H, S, D, n_quant_now)
         z = self._zero_scalar
         if z is None or z.dtype != keys.dtype or z.device != keys.device:
@@ -462,7 +471,8 @@ class KIVIKVCache(FP16KVCache):
     @property
     def nbytes(self) -> int:
         total = 0 if self._memory_bound else FP16KVCache.nbytes.fget(self)
-        for t in (self._kp, self._ks, self._kz, self._vp, self._vs, self._vz, self._tail_k, self._tail_v):
+        for t in (self._kp, self._ks, self._kz, self._vp, self._vs, self._vz, self._tail_k, self._tail_v,
+                  *(self._tail_spare or ())):
             if t is not None:
                 total += t.numel() * t.element_size()
         return total

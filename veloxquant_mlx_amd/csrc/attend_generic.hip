@@ -122,6 +122,48 @@ __global__ void attend_merge_kernel(const float *__restrict__ ws, int64_t rows, 
     }
 }
 
+// Up to four records per row, even D: a thread takes two neighbouring channels (the records'
+// accumulators start 8 bytes into a record whose size is a multiple of 8, so the pairs are
+// aligned) and reads each record's maximum and sum once for both.
+__global__ void attend_merge4_kernel(const float *__restrict__ ws, int64_t rows, int nsplit, int64_t D,
+                                     void *__restrict__ out, int out_dtype) {
+    const int64_t half = D / 2, n = rows * half;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = e / half, d = 2 * (e % half);
+        const float *rec = ws + row * nsplit * (D + 2);
+        float m[4], l[4];
+        float2 o[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float *q = rec + (int64_t)(j < nsplit ? j : 0) * (D + 2);
+            m[j] = j < nsplit ? q[0] : -INFINITY;
+            l[j] = q[1];
+            o[j] = *reinterpret_cast<const float2 *>(q + 2 + d);
+        }
+        const float gm = fmaxf(fmaxf(m[0], m[1]), fmaxf(m[2], m[3]));
+        float den = 0.f, nx = 0.f, ny = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (m[j] != -INFINITY) {
+                const float f = __expf(m[j] - gm);
+                den += l[j] * f;
+                nx += o[j].x * f;
+                ny += o[j].y * f;
+            }
+        st_tag(out, out_dtype, row * D + d, den > 0.f ? nx / den : 0.f);
+        st_tag(out, out_dtype, row * D + d + 1, den > 0.f ? ny / den : 0.f);
+    }
+}
+
+static void launch_merge(const float *ws, int64_t rows, int nparts, int64_t D, void *out, int out_dtype, hipStream_t st) {
+    const bool pairs = nparts <= 4 && D % 2 == 0 && ((uintptr_t)ws & 7u) == 0;
+    int64_t g = cdiv(pairs ? rows * D / 2 : rows * D, 256);
+    if (g > (1 << 20)) g = 1 << 20;
+    if (g < 1) g = 1;
+    if (pairs) hipLaunchKernelGGL(attend_merge4_kernel, dim3((unsigned)g), dim3(256), 0, st, ws, rows, nparts, D, out, out_dtype);
+    else hipLaunchKernelGGL(attend_merge_kernel, dim3((unsigned)g), dim3(256), 0, st, ws, rows, nparts, D, out, out_dtype);
+}
+
 int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len) {
     hipStream_t st = (hipStream_t)a.stream;
     const int64_t rows = a.B * a.Hq * a.Sq;
@@ -132,18 +174,11 @@ int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len
 }
 
 void launch_merge_rows(const float *ws, int64_t rows, int nparts, int64_t D, void *out, int out_dtype, hipStream_t st) {
-    int64_t g = cdiv(rows * D, 256);
-    if (g > (1 << 20)) g = 1 << 20;
-    hipLaunchKernelGGL(attend_merge_kernel, dim3((unsigned)g), dim3(256), 0, st, ws, rows, nparts, D, out, out_dtype);
+    launch_merge(ws, rows, nparts, D, out, out_dtype, st);
 }
 
 int launch_attend_merge(const vq_attend_args &a, int nparts) {
-    hipStream_t st = (hipStream_t)a.stream;
-    const int64_t rows = a.B * a.Hq * a.Sq;
-    int64_t g = cdiv(rows * a.D, 256);
-    if (g > (1 << 20)) g = 1 << 20;
-    hipLaunchKernelGGL(attend_merge_kernel, dim3((unsigned)g), dim3(256), 0, st, (const float *)a.workspace, rows,
-                       nparts, a.D, a.out, a.out_dtype);
+    launch_merge((const float *)a.workspace, a.B * a.Hq * a.Sq, nparts, a.D, a.out, a.out_dtype, (hipStream_t)a.stream);
     return VQ_OK;
 }
 

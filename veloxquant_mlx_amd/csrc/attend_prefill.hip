@@ -597,21 +597,30 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     };
 
     // One unit: scores of the wave's row blocks, softmax against the lazily updated
-    // references, second product.  Returns false, having only noted the maxima, when some row's
-    // scores outgrow its reference: the caller rescales and repeats the unit.
-    auto compute = [&](int buf, int base, bool packed, int full) -> bool {
-        f32x4 S[PR_RB][2];
+    // references (raised in place, with the accumulators rescaled, when some row's scores
+    // outgrow its reference), second product.
+    auto compute = [&](int buf, int base, bool packed, int full) {
+        // the key tile's operands first, then four independent accumulator chains side by side
+        f16x8 A[2][4];
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             const f16 *kr = &s_k[buf][pf_krow(pf_tok(n >> 2, n & 3, T)) * PF_KSTRIDE + 8 * blk];
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const f16x8 A = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
+            for (int ks = 0; ks < 4; ++ks) A[T][ks] = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
+        }
+        f32x4 S[PR_RB][2];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
 #pragma unroll
                 for (int rb = 0; rb < PR_RB; ++rb)
-                    S[rb][T] = VQ_MFMA(A, qn[rb][ks], ks == 0 ? (f32x4{0.f, 0.f, 0.f, 0.f}) : S[rb][T]);
-            }
-        }
+                    S[rb][T] = VQ_MFMA(A[T][ks], qn[rb][ks], ks == 0 ? (f32x4{0.f, 0.f, 0.f, 0.f}) : S[rb][T]);
+        // the value tile's operands are on their way while the softmax runs
+        f16x8 Bv[8];
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt)
+            Bv[nt] = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
         bool grow = false;
 #pragma unroll
         for (int rb = 0; rb < PR_RB; ++rb) {
@@ -628,7 +637,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             m_seen[rb] = mx * c;
             grow |= mx * c > m_run[rb] + RESCALE_SLACK;
         }
-        if (__any(grow)) return false;
+        if (__any(grow)) rescale();
         f16x8 P8[PR_RB];
 #pragma unroll
         for (int rb = 0; rb < PR_RB; ++rb) {
@@ -641,17 +650,14 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             P8[rb] = as_h8(P[0], P[1], P[2], P[3]);
         }
 #pragma unroll
-        for (int nt = 0; nt < 8; ++nt) {
-            const f16x8 Bv = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+        for (int nt = 0; nt < 8; ++nt)
 #pragma unroll
-            for (int rb = 0; rb < PR_RB; ++rb) O[rb][nt] = VQ_MFMA(P8[rb], Bv, O[rb][nt]);
-        }
+            for (int rb = 0; rb < PR_RB; ++rb) O[rb][nt] = VQ_MFMA(P8[rb], Bv[nt], O[rb][nt]);
 #pragma unroll
         for (int rb = 0; rb < PR_RB; ++rb) L[rb] = VQ_MFMA(P8[rb], ones, L[rb]);
-        return true;
     };
 
-    // ---- pipeline over the work units [w0, w1), as in the kernel above
+    // ---- pipeline over the work units [w0, w1): unit w+1 is unpacked and unit w+2 requested while unit w is computed
     Stage st;
     if (w1 > w0) {
         fetch(w0, st);
@@ -659,23 +665,14 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         __syncthreads();
         if (w0 + 1 < w1) fetch(w0 + 1, st);
     }
-    bool staged = false;   // unit w+1 already unpacked (set while a unit is being repeated)
-    for (int w = w0; w < w1;) {
+    for (int w = w0; w < w1; ++w) {
         const int buf = (w - w0) & 1;
-        if (!staged) {
-            if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
-            if (w + 2 < w1) fetch(w + 2, st);
-            staged = true;
-        }
+        if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
+        if (w + 2 < w1) fetch(w + 2, st);
         const bool packed = w < n_punits;
         const int base = packed ? w * 32 : (w - n_punits) * 32;
-        if (!compute(buf, base, packed, packed ? full_vis : full_tvis)) {
-            rescale();
-            continue;
-        }
+        compute(buf, base, packed, packed ? full_vis : full_tvis);
         __syncthreads();
-        staged = false;
-        ++w;
     }
 
     // ---- every wave owns its rows: accumulator register r of lane (n, blk) is row 4 blk + r of the
