@@ -229,3 +229,97 @@ class KiviCacheModel:
             self.tokens_seen = max(0, self.tokens_seen - n)
             self.residual_fp16_bytes = (self.offset - self.n_quantized) * D * 2 * 2 * H * B
         return n
+
+
+class SinkCacheModel(KiviCacheModel):
+    """numpy model of ``SinkProtectedKVCache`` (cache/sink_cache.py:62-225): KIVI with the
+    ``n_sink`` highest-key-norm token positions of every batch element kept in fp16.  The
+    selection signal is the key L2 norm averaged over kv heads (``:97-110``), a running top-k per
+    batch element (``:105-110``); inside a block that is being quantised a sink row is replaced
+    by its nearest non-sink neighbour of the same batch element before the group parameters are
+    computed (``:146-175``) and restored to its fp16 value afterwards (``:178-186``)."""
+
+    def __init__(self, bits=2, group_size=32, residual_length=128, n_sink=5):
+        super().__init__(bits, group_size, residual_length)
+        self.n_sink = n_sink
+        self.sink_norms: list[dict[int, float]] = []
+        self.sink_fp16_bytes = 0
+
+    def _update_sinks(self, keys, start):
+        B = keys.shape[0]
+        while len(self.sink_norms) < B:
+            self.sink_norms.append({})
+        if self.n_sink == 0:
+            return [set() for _ in range(B)]
+        per_tok = np.sqrt((keys.astype(F32) ** 2).sum(-1, dtype=F32)).mean(axis=1)   # [B, S]
+        for b in range(B):
+            d = self.sink_norms[b]
+            for i, v in enumerate(per_tok[b].tolist()):
+                d[start + i] = float(v)
+            if len(d) > self.n_sink:
+                self.sink_norms[b] = dict(sorted(d.items(), key=lambda kv: -kv[1])[: self.n_sink])
+        return [set(self.sink_norms[b]) for b in range(B)]
+
+    @staticmethod
+    def neighbour(idx, sink_set, n):
+        """Row that stands in for sink row ``idx`` of an ``n``-row block, or None (:160-171)."""
+        src = idx - 1
+        while src in sink_set and src > 0:
+            src -= 1
+        if src < 0 or src in sink_set:
+            src = idx + 1
+            while src in sink_set and src < n - 1:
+                src += 1
+        return src if 0 <= src < n and src not in sink_set else None
+
+    def update_and_fetch(self, keys, values):
+        B, H, S, D = keys.shape
+        self.shape_bhd = (B, H, D)
+        start = self.offset
+        sinks = self._update_sinks(keys, start)
+        if self.keys is None:
+            self.keys, self.values = keys.copy(), values.copy()
+        else:
+            self.keys = np.concatenate([self.keys[:, :, : self.offset], keys], axis=2)
+            self.values = np.concatenate([self.values[:, :, : self.offset], values], axis=2)
+        self.offset += S
+        nb = quantization_boundary(self.offset, self.R, self.g)
+        n_now = nb - self.n_quantized
+        n_sink_in_block = 0
+        if n_now > 0:
+            lo, hi = self.n_quantized, nb
+            k_reg, v_reg = self.keys[:, :, lo:hi].copy(), self.values[:, :, lo:hi].copy()
+            local = [sorted(p - lo for p in sinks[b] if lo <= p < hi) for b in range(B)]
+            for b in range(B):
+                ss = set(local[b])
+                for idx in local[b]:
+                    src = self.neighbour(idx, ss, n_now)
+                    if src is not None:
+                        k_reg[b, :, idx] = self.keys[b, :, lo + src]
+                        v_reg[b, :, idx] = self.values[b, :, lo + src]
+            k_q = quant_dequant_along(k_reg, -2, self.g, self.levels)
+            v_q = quant_dequant_along(v_reg, -1, self.g, self.levels)
+            for b in range(B):
+                n_sink_in_block = max(n_sink_in_block, len(local[b]))
+                for idx in local[b]:
+                    k_q[b, :, idx] = self.keys[b, :, lo + idx]
+                    v_q[b, :, idx] = self.values[b, :, lo + idx]
+            self.keys[:, :, lo:hi] = k_q
+            self.values[:, :, lo:hi] = v_q
+            self.n_quantized = nb
+        n_comp = n_now - n_sink_in_block
+        if n_comp > 0:
+            k, v = quantized_bytes(n_comp, B, H, D, self.bits, self.g)
+            self.key_bytes_compressed += k
+            self.value_bytes_compressed += v
+        self.sink_fp16_bytes += n_sink_in_block * D * 2 * 2 * H * B
+        self.residual_fp16_bytes = (self.offset - self.n_quantized) * D * 2 * 2 * H * B
+        self.key_bytes_fp16 += H * B * S * D * 2
+        self.value_bytes_fp16 += H * B * S * D * 2
+        self.tokens_seen += S
+        return self.keys[:, :, : self.offset], self.values[:, :, : self.offset]
+
+    def sink_positions_for(self, b):
+        if b >= len(self.sink_norms):
+            return []
+        return [p for p, _ in sorted(self.sink_norms[b].items(), key=lambda kv: -kv[1])]

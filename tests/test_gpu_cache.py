@@ -196,6 +196,44 @@ def test_packed_state_round_trip_and_prompt_cache_file(mode, bits, g, layout, tm
         K.attend_fixed_order(False)
 
 
+@pytest.mark.parametrize("n_sink", [0, 3])
+def test_sink_protected_cache_matches_model(n_sink):
+    """method="kivi_sink" (veloxquant_mlx/cache/sink_cache.py): prefill, decode steps and a trim
+    against the numpy model, bit for bit; two sequences with their outliers at different places."""
+    require_gpu()
+    rng = np.random.default_rng(7)
+    B, H, D = 2, 2, 128
+    k = rng.standard_normal((B, H, 330, D)).astype(np.float16)
+    v = rng.standard_normal((B, H, 330, D)).astype(np.float16)
+    k[0, :, 3] *= 25
+    k[1, :, 150] *= 25
+    k[1, :, 310] *= 30
+    c = KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=2, kivi_group_size=32,
+                                            residual_length=64, n_sink_tokens=n_sink))
+    m = ok.SinkCacheModel(2, 32, 64, n_sink)
+    steps = [(0, 200)] + [(s, s + 1) for s in range(200, 260)] + [(260, 330)]
+    for s0, s1 in steps:
+        ko, vo = c.update_and_fetch(to_dev(k[:, :, s0:s1]), to_dev(v[:, :, s0:s1]))
+        km, vm = m.update_and_fetch(k[:, :, s0:s1], v[:, :, s0:s1])
+    assert np.array_equal(host(ko), km) and np.array_equal(host(vo), vm)
+    assert c._n_quantized == m.n_quantized and c.offset == 330
+    for b in range(B):
+        assert c.sink_positions_for(b) == m.sink_positions_for(b)
+    assert c.sink_positions == m.sink_positions_for(0)
+    for name, want in (("compressed_key_bytes", m.key_bytes_compressed), ("compressed_value_bytes", m.value_bytes_compressed),
+                       ("sink_fp16_bytes", m.sink_fp16_bytes), ("residual_fp16_bytes", m.residual_fp16_bytes)):
+        assert getattr(c, name) == want, name
+    if n_sink:
+        assert 3 in c.sink_positions_for(0) and 150 in c.sink_positions_for(1) and 310 in c.sink_positions_for(1)
+        assert np.array_equal(host(ko)[0, :, 3], k[0, :, 3])
+    assert c.trim(100) == 100 and c.offset == 230 and c._n_quantized == (230 // 32) * 32
+    assert all(p < 230 for b in range(B) for p in c.sink_positions_for(b))
+    with pytest.raises(ValueError, match="fused_sdpa"):
+        KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, fused_sdpa=True))
+    with pytest.raises(ValueError, match="n_sink_tokens"):
+        KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, n_sink_tokens=-1))
+
+
 def test_chunked_prefill_through_the_cache_matches_oracle():
     """Quantise-on-write prefill: chunks of 64 through a cache with R=32, g=32."""
     require_gpu()

@@ -232,3 +232,54 @@ def test_cache_model_trim_equals_feeding_kept_tokens():
     # frontier snaps down to a group multiple no larger than the kept length
     assert a.offset == 64 and a.n_quantized == min(88, 64) and a.n_quantized % 8 == 0
     assert a.key_bytes_fp16 == b.key_bytes_fp16 and a.tokens_seen == b.tokens_seen
+
+
+def test_sink_cache_model_pins():
+    """SinkCacheModel (veloxquant_mlx/cache/sink_cache.py:62-256) against what the method fixes:
+    without sinks it is the KIVI model; the protected positions are the brute-force top-k of the
+    head-averaged key norms; protected rows keep their fp16 values; a 25x row no longer sets its
+    group's range (the reference's tests/cache/test_sink_cache.py ask exactly for these:
+    sink rows exact, neighbours better than under plain KIVI, per-batch positions)."""
+    rng = np.random.default_rng(0)
+    k = rng.standard_normal((2, 2, 300, 64)).astype(np.float16)
+    v = rng.standard_normal((2, 2, 300, 64)).astype(np.float16)
+    k[0, :, 17] *= 25
+    k[1, :, 200] *= 25
+    plain = kivi.KiviCacheModel(2, 32, 64)
+    kp, vp = plain.update_and_fetch(k, v)
+    none = kivi.SinkCacheModel(2, 32, 64, n_sink=0)
+    k0, v0 = none.update_and_fetch(k, v)
+    assert np.array_equal(k0, kp) and np.array_equal(v0, vp)
+    assert none.key_bytes_compressed == plain.key_bytes_compressed and none.sink_fp16_bytes == 0
+    m = kivi.SinkCacheModel(2, 32, 64, n_sink=3)
+    ks, vs = m.update_and_fetch(k, v)
+    norms = np.sqrt((k.astype(np.float32) ** 2).sum(-1)).mean(1)
+    for b in range(2):
+        assert sorted(m.sink_positions_for(b)) == sorted(np.argsort(-norms[b])[:3].tolist())
+        for p in m.sink_positions_for(b):
+            if p < m.n_quantized:
+                assert np.array_equal(ks[b, :, p], k[b, :, p]) and np.array_equal(vs[b, :, p], v[b, :, p])
+    # keys are grouped along tokens: the group of token 17 (tokens 0..31) of batch 0
+    err_plain = np.abs(kp[0, :, :32].astype(np.float32) - k[0, :, :32].astype(np.float32))
+    err_sink = np.abs(ks[0, :, :32].astype(np.float32) - k[0, :, :32].astype(np.float32))
+    rows = [t for t in range(32) if t != 17]
+    assert err_sink[:, rows].mean() < 0.25 * err_plain[:, rows].mean()
+    # key groups (32 tokens) that hold no protected row are bit-identical to plain KIVI
+    clean = [g for g in range(m.n_quantized // 32) if not any(g * 32 <= p < g * 32 + 32 for p in m.sink_positions_for(0))]
+    assert len(clean) >= 4
+    for g in clean:
+        assert np.array_equal(ks[0, :, g * 32:g * 32 + 32], kp[0, :, g * 32:g * 32 + 32])
+    # accounting: the sinks inside the quantised region moved from the compressed pool to the fp16 pool
+    n_in = max(sum(1 for p in m.sink_positions_for(b) if p < m.n_quantized) for b in range(2))
+    assert m.sink_fp16_bytes == n_in * 64 * 2 * 2 * 2 * 2
+    kq, vq = kivi.quantized_bytes(m.n_quantized - n_in, 2, 2, 64, 2, 32)
+    assert (m.key_bytes_compressed, m.value_bytes_compressed) == (kq, vq)
+    # the stand-in row: nearest non-sink neighbour, left first
+    nb = kivi.SinkCacheModel.neighbour
+    assert nb(5, {5}, 32) == 4 and nb(0, {0}, 32) == 1 and nb(1, {0, 1}, 32) == 2 and nb(0, {0}, 1) is None
+    # streaming: sinks found in a later block are protected from then on; earlier ones stay
+    st = kivi.SinkCacheModel(2, 32, 64, n_sink=1)
+    for s0 in range(0, 300, 50):
+        st.update_and_fetch(k[:, :, s0:s0 + 50], v[:, :, s0:s0 + 50])
+    assert st.sink_positions_for(0) == [17] and st.sink_positions_for(1) == [200]
+    assert np.array_equal(st.keys[1, :, 200], k[1, :, 200])
