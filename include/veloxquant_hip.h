@@ -194,6 +194,16 @@ typedef struct vq_attend_args {
      * block of every kv head merges the split partials); without them (NULL) a separate
      * merge kernel follows.  Calls sharing counters must not overlap. */
     int32_t *sync_counters;
+    /* Optional, both or neither: per-sequence lengths for a batch whose sequences differ in
+     * length (device arrays of B int32).  Sequence b attends over its first packed_lens[b]
+     * packed tokens (a multiple of 32 and of group, <= n_packed) and its first tail_lens[b]
+     * tail tokens (<= n_tail); n_packed and n_tail are then the maxima over the batch, which
+     * size the launch.  With causal != 0 the queries of sequence b align to the end of its own
+     * tokens.  No counterpart in the reference, whose caches carry one offset for the batch
+     * (variable-length batches are the integration it scoped and left open,
+     * docs/KV_KERNEL_ROOFLINE_FINDINGS.md:963-973). */
+    const int32_t *packed_lens;
+    const int32_t *tail_lens;
 } vq_attend_args;
 
 /* The decode kernel balances its waves by handing out token chunks on demand, so the order in

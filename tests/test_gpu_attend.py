@@ -329,3 +329,64 @@ def test_mfma_prefill_lds_kernel_shapes(Hq, Hkv, b, g, meta):
     path = 2 if meta == torch.float16 else 1   # float32 scale / zero stays on the 8-row tiles
     _packed_case(1, Hq, Hkv, 384, 45, 128, b, g, "token", meta, Sq=100, causal=True, seed=Hq + b + g, expect_path=path)
     _packed_case(1, Hq, Hkv, 384, 0, 128, b, g, "token", meta, Sq=16, causal=False, seed=Hq + b + g + 1, expect_path=path)
+
+
+# ------------------------------------------------- sequences of different lengths in one batch
+@pytest.mark.parametrize("Sq,causal,v_layout,num_splits", [(1, False, "token", 0), (1, False, "token", 3), (5, True, "token", 0),
+                                                           (40, True, "token", 0), (80, True, "token", 0), (1, False, "channel", 0),
+                                                           (1, False, "token", -1)])
+def test_ragged_batch_per_sequence_lengths(Sq, causal, v_layout, num_splits):
+    """packed_lens / tail_lens: every sequence attends over its own prefix of the shared buffers
+    (and, causal, aligns its queries to its own end).  Each sequence is checked against the
+    oracle run on that sequence alone; decode tiles, both prefill kernels and the vector kernel."""
+    require_gpu()
+    B, Hq, Hkv, D, b, g = 4, 8, 2, 128, 4, 32
+    NP, NT = 384, 48
+    per = 32 // b
+    p_lens, t_lens = [384, 128, 256, 96], [48, 0, 17, 33]
+    k, v = outlier_kv((B, Hkv, NP + NT, D), seed=Sq + 2)
+    q = np.random.default_rng(Sq).standard_normal((B, Hq, Sq, D)).astype(np.float16)
+    kt, vt = to_dev(k), to_dev(v)
+    dev = "cuda:0"
+    kp = torch.zeros((B, Hkv, NP, D // per), dtype=torch.int32, device=dev)
+    ks = torch.zeros((B, Hkv, NP // g, D), dtype=torch.float16, device=dev)
+    kz = torch.zeros_like(ks)
+    if v_layout == "token":
+        vp = torch.zeros((B, Hkv, NP // per, D), dtype=torch.int32, device=dev)
+        vs = torch.zeros((B, Hkv, D // g, NP), dtype=torch.float16, device=dev)
+    else:
+        vp = torch.zeros((B, Hkv, NP, D // per), dtype=torch.int32, device=dev)
+        vs = torch.zeros((B, Hkv, NP, D // g), dtype=torch.float16, device=dev)
+    vz = torch.zeros_like(vs)
+    K.kivi_quant_pack(kt[:, :, :NP], -2, g, b, out=(kp, ks, kz))
+    K.kivi_quant_pack(vt[:, :, :NP], -1, g, b, v_layout=v_layout, out=(vp, vs, vz))
+    # the tail rows of sequence s are the tokens that follow ITS packed prefix
+    tk = torch.zeros((B, Hkv, 64, D), dtype=torch.float16, device=dev)
+    tv = torch.zeros_like(tk)
+    for s in range(B):
+        tk[s, :, :t_lens[s]] = kt[s, :, p_lens[s]:p_lens[s] + t_lens[s]]
+        tv[s, :, :t_lens[s]] = vt[s, :, p_lens[s]:p_lens[s] + t_lens[s]]
+    plan = {}
+    out = K.kivi_packed_attend(to_dev(q), n_packed=NP, bits=b, group_size=g, v_layout=v_layout, k_packed=kp, k_scale=ks,
+                               k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz, k_tail=tk, v_tail=tv, n_tail=NT,
+                               scale=0.09, causal=causal, out_dtype=torch.float32, num_splits=num_splits,
+                               packed_lens=torch.tensor(p_lens, dtype=torch.int32, device=dev),
+                               tail_lens=torch.tensor(t_lens, dtype=torch.int32, device=dev), _plan_out=plan)
+    rows256 = plan["path"] == 2 and (Hq // Hkv) * Sq >= 256
+    levels = (1 << b) - 1
+    worst = 0.0
+    for s in range(B):
+        n, t = p_lens[s], t_lens[s]
+        kq = ok.group_quant_codes(k[s:s + 1, :, :n], -2, g, levels)
+        vq = ok.group_quant_codes(v[s:s + 1, :, :n], -1, g, levels)
+        f = np.float16
+        ref = oa.kivi_attend(q[s:s + 1], kq[0], kq[1].astype(f), kq[2].astype(f), vq[0], vq[1].astype(f), vq[2].astype(f), g,
+                             k[s:s + 1, :, n:n + t], v[s:s + 1, :, n:n + t], 0.09, causal=causal,
+                             recon_dtype=np.float16 if rows256 else None)
+        worst = max(worst, float(np.max(np.abs(host(out)[s:s + 1] - ref))))
+    print(f"path {plan['path']}, worst max-abs err {worst:.2e}")
+    assert worst < TOL
+    assert int(K._counters(to_dev(q).device).abs().sum()) == 0
+    with pytest.raises(ValueError, match="go together"):
+        K.kivi_packed_attend(to_dev(q), n_packed=NP, bits=b, group_size=g, v_layout=v_layout, k_packed=kp, k_scale=ks, k_zero=kz,
+                             v_packed=vp, v_scale=vs, v_zero=vz, scale=0.09, packed_lens=torch.tensor(p_lens, device=dev))

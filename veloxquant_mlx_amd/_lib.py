@@ -36,6 +36,7 @@ class AttendArgs(C.Structure):
         ("scale", f32), ("causal", i32), ("num_splits", i32),
         ("workspace", vp), ("workspace_bytes", sz), ("stream", vp),
         ("sync_counters", vp),
+        ("packed_lens", vp), ("tail_lens", vp),
     ]
 
 

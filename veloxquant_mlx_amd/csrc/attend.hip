@@ -125,6 +125,8 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a) {
         VQ_REQUIRE(a->k_packed && a->v_packed && a->k_scale && a->k_zero && a->v_scale && a->v_zero, VQ_ERR_INVALID,
                    "%s: null packed-cache pointer", fn);
     if (a->n_tail > 0) VQ_REQUIRE(a->k_tail && a->v_tail, VQ_ERR_INVALID, "%s: null tail pointer", fn);
+    VQ_REQUIRE((a->packed_lens == nullptr) == (a->tail_lens == nullptr), VQ_ERR_INVALID,
+               "%s: packed_lens and tail_lens go together", fn);
     AttendPlan p = plan_attend(*a);
     size_t need = vq_kivi_attend_workspace(a);
     VQ_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, VQ_ERR_WORKSPACE,

@@ -4,6 +4,15 @@
 
 namespace vq {
 
+// a batch whose sequences differ in length: the block's copy of the arguments takes the lengths
+// of its own sequence
+__device__ __forceinline__ void take_sequence_lengths(vq_attend_args &a, int64_t b) {
+    if (a.packed_lens != nullptr) {
+        a.n_packed = a.packed_lens[b];
+        a.n_tail = a.tail_lens[b];
+    }
+}
+
 struct AttendPlan {
     int path;           // 0 generic waves, 1 MFMA decode (row tiles of <= 8), 2 MFMA prefill (LDS-staged, 64-row blocks)
     int nsplit;         // splits along the tokens the main kernel covers

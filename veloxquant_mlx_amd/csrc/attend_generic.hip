@@ -41,6 +41,7 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(vq_attend_args a, i
     const int sp = (int)(wid % nsplit);
     const int64_t iq = row % a.Sq, h = (row / a.Sq) % a.Hq, b = row / (a.Sq * a.Hq);
     const int64_t hpk = a.Hq / a.Hkv, bh = b * a.Hkv + h / hpk;
+    take_sequence_lengths(a, b);
     const int64_t D = a.D, n_total = a.n_packed + a.n_tail;
     const int64_t last = a.causal ? (n_total - a.Sq + iq) : (n_total - 1);
     int64_t t0 = (int64_t)sp * split_len, t1 = t0 + split_len;

@@ -628,6 +628,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int sp = (int)blockIdx.x, nsplit = (int)gridDim.x;
     const int64_t bh = by / tiles;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    take_sequence_lengths(a, b);
     const float c = a.scale * LOG2E;
 
     RowTile tile;
@@ -644,7 +645,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     // the raw query is staged in the (not yet used) output exchange buffer
     f16 *s_qraw = reinterpret_cast<f16 *>(&s_o[0][0][0]);
     build_query_image<BITS>(a, tile, tid, s_qraw, s_q);
-    if (sp == 0 && a.n_tail > 0)
+    if (sp == 0 && nparts > nsplit)   // the launch has a tail slot: filled even when this sequence's tail is empty
         tail_block<PK_WAVES>(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid,
                              wave, single_launch);
 

@@ -103,6 +103,7 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     const int n = lane & 15, blk = lane >> 4;
     const int64_t bh = blockIdx.y;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    take_sequence_lengths(a, b);
     const int R = (int)(a.Hq / a.Hkv);
     const int64_t cap = a.cap_tokens;
     const float c = a.scale * LOG2E;
@@ -452,6 +453,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int n = lane & 15, blk = lane >> 4;
     const int64_t bh = blockIdx.y;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    take_sequence_lengths(a, b);
     const int R = (int)(a.Hq / a.Hkv);
     const int64_t cap = a.cap_tokens;
     const float c = a.scale * LOG2E;

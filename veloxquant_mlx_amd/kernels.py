@@ -533,7 +533,8 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
                        v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
                        scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
-                       num_splits: int = 0, _plan_out: dict | None = None,
+                       num_splits: int = 0, packed_lens: torch.Tensor | None = None,
+                       tail_lens: torch.Tensor | None = None, _plan_out: dict | None = None,
                        _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
@@ -598,6 +599,16 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
+    if (packed_lens is None) != (tail_lens is None):
+        raise ValueError(f"{name}: packed_lens and tail_lens go together")
+    if packed_lens is not None:
+        # sequences of different lengths: int32 [B] on the device; n_packed / n_tail are the maxima
+        lens = []
+        for nm, t in (("packed_lens", packed_lens), ("tail_lens", tail_lens)):
+            if t.shape != (B,) or not t.is_cuda:
+                raise ValueError(f"{name}: {nm} must be a device tensor of shape [{B}]")
+            lens.append(t.to(torch.int32).contiguous())
+        a.packed_lens, a.tail_lens = lens[0].data_ptr(), lens[1].data_ptr()
     lib = _lib.load()
     if _plan_out is not None:
         import ctypes
