@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the KV-cache compression hot path on one MI355X.
 
-Headline workload (BASELINE.json configs[3], the "@32k ctx" decode the metric is
+Headline workload (configuration 3 of the benchmark set, the "@32k ctx" decode the metric is
 quoted on): Qwen3-8B shape, 36 layers, 32 query / 8 kv heads, D=128, batch 16,
 32768 tokens of context per sequence stored as 4-bit packed KIVI codes (keys per
 channel, values per token, group 64) plus an fp16 tail.  One step = one decode

@@ -252,7 +252,7 @@ def test_chunked_prefill_through_the_cache_matches_oracle():
 
 
 def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
-    """BASELINE configs[4]: 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
+    """Benchmark configuration 4: 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
     tokens plus their own tokens (32 query / 8 kv heads, D=128, group 32, residual 128).  The
     oracle is too slow at this size, so the two independent GPU implementations (each checked
     against the oracle at small sizes) are compared on the chunks with the shortest and the
@@ -294,7 +294,7 @@ def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
 
 
 def test_config3_decode_at_full_size_against_the_oracle_and_the_vector_kernel():
-    """BASELINE configs[3], one layer: batch 16, 32 query / 8 kv heads, D=128, 32768 tokens of
+    """Benchmark configuration 3, one layer: batch 16, 32 query / 8 kv heads, D=128, 32768 tokens of
     context in a 4-bit group-64 packed cache plus the fp16 residual, one query token.  The last
     sequence is checked against the scalar C oracle (about a second of CPU), every sequence
     against the independent vector kernel."""
