@@ -204,6 +204,15 @@ typedef struct vq_attend_args {
      * docs/KV_KERNEL_ROOFLINE_FINDINGS.md:963-973). */
     const int32_t *packed_lens;
     const int32_t *tail_lens;
+    /* Optional, both or neither: the newest token's key and value rows, [B, Hkv, D] contiguous in
+     * tail_dtype, 16-byte aligned.  The call first stores them as the LAST of the n_tail tail rows
+     * (row n_tail - 1, or tail_lens[b] - 1) and attends over them from these buffers, so a decode
+     * step appends and attends in one launch.  Single-query MFMA decode path only (Sq == 1, what
+     * vq_kivi_attend_plan reports as path 1); VQ_ERR_UNSUPPORTED otherwise -- append with
+     * vq_kv_tail_append first.  Stands for the concatenation in KIVIKVCache.update_and_fetch
+     * (cache/kivi_cache.py:206-260) followed by the attention call of the same step. */
+    const void *k_new;
+    const void *v_new;
 } vq_attend_args;
 
 /* The decode kernel balances its waves by handing out token chunks on demand, so the order in

@@ -447,3 +447,52 @@ def test_vecinfer_max_ctx_cap():
     c.update_and_fetch(to_dev(k), to_dev(v))
     with pytest.raises(RuntimeError, match="exceeded fused_sdpa_max_ctx=100"):
         c.update_and_fetch(to_dev(k[:, :, :20]), to_dev(v[:, :, :20]))
+
+
+def test_decode_steps_store_the_new_token_in_the_attention_launch():
+    """Memory-bound decode: a step with no flush due hands the new token to the attention launch
+    (vq_attend_args.k_new / v_new), which stores it in the tail and attends in one go.  Sixty
+    steps against the cache model + oracle, across two flushes, with a state read, a trim and a
+    two-token step in between; the tail must hold every token afterwards."""
+    require_gpu()
+    B, Hq, Hkv, D, g, R = 2, 8, 2, 128, 32, 64
+    k, v = outlier_kv((B, Hkv, 400, D), seed=21)
+    rng = np.random.default_rng(3)
+    c = _make(bit_width_inlier=4, kivi_group_size=g, residual_length=R, fused_sdpa=True, fused_sdpa_memory_bound=True)
+    c.update_and_fetch(to_dev(k[:, :, :300]), to_dev(v[:, :, :300]))
+    deferred = 0
+    pos = 300
+    levels = 15
+    for step in range(60):
+        n_new = 2 if step == 17 else 1
+        c.update_and_fetch(to_dev(k[:, :, pos:pos + n_new]), to_dev(v[:, :, pos:pos + n_new]))
+        pos += n_new
+        deferred += c._pending is not None
+        if step == 23:
+            st = c.state            # reading the state stores the token first
+            assert c._pending is None and st[-1].shape[2] == c.offset - c._n_quantized
+            assert np.array_equal(host(st[-2][:, :, -1]), k[:, :, pos - 1])
+        if step == 31:
+            assert c.trim(3) == 3
+            pos -= 3
+        q = rng.standard_normal((B, Hq, 1, D)).astype(np.float16)
+        out = host(c.fused_sdpa(to_dev(q), 0.09)).astype(np.float32)
+        assert c._pending is None and c.offset == pos
+        nq = c._n_quantized
+        assert nq == ((pos - R) // g) * g
+        kq = ok.group_quant_codes(k[:, :, :nq], -2, g, levels)
+        vq = ok.group_quant_codes(v[:, :, :nq], -1, g, levels)
+        f = np.float16
+        ref = oa.kivi_attend(q, kq[0], kq[1].astype(f), kq[2].astype(f), vq[0], vq[1].astype(f), vq[2].astype(f), g,
+                             k[:, :, nq:pos], v[:, :, nq:pos], 0.09)
+        assert np.max(np.abs(out - ref)) < 2e-3, step
+        n_tail = pos - nq
+        assert np.array_equal(host(c._tail_k[:, :, :n_tail]), k[:, :, nq:pos]), step
+        assert np.array_equal(host(c._tail_v[:, :, :n_tail]), v[:, :, nq:pos]), step
+    assert deferred >= 50   # all but the flush steps, the two-token step and the one after the trim... took the fused path
+    # the kernel refuses the pair where it cannot take it
+    with pytest.raises(ValueError, match="k_new"):
+        K.kivi_packed_attend(to_dev(rng.standard_normal((B, Hq, 4, D)).astype(np.float16)), k_packed=c._kp, k_scale=c._ks,
+                             k_zero=c._kz, v_packed=c._vp, v_scale=c._vs, v_zero=c._vz, n_packed=c._n_quantized, bits=4,
+                             group_size=g, v_layout="token", k_tail=c._tail_k, v_tail=c._tail_v, n_tail=8, scale=0.1,
+                             k_new=to_dev(k[:, :, :1]), v_new=to_dev(v[:, :, :1]))

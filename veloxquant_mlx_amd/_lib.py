@@ -37,6 +37,7 @@ class AttendArgs(C.Structure):
         ("workspace", vp), ("workspace_bytes", sz), ("stream", vp),
         ("sync_counters", vp),
         ("packed_lens", vp), ("tail_lens", vp),
+        ("k_new", vp), ("v_new", vp),
     ]
 
 

@@ -109,6 +109,9 @@ class KIVIKVCache(FP16KVCache):
         # fp16 tail (memory-bound mode): tokens [_n_quantized, offset)
         self._tail_k = self._tail_v = None
         self._tail_spare = None   # second pair of tail buffers the kept rows move into at a flush
+        # memory-bound decode: the newest token's (keys, values), counted in ``offset`` but not yet in the
+        # tail; the next fused_sdpa stores them in the same launch that attends, anything else stores them first
+        self._pending = None
         self._zero_scalar = None
 
     # ------------------------------------------------------------------
@@ -198,10 +201,32 @@ class KIVIKVCache(FP16KVCache):
         self._account_bytes(B, H, S, D, n_quant_now)
         return k_all, v_all
 
+    def _store_pending(self) -> None:
+        """Write a deferred newest token into the tail (see ``_pending``)."""
+        if self._pending is not None:
+            k, v = self._pending
+            self._pending = None
+            K.kv_tail_append(k, v, self._tail_k, self._tail_v, self.offset - self._n_quantized - 1)
+
     def _update_memory_bound(self, keys: torch.Tensor, values: torch.Tensor):
         B, H, S, D = keys.shape
+        self._store_pending()
         n_tail = self.offset - self._n_quantized
         need = n_tail + S
+        if (S == 1 and self._n_quantized > 0 and self._tail_k is not None and need <= self._tail_k.shape[2]
+                and keys.dtype == self._tail_k.dtype and values.dtype == keys.dtype and D == 128
+                and keys.is_contiguous() and values.is_contiguous() and keys.data_ptr() % 16 == 0
+                and values.data_ptr() % 16 == 0
+                and (max(0, self.offset + 1 - self._residual_length) // self._group_size) * self._group_size
+                == self._n_quantized):
+            # a plain decode step with no flush due: the attention launch of this step stores the token
+            self._pending = (keys, values)
+            self.offset += 1
+            self._account_bytes(B, H, S, D, 0)
+            z = self._zero_scalar
+            if z is None or z.dtype != keys.dtype or z.device != keys.device:
+                z = self._zero_scalar = torch.zeros((), dtype=keys.dtype, device=keys.device)
+            return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
         if self._tail_k is None or need > self._tail_k.shape[2]:
             cap = max(need, self._residual_length + 2 * self._group_size)
             cap = -(-cap // 64) * 64
@@ -259,15 +284,24 @@ class KIVIKVCache(FP16KVCache):
             raise ValueError("KIVIKVCache.fused_sdpa: sliding_window attention is not supported")
         nq = self._n_quantized
         n_tail = self.offset - nq
+        if self._pending is not None and q.shape[2] != 1:
+            self._store_pending()
         if self._memory_bound:
             tk, tv = self._tail_k, self._tail_v
         else:
             tk, tv = self.keys[:, :, nq:], self.values[:, :, nq:]
-        return K.kivi_packed_attend(
-            q, k_packed=self._kp, k_scale=self._ks, k_zero=self._kz, v_packed=self._vp, v_scale=self._vs,
-            v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
-            k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
-            causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype)
+        kw = dict(k_packed=self._kp, k_scale=self._ks, k_zero=self._kz, v_packed=self._vp, v_scale=self._vs,
+                  v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
+                  k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
+                  causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype)
+        if self._pending is not None:
+            try:   # append and attend in one launch (single-query MFMA decode path)
+                out = K.kivi_packed_attend(q, k_new=self._pending[0], v_new=self._pending[1], **kw)
+                self._pending = None
+                return out
+            except ValueError:   # a shape that path does not take: store the token, then attend
+                self._store_pending()
+        return K.kivi_packed_attend(q, **kw)
 
     # ------------------------------------------------------------------ trim / state
     def _rollback_frontier(self, new_offset: int) -> int:
@@ -292,6 +326,7 @@ class KIVIKVCache(FP16KVCache):
     def trim(self, n: int) -> int:
         """Drop the last ``n`` tokens and roll frontier and accounting back (kivi_cache.py:293-299)."""
         old_nq = self._n_quantized
+        self._store_pending()
         trimmed = super().trim(n)
         if trimmed:
             n_rolled = self._rollback_frontier(self.offset)
@@ -327,6 +362,7 @@ class KIVIKVCache(FP16KVCache):
         rows).  Memory-bound mode: live packed rows followed by the live fp16 tail."""
         if not self._fused_enabled:
             return FP16KVCache.state.fget(self)
+        self._store_pending()
         packed = self._packed_state()
         if not self._memory_bound:
             return (*FP16KVCache.state.fget(self), *packed)
@@ -350,6 +386,7 @@ class KIVIKVCache(FP16KVCache):
         """Inverse of the getter, mode by mode.  The frontier comes from the packed rows' own
         length; byte accounting is rebuilt for the restored token count."""
         v = tuple(v)
+        self._pending = None
         if not self._fused_enabled:
             FP16KVCache.state.fset(self, v)
             if v:

@@ -127,7 +127,16 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a) {
     if (a->n_tail > 0) VQ_REQUIRE(a->k_tail && a->v_tail, VQ_ERR_INVALID, "%s: null tail pointer", fn);
     VQ_REQUIRE((a->packed_lens == nullptr) == (a->tail_lens == nullptr), VQ_ERR_INVALID,
                "%s: packed_lens and tail_lens go together", fn);
+    VQ_REQUIRE((a->k_new == nullptr) == (a->v_new == nullptr), VQ_ERR_INVALID, "%s: k_new and v_new go together", fn);
+    if (a->k_new != nullptr) {
+        VQ_REQUIRE(a->n_tail >= 1, VQ_ERR_INVALID, "%s: k_new / v_new fill the last tail row, so n_tail must be >= 1", fn);
+        VQ_REQUIRE((((uintptr_t)a->k_new | (uintptr_t)a->v_new) & 15u) == 0, VQ_ERR_UNSUPPORTED,
+                   "%s: k_new / v_new must be 16-byte aligned", fn);
+    }
     AttendPlan p = plan_attend(*a);
+    if (a->k_new != nullptr)
+        VQ_REQUIRE(p.path == 1 && a->Sq == 1, VQ_ERR_UNSUPPORTED,
+                   "%s: k_new / v_new need the single-query MFMA decode path; append with vq_kv_tail_append first", fn);
     size_t need = vq_kivi_attend_workspace(a);
     VQ_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, VQ_ERR_WORKSPACE,
                "%s: workspace of %zu bytes required, %zu given", fn, need, a->workspace_bytes);

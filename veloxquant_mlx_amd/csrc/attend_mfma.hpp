@@ -281,21 +281,30 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
     const int n_tu = (int)((a.n_tail + 31) / 32);
 
     struct TUnit { f16x8 kr[2][4], vr[8]; };
+    // the newest token's rows, when the call brings them, are read from where the caller holds
+    // them (row n_tail - 1 of the tail is being written by this block at the same time)
+    const int64_t newest = a.k_new != nullptr ? a.n_tail - 1 : -1;
+    auto key_row = [&](int64_t tok, int64_t col) {
+        if (tok >= a.n_tail) tok = 0;
+        return tok == newest ? ld_tail8(a.k_new, bh * MF_D + col, bf16) : ld_tail8(a.k_tail, tbase + tok * MF_D + col, bf16);
+    };
+    auto value_row = [&](int64_t tok, int64_t col) {
+        if (tok >= a.n_tail) tok = 0;
+        return tok == newest ? ld_tail8(a.v_new, bh * MF_D + col, bf16) : ld_tail8(a.v_tail, tbase + tok * MF_D + col, bf16);
+    };
     // every load of a unit is issued before its first product; clamped rows are masked below
     auto load = [&](int u, TUnit &d) {
         const int64_t base = (int64_t)u * 32;
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             const int64_t tok = base + tail_tok(i >> 2, i & 3, T);
-            const int64_t e = tbase + (tok < a.n_tail ? tok : 0) * MF_D + 32 * blk;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) d.kr[T][ks] = ld_tail8(a.k_tail, e + 8 * ks, bf16);
+            for (int ks = 0; ks < 4; ++ks) d.kr[T][ks] = key_row(tok, 32 * blk + 8 * ks);
         }
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            const int64_t tA = base + tail_tok(blk, p, 0), tB = base + tail_tok(blk, p, 1);
-            d.vr[2 * p] = ld_tail8(a.v_tail, tbase + (tA < a.n_tail ? tA : 0) * MF_D + 8 * i, bf16);
-            d.vr[2 * p + 1] = ld_tail8(a.v_tail, tbase + (tB < a.n_tail ? tB : 0) * MF_D + 8 * i, bf16);
+            d.vr[2 * p] = value_row(base + tail_tok(blk, p, 0), 8 * i);
+            d.vr[2 * p + 1] = value_row(base + tail_tok(blk, p, 1), 8 * i);
         }
     };
     auto compute = [&](int u, const TUnit &d) {

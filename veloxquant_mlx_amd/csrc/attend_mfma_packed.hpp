@@ -645,6 +645,15 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     // the raw query is staged in the (not yet used) output exchange buffer
     f16 *s_qraw = reinterpret_cast<f16 *>(&s_o[0][0][0]);
     build_query_image<BITS>(a, tile, tid, s_qraw, s_q);
+    if (sp == 0 && a.k_new != nullptr && a.n_tail >= 1 && tid < 32) {
+        // the newest token's key and value rows become the last tail row: 16 pieces of 16 bytes each
+        const int piece = tid & 15;
+        const bool val = tid >= 16;
+        const uint4 *src = reinterpret_cast<const uint4 *>(val ? a.v_new : a.k_new) + bh * (MF_D / 8) + piece;
+        uint4 *dst = reinterpret_cast<uint4 *>(const_cast<void *>(val ? a.v_tail : a.k_tail)) +
+                     (bh * a.tail_cap + a.n_tail - 1) * (MF_D / 8) + piece;
+        *dst = *src;
+    }
     if (sp == 0 && nparts > nsplit)   // the launch has a tail slot: filled even when this sequence's tail is empty
         tail_block<PK_WAVES>(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid,
                              wave, single_launch);

@@ -534,7 +534,8 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
                        scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
                        num_splits: int = 0, packed_lens: torch.Tensor | None = None,
-                       tail_lens: torch.Tensor | None = None, _plan_out: dict | None = None,
+                       tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
+                       v_new: torch.Tensor | None = None, _plan_out: dict | None = None,
                        _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
@@ -609,6 +610,14 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                 raise ValueError(f"{name}: {nm} must be a device tensor of shape [{B}]")
             lens.append(t.to(torch.int32).contiguous())
         a.packed_lens, a.tail_lens = lens[0].data_ptr(), lens[1].data_ptr()
+    if (k_new is None) != (v_new is None):
+        raise ValueError(f"{name}: k_new and v_new go together")
+    if k_new is not None:
+        # the newest token's rows [B, Hkv, 1, D]: stored as the last tail row and attended in the same launch
+        for nm, t in (("k_new", k_new), ("v_new", v_new)):
+            if k_tail is None or t.dtype != k_tail.dtype or t.numel() != B * Hkv * D or not t.is_contiguous() or not t.is_cuda:
+                raise ValueError(f"{name}: {nm} must be a contiguous [{B}, {Hkv}, 1, {D}] device tensor in the dtype of the tail")
+        a.k_new, a.v_new = k_new.data_ptr(), v_new.data_ptr()
     lib = _lib.load()
     if _plan_out is not None:
         import ctypes
