@@ -143,7 +143,42 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int n = lane & 15, blk = lane >> 4;
     const int ntiles = (nc + 15) / 16;
 
-    for (int i = tid; i < nc * SUB; i += 256) s_cb[i] = ld_any(cb, ct, i);
+    // thread c fetches centroid c with one or two vector loads (the row is 8 to 32 bytes); a
+    // codebook that is not 16-byte aligned goes element by element
+    if ((reinterpret_cast<uintptr_t>(cb) & 15u) == 0) {
+        if (tid < nc) {
+            float row[SUB];
+            if (ct == VQ_F32) {
+#pragma unroll
+                for (int e = 0; e < SUB; e += 4) {
+                    const float4 v = *reinterpret_cast<const float4 *>((const float *)cb + tid * SUB + e);
+                    row[e] = v.x; row[e + 1] = v.y; row[e + 2] = v.z; row[e + 3] = v.w;
+                }
+            } else {
+                u32 w[SUB / 2];
+                if constexpr (SUB == 8) {
+                    const uint4 v = *reinterpret_cast<const uint4 *>((const u16 *)cb + tid * 8);
+                    w[0] = v.x; w[1] = v.y; w[2] = v.z; w[3] = v.w;
+                } else {
+                    const uint2 v = *reinterpret_cast<const uint2 *>((const u16 *)cb + tid * 4);
+                    w[0] = v.x; w[1] = v.y;
+                }
+#pragma unroll
+                for (int e = 0; e < SUB / 2; ++e) {
+                    if (ct == VQ_F16) {
+                        const f16x2 h = __builtin_bit_cast(f16x2, w[e]);
+                        row[2 * e] = (float)h[0]; row[2 * e + 1] = (float)h[1];
+                    } else {
+                        row[2 * e] = __uint_as_float(w[e] << 16); row[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+                    }
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < SUB; ++e) s_cb[tid * SUB + e] = row[e];
+        }
+    } else {
+        for (int i = tid; i < nc * SUB; i += 256) s_cb[i] = ld_any(cb, ct, i);
+    }
     __syncthreads();
     {
         float c2 = 3.0e38f;
@@ -267,16 +302,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             float k1[4], k2[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) { k1[r] = INFINITY; k2[r] = INFINITY; }
+            // four centroid tiles at a time: their products are issued together, so the tracking
+            // of one tile runs while the next product is still in the matrix unit (tiles past the
+            // last centroid of a started group carry zero operands and a huge |c|^2: never chosen)
 #pragma unroll
-            for (int j = 0; j < VM_TILES; ++j) {
-                if (j < ntiles) {
-                    const f32x4 D = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[j], B, C2[j], 0, 0, 0);
+            for (int j4 = 0; j4 < VM_TILES; j4 += 4) {
+                if (j4 < ntiles) {
+                    f32x4 D[4];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) {
-                        const float key = __uint_as_float((__float_as_uint(D[r]) & 0xfffffff0u) | (u32)j);
-                        k2[r] = vmed3(k1[r], k2[r], key);
-                        k1[r] = vmin(k1[r], key);
-                    }
+                    for (int u = 0; u < 4; ++u) D[u] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[j4 + u], B, C2[j4 + u], 0, 0, 0);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const float key = __uint_as_float((__float_as_uint(D[u][r]) & 0xfffffff0u) | (u32)(j4 + u));
+                            k2[r] = vmed3(k1[r], k2[r], key);
+                            k1[r] = vmin(k1[r], key);
+                        }
                 }
             }
             // lane top-2 over its four rows, then over the four lane groups of the column
