@@ -48,6 +48,12 @@ def _parse():
     return p.parse_args()
 
 
+def _side_ms(fn, iters, torch, rounds=3):
+    """Side measurements: median over ``rounds`` of the average milliseconds per call
+    (the reference's own rule is medians, tests/metal/test_kivi_quant.py:297-347)."""
+    return sorted(_event_ms(fn, iters, torch) for _ in range(rounds))[rounds // 2]
+
+
 def _event_ms(fn, iters, torch):
     """Average milliseconds per call, HIP events on the current stream."""
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -203,8 +209,8 @@ def _extras(torch, K, dev):
     for f in (lambda: dst.copy_(src), lambda: big.view(torch.int32).max(), lambda: ga @ gb):
         for _ in range(3):
             f()
-    ms_c, ms_r, ms_g = (_event_ms(lambda: dst.copy_(src), 20, torch), _event_ms(lambda: big.view(torch.int32).max(), 20, torch),
-                        _event_ms(lambda: ga @ gb, 10, torch))
+    ms_c, ms_r, ms_g = (_side_ms(lambda: dst.copy_(src), 20, torch), _side_ms(lambda: big.view(torch.int32).max(), 20, torch),
+                        _side_ms(lambda: ga @ gb, 10, torch))
     ex["measured_ceilings"] = {"copy_GBps": round((2 << 30) / ms_c / 1e6, 1), "read_GBps_library_reduction": round((2 << 30) / ms_r / 1e6, 1),
                                "gemm_f16_TFLOPs": round(2 * 8192 ** 3 / ms_g / 1e9, 1)}
     del src, dst, big, ga, gb
@@ -220,7 +226,7 @@ def _extras(torch, K, dev):
         fn = lambda: c.fused_sdpa(q, 1 / math.sqrt(D))
         for _ in range(3):
             fn()
-        ms = _event_ms(fn, 30, torch)
+        ms = _side_ms(fn, 30, torch)
         nbytes = _algorithmic_bytes_per_layer(B, Hkv, 32768, D, 2, 32)
         ex[f"decode_2bit_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
                                         "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}
@@ -239,7 +245,7 @@ def _extras(torch, K, dev):
         n = k.numel()
         b_qp = 2 * (n * 2 + n // 2 + (n // 32) * 4)
         b_rt = 2 * (n * 2 + n * 2)
-        ms_qp, ms_rt = _event_ms(qp, 30, torch), _event_ms(rt, 30, torch)
+        ms_qp, ms_rt = _side_ms(qp, 30, torch), _side_ms(rt, 30, torch)
         ex[f"quant_pack_{name}"] = {"ms": round(ms_qp, 5), "GBps": round(b_qp / ms_qp / 1e6, 1), "bytes": b_qp}
         ex[f"quant_dequant_{name}"] = {"ms": round(ms_rt, 5), "GBps": round(b_rt / ms_rt / 1e6, 1), "bytes": b_rt}
     # config 4: causal prefill of 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
@@ -276,7 +282,7 @@ def _extras(torch, K, dev):
     fn = lambda: K.vecinfer_quantize_metal(x, cb, 8, index_dtype=torch.uint8)
     for _ in range(3):
         fn()
-    ms = _event_ms(fn, 20, torch)
+    ms = _side_ms(fn, 20, torch)
     flops = 2 * 524288 * 256 * 8
     ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
                             "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
@@ -300,7 +306,7 @@ def _extras(torch, K, dev):
                                       scale=1 / math.sqrt(D), out_dtype=torch.float16)
     for _ in range(2):
         fn()
-    ms = _event_ms(fn, 5, torch)
+    ms = _side_ms(fn, 5, torch)
     nbytes = NL * _algorithmic_bytes_per_layer(Bs, Hkv, ctx, D, 4, g)
     ex["decode_cfg3_36_layers_one_launch"] = {"ms": round(ms, 4), "ms_per_layer": round(ms / NL, 5), "GBps": round(nbytes / ms / 1e6, 1),
                                               "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}
@@ -316,7 +322,7 @@ def _extras(torch, K, dev):
         fn = lambda: K.vecinfer_encode_decode_metal(x4, cb, 8, Hm, sm, index_dtype=torch.uint8, want_k_hat=hat)
         for _ in range(3):
             fn()
-        ms = _event_ms(fn, 20, torch)
+        ms = _side_ms(fn, 20, torch)
         nbytes = x4.numel() * 2 + x4.numel() // 8 + (x4.numel() * 2 if hat else 0)
         ex[f"vq_encode_keys_cfg2_{name}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1), "bytes": nbytes}
     # attention straight from VecInfer indices: 32768 tokens, 8 kv heads x 4 query heads, D 128 in 16
@@ -329,7 +335,7 @@ def _extras(torch, K, dev):
         fn = lambda: K.metal_fused_sdpa(q, ki, kcb, vi, vcb, 1 / math.sqrt(D))
         for _ in range(3):
             fn()
-        ms = _event_ms(fn, 30, torch)
+        ms = _side_ms(fn, 30, torch)
         nbytes = 2 * ki.numel()
         lds_ops = B * Hq * 32768 * 16 * 2 / 64    # one look-up and one histogram addition per row, token and sub-vector, 64 lanes an instruction
         ex[f"index_attend_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1), "bytes": nbytes,
