@@ -107,6 +107,41 @@ int vq_kv_tail_append(const void *k_new, const void *v_new, const int64_t k_stri
                       void *k_tail, void *v_tail, int elem_bytes, int64_t B, int64_t H, int64_t S, int64_t D,
                       int64_t tail_cap, int64_t pos, void *stream);
 
+/* A whole chunk of a packed KIVI cache in one call: the concatenation, the quantisation of
+ * the tokens that aged out of the fp16 residual window and the start of the next tail
+ * (KIVIKVCache.update_and_fetch, veloxquant_mlx/cache/kivi_cache.py:206-262, on packed
+ * buffers).  In stream order:
+ * With n_flush == 0 the call is vq_kv_tail_append: k_new / v_new [B, H, S, D] (strides as
+ * there) go to rows [n_tail, n_tail + S) of the tails [B, H, tail_cap, D].  With n_flush > 0,
+ * of the rows of [tail ; new]
+ *   1. the first n_flush are quantised and packed as tokens [dst_tok0, dst_tok0 + n_flush) of
+ *      the packed store (keys per channel over token groups, values per token over channel
+ *      groups in v_layout; buffers, cap_tokens and the alignment rules are those of
+ *      vq_kivi_quant_pack; new rows among them pass through the tails, which must have room
+ *      for n_tail + S rows), in one launch for keys and values where D == 128, and
+ *   2. the n_tail + S - n_flush rows that stay are written to the front of the spare tails
+ *      [B, H, spare_cap, D], which the caller uses as the tails from then on (the old tails'
+ *      contents are unspecified afterwards).
+ * dtype is the element type of the new tokens and of all four tail buffers. */
+typedef struct vq_kivi_append_args {
+    const void *k_new, *v_new;
+    int64_t k_strides[3], v_strides[3];
+    int dtype;
+    int64_t B, H, S, D;
+    void *k_tail, *v_tail;
+    int64_t tail_cap, n_tail;
+    int64_t n_flush;
+    void *k_packed, *k_scale, *k_zero, *v_packed, *v_scale, *v_zero;
+    int meta_dtype;
+    int64_t cap_tokens, dst_tok0;
+    int group, levels;
+    float eps;
+    int pack_bits, v_layout;
+    void *k_spare, *v_spare;
+    int64_t spare_cap;
+} vq_kivi_append_args;
+int vq_kivi_cache_append(const vq_kivi_append_args *args, void *stream);
+
 /* ---- bit packing ----------------------------------------------------------- */
 
 /* Trailing-axis word packing, idx[rows, D] uint8 <-> words[rows, ceil(D/per)].

@@ -496,3 +496,72 @@ def test_decode_steps_store_the_new_token_in_the_attention_launch():
                              k_zero=c._kz, v_packed=c._vp, v_scale=c._vs, v_zero=c._vz, n_packed=c._n_quantized, bits=4,
                              group_size=g, v_layout="token", k_tail=c._tail_k, v_tail=c._tail_v, n_tail=8, scale=0.1,
                              k_new=to_dev(k[:, :, :1]), v_new=to_dev(v[:, :, :1]))
+
+
+@pytest.mark.parametrize("dtype,bits,group,v_layout,D,n_tail,S,n_flush", [
+    (torch.float16, 4, 32, "token", 128, 128, 512, 512),     # chunked prefill: the new rows split between store and tail
+    (torch.bfloat16, 4, 64, "token", 128, 160, 96, 128),     # the flush stays inside the old tail
+    (torch.bfloat16, 2, 32, "token", 128, 40, 200, 224),     # everything but a few rows leaves
+    (torch.float16, 2, 32, "channel", 128, 0, 256, 256),     # empty tail, nothing kept
+    (torch.float16, 4, 32, "token", 64, 64, 64, 96),         # head size the one-launch kernel does not take
+    (torch.float32, 4, 32, "channel", 128, 32, 64, 64),      # float32 cache
+    (torch.float16, 4, 32, "token", 128, 100, 7, 0),         # plain append
+])
+def test_cache_append_one_call_matches_the_single_steps(dtype, bits, group, v_layout, D, n_tail, S, n_flush):
+    """``vq_kivi_cache_append`` against ``vq_kv_tail_append`` + two ``vq_kivi_quant_pack`` + a row
+    move: packed words, scale, zero and the kept rows bit for bit."""
+    require_gpu()
+    B, H, cap_t, cap_p, tok0 = 2, 3, 768, 1024, 256
+    g = torch.Generator(device="cuda").manual_seed(5)
+    rnd = lambda *s: torch.randn(s, generator=g, device="cuda").to(dtype)
+    tk, tv = rnd(B, H, cap_t, D), rnd(B, H, cap_t, D)
+    kn, vn = rnd(B, H, S + 8, D)[:, :, 3:3 + S], rnd(B, H, S, D)   # the keys a strided view
+    per = 32 // bits
+    meta = torch.float16
+    def store():
+        W, GV = D // per, D // group
+        z = lambda *s, dt=torch.int32: torch.zeros(s, dtype=dt, device="cuda")
+        if v_layout == "token":
+            return [z(B, H, cap_p, W), z(B, H, cap_p // group, D, dt=meta), z(B, H, cap_p // group, D, dt=meta),
+                    z(B, H, cap_p // per, D), z(B, H, GV, cap_p, dt=meta), z(B, H, GV, cap_p, dt=meta)]
+        return [z(B, H, cap_p, W), z(B, H, cap_p // group, D, dt=meta), z(B, H, cap_p // group, D, dt=meta),
+                z(B, H, cap_p, W), z(B, H, cap_p, GV, dt=meta), z(B, H, cap_p, GV, dt=meta)]
+    need, keep = n_tail + S, n_tail + S - n_flush
+    # the single steps
+    t1k, t1v, st1 = tk.clone(), tv.clone(), store()
+    K.kv_tail_append(kn, vn, t1k, t1v, n_tail)
+    if n_flush:
+        K.kivi_quant_pack(t1k[:, :, :n_flush], -2, group, bits, meta_dtype=meta, out=tuple(st1[:3]), dst_tok0=tok0)
+        K.kivi_quant_pack(t1v[:, :, :n_flush], -1, group, bits, meta_dtype=meta, v_layout=v_layout, out=tuple(st1[3:]),
+                          dst_tok0=tok0)
+    # one call
+    t2k, t2v, st2 = tk.clone(), tv.clone(), store()
+    spare = (torch.zeros_like(tk), torch.zeros_like(tv)) if n_flush else None
+    K.kivi_cache_append(kn, vn, t2k, t2v, n_tail, n_flush, st2, tok0, spare, bits=bits, group_size=group,
+                        levels=(1 << bits) - 1, eps=1e-8, v_layout=v_layout)
+    torch.cuda.synchronize()
+    if n_flush:
+        for x, y in zip(st1, st2):
+            assert torch.equal(x, y)
+        assert torch.equal(spare[0][:, :, :keep], t1k[:, :, n_flush:need])
+        assert torch.equal(spare[1][:, :, :keep], t1v[:, :, n_flush:need])
+        assert not spare[0][:, :, keep:].any() and not spare[1][:, :, keep:].any()
+    else:
+        assert torch.equal(t1k, t2k) and torch.equal(t1v, t2v)
+
+
+def test_cache_append_rejects_bad_arguments():
+    require_gpu()
+    z = lambda *s, dt=torch.float16: torch.zeros(s, dtype=dt, device="cuda")
+    tk, tv, kn, vn = z(1, 1, 64, 128), z(1, 1, 64, 128), z(1, 1, 32, 128), z(1, 1, 32, 128)
+    with pytest.raises(ValueError, match="tail capacity"):
+        K.kivi_cache_append(kn, vn, tk, tv, 40, 0, None, 0, None, bits=4, group_size=32, levels=15, eps=1e-8,
+                            v_layout="token")
+    st = [z(1, 1, 64, 16, dt=torch.int32), z(1, 1, 2, 128), z(1, 1, 2, 128), z(1, 1, 8, 128, dt=torch.int32),
+          z(1, 1, 4, 64), z(1, 1, 4, 64)]
+    with pytest.raises(ValueError, match="spare"):   # the spare tails must not be the tails
+        K.kivi_cache_append(kn, vn, tk, tv, 0, 32, st, 0, (tk, tv), bits=4, group_size=32, levels=15, eps=1e-8,
+                            v_layout="token")
+    with pytest.raises(ValueError, match="n_flush"):
+        K.kivi_cache_append(kn, vn, tk, tv, 0, 64, st, 0, (z(1, 1, 64, 128), z(1, 1, 64, 128)), bits=4, group_size=32,
+                            levels=15, eps=1e-8, v_layout="token")

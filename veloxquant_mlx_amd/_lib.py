@@ -56,6 +56,23 @@ class LutAttendArgs(C.Structure):
     ]
 
 
+class KiviAppendArgs(C.Structure):
+    """Mirror of ``vq_kivi_append_args``."""
+
+    _fields_ = [
+        ("k_new", vp), ("v_new", vp), ("k_strides", i64 * 3), ("v_strides", i64 * 3),
+        ("dtype", i32),
+        ("B", i64), ("H", i64), ("S", i64), ("D", i64),
+        ("k_tail", vp), ("v_tail", vp), ("tail_cap", i64), ("n_tail", i64),
+        ("n_flush", i64),
+        ("k_packed", vp), ("k_scale", vp), ("k_zero", vp), ("v_packed", vp), ("v_scale", vp), ("v_zero", vp),
+        ("meta_dtype", i32),
+        ("cap_tokens", i64), ("dst_tok0", i64),
+        ("group", i32), ("levels", i32), ("eps", f32), ("pack_bits", i32), ("v_layout", i32),
+        ("k_spare", vp), ("v_spare", vp), ("spare_cap", i64),
+    ]
+
+
 _SIGNATURES = {
     "vq_abi_version": (i32, []),
     "vq_last_error": (i32, [C.c_char_p, sz]),
@@ -64,6 +81,7 @@ _SIGNATURES = {
     "vq_kivi_quant_pack": (i32, [vp, i32, i64, i64, i64, i64, i32, i32, i32, f32, i32, i32, vp, vp, vp, i32, i64, i64, vp]),
     "vq_kivi_dequant": (i32, [vp, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, i64, i64, vp, i32, vp]),
     "vq_kv_tail_append": (i32, [vp, vp, C.POINTER(i64), C.POINTER(i64), vp, vp, i32, i64, i64, i64, i64, i64, i64, vp]),
+    "vq_kivi_cache_append": (i32, [C.POINTER(KiviAppendArgs), vp]),
     "vq_pack_words": (i32, [vp, i64, i64, i32, vp, vp]),
     "vq_unpack_words": (i32, [vp, i64, i64, i32, vp, vp]),
     "vq_bit_pack": (i32, [vp, i64, i32, vp, vp]),

@@ -109,6 +109,7 @@ class KIVIKVCache(FP16KVCache):
         # fp16 tail (memory-bound mode): tokens [_n_quantized, offset)
         self._tail_k = self._tail_v = None
         self._tail_spare = None   # second pair of tail buffers the kept rows move into at a flush
+        self._append_args = None  # argument block of the one-call append, refilled from chunk to chunk
         # memory-bound decode: the newest token's (keys, values), counted in ``offset`` but not yet in the
         # tail; the next fused_sdpa stores them in the same launch that attends, anything else stores them first
         self._pending = None
@@ -136,7 +137,10 @@ class KIVIKVCache(FP16KVCache):
         unit = g * per // math.gcd(g, per)
         cap = max(needed, 2 * self._packed_cap, 1024)
         if self._max_ctx is not None:
-            cap = min(cap, self._max_ctx)
+            # a stated limit sizes the store once, as the reference's index buffers are "allocated at
+            # fused_sdpa_max_ctx, not at the live length"
+            # (veloxquant_mlx/tests/cache/test_vecinfer_fused_sdpa.py:342-346)
+            cap = self._max_ctx
         cap = -(-cap // unit) * unit
         W = -(-D // per)
         GV = -(-D // g)
@@ -236,16 +240,18 @@ class KIVIKVCache(FP16KVCache):
                 tk[:, :, :n_tail] = self._tail_k[:, :, :n_tail]
                 tv[:, :, :n_tail] = self._tail_v[:, :, :n_tail]
             self._tail_k, self._tail_v = tk, tv
-        if keys.dtype == self._tail_k.dtype and values.dtype == keys.dtype and (D * keys.element_size()) % 16 == 0:
-            K.kv_tail_append(keys, values, self._tail_k, self._tail_v, n_tail)
-        else:
+        es = keys.element_size()
+        one_call = (keys.dtype == self._tail_k.dtype and values.dtype == keys.dtype and (D * es) % 16 == 0
+                    and keys.stride(3) == 1 and values.stride(3) == 1)
+        if not one_call:
             self._tail_k[:, :, n_tail:need] = keys
             self._tail_v[:, :, n_tail:need] = values
         self.offset += S
         new_boundary = self._quantization_boundary()
         n_quant_now = new_boundary - self._n_quantized
+        spare = None
         if n_quant_now > 0:
-            self._pack_block(self._tail_k[:, :, :n_quant_now], self._tail_v[:, :, :n_quant_now], self._n_quantized)
+            self._ensure_packed_capacity(B, H, D, new_boundary, keys.device)
             keep = need - n_quant_now
             # the rows that stay move to the front of a second buffer (one copy each, no
             # temporaries); a very large prefill chunk leaves an oversized buffer behind, which is
@@ -258,9 +264,23 @@ class KIVIKVCache(FP16KVCache):
             if spare is None or spare[0].shape != (B, H, cap, D) or spare[0].dtype != self._tail_k.dtype:
                 spare = (torch.zeros((B, H, cap, D), dtype=self._tail_k.dtype, device=keys.device),
                          torch.zeros((B, H, cap, D), dtype=self._tail_v.dtype, device=keys.device))
+        if one_call:
+            # append, quantise what aged out and start the next tail in one library call
+            if any((st * es) % 16 for st in keys.stride()[:3]) or keys.data_ptr() % 16:
+                keys = keys.contiguous()
+            if any((st * es) % 16 for st in values.stride()[:3]) or values.data_ptr() % 16:
+                values = values.contiguous()
+            self._append_args = K.kivi_cache_append(
+                keys, values, self._tail_k, self._tail_v, n_tail, max(n_quant_now, 0),
+                (self._kp, self._ks, self._kz, self._vp, self._vs, self._vz), self._n_quantized, spare,
+                bits=self._b, group_size=self._group_size, levels=self._levels, eps=self._eps,
+                v_layout=self._v_layout, args=self._append_args)
+        elif n_quant_now > 0:
+            self._pack_block(self._tail_k[:, :, :n_quant_now], self._tail_v[:, :, :n_quant_now], self._n_quantized)
             if keep:
                 spare[0][:, :, :keep] = self._tail_k[:, :, n_quant_now:need]
                 spare[1][:, :, :keep] = self._tail_v[:, :, n_quant_now:need]
+        if n_quant_now > 0:
             old = (self._tail_k, self._tail_v)
             self._tail_k, self._tail_v = spare
             self._tail_spare = old if old[0].shape[2] == cap else None

@@ -240,9 +240,12 @@ __device__ __forceinline__ void st_partial(float *p, float v, bool device_scope)
 
 // Eight consecutive tail elements as fp16.  A bf16 tail is converted: exact for magnitudes in
 // fp16's normal range, an absolute error below 2^-25 for smaller ones, saturating at 65504.
-__device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool bf16) {
-    if (!bf16) return *reinterpret_cast<const f16x8 *>((const f16 *)base + elem);
-    const uint4 u = *reinterpret_cast<const uint4 *>((const u16 *)base + elem);
+__device__ __forceinline__ f16x8 tail8_from_raw(const uint4 u, bool bf16) {
+    if (!bf16) {
+        union { uint4 u; f16x8 h; } x;
+        x.u = u;
+        return x.h;
+    }
     const u32 w[4] = {u.x, u.y, u.z, u.w};
     f16x8 o;
 #pragma unroll
@@ -252,6 +255,9 @@ __device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool b
         o[2 * j + 1] = (f16)fminf(fmaxf(hi, -65504.f), 65504.f);
     }
     return o;
+}
+__device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool bf16) {
+    return tail8_from_raw(*reinterpret_cast<const uint4 *>((const u16 *)base + elem), bf16);
 }
 
 // NW waves per block.  s_m, s_l: [NW][MF_ROWS] floats; s_o: [NW][MF_ROWS][MF_D] floats of

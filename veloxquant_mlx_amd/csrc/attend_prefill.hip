@@ -442,8 +442,8 @@ template <int BITS> struct PrStage {
 template <int BITS, int GV>
 __global__ __launch_bounds__(PR_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__restrict__ ws) {
-    __shared__ __align__(16) f16 s_k[2][32 * PF_KSTRIDE];
-    __shared__ __align__(16) f16 s_v[2][MF_D * PF_VSTRIDE];
+    __shared__ __align__(16) f16 s_k[3][32 * PF_KSTRIDE];
+    __shared__ __align__(16) f16 s_v[3][MF_D * PF_VSTRIDE];
 
     constexpr int PER = 32 / BITS;
     constexpr int KW = MF_D / PER;
@@ -515,8 +515,15 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     using Stage = PrStage<BITS>;
     f16x8 ksr, kzr;   // key scale / zero of the thread's 8 channels in the token group last fetched
     int meta_group = -1;
-    auto fetch = [&](int w, Stage &st) {   // packed work units only
-        if (w >= n_punits) return;
+    auto fetch = [&](int w, Stage &st) {
+        if (w >= n_punits) {   // tail unit: the thread's key and value row chunks travel in the value-meta slots
+            int64_t tok = (int64_t)(w - n_punits) * 32 + kt;
+            if (tok >= a.n_tail) tok = 0;   // masked in the softmax
+            const int64_t e0 = tbase + tok * MF_D + 8 * kc;
+            st.vs = *reinterpret_cast<const uint4 *>((const u16 *)a.k_tail + e0);
+            st.vz = *reinterpret_cast<const uint4 *>((const u16 *)a.v_tail + e0);
+            return;
+        }
         const int64_t base = (int64_t)w * 32;
         if (BITS == 4) {
             st.kw = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + kc) * 4);
@@ -554,12 +561,9 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             *reinterpret_cast<f16x8 *>(&s_v[buf][vc * PF_VSTRIDE + 8 * vq]) =
                 __builtin_elementwise_fma(codes8(st.vw, vq & 1), as_h8(st.vs), as_h8(st.vz));
         } else {
-            // tail unit (few per block, fetched here): plain key row chunk; value row chunk transposed
-            int64_t tok = (int64_t)(w - n_punits) * 32 + kt;
-            if (tok >= a.n_tail) tok = 0;   // masked in the softmax
-            const int64_t e0 = tbase + tok * MF_D + 8 * kc;
-            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = ld_tail8(a.k_tail, e0, tail_bf16);
-            const f16x8 v0 = ld_tail8(a.v_tail, e0, tail_bf16);
+            // tail unit: plain key row chunk; value row chunk transposed
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = tail8_from_raw(st.vs, tail_bf16);
+            const f16x8 v0 = tail8_from_raw(st.vz, tail_bf16);
 #pragma unroll
             for (int e = 0; e < 8; ++e) s_v[buf][(8 * kc + e) * PF_VSTRIDE + kt] = v0[e];
         }
@@ -598,18 +602,30 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         }
     };
 
-    // One unit: scores of the wave's row blocks, softmax against the lazily updated
-    // references (raised in place, with the accumulators rescaled, when some row's scores
-    // outgrow its reference), second product.
-    auto compute = [&](int buf, int base, bool packed, int full) {
-        // the key tile's operands first, then four independent accumulator chains side by side
-        f16x8 A[2][4];
+    // The operands of a unit live in registers from one iteration to the next: the key tile's
+    // rows (A) and the value tile's rows (Bv) of unit w+1 are read from LDS while unit w is
+    // still being computed, so that the LDS traffic of the eight waves runs beside the products
+    // and the softmax instead of in front of them.
+    f16x8 A[2][4], Bv[8];
+    auto load_keys = [&](int buf) {
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             const f16 *kr = &s_k[buf][pf_krow(pf_tok(n >> 2, n & 3, T)) * PF_KSTRIDE + 8 * blk];
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) A[T][ks] = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
         }
+    };
+    auto load_values = [&](int buf) {
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt)
+            Bv[nt] = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+    };
+
+    // One unit: scores of the wave's row blocks (four independent accumulator chains side by
+    // side), softmax against the lazily updated references (raised in place, with the
+    // accumulators rescaled, when some row's scores outgrow its reference), second product.
+    // `next` is the buffer of the following unit (stale but harmless after the last one).
+    auto compute = [&](int next, int base, bool packed, int full) {
         f32x4 S[PR_RB][2];
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
@@ -618,11 +634,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
 #pragma unroll
                 for (int rb = 0; rb < PR_RB; ++rb)
                     S[rb][T] = VQ_MFMA(A[T][ks], qn[rb][ks], ks == 0 ? (f32x4{0.f, 0.f, 0.f, 0.f}) : S[rb][T]);
-        // the value tile's operands are on their way while the softmax runs
-        f16x8 Bv[8];
-#pragma unroll
-        for (int nt = 0; nt < 8; ++nt)
-            Bv[nt] = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+        load_keys(next);
         bool grow = false;
 #pragma unroll
         for (int rb = 0; rb < PR_RB; ++rb) {
@@ -657,24 +669,41 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             for (int rb = 0; rb < PR_RB; ++rb) O[rb][nt] = VQ_MFMA(P8[rb], Bv[nt], O[rb][nt]);
 #pragma unroll
         for (int rb = 0; rb < PR_RB; ++rb) L[rb] = VQ_MFMA(P8[rb], ones, L[rb]);
+        load_values(next);
     };
 
-    // ---- pipeline over the work units [w0, w1): unit w+1 is unpacked and unit w+2 requested while unit w is computed
+    // ---- pipeline over the work units [w0, w1) on three LDS buffers: while unit w is computed
+    // from registers, unit w+1 is read from its buffer, unit w+2 is unpacked into the third and
+    // unit w+3 is requested from memory.  Half of the waves unpack before they compute and half
+    // after, so that the two waves of a SIMD are not in the same phase after every barrier.
     Stage st;
     if (w1 > w0) {
         fetch(w0, st);
         unpack_to_lds(w0, st, 0);
+        if (w0 + 1 < w1) {
+            fetch(w0 + 1, st);
+            unpack_to_lds(w0 + 1, st, 1);
+        }
+        if (w0 + 2 < w1) fetch(w0 + 2, st);
         __syncthreads();
-        if (w0 + 1 < w1) fetch(w0 + 1, st);
+        load_keys(0);
+        load_values(0);
     }
+    const bool early = wave < PR_THREADS / 128;
+    int cur = 0;
     for (int w = w0; w < w1; ++w) {
-        const int buf = (w - w0) & 1;
-        if (w + 1 < w1) unpack_to_lds(w + 1, st, buf ^ 1);
-        if (w + 2 < w1) fetch(w + 2, st);
+        const int next = cur == 2 ? 0 : cur + 1, third = next == 2 ? 0 : next + 1;
+        auto produce = [&]() {
+            if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
+            if (w + 3 < w1) fetch(w + 3, st);
+        };
+        if (early) produce();
         const bool packed = w < n_punits;
         const int base = packed ? w * 32 : (w - n_punits) * 32;
-        compute(buf, base, packed, packed ? full_vis : full_tvis);
+        compute(next, base, packed, packed ? full_vis : full_tvis);
+        if (!early) produce();
         __syncthreads();
+        cur = next;
     }
 
     // ---- every wave owns its rows: accumulator register r of lane (n, blk) is row 4 blk + r of the

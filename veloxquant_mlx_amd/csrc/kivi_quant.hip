@@ -216,7 +216,7 @@ template <> struct Raw8<f16> {
 constexpr int KT_MAXP = 8;
 
 template <typename T, typename M, int LPR, int MODE, int NP>
-__global__ __launch_bounds__(256) void kivi_key_tile_kernel(
+__device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
     const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
     float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
     int64_t cap_tokens, int64_t dst_tok0, int W) {
@@ -226,8 +226,7 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
     __shared__ __align__(16) float s_mn[RPP][D];
     __shared__ __align__(16) float s_mx[RPP][D];
     __shared__ __align__(16) float s_par[4][D];
-    const int gk = blockIdx.x;
-    const int64_t bh = blockIdx.y;
+    const int gk = bx;
     const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
     const int64_t s0 = (int64_t)gk * group;
     const T *xb = x + bh * x_stride_bh;
@@ -308,6 +307,15 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
     }
 }
 
+template <typename T, typename M, int LPR, int MODE, int NP>
+__global__ __launch_bounds__(256) void kivi_key_tile_kernel(
+    const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
+    float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
+    int64_t cap_tokens, int64_t dst_tok0, int W) {
+    kivi_key_tile_body<T, M, LPR, MODE, NP>((int)blockIdx.x, (int64_t)blockIdx.y, x, out, S, x_stride_bh, group, levels, eps,
+                                            bits, packed, scale, zero, cap_tokens, dst_tok0, W);
+}
+
 // ---------------------------------------------------------------------------
 // Values: groups along channels.  One block per (row tile, bh); a group is
 // reduced across g/8 neighbouring lanes.  MODE 0 reconstruction, MODE 1
@@ -316,7 +324,7 @@ __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
 constexpr int VT_TILES = 4;   // row tiles of 256 / LPR rows one block of the value kernel takes
 
 template <typename T, typename M, int LPR, int MODE>
-__global__ __launch_bounds__(256) void kivi_value_tile_kernel(
+__device__ __forceinline__ void kivi_value_tile_body(int bx, int64_t bh,
     const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
     float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
     int64_t cap_tokens, int64_t dst_tok0, int W) {
@@ -328,9 +336,8 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
     // token-packed scale / zero rows of the tile, staged so that they leave as whole vectors
     constexpr int MAXGV = 4;
     __shared__ __align__(16) M s_meta[MODE == 2 ? 2 * MAXGV * ROWS : 1];
-    const int64_t bh = blockIdx.y;
     const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
-    const int64_t tile_tok0 = (int64_t)blockIdx.x * ROWS;
+    const int64_t tile_tok0 = (int64_t)bx * ROWS;
     const int GL = group / 8;  // lanes per group (power of two <= LPR)
     const int GV = D / group;
 
@@ -428,6 +435,33 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
             packed[(bh * (cap_tokens / per) + wrow) * D + d] = w;
         }
     }
+}
+
+template <typename T, typename M, int LPR, int MODE>
+__global__ __launch_bounds__(256) void kivi_value_tile_kernel(
+    const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
+    float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
+    int64_t cap_tokens, int64_t dst_tok0, int W) {
+    kivi_value_tile_body<T, M, LPR, MODE>((int)blockIdx.x, (int64_t)blockIdx.y, x, out, S, x_stride_bh, group, levels, eps,
+                                          bits, packed, scale, zero, cap_tokens, dst_tok0, W);
+}
+
+// Keys and values of one cache flush in a single launch: blocks [0, key_blocks) of a (b, h)
+// take the key groups, the rest the value row tiles.  The two bodies are those of the kernels
+// above; a chunked prefill flushes a few hundred tokens at a time, where a second launch costs
+// as much as the work.
+struct PackDst { uint32_t *packed; void *scale, *zero; };
+template <typename T, typename M, int LPR, int NP, int VMODE>
+__global__ __launch_bounds__(256) void kivi_kv_tile_kernel(
+    const T *__restrict__ k, const T *__restrict__ v, int64_t S, int64_t x_stride_bh, int group, float levels, float eps,
+    int bits, PackDst kd, PackDst vd, int64_t cap_tokens, int64_t dst_tok0, int W, int key_blocks) {
+    const int bx = (int)blockIdx.x;
+    if (bx < key_blocks)
+        kivi_key_tile_body<T, M, LPR, 1, NP>(bx, (int64_t)blockIdx.y, k, nullptr, S, x_stride_bh, group, levels, eps, bits,
+                                             kd.packed, (M *)kd.scale, (M *)kd.zero, cap_tokens, dst_tok0, W);
+    else
+        kivi_value_tile_body<T, M, LPR, VMODE>(bx - key_blocks, (int64_t)blockIdx.y, v, nullptr, S, x_stride_bh, group, levels,
+                                               eps, bits, vd.packed, (M *)vd.scale, (M *)vd.zero, cap_tokens, dst_tok0, W);
 }
 
 // ---------------------------------------------------------------------------
@@ -654,6 +688,55 @@ static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t 
 #undef VQ_V
     return true;
 }
+
+namespace vq {
+// Keys (groups along tokens) and values (groups along channels, v_layout) of the same S tokens in
+// one launch where the tile kernels take the shape, else as two single calls.
+int pack_kv_pair(const void *k, const void *v, int dtype, int64_t BH, int64_t S, int64_t D, int64_t xs, int group,
+                 int levels, float eps, int bits, int v_layout, void *kp, void *ks, void *kz, void *vp, void *vs, void *vz,
+                 int meta_dtype, int64_t cap, int64_t tok0, void *stream) {
+    const int per = bits >= 1 && bits <= 8 ? 32 / bits : 1;
+    constexpr int LPR = 16, RPP = 256 / LPR, ROWS = RPP * VT_TILES;
+    const bool tokpacked = v_layout == VQ_V_TOKEN_PACKED;
+    const bool fused = D == 128 && (dtype == VQ_F16 || dtype == VQ_BF16) && (meta_dtype == VQ_F16 || meta_dtype == VQ_F32) &&
+                       BH >= 1 && BH <= 65535 && S >= 1 && xs % 8 == 0 && xs >= S * D && aligned16(k) && aligned16(v) &&
+                       aligned16(kp) && aligned16(ks) && aligned16(kz) && aligned16(vp) && aligned16(vs) && aligned16(vz) &&
+                       (bits == 2 || bits == 4 || bits == 8) && levels >= 1 && levels <= (1 << bits) - 1 &&
+                       group >= 8 && group <= KT_MAXP * RPP && group % 8 == 0 && pow2(group / 8) && D % group == 0 &&
+                       (v_layout == VQ_V_CHANNEL_PACKED || (tokpacked && RPP % per == 0)) && tok0 >= 0 && tok0 + S <= cap &&
+                       tok0 % group == 0 && (!tokpacked || (tok0 % per == 0 && S % per == 0 && cap % per == 0));
+    if (!fused) {
+        const int rc = vq_kivi_quant_pack(k, dtype, BH, S, D, xs, VQ_AXIS_TOKEN, group, levels, eps, bits, VQ_V_CHANNEL_PACKED,
+                                          kp, ks, kz, meta_dtype, cap, tok0, stream);
+        if (rc != VQ_OK) return rc;
+        return vq_kivi_quant_pack(v, dtype, BH, S, D, xs, VQ_AXIS_CHANNEL, group, levels, eps, bits, v_layout, vp, vs, vz,
+                                  meta_dtype, cap, tok0, stream);
+    }
+    const int key_blocks = (int)cdiv(S, group), value_blocks = (int)cdiv(S, ROWS);
+    const dim3 grid((unsigned)(key_blocks + value_blocks), (unsigned)BH);
+    const int W = (int)cdiv(LPR * 8, per);
+    const PackDst kd = {(uint32_t *)kp, ks, kz}, vd = {(uint32_t *)vp, vs, vz};
+    hipStream_t st = (hipStream_t)stream;
+#define VQ_KV(T, M, NP, VM)                                                                                              \
+    hipLaunchKernelGGL((kivi_kv_tile_kernel<T, M, LPR, NP, VM>), grid, dim3(256), 0, st, (const T *)k, (const T *)v, S, xs, \
+                       group, (float)levels, eps, bits, kd, vd, cap, tok0, W, key_blocks)
+#define VQ_KV_NP(T, M, VM)                                                                \
+    do {                                                                                  \
+        if (group <= (KT_MAXP / 2) * RPP) VQ_KV(T, M, KT_MAXP / 2, VM); else VQ_KV(T, M, KT_MAXP, VM); \
+    } while (0)
+#define VQ_KV_M(T, VM)                                                                    \
+    do {                                                                                  \
+        if (meta_dtype == VQ_F16) VQ_KV_NP(T, f16, VM); else VQ_KV_NP(T, float, VM);      \
+    } while (0)
+    if (dtype == VQ_F16) { if (tokpacked) VQ_KV_M(f16, 2); else VQ_KV_M(f16, 1); }
+    else { if (tokpacked) VQ_KV_M(bf16_t, 2); else VQ_KV_M(bf16_t, 1); }
+#undef VQ_KV_M
+#undef VQ_KV_NP
+#undef VQ_KV
+    VQ_HIP_CHECK_LAUNCH("vq_kivi_cache_append");
+    return VQ_OK;
+}
+}  // namespace vq
 
 extern "C" int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int axis,
                                      int group, int levels, float eps, void *stream) {

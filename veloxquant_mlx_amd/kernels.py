@@ -204,6 +204,51 @@ def kv_tail_append(k_new: torch.Tensor, v_new: torch.Tensor, k_tail: torch.Tenso
                                              v_tail.data_ptr(), es, B, H, S, D, cap, pos, _stream(k_new)))
 
 
+def kivi_cache_append(k_new: torch.Tensor, v_new: torch.Tensor, k_tail: torch.Tensor, v_tail: torch.Tensor,
+                      n_tail: int, n_flush: int, packed, dst_tok0: int, spare, *, bits: int, group_size: int,
+                      levels: int, eps: float, v_layout: str, args=None):
+    """One chunk of a packed KIVI cache in one library call (``vq_kivi_cache_append``):
+    ``k_new, v_new [B,H,S,D]`` go to rows ``[n_tail, n_tail+S)`` of the tails; with
+    ``n_flush > 0`` the first ``n_flush`` tail rows are quantised into ``packed =
+    (k_packed, k_scale, k_zero, v_packed, v_scale, v_zero)`` at token ``dst_tok0`` and the
+    rest moves to the front of ``spare = (k_spare, v_spare)``.  The steps of
+    ``KIVIKVCache.update_and_fetch`` (veloxquant_mlx/cache/kivi_cache.py:206-262) on packed
+    buffers.  The caller owns the shapes: all tensors share a device, the new tokens and the
+    four tails one dtype, every buffer is contiguous except ``k_new`` / ``v_new``, whose
+    channels are.  ``args`` may carry a ``KiviAppendArgs`` from a previous call to refill."""
+    name = "kivi_cache_append"
+    _need_gpu(name, k_new)
+    a = _lib.KiviAppendArgs() if args is None else args
+    B, H, S, D = k_new.shape
+    if v_new.shape != k_new.shape or k_tail.shape != v_tail.shape or k_tail.ndim != 4:
+        raise ValueError(f"{name}: keys/values must be [B,H,S,D] and the tails [B,H,cap,D]")
+    if not (k_new.dtype == v_new.dtype == k_tail.dtype == v_tail.dtype):
+        raise ValueError(f"{name}: new tokens and tails must share one dtype")
+    a.k_new, a.v_new = k_new.data_ptr(), v_new.data_ptr()
+    ks, vs = k_new.stride(), v_new.stride()
+    if ks[3] != 1 or vs[3] != 1:
+        raise ValueError(f"{name}: channels of the new tokens must be contiguous")
+    a.k_strides[0], a.k_strides[1], a.k_strides[2] = ks[0], ks[1], ks[2]
+    a.v_strides[0], a.v_strides[1], a.v_strides[2] = vs[0], vs[1], vs[2]
+    a.dtype = _FLOAT_TAG[k_new.dtype]
+    a.B, a.H, a.S, a.D = B, H, S, D
+    a.k_tail, a.v_tail, a.tail_cap, a.n_tail = k_tail.data_ptr(), v_tail.data_ptr(), k_tail.shape[2], n_tail
+    a.n_flush = n_flush
+    if n_flush:
+        kp, ksc, kz, vp_, vsc, vz = packed
+        per = 32 // bits
+        a.k_packed, a.k_scale, a.k_zero = kp.data_ptr(), ksc.data_ptr(), kz.data_ptr()
+        a.v_packed, a.v_scale, a.v_zero = vp_.data_ptr(), vsc.data_ptr(), vz.data_ptr()
+        a.meta_dtype = VQ_F16 if ksc.dtype == torch.float16 else VQ_F32
+        a.cap_tokens, a.dst_tok0 = kp.shape[2], dst_tok0
+        if v_layout == "token" and vp_.shape[2] * per != kp.shape[2]:
+            raise ValueError(f"{name}: key and value stores differ in capacity")
+        a.group, a.levels, a.eps, a.pack_bits, a.v_layout = group_size, levels, eps, bits, _V_LAYOUT[v_layout]
+        a.k_spare, a.v_spare, a.spare_cap = spare[0].data_ptr(), spare[1].data_ptr(), spare[0].shape[2]
+    _lib.check(_lib.load().vq_kivi_cache_append(C.byref(a), _stream(k_new)))
+    return a
+
+
 def kivi_dequant(packed: torch.Tensor, scale: torch.Tensor, zero: torch.Tensor, axis: int, group_size: int,
                  bits: int, S: int, D: int, *, v_layout: str = "channel", out_dtype: torch.dtype = torch.float16,
                  src_tok0: int = 0) -> torch.Tensor:
@@ -760,7 +805,7 @@ __all__ = [
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",
-    "kv_tail_append", "attend_fixed_order",
+    "kv_tail_append", "kivi_cache_append", "attend_fixed_order",
     "kivi_packed_attend", "scalar_fused_decode_attend", "scalar_fused_decode_attend_batched",
     "scalar_predecoded_attend", "flash_prefill_attend",
 ]
