@@ -187,6 +187,23 @@ def main() -> int:
 
     if not a.no_extras:
         out["extras"] = _extras(torch, K, dev)
+        # the same step with the layers' caches adopted by a layer-stacked cache (their buffers become
+        # slices of [NL*B, ...] stacks, copied once): 36 appends that launch nothing and ONE launch that
+        # stores every layer's new token and attends for all layers
+        from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+        stack = LayerStackedKIVICache.from_layers(caches)
+
+        def step_all():
+            for l, c in enumerate(caches):
+                c.update_and_fetch(k_new[l], v_new[l])
+            stack.fused_sdpa_all(q, scale)
+        for _ in range(2):
+            step_all()
+        ms = _side_ms(step_all, 5, torch)
+        out["extras"]["decode_cfg3_36_layers_one_launch"] = {
+            "ms": round(ms, 4), "ms_per_layer": round(ms / NL, 5), "GBps": round(step_bytes / ms / 1e6, 1),
+            "frac_hbm": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes,
+            "note": "LayerStackedKIVICache over the resident caches: append + attend of all layers per step"}
     if not a.no_cpu:
         out["cpu_baseline"] = _cpu_baseline(np, torch, caches[0], q[0], ctx, Hkv, D, bits, g, scale)
     print(json.dumps(out))
@@ -287,32 +304,6 @@ def _extras(torch, K, dev):
     flops = 2 * 524288 * 256 * 8
     ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
                             "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
-    # config 3 with the 36 layers' packed caches stacked along the batch axis ([NL*B, ...] buffers, what a
-    # cache that owns all layers would hold) and attended in ONE launch; synthetic random codes, as the
-    # reference's own microbenchmark feeds its kernel (scripts/kv_kernel_roofline_bench.py:245-253)
-    NL, Bs, ctx, g = 36, 16, 32768, 64
-    BB = NL * Bs
-    gen = torch.Generator(device=dev).manual_seed(3)
-    kp = torch.randint(-2 ** 31, 2 ** 31 - 1, (BB, Hkv, ctx, D // 8), dtype=torch.int32, device=dev, generator=gen)
-    vp = torch.randint(-2 ** 31, 2 ** 31 - 1, (BB, Hkv, ctx // 8, D), dtype=torch.int32, device=dev, generator=gen)
-    ks = (torch.rand((BB, Hkv, ctx // g, D), device=dev, generator=gen) * 0.3 + 0.05).half()
-    kz = torch.randn((BB, Hkv, ctx // g, D), device=dev, generator=gen).half()
-    vs = (torch.rand((BB, Hkv, D // g, ctx), device=dev, generator=gen) * 0.3 + 0.05).half()
-    vz = torch.randn((BB, Hkv, D // g, ctx), device=dev, generator=gen).half()
-    kt = torch.randn((BB, Hkv, 192, D), device=dev, generator=gen).half()
-    vt = torch.randn((BB, Hkv, 192, D), device=dev, generator=gen).half()
-    qs = torch.randn((BB, Hq, 1, D), device=dev, generator=gen).half()
-    fn = lambda: K.kivi_packed_attend(qs, n_packed=ctx, bits=4, group_size=g, v_layout="token", k_packed=kp, k_scale=ks,
-                                      k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz, k_tail=kt, v_tail=vt, n_tail=128,
-                                      scale=1 / math.sqrt(D), out_dtype=torch.float16)
-    for _ in range(2):
-        fn()
-    ms = _side_ms(fn, 5, torch)
-    nbytes = NL * _algorithmic_bytes_per_layer(Bs, Hkv, ctx, D, 4, g)
-    ex["decode_cfg3_36_layers_one_launch"] = {"ms": round(ms, 4), "ms_per_layer": round(ms / NL, 5), "GBps": round(nbytes / ms / 1e6, 1),
-                                              "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}
-    del kp, vp, ks, kz, vs, vz, kt, vt, qs
-    torch.cuda.empty_cache()
     # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,
     # and with the reconstruction written as well
     from veloxquant_mlx_amd.allocators.vecinfer import walsh_hadamard_matrix

@@ -565,3 +565,62 @@ def test_cache_append_rejects_bad_arguments():
     with pytest.raises(ValueError, match="n_flush"):
         K.kivi_cache_append(kn, vn, tk, tv, 0, 64, st, 0, (z(1, 1, 64, 128), z(1, 1, 64, 128)), bits=4, group_size=32,
                             levels=15, eps=1e-8, v_layout="token")
+
+
+def test_layer_stacked_cache_attends_for_all_layers_at_once():
+    """``LayerStackedKIVICache``: per-layer updates through the ordinary cache API on slices of the
+    stacked buffers, one attention launch for all layers; against separate per-layer caches fed the
+    same tokens (the layer-batched call of veloxquant_mlx/metal/_scalar_attend.py:496-647 without its
+    stacking step).  Outputs within 1e-3 (the launches may split the context differently), stored
+    codes bit for bit."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    NL, B, Hq, Hkv, D = 3, 2, 8, 2, 128
+    cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=4, kivi_group_size=32, residual_length=64,
+                        fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=1024)
+    stacked = LayerStackedKIVICache(cfg, NL)
+    solo = [KVCacheFactory.create(cfg) for _ in range(NL)]
+    g = torch.Generator(device="cuda").manual_seed(11)
+    rnd = lambda *s: torch.randn(s, generator=g, device="cuda").to(torch.float16)
+    scale = 1 / math.sqrt(D)
+
+    def feed(layer, n):
+        k, v = rnd(B, Hkv, n, D), rnd(B, Hkv, n, D)
+        stacked[layer].update_and_fetch(k, v)
+        solo[layer].update_and_fetch(k, v)
+
+    def check(Sq=1):
+        q = rnd(NL, B, Hq, Sq, D)
+        out = stacked.fused_sdpa_all(q, scale)
+        assert out.shape == (NL, B, Hq, Sq, D)
+        for layer in range(NL):
+            ref = solo[layer].fused_sdpa(q[layer], scale)
+            assert (out[layer].float() - ref.float()).abs().max().item() <= 1e-3, layer
+
+    for layer in range(NL):
+        feed(layer, 200)
+    check()
+    kp = stacked._packed[0]
+    assert all(stacked[layer]._kp.data_ptr() == kp[layer * B:].data_ptr() for layer in range(NL))   # the stack is the storage
+    for step in range(80):   # crosses two flushes: tails swap inside the stack, nothing is copied back
+        for layer in range(NL):
+            feed(layer, 1)
+        check()
+    assert stacked._packed[0] is kp
+    for layer in range(NL):
+        a, b = stacked[layer], solo[layer]
+        n = a._n_quantized
+        assert a.offset == b.offset == 280 and n == b._n_quantized
+        assert torch.equal(a._kp[:, :, :n], b._kp[:, :, :n]) and torch.equal(a._vp[:, :, :n // 8], b._vp[:, :, :n // 8])
+        assert torch.equal(a._ks[:, :, :n // 32], b._ks[:, :, :n // 32]) and torch.equal(a._vz[..., :n], b._vz[..., :n])
+        nt = a.offset - n
+        assert torch.equal(a._tail_k[:, :, :nt], b._tail_k[:, :, :nt])
+    # a forward pass in flight: layer 0 is one token ahead of the others
+    feed(0, 1)
+    check()
+    check(Sq=4)
+    # a layer whose buffers were replaced is copied back into the stack
+    stacked[1].state = solo[1].state
+    check()
+    with pytest.raises(ValueError, match="NL=3"):
+        stacked.fused_sdpa_all(rnd(2, B, Hq, 1, D), scale)

@@ -3,6 +3,7 @@
 from .base import KVCacheBuilder, KVCacheConfig, KVCacheFactory
 from .options import KIVIOptions, VecInferOptions
 from .prompt_cache import load_prompt_cache, save_prompt_cache
+from .stacked_cache import LayerStackedKIVICache
 
 __all__ = ["KVCacheConfig", "KVCacheFactory", "KVCacheBuilder", "KIVIOptions", "VecInferOptions",
-           "save_prompt_cache", "load_prompt_cache"]
+           "save_prompt_cache", "load_prompt_cache", "LayerStackedKIVICache"]
