@@ -304,6 +304,17 @@ def _extras(torch, K, dev):
     flops = 2 * 524288 * 256 * 8
     ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
                             "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
+    # Kitty keys (mixed 4/2-bit by channel variance): two launches of the key-axis round trip plus the ranking
+    kc = KVCacheFactory.create(KVCacheConfig(method="kitty", head_dim=D))
+    kk = (torch.randn((16, Hkv, 8192, D), device=dev) * torch.exp(torch.randn(D, device=dev))).to(torch.float16)
+    fn = lambda: kc._quantize_keys(kk)
+    for _ in range(3):
+        fn()
+    ms = _side_ms(fn, 10, torch)
+    nb = 2 * kk.numel() * 2
+    ex["kitty_keys_[16,8,8192,128]"] = {"ms": round(ms, 5), "GBps": round(nb / ms / 1e6, 1), "bytes": nb,
+                                        "note": "fp16 keys in, fp16 mixed-precision reconstruction out"}
+    del kk, kc
     # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,
     # and with the reconstruction written as well
     from veloxquant_mlx_amd.allocators.vecinfer import walsh_hadamard_matrix

@@ -1,0 +1,105 @@
+"""``method="kitty"`` on the GPU against ``oracle.kitty`` (cases of
+veloxquant_mlx/tests/cache/test_kitty_cache.py and tests/quantizers/test_kitty_batched.py)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import kitty as okt
+from tests._gpu import gpu, host, require_gpu, to_dev
+from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+from veloxquant_mlx_amd.cache.kitty_cache import KittyKVCache
+from veloxquant_mlx_amd.core.exceptions import QuantizerConfigError
+from veloxquant_mlx_amd.quantizers import kitty as qk
+
+pytestmark = gpu
+
+
+def _kv(B, H, S, D, seed):
+    """Keys whose channels differ in spread by clear margins (the ranking is then not a matter of
+    the last bits of a float32 variance), values plain."""
+    rng = np.random.default_rng(seed)
+    spread = np.exp(np.random.default_rng(99).permutation(D) / D * 3.0).astype(np.float32)
+    return ((rng.standard_normal((B, H, S, D)) * spread).astype(np.float16),
+            rng.standard_normal((B, H, S, D)).astype(np.float16))
+
+
+@pytest.mark.parametrize("B,H,D,prefill,kw", [
+    (1, 2, 64, 20, {}),                                                    # ragged last group
+    (2, 2, 128, 100, {}),
+    (1, 4, 128, 64, dict(kitty_hi_fraction=0.5, kitty_hi_bit=8, kitty_lo_bit=3, kitty_group_size=16)),
+    (1, 1, 64, 32, dict(kitty_hi_fraction=0.0)),
+    (1, 1, 64, 32, dict(kitty_hi_fraction=1.0)),
+])
+def test_cache_matches_the_model_bit_for_bit(B, H, D, prefill, kw):
+    require_gpu()
+    c = KVCacheFactory.create(KVCacheConfig(method="kitty", head_dim=D, **kw))
+    assert isinstance(c, KittyKVCache)
+    m = okt.KittyCacheModel(D, kw.get("kitty_hi_fraction", 0.25), kw.get("kitty_hi_bit", 4), kw.get("kitty_lo_bit", 2),
+                            kw.get("kitty_group_size", 32))
+    k, v = _kv(B, H, prefill, D, 1)
+    ko, vo = c.update_and_fetch(to_dev(k), to_dev(v))
+    km, vm = m.update_and_fetch(k, v)
+    assert np.array_equal(host(ko), km) and np.array_equal(host(vo), vm)
+    for step in range(6):
+        k, v = _kv(B, H, 1, D, 10 + step)
+        ko, vo = c.update_and_fetch(to_dev(k), to_dev(v))
+        km, vm = m.update_and_fetch(k, v)
+        assert ko.shape[2] == prefill + step + 1
+        assert np.array_equal(host(ko), km) and np.array_equal(host(vo), vm)
+    k, v = _kv(B, H, 40, D, 30)   # a later multi-token call is ranked by the running sums
+    ko, _ = c.update_and_fetch(to_dev(k), to_dev(v))
+    km, _ = m.update_and_fetch(k, v)
+    assert np.array_equal(host(ko), km)
+    np.testing.assert_allclose(host(c._key_sum), m.key_sum, rtol=1e-5, atol=1e-3)
+    np.testing.assert_allclose(host(c._key_sq_sum), m.key_sq_sum, rtol=1e-5, atol=1e-2)
+    assert (c.compressed_key_bytes, c.fp16_key_bytes, c.value_fp16_bytes) == \
+        (m.compressed_key_bytes, m.fp16_key_bytes, m.value_fp16_bytes)
+    assert c.compressed_key_bytes < c.fp16_key_bytes
+    assert c.trim(40) == m.trim(40) == 40 and c.offset == m.keys.shape[2]
+    np.testing.assert_allclose(host(c._key_sum), m.key_sum, rtol=1e-5, atol=1e-3)
+    assert c.compressed_key_bytes == m.compressed_key_bytes
+    assert c.trim(10 ** 6) == prefill + 6 and c._key_sum is None and c._n_keys == 0
+
+
+def test_bfloat16_keys_round_through_float16():
+    """The reference builds the reconstruction as float16 and casts it to the keys' dtype (kitty_cache.py:141-148)."""
+    require_gpu()
+    k, v = _kv(1, 2, 64, 128, 5)
+    kb = torch.from_numpy(k.astype(np.float32)).to(torch.bfloat16)
+    c = KVCacheFactory.create(KVCacheConfig(method="kitty", head_dim=128))
+    ko, _ = c.update_and_fetch(kb.cuda(), to_dev(v).to(torch.bfloat16))
+    m = okt.KittyCacheModel(128)
+    km, _ = m.update_and_fetch(kb.float().numpy(), v)
+    want = torch.from_numpy(km).to(torch.bfloat16)
+    assert ko.dtype == torch.bfloat16 and torch.equal(ko.cpu(), want)
+
+
+def test_quantizer_functions():
+    require_gpu()
+    data = np.random.default_rng(7).standard_normal((128, 64)).astype(np.float32)
+    data[:, :8] *= 10.0
+    hi, lo = qk.rank_channels_by_sensitivity(torch.from_numpy(data).cuda(), hi_fraction=0.125)
+    assert hi == list(range(8)) and lo == list(range(8, 64))          # test_kitty_cache.py:110-123
+    x = data.astype(np.float16)
+    out = qk.quantize_mixed_channels(to_dev(x), hi, lo)
+    mask = np.zeros((1, 64), bool)
+    mask[0, :8] = True
+    assert np.array_equal(host(out), okt.quantize_mixed_channels_batched(x[None], mask)[0])
+    tie = qk.hi_mask_from_variance_batched(torch.ones((1, 4), device="cuda"), 0.5)
+    assert tie.tolist() == [[True, True, False, False]]
+    s = torch.from_numpy(data.sum(0)).cuda()
+    sq = torch.from_numpy((data * data).sum(0)).cuda()
+    np.testing.assert_allclose(host(qk.compute_running_variance(s, sq, 128)), np.var(data, axis=0), rtol=1e-4, atol=1e-5)
+    assert not qk.compute_running_variance(s, sq, 1).any()
+
+
+def test_configuration():
+    require_gpu()
+    c = KittyKVCache(KVCacheConfig(method="kitty", head_dim=64))
+    assert c.assigned_avg_bits == 2.5 and (c.hi_fraction, c.hi_bit, c.lo_bit, c.group_size) == (0.25, 4, 2, 32)
+    c0 = KittyKVCache(KVCacheConfig(method="kitty", head_dim=64, kitty_hi_fraction=0.0))
+    assert abs(c0.assigned_avg_bits - (4 + 63 * 2) / 64) < 1e-9          # test_kitty_cache.py:248-262
+    for bad in (1.5, -0.1):
+        with pytest.raises(QuantizerConfigError, match="kitty_hi_fraction"):
+            KittyKVCache(KVCacheConfig(method="kitty", head_dim=64, kitty_hi_fraction=bad))

@@ -24,4 +24,14 @@ class KIVIOptions:
     kivi_group_size: int = 32  # min/max group size (KIVI default 32)
 
 
-__all__ = ["VecInferOptions", "KIVIOptions"]
+@dataclass
+class KittyOptions:
+    """Kitty configuration (channel-wise mixed-precision keys; options.py:66-73 in the reference)."""
+
+    kitty_hi_fraction: float = 0.25  # fraction of channels kept at kitty_hi_bit
+    kitty_hi_bit: int = 4
+    kitty_lo_bit: int = 2
+    kitty_group_size: int = 32
+
+
+__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions"]
