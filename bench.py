@@ -314,6 +314,18 @@ def _extras(torch, K, dev):
     nb = 2 * kk.numel() * 2
     ex["kitty_keys_[16,8,8192,128]"] = {"ms": round(ms, 5), "GBps": round(nb / ms / 1e6, 1), "bytes": nb,
                                         "note": "fp16 keys in, fp16 mixed-precision reconstruction out"}
+    # AgeTieredKV: 8192 tokens re-derived at 8 / 4 / 2 bits by age (one launch per stretch of groups of one tier)
+    from veloxquant_mlx_amd.quantizers.age_tiered import age_tier_quantize_batched, assign_age_tiers, default_age_tiers
+    tiers = assign_age_tiers([8192 - (i + 1) for i in range(8192)], 128, 1024)
+    group_tier = [tiers[gi * 32] for gi in range(256)]
+    raw = kk.reshape(16 * Hkv, 8192, D)
+    fn = lambda: age_tier_quantize_batched(raw, group_tier, default_age_tiers(8, 4, 2), 32)
+    for _ in range(3):
+        fn()
+    ms = _side_ms(fn, 10, torch)
+    ex["age_tiered_keys_[16,8,8192,128]"] = {"ms": round(ms, 5), "GBps": round(nb / ms / 1e6, 1), "bytes": nb,
+                                             "note": "fp16 tokens in, fp16 reconstruction out, three tiers"}
+    del raw
     del kk, kc
     # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,
     # and with the reconstruction written as well

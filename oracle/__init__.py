@@ -12,7 +12,7 @@ lives in tests/test_oracle_*.py):
 * group quantisation, packing, dequantisation, decode attention, causal
   prefill attention, attention from codebook indices with its sliding-window
   mask, cache frontier arithmetic, the Kitty channel ranking / mixed round trip /
-  accounting: pinned (hand-computed known answers, the reference tests' own seeded
+  accounting, the AgeTieredKV tiers / windows / bytes: pinned (hand-computed known answers, the reference tests' own seeded
   cases, closed forms, invariants, brute force, library SDPA).
 * ``quantize_vq`` on exact fp32 near-ties: PARITY UNPINNED against MLX's
   ``mx.sum`` reduction order and ``mx.argmin`` tie order (MLX is not

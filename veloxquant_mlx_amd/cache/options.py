@@ -34,4 +34,16 @@ class KittyOptions:
     kitty_group_size: int = 32
 
 
-__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions"]
+@dataclass
+class AgeTieredKVOptions:
+    """AgeTieredKV configuration (three precision tiers by token age; options.py in the reference)."""
+
+    age_recent_boundary: int = 128
+    age_mid_boundary: int = 1024
+    age_bits_recent: int = 8
+    age_bits_mid: int = 4
+    age_bits_old: int = 2
+    age_group_size: int = 32
+
+
+__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions", "AgeTieredKVOptions"]
