@@ -316,6 +316,20 @@ typedef struct vq_lut_attend_args {
 size_t vq_vecinfer_attend_workspace(const vq_lut_attend_args *a);
 int vq_vecinfer_attend(const vq_lut_attend_args *a);
 
+/* ---- SKVQ clipped group quantisation ------------------------------------- */
+
+/* Round trip of rows through per-token, per-channel-group asymmetric quantisation with a
+ * grid-searched clip factor: out = cast(code*scale + lo) under the first of `alphas` with the
+ * smallest group error.  Replaces clipped_group_quant followed by clipped_group_dequant
+ * (veloxquant_mlx/quantizers/skvq.py:105-183) together with the channel gather and inverse
+ * gather around them in SKVQKVCache._round_trip (veloxquant_mlx/cache/skvq_cache.py:236-251).
+ * x/out: B*H slabs of [r, D] rows, slab b*H+h at element offset (b*H+h)*stride_bh; same dtype;
+ * out may alias x.  perm: device int32 [H, D] channel order per head, or NULL for the identity.
+ * alphas: host array of n_alphas (1..8) clip factors in (0, 1]. */
+int vq_skvq_clipped_roundtrip(const void *x, void *out, int dtype, int64_t B, int64_t H, int64_t r, int64_t D,
+                              int64_t x_stride_bh, int64_t out_stride_bh, const int32_t *perm, int bits,
+                              int group, const float *alphas, int n_alphas, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -46,4 +46,19 @@ class AgeTieredKVOptions:
     age_group_size: int = 32
 
 
-__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions", "AgeTieredKVOptions"]
+@dataclass
+class SKVQOptions:
+    """SKVQ configuration (sliding window, channel reorder, clipped groups; options.py in the reference)."""
+
+    skvq_bits_key: int = 4
+    skvq_bits_value: int = 4
+    skvq_group_size: int = 32
+    skvq_window: int = 128
+    skvq_n_sink: int = 5
+    skvq_reorder: bool = True
+    skvq_clip_search: bool = True
+    skvq_clip_alpha: float = 1.0
+    skvq_max_ctx: int | None = None
+
+
+__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions", "AgeTieredKVOptions", "SKVQOptions"]

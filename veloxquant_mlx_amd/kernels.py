@@ -94,6 +94,61 @@ def kivi_group_quant_dequant(x: torch.Tensor, axis: int, group_size: int, levels
     return out.view(x.shape)
 
 
+def skvq_clipped_round_trip(x: torch.Tensor, bits: int, group_size: int, alphas, perm: torch.Tensor | None = None,
+                            out: torch.Tensor | None = None) -> torch.Tensor:
+    """Round-trip ``x [B, H, r, D]`` through SKVQ's clipped group quantisation.
+
+    ``clipped_group_quant`` then ``clipped_group_dequant`` (veloxquant_mlx/quantizers/skvq.py:105-183)
+    on the channels taken in the order ``perm [H, D]`` (int32; ``None`` = as stored), with the result
+    put back on the channels it came from, as ``SKVQKVCache._round_trip`` does
+    (veloxquant_mlx/cache/skvq_cache.py:236-251).  ``x`` may be a token slice of a larger
+    ``[B, H, cap, D]`` buffer; ``out`` (same shape and dtype, may be ``x`` itself) likewise.
+    """
+    name = "skvq_clipped_round_trip"
+    if x.ndim != 4:
+        raise ValueError(f"{name}: x must be [B, H, r, D], got {tuple(x.shape)}")
+    if not 1 <= int(bits) <= 8:
+        raise ValueError(f"{name}: bits must be in [1, 8], got {bits}")
+    if group_size < 1:
+        raise ValueError(f"{name}: group_size must be >= 1, got {group_size}")
+    al = [float(a) for a in alphas]
+    if not al or len(al) > 8 or any(not 0.0 < a <= 1.0 for a in al):
+        raise ValueError(f"{name}: alphas must be 1..8 values in (0, 1], got {al}")
+    tag = _ftag(name, x)
+    B, H, r, D = x.shape
+
+    def slab(t: torch.Tensor, what: str) -> int:
+        """Elements between consecutive (b, h) slabs of a token slice of a contiguous [B, H, cap, D] buffer."""
+        st = t.stride()
+        step = st[1] if H > 1 else (st[0] if B > 1 else r * D)
+        ok = (D == 1 or st[3] == 1) and (r == 1 or st[2] == D) and (B == 1 or H == 1 or st[0] == H * st[1]) \
+            and step >= r * D
+        if not ok:
+            raise ValueError(f"{name}: {what} must be a token slice of a contiguous [B, H, cap, D] buffer, strides {st}")
+        return step
+
+    if out is None:
+        out = torch.empty((B, H, r, D), dtype=x.dtype, device=x.device)
+    elif out.shape != x.shape or out.dtype != x.dtype:
+        raise ValueError(f"{name}: out must match x in shape and dtype")
+    if x.numel() == 0:
+        return out
+    _need_gpu(name, x, out)
+    xs, os_ = slab(x, "x"), slab(out, "out")
+    pp = None
+    if perm is not None:
+        if perm.shape != (H, D) or perm.dtype != torch.int32:
+            raise ValueError(f"{name}: perm must be int32 [H, D] = {(H, D)}, got {perm.dtype} {tuple(perm.shape)}")
+        _need_gpu(name, perm)
+        perm = perm.contiguous()
+        pp = perm.data_ptr()
+    arr = (_lib.C.c_float * len(al))(*al)
+    rc = _lib.load().vq_skvq_clipped_roundtrip(x.data_ptr(), out.data_ptr(), tag, B, H, r, D, xs, os_, pp, int(bits),
+                                               int(group_size), arr, len(al), _stream(x))
+    _lib.check(rc)
+    return out
+
+
 def kivi_quant_pack(x: torch.Tensor, axis: int, group_size: int, bits: int, *, levels: int | None = None,
                     eps: float = 1e-8, meta_dtype: torch.dtype = torch.float16, v_layout: str = "channel",
                     out: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
