@@ -329,15 +329,16 @@ def _extras(torch, K, dev):
     # SKVQ flush arithmetic: clipped group round trip with the five-factor clip search and a per-head channel order
     from veloxquant_mlx_amd.quantizers.skvq import DEFAULT_ALPHA_GRID
     perm = torch.stack([torch.randperm(D, device=dev) for _ in range(Hkv)]).to(torch.int32)
+    sk_inv = torch.argsort(perm.long(), dim=-1).to(torch.int32)
     sk_out = torch.empty_like(kk)
-    fn = lambda: K.skvq_clipped_round_trip(kk, 4, 32, DEFAULT_ALPHA_GRID, perm=perm, out=sk_out)
+    fn = lambda: K.skvq_clipped_round_trip(kk, 4, 32, DEFAULT_ALPHA_GRID, perm=perm, inv=sk_inv, out=sk_out)
     for _ in range(3):
         fn()
     ms = _side_ms(fn, 10, torch)
     ex["skvq_round_trip_[16,8,8192,128]"] = {"ms": round(ms, 5), "GBps": round(nb / ms / 1e6, 1), "bytes": nb,
                                              "note": "fp16 rows in, fp16 reconstruction out, 4-bit, group 32, "
                                                      "five clip factors searched per group, permuted channels"}
-    del sk_out, perm
+    del sk_out, perm, sk_inv
     del kk, kc
     # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,
     # and with the reconstruction written as well

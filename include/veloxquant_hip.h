@@ -325,10 +325,12 @@ int vq_vecinfer_attend(const vq_lut_attend_args *a);
  * gather around them in SKVQKVCache._round_trip (veloxquant_mlx/cache/skvq_cache.py:236-251).
  * x/out: B*H slabs of [r, D] rows, slab b*H+h at element offset (b*H+h)*stride_bh; same dtype;
  * out may alias x.  perm: device int32 [H, D] channel order per head, or NULL for the identity.
+ * inv: optional device int32 [H, D] inverse of perm (inv[h][perm[h][j]] = j); with it rows move as
+ * 16-byte pieces under a channel order too (results are the same).
  * alphas: host array of n_alphas (1..8) clip factors in (0, 1]. */
 int vq_skvq_clipped_roundtrip(const void *x, void *out, int dtype, int64_t B, int64_t H, int64_t r, int64_t D,
-                              int64_t x_stride_bh, int64_t out_stride_bh, const int32_t *perm, int bits,
-                              int group, const float *alphas, int n_alphas, void *stream);
+                              int64_t x_stride_bh, int64_t out_stride_bh, const int32_t *perm, const int32_t *inv,
+                              int bits, int group, const float *alphas, int n_alphas, void *stream);
 
 #ifdef __cplusplus
 }

@@ -72,6 +72,9 @@ def test_round_trip_kernel_matches_the_oracle_bit_for_bit(dtype, B, H, r, D, bit
     assert out.dtype == dtype and out.shape == xt.shape
     assert torch.equal(out.cpu().view(torch.int16 if dtype != torch.float32 else torch.int32),
                        ref.view(torch.int16 if dtype != torch.float32 else torch.int32))
+    if with_perm:   # with the inverse order the rows move as 16-byte pieces; same bits
+        out_inv = K.skvq_clipped_round_trip(xt, bits, g, o.DEFAULT_ALPHA_GRID, perm=to_dev(perm), inv=to_dev(inv))
+        assert torch.equal(out_inv, out)
     # some group took a clipped window (the search is live), and a single alpha = 1 differs
     plain = K.skvq_clipped_round_trip(xt, bits, g, (1.0,), perm=None if perm is None else to_dev(perm))
     if bits <= 4 and g > 1:
@@ -103,6 +106,8 @@ def test_wrapper_rejects_bad_arguments():
         K.skvq_clipped_round_trip(x, 2, 16, (1.2,))
     with pytest.raises(ValueError, match="perm"):
         K.skvq_clipped_round_trip(x, 2, 16, (1.0,), perm=torch.zeros((2, 64), dtype=torch.int64, device="cuda:0"))
+    with pytest.raises(ValueError, match="inv"):
+        K.skvq_clipped_round_trip(x, 2, 16, (1.0,), inv=torch.zeros((2, 64), dtype=torch.int32, device="cuda:0"))
     with pytest.raises(ValueError, match="token slice"):
         K.skvq_clipped_round_trip(x.transpose(1, 2), 2, 16, (1.0,))
     assert K.skvq_clipped_round_trip(x[:, :, :0], 2, 16, (1.0,)).shape == (1, 2, 0, 64)

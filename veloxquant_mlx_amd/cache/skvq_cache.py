@@ -68,9 +68,8 @@ class SKVQKVCache(FP16KVCache):
 
     # ------------------------------------------------------------------ permutations
     def _round_trip(self, x: torch.Tensor, perm, inv, bits: int, out: torch.Tensor | None = None) -> torch.Tensor:
-        """Reorder -> clipped quantise -> dequantise -> inverse reorder (skvq_cache.py:236-251); the kernel
-        scatters through ``perm``, so ``inv`` is carried for the reference's signature only."""
-        return skvq_round_trip_batched(x, perm, bits, self._group_size, self._alphas, out=out)
+        """Reorder -> clipped quantise -> dequantise -> inverse reorder (skvq_cache.py:236-251), one launch."""
+        return skvq_round_trip_batched(x, perm, bits, self._group_size, self._alphas, out=out, inv=inv)
 
     def _per_head_perms(self, chunk: torch.Tensor, bits: int):
         """Channels of each head sorted by range over the chunk's non-sink rows, kept only where that lowers the

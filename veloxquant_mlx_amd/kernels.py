@@ -95,14 +95,15 @@ def kivi_group_quant_dequant(x: torch.Tensor, axis: int, group_size: int, levels
 
 
 def skvq_clipped_round_trip(x: torch.Tensor, bits: int, group_size: int, alphas, perm: torch.Tensor | None = None,
-                            out: torch.Tensor | None = None) -> torch.Tensor:
+                            out: torch.Tensor | None = None, inv: torch.Tensor | None = None) -> torch.Tensor:
     """Round-trip ``x [B, H, r, D]`` through SKVQ's clipped group quantisation.
 
     ``clipped_group_quant`` then ``clipped_group_dequant`` (veloxquant_mlx/quantizers/skvq.py:105-183)
     on the channels taken in the order ``perm [H, D]`` (int32; ``None`` = as stored), with the result
     put back on the channels it came from, as ``SKVQKVCache._round_trip`` does
     (veloxquant_mlx/cache/skvq_cache.py:236-251).  ``x`` may be a token slice of a larger
-    ``[B, H, cap, D]`` buffer; ``out`` (same shape and dtype, may be ``x`` itself) likewise.
+    ``[B, H, cap, D]`` buffer; ``out`` (same shape and dtype, may be ``x`` itself) likewise.  ``inv``
+    (the inverse of ``perm``, as the cache keeps it) only makes the launch faster.
     """
     name = "skvq_clipped_round_trip"
     if x.ndim != 4:
@@ -142,8 +143,15 @@ def skvq_clipped_round_trip(x: torch.Tensor, bits: int, group_size: int, alphas,
         _need_gpu(name, perm)
         perm = perm.contiguous()
         pp = perm.data_ptr()
+    ip = None
+    if inv is not None:
+        if perm is None or inv.shape != (H, D) or inv.dtype != torch.int32:
+            raise ValueError(f"{name}: inv goes with perm and must be int32 [H, D]")
+        _need_gpu(name, inv)
+        inv = inv.contiguous()
+        ip = inv.data_ptr()
     arr = (_lib.C.c_float * len(al))(*al)
-    rc = _lib.load().vq_skvq_clipped_roundtrip(x.data_ptr(), out.data_ptr(), tag, B, H, r, D, xs, os_, pp, int(bits),
+    rc = _lib.load().vq_skvq_clipped_roundtrip(x.data_ptr(), out.data_ptr(), tag, B, H, r, D, xs, os_, pp, ip, int(bits),
                                                int(group_size), arr, len(al), _stream(x))
     _lib.check(rc)
     return out

@@ -15,11 +15,12 @@ DEFAULT_ALPHA_GRID: tuple = (1.0, 0.97, 0.94, 0.90, 0.85)   # skvq.py:61
 
 
 def skvq_round_trip_batched(x: torch.Tensor, perm: torch.Tensor | None, bits: int, group_size: int,
-                            alphas=DEFAULT_ALPHA_GRID, out: torch.Tensor | None = None) -> torch.Tensor:
+                            alphas=DEFAULT_ALPHA_GRID, out: torch.Tensor | None = None,
+                            inv: torch.Tensor | None = None) -> torch.Tensor:
     """``[B, H, r, D]`` -> same shape and dtype: channels gathered by ``perm [H, D]``, clipped group
     quantise -> dequantise per token, channels put back (skvq.py:105-207 under
     SKVQKVCache._round_trip, veloxquant_mlx/cache/skvq_cache.py:236-251)."""
-    return K.skvq_clipped_round_trip(x, bits, group_size, alphas, perm=perm, out=out)
+    return K.skvq_clipped_round_trip(x, bits, group_size, alphas, perm=perm, out=out, inv=inv)
 
 
 def skvq_compressed_bytes(n_tokens: int, d: int, bits: int, group_size: int) -> int:
