@@ -1,0 +1,88 @@
+"""``method="zipcache"`` on the GPU against ``oracle.zipcache`` (cases of
+veloxquant_mlx/tests/cache/test_zipcache_cache.py); reconstructions bit for bit."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import zipcache as oz
+from tests._gpu import gpu, host, require_gpu, to_dev
+from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+from veloxquant_mlx_amd.cache.zipcache_cache import ZipCacheKVCache
+
+pytestmark = gpu
+
+
+def _kv(B, H, S, D, seed):
+    rng = np.random.default_rng(seed)
+    amp = (1.0 + 0.05 * rng.permutation(S)).astype(np.float32)[None, None, :, None]
+    return ((rng.standard_normal((B, H, S, D)).astype(np.float32) * amp).astype(np.float16),
+            rng.standard_normal((B, H, S, D)).astype(np.float16))
+
+
+def _make(**kw):
+    return KVCacheFactory.create(KVCacheConfig(method="zipcache", head_dim=kw.pop("head_dim", 64), **kw))
+
+
+@pytest.mark.parametrize("B,H,S,D,kw", [
+    (1, 2, 64, 64, {}),
+    (2, 3, 50, 128, dict(zipcache_hi_bits=8, zipcache_lo_bits=3, zipcache_hi_fraction=0.5, zipcache_group_size=16)),
+    (1, 2, 33, 64, dict(zipcache_hi_fraction=0.0)),
+    (1, 2, 33, 64, dict(zipcache_hi_fraction=1.0)),
+    (1, 4, 200, 128, dict(zipcache_quantize_values=False)),
+])
+def test_cache_matches_the_model_bit_for_bit(B, H, S, D, kw):
+    require_gpu()
+    c = _make(head_dim=D, **kw)
+    assert isinstance(c, ZipCacheKVCache) and not hasattr(c, "bits")
+    hb, lb = kw.get("zipcache_hi_bits", 4), kw.get("zipcache_lo_bits", 2)
+    fr, gs = kw.get("zipcache_hi_fraction", 0.2), kw.get("zipcache_group_size", 32)
+    k, v = _kv(B, H, S, D, seed=S)
+    ko, vo = c.update_and_fetch(to_dev(k), to_dev(v))
+    kr, _, (kc, kb, kf) = oz.compress(k, True, hb, lb, fr, gs)
+    assert ko.dtype == torch.float16 and np.array_equal(host(ko).view(np.uint16), kr.view(np.uint16))
+    assert (c.compressed_key_bytes, c.baseline_key_bytes, c.fp16_key_bytes) == (kc, kb, kf)
+    if kw.get("zipcache_quantize_values", True):
+        vr, _, (vc, vb, vf) = oz.compress(v, False, hb, lb, fr, gs)
+        assert np.array_equal(host(vo).view(np.uint16), vr.view(np.uint16))
+        assert (c.compressed_value_bytes, c.baseline_value_bytes, c.fp16_value_bytes) == (vc, vb, vf)
+    else:
+        assert np.array_equal(host(vo), v) and c.compressed_value_bytes == 0 and c.fp16_value_bytes > 0
+    assert c.baseline_key_bytes <= c.compressed_key_bytes < c.fp16_key_bytes and c.compression_ratio > 1.0
+    # decode steps: a single token is its own block (one group, exact at any bit width >= 1 only when constant)
+    for t in range(3):
+        k1, v1 = _kv(B, H, 1, D, seed=100 + t)
+        ko, vo = c.update_and_fetch(to_dev(k1), to_dev(v1))
+        assert np.array_equal(host(ko)[:, :, -1:].view(np.uint16), oz.compress(k1, True, hb, lb, fr, gs)[0].view(np.uint16))
+    assert ko.shape[2] == S + 3 and len(c._ledger) == 2 and c._ledger[-1][1] == 3
+
+
+def test_trim_takes_charges_back_and_nan_chunk_is_reported_by_the_next_call():
+    require_gpu()
+    c = _make()
+    k, v = _kv(1, 2, 32, 64, seed=1)
+    c.update_and_fetch(to_dev(k), to_dev(v))
+    after_prefill = (c.compressed_key_bytes, c.fp16_key_bytes)
+    for t in range(4):
+        c.update_and_fetch(*map(to_dev, _kv(1, 2, 1, 64, seed=50 + t)))
+    assert c.trim(4) == 4 and (c.compressed_key_bytes, c.fp16_key_bytes) == after_prefill and c.offset == 32
+    assert c.trim(16) == 16 and c.fp16_key_bytes == after_prefill[1] // 2     # pro-rated
+    bad = k.copy()
+    bad[0, 0, 3, 5] = np.nan
+    c2 = _make()
+    c2.update_and_fetch(to_dev(bad), to_dev(v))
+    with pytest.raises(ValueError, match="NaN or Inf"):
+        c2.update_and_fetch(*map(to_dev, _kv(1, 2, 1, 64, seed=9)))
+    assert c2.offset == 0 and c2.fp16_key_bytes == 0
+
+
+def test_validation():
+    require_gpu()
+    for bad, what in ((dict(zipcache_hi_fraction=1.5), "zipcache_hi_fraction"), (dict(zipcache_hi_fraction=-0.1), "zipcache_hi_fraction"),
+                      (dict(zipcache_hi_bits=9), "zipcache_hi_bits"), (dict(zipcache_lo_bits=0), "zipcache_lo_bits"),
+                      (dict(zipcache_hi_bits=2, zipcache_lo_bits=4), "must not exceed"),
+                      (dict(zipcache_group_size=0), "zipcache_group_size"), (dict(zipcache_quantize_values=1), "zipcache_quantize_values")):
+        with pytest.raises(ValueError, match=what):
+            _make(**bad)
+    with pytest.raises(ValueError, match=r"\[B, H, S, D\]"):
+        _make()._compress(torch.zeros((2, 4, 8), device="cuda:0"), True)

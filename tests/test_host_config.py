@@ -71,7 +71,7 @@ def test_inlier_bits_warning_for_methods_that_ignore_it():
 
 
 def test_factory_dispatch_and_rejections():
-    assert set(_CACHE_CLASS_BY_METHOD) == {"kivi", "kivi_sink", "kitty", "age_tiered", "skvq", "vecinfer"}
+    assert set(_CACHE_CLASS_BY_METHOD) == {"kivi", "kivi_sink", "kitty", "age_tiered", "skvq", "zipcache", "vecinfer"}
     assert isinstance(KVCacheFactory.create(KVCacheConfig(method="kivi")), KIVIKVCache)
     with pytest.warns(UserWarning, match="random N"):
         assert isinstance(KVCacheFactory.create(KVCacheConfig(method="vecinfer")), VecInferKVCache)

@@ -61,4 +61,15 @@ class SKVQOptions:
     skvq_max_ctx: int | None = None
 
 
-__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions", "AgeTieredKVOptions", "SKVQOptions"]
+@dataclass
+class ZipCacheOptions:
+    """ZipCache-adapted configuration (per-token mixed precision by key norm; options.py in the reference)."""
+
+    zipcache_hi_bits: int = 4
+    zipcache_lo_bits: int = 2
+    zipcache_hi_fraction: float = 0.20
+    zipcache_group_size: int = 32
+    zipcache_quantize_values: bool = True
+
+
+__all__ = ["VecInferOptions", "KIVIOptions", "KittyOptions", "AgeTieredKVOptions", "SKVQOptions", "ZipCacheOptions"]
