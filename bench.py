@@ -339,6 +339,16 @@ def _extras(torch, K, dev):
                                              "note": "fp16 rows in, fp16 reconstruction out, 4-bit, group 32, "
                                                      "five clip factors searched per group, permuted channels"}
     del sk_out, perm, sk_inv
+    # ZipCache-adapted keys: norms, stable ranks, gather, two token-axis round trips (4 / 2 bits), scatter
+    zc = KVCacheFactory.create(KVCacheConfig(method="zipcache", head_dim=D))
+    fn = lambda: zc._compress(kk, True)
+    for _ in range(2):
+        fn()
+    ms = _side_ms(fn, 5, torch)
+    ex["zipcache_keys_[16,8,8192,128]"] = {"ms": round(ms, 5), "GBps": round(nb / ms / 1e6, 1), "bytes": nb,
+                                           "note": "fp16 keys in, fp16 mixed-precision reconstruction out; the routing "
+                                                   "(norms, ranks, gather, scatter) is torch around two kernel launches"}
+    del zc
     del kk, kc
     # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,
     # and with the reconstruction written as well
