@@ -248,14 +248,19 @@ typedef struct vq_attend_args {
      * (cache/kivi_cache.py:206-260) followed by the attention call of the same step. */
     const void *k_new;
     const void *v_new;
+    /* Order in which the decode kernel's waves take token chunks, for this call:
+     * 0 = the process default (vq_kivi_attend_fixed_order), 1 = a fixed order (identical bits
+     * from run to run), 2 = on demand (fastest; the last bits can differ between runs). */
+    int32_t fixed_order;
 } vq_attend_args;
 
 /* The decode kernel balances its waves by handing out token chunks on demand, so the order in
  * which partial sums are formed, and with it the last bits of the output, can differ from one
- * run to the next (well inside the 2e-3 bar).  enable != 0 makes every later vq_kivi_attend
- * of the process deal the chunks in a fixed order instead: identical bits from run to run, a
- * few percent slower.  Returns the previous setting.  No counterpart in the reference (its
- * kernels use a fixed split order); for callers that compare runs bit for bit. */
+ * run to the next (well inside the 2e-3 bar).  enable != 0 changes the process default, which
+ * calls with vq_attend_args.fixed_order == 0 take: chunks are dealt in a fixed order instead,
+ * identical bits from run to run, a few percent slower.  Returns the previous setting.  No
+ * counterpart in the reference (its kernels use a fixed split order); for callers that compare
+ * runs bit for bit. */
 int vq_kivi_attend_fixed_order(int enable);
 
 /* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the

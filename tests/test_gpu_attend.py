@@ -84,6 +84,39 @@ def test_batched_layers_equal_per_layer_calls_bit_for_bit():
         assert torch.equal(out[l], one)
 
 
+def test_packed_layers_folded_into_the_batch_equal_per_layer_calls_bit_for_bit():
+    """The reference asserts batched == per-layer bit-identical
+    (veloxquant_mlx/tests/metal/test_scalar_attend.py:660-707).  Here on the packed MFMA decode
+    path: three layers' packed stores and fp16 tails stacked along the batch axis and attended in
+    one launch, against one launch per layer, with the token chunks dealt in a fixed order and the
+    same split count on both sides."""
+    require_gpu()
+    NL, B, Hq, Hkv, D, b, g, n_packed, n_tail = 3, 2, 8, 2, 128, 2, 32, 1024, 45
+    per = 32 // b
+    layers = []
+    for l in range(NL):
+        k, v = outlier_kv((B, Hkv, n_packed + n_tail, D), seed=70 + l)
+        kt, vt = to_dev(k), to_dev(v)
+        kq = K.kivi_quant_pack(kt[:, :, :n_packed], -2, g, b, meta_dtype=torch.float16)
+        vq = K.kivi_quant_pack(vt[:, :, :n_packed], -1, g, b, meta_dtype=torch.float16, v_layout="token")
+        q = to_dev(np.random.default_rng(80 + l).standard_normal((B, Hq, 1, D)).astype(np.float16))
+        layers.append((q, kq, vq, kt[:, :, n_packed:].contiguous(), vt[:, :, n_packed:].contiguous()))
+    cat = lambda f: torch.cat([f(L) for L in layers]).contiguous()
+    common = dict(n_packed=n_packed, bits=b, group_size=g, v_layout="token", n_tail=n_tail, scale=0.09,
+                  num_splits=4, fixed_order=True)
+    plan = {}
+    out = K.kivi_packed_attend(cat(lambda L: L[0]), k_packed=cat(lambda L: L[1][0]), k_scale=cat(lambda L: L[1][1]),
+                               k_zero=cat(lambda L: L[1][2]), v_packed=cat(lambda L: L[2][0]),
+                               v_scale=cat(lambda L: L[2][1]), v_zero=cat(lambda L: L[2][2]),
+                               k_tail=cat(lambda L: L[3]), v_tail=cat(lambda L: L[4]), _plan_out=plan, **common)
+    assert plan["path"] == 1
+    assert vq[0].shape == (B, Hkv, n_packed // per, D)
+    for l, (q, kq, vq, tk, tv) in enumerate(layers):
+        one = K.kivi_packed_attend(q, k_packed=kq[0], k_scale=kq[1], k_zero=kq[2], v_packed=vq[0], v_scale=vq[1],
+                                   v_zero=vq[2], k_tail=tk, v_tail=tv, **common)
+        assert torch.equal(out[l * B:(l + 1) * B], one), l
+
+
 def test_predecoded_and_flash_prefill_forms():
     require_gpu()
     rng = np.random.default_rng(20)
@@ -169,14 +202,10 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
         # separate merge kernel run the same arithmetic (compared with the token chunks dealt in
         # a fixed order: handed out on demand, the last bits depend on timing); the sync
         # counters end up zero again
-        prev = K.attend_fixed_order(True)
-        try:
-            args = dict(n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k, v_tail=tail_v,
-                        n_tail=n_tail, scale=scale, causal=causal, out_dtype=torch.float32, **kw)
-            out1 = K.kivi_packed_attend(qt, **args)
-            out2 = K.kivi_packed_attend(qt, _single_launch=False, **args)
-        finally:
-            K.attend_fixed_order(prev)
+        args = dict(n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k, v_tail=tail_v,
+                    n_tail=n_tail, scale=scale, causal=causal, out_dtype=torch.float32, fixed_order=True, **kw)
+        out1 = K.kivi_packed_attend(qt, **args)
+        out2 = K.kivi_packed_attend(qt, _single_launch=False, **args)
         assert torch.equal(out1, out2)
         assert float((out - out1).abs().max()) < TOL
         assert int(K._counters(qt.device).abs().sum()) == 0

@@ -153,7 +153,7 @@ def test_packed_state_round_trip_and_prompt_cache_file(mode, bits, g, layout, tm
     from veloxquant_mlx_amd.cache import load_prompt_cache, save_prompt_cache
     kw = dict(bit_width_inlier=bits, kivi_group_size=g, residual_length=128, kivi_value_layout=layout,
               fused_sdpa=mode != "standard", fused_sdpa_memory_bound=mode == "memory_bound")
-    K.attend_fixed_order(True)
+    prev_order = K.attend_fixed_order(True)   # the process default, restored below
     try:
         c = _make(**kw)
         k, v = outlier_kv((2, 2, 333, 128), seed=bits + g)
@@ -193,7 +193,7 @@ def test_packed_state_round_trip_and_prompt_cache_file(mode, bits, g, layout, tm
         empty.state = ()
         assert empty.offset == 0 and empty.empty()
     finally:
-        K.attend_fixed_order(False)
+        K.attend_fixed_order(prev_order)
 
 
 @pytest.mark.parametrize("n_sink", [0, 3])
@@ -327,11 +327,7 @@ def test_config3_decode_at_full_size_against_the_oracle_and_the_vector_kernel():
     assert err < 2e-3
     # chunks handed out on demand: repeated runs agree to rounding; dealt in a fixed order: bit for bit
     assert float((c.fused_sdpa(q, scale).float() - o1).abs().max()) < 2e-3   # fp16 output
-    prev = K.attend_fixed_order(True)
-    try:
-        f1, f2 = K.kivi_packed_attend(q, **kw), K.kivi_packed_attend(q, **kw)
-    finally:
-        K.attend_fixed_order(prev)
+    f1, f2 = K.kivi_packed_attend(q, fixed_order=True, **kw), K.kivi_packed_attend(q, fixed_order=True, **kw)
     assert torch.equal(f1, f2) and float((f1 - o1).abs().max()) < 2e-3
 
     b, per = B - 1, 32 // bits

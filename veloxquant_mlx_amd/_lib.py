@@ -38,6 +38,7 @@ class AttendArgs(C.Structure):
         ("sync_counters", vp),
         ("packed_lens", vp), ("tail_lens", vp),
         ("k_new", vp), ("v_new", vp),
+        ("fixed_order", C.c_int32),
     ]
 
 

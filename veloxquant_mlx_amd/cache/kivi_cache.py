@@ -291,10 +291,13 @@ class KIVIKVCache(FP16KVCache):
             z = self._zero_scalar = torch.zeros((), dtype=keys.dtype, device=keys.device)
         return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
 
-    def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0):
+    def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0,
+                   fixed_order: bool | None = None):
         """Attention of ``q [B,H_q,S_q,D]`` over the packed prefix and the fp16 tail,
         queries aligned to the end of the cache (the contract of
-        ``VecInferKVCache.fused_sdpa``, veloxquant_mlx/cache/vecinfer_cache.py:670-731)."""
+        ``VecInferKVCache.fused_sdpa``, veloxquant_mlx/cache/vecinfer_cache.py:670-731).
+        ``fixed_order=True`` asks for results that are identical from run to run (see
+        :func:`veloxquant_mlx_amd.kernels.kivi_packed_attend`)."""
         if not self._fused_enabled:
             raise RuntimeError("KIVIKVCache.fused_sdpa called but fused_sdpa was not enabled via "
                                "KVCacheConfig.fused_sdpa=True.")
@@ -313,7 +316,7 @@ class KIVIKVCache(FP16KVCache):
         kw = dict(k_packed=self._kp, k_scale=self._ks, k_zero=self._kz, v_packed=self._vp, v_scale=self._vs,
                   v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
                   k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
-                  causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype)
+                  causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order)
         if self._pending is not None:
             try:   # append and attend in one launch (single-query MFMA decode path)
                 out = K.kivi_packed_attend(q, k_new=self._pending[0], v_new=self._pending[1], **kw)

@@ -144,9 +144,11 @@ class LayerStackedKIVICache:
         return 0
 
     # ------------------------------------------------------------------ attention
-    def fused_sdpa_all(self, q: torch.Tensor, scale: float, *, causal: bool = True) -> torch.Tensor:
+    def fused_sdpa_all(self, q: torch.Tensor, scale: float, *, causal: bool = True,
+                       fixed_order: bool | None = None) -> torch.Tensor:
         """Attention of ``q [NL, B, H_q, S_q, D]`` over every layer's cache in one launch; layer
-        ``l``'s queries align to the end of layer ``l``'s tokens."""
+        ``l``'s queries align to the end of layer ``l``'s tokens.  ``fixed_order`` as in
+        ``KIVIKVCache.fused_sdpa``."""
         NL = len(self.layers)
         if q.ndim != 5 or q.shape[0] != NL:
             raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: q must be [NL={NL},B,H_q,S_q,D], got {tuple(q.shape)}")
@@ -186,7 +188,7 @@ class LayerStackedKIVICache:
         kw = dict(k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz, n_packed=max(nq), bits=c0._b,
                   group_size=c0._group_size, v_layout=c0._v_layout, k_tail=tk if max(nt) else None,
                   v_tail=tv if max(nt) else None, n_tail=max(nt), scale=float(scale),
-                  causal=bool(causal) and q.shape[3] > 1, out_dtype=q.dtype, **lens)
+                  causal=bool(causal) and q.shape[3] > 1, out_dtype=q.dtype, fixed_order=fixed_order, **lens)
         qf = q.reshape((NL * B,) + tuple(q.shape[2:]))
         if k_new is not None:
             try:

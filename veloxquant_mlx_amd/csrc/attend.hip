@@ -10,7 +10,7 @@ static std::atomic<int> g_fixed_order{0};
 
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
-    p.fixed_order = g_fixed_order.load(std::memory_order_relaxed);
+    p.fixed_order = a.fixed_order == 1 ? 1 : a.fixed_order == 2 ? 0 : g_fixed_order.load(std::memory_order_relaxed);
     p.path = (a.num_splits >= 0 && mfma_decode_supported(a)) ? 1 : 0;
     p.tail_equiv = 0;
     p.pq = 1;
@@ -73,6 +73,7 @@ static int validate(const vq_attend_args *a, const char *fn) {
                (long long)a->Hkv);
     VQ_REQUIRE(a->n_packed >= 0 && a->n_tail >= 0, VQ_ERR_INVALID, "%s: negative token count", fn);
     VQ_REQUIRE(a->n_packed + a->n_tail >= 1, VQ_ERR_INVALID, "%s: no key/value slots to attend to", fn);
+    VQ_REQUIRE(a->fixed_order >= 0 && a->fixed_order <= 2, VQ_ERR_INVALID, "%s: fixed_order must be 0, 1 or 2", fn);
     VQ_REQUIRE(a->Sq <= a->n_packed + a->n_tail || !a->causal, VQ_ERR_INVALID,
                "%s: S_q=%lld exceeds S_kv=%lld; queries align to the tail of the KV cache", fn, (long long)a->Sq,
                (long long)(a->n_packed + a->n_tail));
@@ -102,7 +103,10 @@ extern "C" int vq_kivi_attend_fixed_order(int enable) {
 }
 
 extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
-    if (!a) return 0;
+    // the plan divides by the shapes: arguments that would not pass vq_kivi_attend need no workspace
+    if (!a || a->B < 1 || a->Hq < 1 || a->Hkv < 1 || a->Sq < 1 || a->D < 1 || a->Hq % a->Hkv != 0 ||
+        a->n_packed < 0 || a->n_tail < 0 || (a->n_packed > 0 && (a->pack_bits < 1 || a->pack_bits > 8 || a->group < 1)))
+        return 0;
     AttendPlan p = plan_attend(*a);
     return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nparts * (size_t)(a->D + 2) * sizeof(float);
 }

@@ -161,12 +161,8 @@ template <int BITS, typename M, int GV> struct Ring {
     // the block has the CU's 160 KB to itself: the waves' rings next to the query image
     static constexpr int BUDGET = (160 * 1024 - MF_QIMG_BYTES - 256) / PK_WAVES;
     static constexpr int bytes_at(int depth) { return depth * SLOT + ((depth + UPG - 1) / UPG) * GROUP_SLOT; }
-#ifdef VQ_X_DEPTH
-    static constexpr int DEPTH = VQ_X_DEPTH;
-#else
     // one slot in use, at least one in flight
     static constexpr int DEPTH = bytes_at(5) <= BUDGET ? 5 : bytes_at(4) <= BUDGET ? 4 : bytes_at(3) <= BUDGET ? 3 : 2;
-#endif
     static constexpr int GROUP_SLOTS = (DEPTH + UPG - 1) / UPG;
     static constexpr int GROUP_OFF = DEPTH * SLOT;
     // copies issued after those of the unit about to be read: DEPTH - 1 later units, of which at
@@ -724,10 +720,14 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     }
 
     // ---- last block of this tile merges the splits (no block ever waits for another).
-    // Partials travel as device-scope stores and loads, so no cache-wide write-back or
-    // invalidate is needed: the barrier below waits until this block's stores are
-    // acknowledged, then one thread takes a ticket.
+    // Partials travel as device-scope (write-through) stores and device-scope loads, so no
+    // cache-wide write-back or invalidate is needed.  What orders them against the ticket:
+    // every thread waits until its own stores (these and the tail's) have been acknowledged
+    // -- stores count in vmcnt on this target, and a barrier alone does not wait for them --
+    // then the barrier collects the block, then one thread takes a ticket.  The merging
+    // block's loads depend on the ticket's value, so they are issued after it returned.
     if (!single_launch) return;
+    wait_copies<0>();
     __syncthreads();
     if (tid == 0)
         s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

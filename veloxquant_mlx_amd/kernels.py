@@ -643,14 +643,17 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
                        num_splits: int = 0, packed_lens: torch.Tensor | None = None,
                        tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
-                       v_new: torch.Tensor | None = None, _plan_out: dict | None = None,
-                       _single_launch: bool = True) -> torch.Tensor:
+                       v_new: torch.Tensor | None = None, fixed_order: bool | None = None,
+                       _plan_out: dict | None = None, _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
     q ``[B,Hq,Sq,D]``; packed buffers as :func:`kivi_quant_pack` lays them out
     with capacity read from their shapes, of which the first ``n_packed`` tokens
     are live; tails ``[B,Hkv,tail_cap,D]`` with ``n_tail`` live tokens.  GQA by
-    repeat-interleave.  ``causal`` aligns queries to the end of the slots."""
+    repeat-interleave.  ``causal`` aligns queries to the end of the slots.
+    ``fixed_order`` (this call only): True deals the decode kernel's token chunks to its waves
+    in a fixed order (identical bits from run to run), False on demand, None takes the process
+    default set by :func:`attend_fixed_order`."""
     name = "kivi_packed_attend"
     if q.ndim != 4:
         raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
@@ -708,6 +711,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
+    a.fixed_order = 0 if fixed_order is None else (1 if fixed_order else 2)
     if (packed_lens is None) != (tail_lens is None):
         raise ValueError(f"{name}: packed_lens and tail_lens go together")
     if packed_lens is not None:
@@ -732,11 +736,11 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         pth, npt = ctypes.c_int(0), ctypes.c_int(0)
         _lib.check(lib.vq_kivi_attend_plan(a, ctypes.byref(pth), ctypes.byref(npt)))
         _plan_out["path"], _plan_out["nparts"] = pth.value, npt.value
+    a.stream = _stream(q)
     need = lib.vq_kivi_attend_workspace(a)
     ws = _workspace(q.device, need)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
     a.sync_counters = _counters(q.device).data_ptr() if _single_launch else None
-    a.stream = _stream(q)
     _lib.check(lib.vq_kivi_attend(a))
     return out
 
