@@ -284,6 +284,17 @@ int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts);
  * flash_prefill_attend (veloxquant_mlx/metal/_flash_prefill.py:171-237). */
 int vq_kivi_attend(const vq_attend_args *a);
 
+/* vq_kivi_attend for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * split partials and the sync counters come from a device array built into the library (8 MiB +
+ * 64 KiB per GPU, held until the process ends); a->workspace, a->workspace_bytes and
+ * a->sync_counters are ignored.  Shapes whose partials exceed 8 MiB (vq_kivi_attend_workspace) or
+ * with more than 16384 (sequence, kv head, row tile) triples return VQ_ERR_WORKSPACE.  The call
+ * itself allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads) race -- serialise them, or use vq_kivi_attend
+ * with a workspace per stream. */
+int vq_kivi_attend_static(const vq_attend_args *a);
+
 /* ---- attention over VecInfer indices ----------------------------------------- */
 
 typedef struct vq_lut_attend_args {

@@ -95,6 +95,7 @@ _SIGNATURES = {
     "vq_kivi_attend_workspace": (sz, [C.POINTER(AttendArgs)]),
     "vq_kivi_attend_plan": (i32, [C.POINTER(AttendArgs), C.POINTER(i32), C.POINTER(i32)]),
     "vq_kivi_attend": (i32, [C.POINTER(AttendArgs)]),
+    "vq_kivi_attend_static": (i32, [C.POINTER(AttendArgs)]),
     "vq_vecinfer_attend_workspace": (sz, [C.POINTER(LutAttendArgs)]),
     "vq_vecinfer_attend": (i32, [C.POINTER(LutAttendArgs)]),
 }

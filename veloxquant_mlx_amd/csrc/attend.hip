@@ -3,6 +3,7 @@
 #include "attend.hpp"
 
 #include <atomic>
+#include <mutex>
 
 namespace vq {
 
@@ -159,4 +160,54 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a) {
     rc = launch_attend_merge(*a, p.nparts);
     VQ_HIP_CHECK_LAUNCH(fn);
     return rc;
+}
+
+// ---------------------------------------------------------------------------
+// vq_kivi_attend for callers that cannot allocate: the split partials and the sync counters
+// live in a file-scope device array instead of a caller-provided workspace.
+// ---------------------------------------------------------------------------
+namespace {
+constexpr size_t STATIC_WS_BYTES = (size_t)8 << 20;   // split partials
+constexpr size_t STATIC_COUNTERS = 16384;             // int32 sync counters, one per (sequence, kv head, row tile)
+// Every GPU the library runs on holds its own copy of this array until the process ends.  In host
+// code the array's name is only a stand-in: the address kernels may use comes from
+// hipGetSymbolAddress, per device.
+static __device__ __align__(256) unsigned char scratch[STATIC_WS_BYTES + STATIC_COUNTERS * sizeof(int32_t)];
+std::mutex g_scratch_mutex;
+unsigned char *g_scratch_ptr[64] = {};
+}  // namespace
+
+extern "C" int vq_kivi_attend_static(const vq_attend_args *a) {
+    const char *fn = "vq_kivi_attend_static";
+    int rc = validate(a, fn);
+    if (rc != VQ_OK) return rc;
+    const size_t need = vq_kivi_attend_workspace(a);
+    VQ_REQUIRE(need <= STATIC_WS_BYTES, VQ_ERR_WORKSPACE,
+               "%s: these shapes need %zu bytes of split partials, the built-in scratch holds %zu; use vq_kivi_attend "
+               "with a workspace of its own", fn, need, STATIC_WS_BYTES);
+    const AttendPlan p = plan_attend(*a);
+    VQ_REQUIRE((size_t)(a->B * a->Hkv * p.tiles) <= STATIC_COUNTERS, VQ_ERR_WORKSPACE,
+               "%s: B * H_kv * row tiles = %lld exceeds the %zu built-in sync counters", fn,
+               (long long)(a->B * a->Hkv * p.tiles), STATIC_COUNTERS);
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    VQ_REQUIRE(e == hipSuccess && dev >= 0 && dev < 64, VQ_ERR_HIP, "%s: no current device (%s)", fn, hipGetErrorString(e));
+    unsigned char *ptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_ptr[dev] == nullptr) {   // once per device, with that device current
+            void *sym = nullptr;
+            e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+            VQ_REQUIRE(e == hipSuccess && sym != nullptr, VQ_ERR_HIP, "%s: hipGetSymbolAddress failed: %s", fn,
+                       hipGetErrorString(e));
+            g_scratch_ptr[dev] = static_cast<unsigned char *>(sym);
+        }
+        ptr = g_scratch_ptr[dev];
+    }
+    vq_attend_args b = *a;
+    b.workspace = ptr;
+    b.workspace_bytes = STATIC_WS_BYTES;
+    // the counters start at zero (static storage) and every finished call leaves them at zero
+    b.sync_counters = reinterpret_cast<int32_t *>(ptr + STATIC_WS_BYTES);
+    return vq_kivi_attend(&b);
 }

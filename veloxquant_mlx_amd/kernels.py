@@ -644,6 +644,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        num_splits: int = 0, packed_lens: torch.Tensor | None = None,
                        tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
                        v_new: torch.Tensor | None = None, fixed_order: bool | None = None,
+                       out: torch.Tensor | None = None, static_scratch: bool = False,
                        _plan_out: dict | None = None, _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
@@ -653,7 +654,10 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     repeat-interleave.  ``causal`` aligns queries to the end of the slots.
     ``fixed_order`` (this call only): True deals the decode kernel's token chunks to its waves
     in a fixed order (identical bits from run to run), False on demand, None takes the process
-    default set by :func:`attend_fixed_order`."""
+    default set by :func:`attend_fixed_order`.  ``out`` receives the result when given (a
+    contiguous ``[B,Hq,Sq,D]`` tensor).  ``static_scratch=True`` goes through
+    ``vq_kivi_attend_static``: the library's built-in scratch instead of a torch workspace, for
+    callers that may not allocate (give ``out`` too; calls on one GPU must not overlap)."""
     name = "kivi_packed_attend"
     if q.ndim != 4:
         raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
@@ -663,7 +667,12 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     if out_dtype is None:
         out_dtype = q.dtype
     a = AttendArgs()
-    out = torch.empty((B, Hq, Sq, D), dtype=out_dtype, device=q.device)
+    if out is None:
+        out = torch.empty((B, Hq, Sq, D), dtype=out_dtype, device=q.device)
+    elif tuple(out.shape) != (B, Hq, Sq, D) or not out.is_contiguous() or out.device != q.device:
+        raise ValueError(f"{name}: out must be a contiguous [{B}, {Hq}, {Sq}, {D}] tensor on the device of q")
+    else:
+        out_dtype = out.dtype
     a.q, a.out = q.data_ptr(), out.data_ptr()
     a.q_dtype, a.out_dtype = _ftag(name, q), _FLOAT_TAG[out_dtype]
     Hkv = None
@@ -737,6 +746,9 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         _lib.check(lib.vq_kivi_attend_plan(a, ctypes.byref(pth), ctypes.byref(npt)))
         _plan_out["path"], _plan_out["nparts"] = pth.value, npt.value
     a.stream = _stream(q)
+    if static_scratch:
+        _lib.check(lib.vq_kivi_attend_static(a))
+        return out
     need = lib.vq_kivi_attend_workspace(a)
     ws = _workspace(q.device, need)
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
