@@ -11,7 +11,8 @@ static std::atomic<int> g_fixed_order{0};
 
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
-    p.fixed_order = a.fixed_order == 1 ? 1 : a.fixed_order == 2 ? 0 : g_fixed_order.load(std::memory_order_relaxed);
+    // bit 0: fixed chunk order; bit 1 (fixed_order == 3): the decode kernel also waits for every copy in flight
+    p.fixed_order = a.fixed_order == 1 ? 1 : a.fixed_order == 3 ? 3 : a.fixed_order == 2 ? 0 : g_fixed_order.load(std::memory_order_relaxed);
     p.path = (a.num_splits >= 0 && mfma_decode_supported(a)) ? 1 : 0;
     p.tail_equiv = 0;
     p.pq = 1;
@@ -74,7 +75,7 @@ static int validate(const vq_attend_args *a, const char *fn) {
                (long long)a->Hkv);
     VQ_REQUIRE(a->n_packed >= 0 && a->n_tail >= 0, VQ_ERR_INVALID, "%s: negative token count", fn);
     VQ_REQUIRE(a->n_packed + a->n_tail >= 1, VQ_ERR_INVALID, "%s: no key/value slots to attend to", fn);
-    VQ_REQUIRE(a->fixed_order >= 0 && a->fixed_order <= 2, VQ_ERR_INVALID, "%s: fixed_order must be 0, 1 or 2", fn);
+    VQ_REQUIRE(a->fixed_order >= 0 && a->fixed_order <= 3, VQ_ERR_INVALID, "%s: fixed_order must be 0, 1, 2 or 3", fn);
     VQ_REQUIRE(a->Sq <= a->n_packed + a->n_tail || !a->causal, VQ_ERR_INVALID,
                "%s: S_q=%lld exceeds S_kv=%lld; queries align to the tail of the KV cache", fn, (long long)a->Sq,
                (long long)(a->n_packed + a->n_tail));

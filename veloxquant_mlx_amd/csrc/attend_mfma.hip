@@ -34,8 +34,15 @@ bool mfma_decode_supported(const vq_attend_args &a) {
 bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p) {
     hipStream_t st = (hipStream_t)a.stream;
     float *ws = (float *)a.workspace;
-    if (a.meta_dtype == VQ_F16) launch_mfma_packed_f16meta(a, p, ws, st);
-    else launch_mfma_packed_f32meta(a, p, ws, st);
+    // rows a block carries: the GQA group at p.pq positions, padded to 4 or 8
+    const bool wide = (a.Hq / a.Hkv) * p.pq > 4;
+    if (a.meta_dtype == VQ_F16) {
+        if (wide) launch_mfma_packed_f16meta_r8(a, p, ws, st);
+        else launch_mfma_packed_f16meta_r4(a, p, ws, st);
+    } else {
+        if (wide) launch_mfma_packed_f32meta_r8(a, p, ws, st);
+        else launch_mfma_packed_f32meta_r4(a, p, ws, st);
+    }
     return a.sync_counters != nullptr;
 }
 

@@ -25,6 +25,18 @@ __device__ __forceinline__ f16x2 h2(float a) { f16x2 r = {(f16)a, (f16)a}; retur
 // A constant the optimiser must keep in a vector register, so that
 // (w & mask) | magic becomes one v_and_or_b32 (mask in a scalar register).
 __device__ __forceinline__ u32 vreg_const(u32 x) { asm volatile("" : "+v"(x)); return x; }
+// The fp16 high part of a float32 product, pinned to the value that sits in the register.  Without
+// the barrier the compiler is free to evaluate `(f16)(a * b)` twice in two ways -- a float32
+// multiply followed by a conversion (two roundings) where the pair is packed, and a mixed-precision
+// fused multiply-add that rounds the exact product once (v_fma_mixlo_f16) where a single element
+// is widened again.  When the float32 product lies exactly half-way between two fp16 numbers the
+// two disagree by one fp16 step, and a remainder `t - (float)hi` formed from the second no longer
+// complements the high part stored from the first (error 2^-11 relative instead of 2^-22).
+__device__ __forceinline__ f16x2 pinned_h2(f16x2 h) {
+    u32 u = __builtin_bit_cast(u32, h);
+    asm volatile("" : "+v"(u));
+    return __builtin_bit_cast(f16x2, u);
+}
 // {lo half of a, lo half of b} and {hi half of a, hi half of b}
 __device__ __forceinline__ u32 pair_lo(u32 a, u32 b) { return __builtin_amdgcn_perm(b, a, 0x05040100u); }
 __device__ __forceinline__ u32 pair_hi(u32 a, u32 b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
@@ -261,12 +273,13 @@ __device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool b
 }
 
 // NW waves per block.  s_m, s_l: [NW][MF_ROWS] floats; s_o: [NW][MF_ROWS][MF_D] floats of
-// block-shared memory.  s_qraw: the query rows of this kv head as fp16 [MF_ROWS][MF_D] (rows >= R
-// zero); it may alias s_o: it is read into registers before s_o is written.
+// block-shared memory.  s_qraw: the query rows of this kv head as fp16, q_stride halves apart (rows
+// the tile does not have are zero or absent); it may alias s_o: it is read into registers before
+// s_o is written.
 template <int NW>
 __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, const RowTile &tile, float c, int slot,
                                            int nparts, float *__restrict__ ws, float *s_m, float *s_l, float *s_o,
-                                           const f16 *s_qraw, int tid, int wave, bool device_scope) {
+                                           const f16 *s_qraw, int q_stride, int tid, int wave, bool device_scope) {
     const int lane = tid & 63, i = lane & 15, blk = lane >> 4;
     const int R = tile.RT;
     // tail tokens this lane's query row sees
@@ -281,7 +294,10 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
     const int64_t tbase = bh * a.tail_cap * MF_D;
     f16x8 qT[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * MF_D + 32 * blk + 8 * ks);
+    for (int ks = 0; ks < 4; ++ks) {
+        qT[ks] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (i < R) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * q_stride + 32 * blk + 8 * ks);
+    }
     __syncthreads();   // s_qraw may alias s_o
     const f16x8 ones = ones8();
     const int n_tu = (int)((a.n_tail + 31) / 32);
@@ -400,7 +416,10 @@ __device__ __forceinline__ void merge_rows(const vq_attend_args &a, const RowTil
 
 // launchers of the packed-prefix kernel (it also runs the fp16 tail and, given sync counters,
 // the final merge); partials are [rows][nparts][MF_PART] floats of (max, sum, accumulator)
-void launch_mfma_packed_f16meta(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
-void launch_mfma_packed_f32meta(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+// (one translation unit per scale / zero type and per number of query rows a block carries: 4 or 8)
+void launch_mfma_packed_f16meta_r4(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_f16meta_r8(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_f32meta_r4(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_f32meta_r8(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
 
 }  // namespace vq

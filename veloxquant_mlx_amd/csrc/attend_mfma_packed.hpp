@@ -6,44 +6,46 @@
 // constant by one and-or per two codes (value = offset + code, exact), and every
 // affine term is pushed onto the matrix unit:
 //
-//   scores   S^T[token, row] = sum_d (off + c_td) (q s)_d          A = codes, B = folded query
-//                            + sum_d z_d q_d - off * sum_d (q s)_d   the accumulator the product starts from
-//   output   O[row, chan]    = sum_t (P s_g)[row, t] (off + c_t,chan)     A = P scaled per channel group (hi + remainder)
-//                            - off * sum_t P[row, t] s_g[t]          extra tile, A = P, B = value scales
-//                                                                    (float32 scale / zero: against ones, same A)
-//                            + sum_t P[row, t] z_g[t]                same tile, B = value zeros
-//   denominator               sum_t P[row, t]                        extra tile against ones
+//   scores   S^T[token, col]  = sum_d (off + c_td) (q s)_d           A = codes, B = folded query
+//                             + sum_d z_d q_d - off * sum_d s_d q_d    the accumulator the product starts from
+//   output   O^T[chan, col]   = sum_t (off + c_t,chan) (P s_g)[t, col]   A = codes, B = P scaled by the column's
+//                                                                      channel group (hi + remainder)
+//   sums     Z[i, col]        = sum_t A_z[i, t] P[t, col]             rows i: value zeros of group i, value
+//                                                                      scales of group i, ones (the denominator)
 //
-// Keys (per-channel scale s_d, zero z_d per token group): the scale is folded into
-// the query, carried as an fp16 high part in columns [0, R) of the 16-wide tile and
-// the exact fp16 remainder in columns [R, 2R), so the product is as accurate as a
-// float32 one although keys carry outlier channels; the two columns are added with
-// one DPP add per score.  The per-group row bias is itself a small MFMA chain
-// (A = the group's zeros / a constant -off, B = the query) whose result seeds the
-// score accumulators, so opening a token group costs no reductions.
+// The 16 columns of a tile carry the RTP (4 or 8) query rows of the block several times over:
+//   * first product: column n is query row n % RTP; columns with (n / RTP) even hold the fp16
+//     high part of q*s, those with (n / RTP) odd its exact fp16 remainder, so the product is as
+//     accurate as a float32 one although keys carry outlier channels.  One DPP add (rotate the
+//     row of 16 lanes by RTP) gives EVERY column the full score of its row.
+//   * second product: column n stands for (channel group (n / RTP) % GPP, row n % RTP): the lane
+//     scales its probabilities by the value scale of ITS group only -- one operand serves all
+//     channel groups at once, and a tile of 16 channels reads the columns of its own group.
+//     (Per-token value scales cost 8 packed operations per unit this way, whatever the number
+//     of groups.)
+// Accumulators therefore sit as [channel][column]: a rescale of the running maximum is a
+// per-lane factor, no cross-lane traffic.
 //
-// Values (per-token scale s_g[t], zero z_g[t] per channel group g): the scale is
-// folded into the probabilities (fp16 product plus its exact fp16 remainder, so that a
-// sharply peaked softmax still returns code*scale+zero to float32 accuracy).  A value
-// tile covers 16 consecutive channels, which lie in one group.
+// Opening a token group (keys: per-channel scale s_d, zero z_d per group of tokens) is shared
+// work of the wave: every lane forms q*s (high part and remainder) for eight channels of one
+// row, the pieces go through a small LDS image and come back in operand order; the row bias is
+// one MFMA chain with the group's zeros in operand rows 0-7 and its scales in rows 8-15.
 //
-// Query rows (the H_q/H_kv heads sharing the kv head) sit in the 16-wide M/N
-// dimension.  Keys are packed along channels, so a lane's eight k-slots of the
-// first product are eight channels of one token; values are packed along tokens
-// (VQ_V_TOKEN_PACKED), so a lane's eight k-slots of the second product are eight
-// tokens of one channel; token rows of the two score tiles interleave so that the
-// accumulator layout of S^T is the A-operand layout of P.
+// Keys are packed along channels, so a lane's eight k-slots of the first product are eight
+// channels of one token; values are packed along tokens (VQ_V_TOKEN_PACKED), so a lane's eight
+// k-slots of the second product are eight tokens of one channel; token rows of the two score
+// tiles interleave so that the accumulator layout of S^T is the B-operand layout of P.
 //
-// Every wave streams its units through its own ring of LDS slots, filled by copies
-// that go from global memory straight into LDS and run DEPTH - 1 units ahead of the
-// arithmetic: the bytes in flight per wave are set by the ring, not by the register
-// file, and a unit is read into registers only when its turn comes.  The softmax
-// keeps a lazily updated reference maximum, so the common path has no cross-lane
-// traffic at all.
+// Every wave streams its units through its own ring of LDS slots, filled by copies that go
+// from global memory straight into LDS: a slot is refilled as soon as its unit has been read
+// into registers, so DEPTH units are in flight behind the arithmetic; the bytes in flight per
+// wave are set by the ring, not by the register file.  The softmax keeps a lazily updated
+// reference maximum, so the common path has no cross-lane traffic at all.
 #pragma once
 #include "attend_mfma.hpp"
 
 namespace vq {
+
 
 // One block of PK_WAVES waves per CU (two waves per SIMD, the register file split in two).
 constexpr int PK_WAVES = 8;
@@ -77,77 +79,53 @@ template <> struct TokMeta<float> {
     __device__ __forceinline__ float hi(int p) const { return p == 0 ? b.x : p == 1 ? b.y : p == 2 ? b.z : b.w; }
 };
 
-// ---- key scale / zero of a lane's 32 channels for one token group, memory order
-template <typename M> struct ChanMeta;
-template <> struct ChanMeta<f16> {
-    uint4 s[4], z[4];
-    __device__ __forceinline__ void read(const char *sp, const char *zp) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            s[j] = *reinterpret_cast<const uint4 *>(sp + 16 * j);
-            z[j] = *reinterpret_cast<const uint4 *>(zp + 16 * j);
-        }
-    }
-    __device__ __forceinline__ u32 sword(int w) const {   // channels 2w, 2w+1
-        const uint4 &q = s[w / 4];
-        return w % 4 == 0 ? q.x : w % 4 == 1 ? q.y : w % 4 == 2 ? q.z : q.w;
-    }
-    // {scale[lo], scale[hi]} for two channels of equal parity
-    __device__ __forceinline__ u32 spair(int lo, int hi) const {
-        return (lo & 1) ? pair_hi(sword(lo / 2), sword(hi / 2)) : pair_lo(sword(lo / 2), sword(hi / 2));
-    }
-};
-template <> struct ChanMeta<float> {
-    float4 s[8], z[8];
-    __device__ __forceinline__ void read(const char *sp, const char *zp) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            s[j] = *reinterpret_cast<const float4 *>(sp + 16 * j);
-            z[j] = *reinterpret_cast<const float4 *>(zp + 16 * j);
-        }
-    }
-    static __device__ __forceinline__ float pick(const float4 &q, int e) { return e == 0 ? q.x : e == 1 ? q.y : e == 2 ? q.z : q.w; }
-    __device__ __forceinline__ float sval(int ch) const { return pick(s[ch / 4], ch % 4); }
-    __device__ __forceinline__ float zval(int ch) const { return pick(z[ch / 4], ch % 4); }
+// How the 16 columns of the second product map to channel groups: GPP groups per probability
+// operand, NP operands per unit, TPP value tiles (of 16 channels) per operand.
+template <int GV, int RTP> struct Cols {
+    static constexpr int GPP = GV < 16 / RTP ? GV : 16 / RTP;
+    static constexpr int NP = GV / GPP;
+    static constexpr int TPG = 8 / GV;
+    static constexpr int TPP = 8 / NP;
 };
 
-// Per-wave state of the packed kernel.  GV = channel groups per value row.
-template <int GV, bool OFF_TILES> struct PackedAcc {
-    f32x4 O[8];     // tile nt: channels 16*nt + n, still carrying off * sum_t (P s_g)[row, t]
-    f32x4 Z;        // column g < GV: sum_t P[row, t] z_g[t]; column GV + g: sum_t P[row, t] s_g[t]
-    f32x4 Off[OFF_TILES ? GV : 1];  // float32 scale / zero only: sum_t (P s_g)[row, t] from the same A operands, every column alike
-    f32x4 L;        // sum_t P[row, t], every column alike
-    float m_run;    // softmax reference, log2 domain, per lane column (query row)
+// Per-wave state of the packed kernel.
+template <int NP, bool OFF_TILES> struct PackedAcc {
+    f32x4 O[8];     // tile nt, register r: channel 16*nt + 4*blk + r of the lane's column, still carrying
+                    // off * sum_t (P s_g)[t]
+    f32x4 Z;        // register r = operand row 4*blk + r: sum_t P z_g (rows g < GV), sum_t P s_g (rows GV + g),
+                    // sum_t P (rows >= 8)
+    f32x4 Off[OFF_TILES ? NP : 1];   // float32 scale / zero only: sum_t (P s_g)[t] from the very operands of O
+    float m_run;    // softmax reference, log2 domain, of the lane's column (query row)
 };
 
-template <int BITS, typename M, int GV> struct PackedUnit {
+template <int BITS, typename M, int NP> struct PackedUnit {
     u32 kw[2][(MF_D * BITS / 32) / 4];   // key words of the lane's 32 channels, two token rows
     u32 vw[8];                           // value words, one per 16-channel tile
-    TokMeta<M> s[GV];                    // value scales of the lane's eight tokens, every group
-    TokMeta<M> z;                        // lane column n < GV: value zeros of group n, else value scales of
-                                         // group n % GV, of the lane's eight tokens
+    TokMeta<M> s[NP];                    // value scales of the lane's eight tokens, the lane's group of each operand
+    TokMeta<M> z;                        // operand row of the sums product (see PackedAcc::Z)
 };
 
-constexpr int MF_QIMG = 8 * 64;               // uint4 entries of the query image (below)
-constexpr int MF_QIMG_BYTES = MF_QIMG * 16;
+constexpr int PK_QROW = 136;                  // halves between query rows in LDS (128 + 8: rows on different banks)
+constexpr int PK_QIMG_ROW = 272;              // bytes between rows of a wave's folded-query image
 
-// A wave's ring: DEPTH unit slots, then GROUP_SLOTS group slots.  A unit slot holds what every
-// unit needs, as it lies in memory:
+// A wave's ring: DEPTH unit slots, then GROUP_SLOTS group slots, then the folded-query image.
+// A unit slot holds what every unit needs, as it lies in memory:
 //   key codes    32 tokens x 16*BITS bytes (4-bit: lane l's two 16-byte pieces at 16 l and 1024 + 16 l;
 //                2-bit: the 16-byte piece lane l asked for at 16 l)
 //   value codes  the unit's word rows, 512 bytes each
 //   value scale rows (one per channel group, 32 tokens), then value zero rows
 // A group slot holds the key scale and key zero (128 channels each) of a token group; the unit
 // that opens a group brings them along.  Blocks start on a group boundary, so units open a
-// group every UPG units and at most ceil(DEPTH / UPG) group slots are live at a time.
+// group every UPG units.
 // The exchange arrays of the waves (tail, cross-wave merge) share the rings' bytes:
 // accumulators [PK_WAVES][MF_ROWS][MF_D], zero-point sums [PK_WAVES][MF_ROWS][8], maxima and
 // sums [PK_WAVES][MF_ROWS]
 constexpr int EX_O = PK_WAVES * MF_ROWS * MF_D * 4, EX_Z = PK_WAVES * MF_ROWS * 8 * 4, EX_M = PK_WAVES * MF_ROWS * 4;
 constexpr int EX_BYTES = EX_O + EX_Z + 2 * EX_M;
 constexpr int PK_ALIGN = 128;                 // tokens: blocks start on a multiple of the largest token group
+constexpr int PK_STATIC_LDS = 4096;           // query rows, constant rows, counters (static block-shared memory)
 
-template <int BITS, typename M, int GV> struct Ring {
+template <int BITS, typename M, int GV, int RTP> struct Ring {
     static constexpr int MSZ = sizeof(M);
     static constexpr int KB = 512 * BITS, VB = 512 * BITS;
     static constexpr int VMR = GV * 32 * MSZ;      // bytes of the scale rows (and of the zero rows)
@@ -158,35 +136,33 @@ template <int BITS, typename M, int GV> struct Ring {
     static constexpr int VM_COPIES = VMR > 256 ? VMR / 256 : 1, KM_COPIES = KMR / 256;
     static constexpr int UNIT_COPIES = (BITS == 4 ? 4 : 2) + 2 * VM_COPIES, GROUP_COPIES = 2 * KM_COPIES;
     static constexpr int UPG = 4 / GV;             // units per token group
-    // the block has the CU's 160 KB to itself: the waves' rings next to the query image
-    static constexpr int BUDGET = (160 * 1024 - MF_QIMG_BYTES - 256) / PK_WAVES;
-    static constexpr int bytes_at(int depth) { return depth * SLOT + ((depth + UPG - 1) / UPG) * GROUP_SLOT; }
-    // one slot in use, at least one in flight
+    static constexpr int QIMG = 2 * RTP * PK_QIMG_ROW;
+    // the block has the CU's 160 KB to itself
+    static constexpr int BUDGET = (160 * 1024 - PK_STATIC_LDS) / PK_WAVES - QIMG;
+    // a group slot is read only while its group is opened, and refilled by the opener issued
+    // ceil(DEPTH / UPG) openers later -- at the earliest in the same pass, after that read
+    static constexpr int group_slots(int depth) { return (depth + UPG - 1) / UPG; }
+    static constexpr int bytes_at(int depth) { return depth * SLOT + group_slots(depth) * GROUP_SLOT; }
     static constexpr int DEPTH = bytes_at(5) <= BUDGET ? 5 : bytes_at(4) <= BUDGET ? 4 : bytes_at(3) <= BUDGET ? 3 : 2;
-    static constexpr int GROUP_SLOTS = (DEPTH + UPG - 1) / UPG;
+    static constexpr int GROUP_SLOTS = group_slots(DEPTH);
     static constexpr int GROUP_OFF = DEPTH * SLOT;
+    static constexpr int QIMG_OFF = GROUP_OFF + GROUP_SLOTS * GROUP_SLOT;
     // copies issued after those of the unit about to be read: DEPTH - 1 later units, of which at
     // least (DEPTH - 1) / UPG open a group
     static constexpr int LATER = (DEPTH - 1) * UNIT_COPIES + ((DEPTH - 1) / UPG) * GROUP_COPIES;
-    static constexpr int WAVE_BYTES = bytes_at(DEPTH);
+    static constexpr int WAVE_BYTES = QIMG_OFF + QIMG;
     static constexpr int BYTES = PK_WAVES * WAVE_BYTES > EX_BYTES ? PK_WAVES * WAVE_BYTES : EX_BYTES;
     // Units are handed out to the waves in chunks of CHUNK consecutive units: whole token groups,
-    // and at least DEPTH - 1 units, so that the copies never run more than one chunk ahead of
+    // and at least DEPTH units, so that the copies never run more than one chunk ahead of
     // the arithmetic.
-    static constexpr int CHUNK = ((DEPTH - 1 + UPG - 1) / UPG) * UPG;
+    static constexpr int CHUNK = ((DEPTH + UPG - 1) / UPG) * UPG;
+    static_assert(LATER < 64, "the outstanding-copy counter has six bits");
 };
 
-// LDS image of the query, two operand forms of 4 k-steps x 64 lanes each:
-//   [0..3]  memory order, rows in columns [0, R) only       (B operand of the zero-point product)
-//   [4..7]  k-slot pair order, q in columns [0, R) and again in columns [R, 2R)
-// so that  t = [4..7] * s  is the rounded product and  fma([4..7], s, -t)  its exact remainder;
-// columns [0, R) keep the first, columns [R, 2R) the second.
-template <int BITS>
-__device__ __forceinline__ void build_query_image(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw,
-                                                  uint4 *s_q) {
-    const int R = tile.RT;
-    // raw rows: eight consecutive channels per thread, one load each
-    for (int e = tid; e < MF_ROWS * MF_D / 8; e += PK_THREADS) {
+// The query rows of the block as fp16 in LDS, PK_QROW halves apart; rows the tile does not have are zero.
+template <int RTP>
+__device__ __forceinline__ void stage_query(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw) {
+    for (int e = tid; e < RTP * MF_D / 8; e += PK_THREADS) {
         const int row = e / (MF_D / 8), d = 8 * (e % (MF_D / 8));
         f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (tile.valid(row)) {
@@ -197,44 +173,34 @@ __device__ __forceinline__ void build_query_image(const vq_attend_args &a, const
                 for (int j = 0; j < 8; ++j) v[j] = (f16)ldq(a.q, a.q_dtype, i + j);
             }
         }
-        *reinterpret_cast<f16x8 *>(s_qraw + 8 * e) = v;
+        *reinterpret_cast<f16x8 *>(s_qraw + row * PK_QROW + d) = v;
     }
-    __syncthreads();
-    for (int e = tid; e < MF_QIMG; e += PK_THREADS) {
-        const int form = e / 256, ks = (e / 64) % 4, l = e % 64;   // 256 entries per form
-        const int n = l & 15, blk = l >> 4;
-        const int rq = n < R ? n : n - R;
-        const bool hi_col = n < R, lo_col = n >= R && n < 2 * R;
-        f16 v[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            int ch;
-            if (form == 0) ch = 8 * ks + j;
-            else ch = (j & 1) ? kchan_hi<BITS>(ks, j >> 1) : kchan_lo<BITS>(ks, j >> 1);
-            const f16 q = (hi_col || lo_col) ? s_qraw[rq * MF_D + 32 * blk + ch] : (f16)0.f;
-            v[j] = (form == 0 && !hi_col) ? (f16)0.f : q;
-        }
-        f16x8 o = {v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7]};
-        s_q[e] = __builtin_bit_cast(uint4, o);
-    }
-    __syncthreads();
 }
 
-template <int BITS, typename M, int GV>
-__device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, int R, float c, int64_t t_begin,
+// value of lane (lane + N) % 16 of the same row of 16 lanes
+template <int N> __device__ __forceinline__ float row_ror(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 + N, 0xF, 0xF, true));
+}
+
+// order: bit 0 = deal the chunks round robin, bit 1 = wait for every copy in flight instead of the
+// counted ones (a slower, count-free cross-check of the ring's accounting)
+template <int BITS, typename M, int GV, int RTP>
+__device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, float c, int64_t t_begin,
                                              int n_units, int64_t lane_vis, int64_t full_vis, int lane, int wave,
-                                             PackedAcc<GV, sizeof(M) != 2> &acc, const uint4 *s_q, char *ring,
-                                             int *s_next, bool fixed_order) {
+                                             PackedAcc<Cols<GV, RTP>::NP, sizeof(M) != 2> &acc, const f16 *s_qraw,
+                                             const char *s_const, char *ring, int *s_next, int order) {
+    using CL = Cols<GV, RTP>;
     constexpr int PER = 32 / BITS;           // codes per word
     constexpr int KW = MF_D / PER;           // key words per token row
     constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
     constexpr int GAP = vtok_gap<BITS>();
     constexpr int G = MF_D / GV;             // tokens per key group = channels per value group
-    constexpr int TPG = 8 / GV;              // value tiles per channel group
     constexpr u32 MSZ = sizeof(M);
+    constexpr bool F32META = sizeof(M) != 2;
     const int n = lane & 15, blk = lane >> 4;
     const u32 magic = vreg_const(Magic<BITS>::bits);
     const int64_t cap = a.cap_tokens;
+    const bool fixed_order = (order & 1) != 0, wait_all = (order & 2) != 0;
 
     // block-uniform bases, 32-bit per-lane byte offsets
     const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
@@ -244,8 +210,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const char *vsb = (const char *)a.v_scale + bh * GV * cap * MSZ;
     const char *vzb = (const char *)a.v_zero + bh * GV * cap * MSZ;
 
-    using RG = Ring<BITS, M, GV>;
-    using Unit = PackedUnit<BITS, M, GV>;
+    using RG = Ring<BITS, M, GV, RTP>;
+    using Unit = PackedUnit<BITS, M, CL::NP>;
     char *wring = ring + wave * RG::WAVE_BYTES;
     const u32 wring_lds = lds_addr(wring);
     // ---- what a lane copies.  Key codes: token of S^T row n in tile T is vtok_lo(n / 4, n % 4) + T * GAP.
@@ -304,7 +270,14 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const int vrow = BITS == 4 ? blk : blk >> 1;          // word row of the lane's eight tokens
     const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
     const int tok_a = vtok_lo<BITS>(blk, 0);
-    const int zrow = n < GV ? GV + n : n % GV;            // row of the [scale rows | zero rows] image
+    // column n of the second product: channel group vgrp of every probability operand, query row n % RTP
+    const int col_row = n % RTP, col_lo = (n / RTP) & 1, vgrp = (n / RTP) % CL::GPP;
+    // operand row n of the sums product: zeros of group n, scales of group n - GV, ones from row 8 on
+    // (rows 2 GV .. 7 are not used: they read scales).  Byte offset inside a slot, or inside the
+    // block's constants when the row is ones.
+    const bool zs_ones = n >= 8;
+    const int zs_off = (zs_ones ? 0 : (n < GV ? RG::VZ_OFF + n * VROW : RG::VS_OFF + (n < 2 * GV ? n - GV : 0) * VROW)) +
+                       tok_a * (int)MSZ;
     auto read_unit = [&](int slot, Unit &d) VQ_INLINE_LAMBDA {
         const char *sl = wring + slot * RG::SLOT;
         if constexpr (BITS == 4) {
@@ -324,80 +297,127 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         for (int nt = 0; nt < 8; ++nt)
             d.vw[nt] = *reinterpret_cast<const u32 *>(sl + RG::V_OFF + vrow * 512 + (16 * nt + n) * 4);
 #pragma unroll
-        for (int g = 0; g < GV; ++g) d.s[g].read(sl + RG::VS_OFF + g * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
-        d.z.read(sl + RG::VS_OFF + zrow * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
+        for (int p = 0; p < CL::NP; ++p)
+            d.s[p].read(sl + RG::VS_OFF + (p * CL::GPP + vgrp) * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
+        d.z.read((zs_ones ? s_const : sl) + zs_off, GAP * (int)MSZ);
     };
-    auto read_group = [&](int gslot, ChanMeta<M> &km) VQ_INLINE_LAMBDA {
-        const char *gs = wring + RG::GROUP_OFF + gslot * RG::GROUP_SLOT;
-        km.read(gs + 32 * blk * (int)MSZ, gs + RG::KMR + 32 * blk * (int)MSZ);
-    };
+
+    // ---- opening a token group
+    // Writer role: lane w forms q * s for row w / 16 (+ 4 with eight rows), the eight channels of
+    // k-step w % 4 of lane group (w / 4) % 4, and stores the high parts and the remainders as
+    // 16-byte pieces of the folded-query image.  Reader role: lane (n, blk) fetches the four
+    // pieces of its column.
+    constexpr int WR = RTP / 4;                       // rows a lane writes
+    const int w_row = lane >> 4, w_blk = (lane >> 2) & 3, w_ks = lane & 3;
+    // first channel of the piece in k-slot pair order: pair p = (ch0 + p, ch0 + p + PAIR_GAP)
+    constexpr int PAIR_GAP = BITS == 4 ? 4 : 8;
+    const int w_ch0 = 32 * w_blk + (BITS == 4 ? 8 * w_ks : 16 * (w_ks >> 1) + 4 * (w_ks & 1));
+    u32 qpair[WR][4];
+#pragma unroll
+    for (int u = 0; u < WR; ++u)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const f16 *qr = s_qraw + (w_row + 4 * u) * PK_QROW + w_ch0 + p;
+            qpair[u][p] = as_u(f16x2{qr[0], qr[PAIR_GAP]});
+        }
+    char *qimg = wring + RG::QIMG_OFF;
+    const int w_off = w_row * PK_QIMG_ROW + w_blk * 64 + w_ks * 16;
+    const int r_off = (col_lo * RTP + col_row) * PK_QIMG_ROW + blk * 64;
+    // bias chain: operand rows 0-7 carry the group's zeros, rows 8-15 its scales (fp16 scale / zero);
+    // the query rows (high columns only; remainder columns read zeros) are the other operand
+    const f16 *q0_src = col_lo ? reinterpret_cast<const f16 *>(s_const + 256) : s_qraw + col_row * PK_QROW + 32 * blk;
+    const int q0_step = col_lo ? 0 : 8;
 
     f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
     f32x4 bias;    // what the score accumulators start from; every register alike
     const f16x8 ones = ones8();
-    const f16x8 negoff = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair,
-                               Magic<BITS>::neg_off_pair);
 
-    auto open_group = [&](const ChanMeta<M> &km) VQ_INLINE_LAMBDA {
+    auto open_group = [&](int gslot) VQ_INLINE_LAMBDA {
+        const char *gs = wring + RG::GROUP_OFF + gslot * RG::GROUP_SLOT;
         f32x4 bt = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (sizeof(M) == 2) {
+        if constexpr (!F32META) {
+            // ---- folded query, writer role
+            u32 sp[4];
+            if constexpr (BITS == 4) {
+                const uint4 x = *reinterpret_cast<const uint4 *>(gs + w_ch0 * 2);
+                sp[0] = pair_lo(x.x, x.z); sp[1] = pair_hi(x.x, x.z); sp[2] = pair_lo(x.y, x.w); sp[3] = pair_hi(x.y, x.w);
+            } else {
+                const uint2 x = *reinterpret_cast<const uint2 *>(gs + w_ch0 * 2);
+                const uint2 y = *reinterpret_cast<const uint2 *>(gs + (w_ch0 + 8) * 2);
+                sp[0] = pair_lo(x.x, y.x); sp[1] = pair_hi(x.x, y.x); sp[2] = pair_lo(x.y, y.y); sp[3] = pair_hi(x.y, y.y);
+            }
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) bt = VQ_MFMA(as_h8(km.z[ks]), as_h8(s_q[ks * 64 + lane]), bt);
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const uint4 qs = s_q[(4 + ks) * 64 + lane];
-                const u32 qsw[4] = {qs.x, qs.y, qs.z, qs.w};
-                u32 o[4];
+            for (int u = 0; u < WR; ++u) {
+                u32 hi[4], lo[4];
 #pragma unroll
                 for (int p = 0; p < 4; ++p) {
-                    const f16x2 sp = as_h2(km.spair(kchan_lo<BITS>(ks, p), kchan_hi<BITS>(ks, p)));
-                    const f16x2 t = as_h2(qsw[p]) * sp;   // round(q s)
+                    const f16x2 t = as_h2(qpair[u][p]) * as_h2(sp[p]);   // round(q s)
                     // q*s has at most 22 significant bits: the remainder after the fp16
                     // high part is itself an fp16 number, so this fma is exact
-                    const f16x2 rem = __builtin_elementwise_fma(as_h2(qsw[p]), sp, -t);
-                    o[p] = n < R ? as_u(t) : as_u(rem);
+                    hi[p] = as_u(t);
+                    lo[p] = as_u(__builtin_elementwise_fma(as_h2(qpair[u][p]), as_h2(sp[p]), -t));
                 }
-                qB[ks] = as_h8(o[0], o[1], o[2], o[3]);
+                *reinterpret_cast<uint4 *>(qimg + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
+                *reinterpret_cast<uint4 *>(qimg + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
             }
-        } else {
-            // float32 scale / zero: zeros split into an fp16 pair, the folded query formed
-            // in float32 and split the same way
-            f16x8 zh[4], zl[4];
+            // ---- bias chain
+            const char *zs = gs + (n < 8 ? RG::KMR : 0) + 64 * blk;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
+                bt = VQ_MFMA(as_h8(*reinterpret_cast<const uint4 *>(zs + 16 * ks)),
+                             *reinterpret_cast<const f16x8 *>(q0_src + q0_step * ks), bt);
+        } else {
+            // float32 scale / zero: q * s formed in float32 and split into an fp16 pair
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float z = km.zval(8 * ks + j);
-                    zh[ks][j] = (f16)z;
-                    zl[ks][j] = (f16)(z - (float)zh[ks][j]);
+            for (int u = 0; u < WR; ++u) {
+                u32 hi[4], lo[4];
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const float s0 = *reinterpret_cast<const float *>(gs + (w_ch0 + p) * 4);
+                    const float s1 = *reinterpret_cast<const float *>(gs + (w_ch0 + p + PAIR_GAP) * 4);
+                    const float t0 = (float)as_h2(qpair[u][p])[0] * s0, t1 = (float)as_h2(qpair[u][p])[1] * s1;
+                    const f16x2 h = pinned_h2(f16x2{(f16)t0, (f16)t1});
+                    hi[p] = as_u(h);
+                    lo[p] = as_u(f16x2{(f16)(t0 - (float)h[0]), (f16)(t1 - (float)h[1])});
                 }
+                *reinterpret_cast<uint4 *>(qimg + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
+                *reinterpret_cast<uint4 *>(qimg + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
+            }
+            // bias chain: operand rows 0-3 high parts of the zeros, 4-7 their remainders, 8-11 and 12-15
+            // the same of the scales
+            const char *zs = gs + (n < 8 ? RG::KMR : 0) + 128 * blk;
+            const bool rem = (n & 4) != 0;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
-                const f16x8 qz = as_h8(s_q[ks * 64 + lane]);
-                bt = VQ_MFMA(zh[ks], qz, bt);
-                bt = VQ_MFMA(zl[ks], qz, bt);
-            }
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const f16x8 qs = as_h8(s_q[(4 + ks) * 64 + lane]);
+                const float4 x0 = *reinterpret_cast<const float4 *>(zs + 32 * ks);
+                const float4 x1 = *reinterpret_cast<const float4 *>(zs + 32 * ks + 16);
+                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                f16x8 o;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const int ch = (j & 1) ? kchan_hi<BITS>(ks, j >> 1) : kchan_lo<BITS>(ks, j >> 1);
-                    const float t = (float)qs[j] * km.sval(ch);
-                    const f16 hi = (f16)t;
-                    const f16 lo = (f16)(t - (float)hi);
-                    qB[ks][j] = n < R ? hi : lo;
+                    const f16 h = (f16)x[j];
+                    const f16 l = (f16)(x[j] - (float)h);
+                    o[j] = rem ? l : h;
                 }
+                bt = VQ_MFMA(o, *reinterpret_cast<const f16x8 *>(q0_src + q0_step * ks), bt);
             }
+            bt[0] += __shfl_xor(bt[0], 16);   // high part + remainder
         }
+        // lanes 0-31 hold sum z q of their column, lanes 32-63 sum s q
+        const float other = __shfl_xor(bt[0], 32);
+        const float zq = blk < 2 ? bt[0] : other, sq = blk < 2 ? other : bt[0];
+        const float b = zq - Magic<BITS>::off * sq;
+        bias = f32x4{b, b, b, b};
+        // ---- folded query, reader role (the image is this wave's own: its LDS accesses run in order)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) bt = VQ_MFMA(negoff, qB[ks], bt);
-        bias = bt;
+        for (int ks = 0; ks < 4; ++ks) qB[ks] = as_h8(*reinterpret_cast<const uint4 *>(qimg + r_off + 16 * ks));
     };
 
-    // ---- one unit: scores, softmax, output
-    auto compute = [&](const Unit &cur, int64_t base) VQ_INLINE_LAMBDA {
-        f32x4 S[2];
+    // ---- one unit, first half: scores
+    auto scores = [&](const Unit &cur, f32x4 (&S)[2]) VQ_INLINE_LAMBDA {
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
             f16x8 A[4];   // per k-step
@@ -411,22 +431,15 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) S[T] = VQ_MFMA(A[ks], qB[ks], ks == 0 ? bias : S[T]);
         }
-        // column n < R: add the remainder column n + R; other columns idle
-#define VQ_ADD_SHL(N)                                                                         \
-    _Pragma("unroll") for (int T = 0; T < 2; ++T) _Pragma("unroll") for (int r = 0; r < 4; ++r) \
-        S[T][r] += row_shl<N>(S[T][r]);
-        switch (R) {   // block-uniform
-            case 1: VQ_ADD_SHL(1) break;
-            case 2: VQ_ADD_SHL(2) break;
-            case 4: VQ_ADD_SHL(4) break;
-            case 8: VQ_ADD_SHL(8) break;
-            default:
+    };
+
+    // ---- second half: softmax, output
+    auto finish = [&](const Unit &cur, f32x4 (&S)[2], int64_t base) VQ_INLINE_LAMBDA {
+        // high + remainder column: every column ends up with the full score of its row
 #pragma unroll
-                for (int T = 0; T < 2; ++T)
+        for (int T = 0; T < 2; ++T)
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) S[T][r] += __shfl(S[T][r], (lane & ~15) | ((n + R) & 15));
-        }
-#undef VQ_ADD_SHL
+            for (int r = 0; r < 4; ++r) S[T][r] += row_ror<RTP>(S[T][r]);
         // causal edge: tokens this lane's query row does not see (units below full_vis are
         // visible to every row of the tile)
         if (base + 32 > full_vis) {
@@ -446,95 +459,94 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 32));
             const float m_new = fmaxf(acc.m_run, m_seen);
             const float alpha = m_new == -INFINITY ? 1.f : exp2f(acc.m_run - m_new);   // 0 on the first unit
-            float al[4];
+            // accumulators are [channel][column]: the factor is the lane's own
 #pragma unroll
-            for (int r = 0; r < 4; ++r) al[r] = __shfl(alpha, 4 * blk + r);
+            for (int nt = 0; nt < 8; ++nt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
+                for (int r = 0; r < 4; ++r) acc.O[nt][r] *= alpha;
 #pragma unroll
-                for (int nt = 0; nt < 8; ++nt) acc.O[nt][r] *= al[r];
-                acc.Z[r] *= al[r];
-                acc.L[r] *= al[r];
-                if constexpr (sizeof(M) != 2) {
+            for (int r = 0; r < 4; ++r) acc.Z[r] *= alpha;
+            if constexpr (F32META) {
 #pragma unroll
-                    for (int g = 0; g < GV; ++g) acc.Off[g][r] *= al[r];
-                }
+                for (int p = 0; p < CL::NP; ++p)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc.Off[p][r] *= alpha;
             }
             acc.m_run = m_new;
         }
         const float nm = acc.m_run == -INFINITY ? 0.f : -acc.m_run;   // a row with no visible token yet
-        float Pf[2][4];
         u32 P[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            Pf[0][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], c, nm));
-            Pf[1][r] = __builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], c, nm));
-            P[r] = as_u(f16x2{(f16)Pf[0][r], (f16)Pf[1][r]});
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], c, nm));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], c, nm));
+            P[r] = as_u(f16x2{(f16)p0, (f16)p1});
         }
         const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
 
-        // output: per channel group, A = P * s_g as an fp16 high part plus its exact fp16
+        // output: B = P * s_g of the lane's channel group as an fp16 high part plus its exact fp16
         // remainder (P and s have 11 significant bits each), both multiplied into the codes
 #pragma unroll
-        for (int g = 0; g < GV; ++g) {
-            u32 ah[4], al[4];
+        for (int p = 0; p < CL::NP; ++p) {
+            u32 bh[4], bl[4];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                if constexpr (sizeof(M) == 2) {
-                    const f16x2 sp = as_h2(cur.s[g].pair(p));
-                    const f16x2 hi = as_h2(P[p]) * sp;
-                    ah[p] = as_u(hi);
-                    al[p] = as_u(__builtin_elementwise_fma(as_h2(P[p]), sp, -hi));
+            for (int j = 0; j < 4; ++j) {
+                if constexpr (!F32META) {
+                    const f16x2 sp = as_h2(cur.s[p].pair(j));
+                    const f16x2 hi = as_h2(P[j]) * sp;
+                    bh[j] = as_u(hi);
+                    bl[j] = as_u(__builtin_elementwise_fma(as_h2(P[j]), sp, -hi));
                 } else {
-                    const float t0 = (float)as_h2(P[p])[0] * cur.s[g].lo(p), t1 = (float)as_h2(P[p])[1] * cur.s[g].hi(p);
-                    const f16x2 hi = {(f16)t0, (f16)t1};
-                    ah[p] = as_u(hi);
-                    al[p] = as_u(f16x2{(f16)(t0 - (float)hi[0]), (f16)(t1 - (float)hi[1])});
+                    const float t0 = (float)as_h2(P[j])[0] * cur.s[p].lo(j), t1 = (float)as_h2(P[j])[1] * cur.s[p].hi(j);
+                    const f16x2 hi = pinned_h2(f16x2{(f16)t0, (f16)t1});
+                    bh[j] = as_u(hi);
+                    bl[j] = as_u(f16x2{(f16)(t0 - (float)hi[0]), (f16)(t1 - (float)hi[1])});
                 }
             }
-            const f16x8 Ah = as_h8(ah[0], ah[1], ah[2], ah[3]), Al = as_h8(al[0], al[1], al[2], al[3]);
+            const f16x8 Bh = as_h8(bh[0], bh[1], bh[2], bh[3]), Bl = as_h8(bl[0], bl[1], bl[2], bl[3]);
 #pragma unroll
-            for (int j = 0; j < TPG; j += 2) {
-                const int nt = g * TPG + j;
-                f16x8 Bv0, Bv1;
-                if constexpr (BITS == 4) unpack8_pair<4>(cur.vw[nt], cur.vw[nt + 1], magic, Bv0, Bv1);
+            for (int j = 0; j < CL::TPP; j += 2) {
+                const int nt = p * CL::TPP + j;
+                f16x8 Av0, Av1;
+                if constexpr (BITS == 4) unpack8_pair<4>(cur.vw[nt], cur.vw[nt + 1], magic, Av0, Av1);
                 else {
                     const u64 x = pack64(cur.vw[nt], cur.vw[nt + 1]) >> vshift;   // the lane's byte of each 16-token word
-                    unpack8_pair<2>((u32)x, (u32)(x >> 32), magic, Bv0, Bv1);
+                    unpack8_pair<2>((u32)x, (u32)(x >> 32), magic, Av0, Av1);
                 }
-                acc.O[nt] = VQ_MFMA(Ah, Bv0, acc.O[nt]);
-                acc.O[nt] = VQ_MFMA(Al, Bv0, acc.O[nt]);
-                acc.O[nt + 1] = VQ_MFMA(Ah, Bv1, acc.O[nt + 1]);
-                acc.O[nt + 1] = VQ_MFMA(Al, Bv1, acc.O[nt + 1]);
+                acc.O[nt] = VQ_MFMA(Av0, Bh, acc.O[nt]);
+                acc.O[nt] = VQ_MFMA(Av0, Bl, acc.O[nt]);
+                acc.O[nt + 1] = VQ_MFMA(Av1, Bh, acc.O[nt + 1]);
+                acc.O[nt + 1] = VQ_MFMA(Av1, Bl, acc.O[nt + 1]);
             }
-            if constexpr (sizeof(M) != 2) {
-                acc.Off[g] = VQ_MFMA(Ah, ones, acc.Off[g]);
-                acc.Off[g] = VQ_MFMA(Al, ones, acc.Off[g]);
+            if constexpr (F32META) {
+                acc.Off[p] = VQ_MFMA(ones, Bh, acc.Off[p]);
+                acc.Off[p] = VQ_MFMA(ones, Bl, acc.Off[p]);
             }
         }
-        if constexpr (sizeof(M) == 2) {
-            acc.Z = VQ_MFMA(P8, as_h8(cur.z.pair(0), cur.z.pair(1), cur.z.pair(2), cur.z.pair(3)), acc.Z);
+        // sums: operand rows = zeros of each group, scales of each group, ones
+        if constexpr (!F32META) {
+            acc.Z = VQ_MFMA(as_h8(cur.z.pair(0), cur.z.pair(1), cur.z.pair(2), cur.z.pair(3)), P8, acc.Z);
         } else {
             u32 zh[4], zl[4];
 #pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const f16x2 h = {(f16)cur.z.lo(p), (f16)cur.z.hi(p)};
-                zh[p] = as_u(h);
-                zl[p] = as_u(f16x2{(f16)(cur.z.lo(p) - (float)h[0]), (f16)(cur.z.hi(p) - (float)h[1])});
+            for (int j = 0; j < 4; ++j) {
+                const f16x2 h = {(f16)cur.z.lo(j), (f16)cur.z.hi(j)};
+                zh[j] = as_u(h);
+                zl[j] = as_u(f16x2{(f16)(cur.z.lo(j) - (float)h[0]), (f16)(cur.z.hi(j) - (float)h[1])});
             }
-            acc.Z = VQ_MFMA(P8, as_h8(zh[0], zh[1], zh[2], zh[3]), acc.Z);
-            acc.Z = VQ_MFMA(P8, as_h8(zl[0], zl[1], zl[2], zl[3]), acc.Z);
+            acc.Z = VQ_MFMA(as_h8(zh[0], zh[1], zh[2], zh[3]), P8, acc.Z);
+            acc.Z = VQ_MFMA(as_h8(zl[0], zl[1], zl[2], zl[3]), P8, acc.Z);
         }
-        acc.L = VQ_MFMA(P8, ones, acc.L);
     };
 
     // ---- the waves of a block draw chunks of CHUNK units from a shared counter (a wave that
     // is ahead simply draws more), so no wave waits for a slower one until the block's units are
     // used up.  Which wave meets which tokens then depends on timing, and with it the last bits
-    // of the result; `fixed_order` deals the chunks round robin instead.  Copies run DEPTH - 1 units ahead of the arithmetic: `i_*` is where the copies are,
-    // `c_*` where the arithmetic is.  Chunks being at least DEPTH - 1 units long (but for the
-    // block's last), the copies have entered at most two chunks beyond the one being computed:
-    // `c_next`, `c_after` queue them (NONE = nothing queued, END = the block has no more).
+    // of the result; `fixed_order` deals the chunks round robin instead.  Copies run DEPTH units
+    // ahead of the arithmetic: `i_*` is where the copies are, `c_*` where the arithmetic is.
+    // Chunks being at least DEPTH units long (but for the block's last), the copies have entered
+    // at most two chunks beyond the one being computed: `c_next`, `c_after` queue them (NONE =
+    // nothing queued, END = the block has no more).
     constexpr int CH = RG::CHUNK;
     const int n_chunks = (n_units + CH - 1) / CH;
     int dealt = wave;   // fixed order: wave w takes chunks w, w + PK_WAVES, ...
@@ -567,27 +579,30 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             if (i_chunk >= 0) drawn = draw();
         }
     };
-    // the first DEPTH - 1 passes only issue copies
-    for (int pass = 1 - RG::DEPTH; c_chunk >= 0; ++pass) {
-        if (i_chunk >= 0) issue_next();
-        if (pass < 0) continue;
+    // the ring is filled first; from then on a slot is refilled as soon as its unit sits in registers
+    for (int d = 0; d < RG::DEPTH && i_chunk >= 0; ++d) issue_next();
+    while (c_chunk >= 0) {
         // with a full ring exactly DEPTH - 1 units were issued behind the one awaited
-        if (in_flight == RG::DEPTH) wait_copies<RG::LATER>();
+        if (in_flight == RG::DEPTH && !wait_all) wait_copies<RG::LATER>();
         else wait_copies<0>();
         const int u = c_chunk * CH + c_pos;
         Unit cur;
         read_unit(c_slot, cur);
         const bool opens = c_pos % RG::UPG == 0;
-        if (opens) {
-            ChanMeta<M> km;
-            read_group(c_gslot, km);
-            open_group(km);
-        }
+        if (opens) open_group(c_gslot);
         const int cg_next = c_gslot + 1 == RG::GROUP_SLOTS ? 0 : c_gslot + 1;
         c_gslot = opens ? cg_next : c_gslot;
-        compute(cur, t_begin + (int64_t)u * 32);
-        c_slot = c_slot + 1 == RG::DEPTH ? 0 : c_slot + 1;
+        f32x4 S[2];
+        scores(cur, S);
+        // everything of the slot (and of the group slot) has been read: refill it.  The wait is for
+        // LDS reads only, whose results the products above already consumed or are about to.
         --in_flight;
+        if (i_chunk >= 0) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            issue_next();
+        }
+        finish(cur, S, t_begin + (int64_t)u * 32);
+        c_slot = c_slot + 1 == RG::DEPTH ? 0 : c_slot + 1;
         if (++c_pos == chunk_len(c_chunk)) {
             c_chunk = c_next;   // queued by then: the copies are ahead
             c_next = c_after;
@@ -602,11 +617,14 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 // [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)), cut to what the
 // tile sees; block 0 first runs the fp16 tail, whose partial goes to slot nsplit.  With sync
 // counters the block that finishes last for its tile merges the nparts partials into the output.
-template <int BITS, typename M, int GV>
+template <int BITS, typename M, int GV, int RTP>
 __global__ __launch_bounds__(PK_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
-                               int fixed_order, float *__restrict__ ws) {
-    __shared__ uint4 s_q[MF_QIMG];
+                               int order, float *__restrict__ ws) {
+    using CL = Cols<GV, RTP>;
+    // query rows of the block; constants: [0, 128) ones for 32 tokens in the scale / zero type, then zeros
+    __shared__ __align__(16) f16 s_qraw[8 * PK_QROW];
+    __shared__ __align__(16) char s_const[512];
     // the waves' rings; before and after the units the same bytes are the exchange buffer
     // s_o[PK_WAVES][MF_ROWS][MF_D] of the tail and of the cross-wave merge
     extern __shared__ __align__(16) char s_ring[];
@@ -619,6 +637,10 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: loops below stay scalar
     if (tid == 0) s_next = PK_WAVES;   // chunks 0 .. PK_WAVES - 1 are dealt to the waves up front
+    if (tid < 128) {
+        if (sizeof(M) == 2) reinterpret_cast<u32 *>(s_const)[tid] = tid < 16 ? 0x3C003C00u : 0u;
+        else reinterpret_cast<u32 *>(s_const)[tid] = tid < 32 ? __float_as_uint(1.f) : 0u;
+    }
     const int n = lane & 15, blk = lane >> 4;
     const int by = blockIdx.y;
     const int sp = (int)blockIdx.x, nsplit = (int)gridDim.x;
@@ -638,9 +660,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int RT = tile.RT;
 
     const bool single_launch = a.sync_counters != nullptr;
-    // the raw query is staged in the (not yet used) output exchange buffer
-    f16 *s_qraw = reinterpret_cast<f16 *>(&s_o[0][0][0]);
-    build_query_image<BITS>(a, tile, tid, s_qraw, s_q);
+    stage_query<RTP>(a, tile, tid, s_qraw);
     if (sp == 0 && a.k_new != nullptr && a.n_tail >= 1 && tid < 32) {
         // the newest token's key and value rows become the last tail row: 16 pieces of 16 bytes each
         const int piece = tid & 15;
@@ -650,26 +670,26 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
                      (bh * a.tail_cap + a.n_tail - 1) * (MF_D / 8) + piece;
         *dst = *src;
     }
+    __syncthreads();
     if (sp == 0 && nparts > nsplit)   // the launch has a tail slot: filled even when this sequence's tail is empty
-        tail_block<PK_WAVES>(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, tid,
-                             wave, single_launch);
+        tail_block<PK_WAVES>(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, PK_QROW,
+                             tid, wave, single_launch);
 
-    PackedAcc<GV, sizeof(M) != 2> acc;
+    PackedAcc<CL::NP, sizeof(M) != 2> acc;
 #pragma unroll
     for (int nt = 0; nt < 8; ++nt) acc.O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.Z = f32x4{0.f, 0.f, 0.f, 0.f};
-    acc.L = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
     if constexpr (sizeof(M) != 2) {
 #pragma unroll
-        for (int g = 0; g < GV; ++g) acc.Off[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < CL::NP; ++p) acc.Off[p] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
 
     // packed tokens the rows of the tile see: all of them up to full_vis, none from max_vis on
     int64_t full_vis = tile.visible(0), max_vis = tile.visible(RT - 1);
     if (full_vis > a.n_packed) full_vis = a.n_packed;
     if (max_vis > a.n_packed) max_vis = a.n_packed;
-    int64_t lane_vis = tile.visible(n < RT ? n : (n < 2 * RT ? n - RT : 0));
+    int64_t lane_vis = tile.visible(n % RTP < RT ? n % RTP : 0);
     if (lane_vis > a.n_packed) lane_vis = a.n_packed;
 
     int64_t t_begin = (int64_t)sp * split_len - tail_equiv;
@@ -677,24 +697,34 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (t_begin < 0) t_begin = 0;
     if (t_end > (max_vis + 31) / 32 * 32) t_end = (max_vis + 31) / 32 * 32;
     const int n_units = t_end > t_begin ? (int)((t_end - t_begin) / 32) : 0;
-    __syncthreads();   // the query staging and the tail are done with the ring's bytes
-    packed_units<BITS, M, GV>(a, bh, RT, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_q, s_ring,
-                              &s_next, fixed_order != 0);
+    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_qraw, s_const,
+                                   s_ring, &s_next, order);
     __syncthreads();   // every wave has read its last slot
 
-    // ---- merge the waves: accumulator register r of lane (n, blk) is row 4*blk + r,
-    // tile nt column n is channel 16*nt + n
-    if (blk == 0) s_m[wave][n] = acc.m_run;
+    // ---- merge the waves.  Lane (n, blk): column n is query row n % RTP; tile nt, register r is
+    // channel 16*nt + 4*blk + r, valid in the columns of the tile's channel group (first copy)
+    const int col_row = n % RTP, col_set = n / RTP;
+    if (n < RTP && blk == 0) s_m[wave][n] = acc.m_run;
+    if (col_row < RT) {
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int row = 4 * blk + r;
-        if (row < RT) {
-            if (n == 0) s_l[wave][row] = acc.L[r];
-            if (n < 2 * GV) s_z[wave][row][n] = acc.Z[r];
+        for (int nt = 0; nt < 8; ++nt) {
+            const int g = nt / CL::TPG;
+            if (col_set == g % CL::GPP) {
 #pragma unroll
-            for (int nt = 0; nt < 8; ++nt)
-                if constexpr (sizeof(M) == 2) s_o[wave][row][16 * nt + n] = acc.O[nt][r];
-                else s_o[wave][row][16 * nt + n] = acc.O[nt][r] - Magic<BITS>::off * acc.Off[nt / (8 / GV)][r];
+                for (int r = 0; r < 4; ++r) {
+                    float v = acc.O[nt][r];
+                    if constexpr (sizeof(M) != 2) v -= Magic<BITS>::off * acc.Off[g / CL::GPP][r];
+                    s_o[wave][col_row][16 * nt + 4 * blk + r] = v;
+                }
+            }
+        }
+        if (col_set == 0) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * blk + r;
+                if (i < 2 * GV) s_z[wave][col_row][i] = acc.Z[r];
+                if (i == 8) s_l[wave][col_row] = acc.Z[r];
+            }
         }
     }
     __syncthreads();
@@ -737,24 +767,24 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (tid == 0) __hip_atomic_store(a.sync_counters + by, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename M>
+template <typename M, int RTP>
 static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
     const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles)), block(PK_THREADS);
     const int gv = (int)(MF_D / a.group);
     // more than 64 KB of block-shared memory has to be allowed per kernel and device, once
-#define VQ_LAUNCH(BITS, GV)                                                                                       \
-    do {                                                                                                          \
-        constexpr int ring_bytes = Ring<BITS, M, GV>::BYTES;                                                      \
-        static bool allowed[64] = {};                                                                             \
-        int dev = 0;                                                                                              \
-        (void)hipGetDevice(&dev);                                                                                 \
-        if (dev < 0 || dev >= 64 || !allowed[dev]) {                                                              \
-            (void)hipFuncSetAttribute((const void *)attend_mfma_packed_kernel<BITS, M, GV>,                       \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);                    \
-            if (dev >= 0 && dev < 64) allowed[dev] = true;                                                        \
-        }                                                                                                         \
-        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV>), grid, block, ring_bytes, st, a, p.split_len, \
-                           p.tail_equiv, p.nparts, p.pq, p.tiles, p.fixed_order, ws);                             \
+#define VQ_LAUNCH(BITS, GV)                                                                                            \
+    do {                                                                                                               \
+        constexpr int ring_bytes = Ring<BITS, M, GV, RTP>::BYTES;                                                      \
+        static bool allowed[64] = {};                                                                                  \
+        int dev = 0;                                                                                                   \
+        (void)hipGetDevice(&dev);                                                                                      \
+        if (dev < 0 || dev >= 64 || !allowed[dev]) {                                                                   \
+            (void)hipFuncSetAttribute((const void *)attend_mfma_packed_kernel<BITS, M, GV, RTP>,                       \
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);                         \
+            if (dev >= 0 && dev < 64) allowed[dev] = true;                                                             \
+        }                                                                                                              \
+        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV, RTP>), grid, block, ring_bytes, st, a, p.split_len, \
+                           p.tail_equiv, p.nparts, p.pq, p.tiles, p.fixed_order, ws);                                  \
     } while (0)
     if (a.pack_bits == 4) {
         if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);

@@ -720,7 +720,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
-    a.fixed_order = 0 if fixed_order is None else (1 if fixed_order else 2)
+    a.fixed_order = 0 if fixed_order is None else (int(fixed_order) if fixed_order is not True and fixed_order is not False and int(fixed_order) > 2 else (1 if fixed_order else 2))
     if (packed_lens is None) != (tail_lens is None):
         raise ValueError(f"{name}: packed_lens and tail_lens go together")
     if packed_lens is not None:
