@@ -43,6 +43,9 @@ def _parse():
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extras", action="store_true", help="skip the per-kernel side measurements")
     p.add_argument("--only-kernel", action="store_true", help="time the attention kernel loop only (profiling)")
+    p.add_argument("--only", default=None, metavar="NAME",
+                   help="run one side workload in a loop and print its timing (for rocprofv3): "
+                        "decode_2bit_B16, decode_2bit_B1, vq_assign, prefill, quant_pack, quant_dequant")
     p.add_argument("--copy-calib", action="store_true",
                    help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
@@ -104,6 +107,8 @@ def main() -> int:
         print(json.dumps({"copy_bytes_read": 1 << 30, "copy_bytes_written": 1 << 30, "ms": ms,
                           "GBps": (2 << 30) / ms / 1e6}))
         return 0
+    if a.only:
+        return _only(a, torch, K, dev)
     NL, B, Hq, Hkv, D, ctx, bits, g = a.layers, a.batch, 32, 8, 128, a.ctx, a.bits, a.group
     R = 128
     scale = 1.0 / math.sqrt(D)
@@ -210,6 +215,97 @@ def main() -> int:
     return 0
 
 
+def _decode_2bit_case(torch, dev, B):
+    """2-bit group-32 packed cache of 32768 tokens plus the fp16 residual, one query token (the "@32k" target)."""
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+    D, Hq, Hkv = 128, 32, 8
+    cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=2, kivi_group_size=32, residual_length=128,
+                        fused_sdpa=True, fused_sdpa_memory_bound=True)
+    c = KVCacheFactory.create(cfg)
+    for s0 in range(0, 32768 + 128, 8192):
+        n = min(8192, 32768 + 128 - s0)
+        k, v = _synthetic_layer(torch, B, Hkv, n, D, 5 + s0, dev)
+        c.update_and_fetch(k, v)
+    q = torch.randn((B, Hq, 1, D), device=dev).to(torch.float16)
+    return c, (lambda: c.fused_sdpa(q, 1 / math.sqrt(D))), _algorithmic_bytes_per_layer(B, Hkv, 32768, D, 2, 32)
+
+
+def _prefill_case(torch, dev):
+    """Config 4: 8 chunks of 512 bf16 queries over a 4-bit packed prefix of 4096 tokens plus their own,
+    quantise-on-write (group 32, residual 128).  Returns a function that runs one whole pass and
+    gives its milliseconds."""
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+    D, Hq, Hkv = 128, 32, 8
+
+    def prefill_pass():
+        cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=4, kivi_group_size=32, residual_length=128,
+                            fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=8192)
+        c = KVCacheFactory.create(cfg)
+        k, v = _synthetic_layer(torch, 1, Hkv, 4096, D, 77, dev)
+        c.update_and_fetch(k.to(torch.bfloat16), v.to(torch.bfloat16))
+        chunks = []
+        for ci in range(8):
+            k, v = _synthetic_layer(torch, 1, Hkv, 512, D, 78 + ci, dev)
+            chunks.append((k.to(torch.bfloat16), v.to(torch.bfloat16),
+                           torch.randn((1, Hq, 512, D), device=dev).to(torch.bfloat16)))
+        torch.cuda.synchronize()
+        s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s_.record()
+        for k, v, q in chunks:
+            c.update_and_fetch(k, v)
+            c.fused_sdpa(q, 1 / math.sqrt(D), causal=True)
+        e_.record()
+        torch.cuda.synchronize()
+        return s_.elapsed_time(e_)
+    return prefill_pass
+
+
+def _vq_assign_case(torch, K, dev):
+    """Config 2: keys [4, 4096, 256] fp16 with channel outliers, 256 centroids of 8 dims, uint8 indices."""
+    x = (torch.randn((4, 4096, 256), device=dev) * torch.exp(torch.randn(256, device=dev))).to(torch.float16)
+    cb = torch.randn((256, 8), device=dev).to(torch.float16)
+    return x, cb, (lambda: K.vecinfer_quantize_metal(x, cb, 8, index_dtype=torch.uint8))
+
+
+def _only(a, torch, K, dev):
+    """One side workload in a loop, for profilers: prints its average milliseconds."""
+    name = a.only
+    if name in ("decode_2bit_B16", "decode_2bit_B1"):
+        c, fn, nbytes = _decode_2bit_case(torch, dev, 16 if name.endswith("16") else 1)
+    elif name == "vq_assign":
+        x, cb, fn = _vq_assign_case(torch, K, dev)
+        nbytes = None
+    elif name == "prefill":
+        run = _prefill_case(torch, dev)
+        run()
+        ms = min(run() for _ in range(max(1, a.steps)))
+        print(json.dumps({"only": name, "ms": ms}))
+        return 0
+    elif name in ("quant_pack", "quant_dequant"):
+        k, v = _synthetic_layer(torch, 16, 8, 8192, 128, 11, dev)
+        if name == "quant_pack":
+            def fn():
+                K.kivi_quant_pack(k, -2, 32, 4)
+                K.kivi_quant_pack(v, -1, 32, 4, v_layout="token")
+            nbytes = 2 * (k.numel() * 2 + k.numel() // 2 + (k.numel() // 32) * 4)
+        else:
+            def fn():
+                K.kivi_group_quant_dequant(k, -2, 32, 15)
+                K.kivi_group_quant_dequant(v, -1, 32, 15)
+            nbytes = 2 * (k.numel() * 2 + k.numel() * 2)
+    else:
+        print(f"bench.py: unknown --only {name!r}", file=sys.stderr)
+        return 2
+    for _ in range(a.warmup):
+        fn()
+    ms = _event_ms(fn, max(1, a.steps), torch)
+    out = {"only": name, "ms": ms}
+    if nbytes:
+        out["GBps"] = nbytes / ms / 1e6
+    print(json.dumps(out))
+    return 0
+
+
 def _extras(torch, K, dev):
     """Side measurements the metric string also names: 2-bit 32k decode, quantise GB/s,
     VQ assignment MFMA utilisation.  Each is an event-timed loop of one kernel."""
@@ -232,19 +328,10 @@ def _extras(torch, K, dev):
                                "gemm_f16_TFLOPs": round(2 * 8192 ** 3 / ms_g / 1e9, 1)}
     del src, dst, big, ga, gb
     for B in (1, 16):
-        cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=2, kivi_group_size=32, residual_length=128,
-                            fused_sdpa=True, fused_sdpa_memory_bound=True)
-        c = KVCacheFactory.create(cfg)
-        for s0 in range(0, 32768 + 128, 8192):
-            n = min(8192, 32768 + 128 - s0)
-            k, v = _synthetic_layer(torch, B, Hkv, n, D, 5 + s0, dev)
-            c.update_and_fetch(k, v)
-        q = torch.randn((B, Hq, 1, D), device=dev).to(torch.float16)
-        fn = lambda: c.fused_sdpa(q, 1 / math.sqrt(D))
+        c, fn, nbytes = _decode_2bit_case(torch, dev, B)
         for _ in range(3):
             fn()
         ms = _side_ms(fn, 30, torch)
-        nbytes = _algorithmic_bytes_per_layer(B, Hkv, 32768, D, 2, 32)
         ex[f"decode_2bit_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
                                         "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}
         del c
@@ -267,37 +354,16 @@ def _extras(torch, K, dev):
         ex[f"quant_dequant_{name}"] = {"ms": round(ms_rt, 5), "GBps": round(b_rt / ms_rt / 1e6, 1), "bytes": b_rt}
     # config 4: causal prefill of 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
     # tokens plus their own tokens, quantise-on-write (group 32, residual 128)
-    def prefill_pass(timed):
-        cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=4, kivi_group_size=32, residual_length=128,
-                            fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=8192)
-        c = KVCacheFactory.create(cfg)
-        k, v = _synthetic_layer(torch, 1, Hkv, 4096, D, 77, dev)
-        c.update_and_fetch(k.to(torch.bfloat16), v.to(torch.bfloat16))
-        chunks = []
-        for ci in range(8):
-            k, v = _synthetic_layer(torch, 1, Hkv, 512, D, 78 + ci, dev)
-            chunks.append((k.to(torch.bfloat16), v.to(torch.bfloat16),
-                           torch.randn((1, Hq, 512, D), device=dev).to(torch.bfloat16)))
-        torch.cuda.synchronize()
-        s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s_.record()
-        for k, v, q in chunks:
-            c.update_and_fetch(k, v)
-            c.fused_sdpa(q, 1 / math.sqrt(D), causal=True)
-        e_.record()
-        torch.cuda.synchronize()
-        return s_.elapsed_time(e_)
-    prefill_pass(False)
-    ms = min(prefill_pass(True) for _ in range(3))
+    prefill_pass = _prefill_case(torch, dev)
+    prefill_pass()
+    ms = min(prefill_pass() for _ in range(3))
     flops = 412350414848
     ex["prefill_cfg4"] = {"ms": round(ms, 4), "TFLOPs": round(flops / ms / 1e9, 1),
                           "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
                           "note": "8 chunks of 512 queries: quantise-on-write append + attention per chunk; "
                                   "the packed store is sized once by fused_sdpa_max_ctx=8192"}
     # config 2: VQ assignment, keys [4,4096,256], 256 centroids x 8 dims
-    x = (torch.randn((4, 4096, 256), device=dev) * torch.exp(torch.randn(256, device=dev))).to(torch.float16)
-    cb = torch.randn((256, 8), device=dev).to(torch.float16)
-    fn = lambda: K.vecinfer_quantize_metal(x, cb, 8, index_dtype=torch.uint8)
+    x, cb, fn = _vq_assign_case(torch, K, dev)
     for _ in range(3):
         fn()
     ms = _side_ms(fn, 20, torch)

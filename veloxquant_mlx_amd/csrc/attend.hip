@@ -9,6 +9,11 @@ namespace vq {
 
 static std::atomic<int> g_fixed_order{0};
 
+// what a tail token costs the block of split 0, in packed tokens, when the plan balances the splits
+#ifndef VQ_TAIL_EQUIV
+#define VQ_TAIL_EQUIV 2
+#endif
+
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
     // bit 0: fixed chunk order; bit 1 (fixed_order == 3): the decode kernel also waits for every copy in flight
@@ -33,14 +38,13 @@ AttendPlan plan_attend(const vq_attend_args &a) {
         p.nparts = p.nsplit;
         return p;
     }
-    // tokens the kernel splits: the MFMA path hands the tail to the block of split 0 and
-    // prices a tail token at five packed tokens when it balances the splits (the tail pass
-    // is short but latency-bound: about 5 us, the time a block streams 500-800 packed tokens)
+    // tokens the kernel splits: the MFMA path hands the tail to a few waves of the block of split 0
+    // and prices a tail token at VQ_TAIL_EQUIV packed tokens when it balances the splits
     int64_t n_split = a.n_packed + a.n_tail;
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
         p.tiles = (int)cdiv(a.Sq, p.pq);
-                p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * 5, 128) * 128 : 0;
+        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * VQ_TAIL_EQUIV, 128) * 128 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
     // the MFMA kernel wants every block to start on a boundary of the largest token group (128)
@@ -60,7 +64,13 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     if (p.path == 0) ns = n_split > 0 ? cdiv(n_split, len) : 1;
     p.nsplit = (int)ns;
     p.split_len = len;
-    p.nparts = p.nsplit + ((p.path == 1 && a.n_tail > 0) ? 1 : 0);
+    // MFMA decode path: the tail is run by up to eight waves of split 0, two units of 32 tokens each
+    // where there are that many, every wave into a partial of its own
+    p.nparts = p.nsplit;
+    if (p.path == 1 && a.n_tail > 0) {
+        int64_t tw = cdiv(cdiv(a.n_tail, 32), 2);
+        p.nparts += (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw);
+    }
     return p;
 }
 

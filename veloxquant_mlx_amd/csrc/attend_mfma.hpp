@@ -272,15 +272,15 @@ __device__ __forceinline__ f16x8 ld_tail8(const void *base, int64_t elem, bool b
     return tail8_from_raw(*reinterpret_cast<const uint4 *>((const u16 *)base + elem), bf16);
 }
 
-// NW waves per block.  s_m, s_l: [NW][MF_ROWS] floats; s_o: [NW][MF_ROWS][MF_D] floats of
-// block-shared memory.  s_qraw: the query rows of this kv head as fp16, q_stride halves apart (rows
-// the tile does not have are zero or absent); it may alias s_o: it is read into registers before
-// s_o is written.
-template <int NW>
-__device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, const RowTile &tile, float c, int slot,
-                                           int nparts, float *__restrict__ ws, float *s_m, float *s_l, float *s_o,
-                                           const f16 *s_qraw, int q_stride, int tid, int wave, bool device_scope) {
-    const int lane = tid & 63, i = lane & 15, blk = lane >> 4;
+// One wave's share of the tail: units w, w + T, ... of 32 tokens (w = which of the T tail waves this
+// is), written as a partial of its own into slot `slot` straight from the accumulators -- no
+// block-shared memory and no barrier, so the other waves of the block stream the packed prefix
+// meanwhile.  s_qraw: the query rows of this kv head as fp16, q_stride halves apart.  A wave
+// without units (a sequence with a shorter tail) writes an empty partial (max -inf, sum 0).
+__device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, const RowTile &tile, float c, int slot,
+                                          int nparts, float *__restrict__ ws, const f16 *s_qraw, int q_stride, int lane,
+                                          int w, int T, bool device_scope) {
+    const int i = lane & 15, blk = lane >> 4;
     const int R = tile.RT;
     // tail tokens this lane's query row sees
     int64_t n_vis = tile.visible(i < R ? i : 0) - a.n_packed;
@@ -298,7 +298,6 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
         qT[ks] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
         if (i < R) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * q_stride + 32 * blk + 8 * ks);
     }
-    __syncthreads();   // s_qraw may alias s_o
     const f16x8 ones = ones8();
     const int n_tu = (int)((a.n_tail + 31) / 32);
 
@@ -318,10 +317,10 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
     auto load = [&](int u, TUnit &d) {
         const int64_t base = (int64_t)u * 32;
 #pragma unroll
-        for (int T = 0; T < 2; ++T) {
-            const int64_t tok = base + tail_tok(i >> 2, i & 3, T);
+        for (int Tt = 0; Tt < 2; ++Tt) {
+            const int64_t tok = base + tail_tok(i >> 2, i & 3, Tt);
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) d.kr[T][ks] = key_row(tok, 32 * blk + 8 * ks);
+            for (int ks = 0; ks < 4; ++ks) d.kr[Tt][ks] = key_row(tok, 32 * blk + 8 * ks);
         }
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
@@ -333,16 +332,16 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
         const int64_t base = (int64_t)u * 32;
         f32x4 S[2];
 #pragma unroll
-        for (int T = 0; T < 2; ++T) {
-            S[T] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int Tt = 0; Tt < 2; ++Tt) {
+            S[Tt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) S[T] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.kr[T][ks], qT[ks], S[T], 0, 0, 0);
+            for (int ks = 0; ks < 4; ++ks) S[Tt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.kr[Tt][ks], qT[ks], S[Tt], 0, 0, 0);
         }
 #pragma unroll
-        for (int T = 0; T < 2; ++T)
+        for (int Tt = 0; Tt < 2; ++Tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                if (i < R && base + tail_tok(blk, r, T) >= n_vis) S[T][r] = -INFINITY;
+                if (i < R && base + tail_tok(blk, r, Tt) >= n_vis) S[Tt][r] = -INFINITY;
         const f16x8 P = tail_softmax_unit(S, c, acc, blk);
 #pragma unroll
         for (int nt = 0; nt < 8; ++nt) {   // lane column i is channel 8*i + nt
@@ -353,47 +352,26 @@ __device__ __forceinline__ void tail_block(const vq_attend_args &a, int64_t bh, 
         }
         acc.O[8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(P, ones, acc.O[8], 0, 0, 0);
     };
-    // two units of a wave in flight at a time
-    for (int u = wave; u < n_tu; u += 2 * NW) {
+    // two units of the wave in flight at a time
+    for (int u = w; u < n_tu; u += 2 * T) {
         TUnit d0, d1;
         load(u, d0);
-        if (u + NW < n_tu) load(u + NW, d1);
+        if (u + T < n_tu) load(u + T, d1);
         compute(u, d0);
-        if (u + NW < n_tu) compute(u + NW, d1);
+        if (u + T < n_tu) compute(u + T, d1);
     }
-
-    // merge the waves: accumulator register r of lane (i, blk) is row 4*blk + r, channel 8*i + nt
-    if (blk == 0) s_m[wave * MF_ROWS + i] = acc.m_run;
+    // the partial: accumulator register r of lane (i, blk) is row 4*blk + r, channels 8*i .. 8*i + 7;
+    // the maximum of row i sits in lane i of every lane group
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
         const int row = 4 * blk + r;
-        if (row < R) {
-            if (i == 0) s_l[wave * MF_ROWS + row] = acc.O[8][r];
-#pragma unroll
-            for (int nt = 0; nt < 8; ++nt) s_o[(wave * MF_ROWS + row) * MF_D + 8 * i + nt] = acc.O[nt][r];
-        }
-    }
-    __syncthreads();
-    for (int e = tid; e < R * MF_D; e += 64 * NW) {
-        const int row = e / MF_D, d = e % MF_D;
-        float gm = -INFINITY;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) gm = fmaxf(gm, s_m[w * MF_ROWS + row]);
-        float num = 0.f, den = 0.f;
-#pragma unroll
-        for (int w = 0; w < NW; ++w) {
-            const float mw = s_m[w * MF_ROWS + row];
-            if (mw == -INFINITY) continue;
-            const float f = exp2f(mw - gm);
-            num += s_o[(w * MF_ROWS + row) * MF_D + d] * f;
-            den += s_l[w * MF_ROWS + row] * f;
-        }
         if (!tile.valid(row)) continue;
         float *o = ws + (tile.row(row) * nparts + slot) * MF_PART;
-        st_partial(o + 2 + d, num, device_scope);
-        if (d == 0) { st_partial(o, gm * LN2, device_scope); st_partial(o + 1, den, device_scope); }
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) st_partial(o + 2 + 8 * i + nt, acc.O[nt][r], device_scope);
+        if (i == 0) st_partial(o + 1, acc.O[8][r], device_scope);
     }
-    __syncthreads();   // the exchange buffers are free again
+    if (blk == 0 && tile.valid(i)) st_partial(ws + (tile.row(i) * nparts + slot) * MF_PART, acc.m_run * LN2, device_scope);
 }
 
 // Combine the nparts partials of the tile's query rows into the output (the

@@ -48,7 +48,10 @@ namespace vq {
 
 
 // One block of PK_WAVES waves per CU (two waves per SIMD, the register file split in two).
-constexpr int PK_WAVES = 8;
+#ifndef VQ_PK_WAVES
+#define VQ_PK_WAVES 8
+#endif
+constexpr int PK_WAVES = VQ_PK_WAVES;
 constexpr int PK_THREADS = 64 * PK_WAVES;
 // Every lambda below must be inlined at every call: a closure left in memory would be read back
 // with vector loads, whose completion the ring's copy counter cannot tell from its own.
@@ -117,7 +120,7 @@ constexpr int PK_QIMG_ROW = 272;              // bytes between rows of a wave's 
 // A group slot holds the key scale and key zero (128 channels each) of a token group; the unit
 // that opens a group brings them along.  Blocks start on a group boundary, so units open a
 // group every UPG units.
-// The exchange arrays of the waves (tail, cross-wave merge) share the rings' bytes:
+// The exchange arrays of the waves (cross-wave merge) share the rings' bytes:
 // accumulators [PK_WAVES][MF_ROWS][MF_D], zero-point sums [PK_WAVES][MF_ROWS][8], maxima and
 // sums [PK_WAVES][MF_ROWS]
 constexpr int EX_O = PK_WAVES * MF_ROWS * MF_D * 4, EX_Z = PK_WAVES * MF_ROWS * 8 * 4, EX_M = PK_WAVES * MF_ROWS * 4;
@@ -186,7 +189,7 @@ template <int N> __device__ __forceinline__ float row_ror(float x) {
 // counted ones (a slower, count-free cross-check of the ring's accounting)
 template <int BITS, typename M, int GV, int RTP>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, float c, int64_t t_begin,
-                                             int n_units, int64_t lane_vis, int64_t full_vis, int lane, int wave,
+                                             int n_units, int lane_vis, int full_vis, int lane, int wave,
                                              PackedAcc<Cols<GV, RTP>::NP, sizeof(M) != 2> &acc, const f16 *s_qraw,
                                              const char *s_const, char *ring, int *s_next, int order) {
     using CL = Cols<GV, RTP>;
@@ -325,8 +328,12 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const int r_off = (col_lo * RTP + col_row) * PK_QIMG_ROW + blk * 64;
     // bias chain: operand rows 0-7 carry the group's zeros, rows 8-15 its scales (fp16 scale / zero);
     // the query rows (high columns only; remainder columns read zeros) are the other operand
-    const f16 *q0_src = col_lo ? reinterpret_cast<const f16 *>(s_const + 256) : s_qraw + col_row * PK_QROW + 32 * blk;
-    const int q0_step = col_lo ? 0 : 8;
+    f16x8 q0[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        q0[ks] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (!col_lo) q0[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + col_row * PK_QROW + 32 * blk + 8 * ks);
+    }
 
     f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
     f32x4 bias;    // what the score accumulators start from; every register alike
@@ -364,8 +371,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             const char *zs = gs + (n < 8 ? RG::KMR : 0) + 64 * blk;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
-                bt = VQ_MFMA(as_h8(*reinterpret_cast<const uint4 *>(zs + 16 * ks)),
-                             *reinterpret_cast<const f16x8 *>(q0_src + q0_step * ks), bt);
+                bt = VQ_MFMA(as_h8(*reinterpret_cast<const uint4 *>(zs + 16 * ks)), q0[ks], bt);
         } else {
             // float32 scale / zero: q * s formed in float32 and split into an fp16 pair
 #pragma unroll
@@ -399,7 +405,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                     const f16 l = (f16)(x[j] - (float)h);
                     o[j] = rem ? l : h;
                 }
-                bt = VQ_MFMA(o, *reinterpret_cast<const f16x8 *>(q0_src + q0_step * ks), bt);
+                bt = VQ_MFMA(o, q0[ks], bt);
             }
             bt[0] += __shfl_xor(bt[0], 16);   // high part + remainder
         }
@@ -434,20 +440,24 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     };
 
     // ---- second half: softmax, output
-    auto finish = [&](const Unit &cur, f32x4 (&S)[2], int64_t base) VQ_INLINE_LAMBDA {
+    // lane_vis, full_vis, base: token positions counted from the block's first token
+    const int lane_vis0 = lane_vis - tok_a;   // visible tokens counted from the lane's first token of a unit
+    auto finish = [&](const Unit &cur, f32x4 (&S)[2], int base) VQ_INLINE_LAMBDA {
         // high + remainder column: every column ends up with the full score of its row
 #pragma unroll
         for (int T = 0; T < 2; ++T)
 #pragma unroll
             for (int r = 0; r < 4; ++r) S[T][r] += row_ror<RTP>(S[T][r]);
         // causal edge: tokens this lane's query row does not see (units below full_vis are
-        // visible to every row of the tile)
+        // visible to every row of the tile); a real branch, taken by the last units of a block only
         if (base + 32 > full_vis) {
+            asm volatile("" ::: "memory");
+            const int lv = lane_vis0 - base;
 #pragma unroll
             for (int T = 0; T < 2; ++T)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (base + vtok_lo<BITS>(blk, r) + T * GAP >= lane_vis) S[T][r] = -INFINITY;
+                    if (r + T * GAP >= lv) S[T][r] = -INFINITY;
         }
 
         // softmax against a lazily updated reference: the fast path touches no other lane
@@ -514,8 +524,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                     unpack8_pair<2>((u32)x, (u32)(x >> 32), magic, Av0, Av1);
                 }
                 acc.O[nt] = VQ_MFMA(Av0, Bh, acc.O[nt]);
-                acc.O[nt] = VQ_MFMA(Av0, Bl, acc.O[nt]);
                 acc.O[nt + 1] = VQ_MFMA(Av1, Bh, acc.O[nt + 1]);
+                acc.O[nt] = VQ_MFMA(Av0, Bl, acc.O[nt]);
                 acc.O[nt + 1] = VQ_MFMA(Av1, Bl, acc.O[nt + 1]);
             }
             if constexpr (F32META) {
@@ -601,7 +611,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             issue_next();
         }
-        finish(cur, S, t_begin + (int64_t)u * 32);
+        finish(cur, S, u * 32);
         c_slot = c_slot + 1 == RG::DEPTH ? 0 : c_slot + 1;
         if (++c_pos == chunk_len(c_chunk)) {
             c_chunk = c_next;   // queued by then: the copies are ahead
@@ -615,18 +625,19 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 // grid (nsplit, B*Hkv*tiles), PK_THREADS threads.  A block works on one tile of query rows (the GQA
 // group at pq consecutive positions) and on packed tokens
 // [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)), cut to what the
-// tile sees; block 0 first runs the fp16 tail, whose partial goes to slot nsplit.  With sync
-// counters the block that finishes last for its tile merges the nparts partials into the output.
+// tile sees; in the block of split 0 the last nparts - nsplit waves first run the fp16 tail, each
+// into a partial slot of its own.  With sync counters the block that finishes last for its tile
+// merges the nparts partials into the output.
 template <int BITS, typename M, int GV, int RTP>
-__global__ __launch_bounds__(PK_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+__global__ __launch_bounds__(PK_THREADS) __attribute__((amdgpu_waves_per_eu(VQ_PK_WAVES / 4, VQ_PK_WAVES / 4)))
 void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
                                int order, float *__restrict__ ws) {
     using CL = Cols<GV, RTP>;
     // query rows of the block; constants: [0, 128) ones for 32 tokens in the scale / zero type, then zeros
     __shared__ __align__(16) f16 s_qraw[8 * PK_QROW];
     __shared__ __align__(16) char s_const[512];
-    // the waves' rings; before and after the units the same bytes are the exchange buffer
-    // s_o[PK_WAVES][MF_ROWS][MF_D] of the tail and of the cross-wave merge
+    // the waves' rings; after the units the same bytes are the exchange buffer
+    // s_o[PK_WAVES][MF_ROWS][MF_D] of the cross-wave merge
     extern __shared__ __align__(16) char s_ring[];
     float (*s_o)[MF_ROWS][MF_D] = reinterpret_cast<float (*)[MF_ROWS][MF_D]>(s_ring);
     float (*s_z)[MF_ROWS][8] = reinterpret_cast<float (*)[MF_ROWS][8]>(s_ring + EX_O);
@@ -671,9 +682,12 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         *dst = *src;
     }
     __syncthreads();
-    if (sp == 0 && nparts > nsplit)   // the launch has a tail slot: filled even when this sequence's tail is empty
-        tail_block<PK_WAVES>(a, bh, tile, c, nsplit, nparts, ws, &s_m[0][0], &s_l[0][0], &s_o[0][0][0], s_qraw, PK_QROW,
-                             tid, wave, single_launch);
+    // the launch has nparts - nsplit tail slots (filled even when this sequence's tail is empty): the
+    // last waves of split 0 run the tail first, each into a slot of its own, while the others stream
+    const int tail_waves = nparts - nsplit;
+    if (sp == 0 && wave >= PK_WAVES - tail_waves)
+        tail_wave(a, bh, tile, c, nsplit + wave - (PK_WAVES - tail_waves), nparts, ws, s_qraw, PK_QROW, lane,
+                  wave - (PK_WAVES - tail_waves), tail_waves, single_launch);
 
     PackedAcc<CL::NP, sizeof(M) != 2> acc;
 #pragma unroll
@@ -697,7 +711,11 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (t_begin < 0) t_begin = 0;
     if (t_end > (max_vis + 31) / 32 * 32) t_end = (max_vis + 31) / 32 * 32;
     const int n_units = t_end > t_begin ? (int)((t_end - t_begin) / 32) : 0;
-    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_vis, full_vis, lane, wave, acc, s_qraw, s_const,
+    // visibility counted from the block's first token (a block holds fewer than 2^31 tokens)
+    const int64_t rel_cap = (int64_t)n_units * 32 + 64;
+    const int lane_rel = (int)(lane_vis - t_begin < 0 ? 0 : lane_vis - t_begin > rel_cap ? rel_cap : lane_vis - t_begin);
+    const int full_rel = (int)(full_vis - t_begin < 0 ? 0 : full_vis - t_begin > rel_cap ? rel_cap : full_vis - t_begin);
+    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lane, wave, acc, s_qraw, s_const,
                                    s_ring, &s_next, order);
     __syncthreads();   // every wave has read its last slot
 
