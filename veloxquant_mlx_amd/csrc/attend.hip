@@ -10,9 +10,7 @@ namespace vq {
 static std::atomic<int> g_fixed_order{0};
 
 // what a tail token costs the block of split 0, in packed tokens, when the plan balances the splits
-#ifndef VQ_TAIL_EQUIV
-#define VQ_TAIL_EQUIV 2
-#endif
+constexpr int64_t TAIL_EQUIV = 4;
 
 AttendPlan plan_attend(const vq_attend_args &a) {
     AttendPlan p;
@@ -39,12 +37,12 @@ AttendPlan plan_attend(const vq_attend_args &a) {
         return p;
     }
     // tokens the kernel splits: the MFMA path hands the tail to a few waves of the block of split 0
-    // and prices a tail token at VQ_TAIL_EQUIV packed tokens when it balances the splits
+    // and prices a tail token at TAIL_EQUIV packed tokens when it balances the splits
     int64_t n_split = a.n_packed + a.n_tail;
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
         p.tiles = (int)cdiv(a.Sq, p.pq);
-        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * VQ_TAIL_EQUIV, 128) * 128 : 0;
+        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * TAIL_EQUIV, 128) * 128 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
     // the MFMA kernel wants every block to start on a boundary of the largest token group (128)
@@ -64,11 +62,12 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     if (p.path == 0) ns = n_split > 0 ? cdiv(n_split, len) : 1;
     p.nsplit = (int)ns;
     p.split_len = len;
-    // MFMA decode path: the tail is run by up to eight waves of split 0, two units of 32 tokens each
-    // where there are that many, every wave into a partial of its own
+    // MFMA decode path: the tail is run by up to eight waves of split 0, every wave into a partial of
+    // its own.  A launch with many blocks is bound by throughput: one wave takes eight units of 32
+    // tokens (the other waves stream meanwhile); a launch with few is bound by latency: two units a wave.
     p.nparts = p.nsplit;
     if (p.path == 1 && a.n_tail > 0) {
-        int64_t tw = cdiv(cdiv(a.n_tail, 32), 2);
+        int64_t tw = cdiv(cdiv(a.n_tail, 32), units >= 64 ? 8 : 2);
         p.nparts += (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw);
     }
     return p;
