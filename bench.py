@@ -10,8 +10,10 @@ flush a 64-token block into the packed store when one is due, attend.
 
 Prints ONE JSON line.  ``value`` is algorithmic HBM bytes per step divided by
 the step time, inputs resident in HBM.  ``roofline`` prices the attention
-kernel alone (HIP events on the launch stream); ``cpu_baseline`` times the
-scalar C oracle on a bounded sample of the same workload on the host.
+kernel alone (HIP events on the launch stream); ``cpu_baseline`` times the reference's
+CPU path (its operations restated on torch CPU, all host threads torch is given) on a
+bounded sample of the same workload; ``extras.cpu_baselines`` holds the same for the
+other workloads and the one-thread scalar C port.
 """
 
 from __future__ import annotations
@@ -67,6 +69,32 @@ def _event_ms(fn, iters, torch):
     e.record()
     torch.cuda.synchronize()
     return s.elapsed_time(e) / iters
+
+
+def _graph_ms(fn, torch, calls=20, replays=5):
+    """Milliseconds per call with the calls replayed from a HIP graph: what the GPU needs when the
+    host's per-call cost (argument marshalling in Python, ~20 us) is out of the way."""
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+        side.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for _ in range(calls):
+                fn()
+    graph.replay()
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(replays):
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        graph.replay()
+        e.record()
+        torch.cuda.synchronize()
+        ms = s.elapsed_time(e) / calls
+        best = ms if best is None else min(best, ms)
+    return best
 
 
 def _algorithmic_bytes_per_layer(B, Hkv, ctx, D, bits, g):
@@ -168,12 +196,12 @@ def main() -> int:
     kern_ms = _event_ms(attend_only, max(3, a.steps // 2), torch) / NL
     achieved = layer_bytes / (kern_ms * 1e-3) / 1e9
     # HBM bytes one attention launch moved under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated
-    # against a 1 GiB device copy); measured at the default workload only
-    # (profiles/attend_mfma_packed_4bit_cfg3_hbm_traffic.md)
+    # against a 1 GiB device copy): read from profiles/hbm_traffic.json, which records the hash of the
+    # attention sources it was measured on -- a kernel changed since then reports null
     default_workload = (B, ctx, bits, g) == (16, 32768, 4, 64)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": 618432102 if default_workload else None,
-                "kernel": "attend_mfma_packed_kernel<4, f16, 2>: one launch per layer does the fp16 tail, "
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _recorded_traffic("decode_cfg3_4bit_g64_B16") if default_workload else None,
+                "kernel": "attend_mfma_packed_kernel<4, f16, 2, 4>: one launch per layer does the fp16 tail, "
                           "the packed prefix and the split merge (vq_kivi_attend with sync counters)",
                 "bytes_per_launch": layer_bytes, "ms_per_launch": round(kern_ms, 5)}
 
@@ -210,7 +238,9 @@ def main() -> int:
             "frac_hbm": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes,
             "note": "LayerStackedKIVICache over the resident caches: append + attend of all layers per step"}
     if not a.no_cpu:
-        out["cpu_baseline"] = _cpu_baseline(np, torch, caches[0], q[0], ctx, Hkv, D, bits, g, scale)
+        head, others = _cpu_baselines(np, torch, caches[0], q[0], ctx, Hkv, D, bits, g, scale)
+        out["cpu_baseline"] = head
+        out.setdefault("extras", {})["cpu_baselines"] = others
     print(json.dumps(out))
     return 0
 
@@ -332,8 +362,11 @@ def _extras(torch, K, dev):
         for _ in range(3):
             fn()
         ms = _side_ms(fn, 30, torch)
+        ms_g = _graph_ms(fn, torch)
         ex[f"decode_2bit_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1),
-                                        "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}
+                                        "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes,
+                                        "ms_graph": round(ms_g, 5), "frac_hbm_graph": round(nbytes / ms_g / 1e6 / HBM_PEAK_GBS, 4),
+                                        "note": "ms: one Python call per launch; ms_graph: the same launches replayed from a HIP graph"}
         del c
     # config 0: quantise + pack of one layer's K and V [1,8,2048,128], 4-bit, group 32; and a large flush
     for name, shape in (("cfg0_[1,8,2048,128]", (1, 8, 2048, 128)), ("large_[16,8,8192,128]", (16, 8, 8192, 128))):
@@ -447,32 +480,116 @@ def _extras(torch, K, dev):
     return ex
 
 
-def _cpu_baseline(np, torch, cache, q_layer, ctx, Hkv, D, bits, g, scale):
-    """Scalar C oracle (one thread) on one sequence of one layer: dequantise each
-    slot and attend, the same arithmetic the GPU step does for that slice."""
-    from oracle import cref, kivi as ok
-    n = ctx
-    kp = cache._kp[:1, :, :n].cpu().numpy().view(np.uint32)
-    codes_k = ok.unpack_indices(kp, bits, D)
-    ks = cache._ks[:1, :, : n // g].float().cpu().numpy()
-    kz = cache._kz[:1, :, : n // g].float().cpu().numpy()
+def _unpacked_sequences(np, torch, cache, n_seq, ctx, D, bits, g):
+    """Codes (uint8) and float32 scale / zero of the first ``n_seq`` sequences of a resident packed
+    cache, in the reference's layout: keys ``[B,H,S,D]`` + ``[B,H,S/g,D]``, values ``[B,H,S,D]`` +
+    ``[B,H,S,D/g]``."""
+    from oracle import kivi as ok
     per = 32 // bits
-    vp = cache._vp[:1, :, : n // per].cpu().numpy().view(np.uint32)       # [1,H,n/per,D]
-    codes_v = ok.unpack_indices(np.ascontiguousarray(vp.swapaxes(-1, -2)), bits, n).swapaxes(-1, -2)
-    vs = np.ascontiguousarray(cache._vs[:1, :, :, :n].float().cpu().numpy().swapaxes(-1, -2))
-    vz = np.ascontiguousarray(cache._vz[:1, :, :, :n].float().cpu().numpy().swapaxes(-1, -2))
-    qn = q_layer[:1].float().cpu().numpy()
-    cref.lib()
+    kp = cache._kp[:n_seq, :, :ctx].cpu().numpy().view(np.uint32)
+    codes_k = ok.unpack_indices(kp, bits, D)
+    ks = cache._ks[:n_seq, :, : ctx // g].float().cpu().numpy()
+    kz = cache._kz[:n_seq, :, : ctx // g].float().cpu().numpy()
+    vp = cache._vp[:n_seq, :, : ctx // per].cpu().numpy().view(np.uint32)       # [n,H,ctx/per,D]
+    codes_v = np.ascontiguousarray(ok.unpack_indices(np.ascontiguousarray(vp.swapaxes(-1, -2)), bits, ctx).swapaxes(-1, -2))
+    vs = np.ascontiguousarray(cache._vs[:n_seq, :, :, :ctx].float().cpu().numpy().swapaxes(-1, -2))
+    vz = np.ascontiguousarray(cache._vz[:n_seq, :, :, :ctx].float().cpu().numpy().swapaxes(-1, -2))
+    return codes_k, ks, kz, codes_v, vs, vz
+
+
+def _timed(fn, min_seconds, max_reps=50):
+    fn()                                  # warm-up (allocator, thread pool)
     t0 = time.perf_counter()
     reps = 0
-    while time.perf_counter() - t0 < 10.0:
-        cref.attend(qn, codes_k, ks, kz, np.ascontiguousarray(codes_v), vs, vz, g, scale)
+    while reps < max_reps and (reps == 0 or time.perf_counter() - t0 < min_seconds):
+        fn()
         reps += 1
-    dt = (time.perf_counter() - t0) / reps
+    return (time.perf_counter() - t0) / reps, reps
+
+
+def _cpu_baselines(np, torch, cache, q_layer, ctx, Hkv, D, bits, g, scale):
+    """The reference's CPU path (oracle/cpu_path.py: its pure-MLX operations restated one for one on
+    torch CPU tensors, same materialised intermediates) timed on this box's host cores on bounded
+    samples of the four workloads, and the scalar C oracle (one thread) on the decode sample.
+    Returns (headline cpu_baseline = decode, dict of the others)."""
+    from oracle import cpu_path as cp, cref
+    cores = torch.get_num_threads()
+    model = cp.cpu_model()
+    t = lambda a: torch.from_numpy(np.ascontiguousarray(a))
+
+    # decode (the headline workload): one sequence of one layer, dequantise-then-SDPA
+    codes_k, ks, kz, codes_v, vs, vz = _unpacked_sequences(np, torch, cache, 1, ctx, D, bits, g)
+    qn = q_layer[:1].cpu()
+    args = [t(a) for a in (codes_k, ks, kz, codes_v, vs, vz)]
+    dt, reps = _timed(lambda: cp.decode_dequant_then_sdpa(qn, *args, g, scale), 6.0)
     nbytes = _algorithmic_bytes_per_layer(1, Hkv, ctx, D, bits, g)
-    return {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
-            "sample": f"one sequence of one layer ({Hkv} kv heads x {ctx} tokens, 32 query heads), scalar C oracle "
-                      f"oracle/c/kv_oracle.c:kvo_attend, {reps} repetitions, {dt:.3f} s each"}
+    head = {"value": round(nbytes / dt / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port", "cpu_model": model,
+            "sample": f"one sequence of one layer ({Hkv} kv heads x {ctx} tokens, 32 query heads): the reference's "
+                      f"dequantise-then-SDPA arm (benchmark_real_model_scalar_attend.py:194-217) restated on torch CPU "
+                      f"(oracle/cpu_path.py), {cores} threads, {reps} repetitions of {dt:.3f} s; GB/s of the same "
+                      f"algorithmic packed bytes the GPU figure counts"}
+    others = {}
+    # the scalar C port of the fused decode arithmetic, one thread, same sample
+    cref.lib()
+    qf = qn.float().numpy()
+    cargs = (codes_k, ks, kz, np.ascontiguousarray(codes_v), vs, vz)
+    dtc, repsc = _timed(lambda: cref.attend(qf, *cargs, g, scale), 3.0, max_reps=5)
+    others["decode_scalar_c_port"] = {"GBps": round(nbytes / dtc / 1e9, 4), "cores": 1, "seconds": round(dtc, 3),
+                                      "note": "oracle/c/kv_oracle.c:kvo_attend, one thread, same sample"}
+    del codes_k, codes_v, args, cargs
+
+    # config 0: 4-bit group-32 round trip of K (per channel) and V (per token), [1,8,2048,128] fp16
+    rng = np.random.default_rng(0)
+    f = np.exp(rng.standard_normal(128)).astype(np.float32)
+    k0 = t((rng.standard_normal((1, 8, 2048, 128)).astype(np.float32) * f).astype(np.float16))
+    v0 = t(rng.standard_normal((1, 8, 2048, 128)).astype(np.float16))
+    dt0, reps0 = _timed(lambda: (cp.kivi_round_trip(k0, -2, 32, 15), cp.kivi_round_trip(v0, -1, 32, 15)), 3.0)
+    others["cfg0_round_trip"] = {"GBps": round(16777216 / dt0 / 1e9, 3), "ms": round(dt0 * 1e3, 3), "cores": cores, "bytes": 16777216,
+                                 "note": "KIVIKVCache._quant_dequant_along (kivi_cache.py:181-201), K and V of config 0, full size"}
+    # config 2: VQ assignment at full size, chunked difference tensor
+    x2 = t((rng.standard_normal((4, 4096, 256)).astype(np.float32) * np.exp(rng.standard_normal(256)).astype(np.float32)).astype(np.float16))
+    cb2 = t(rng.standard_normal((256, 8)).astype(np.float16))
+    dt2, reps2 = _timed(lambda: cp.quantize_vq(x2, cb2, 8), 4.0, max_reps=10)
+    others["cfg2_vq_assign"] = {"ms": round(dt2 * 1e3, 2), "TFLOPs_gemm_form": round(2 * 524288 * 256 * 8 / dt2 / 1e12, 4), "cores": cores,
+                                "note": "quantize_vq (allocators/vecinfer.py:281-318), 524288 sub-vectors x 256 centroids, full size"}
+    # config 4: chunked quantise-on-write prefill at full size (float32 arithmetic over the fp16 history)
+    kc = [t((rng.standard_normal((1, 8, 512, 128)).astype(np.float32) * f).astype(np.float16)) for _ in range(8)]
+    vc = [t(rng.standard_normal((1, 8, 512, 128)).astype(np.float16)) for _ in range(8)]
+    qc = [t(rng.standard_normal((1, 32, 512, 128)).astype(np.float16)) for _ in range(8)]
+    pk = t((rng.standard_normal((1, 8, 4096, 128)).astype(np.float32) * f).astype(np.float16))
+    pv = t(rng.standard_normal((1, 8, 4096, 128)).astype(np.float16))
+    dt4, reps4 = _timed(lambda: cp.chunked_prefill(qc, kc, vc, pk, pv, 4, 32, 128, 1 / math.sqrt(128)), 4.0, max_reps=5)
+    others["cfg4_prefill"] = {"ms": round(dt4 * 1e3, 1), "TFLOPs": round(412350414848 / dt4 / 1e12, 4), "cores": cores,
+                              "note": "KIVIKVCache.update_and_fetch per chunk (kivi_cache.py:206-262) + dense causal SDPA over the "
+                                      "whole history, 8 chunks of 512 queries, full size"}
+    others["cpu_model"] = model
+    return head, others
+
+
+# ---- HBM traffic of the headline kernel, measured with rocprofv3 --pmc and kept under profiles/
+def _kernel_source_sha():
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "veloxquant_mlx_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.startswith("attend") and name.endswith((".hip", ".hpp")):
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(name.encode())
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def _recorded_traffic(key):
+    """Bytes per launch from profiles/hbm_traffic.json, or None when the attention sources have
+    changed since the counters were taken (the figure would be stale)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            rec = json.load(f).get(key)
+    except (OSError, ValueError):
+        return None
+    if not rec or rec.get("attend_sources_sha256") != _kernel_source_sha():
+        return None
+    return rec.get("traffic_bytes")
 
 
 if __name__ == "__main__":
