@@ -293,6 +293,120 @@ def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
         assert torch.equal(c.fused_sdpa(q, scale, causal=True), o1.to(torch.bfloat16))
 
 
+def test_config4_every_chunk_against_the_oracle_on_sampled_rows():
+    """Benchmark configuration 4 at full size, every one of the 8 chunks: for one kv head the host
+    quantises the same bf16 keys and values with the numpy oracle (one shot over the packed prefix:
+    whole groups are independent of how the cache was flushed), and sampled query rows -- first,
+    last and two inner positions of the chunk, all four query heads of the group -- are attended
+    over (reconstruction | residual rows) in float64.  The 256-row MFMA blocks attend over the
+    reconstruction rounded to fp16, which is the oracle's ``recon_dtype``."""
+    require_gpu()
+    B, Hq, Hkv, D, P, C, g = 1, 32, 8, 128, 4096, 512, 32
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(41)
+    f = torch.exp(torch.randn(D, generator=gen, device=dev))
+    c = _make(bit_width_inlier=4, kivi_group_size=g, residual_length=128, fused_sdpa=True,
+              fused_sdpa_memory_bound=True)
+    mk = lambda n: ((torch.randn((B, Hkv, n, D), generator=gen, device=dev) * f).to(torch.bfloat16),
+                    torch.randn((B, Hkv, n, D), generator=gen, device=dev).to(torch.bfloat16))
+    hk = 5                                        # the kv head the host follows
+    k0, v0 = mk(P)
+    c.update_and_fetch(k0, v0)
+    k_all, v_all = [host(k0[:, hk:hk + 1])], [host(v0[:, hk:hk + 1])]
+    scale = 1 / math.sqrt(D)
+    rng = np.random.default_rng(8)
+    worst = 0.0
+    for ci in range(8):
+        kc_, vc_ = mk(C)
+        c.update_and_fetch(kc_, vc_)
+        k_all.append(host(kc_[:, hk:hk + 1]))
+        v_all.append(host(vc_[:, hk:hk + 1]))
+        q = torch.randn((B, Hq, C, D), generator=gen, device=dev).to(torch.bfloat16)
+        out = host(c.fused_sdpa(q, scale, causal=True))
+        nq = c._n_quantized
+        kh, vh = np.concatenate(k_all, axis=2), np.concatenate(v_all, axis=2)     # float32 views of the bf16 rows
+        n_total = kh.shape[2]
+        assert n_total == c.offset and nq == (n_total - 128) // g * g
+        kcodes, ksc, kzr = ok.group_quant_codes(kh[:, :, :nq], -2, g, 15)
+        vcodes, vsc, vzr = ok.group_quant_codes(vh[:, :, :nq], -1, g, 15)
+        meta = [a.astype(np.float16) for a in (ksc, kzr, vsc, vzr)]
+        heads = slice(hk * (Hq // Hkv), (hk + 1) * (Hq // Hkv))
+        for pos in sorted({0, C - 1, *rng.integers(1, C - 1, 2).tolist()}):
+            vis = n_total - C + pos + 1
+            npk = min(vis, nq)
+            ref = oa.kivi_attend(host(q[:, heads, pos:pos + 1]), kcodes[:, :, :npk], meta[0][:, :, : -(-npk // g)], meta[1][:, :, : -(-npk // g)],
+                                 vcodes[:, :, :npk], meta[2][:, :, :npk], meta[3][:, :, :npk], g,
+                                 kh[:, :, nq:vis], vh[:, :, nq:vis], scale, recon_dtype=np.float16)
+            err = float(np.max(np.abs(out[:, heads, pos:pos + 1] - ref)))
+            worst = max(worst, err)
+            # the output is bf16 (8 significant bits): half an ulp of values up to ~1 on top of the 2e-3 bar
+            assert err < 2e-3 + 2.0 ** -9, (ci, pos, err)
+    print(f"8 chunks, sampled rows: max |out - oracle| = {worst:.2e}")
+
+
+@pytest.mark.parametrize("chunk,g", [(128, 32), (80, 32), (96, 64)])
+def test_chunked_prefill_with_no_residual_window(chunk, g):
+    """The other reading of quantise-on-write: ``residual_length=0``, every whole group is packed
+    as soon as it is complete, so a chunk's queries see (nearly) all tokens, their own included, in
+    quantised form and the causal edge runs through the packed prefix."""
+    require_gpu()
+    B, Hq, Hkv, S, D = 1, 8, 2, 480, 128
+    k, v = outlier_kv((B, Hkv, S, D), seed=14)
+    q = np.random.default_rng(6).standard_normal((B, Hq, S, D)).astype(np.float16)
+    c = _make(bit_width_inlier=4, kivi_group_size=g, residual_length=0, fused_sdpa=True,
+              fused_sdpa_memory_bound=True, kivi_meta_dtype="float32")
+    outs, refs = [], []
+    kc_, ks_, kz_ = ok.group_quant_codes(k, -2, g, 15)     # whole groups do not depend on when they were flushed
+    vc_, vs_, vz_ = ok.group_quant_codes(v, -1, g, 15)
+    for s0 in range(0, S, chunk):
+        s1 = min(S, s0 + chunk)
+        c.update_and_fetch(to_dev(k[:, :, s0:s1]), to_dev(v[:, :, s0:s1]))
+        nq = s1 // g * g
+        assert c._n_quantized == nq and c.offset - nq < g
+        outs.append(host(c.fused_sdpa(to_dev(q[:, :, s0:s1]), 1 / math.sqrt(D), causal=True)))
+        refs.append(oa.kivi_attend(q[:, :, s0:s1], kc_[:, :, :nq], ks_[:, :, : nq // g], kz_[:, :, : nq // g], vc_[:, :, :nq],
+                                   vs_[:, :, :nq], vz_[:, :, :nq], g, k[:, :, nq:s1], v[:, :, nq:s1], 1 / math.sqrt(D), causal=True))
+    got = np.concatenate(outs, axis=2).astype(np.float32)
+    # float32 scale / zero: the kernels attend over code * scale + zero itself
+    assert np.max(np.abs(got - np.concatenate(refs, axis=2))) < 2e-3
+    # the cache model holds that reconstruction rounded to fp16 (kivi_cache.py:198-201); with every
+    # token quantised the rounding shows, inside the 1e-2 bar of the reference's own fused-attention tests
+    assert np.max(np.abs(got - oa.chunked_prefill(q, k, v, chunk, 4, g, 0, 1 / math.sqrt(D)))) < 1e-2
+
+
+def test_bf16_history_holds_the_reconstruction_rounded_to_bf16():
+    """Keys and values that arrive in bf16: the standard cache returns, below the frontier, the
+    float32 reconstruction cast to bf16 -- ``recon.astype(x.dtype)``, kivi_cache.py:198-201 -- bit
+    for bit; the packed cache never forms those rows: its attention works on code * scale + zero
+    with scale / zero in the configured storage type, and differs from attention over the bf16
+    history by less than bf16 rounding of keys and values allows."""
+    require_gpu()
+    B, Hq, Hkv, S, D, g = 1, 8, 2, 320, 128, 32
+    k, v = outlier_kv((B, Hkv, S, D), seed=15)
+    bf = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.bfloat16)
+    kb, vb = bf(k), bf(v)
+    cast = lambda a: torch.from_numpy(a).to(torch.bfloat16).float().numpy()
+    std = _make(bit_width_inlier=4, kivi_group_size=g, residual_length=64)
+    ko, vo = std.update_and_fetch(kb.to("cuda:0"), vb.to("cuda:0"))
+    assert ko.dtype == torch.bfloat16
+    nq = std._n_quantized
+    assert nq == 256
+    k32, v32 = kb.float().numpy(), vb.float().numpy()
+    assert np.array_equal(host(ko)[:, :, :nq], ok.quant_dequant_along(k32[:, :, :nq], -2, g, 15, cast=cast))
+    assert np.array_equal(host(vo)[:, :, :nq], ok.quant_dequant_along(v32[:, :, :nq], -1, g, 15, cast=cast))
+    assert np.array_equal(host(ko)[:, :, nq:], k32[:, :, nq:])
+    packed = _make(bit_width_inlier=4, kivi_group_size=g, residual_length=64, fused_sdpa=True, fused_sdpa_memory_bound=True,
+                   kivi_meta_dtype="float32")
+    packed.update_and_fetch(kb.to("cuda:0"), vb.to("cuda:0"))
+    q = np.random.default_rng(7).standard_normal((B, Hq, 1, D)).astype(np.float16)
+    got = host(packed.fused_sdpa(to_dev(q), 1 / math.sqrt(D), causal=False)).astype(np.float32)
+    exact = oa.sdpa(q, np.concatenate([ok.quant_dequant_along(k32[:, :, :nq], -2, g, 15), k32[:, :, nq:]], axis=2),
+                    np.concatenate([ok.quant_dequant_along(v32[:, :, :nq], -1, g, 15), v32[:, :, nq:]], axis=2), 1 / math.sqrt(D))
+    over_bf16 = oa.sdpa(q, host(ko), host(vo), 1 / math.sqrt(D))
+    assert np.max(np.abs(got - exact)) < 2e-3
+    assert np.max(np.abs(got - over_bf16)) < 1e-2
+
+
 def test_config3_decode_at_full_size_against_the_oracle_and_the_vector_kernel():
     """Benchmark configuration 3, one layer: batch 16, 32 query / 8 kv heads, D=128, 32768 tokens of
     context in a 4-bit group-64 packed cache plus the fp16 residual, one query token.  The last

@@ -509,6 +509,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int kt = tid >> 4, kc = tid & 15;       // key tile: token, 8-channel chunk
     const int vc = tid & 127, vq = tid >> 7;      // value tile: channel, 8-token quarter
     const int vg = vc >> gshift;                  // channel group of the thread's value channel
+    const int tp = lane & 15, cq = 4 * wave + (lane >> 4);   // tail values: token pair, channel quad
     const bool tail_bf16 = a.tail_dtype == VQ_BF16;
     const int64_t tbase = bh * a.tail_cap * MF_D;
     const f16x8 off8 = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair);
@@ -516,12 +517,18 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     f16x8 ksr, kzr;   // key scale / zero of the thread's 8 channels in the token group last fetched
     int meta_group = -1;
     auto fetch = [&](int w, Stage &st) {
-        if (w >= n_punits) {   // tail unit: the thread's key and value row chunks travel in the value-meta slots
-            int64_t tok = (int64_t)(w - n_punits) * 32 + kt;
+        if (w >= n_punits) {   // tail unit: the thread's key and value pieces travel in the value-meta slots
+            const int64_t t0 = (int64_t)(w - n_punits) * 32;
+            int64_t tok = t0 + kt;
             if (tok >= a.n_tail) tok = 0;   // masked in the softmax
-            const int64_t e0 = tbase + tok * MF_D + 8 * kc;
-            st.vs = *reinterpret_cast<const uint4 *>((const u16 *)a.k_tail + e0);
-            st.vz = *reinterpret_cast<const uint4 *>((const u16 *)a.v_tail + e0);
+            st.vs = *reinterpret_cast<const uint4 *>((const u16 *)a.k_tail + tbase + tok * MF_D + 8 * kc);
+            // values: four channels of a token pair, so that the transposed tile is written in whole words
+            int64_t ta = t0 + 2 * tp, tb = ta + 1;
+            if (ta >= a.n_tail) ta = 0;
+            if (tb >= a.n_tail) tb = 0;
+            const uint2 va = *reinterpret_cast<const uint2 *>((const u16 *)a.v_tail + tbase + ta * MF_D + 4 * cq);
+            const uint2 vb2 = *reinterpret_cast<const uint2 *>((const u16 *)a.v_tail + tbase + tb * MF_D + 4 * cq);
+            st.vz = make_uint4(va.x, va.y, vb2.x, vb2.y);
             return;
         }
         const int64_t base = (int64_t)w * 32;
@@ -561,11 +568,13 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             *reinterpret_cast<f16x8 *>(&s_v[buf][vc * PF_VSTRIDE + 8 * vq]) =
                 __builtin_elementwise_fma(codes8(st.vw, vq & 1), as_h8(st.vs), as_h8(st.vz));
         } else {
-            // tail unit: plain key row chunk; value row chunk transposed
+            // tail unit: plain key row chunk; values transposed, one word (a token pair of one channel)
+            // at a time: the lanes of a wave cover 16 token pairs x 4 channel quads = 64 different banks
             *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = tail8_from_raw(st.vs, tail_bf16);
-            const f16x8 v0 = tail8_from_raw(st.vz, tail_bf16);
+            const f16x8 v0 = tail8_from_raw(st.vz, tail_bf16);   // channels 0..3 of the first token, then of the second
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s_v[buf][(8 * kc + e) * PF_VSTRIDE + kt] = v0[e];
+            for (int e = 0; e < 4; ++e)
+                *reinterpret_cast<f16x2 *>(&s_v[buf][(4 * cq + e) * PF_VSTRIDE + 2 * tp]) = f16x2{v0[e], v0[4 + e]};
         }
     };
 
@@ -728,22 +737,28 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
 int mfma_prefill_block_rows(const vq_attend_args &a);
 
 bool mfma_prefill_supported(const vq_attend_args &a) {
-    if (a.D != MF_D || a.n_packed <= 0 || a.Sq < 16) return false;
+    if (a.D != MF_D || a.n_packed < 0 || a.Sq < 16) return false;
     if (a.Hq % a.Hkv != 0) return false;
     const int64_t R = a.Hq / a.Hkv;
     if (!(R == 1 || R == 2 || R == 4 || R == 8)) return false;
-    if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
-    if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
-    if (a.meta_dtype != VQ_F16) return false;   // float32 scale / zero stays on the 8-row tiles of the decode kernel
-    if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
-    if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
+    if (a.n_packed > 0) {
+        if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
+        if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
+        if (a.meta_dtype != VQ_F16) return false;   // float32 scale / zero stays on the 8-row tiles of the decode kernel
+        if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
+        if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
+    } else {
+        // plain keys and values only (the tail units of the same kernels): worth the matrix unit
+        // from a few hundred tokens on
+        if (a.n_tail < 64 || a.packed_lens != nullptr) return false;
+    }
     if (!(a.scale > 0.f)) return false;
     if (a.n_tail > 0 && (!(a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
     if (a.B * a.Hkv > 65535) return false;
     if (a.n_tail > 0 && a.tail_cap * MF_D % 8 != 0) return false;
     const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
                          (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
-    if (al & 15u) return false;
+    if (a.n_packed > 0 && (al & 15u)) return false;
     if (mfma_prefill_block_rows(a) == 256 && a.q_dtype != VQ_F32 && ((uintptr_t)a.q & 15u)) return false;
     return true;
 }
@@ -758,7 +773,7 @@ void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     const int R = (int)(a.Hq / a.Hkv);
     const int rows = mfma_prefill_block_rows(a);
     const int qp = rows / R, tiles = (int)cdiv(a.Sq, qp);
-    const int gv = (int)(MF_D / a.group);
+    const int gv = a.n_packed > 0 ? (int)(MF_D / a.group) : 4;   // without packed units any instantiation serves
     const dim3 grid((unsigned)tiles, (unsigned)(a.B * a.Hkv), (unsigned)p.nsplit), block(256);
 #define VQ_LAUNCH(BITS, GV)                                                                                          \
     do {                                                                                                             \
@@ -767,7 +782,7 @@ void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
         else                                                                                                         \
             hipLaunchKernelGGL((attend_prefill_kernel<BITS, GV>), grid, block, 0, st, a, qp, p.nparts, ws);           \
     } while (0)
-    if (a.pack_bits == 4) { if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4); }
+    if (a.pack_bits == 4 || a.n_packed == 0) { if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4); }
     else { if (gv == 1) VQ_LAUNCH(2, 1); else if (gv == 2) VQ_LAUNCH(2, 2); else VQ_LAUNCH(2, 4); }
 #undef VQ_LAUNCH
 }
