@@ -47,7 +47,7 @@ def _parse():
     p.add_argument("--only-kernel", action="store_true", help="time the attention kernel loop only (profiling)")
     p.add_argument("--only", default=None, metavar="NAME",
                    help="run one side workload in a loop and print its timing (for rocprofv3): "
-                        "decode_2bit_B16, decode_2bit_B1, vq_assign, prefill, quant_pack, quant_dequant")
+                        "decode_2bit_B16, decode_2bit_B1, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant")
     p.add_argument("--copy-calib", action="store_true",
                    help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
@@ -290,6 +290,17 @@ def _prefill_case(torch, dev):
     return prefill_pass
 
 
+def _flash_prefill_case(torch, K, dev, S, H=32, D=128):
+    """Causal self-attention over plain fp16 K/V, one sequence, H heads (no GQA), S_q = S_kv = S: the
+    shape the reference quotes its flash-prefill kernel on.  Returns (call, flops)."""
+    q = torch.randn((1, H, S, D), device=dev).to(torch.float16)
+    k = torch.randn((1, H, S, D), device=dev).to(torch.float16)
+    v = torch.randn((1, H, S, D), device=dev).to(torch.float16)
+    out = torch.empty_like(q)
+    fn = lambda: K.kivi_packed_attend(q, k_tail=k, v_tail=v, n_tail=S, scale=D ** -0.5, causal=True, out=out)
+    return fn, 4 * D * H * (S * (S + 1) // 2)
+
+
 def _vq_assign_case(torch, K, dev):
     """Config 2: keys [4, 4096, 256] fp16 with channel outliers, 256 centroids of 8 dims, uint8 indices."""
     x = (torch.randn((4, 4096, 256), device=dev) * torch.exp(torch.randn(256, device=dev))).to(torch.float16)
@@ -305,6 +316,13 @@ def _only(a, torch, K, dev):
     elif name == "vq_assign":
         x, cb, fn = _vq_assign_case(torch, K, dev)
         nbytes = None
+    elif name.startswith("flash_prefill"):
+        fn, flops = _flash_prefill_case(torch, K, dev, int(name.rsplit("_", 1)[1]) if name[-1].isdigit() else 8192)
+        for _ in range(a.warmup):
+            fn()
+        ms = _event_ms(fn, max(1, a.steps), torch)
+        print(json.dumps({"only": name, "ms": ms, "TFLOPs": flops / ms / 1e9}))
+        return 0
     elif name == "prefill":
         run = _prefill_case(torch, dev)
         run()
@@ -395,6 +413,15 @@ def _extras(torch, K, dev):
                           "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
                           "note": "8 chunks of 512 queries: quantise-on-write append + attention per chunk; "
                                   "the packed store is sized once by fused_sdpa_max_ctx=8192"}
+    # causal attention over plain fp16 K/V (the reference's flash-prefill shape: 32 heads, D 128, S_q = S_kv)
+    for S in (2048, 8192):
+        fn, flops = _flash_prefill_case(torch, K, dev, S)
+        for _ in range(3):
+            fn()
+        ms = _side_ms(fn, 10, torch)
+        ex[f"flash_prefill_S{S}_H32"] = {"ms": round(ms, 4), "TFLOPs": round(flops / ms / 1e9, 1),
+                                         "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
+                                         "note": "flops count the causal half only"}
     # config 2: VQ assignment, keys [4,4096,256], 256 centroids x 8 dims
     x, cb, fn = _vq_assign_case(torch, K, dev)
     for _ in range(3):

@@ -468,3 +468,25 @@ def test_ragged_batch_per_sequence_lengths(Sq, causal, v_layout, num_splits):
     with pytest.raises(ValueError, match="go together"):
         K.kivi_packed_attend(to_dev(q), n_packed=NP, bits=b, group_size=g, v_layout=v_layout, k_packed=kp, k_scale=ks, k_zero=kz,
                              v_packed=vp, v_scale=vs, v_zero=vz, scale=0.09, packed_lens=torch.tensor(p_lens, device=dev))
+
+
+@pytest.mark.parametrize("bits,g,meta,Hq,Hkv", [(2, 32, "float16", 32, 8), (4, 64, "float16", 32, 8), (4, 32, "float32", 8, 1),
+                                                 (2, 64, "float32", 16, 4)])
+def test_counted_copy_waits_equal_waiting_for_every_copy(bits, g, meta, Hq, Hkv):
+    """The decode kernel fills its LDS ring with asynchronous copies and waits for exactly the copies
+    a unit needs (a hand-counted outstanding-load count).  ``fixed_order=3`` runs the same kernel
+    waiting for every copy in flight instead; with the chunks dealt in the same fixed order the two
+    must agree bit for bit -- a miscounted wait would read a slot before its copy has landed."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+    B, D, ctx = 2, 128, 4096 + 128 + 19
+    c = KVCacheFactory.create(KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=bits, kivi_group_size=g,
+                                            residual_length=128, fused_sdpa=True, fused_sdpa_memory_bound=True,
+                                            kivi_meta_dtype=meta))
+    k, v = outlier_kv((B, Hkv, ctx, D), seed=bits + g)
+    c.update_and_fetch(to_dev(k), to_dev(v))
+    for Sq in (1, 3):
+        q = to_dev(np.random.default_rng(Sq).standard_normal((B, Hq, Sq, D)).astype(np.float16))
+        counted = c.fused_sdpa(q, D ** -0.5, fixed_order=1)
+        wait_all = c.fused_sdpa(q, D ** -0.5, fixed_order=3)
+        assert torch.equal(counted, wait_all)
