@@ -31,6 +31,14 @@ namespace vq {
 
 #define VQ_MFMA(A, B, C) __builtin_amdgcn_mfma_f32_16x16x32_f16((A), (B), (C), 0, 0, 0)
 
+// Bare three-way maximum: the scores are never NaN, so the canonicalising moves the compiler
+// wraps around fmaxf would only cost issue slots in the softmax.
+__device__ __forceinline__ float vmax3(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
 constexpr int PF_KSTRIDE = MF_D + 8;   // fp16 per token row of the key-code tile (272 B: conflict-free b128 reads)
 constexpr int PF_VSTRIDE = 32 + 8;     // fp16 per channel row of the value tile (80 B)
 
@@ -108,7 +116,8 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     const int64_t cap = a.cap_tokens;
     const float c = a.scale * LOG2E;
     const u32 magic = vreg_const(Magic<BITS>::bits);
-    const int pos0 = (int)blockIdx.x * qp;
+    // under a causal mask the last tiles see the most tokens: they are started first
+    const int pos0 = (int)(a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * qp;
     const int64_t n_total = a.n_packed + a.n_tail;
 
     // ---- this lane's query row (as a score column): row j = 16 wave + n of the block
@@ -458,7 +467,8 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int64_t cap = a.cap_tokens;
     const float c = a.scale * LOG2E;
     const u32 magic = vreg_const(Magic<BITS>::bits);
-    const int pos0 = (int)blockIdx.x * qp;
+    // under a causal mask the last tiles see the most tokens: they are started first
+    const int pos0 = (int)(a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * qp;
     const int64_t n_total = a.n_packed + a.n_tail;
     auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
 
@@ -509,6 +519,10 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int kt = tid >> 4, kc = tid & 15;       // key tile: token, 8-channel chunk
     const int vc = tid & 127, vq = tid >> 7;      // value tile: channel, 8-token quarter
     const int vg = vc >> gshift;                  // channel group of the thread's value channel
+    // byte offsets of the thread's key word, value word and value scale / zero piece inside a unit
+    const unsigned k_off = (unsigned)((kt * KW + (BITS == 4 ? kc : kc >> 1)) * 4);
+    const unsigned v_off = (unsigned)(((BITS == 4 ? vq : vq >> 1) * MF_D + vc) * 4);
+    const unsigned m_off = (unsigned)(((int64_t)vg * cap + 8 * vq) * 2);
     const int tp = lane & 15, cq = 4 * wave + (lane >> 4);   // tail values: token pair, channel quad
     const bool tail_bf16 = a.tail_dtype == VQ_BF16;
     const int64_t tbase = bh * a.tail_cap * MF_D;
@@ -531,21 +545,18 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             st.vz = make_uint4(va.x, va.y, vb2.x, vb2.y);
             return;
         }
+        // a block-uniform base that moves with the unit plus a 32-bit offset of the thread's own: the
+        // per-unit address arithmetic stays on the scalar unit
         const int64_t base = (int64_t)w * 32;
-        if (BITS == 4) {
-            st.kw = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + kc) * 4);
-            st.vw = *reinterpret_cast<const u32 *>(vb + ((base / 8 + vq) * MF_D + vc) * 4);
-        } else {
-            st.kw = *reinterpret_cast<const u32 *>(kb + ((base + kt) * KW + (kc >> 1)) * 4);
-            st.vw = *reinterpret_cast<const u32 *>(vb + ((base / 16 + (vq >> 1)) * MF_D + vc) * 4);
-        }
-        st.vs = *reinterpret_cast<const uint4 *>(vsb + (int64_t)vg * cap + base + 8 * vq);
-        st.vz = *reinterpret_cast<const uint4 *>(vzb + (int64_t)vg * cap + base + 8 * vq);
+        st.kw = *reinterpret_cast<const u32 *>(kb + base * (KW * 4) + k_off);
+        st.vw = *reinterpret_cast<const u32 *>(vb + (base / PER) * (MF_D * 4) + v_off);
+        st.vs = *reinterpret_cast<const uint4 *>((const char *)vsb + base * 2 + m_off);
+        st.vz = *reinterpret_cast<const uint4 *>((const char *)vzb + base * 2 + m_off);
         const int grp = (int)(base >> gshift);
         if (grp != meta_group) {   // block-uniform
             meta_group = grp;
-            ksr = *reinterpret_cast<const f16x8 *>(ksb + (int64_t)grp * MF_D + 8 * kc);
-            kzr = *reinterpret_cast<const f16x8 *>(kzb + (int64_t)grp * MF_D + 8 * kc);
+            ksr = *reinterpret_cast<const f16x8 *>((const char *)ksb + (int64_t)grp * (MF_D * 2) + 16u * (unsigned)kc);
+            kzr = *reinterpret_cast<const f16x8 *>((const char *)kzb + (int64_t)grp * (MF_D * 2) + 16u * (unsigned)kc);
         }
     };
     // the thread's eight codes of a word, in order, as exact fp16 numbers
@@ -655,8 +666,8 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
                     for (int r = 0; r < 4; ++r)
                         if (base + pf_tok(blk, r, T) >= lim) S[rb][T][r] = -INFINITY;
             }
-            const float mx = fmaxf(fmaxf(fmaxf(S[rb][0][0], S[rb][0][1]), fmaxf(S[rb][0][2], S[rb][0][3])),
-                                   fmaxf(fmaxf(S[rb][1][0], S[rb][1][1]), fmaxf(S[rb][1][2], S[rb][1][3])));
+            const float mx = vmax3(vmax3(S[rb][0][0], S[rb][0][1], S[rb][0][2]), vmax3(S[rb][0][3], S[rb][1][0], S[rb][1][1]),
+                                   vmax3(S[rb][1][2], S[rb][1][3], S[rb][1][3]));
             m_seen[rb] = mx * c;
             grow |= mx * c > m_run[rb] + RESCALE_SLACK;
         }
@@ -747,6 +758,7 @@ bool mfma_prefill_supported(const vq_attend_args &a) {
         if (a.meta_dtype != VQ_F16) return false;   // float32 scale / zero stays on the 8-row tiles of the decode kernel
         if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
         if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
+        if (a.cap_tokens > ((int64_t)1 << 28)) return false;   // 32-bit byte offsets inside one (sequence, kv head) slab
     } else {
         // plain keys and values only (the tail units of the same kernels): worth the matrix unit
         // from a few hundred tokens on
