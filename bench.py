@@ -329,9 +329,12 @@ def _only(a, torch, K, dev):
         ms = min(run() for _ in range(max(1, a.steps)))
         print(json.dumps({"only": name, "ms": ms}))
         return 0
-    elif name in ("quant_pack", "quant_dequant"):
+    elif name in ("quant_pack", "quant_pack_2calls", "quant_dequant"):
         k, v = _synthetic_layer(torch, 16, 8, 8192, 128, 11, dev)
         if name == "quant_pack":
+            fn = lambda: K.kivi_quant_pack_kv(k, v, 32, 4, v_layout="token")
+            nbytes = 2 * (k.numel() * 2 + k.numel() // 2 + (k.numel() // 32) * 4)
+        elif name == "quant_pack_2calls":
             def fn():
                 K.kivi_quant_pack(k, -2, 32, 4)
                 K.kivi_quant_pack(v, -1, 32, 4, v_layout="token")
@@ -389,9 +392,7 @@ def _extras(torch, K, dev):
     # config 0: quantise + pack of one layer's K and V [1,8,2048,128], 4-bit, group 32; and a large flush
     for name, shape in (("cfg0_[1,8,2048,128]", (1, 8, 2048, 128)), ("large_[16,8,8192,128]", (16, 8, 8192, 128))):
         k, v = _synthetic_layer(torch, shape[0], shape[1], shape[2], shape[3], 11, dev)
-        def qp():
-            K.kivi_quant_pack(k, -2, 32, 4)
-            K.kivi_quant_pack(v, -1, 32, 4, v_layout="token")
+        qp = lambda: K.kivi_quant_pack_kv(k, v, 32, 4, v_layout="token")   # keys and values of a flush: one launch
         def rt():
             K.kivi_group_quant_dequant(k, -2, 32, 15)
             K.kivi_group_quant_dequant(v, -1, 32, 15)
@@ -401,7 +402,14 @@ def _extras(torch, K, dev):
         b_qp = 2 * (n * 2 + n // 2 + (n // 32) * 4)
         b_rt = 2 * (n * 2 + n * 2)
         ms_qp, ms_rt = _side_ms(qp, 30, torch), _side_ms(rt, 30, torch)
-        ex[f"quant_pack_{name}"] = {"ms": round(ms_qp, 5), "GBps": round(b_qp / ms_qp / 1e6, 1), "bytes": b_qp}
+        ex[f"quant_pack_{name}"] = {"ms": round(ms_qp, 5), "GBps": round(b_qp / ms_qp / 1e6, 1), "bytes": b_qp,
+                                    "note": "keys and values of the layer in one launch (kivi_quant_pack_kv)"}
+        def qp2():
+            K.kivi_quant_pack(k, -2, 32, 4)
+            K.kivi_quant_pack(v, -1, 32, 4, v_layout="token")
+        qp2()
+        ms_qp2 = _side_ms(qp2, 30, torch)
+        ex[f"quant_pack_two_calls_{name}"] = {"ms": round(ms_qp2, 5), "GBps": round(b_qp / ms_qp2 / 1e6, 1), "bytes": b_qp}
         ex[f"quant_dequant_{name}"] = {"ms": round(ms_rt, 5), "GBps": round(b_rt / ms_rt / 1e6, 1), "bytes": b_rt}
     # config 4: causal prefill of 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
     # tokens plus their own tokens, quantise-on-write (group 32, residual 128)

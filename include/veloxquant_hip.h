@@ -87,6 +87,18 @@ int vq_kivi_quant_pack(const void *x, int dtype, int64_t BH, int64_t S, int64_t 
                        int pack_bits, int v_layout, void *packed, void *scale, void *zero,
                        int meta_dtype, int64_t cap_tokens, int64_t dst_tok0, void *stream);
 
+/* Keys and values of the same S tokens in one call: vq_kivi_quant_pack of k along the TOKEN
+ * axis and of v along the CHANNEL axis in v_layout, into destination buffers of the same
+ * cap_tokens at the same dst_tok0 -- the pair of calls every flush of a cache makes
+ * (KIVIKVCache.update_and_fetch, veloxquant_mlx/cache/kivi_cache.py:242-262, quantises keys and
+ * values of one block back to back).  One launch where D == 128, the inputs are fp16 or bf16
+ * and the shapes meet the alignment rules above; otherwise the two single calls. */
+int vq_kivi_quant_pack_kv(const void *k, const void *v, int dtype, int64_t BH, int64_t S, int64_t D,
+                          int64_t x_stride_bh, int group, int levels, float eps, int pack_bits,
+                          int v_layout, void *k_packed, void *k_scale, void *k_zero, void *v_packed,
+                          void *v_scale, void *v_zero, int meta_dtype, int64_t cap_tokens,
+                          int64_t dst_tok0, void *stream);
+
 /* Packed codes -> reconstruction, out[BH, S, D] = cast(code*scale + zero).
  * Replaces scalar_decode_once(codes, scale, zero, group_size, mode)
  * (veloxquant_mlx/metal/_scalar_attend.py:650-699).  Source buffers are laid

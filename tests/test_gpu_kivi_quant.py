@@ -276,3 +276,35 @@ def test_byte_pack_round_trip(b):
         K.turboquant_bit_pack(to_dev(idx[:4095]), b)
     with pytest.raises(ValueError, match="needs"):
         K.turboquant_bit_unpack(p[:10], 4096, b)
+
+
+@pytest.mark.parametrize("dtype,b,g,D,S,v_layout,meta", [
+    (torch.float16, 4, 32, 128, 2048, "token", torch.float16),     # config 0's layer
+    (torch.bfloat16, 2, 64, 128, 320, "token", torch.float32),
+    (torch.float16, 4, 128, 128, 384, "channel", torch.float16),   # the longest key group the tile kernel holds
+    (torch.float16, 2, 32, 64, 96, "token", torch.float16),        # head_dim 64: the two single calls
+    (torch.float16, 8, 32, 128, 100, "channel", torch.float16),    # ragged last key group
+])
+def test_keys_and_values_in_one_call_equal_the_single_calls(dtype, b, g, D, S, v_layout, meta):
+    """``kivi_quant_pack_kv`` is ``kivi_quant_pack`` of keys and values (each checked bit for bit
+    against the oracle above), in fresh buffers and at an offset of pre-allocated ones."""
+    require_gpu()
+    k, v = outlier_kv((2, 3, S, D), seed=S + b)
+    kt, vt = to_dev(k, dtype), to_dev(v, dtype)
+    (kp, ks, kz), (vp, vs, vz) = K.kivi_quant_pack_kv(kt, vt, g, b, meta_dtype=meta, v_layout=v_layout)
+    want_k = K.kivi_quant_pack(kt, -2, g, b, meta_dtype=meta)
+    want_v = K.kivi_quant_pack(vt, -1, g, b, meta_dtype=meta, v_layout=v_layout)
+    for got, want in zip((kp, ks, kz, vp, vs, vz), (*want_k, *want_v)):
+        assert got.shape == want.shape and torch.equal(got, want)
+    if S % g == 0 and S % (32 // b) == 0:
+        cap, off = 2 * S, S
+        bufs = K.kivi_quant_pack_kv(torch.zeros((2, 3, cap, D), dtype=dtype, device=kt.device),
+                                    torch.zeros((2, 3, cap, D), dtype=dtype, device=kt.device), g, b, meta_dtype=meta,
+                                    v_layout=v_layout)
+        K.kivi_quant_pack_kv(kt, vt, g, b, meta_dtype=meta, v_layout=v_layout, out=bufs, dst_tok0=off)
+        per = 32 // b
+        assert torch.equal(bufs[0][0][:, :, off:], kp) and torch.equal(bufs[0][1][:, :, off // g:], ks)
+        if v_layout == "token":
+            assert torch.equal(bufs[1][0][:, :, off // per:], vp) and torch.equal(bufs[1][1][..., off:], vs)
+        else:
+            assert torch.equal(bufs[1][0][:, :, off:], vp) and torch.equal(bufs[1][2][:, :, off:], vz)

@@ -192,17 +192,36 @@ template <> struct Raw8<f16> {
 #pragma unroll
         for (int i = 0; i < 8; ++i) { a.mn[i] = (f16)INFINITY; a.mx[i] = (f16)-INFINITY; }
     }
+    // bare packed min / max: the compiler's own forms quiet signalling NaNs first, two more
+    // instructions per pair, and inputs with NaNs are rejected before they get here
+    static __device__ __forceinline__ uint32_t pk_min(uint32_t a, uint32_t b) {
+        uint32_t d;
+        asm("v_pk_min_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+        return d;
+    }
+    static __device__ __forceinline__ uint32_t pk_max(uint32_t a, uint32_t b) {
+        uint32_t d;
+        asm("v_pk_max_f16 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b));
+        return d;
+    }
     __device__ __forceinline__ void fold(Acc &a) const {
-        a.mn = __builtin_elementwise_min(a.mn, h);
-        a.mx = __builtin_elementwise_max(a.mx, h);
+        typedef uint32_t w4 __attribute__((ext_vector_type(4)));
+        w4 mn = __builtin_bit_cast(w4, a.mn), mx = __builtin_bit_cast(w4, a.mx);
+        const w4 x = __builtin_bit_cast(w4, h);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { mn[i] = pk_min(mn[i], x[i]); mx[i] = pk_max(mx[i], x[i]); }
+        a.mn = __builtin_bit_cast(f16x8, mn);
+        a.mx = __builtin_bit_cast(f16x8, mx);
     }
     static __device__ __forceinline__ void result(const Acc &a, float (&mn)[8], float (&mx)[8]) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) { mn[i] = (float)a.mn[i]; mx[i] = (float)a.mx[i]; }
     }
     __device__ __forceinline__ void span(float &mn, float &mx) const {
-        const f16x4 a = __builtin_elementwise_min(h.lo, h.hi), b = __builtin_elementwise_max(h.lo, h.hi);
-        const f16x2 a2 = __builtin_elementwise_min(a.lo, a.hi), b2 = __builtin_elementwise_max(b.lo, b.hi);
+        typedef uint32_t w4 __attribute__((ext_vector_type(4)));
+        const w4 x = __builtin_bit_cast(w4, h);
+        const uint32_t a = pk_min(pk_min(x[0], x[1]), pk_min(x[2], x[3])), b = pk_max(pk_max(x[0], x[1]), pk_max(x[2], x[3]));
+        const f16x2 a2 = __builtin_bit_cast(f16x2, a), b2 = __builtin_bit_cast(f16x2, b);
         mn = fminf((float)a2[0], (float)a2[1]);
         mx = fmaxf((float)b2[0], (float)b2[1]);
     }
@@ -737,6 +756,15 @@ int pack_kv_pair(const void *k, const void *v, int dtype, int64_t BH, int64_t S,
     return VQ_OK;
 }
 }  // namespace vq
+
+extern "C" int vq_kivi_quant_pack_kv(const void *k, const void *v, int dtype, int64_t BH, int64_t S, int64_t D,
+                                     int64_t x_stride_bh, int group, int levels, float eps, int pack_bits, int v_layout,
+                                     void *k_packed, void *k_scale, void *k_zero, void *v_packed, void *v_scale,
+                                     void *v_zero, int meta_dtype, int64_t cap_tokens, int64_t dst_tok0, void *stream) {
+    // argument checks are those of the single calls; an invalid pair fails there
+    return pack_kv_pair(k, v, dtype, BH, S, D, x_stride_bh, group, levels, eps, pack_bits, v_layout, k_packed, k_scale, k_zero,
+                        v_packed, v_scale, v_zero, meta_dtype, cap_tokens, dst_tok0, stream);
+}
 
 extern "C" int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int axis,
                                      int group, int levels, float eps, void *stream) {

@@ -225,6 +225,63 @@ def kivi_quant_pack(x: torch.Tensor, axis: int, group_size: int, bits: int, *, l
     return packed, scale, zero
 
 
+def kivi_quant_pack_kv(k: torch.Tensor, v: torch.Tensor, group_size: int, bits: int, *, levels: int | None = None,
+                       eps: float = 1e-8, meta_dtype: torch.dtype = torch.float16, v_layout: str = "token",
+                       out: tuple | None = None, dst_tok0: int = 0):
+    """:func:`kivi_quant_pack` of the keys (``axis=-2``) and of the values (``axis=-1``, ``v_layout``) of
+    the same tokens in one library call -- one launch at head_dim 128.  ``k`` and ``v`` are
+    ``[B, H, S, D]`` of one dtype and one layout.  Returns ``((k_packed, k_scale, k_zero),
+    (v_packed, v_scale, v_zero))``; ``out`` takes the same pair of triples (buffers of one token
+    capacity) and ``dst_tok0`` the token offset, as there."""
+    name = "kivi_quant_pack_kv"
+    if k.ndim != 4 or tuple(v.shape) != tuple(k.shape) or v.dtype != k.dtype:
+        raise ValueError(f"{name}: k and v must be 4D [B,H,S,D] of one shape and dtype, got {tuple(k.shape)} {k.dtype} "
+                         f"and {tuple(v.shape)} {v.dtype}")
+    if v_layout not in _V_LAYOUT:
+        raise ValueError(f"{name}: v_layout must be 'channel' or 'token', got {v_layout!r}")
+    if not (1 <= bits <= 8):
+        raise ValueError(f"{name}: bits must be in 1..8, got {bits}")
+    if meta_dtype not in (torch.float16, torch.float32):
+        raise ValueError(f"{name}: meta_dtype must be float16 or float32, got {meta_dtype}")
+    tag = _ftag(name, k)
+    _need_gpu(name, k)
+    B, H, S, D = k.shape
+    per = 32 // bits
+    levels = (1 << bits) - 1 if levels is None else int(levels)
+    tokpacked = v_layout == "token"
+    if not (k.is_contiguous() and v.is_contiguous()):
+        k, v = k.contiguous(), v.contiguous()
+    W, GV, g = -(-D // per), -(-D // group_size), int(group_size)
+    if out is None:
+        if tokpacked and S % per:
+            raise ValueError(f"{name}: token-packed values need S % {per} == 0, got S={S}")
+        new = lambda shape, dt: torch.empty(shape, dtype=dt, device=k.device)
+        kd = (new((B, H, S, W), torch.int32), new((B, H, -(-S // g), D), meta_dtype), new((B, H, -(-S // g), D), meta_dtype))
+        if tokpacked:
+            vd = (new((B, H, S // per, D), torch.int32), new((B, H, GV, S), meta_dtype), new((B, H, GV, S), meta_dtype))
+        else:
+            vd = (new((B, H, S, W), torch.int32), new((B, H, S, GV), meta_dtype), new((B, H, S, GV), meta_dtype))
+        cap = S
+    else:
+        kd, vd = out
+        cap = kd[0].shape[2]
+        v_cap = vd[0].shape[2] * per if tokpacked else vd[0].shape[2]
+        if v_cap != cap:
+            raise ValueError(f"{name}: key and value buffers hold {cap} and {v_cap} tokens")
+        for t in (*kd[1:], *vd[1:]):
+            if t.dtype != meta_dtype:
+                raise ValueError(f"{name}: out scale/zero dtype must equal meta_dtype")
+        for t in (*kd, *vd):
+            if not t.is_contiguous():
+                raise ValueError(f"{name}: out buffers must be contiguous")
+    rc = _lib.load().vq_kivi_quant_pack_kv(
+        k.data_ptr(), v.data_ptr(), tag, B * H, S, D, S * D, g, levels, float(eps), int(bits), _V_LAYOUT[v_layout],
+        kd[0].data_ptr(), kd[1].data_ptr(), kd[2].data_ptr(), vd[0].data_ptr(), vd[1].data_ptr(), vd[2].data_ptr(),
+        VQ_F16 if meta_dtype == torch.float16 else VQ_F32, cap, int(dst_tok0), _stream(k))
+    _lib.check(rc)
+    return kd, vd
+
+
 def kivi_quant_codes(x: torch.Tensor, axis: int, group_size: int, levels: int, eps: float = 1e-8):
     """``(codes uint8, scale f32, zero f32)`` exactly as the reference's split
     form returns them (test_scalar_attend.py:51-82)."""
@@ -880,7 +937,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "kivi_group_quant_dequant", "kivi_quant_pack", "kivi_quant_codes", "kivi_dequant",
+    "hip_available", "kivi_group_quant_dequant", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",
