@@ -264,6 +264,12 @@ typedef struct vq_attend_args {
      * 0 = the process default (vq_kivi_attend_fixed_order), 1 = a fixed order (identical bits
      * from run to run), 2 = on demand (fastest; the last bits can differ between runs). */
     int32_t fixed_order;
+    /* > 0: a query at position p of the sequence (queries align to the end of the slots) sees
+     * only the slots (p - sliding_window, p], with or without `causal` -- the window of
+     * VecInferKVCache.fused_sdpa(..., sliding_window) (veloxquant_mlx/cache/vecinfer_cache.py:670-731,
+     * metal/src/fused_sdpa.metal).  Whole stretches of packed tokens below the window of every
+     * query are not read. */
+    int64_t sliding_window;
 } vq_attend_args;
 
 /* The decode kernel balances its waves by handing out token chunks on demand, so the order in

@@ -64,7 +64,7 @@ def reference_attend(q, kc, ks, kz, vc, vs, vz, g: int, scale: float) -> np.ndar
 
 
 def kivi_attend(q, kc, ks, kz, vc, vs, vz, g: int, k_tail, v_tail, scale: float,
-                causal: bool = False, acc=np.float64, recon_dtype=None) -> np.ndarray:
+                causal: bool = False, acc=np.float64, recon_dtype=None, sliding_window: int = 0) -> np.ndarray:
     """Attention over a quantised prefix followed by an fp16 tail.
 
     The tail is what ``KIVIKVCache`` keeps un-quantised (residual window plus
@@ -85,7 +85,7 @@ def kivi_attend(q, kc, ks, kz, vc, vs, vz, g: int, k_tail, v_tail, scale: float,
         parts_v.append(np.asarray(v_tail).astype(F32))
     k = np.concatenate(parts_k, axis=2)
     v = np.concatenate(parts_v, axis=2)
-    return sdpa(q, k, v, scale, causal=causal, acc=acc)
+    return sdpa(q, k, v, scale, causal=causal, acc=acc, sliding_window=sliding_window)
 
 
 def chunked_prefill(q, k, v, chunk: int, bits: int, group_size: int,

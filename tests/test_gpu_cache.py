@@ -407,6 +407,43 @@ def test_bf16_history_holds_the_reconstruction_rounded_to_bf16():
     assert np.max(np.abs(got - over_bf16)) < 1e-2
 
 
+@pytest.mark.parametrize("memory_bound", [True, False])
+def test_cache_attention_under_a_window_and_with_sequence_lengths(memory_bound):
+    """``KIVIKVCache.fused_sdpa`` with ``sliding_window`` (the parameter the fused dispatcher passes on)
+    and with per-sequence ``lengths`` of a right-padded batch, in the packed-only and the stash mode,
+    against the oracle over (reconstruction | fp16 rows)."""
+    require_gpu()
+    B, Hq, Hkv, D, g, n = 3, 8, 2, 128, 32, 700
+    k, v = outlier_kv((B, Hkv, n, D), seed=44)
+    c = _make(bit_width_inlier=4, kivi_group_size=g, residual_length=64, fused_sdpa=True,
+              fused_sdpa_memory_bound=memory_bound, kivi_meta_dtype="float32")
+    c.update_and_fetch(to_dev(k), to_dev(v))
+    nq = c._n_quantized
+    assert nq == (n - 64) // g * g
+    kc_, ks_, kz_ = ok.group_quant_codes(k[:, :, :nq], -2, g, 15)
+    vc_, vs_, vz_ = ok.group_quant_codes(v[:, :, :nq], -1, g, 15)
+    scale = 1 / math.sqrt(D)
+    rng = np.random.default_rng(45)
+    for Sq, causal in ((1, False), (5, True), (40, True)):
+        q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float16)
+        for w in (0, 17, 90, 400):
+            got = host(c.fused_sdpa(to_dev(q), scale, causal=causal, sliding_window=w)).astype(np.float32)
+            ref = oa.kivi_attend(q, kc_, ks_, kz_, vc_, vs_, vz_, g, k[:, :, nq:], v[:, :, nq:], scale, causal=causal,
+                                 sliding_window=w)
+            assert np.max(np.abs(got - ref)) < 2e-3, (Sq, w)
+        lengths = [n, 655, 300]
+        for lens in (torch.tensor(lengths), torch.tensor(lengths, device="cuda:0", dtype=torch.int32)):
+            got = host(c.fused_sdpa(to_dev(q), scale, causal=causal, lengths=lens)).astype(np.float32)
+            for b, nb in enumerate(lengths):
+                npk = min(nb, nq)
+                ref = oa.kivi_attend(q[b:b + 1], kc_[b:b + 1, :, :npk], ks_[b:b + 1, :, : -(-npk // g)], kz_[b:b + 1, :, : -(-npk // g)],
+                                     vc_[b:b + 1, :, :npk], vs_[b:b + 1, :, :npk], vz_[b:b + 1, :, :npk], g,
+                                     k[b:b + 1, :, nq:nb], v[b:b + 1, :, nq:nb], scale, causal=causal)
+                assert np.max(np.abs(got[b:b + 1] - ref)) < 2e-3, (Sq, b)
+    with pytest.raises(ValueError, match="lengths has"):
+        c.fused_sdpa(to_dev(q), scale, lengths=torch.tensor([1, 2]))
+
+
 def test_config3_decode_at_full_size_against_the_oracle_and_the_vector_kernel():
     """Benchmark configuration 3, one layer: batch 16, 32 query / 8 kv heads, D=128, 32768 tokens of
     context in a 4-bit group-64 packed cache plus the fp16 residual, one query token.  The last

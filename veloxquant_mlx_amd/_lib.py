@@ -39,6 +39,7 @@ class AttendArgs(C.Structure):
         ("packed_lens", vp), ("tail_lens", vp),
         ("k_new", vp), ("v_new", vp),
         ("fixed_order", C.c_int32),
+        ("sliding_window", C.c_int64),
     ]
 
 

@@ -292,19 +292,21 @@ class KIVIKVCache(FP16KVCache):
         return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
 
     def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0,
-                   fixed_order: bool | None = None):
+                   fixed_order: bool | None = None, lengths: torch.Tensor | None = None):
         """Attention of ``q [B,H_q,S_q,D]`` over the packed prefix and the fp16 tail,
         queries aligned to the end of the cache (the contract of
-        ``VecInferKVCache.fused_sdpa``, veloxquant_mlx/cache/vecinfer_cache.py:670-731).
+        ``VecInferKVCache.fused_sdpa``, veloxquant_mlx/cache/vecinfer_cache.py:670-731), under an
+        optional ``sliding_window`` (a query sees only that many last slots up to its own).
         ``fixed_order=True`` asks for results that are identical from run to run (see
-        :func:`veloxquant_mlx_amd.kernels.kivi_packed_attend`)."""
+        :func:`veloxquant_mlx_amd.kernels.kivi_packed_attend`).  ``lengths`` (int ``[B]``, on the
+        device or the host) gives every sequence of a right-padded batch its own number of live
+        tokens: sequence ``b`` attends over its first ``lengths[b]`` slots, its queries aligned to
+        the end of those."""
         if not self._fused_enabled:
             raise RuntimeError("KIVIKVCache.fused_sdpa called but fused_sdpa was not enabled via "
                                "KVCacheConfig.fused_sdpa=True.")
         if self.offset == 0:
             raise RuntimeError("KIVIKVCache.fused_sdpa called before any tokens were cached via update_and_fetch.")
-        if sliding_window:
-            raise ValueError("KIVIKVCache.fused_sdpa: sliding_window attention is not supported")
         nq = self._n_quantized
         n_tail = self.offset - nq
         if self._pending is not None and q.shape[2] != 1:
@@ -316,7 +318,14 @@ class KIVIKVCache(FP16KVCache):
         kw = dict(k_packed=self._kp, k_scale=self._ks, k_zero=self._kz, v_packed=self._vp, v_scale=self._vs,
                   v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
                   k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
-                  causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order)
+                  causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
+                  sliding_window=int(sliding_window or 0))
+        if lengths is not None:
+            self._store_pending()
+            n = torch.as_tensor(lengths, device=q.device).to(torch.int64).reshape(-1)
+            if n.numel() != q.shape[0]:
+                raise ValueError(f"KIVIKVCache.fused_sdpa: lengths has {n.numel()} entries for a batch of {q.shape[0]}")
+            kw.update(packed_lens=torch.clamp(n, max=nq), tail_lens=torch.clamp(n - nq, min=0, max=n_tail))
         if self._pending is not None:
             try:   # append and attend in one launch (single-query MFMA decode path)
                 out = K.kivi_packed_attend(q, k_new=self._pending[0], v_new=self._pending[1], **kw)

@@ -73,6 +73,41 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     return p;
 }
 
+static int64_t gcd64(int64_t x, int64_t y) { while (y) { const int64_t t = x % y; x = y; y = t; } return x; }
+
+// Sliding window: packed tokens below the window of the call's first query are seen by none of
+// its queries.  Whole stretches of them (a common multiple of 128 tokens, the token group and the
+// codes of a word) are dropped by moving the buffer bases forward; the strides between sequences
+// and heads stay those of cap_tokens, so the kernels address the rest as before.  What is left
+// below the window inside the first stretch is masked in the kernels.
+static vq_attend_args skip_below_window(const vq_attend_args &a) {
+    if (a.sliding_window <= 0 || a.packed_lens != nullptr || a.n_packed <= 0) return a;
+    int64_t first = a.n_packed + a.n_tail - a.Sq + 1 - a.sliding_window;   // first slot of the first query
+    if (first > a.n_packed) first = a.n_packed;
+    const int64_t per = 32 / a.pack_bits;
+    int64_t unit = 128 / gcd64(128, a.group) * a.group;
+    unit = unit / gcd64(unit, per) * per;
+    const int64_t skip = first > 0 ? first / unit * unit : 0;
+    if (skip <= 0) return a;
+    vq_attend_args b = a;
+    const int64_t W = cdiv(a.D, per), GV = cdiv(a.D, a.group), es = a.meta_dtype == VQ_F16 ? 2 : 4;
+    auto fwd = [](const void *p, int64_t bytes) { return (const void *)((const char *)p + bytes); };
+    b.k_packed = fwd(a.k_packed, skip * W * 4);
+    b.k_scale = fwd(a.k_scale, skip / a.group * a.D * es);
+    b.k_zero = fwd(a.k_zero, skip / a.group * a.D * es);
+    if (a.v_layout == VQ_V_TOKEN_PACKED) {
+        b.v_packed = fwd(a.v_packed, skip / per * a.D * 4);
+        b.v_scale = fwd(a.v_scale, skip * es);
+        b.v_zero = fwd(a.v_zero, skip * es);
+    } else {
+        b.v_packed = fwd(a.v_packed, skip * W * 4);
+        b.v_scale = fwd(a.v_scale, skip * GV * es);
+        b.v_zero = fwd(a.v_zero, skip * GV * es);
+    }
+    b.n_packed = a.n_packed - skip;
+    return b;
+}
+
 static int validate(const vq_attend_args *a, const char *fn) {
     VQ_REQUIRE(a != nullptr, VQ_ERR_INVALID, "%s: null argument block", fn);
     VQ_REQUIRE(a->B >= 1 && a->Hq >= 1 && a->Hkv >= 1 && a->Sq >= 1 && a->D >= 1, VQ_ERR_INVALID,
@@ -85,6 +120,7 @@ static int validate(const vq_attend_args *a, const char *fn) {
     VQ_REQUIRE(a->n_packed >= 0 && a->n_tail >= 0, VQ_ERR_INVALID, "%s: negative token count", fn);
     VQ_REQUIRE(a->n_packed + a->n_tail >= 1, VQ_ERR_INVALID, "%s: no key/value slots to attend to", fn);
     VQ_REQUIRE(a->fixed_order >= 0 && a->fixed_order <= 3, VQ_ERR_INVALID, "%s: fixed_order must be 0, 1, 2 or 3", fn);
+    VQ_REQUIRE(a->sliding_window >= 0, VQ_ERR_INVALID, "%s: negative sliding window", fn);
     VQ_REQUIRE(a->Sq <= a->n_packed + a->n_tail || !a->causal, VQ_ERR_INVALID,
                "%s: S_q=%lld exceeds S_kv=%lld; queries align to the tail of the KV cache", fn, (long long)a->Sq,
                (long long)(a->n_packed + a->n_tail));
@@ -118,23 +154,25 @@ extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
     if (!a || a->B < 1 || a->Hq < 1 || a->Hkv < 1 || a->Sq < 1 || a->D < 1 || a->Hq % a->Hkv != 0 ||
         a->n_packed < 0 || a->n_tail < 0 || (a->n_packed > 0 && (a->pack_bits < 1 || a->pack_bits > 8 || a->group < 1)))
         return 0;
-    AttendPlan p = plan_attend(*a);
+    AttendPlan p = plan_attend(skip_below_window(*a));
     return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nparts * (size_t)(a->D + 2) * sizeof(float);
 }
 
 extern "C" int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts) {
     int rc = validate(a, "vq_kivi_attend_plan");
     if (rc != VQ_OK) return rc;
-    AttendPlan p = plan_attend(*a);
+    AttendPlan p = plan_attend(skip_below_window(*a));
     if (path) *path = p.path;
     if (nparts) *nparts = p.nparts;
     return VQ_OK;
 }
 
-extern "C" int vq_kivi_attend(const vq_attend_args *a) {
+extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
     const char *fn = "vq_kivi_attend";
-    int rc = validate(a, fn);
+    int rc = validate(a_in, fn);
     if (rc != VQ_OK) return rc;
+    const vq_attend_args windowed = skip_below_window(*a_in);
+    const vq_attend_args *a = &windowed;
     VQ_REQUIRE(a->q && a->out, VQ_ERR_INVALID, "%s: null q/out", fn);
     if (a->n_packed > 0)
         VQ_REQUIRE(a->k_packed && a->v_packed && a->k_scale && a->k_zero && a->v_scale && a->v_zero, VQ_ERR_INVALID,
@@ -195,7 +233,7 @@ extern "C" int vq_kivi_attend_static(const vq_attend_args *a) {
     VQ_REQUIRE(need <= STATIC_WS_BYTES, VQ_ERR_WORKSPACE,
                "%s: these shapes need %zu bytes of split partials, the built-in scratch holds %zu; use vq_kivi_attend "
                "with a workspace of its own", fn, need, STATIC_WS_BYTES);
-    const AttendPlan p = plan_attend(*a);
+    const AttendPlan p = plan_attend(skip_below_window(*a));
     VQ_REQUIRE((size_t)(a->B * a->Hkv * p.tiles) <= STATIC_COUNTERS, VQ_ERR_WORKSPACE,
                "%s: B * H_kv * row tiles = %lld exceeds the %zu built-in sync counters", fn,
                (long long)(a->B * a->Hkv * p.tiles), STATIC_COUNTERS);

@@ -13,6 +13,13 @@ __device__ __forceinline__ void take_sequence_lengths(vq_attend_args &a, int64_t
     }
 }
 
+// first slot a query at position `pos` (of Sq, aligned to the end of n_total slots) sees under a
+// sliding window; 0 without one
+__device__ __host__ __forceinline__ int64_t window_first(const vq_attend_args &a, int64_t n_total, int64_t pos) {
+    const int64_t lo = n_total - a.Sq + pos + 1 - a.sliding_window;
+    return a.sliding_window > 0 && lo > 0 ? lo : 0;
+}
+
 struct AttendPlan {
     int path;           // 0 generic waves, 1 MFMA decode (row tiles of <= 8), 2 MFMA prefill (LDS-staged, 64-row blocks)
     int nsplit;         // splits along the tokens the main kernel covers

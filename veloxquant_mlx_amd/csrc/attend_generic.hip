@@ -46,6 +46,8 @@ __global__ __launch_bounds__(256) void attend_generic_kernel(vq_attend_args a, i
     const int64_t last = a.causal ? (n_total - a.Sq + iq) : (n_total - 1);
     int64_t t0 = (int64_t)sp * split_len, t1 = t0 + split_len;
     if (t1 > last + 1) t1 = last + 1;
+    const int64_t first = window_first(a, n_total, iq);
+    if (t0 < first) t0 = first;
 
     const int bits = a.pack_bits, per = 32 / bits, g = a.group;
     const uint32_t mask = (1u << bits) - 1u;

@@ -187,7 +187,15 @@ struct RowTile {
     int64_t base_row;   // flattened [B, Hq, Sq] row of (b, first head of the group, position 0)
     int64_t Sq, n_total;
     int R, RT, pos0, causal;
+    int64_t window;     // sliding window (0: none)
     __device__ __forceinline__ bool valid(int j) const { return j < RT && pos0 + j / R < Sq; }
+    // first visible slot of tile row j
+    __device__ __forceinline__ int64_t first(int j) const {
+        int64_t pos = pos0 + j / R;
+        if (pos > Sq - 1) pos = Sq - 1;
+        const int64_t lo = n_total - Sq + pos + 1 - window;
+        return window > 0 && lo > 0 ? lo : 0;
+    }
     __device__ __forceinline__ int64_t row(int j) const { return base_row + (int64_t)(j % R) * Sq + pos0 + j / R; }
     // number of visible slots of tile row j (queries align to the end of the slots)
     __device__ __forceinline__ int64_t visible(int j) const {
@@ -285,6 +293,8 @@ __device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, c
     // tail tokens this lane's query row sees
     int64_t n_vis = tile.visible(i < R ? i : 0) - a.n_packed;
     if (n_vis > a.n_tail) n_vis = a.n_tail;
+    int64_t n_lo = tile.first(i < R ? i : 0) - a.n_packed;   // first tail token the row sees
+    if (n_lo < 0) n_lo = 0;
     TailAcc acc;
 #pragma unroll
     for (int n = 0; n < 9; ++n) acc.O[n] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -341,7 +351,7 @@ __device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, c
         for (int Tt = 0; Tt < 2; ++Tt)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                if (i < R && base + tail_tok(blk, r, Tt) >= n_vis) S[Tt][r] = -INFINITY;
+                if (i < R && (base + tail_tok(blk, r, Tt) >= n_vis || base + tail_tok(blk, r, Tt) < n_lo)) S[Tt][r] = -INFINITY;
         const f16x8 P = tail_softmax_unit(S, c, acc, blk);
 #pragma unroll
         for (int nt = 0; nt < 8; ++nt) {   // lane column i is channel 8*i + nt

@@ -189,7 +189,7 @@ template <int N> __device__ __forceinline__ float row_ror(float x) {
 // counted ones (a slower, count-free cross-check of the ring's accounting)
 template <int BITS, typename M, int GV, int RTP>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, float c, int64_t t_begin,
-                                             int n_units, int lane_vis, int full_vis, int lane, int wave,
+                                             int n_units, int lane_vis, int full_vis, int lane_lo, int lo_edge, int lane, int wave,
                                              PackedAcc<Cols<GV, RTP>::NP, sizeof(M) != 2> &acc, const f16 *s_qraw,
                                              const char *s_const, char *ring, int *s_next, int order) {
     using CL = Cols<GV, RTP>;
@@ -442,6 +442,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     // ---- second half: softmax, output
     // lane_vis, full_vis, base: token positions counted from the block's first token
     const int lane_vis0 = lane_vis - tok_a;   // visible tokens counted from the lane's first token of a unit
+    const int lane_lo0 = lane_lo - tok_a;     // first visible token (sliding window), counted the same way
     auto finish = [&](const Unit &cur, f32x4 (&S)[2], int base) VQ_INLINE_LAMBDA {
         // high + remainder column: every column ends up with the full score of its row
 #pragma unroll
@@ -450,14 +451,16 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             for (int r = 0; r < 4; ++r) S[T][r] += row_ror<RTP>(S[T][r]);
         // causal edge: tokens this lane's query row does not see (units below full_vis are
         // visible to every row of the tile); a real branch, taken by the last units of a block only
-        if (base + 32 > full_vis) {
+        // (and, under a sliding window, the first units of the sequence: tokens below lo_edge are
+        // hidden from some row)
+        if (base + 32 > full_vis || base < lo_edge) {
             asm volatile("" ::: "memory");
-            const int lv = lane_vis0 - base;
+            const int lv = lane_vis0 - base, ll = lane_lo0 - base;
 #pragma unroll
             for (int T = 0; T < 2; ++T)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (r + T * GAP >= lv) S[T][r] = -INFINITY;
+                    if (r + T * GAP >= lv || r + T * GAP < ll) S[T][r] = -INFINITY;
         }
 
         // softmax against a lazily updated reference: the fast path touches no other lane
@@ -667,6 +670,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     tile.Sq = a.Sq;
     tile.n_total = a.n_packed + a.n_tail;
     tile.causal = a.causal;
+    tile.window = a.sliding_window;
     tile.base_row = (b * a.Hq + hkv * tile.R) * a.Sq;
     const int RT = tile.RT;
 
@@ -715,7 +719,11 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int64_t rel_cap = (int64_t)n_units * 32 + 64;
     const int lane_rel = (int)(lane_vis - t_begin < 0 ? 0 : lane_vis - t_begin > rel_cap ? rel_cap : lane_vis - t_begin);
     const int full_rel = (int)(full_vis - t_begin < 0 ? 0 : full_vis - t_begin > rel_cap ? rel_cap : full_vis - t_begin);
-    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lane, wave, acc, s_qraw, s_const,
+    // sliding window: first token the lane's row sees, and the first token every row sees
+    const int64_t lane_first = tile.first(n % RTP < RT ? n % RTP : 0) - t_begin, edge_first = tile.first(RT - 1) - t_begin;
+    const int lo_rel = (int)(lane_first < 0 ? 0 : lane_first > rel_cap ? rel_cap : lane_first);
+    const int edge_rel = (int)(edge_first < 0 ? 0 : edge_first > rel_cap ? rel_cap : edge_first);
+    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lo_rel, edge_rel, lane, wave, acc, s_qraw, s_const,
                                    s_ring, &s_next, order);
     __syncthreads();   // every wave has read its last slot
 

@@ -140,7 +140,17 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     const int n_tunits = (max_tvis + 31) / 32;
     const int n_work = n_punits + n_tunits;
     const int nsplit = (int)gridDim.z, sp = (int)blockIdx.z;
-    const int w0 = (int)((int64_t)n_work * sp / nsplit), w1 = (int)((int64_t)n_work * (sp + 1) / nsplit);
+    // units below the window of the block's first row are seen by none of its rows
+    const int64_t first_blk = window_first(a, n_total, pos0);
+    const int w_lo = first_blk < a.n_packed ? (int)(first_blk / 32) : n_punits + (int)((first_blk - a.n_packed) / 32);
+    const int w_n = n_work > w_lo ? n_work - w_lo : 0;
+    const int w0 = w_lo + (int)((int64_t)w_n * sp / nsplit), w1 = w_lo + (int)((int64_t)w_n * (sp + 1) / nsplit);
+    // sliding window: first packed / tail token this lane's row sees, and the first every row sees
+    const int64_t first_lane = window_first(a, n_total, row_ok ? pos : a.Sq - 1), first_all = window_first(a, n_total, last_pos);
+    const int lane_lo = (int)(first_lane < a.n_packed ? first_lane : a.n_packed);
+    const int edge_lo = (int)(first_all < a.n_packed ? first_all : a.n_packed);
+    const int lane_tlo = (int)(first_lane > a.n_packed ? first_lane - a.n_packed : 0);
+    const int edge_tlo = (int)(first_all > a.n_packed ? first_all - a.n_packed : 0);
 
     // query as the B operand: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of row n
     f16x8 qn[4];
@@ -276,13 +286,13 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
     // and repeats the unit.  Otherwise P is the A operand of the second product (pair r =
     // tokens 8 blk + 2 r, 8 blk + 2 r + 1).
     float m_seen = -INFINITY;
-    auto softmax = [&](f32x4 (&S)[2], int base, int lim, int full, u32 (&P)[4]) -> bool {
-        if (base + 32 > full) {
+    auto softmax = [&](f32x4 (&S)[2], int base, int lim, int full, int lo, int lo_edge, u32 (&P)[4]) -> bool {
+        if (base + 32 > full || base < lo_edge) {
 #pragma unroll
             for (int T = 0; T < 2; ++T)
 #pragma unroll
                 for (int r = 0; r < 4; ++r)
-                    if (base + pf_tok(blk, r, T) >= lim) S[T][r] = -INFINITY;
+                    if (base + pf_tok(blk, r, T) >= lim || base + pf_tok(blk, r, T) < lo) S[T][r] = -INFINITY;
         }
         const float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
                                fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
@@ -317,7 +327,7 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
         m_run = m_new;
     };
 
-    auto compute = [&](int buf, int base, int lim, int full, const Meta &vm) -> bool {
+    auto compute = [&](int buf, int base, int lim, int full, int lo, int lo_edge, const Meta &vm) -> bool {
         // two accumulator chains per score tile (high and remainder part of the folded query)
         f32x4 S[2], Sl[2];
 #pragma unroll
@@ -333,7 +343,7 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
             S[T] += Sl[T];
         }
         u32 P[4];
-        if (!softmax(S, base, lim, full, P)) return false;
+        if (!softmax(S, base, lim, full, lo, lo_edge, P)) return false;
         const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
         // per channel group: A = P * s_g as fp16 high part plus exact fp16 remainder
 #pragma unroll
@@ -392,7 +402,8 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
             cur_group = grp;
             open_group(buf);
         }
-        if (!compute(buf, base, packed ? lane_vis : lane_tvis, packed ? full_vis : full_tvis, vm)) {
+        if (!compute(buf, base, packed ? lane_vis : lane_tvis, packed ? full_vis : full_tvis, packed ? lane_lo : lane_tlo,
+                     packed ? edge_lo : edge_tlo, vm)) {
             rescale();
             continue;
         }
@@ -474,6 +485,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
 
     // ---- this lane's query rows (score columns): row j = 32 wave + 16 rb + n of the block
     int lane_vis[PR_RB], lane_tvis[PR_RB];
+    int lane_lo[PR_RB], lane_tlo[PR_RB];   // sliding window: first packed / tail token the row sees
     f16x8 qn[PR_RB][4];   // B operands: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of its row
 #pragma unroll
     for (int rb = 0; rb < PR_RB; ++rb) {
@@ -485,6 +497,9 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         lane_vis[rb] = (int)(vis < a.n_packed ? vis : a.n_packed);
         const int64_t tv = vis - a.n_packed;
         lane_tvis[rb] = (int)(tv < 0 ? 0 : tv < a.n_tail ? tv : a.n_tail);
+        const int64_t first = window_first(a, n_total, row_ok ? pos : a.Sq - 1);
+        lane_lo[rb] = (int)(first < a.n_packed ? first : a.n_packed);
+        lane_tlo[rb] = (int)(first > a.n_packed ? first - a.n_packed : 0);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const int64_t e0 = qrow * MF_D + 32 * ks + 8 * blk;
@@ -507,7 +522,14 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int n_tunits = (max_tvis + 31) / 32;
     const int n_work = n_punits + n_tunits;
     const int nsplit = (int)gridDim.z, sp = (int)blockIdx.z;
-    const int w0 = (int)((int64_t)n_work * sp / nsplit), w1 = (int)((int64_t)n_work * (sp + 1) / nsplit);
+    // units below the window of the block's first row are seen by none of its rows
+    const int64_t first_blk = window_first(a, n_total, pos0);
+    const int w_lo = first_blk < a.n_packed ? (int)(first_blk / 32) : n_punits + (int)((first_blk - a.n_packed) / 32);
+    const int w_n = n_work > w_lo ? n_work - w_lo : 0;
+    const int w0 = w_lo + (int)((int64_t)w_n * sp / nsplit), w1 = w_lo + (int)((int64_t)w_n * (sp + 1) / nsplit);
+    const int64_t first_all = window_first(a, n_total, last_pos);   // below it some row of the block sees nothing
+    const int edge_lo = (int)(first_all < a.n_packed ? first_all : a.n_packed);
+    const int edge_tlo = (int)(first_all > a.n_packed ? first_all - a.n_packed : 0);
 
     // ---- producer side
     const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
@@ -645,7 +667,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     // side), softmax against the lazily updated references (raised in place, with the
     // accumulators rescaled, when some row's scores outgrow its reference), second product.
     // `next` is the buffer of the following unit (stale but harmless after the last one).
-    auto compute = [&](int next, int base, bool packed, int full) {
+    auto compute = [&](int next, int base, bool packed, int full, int lo_edge) {
         f32x4 S[PR_RB][2];
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
@@ -658,13 +680,13 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         bool grow = false;
 #pragma unroll
         for (int rb = 0; rb < PR_RB; ++rb) {
-            if (base + 32 > full) {
-                const int lim = packed ? lane_vis[rb] : lane_tvis[rb];
+            if (base + 32 > full || base < lo_edge) {
+                const int lim = packed ? lane_vis[rb] : lane_tvis[rb], lo = packed ? lane_lo[rb] : lane_tlo[rb];
 #pragma unroll
                 for (int T = 0; T < 2; ++T)
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
-                        if (base + pf_tok(blk, r, T) >= lim) S[rb][T][r] = -INFINITY;
+                        if (base + pf_tok(blk, r, T) >= lim || base + pf_tok(blk, r, T) < lo) S[rb][T][r] = -INFINITY;
             }
             const float mx = vmax3(vmax3(S[rb][0][0], S[rb][0][1], S[rb][0][2]), vmax3(S[rb][0][3], S[rb][1][0], S[rb][1][1]),
                                    vmax3(S[rb][1][2], S[rb][1][3], S[rb][1][3]));
@@ -720,7 +742,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         if (early) produce();
         const bool packed = w < n_punits;
         const int base = packed ? w * 32 : (w - n_punits) * 32;
-        compute(next, base, packed, packed ? full_vis : full_tvis);
+        compute(next, base, packed, packed ? full_vis : full_tvis, packed ? edge_lo : edge_tlo);
         if (!early) produce();
         __syncthreads();
         cur = next;

@@ -701,7 +701,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        num_splits: int = 0, packed_lens: torch.Tensor | None = None,
                        tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
                        v_new: torch.Tensor | None = None, fixed_order: bool | None = None,
-                       out: torch.Tensor | None = None, static_scratch: bool = False,
+                       out: torch.Tensor | None = None, static_scratch: bool = False, sliding_window: int = 0,
                        _plan_out: dict | None = None, _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
@@ -777,6 +777,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
+    a.sliding_window = int(sliding_window or 0)
     a.fixed_order = 0 if fixed_order is None else (int(fixed_order) if fixed_order is not True and fixed_order is not False and int(fixed_order) > 2 else (1 if fixed_order else 2))
     if (packed_lens is None) != (tail_lens is None):
         raise ValueError(f"{name}: packed_lens and tail_lens go together")
