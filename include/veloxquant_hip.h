@@ -270,6 +270,20 @@ typedef struct vq_attend_args {
      * metal/src/fused_sdpa.metal).  Whole stretches of packed tokens below the window of every
      * query are not read. */
     int64_t sliding_window;
+    /* Protected rows of a sink-protecting cache (SinkProtectedKVCache,
+     * veloxquant_mlx/cache/sink_cache.py:117-198, on packed storage -- the reference keeps such rows
+     * exact inside its fp16 history and has no packed form).  The packed store holds a stand-in at
+     * every protected position (the neighbouring row that took its place when the group was
+     * quantised) whose value scale and zero are 0, so it adds nothing to the output sums; the exact
+     * rows sit here: sink_k / sink_v [B, Hkv, sink_cap, D] in sink_dtype, sink_pos int32
+     * [B, sink_cap] with the position of each row in its sequence (-1: unused slot; positions are
+     * below n_packed).  After the attention kernels a patch pass takes the stand-ins' weights out of
+     * every query row's softmax sum and puts the exact rows in, under the same causal / window
+     * visibility.  NULL sink_k: none. */
+    const void *sink_k, *sink_v;
+    const int32_t *sink_pos;
+    int64_t sink_cap;
+    int32_t sink_dtype;
 } vq_attend_args;
 
 /* The decode kernel balances its waves by handing out token chunks on demand, so the order in

@@ -319,6 +319,35 @@ class SinkCacheModel(KiviCacheModel):
         self.tokens_seen += S
         return self.keys[:, :, : self.offset], self.values[:, :, : self.offset]
 
+    def trim(self, n: int) -> int:
+        """sink_cache.py:200-225: the frontier snaps down to a group multiple; protected rows of the
+        stretch that is live again (largest count over the batch, as the flush counted them) leave
+        the fp16 pool; candidates at dropped positions are forgotten."""
+        n = min(self.offset, n)
+        if not n:
+            return n
+        old_nq = self.n_quantized
+        self.offset -= n
+        B, H, D = self.shape_bhd
+        new_nq = min(old_nq, (max(self.offset, 0) // self.g) * self.g)
+        rolled = old_nq - new_nq
+        self.n_quantized = new_nq
+        back = 0
+        for b, norms in enumerate(self.sink_norms):
+            back = max(back, sum(1 for p in norms if new_nq <= p < old_nq))
+            self.sink_norms[b] = {p: x for p, x in norms.items() if p < self.offset}
+        back = min(back, rolled)
+        if rolled - back > 0:
+            k, v = quantized_bytes(rolled - back, B, H, D, self.bits, self.g)
+            self.key_bytes_compressed = max(0, self.key_bytes_compressed - k)
+            self.value_bytes_compressed = max(0, self.value_bytes_compressed - v)
+        self.key_bytes_fp16 = max(0, self.key_bytes_fp16 - H * B * n * D * 2)
+        self.value_bytes_fp16 = max(0, self.value_bytes_fp16 - H * B * n * D * 2)
+        self.tokens_seen = max(0, self.tokens_seen - n)
+        self.residual_fp16_bytes = (self.offset - self.n_quantized) * D * 2 * 2 * H * B
+        self.sink_fp16_bytes = max(0, self.sink_fp16_bytes - back * D * 2 * 2 * H * B)
+        return n
+
     def sink_positions_for(self, b):
         if b >= len(self.sink_norms):
             return []

@@ -226,12 +226,81 @@ def test_sink_protected_cache_matches_model(n_sink):
     if n_sink:
         assert 3 in c.sink_positions_for(0) and 150 in c.sink_positions_for(1) and 310 in c.sink_positions_for(1)
         assert np.array_equal(host(ko)[0, :, 3], k[0, :, 3])
-    assert c.trim(100) == 100 and c.offset == 230 and c._n_quantized == (230 // 32) * 32
+    assert c.trim(100) == m.trim(100) == 100 and c.offset == 230 and c._n_quantized == m.n_quantized == (230 // 32) * 32
     assert all(p < 230 for b in range(B) for p in c.sink_positions_for(b))
-    with pytest.raises(ValueError, match="fused_sdpa"):
-        KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, fused_sdpa=True))
+    for b in range(B):
+        assert c.sink_positions_for(b) == m.sink_positions_for(b)
+    for name, want in (("compressed_key_bytes", m.key_bytes_compressed), ("sink_fp16_bytes", m.sink_fp16_bytes),
+                       ("residual_fp16_bytes", m.residual_fp16_bytes)):
+        assert getattr(c, name) == want, name
     with pytest.raises(ValueError, match="n_sink_tokens"):
         KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, n_sink_tokens=-1))
+
+
+@pytest.mark.parametrize("mode", ["memory_bound", "stash"])
+@pytest.mark.parametrize("bits,g,v_layout", [(4, 32, "token"), (2, 32, "token"), (4, 64, "channel")])
+def test_sink_protected_cache_on_packed_storage(mode, bits, g, v_layout):
+    """``kivi_sink`` with ``fused_sdpa``: the packed store holds stand-ins at the protected positions and
+    the attention call swaps the exact rows in.  The oracle is attention over the history the numpy
+    model of the reference's cache returns (sink_cache.py:117-198: protected rows exact, the rest
+    round-tripped with the stand-ins setting the group parameters), at every stage of prefill,
+    decode steps that flush, a trim and more decode; queries are aimed at the protected keys, so
+    the weights that are swapped are the large ones.  Accounting and protected positions equal the
+    model's as in the unpacked cache."""
+    require_gpu()
+    rng = np.random.default_rng(17)
+    B, Hq, H, D, R = 2, 8, 2, 128, 64
+    n = 420
+    k = rng.standard_normal((B, H, n, D)).astype(np.float16)
+    v = rng.standard_normal((B, H, n, D)).astype(np.float16)
+    for b, p, f in ((0, 3, 12), (0, 40, 9), (1, 150, 12), (1, 151, 10), (1, 310, 14), (0, 333, 8)):
+        k[b, :, p] *= f
+    c = KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=g,
+                                            residual_length=R, n_sink_tokens=3, fused_sdpa=True,
+                                            fused_sdpa_memory_bound=(mode == "memory_bound"), kivi_meta_dtype="float32",
+                                            kivi_value_layout=v_layout))
+    m = ok.SinkCacheModel(bits, g, R, 3)
+    scale = 1 / math.sqrt(D)
+
+    def check(Sq, tag):
+        km, vm = m.keys[:, :, : m.offset], m.values[:, :, : m.offset]
+        q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float16)
+        # half of the query heads look at a protected key of their sequence
+        for b in range(B):
+            for p in m.sink_positions_for(b)[:2]:
+                q[b, ::2, -1] += (0.4 * km[b, 0, p] / np.linalg.norm(km[b, 0, p].astype(np.float32)) * 8).astype(np.float16)
+        for causal, w in ((Sq > 1, 0), (Sq > 1, 130)):
+            got = host(c.fused_sdpa(to_dev(q), scale, causal=causal, sliding_window=w)).astype(np.float32)
+            ref = oa.sdpa(q, km, vm, scale, causal=causal, sliding_window=w)
+            err = float(np.max(np.abs(got - ref)))
+            print(f"{tag}: Sq={Sq} window={w}: {len(c._side_pos[0]) if c._side_pos else 0}+{len(c._side_pos[1]) if len(c._side_pos) > 1 else 0} "
+                  f"rows in the side store, max err {err:.2e}")
+            assert err < 2e-3, (tag, Sq, causal, w, err)
+
+    steps = [(0, 200)] + [(s, s + 1) for s in range(200, 300)] + [(300, 420)]
+    for i, (s0, s1) in enumerate(steps):
+        c.update_and_fetch(to_dev(k[:, :, s0:s1]), to_dev(v[:, :, s0:s1]))
+        m.update_and_fetch(k[:, :, s0:s1], v[:, :, s0:s1])
+        if i in (0, 40, 100):
+            check(1, f"step {i}")
+        if i in (0, 101):
+            check(s1 - s0 if s1 - s0 < 100 else 24, f"chunk {i}")
+    assert c._n_quantized == m.n_quantized and c.offset == m.offset
+    for b in range(B):
+        assert c.sink_positions_for(b) == m.sink_positions_for(b)
+    for name, want in (("compressed_key_bytes", m.key_bytes_compressed), ("compressed_value_bytes", m.value_bytes_compressed),
+                       ("sink_fp16_bytes", m.sink_fp16_bytes), ("residual_fp16_bytes", m.residual_fp16_bytes)):
+        assert getattr(c, name) == want, name
+    assert any(c._side_pos[b] for b in range(B))
+    assert c.trim(130) == m.trim(130)
+    assert c._n_quantized == m.n_quantized and all(p < c._n_quantized for ps in c._side_pos for p in ps)
+    check(1, "after trim")
+    for s in range(290, 330):
+        c.update_and_fetch(to_dev(k[:, :, s:s + 1]), to_dev(v[:, :, s:s + 1]))
+        m.update_and_fetch(k[:, :, s:s + 1], v[:, :, s:s + 1])
+    check(1, "decode after trim")
+    check(16, "chunk after trim")
+    assert c.sink_fp16_bytes == m.sink_fp16_bytes and c.compressed_key_bytes == m.key_bytes_compressed
 
 
 def test_chunked_prefill_through_the_cache_matches_oracle():

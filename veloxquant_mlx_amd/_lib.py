@@ -40,6 +40,8 @@ class AttendArgs(C.Structure):
         ("k_new", vp), ("v_new", vp),
         ("fixed_order", C.c_int32),
         ("sliding_window", C.c_int64),
+        ("sink_k", C.c_void_p), ("sink_v", C.c_void_p), ("sink_pos", C.c_void_p),
+        ("sink_cap", C.c_int64), ("sink_dtype", C.c_int32),
     ]
 
 

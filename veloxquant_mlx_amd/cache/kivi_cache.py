@@ -39,6 +39,10 @@ class KIVIKVCache(FP16KVCache):
     natively quantised cache, kivi_cache.py:93-95); see ``assigned_avg_bits``.
     """
 
+    # append + flush + next tail in one library call; a subclass that works on the rows of a flush
+    # before they are packed turns it off and gets them through _pack_block
+    _one_call_append = True
+
     def __init__(self, config: Any) -> None:
         super().__init__()
         self._head_dim = int(config.head_dim)
@@ -241,8 +245,8 @@ class KIVIKVCache(FP16KVCache):
                 tv[:, :, :n_tail] = self._tail_v[:, :, :n_tail]
             self._tail_k, self._tail_v = tk, tv
         es = keys.element_size()
-        one_call = (keys.dtype == self._tail_k.dtype and values.dtype == keys.dtype and (D * es) % 16 == 0
-                    and keys.stride(3) == 1 and values.stride(3) == 1)
+        one_call = (self._one_call_append and keys.dtype == self._tail_k.dtype and values.dtype == keys.dtype
+                    and (D * es) % 16 == 0 and keys.stride(3) == 1 and values.stride(3) == 1)
         if not one_call:
             self._tail_k[:, :, n_tail:need] = keys
             self._tail_v[:, :, n_tail:need] = values
@@ -320,6 +324,7 @@ class KIVIKVCache(FP16KVCache):
                   k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
                   causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
                   sliding_window=int(sliding_window or 0))
+        kw.update(self._extra_attend_args())
         if lengths is not None:
             self._store_pending()
             n = torch.as_tensor(lengths, device=q.device).to(torch.int64).reshape(-1)
@@ -334,6 +339,10 @@ class KIVIKVCache(FP16KVCache):
             except ValueError:   # a shape that path does not take: store the token, then attend
                 self._store_pending()
         return K.kivi_packed_attend(q, **kw)
+
+    def _extra_attend_args(self) -> dict:
+        """Further arguments of the attention call (subclasses with rows kept outside the packed store)."""
+        return {}
 
     # ------------------------------------------------------------------ trim / state
     def _rollback_frontier(self, new_offset: int) -> int:

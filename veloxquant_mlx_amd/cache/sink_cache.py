@@ -11,9 +11,14 @@ How it is done here: the running top-k lives in two small host tensors ``[B, n]`
 by (norm descending, position ascending), which is the order the reference's stable sort of its
 position->norm mapping yields; a flush turns the protected positions of the block into one
 gather index and one row mask per batch element and runs gather -> group round trip -> select
-on the device for the whole batch at once.  The packed (``fused_sdpa``) modes of ``KIVIKVCache``
-are not offered: a protected row would have to be hidden from the packed prefix inside the
-attention kernels.
+on the device for the whole batch at once.
+
+The packed (``fused_sdpa``) modes of ``KIVIKVCache`` work as well, which the reference does not
+offer: the block is packed with the stand-ins in place, the value scale / zero of a protected
+position are stored as zeros (its stand-in then adds nothing to the attention output), the exact
+rows go to a small side store ``[B, H, n, D]`` with their positions, and the attention call takes
+the stand-ins' softmax weights out and puts the exact rows in (``sinks`` of
+:func:`veloxquant_mlx_amd.kernels.kivi_packed_attend`).
 """
 
 from __future__ import annotations
@@ -93,17 +98,21 @@ def _stand_in_index(protected: torch.Tensor) -> torch.Tensor:
 
 
 class SinkProtectedKVCache(KIVIKVCache):
+    _one_call_append = False     # the rows of a flush pass through _pack_block
+
     def __init__(self, config: Any) -> None:
         super().__init__(config)
-        if self._fused_enabled:
-            raise QuantizerConfigError(
-                "SinkProtectedKVCache: fused_sdpa / packed storage is not available for method='kivi_sink'; "
-                "use method='kivi' for the packed cache.")
         self._n_sink = int(getattr(config, "n_sink_tokens", 5))
         if self._n_sink < 0:
             raise QuantizerConfigError(f"SinkProtectedKVCache: n_sink_tokens={self._n_sink} must be >= 0.")
         self._top = _TopNorms(self._n_sink)
         self._sink_fp16_bytes = 0
+        self._flush_protected = 0        # protected rows of the flush in progress (largest count over the batch)
+        self._frontier_before_trim = 0
+        # packed modes: exact rows of the protected positions below the frontier
+        self._side_k = self._side_v = None     # [B, H, cap, D]
+        self._side_pos: list[list[int]] = []   # per sequence, slot order
+        self._side_pos_dev = None              # int32 [B, cap], -1 for an unused slot
 
     # ------------------------------------------------------------------ protocol
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
@@ -112,15 +121,18 @@ class SinkProtectedKVCache(KIVIKVCache):
         if self._n_sink:
             token_norm = torch.linalg.vector_norm(keys.float(), dim=-1).mean(dim=1)      # [B, S]
             self._top.fold(token_norm.cpu(), self.offset)
+        if self._memory_bound:
+            return self._update_memory_bound(keys, values)
         k_all, v_all = FP16KVCache.update_and_fetch(self, keys, values)
 
         lo, hi = self._n_quantized, self._quantization_boundary()
-        n_protected = 0
         if hi > lo:
             k_blk, v_blk = self.keys[:, :, lo:hi], self.values[:, :, lo:hi]
+            if self._fused_enabled:
+                self._pack_block(k_blk, v_blk, lo)       # from the still-exact rows
             protected = self._top.inside(lo, hi)[:B] if self._n_sink else None
             if protected is not None and bool(protected.any()):
-                n_protected = int(protected.sum(dim=1).max())
+                self._flush_protected = int(protected.sum(dim=1).max())
                 take = _stand_in_index(protected).to(keys.device)[:, None, :, None].expand(B, H, hi - lo, D)
                 keep = protected.to(keys.device)[:, None, :, None]
                 k_new = torch.where(keep, k_blk, self._quant_dequant_along(k_blk.gather(2, take), axis=-2))
@@ -131,12 +143,16 @@ class SinkProtectedKVCache(KIVIKVCache):
             self.keys[:, :, lo:hi], self.values[:, :, lo:hi] = k_new, v_new
             self._n_quantized = hi
             k_all, v_all = self.keys[:, :, : self.offset], self.values[:, :, : self.offset]
+        self._account_bytes(B, H, S, D, hi - lo if hi > lo else 0)
+        return k_all, v_all
 
-        # accounting (sink_cache.py:227-256): of the rows flushed now, the protected ones (the largest
-        # count over the batch) go to the fp16 pool, the rest are priced as plain KIVI rows
+    def _account_bytes(self, B: int, H: int, S: int, D: int, n_quant_now: int) -> None:
+        """sink_cache.py:227-256: of the rows flushed now, the protected ones (the largest count over
+        the batch) go to the fp16 pool, the rest are priced as plain KIVI rows."""
+        n_protected, self._flush_protected = min(self._flush_protected, max(n_quant_now, 0)), 0
         row_bytes = D * 2 * 2 * H * B
-        if hi - lo > n_protected:
-            k_bytes, v_bytes = self._quantized_bytes(hi - lo - n_protected, B, H, D)
+        if n_quant_now > n_protected:
+            k_bytes, v_bytes = self._quantized_bytes(n_quant_now - n_protected, B, H, D)
             self._key_bytes_compressed += k_bytes
             self._value_bytes_compressed += v_bytes
         self._sink_fp16_bytes += n_protected * row_bytes
@@ -144,24 +160,107 @@ class SinkProtectedKVCache(KIVIKVCache):
         self._key_bytes_fp16 += H * B * S * D * 2
         self._value_bytes_fp16 += H * B * S * D * 2
         self._tokens_seen += S
-        return k_all, v_all
+
+    # ------------------------------------------------------------------ packed modes
+    def _pack_block(self, k_blk: torch.Tensor, v_blk: torch.Tensor, lo: int) -> None:
+        B, H, n, D = k_blk.shape
+        protected = self._top.inside(lo, lo + n)[:B] if self._n_sink else None
+        if protected is None or not bool(protected.any()):
+            return super()._pack_block(k_blk, v_blk, lo)
+        self._flush_protected = int(protected.sum(dim=1).max())
+        dev = k_blk.device
+        take = _stand_in_index(protected).to(dev)[:, None, :, None].expand(B, H, n, D)
+        super()._pack_block(k_blk.gather(2, take), v_blk.gather(2, take), lo)
+        seqs, rows = protected.nonzero(as_tuple=True)
+        seqs_d, rows_d = seqs.to(dev), rows.to(dev)
+        # the stand-ins add nothing to the attention output: value scale and zero of their positions are zeros
+        if self._v_layout == "token":
+            self._vs[seqs_d, :, :, rows_d + lo] = 0
+            self._vz[seqs_d, :, :, rows_d + lo] = 0
+        else:
+            self._vs[seqs_d, :, rows_d + lo] = 0
+            self._vz[seqs_d, :, rows_d + lo] = 0
+        self._side_add(seqs.tolist(), [lo + r for r in rows.tolist()], k_blk[seqs_d, :, rows_d], v_blk[seqs_d, :, rows_d])
+
+    def _side_add(self, seqs: list, positions: list, k_rows: torch.Tensor, v_rows: torch.Tensor) -> None:
+        """Append exact rows ``[n, H, D]`` of (sequence, position) pairs to the side store."""
+        B, H, D = self._shape_bhd
+        while len(self._side_pos) < B:
+            self._side_pos.append([])
+        slots = []
+        for b, p in zip(seqs, positions):
+            slots.append(len(self._side_pos[b]))
+            self._side_pos[b].append(p)
+        need = max(len(ps) for ps in self._side_pos)
+        cap = 0 if self._side_k is None else self._side_k.shape[2]
+        if need > cap:
+            new_cap = max(8, 2 * cap, need)
+            side_k = torch.zeros((B, H, new_cap, D), dtype=k_rows.dtype, device=k_rows.device)
+            side_v = torch.zeros_like(side_k)
+            if cap:
+                side_k[:, :, :cap], side_v[:, :, :cap] = self._side_k, self._side_v
+            self._side_k, self._side_v = side_k, side_v
+        dev = k_rows.device
+        b_idx, s_idx = torch.tensor(seqs, device=dev), torch.tensor(slots, device=dev)
+        self._side_k[b_idx, :, s_idx] = k_rows
+        self._side_v[b_idx, :, s_idx] = v_rows
+        self._side_pos_dev = None
+
+    def _extra_attend_args(self) -> dict:
+        if self._side_k is None or not any(self._side_pos):
+            return {}
+        if self._side_pos_dev is None:
+            cap = self._side_k.shape[2]
+            table = [ps + [-1] * (cap - len(ps)) for ps in self._side_pos]
+            self._side_pos_dev = torch.tensor(table, dtype=torch.int32, device=self._side_k.device)
+        return {"sinks": (self._side_k, self._side_v, self._side_pos_dev)}
+
+    def _rollback_bytes(self, n_tokens: int, n_rolled: int) -> None:
+        # protected rows of the flushed stretch that is live again, counted as the flush counted them
+        back = (self._top.pos >= self._n_quantized) & (self._top.pos < self._frontier_before_trim)
+        n_back = min(int(back.sum(dim=1).max()) if back.numel() else 0, n_rolled)
+        B, H, D = self._shape_bhd
+        super()._rollback_bytes(n_tokens, n_rolled - n_back)
+        self._sink_fp16_bytes = max(0, self._sink_fp16_bytes - n_back * D * 2 * 2 * H * B)
 
     def trim(self, n: int) -> int:
-        """Drop the last ``n`` tokens; frontier, candidates and accounting roll back
+        """Drop the last ``n`` tokens; frontier, candidates, side store and accounting roll back
         (sink_cache.py:200-225).  Candidates that had lost their place earlier do not come back."""
-        frontier_before = self._n_quantized
-        trimmed = FP16KVCache.trim(self, n)
+        self._frontier_before_trim = self._n_quantized
+        trimmed = KIVIKVCache.trim(self, n)
         if not trimmed:
             return trimmed
-        n_rolled = self._rollback_frontier(self.offset)
-        # protected rows of the flushed region that is live again, counted as the flush counted them
-        back = (self._top.pos >= self._n_quantized) & (self._top.pos < frontier_before)
-        n_back = min(int(back.sum(dim=1).max()) if back.numel() else 0, n_rolled)
+        frontier = self._n_quantized
+        if self._side_k is not None and any(self._side_pos):
+            # rows of the side store at or past the new frontier: back into the fp16 rows they came
+            # from (the memory-bound tail was just rebuilt from the packed store, stand-ins and all)
+            for b, ps in enumerate(self._side_pos):
+                for slot, p in enumerate(ps):
+                    if frontier <= p < self.offset and self._memory_bound and self._tail_k is not None:
+                        self._tail_k[b, :, p - frontier] = self._side_k[b, :, slot]
+                        self._tail_v[b, :, p - frontier] = self._side_v[b, :, slot]
+            kept = [[(slot, p) for slot, p in enumerate(ps) if p < frontier] for ps in self._side_pos]
+            for b, pairs in enumerate(kept):
+                for new_slot, (slot, _) in enumerate(pairs):
+                    if new_slot != slot:
+                        self._side_k[b, :, new_slot] = self._side_k[b, :, slot]
+                        self._side_v[b, :, new_slot] = self._side_v[b, :, slot]
+            self._side_pos = [[p for _, p in pairs] for pairs in kept]
+            self._side_pos_dev = None
         self._top.drop_from(self.offset)
-        B, H, D = self._shape_bhd
-        self._rollback_bytes(trimmed, n_rolled - n_back)
-        self._sink_fp16_bytes = max(0, self._sink_fp16_bytes - n_back * D * 2 * 2 * H * B)
         return trimmed
+
+    @property
+    def state(self):
+        if self._fused_enabled:
+            raise NotImplementedError("SinkProtectedKVCache: saving a packed cache with protected rows is not supported")
+        return KIVIKVCache.state.fget(self)
+
+    @state.setter
+    def state(self, v) -> None:
+        if self._fused_enabled:
+            raise NotImplementedError("SinkProtectedKVCache: restoring a packed cache with protected rows is not supported")
+        KIVIKVCache.state.fset(self, v)
 
     # ------------------------------------------------------------------ reporting
     @property

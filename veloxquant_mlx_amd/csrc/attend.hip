@@ -121,6 +121,12 @@ static int validate(const vq_attend_args *a, const char *fn) {
     VQ_REQUIRE(a->n_packed + a->n_tail >= 1, VQ_ERR_INVALID, "%s: no key/value slots to attend to", fn);
     VQ_REQUIRE(a->fixed_order >= 0 && a->fixed_order <= 3, VQ_ERR_INVALID, "%s: fixed_order must be 0, 1, 2 or 3", fn);
     VQ_REQUIRE(a->sliding_window >= 0, VQ_ERR_INVALID, "%s: negative sliding window", fn);
+    if (a->sink_k != nullptr) {
+        VQ_REQUIRE(a->sink_v != nullptr && a->sink_pos != nullptr && a->sink_cap >= 1, VQ_ERR_INVALID,
+                   "%s: sink_k needs sink_v, sink_pos and sink_cap >= 1", fn);
+        VQ_REQUIRE(is_float_tag(a->sink_dtype), VQ_ERR_INVALID, "%s: unsupported sink dtype", fn);
+        VQ_REQUIRE(a->n_packed > 0, VQ_ERR_INVALID, "%s: protected rows stand for positions of the packed prefix", fn);
+    }
     VQ_REQUIRE(a->Sq <= a->n_packed + a->n_tail || !a->causal, VQ_ERR_INVALID,
                "%s: S_q=%lld exceeds S_kv=%lld; queries align to the tail of the KV cache", fn, (long long)a->Sq,
                (long long)(a->n_packed + a->n_tail));
@@ -193,10 +199,19 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
     size_t need = vq_kivi_attend_workspace(a);
     VQ_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, VQ_ERR_WORKSPACE,
                "%s: workspace of %zu bytes required, %zu given", fn, need, a->workspace_bytes);
+    // protected rows: the patch pass reads the partials and the original (unshifted) packed store
+    auto finish = [&]() -> int {
+        if (a_in->sink_k == nullptr) return VQ_OK;
+        vq_attend_args full = *a_in;
+        full.workspace = a->workspace;
+        launch_sink_patch(full, p.nparts);
+        VQ_HIP_CHECK_LAUNCH(fn);
+        return VQ_OK;
+    };
     if (p.path == 1) {
         const bool merged = launch_attend_mfma_decode(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
-        if (merged) return VQ_OK;
+        if (merged) return finish();
     } else if (p.path == 2) {
         launch_attend_mfma_prefill(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
@@ -205,6 +220,7 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         if (rc != VQ_OK) return rc;
         VQ_HIP_CHECK_LAUNCH(fn);
     }
+    if (a_in->sink_k != nullptr) return finish();   // the patch pass does the merge as well
     rc = launch_attend_merge(*a, p.nparts);
     VQ_HIP_CHECK_LAUNCH(fn);
     return rc;

@@ -96,6 +96,9 @@ AttendPlan plan_attend(const vq_attend_args &a);
 
 int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len);
 int launch_attend_merge(const vq_attend_args &a, int nparts);
+// protected rows (vq_attend_args.sink_k): rewrites every output row from the partials in the
+// workspace, with the stand-ins' weights taken out and the exact rows put in
+void launch_sink_patch(const vq_attend_args &a, int nparts);
 // merges partials [rows][nparts][D + 2] of (max, sum, accumulator) into out [rows][D]
 void launch_merge_rows(const float *ws, int64_t rows, int nparts, int64_t D, void *out, int out_dtype, hipStream_t st);
 

@@ -158,6 +158,100 @@ __global__ void attend_merge4_kernel(const float *__restrict__ ws, int64_t rows,
     }
 }
 
+// Protected rows: one wave per query row redoes the merge of the row's partials keeping the sums
+// apart, takes the weight of every visible stand-in out of the softmax sum (its values are stored
+// as zeros, so the numerators never saw it; its key is rebuilt from the packed store as
+// code * scale + zero), then folds the exact rows in with a running maximum and writes the row.
+__global__ __launch_bounds__(256) void attend_sink_patch_kernel(vq_attend_args a, int nparts, const float *__restrict__ ws) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int64_t rows = a.B * a.Hq * a.Sq;
+    if (row >= rows) return;
+    const int64_t iq = row % a.Sq, h = (row / a.Sq) % a.Hq, b = row / (a.Sq * a.Hq);
+    const int64_t hpk = a.Hq / a.Hkv, bh = b * a.Hkv + h / hpk;
+    take_sequence_lengths(a, b);
+    const int64_t D = a.D, n_total = a.n_packed + a.n_tail;
+    const int64_t last = a.causal ? (n_total - a.Sq + iq) : (n_total - 1);
+    const int64_t first = window_first(a, n_total, iq);
+    const int bits = a.pack_bits, per = 32 / bits, g = a.group;
+    const uint32_t mask = (1u << bits) - 1u;
+    const int64_t W = (D + per - 1) / per, GKcap = (a.cap_tokens + g - 1) / g;
+    const uint32_t *kp = (const uint32_t *)a.k_packed;
+
+    const float *rec = ws + row * nparts * (D + 2);
+    float gm = -INFINITY;
+    for (int s = 0; s < nparts; ++s) gm = fmaxf(gm, rec[(int64_t)s * (D + 2)]);
+    float qv[4], num[4] = {0.f, 0.f, 0.f, 0.f}, den = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t d = lane + 64 * j;
+        qv[j] = d < D ? ld_tag(a.q, a.q_dtype, row * D + d) : 0.0f;
+    }
+    for (int s = 0; s < nparts; ++s) {
+        const float *r = rec + (int64_t)s * (D + 2);
+        if (r[0] == -INFINITY) continue;
+        const float f = __expf(r[0] - gm);
+        den += r[1] * f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int64_t d = lane + 64 * j;
+            if (d < D) num[j] += r[2 + d] * f;
+        }
+    }
+    auto visible = [&](int64_t pos) { return pos >= 0 && pos < a.n_packed && pos <= last && pos >= first; };
+    if (gm != -INFINITY) {
+        for (int64_t j = 0; j < a.sink_cap; ++j) {
+            const int64_t t = a.sink_pos[b * a.sink_cap + j];
+            if (!visible(t)) continue;
+            float dot = 0.f;
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj) {
+                const int64_t d = lane + 64 * jj;
+                if (d >= D) continue;
+                const uint32_t kw = kp[(bh * a.cap_tokens + t) * W + d / per];
+                const float kc = (float)((kw >> ((d % per) * bits)) & mask);
+                const int64_t kmi = (bh * GKcap + t / g) * D + d;
+                dot += qv[jj] * __fadd_rn(__fmul_rn(kc, ld_tag(a.k_scale, a.meta_dtype, kmi)), ld_tag(a.k_zero, a.meta_dtype, kmi));
+            }
+            den -= __expf(wave_sum(dot) * a.scale - gm);
+        }
+        if (den < 0.f) den = 0.f;
+    }
+    for (int64_t j = 0; j < a.sink_cap; ++j) {
+        const int64_t t = a.sink_pos[b * a.sink_cap + j];
+        if (!visible(t)) continue;
+        float kh[4], vh[4], dot = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+            const int64_t d = lane + 64 * jj;
+            kh[jj] = vh[jj] = 0.f;
+            if (d >= D) continue;
+            const int64_t si = (bh * a.sink_cap + j) * D + d;
+            kh[jj] = ld_tag(a.sink_k, a.sink_dtype, si);
+            vh[jj] = ld_tag(a.sink_v, a.sink_dtype, si);
+            dot += qv[jj] * kh[jj];
+        }
+        const float sc = wave_sum(dot) * a.scale;
+        const float mn = fmaxf(gm, sc);
+        const float f = gm == -INFINITY ? 0.f : __expf(gm - mn), w = __expf(sc - mn);
+        den = den * f + w;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) num[jj] = num[jj] * f + w * vh[jj];
+        gm = mn;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int64_t d = lane + 64 * j;
+        if (d < D) st_tag(a.out, a.out_dtype, row * D + d, den > 0.f ? num[j] / den : 0.f);
+    }
+}
+
+void launch_sink_patch(const vq_attend_args &a, int nparts) {
+    const int64_t rows = a.B * a.Hq * a.Sq;
+    hipLaunchKernelGGL(attend_sink_patch_kernel, dim3((unsigned)cdiv(rows, 4)), dim3(256), 0, (hipStream_t)a.stream, a, nparts,
+                       (const float *)a.workspace);
+}
+
 static void launch_merge(const float *ws, int64_t rows, int nparts, int64_t D, void *out, int out_dtype, hipStream_t st) {
     const bool pairs = nparts <= 4 && D % 2 == 0 && ((uintptr_t)ws & 7u) == 0;
     int64_t g = cdiv(pairs ? rows * D / 2 : rows * D, 256);

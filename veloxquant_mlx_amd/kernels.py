@@ -702,6 +702,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
                        tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
                        v_new: torch.Tensor | None = None, fixed_order: bool | None = None,
                        out: torch.Tensor | None = None, static_scratch: bool = False, sliding_window: int = 0,
+                       sinks: tuple | None = None,
                        _plan_out: dict | None = None, _single_launch: bool = True) -> torch.Tensor:
     """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
 
@@ -714,7 +715,11 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     default set by :func:`attend_fixed_order`.  ``out`` receives the result when given (a
     contiguous ``[B,Hq,Sq,D]`` tensor).  ``static_scratch=True`` goes through
     ``vq_kivi_attend_static``: the library's built-in scratch instead of a torch workspace, for
-    callers that may not allocate (give ``out`` too; calls on one GPU must not overlap)."""
+    callers that may not allocate (give ``out`` too; calls on one GPU must not overlap).
+    ``sliding_window > 0``: a query sees only that many last slots up to its own position.
+    ``sinks=(sink_k, sink_v, sink_pos)``: exact rows ``[B,Hkv,cap,D]`` standing for the packed
+    positions ``sink_pos`` (int32 ``[B,cap]``, -1 for an unused slot) whose packed stand-ins carry
+    zero value scale / zero: the stand-ins' softmax weights are taken out and the exact rows put in."""
     name = "kivi_packed_attend"
     if q.ndim != 4:
         raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
@@ -778,6 +783,16 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
     a.sliding_window = int(sliding_window or 0)
+    if sinks is not None:
+        sk, sv, sp = sinks
+        cap_s = sk.shape[2]
+        if (sk.ndim != 4 or tuple(sv.shape) != tuple(sk.shape) or sk.shape[0] != B or sk.shape[3] != D or sv.dtype != sk.dtype
+                or tuple(sp.shape) != (B, cap_s) or sp.dtype != torch.int32
+                or not (sk.is_contiguous() and sv.is_contiguous() and sp.is_contiguous() and sk.is_cuda and sp.is_cuda)):
+            raise ValueError(f"{name}: sinks must be (k [B,Hkv,cap,D], v like k, positions int32 [B,cap]), contiguous, on the device")
+        a.sink_k, a.sink_v, a.sink_pos = sk.data_ptr(), sv.data_ptr(), sp.data_ptr()
+        a.sink_cap, a.sink_dtype = int(cap_s), _FLOAT_TAG[sk.dtype]
+        keep += [sk, sv, sp]
     a.fixed_order = 0 if fixed_order is None else (int(fixed_order) if fixed_order is not True and fixed_order is not False and int(fixed_order) > 2 else (1 if fixed_order else 2))
     if (packed_lens is None) != (tail_lens is None):
         raise ValueError(f"{name}: packed_lens and tail_lens go together")
