@@ -406,9 +406,21 @@ def test_mfma_path_takes_bf16_tails():
                                       (2, 32, torch.float32)])
 def test_mfma_prefill_lds_kernel_shapes(Hq, Hkv, b, g, meta):
     """64-row blocks over several units and token groups, ragged last tile, not-causal and causal."""
-    path = 2 if meta == torch.float16 else 1   # float32 scale / zero stays on the 8-row tiles
-    _packed_case(1, Hq, Hkv, 384, 45, 128, b, g, "token", meta, Sq=100, causal=True, seed=Hq + b + g, expect_path=path)
-    _packed_case(1, Hq, Hkv, 384, 0, 128, b, g, "token", meta, Sq=16, causal=False, seed=Hq + b + g + 1, expect_path=path)
+    # float32 scale / zero: the 256-row blocks take it, fewer rows stay on the 8-row tiles of the decode kernel
+    path = lambda Sq: 2 if meta == torch.float16 or (Hq // Hkv) * Sq >= 256 else 1
+    _packed_case(1, Hq, Hkv, 384, 45, 128, b, g, "token", meta, Sq=100, causal=True, seed=Hq + b + g, expect_path=path(100))
+    _packed_case(1, Hq, Hkv, 384, 0, 128, b, g, "token", meta, Sq=16, causal=False, seed=Hq + b + g + 1, expect_path=path(16))
+
+
+@pytest.mark.parametrize("b,g", [(4, 32), (2, 64), (4, 128)])
+def test_mfma_prefill_rows_kernel_with_float32_scale_and_zero(b, g):
+    """256-row prefill blocks with float32 scale / zero: the producer forms code * scale + zero in float32
+    (one rounding per operation) and rounds it to fp16 -- the reconstruction a cache that stores fp16
+    holds -- where the fp16 form uses one fused step; causal edge inside the packed prefix, bf16 tail."""
+    _packed_case(1, 32, 8, 1024, 150, 128, b, g, "token", torch.float32, Sq=128, causal=True, seed=b * g, expect_path=2)
+    _packed_case(2, 8, 1, 512, 0, 128, b, g, "token", torch.float32, Sq=64, causal=True, seed=b * g + 1, expect_path=2)
+    _packed_case(1, 16, 4, 640, 90, 128, b, g, "token", torch.float32, Sq=80, causal=False, seed=b * g + 2, expect_path=2,
+                 tail_dtype=torch.bfloat16)
 
 
 # ------------------------------------------------- sequences of different lengths in one batch

@@ -436,11 +436,13 @@ def test_chunked_prefill_with_no_residual_window(chunk, g):
         refs.append(oa.kivi_attend(q[:, :, s0:s1], kc_[:, :, :nq], ks_[:, :, : nq // g], kz_[:, :, : nq // g], vc_[:, :, :nq],
                                    vs_[:, :, :nq], vz_[:, :, :nq], g, k[:, :, nq:s1], v[:, :, nq:s1], 1 / math.sqrt(D), causal=True))
     got = np.concatenate(outs, axis=2).astype(np.float32)
-    # float32 scale / zero: the kernels attend over code * scale + zero itself
-    assert np.max(np.abs(got - np.concatenate(refs, axis=2))) < 2e-3
-    # the cache model holds that reconstruction rounded to fp16 (kivi_cache.py:198-201); with every
-    # token quantised the rounding shows, inside the 1e-2 bar of the reference's own fused-attention tests
-    assert np.max(np.abs(got - oa.chunked_prefill(q, k, v, chunk, 4, g, 0, 1 / math.sqrt(D)))) < 1e-2
+    # every chunk here has 256 query rows or more per kv head and runs on the 256-row prefill blocks,
+    # which attend over the reconstruction rounded to fp16: what the cache model holds
+    # (kivi_cache.py:198-201) and the oracle at the usual bar.  With every token quantised that
+    # rounding shows against code * scale + zero itself, inside the 1e-2 bar of the reference's own
+    # fused-attention tests.
+    assert np.max(np.abs(got - oa.chunked_prefill(q, k, v, chunk, 4, g, 0, 1 / math.sqrt(D)))) < 2e-3
+    assert np.max(np.abs(got - np.concatenate(refs, axis=2))) < 1e-2
 
 
 def test_bf16_history_holds_the_reconstruction_rounded_to_bf16():
@@ -840,3 +842,23 @@ def test_layer_stacked_cache_attends_for_all_layers_at_once():
     check()
     with pytest.raises(ValueError, match="NL=3"):
         stacked.fused_sdpa_all(rnd(2, B, Hq, 1, D), scale)
+
+
+def test_context_limit_error_leaves_the_cache_as_it_was():
+    """An append whose flush would pass ``fused_sdpa_max_ctx`` raises before offset, rows or packed
+    store change: the cache answers the same query with the same bits afterwards."""
+    require_gpu()
+    B, Hq, Hkv, D = 1, 8, 2, 128
+    k, v = outlier_kv((B, Hkv, 600, D), seed=71)
+    c = _make(bit_width_inlier=4, kivi_group_size=32, residual_length=64, fused_sdpa=True, fused_sdpa_memory_bound=True,
+              fused_sdpa_max_ctx=256)
+    c.update_and_fetch(to_dev(k[:, :, :300]), to_dev(v[:, :, :300]))
+    q = to_dev(np.random.default_rng(72).standard_normal((B, Hq, 1, D)).astype(np.float16))
+    before = c.fused_sdpa(q, 0.09, fixed_order=True)
+    state = (c.offset, c._n_quantized, c.nbytes)
+    with pytest.raises(RuntimeError, match="fused_sdpa_max_ctx"):
+        c.update_and_fetch(to_dev(k[:, :, 300:600]), to_dev(v[:, :, 300:600]))
+    assert (c.offset, c._n_quantized, c.nbytes) == state
+    assert torch.equal(c.fused_sdpa(q, 0.09, fixed_order=True), before)
+    c.update_and_fetch(to_dev(k[:, :, 300:310]), to_dev(v[:, :, 300:310]))      # a step that still fits goes through
+    assert c.offset == 310

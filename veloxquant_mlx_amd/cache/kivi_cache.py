@@ -227,7 +227,9 @@ class KIVIKVCache(FP16KVCache):
                 and values.data_ptr() % 16 == 0
                 and (max(0, self.offset + 1 - self._residual_length) // self._group_size) * self._group_size
                 == self._n_quantized):
-            # a plain decode step with no flush due: the attention launch of this step stores the token
+            # a plain decode step with no flush due: the attention launch of this step stores the token.
+            # Until then the cache holds the caller's tensors, not a copy: a caller that reuses its key /
+            # value buffers between update_and_fetch and fused_sdpa must pass clones.
             self._pending = (keys, values)
             self.offset += 1
             self._account_bytes(B, H, S, D, 0)
@@ -235,6 +237,11 @@ class KIVIKVCache(FP16KVCache):
             if z is None or z.dtype != keys.dtype or z.device != keys.device:
                 z = self._zero_scalar = torch.zeros((), dtype=keys.dtype, device=keys.device)
             return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
+        # a flush that would pass fused_sdpa_max_ctx is refused here, before offset or rows change
+        new_boundary = (max(0, self.offset + S - self._residual_length) // self._group_size) * self._group_size
+        n_quant_now = new_boundary - self._n_quantized
+        if n_quant_now > 0:
+            self._ensure_packed_capacity(B, H, D, new_boundary, keys.device)
         if self._tail_k is None or need > self._tail_k.shape[2]:
             cap = max(need, self._residual_length + 2 * self._group_size)
             cap = -(-cap // 64) * 64
@@ -251,11 +258,8 @@ class KIVIKVCache(FP16KVCache):
             self._tail_k[:, :, n_tail:need] = keys
             self._tail_v[:, :, n_tail:need] = values
         self.offset += S
-        new_boundary = self._quantization_boundary()
-        n_quant_now = new_boundary - self._n_quantized
         spare = None
         if n_quant_now > 0:
-            self._ensure_packed_capacity(B, H, D, new_boundary, keys.device)
             keep = need - n_quant_now
             # the rows that stay move to the front of a second buffer (one copy each, no
             # temporaries); a very large prefill chunk leaves an oversized buffer behind, which is

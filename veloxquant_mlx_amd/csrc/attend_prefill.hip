@@ -453,13 +453,41 @@ void attend_prefill_kernel(vq_attend_args a, int qp, int nparts, float *__restri
 constexpr int PR_RB = 2;          // 16-row blocks per wave
 constexpr int PR_THREADS = 512;
 
-template <int BITS> struct PrStage {
+// eight scale or zero values of the storage type M as raw 16-byte pieces
+template <typename M> struct Meta8 {
+    static constexpr int N = (int)sizeof(M) / 2;   // pieces: 1 for fp16, 2 for float32
+    uint4 u[N];
+    __device__ __forceinline__ void load(const void *p) {
+#pragma unroll
+        for (int i = 0; i < N; ++i) u[i] = reinterpret_cast<const uint4 *>(p)[i];
+    }
+};
+// c * s + z for eight exact fp16 codes: formed exactly and rounded once with fp16 scale / zero; in
+// float32 with one rounding per operation and then rounded to fp16 with float32 scale / zero --
+// in both cases what a cache that stores the reconstruction in fp16 holds
+// (veloxquant_mlx/cache/kivi_cache.py:198-201)
+__device__ __forceinline__ f16x8 recon8(f16x8 c, const Meta8<f16> &s, const Meta8<f16> &z) {
+    return __builtin_elementwise_fma(c, as_h8(s.u[0]), as_h8(z.u[0]));
+}
+__device__ __forceinline__ f16x8 recon8(f16x8 c, const Meta8<float> &s, const Meta8<float> &z) {
+    const float sf[8] = {__uint_as_float(s.u[0].x), __uint_as_float(s.u[0].y), __uint_as_float(s.u[0].z), __uint_as_float(s.u[0].w),
+                         __uint_as_float(s.u[1].x), __uint_as_float(s.u[1].y), __uint_as_float(s.u[1].z), __uint_as_float(s.u[1].w)};
+    const float zf[8] = {__uint_as_float(z.u[0].x), __uint_as_float(z.u[0].y), __uint_as_float(z.u[0].z), __uint_as_float(z.u[0].w),
+                         __uint_as_float(z.u[1].x), __uint_as_float(z.u[1].y), __uint_as_float(z.u[1].z), __uint_as_float(z.u[1].w)};
+    f16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (f16)__fadd_rn(__fmul_rn((float)c[e], sf[e]), zf[e]);
+    return o;
+}
+
+template <int BITS, typename M> struct PrStage {
     u32 kw;          // key word: the thread's 8 channels of one token (2-bit: the word holding them)
     u32 vw;          // value word: the thread's 8 tokens of one channel (2-bit: the word holding them)
-    uint4 vs, vz;    // value scale / zero of those 8 tokens (the thread's channel group)
+    Meta8<M> vs, vz; // value scale / zero of those 8 tokens (the thread's channel group); a tail unit's
+                     // raw key and value pieces travel in the first piece of each
 };
 
-template <int BITS, int GV>
+template <int BITS, int GV, typename M>
 __global__ __launch_bounds__(PR_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__restrict__ ws) {
     __shared__ __align__(16) f16 s_k[3][32 * PF_KSTRIDE];
@@ -534,37 +562,37 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     // ---- producer side
     const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
     const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
-    const f16 *ksb = (const f16 *)a.k_scale + bh * (cap >> gshift) * MF_D;
-    const f16 *kzb = (const f16 *)a.k_zero + bh * (cap >> gshift) * MF_D;
-    const f16 *vsb = (const f16 *)a.v_scale + bh * GV * cap;
-    const f16 *vzb = (const f16 *)a.v_zero + bh * GV * cap;
+    const M *ksb = (const M *)a.k_scale + bh * (cap >> gshift) * MF_D;
+    const M *kzb = (const M *)a.k_zero + bh * (cap >> gshift) * MF_D;
+    const M *vsb = (const M *)a.v_scale + bh * GV * cap;
+    const M *vzb = (const M *)a.v_zero + bh * GV * cap;
     const int kt = tid >> 4, kc = tid & 15;       // key tile: token, 8-channel chunk
     const int vc = tid & 127, vq = tid >> 7;      // value tile: channel, 8-token quarter
     const int vg = vc >> gshift;                  // channel group of the thread's value channel
     // byte offsets of the thread's key word, value word and value scale / zero piece inside a unit
     const unsigned k_off = (unsigned)((kt * KW + (BITS == 4 ? kc : kc >> 1)) * 4);
     const unsigned v_off = (unsigned)(((BITS == 4 ? vq : vq >> 1) * MF_D + vc) * 4);
-    const unsigned m_off = (unsigned)(((int64_t)vg * cap + 8 * vq) * 2);
+    const unsigned m_off = (unsigned)(((int64_t)vg * cap + 8 * vq) * sizeof(M));
     const int tp = lane & 15, cq = 4 * wave + (lane >> 4);   // tail values: token pair, channel quad
     const bool tail_bf16 = a.tail_dtype == VQ_BF16;
     const int64_t tbase = bh * a.tail_cap * MF_D;
     const f16x8 off8 = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair);
-    using Stage = PrStage<BITS>;
-    f16x8 ksr, kzr;   // key scale / zero of the thread's 8 channels in the token group last fetched
+    using Stage = PrStage<BITS, M>;
+    Meta8<M> ksr, kzr;   // key scale / zero of the thread's 8 channels in the token group last fetched
     int meta_group = -1;
     auto fetch = [&](int w, Stage &st) {
         if (w >= n_punits) {   // tail unit: the thread's key and value pieces travel in the value-meta slots
             const int64_t t0 = (int64_t)(w - n_punits) * 32;
             int64_t tok = t0 + kt;
             if (tok >= a.n_tail) tok = 0;   // masked in the softmax
-            st.vs = *reinterpret_cast<const uint4 *>((const u16 *)a.k_tail + tbase + tok * MF_D + 8 * kc);
+            st.vs.u[0] = *reinterpret_cast<const uint4 *>((const u16 *)a.k_tail + tbase + tok * MF_D + 8 * kc);
             // values: four channels of a token pair, so that the transposed tile is written in whole words
             int64_t ta = t0 + 2 * tp, tb = ta + 1;
             if (ta >= a.n_tail) ta = 0;
             if (tb >= a.n_tail) tb = 0;
             const uint2 va = *reinterpret_cast<const uint2 *>((const u16 *)a.v_tail + tbase + ta * MF_D + 4 * cq);
             const uint2 vb2 = *reinterpret_cast<const uint2 *>((const u16 *)a.v_tail + tbase + tb * MF_D + 4 * cq);
-            st.vz = make_uint4(va.x, va.y, vb2.x, vb2.y);
+            st.vz.u[0] = make_uint4(va.x, va.y, vb2.x, vb2.y);
             return;
         }
         // a block-uniform base that moves with the unit plus a 32-bit offset of the thread's own: the
@@ -572,13 +600,13 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         const int64_t base = (int64_t)w * 32;
         st.kw = *reinterpret_cast<const u32 *>(kb + base * (KW * 4) + k_off);
         st.vw = *reinterpret_cast<const u32 *>(vb + (base / PER) * (MF_D * 4) + v_off);
-        st.vs = *reinterpret_cast<const uint4 *>((const char *)vsb + base * 2 + m_off);
-        st.vz = *reinterpret_cast<const uint4 *>((const char *)vzb + base * 2 + m_off);
+        st.vs.load((const char *)vsb + base * sizeof(M) + m_off);
+        st.vz.load((const char *)vzb + base * sizeof(M) + m_off);
         const int grp = (int)(base >> gshift);
         if (grp != meta_group) {   // block-uniform
             meta_group = grp;
-            ksr = *reinterpret_cast<const f16x8 *>((const char *)ksb + (int64_t)grp * (MF_D * 2) + 16u * (unsigned)kc);
-            kzr = *reinterpret_cast<const f16x8 *>((const char *)kzb + (int64_t)grp * (MF_D * 2) + 16u * (unsigned)kc);
+            ksr.load((const char *)ksb + (int64_t)grp * (MF_D * sizeof(M)) + 8u * (unsigned)sizeof(M) * (unsigned)kc);
+            kzr.load((const char *)kzb + (int64_t)grp * (MF_D * sizeof(M)) + 8u * (unsigned)sizeof(M) * (unsigned)kc);
         }
     };
     // the thread's eight codes of a word, in order, as exact fp16 numbers
@@ -595,16 +623,14 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     auto unpack_to_lds = [&](int w, const Stage &st, int buf) {
         if (w < n_punits) {
             // keys: 8 channels of token kt; c s + z is formed exactly and rounded once
-            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) =
-                __builtin_elementwise_fma(codes8(st.kw, kc & 1), ksr, kzr);
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = recon8(codes8(st.kw, kc & 1), ksr, kzr);
             // values: 8 tokens of channel vc
-            *reinterpret_cast<f16x8 *>(&s_v[buf][vc * PF_VSTRIDE + 8 * vq]) =
-                __builtin_elementwise_fma(codes8(st.vw, vq & 1), as_h8(st.vs), as_h8(st.vz));
+            *reinterpret_cast<f16x8 *>(&s_v[buf][vc * PF_VSTRIDE + 8 * vq]) = recon8(codes8(st.vw, vq & 1), st.vs, st.vz);
         } else {
             // tail unit: plain key row chunk; values transposed, one word (a token pair of one channel)
             // at a time: the lanes of a wave cover 16 token pairs x 4 channel quads = 64 different banks
-            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = tail8_from_raw(st.vs, tail_bf16);
-            const f16x8 v0 = tail8_from_raw(st.vz, tail_bf16);   // channels 0..3 of the first token, then of the second
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = tail8_from_raw(st.vs.u[0], tail_bf16);
+            const f16x8 v0 = tail8_from_raw(st.vz.u[0], tail_bf16);   // channels 0..3 of the first token, then of the second
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 *reinterpret_cast<f16x2 *>(&s_v[buf][(4 * cq + e) * PF_VSTRIDE + 2 * tp]) = f16x2{v0[e], v0[4 + e]};
@@ -777,7 +803,9 @@ bool mfma_prefill_supported(const vq_attend_args &a) {
     if (a.n_packed > 0) {
         if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
         if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
-        if (a.meta_dtype != VQ_F16) return false;   // float32 scale / zero stays on the 8-row tiles of the decode kernel
+        // float32 scale / zero: the 256-row blocks take it (they reconstruct in the producer); fewer rows stay on
+        // the 8-row tiles of the decode kernel
+        if (a.meta_dtype != VQ_F16 && !(a.meta_dtype == VQ_F32 && (a.Hq / a.Hkv) * a.Sq >= 256)) return false;
         if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
         if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
         if (a.cap_tokens > ((int64_t)1 << 28)) return false;   // 32-bit byte offsets inside one (sequence, kv head) slab
@@ -811,8 +839,10 @@ void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     const dim3 grid((unsigned)tiles, (unsigned)(a.B * a.Hkv), (unsigned)p.nsplit), block(256);
 #define VQ_LAUNCH(BITS, GV)                                                                                          \
     do {                                                                                                             \
-        if (rows == 256)                                                                                             \
-            hipLaunchKernelGGL((attend_prefill_rows_kernel<BITS, GV>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \
+        if (rows == 256 && a.n_packed > 0 && a.meta_dtype == VQ_F32)                                                 \
+            hipLaunchKernelGGL((attend_prefill_rows_kernel<BITS, GV, float>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \
+        else if (rows == 256)                                                                                        \
+            hipLaunchKernelGGL((attend_prefill_rows_kernel<BITS, GV, f16>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \
         else                                                                                                         \
             hipLaunchKernelGGL((attend_prefill_kernel<BITS, GV>), grid, block, 0, st, a, qp, p.nparts, ws);           \
     } while (0)
