@@ -606,8 +606,10 @@ def _kernel_source_sha():
     import hashlib
     h = hashlib.sha256()
     d = os.path.join(ROOT, "veloxquant_mlx_amd", "csrc")
+    # the sources of the decode launch the traffic figure belongs to (the prefill and vector kernels may change freely)
+    decode_sources = ("attend.hip", "attend.hpp", "attend_mfma.hip", "attend_mfma.hpp", "attend_mfma_packed.hpp")
     for name in sorted(os.listdir(d)):
-        if name.startswith("attend") and name.endswith((".hip", ".hpp")):
+        if name in decode_sources or (name.startswith("attend_mfma_packed_") and name.endswith(".hip")):
             with open(os.path.join(d, name), "rb") as f:
                 h.update(name.encode())
                 h.update(f.read())
