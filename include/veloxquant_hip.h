@@ -64,6 +64,29 @@ int vq_device_count(void);
 int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D,
                           int axis, int group, int levels, float eps, void *stream);
 
+/* out[r] = L2 norm of row r of x [n_rows, D], float32 arithmetic (head_dim 64 / 128 / 256).  The salience
+ * signal of ZipCacheKVCache (mx.linalg.norm over the channels of the float32 copy,
+ * veloxquant_mlx/cache/zipcache_cache.py:176-180) without materialising that copy. */
+int vq_row_norms(const void *x, int dtype, int64_t n_rows, int64_t D, float *out, void *stream);
+
+/* Routing order of a salience split: order[bh] = the positions of the S - n_hi rows outside the n_hi largest
+ * norms[bh] (non-negative float32, [BH, S]) in ascending order, then the positions of the n_hi largest in
+ * ascending order; of rows with equal norms at the threshold the later ones are taken first.  Replaces
+ * ZipCacheKVCache._batched_saliency_mask followed by the stable argsort of its mask
+ * (veloxquant_mlx/cache/zipcache_cache.py:106-116, 186-190): two stable argsorts and a third over [BH, S]. */
+int vq_zip_route(const float *norms, int64_t BH, int64_t S, int64_t n_hi, int32_t *order, void *stream);
+
+/* The round trip along the token axis over ROUTED rows: position s of slab bh stands for row
+ * rows[bh * rows_stride + s] of x and of out (both [BH, *, D] with element stride stride_bh between slabs);
+ * groups of `group` consecutive positions are quantised together and every reconstructed row is written
+ * where its source row lies; rows that no position names are left alone.  Replaces, in one launch and
+ * without the gathered copy, the gather -> _group_quant_dequant_batched -> scatter of one salience block
+ * of ZipCacheKVCache._compress_tensor (veloxquant_mlx/cache/zipcache_cache.py:118-244): the caller passes
+ * the low or the high block's slice of its routing order.  head_dim 64 / 128 / 256. */
+int vq_kivi_quant_dequant_rows(const void *x, void *out, int dtype, int64_t BH, int64_t n_rows, int64_t D,
+                               int64_t stride_bh, const int32_t *rows, int64_t rows_stride, int group,
+                               int levels, float eps, void *stream);
+
 /* Quantise and bit-pack.  Codes follow _quant_keys/_quant_values
  * (benchmark_scripts/benchmark_real_model_scalar_attend.py:115-153;
  * veloxquant_mlx/quantizers/_quant_utils.py:9-46) and the word image follows

@@ -8,6 +8,7 @@ import torch
 from oracle import zipcache as oz
 from tests._gpu import gpu, host, require_gpu, to_dev
 from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+from veloxquant_mlx_amd import kernels as K
 from veloxquant_mlx_amd.cache.zipcache_cache import ZipCacheKVCache
 
 pytestmark = gpu
@@ -86,3 +87,35 @@ def test_validation():
             _make(**bad)
     with pytest.raises(ValueError, match=r"\[B, H, S, D\]"):
         _make()._compress(torch.zeros((2, 4, 8), device="cuda:0"), True)
+
+
+def test_row_norms_kernel_matches_float64():
+    """``vq_row_norms``: float32 norms of fp16 / bf16 / float32 rows at the three head sizes, within float32
+    rounding of the float64 value (the routing only needs their order; exact ties are broken by position)."""
+    require_gpu()
+    rng = np.random.default_rng(3)
+    for D in (64, 128, 256):
+        for dt in (torch.float16, torch.bfloat16, torch.float32):
+            x = to_dev(rng.standard_normal((3, 5, 77, D)).astype(np.float32) * 4, dt)
+            got = host(K.row_norms(x))
+            want = np.sqrt((host(x).astype(np.float64) ** 2).sum(-1))
+            assert got.shape == (3, 5, 77) and np.max(np.abs(got - want) / want) < 1e-6
+
+
+def test_routing_kernel_equals_the_stable_sorts():
+    """``vq_zip_route`` against the reference's definition (two stable argsorts for the mask, a third for the order,
+    zipcache_cache.py:106-116, 186-190): norms with many exact ties, zeros, one NaN, lengths that do not divide the
+    block, every block size from 1 to S - 1 at the small lengths."""
+    require_gpu()
+    g = torch.Generator().manual_seed(4)
+    for S in (2, 7, 255, 256, 257, 1000, 8192):
+        norms = torch.randint(0, 9, (5, S), generator=g).float() * 0.37
+        norms[1] = torch.rand(S, generator=g)
+        if S > 10:
+            norms[2, 5] = float("nan")
+        for n_hi in (range(1, S) if S <= 7 else (1, 2, S // 5, S // 2, S - 1)):
+            clean = torch.nan_to_num(norms, nan=float("inf"))       # the sorts put a NaN last, the bit order above inf
+            rank = torch.argsort(torch.argsort(clean, dim=-1, stable=True), dim=-1, stable=True)
+            want = torch.argsort((rank >= S - n_hi).to(torch.int32), dim=-1, stable=True)
+            got = K.zip_route(norms.to("cuda:0"), n_hi).cpu().long()
+            assert torch.equal(got, want), (S, n_hi)

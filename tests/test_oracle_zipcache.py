@@ -49,3 +49,20 @@ def test_bytes_by_hand_and_orderings():
     assert stored == (416 + 256 + 816 + 512 + 64) * 2 and base == (64 * 64 * 2 // 8 + 2 * 256) * 2 and fp16 == 2 * 64 * 64 * 2
     assert base <= stored < fp16 and 2.0 <= 16.0 * stored / fp16 <= 4.0 + 1.0
     assert oz.base_only_bytes(10, 64, 2, 32) == 160 + 256
+
+
+def test_sort_free_routing_equals_the_stable_sorts():
+    """The cache's routing helpers (threshold + prefix sums) against the reference's definition by stable argsorts
+    (zipcache_cache.py:106-116, 186-190), on norms with many ties and every block size."""
+    import torch
+    from veloxquant_mlx_amd.cache.zipcache_cache import ZipCacheKVCache as Z
+    torch.manual_seed(0)
+    for S in (1, 5, 64, 257):
+        for n_hi in range(0, S + 1, max(1, S // 7)):
+            norms = torch.randint(0, 6, (9, S)).float()
+            rank = torch.argsort(torch.argsort(norms, dim=-1, stable=True), dim=-1, stable=True)
+            want = rank >= (S - n_hi)
+            got = Z._batched_saliency_mask(norms, n_hi, S)
+            assert torch.equal(got, want), (S, n_hi)
+            if 0 < n_hi < S:
+                assert torch.equal(Z._routing_order(got, n_hi).long(), torch.argsort(got.to(torch.int32), dim=-1, stable=True))

@@ -84,6 +84,9 @@ _SIGNATURES = {
     "vq_kivi_quant_dequant": (i32, [vp, vp, i32, i64, i64, i64, i32, i32, i32, f32, vp]),
     "vq_skvq_clipped_roundtrip": (i32, [vp, vp, i32, i64, i64, i64, i64, i64, i64, vp, vp, i32, i32, C.POINTER(f32), i32, vp]),
     "vq_kivi_quant_pack": (i32, [vp, i32, i64, i64, i64, i64, i32, i32, i32, f32, i32, i32, vp, vp, vp, i32, i64, i64, vp]),
+    "vq_zip_route": (i32, [vp, i64, i64, i64, vp, vp]),
+    "vq_row_norms": (i32, [vp, i32, i64, i64, vp, vp]),
+    "vq_kivi_quant_dequant_rows": (i32, [vp, vp, i32, i64, i64, i64, i64, vp, i64, i32, i32, f32, vp]),
     "vq_kivi_quant_pack_kv": (i32, [vp, vp, i32, i64, i64, i64, i64, i32, i32, f32, i32, i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, vp]),
     "vq_kivi_dequant": (i32, [vp, vp, vp, i32, i64, i64, i64, i32, i32, i32, i32, i64, i64, vp, i32, vp]),
     "vq_kv_tail_append": (i32, [vp, vp, C.POINTER(i64), C.POINTER(i64), vp, vp, i32, i64, i64, i64, i64, i64, i64, vp]),

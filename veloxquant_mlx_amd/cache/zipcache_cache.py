@@ -75,9 +75,21 @@ class ZipCacheKVCache(FP16KVCache):
             return torch.zeros((BH, S), dtype=torch.bool, device=norms.device)
         if n_hi >= S:
             return torch.ones((BH, S), dtype=torch.bool, device=norms.device)
-        order = torch.argsort(norms, dim=-1, stable=True)
-        rank = torch.argsort(order, dim=-1, stable=True)
-        return rank >= (S - n_hi)
+        # the reference ranks by two stable argsorts; the same set without a sort: rank by (norm, position) as one
+        # integer key -- the bits of a non-negative float order like the float, the position breaks ties in favour of
+        # later rows -- and keep what reaches the n_hi-th largest key
+        key = (norms.contiguous().view(torch.int32).to(torch.int64) << 32) | torch.arange(S, device=norms.device)
+        kth = torch.kthvalue(key, S - n_hi + 1, dim=-1, keepdim=True).values
+        return key >= kth
+
+    @staticmethod
+    def _routing_order(mask: torch.Tensor, n_hi: int) -> torch.Tensor:
+        """int32 ``[BH, S]``: the rows outside ``mask`` in their own order, then the ``n_hi`` rows inside it in theirs
+        (what a stable argsort of the mask gives, zipcache_cache.py:186-190).  Every row of the mask holds exactly
+        ``n_hi`` set entries, so a flat selection of the positions falls apart into equal pieces per row."""
+        BH, S = mask.shape
+        pos = torch.arange(S, dtype=torch.int32, device=mask.device).expand(BH, S)
+        return torch.cat([pos[~mask].view(BH, S - n_hi), pos[mask].view(BH, n_hi)], dim=1)
 
     def _compress(self, t: torch.Tensor, is_key: bool, out_dtype: torch.dtype = torch.float16):
         """``[B,H,S,D]`` -> (reconstruction, row norms ``[BH,S]``, (stored, baseline, fp16) bytes); no state touched
@@ -89,10 +101,28 @@ class ZipCacheKVCache(FP16KVCache):
         lo_bits = self._lo_bits if is_key else self._hi_bits
         hi_fraction = self._hi_fraction if is_key else 1.0
         gs, BH = self._gs, B * H
-        x32 = t.reshape(BH, S, D).float()
-        norms = torch.linalg.vector_norm(x32, dim=-1)
+        rows3 = t.reshape(BH, S, D)
         n_hi = max(0, min(S, int(math.ceil(S * hi_fraction))))
         n_lo = S - n_hi
+        direct = (out_dtype == t.dtype and t.dtype in (torch.float16, torch.bfloat16, torch.float32) and D in (64, 128, 256)
+                  and gs <= 8 * (256 // (D // 8)) and BH <= 65535 and rows3.is_contiguous() and rows3.data_ptr() % 16 == 0)
+        if direct:
+            # float32 arithmetic on the stored rows themselves: the kernels widen every element on load and round
+            # the reconstruction once on store, which is what a float32 copy, round trip and cast give
+            norms = K.row_norms(rows3)
+            if n_lo == 0 or n_hi == 0:
+                out = K.kivi_group_quant_dequant(rows3, -2, gs, (1 << (hi_bits if n_hi else lo_bits)) - 1)
+            else:
+                order = K.zip_route(norms, n_hi)   # low block, then high block
+                out = torch.empty_like(rows3)
+                K.kivi_group_quant_dequant_rows(rows3, out, order, 0, n_lo, gs, (1 << lo_bits) - 1)
+                K.kivi_group_quant_dequant_rows(rows3, out, order, n_lo, n_hi, gs, (1 << hi_bits) - 1)
+            per_slab = (math.ceil(n_hi * D * hi_bits / 8) + math.ceil(n_lo * D * lo_bits / 8)
+                        + (math.ceil(n_hi / gs) if n_hi else 0) * D * 4 + (math.ceil(n_lo / gs) if n_lo else 0) * D * 4 + S)
+            bytes_ = (per_slab * BH, base_only_bytes(S, D, self._lo_bits, gs) * BH, B * H * S * D * 2)
+            return out.reshape(B, H, S, D), norms, bytes_
+        x32 = rows3.float()
+        norms = torch.linalg.vector_norm(x32, dim=-1)
         if n_lo == 0 or n_hi == 0:   # one block in original order: no gather needed
             out = K.kivi_group_quant_dequant(x32, -2, gs, (1 << (hi_bits if n_hi else lo_bits)) - 1)
         else:

@@ -238,9 +238,12 @@ template <typename T, typename M, int LPR, int MODE, int NP>
 __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
     const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
     float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
-    int64_t cap_tokens, int64_t dst_tok0, int W) {
+    int64_t cap_tokens, int64_t dst_tok0, int W, const int32_t *__restrict__ rows = nullptr, int64_t rows_stride = 0) {
     constexpr int D = LPR * 8;
     constexpr int RPP = 256 / LPR;
+    // `rows` (MODE 0 only): position s of the (b, h) slab stands for row rows[bh * rows_stride + s] of x and of
+    // out -- groups are formed over the routed order, rows are read and written where they lie
+    auto routed = [&](int64_t s) -> int64_t { return rows != nullptr ? (int64_t)rows[bh * rows_stride + s] : s; };
     // per-row-slot minima / maxima, then the group's (zero, scale, 1 / scale) per channel
     __shared__ __align__(16) float s_mn[RPP][D];
     __shared__ __align__(16) float s_mx[RPP][D];
@@ -258,7 +261,7 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
         if (rl < group && s < S) {
-            v[p].load(xb + s * D + 8 * o);
+            v[p].load(xb + routed(s) * D + 8 * o);
             v[p].fold(acc);
         }
     }
@@ -317,7 +320,7 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
                 float y[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) y[i] = recon(q[i], sc[i], mn[i]);
-                store8<T>(out + (bh * S + s) * D + 8 * o, y);
+                store8<T>(rows != nullptr ? out + bh * x_stride_bh + routed(s) * D + 8 * o : out + (bh * S + s) * D + 8 * o, y);
             }
         } else {
             uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;
@@ -330,9 +333,9 @@ template <typename T, typename M, int LPR, int MODE, int NP>
 __global__ __launch_bounds__(256) void kivi_key_tile_kernel(
     const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, int group, float levels,
     float eps, int bits, uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
-    int64_t cap_tokens, int64_t dst_tok0, int W) {
+    int64_t cap_tokens, int64_t dst_tok0, int W, const int32_t *__restrict__ rows, int64_t rows_stride) {
     kivi_key_tile_body<T, M, LPR, MODE, NP>((int)blockIdx.x, (int64_t)blockIdx.y, x, out, S, x_stride_bh, group, levels, eps,
-                                            bits, packed, scale, zero, cap_tokens, dst_tok0, W);
+                                            bits, packed, scale, zero, cap_tokens, dst_tok0, W, rows, rows_stride);
 }
 
 // ---------------------------------------------------------------------------
@@ -641,6 +644,98 @@ static inline int grid_for(int64_t n, int block) {
     if (g > 65536 * 16) g = 65536 * 16;
     return (int)g;
 }
+// L2 norm of every row of x [n_rows, D] in float32: LPR = D / 8 lanes per row, 16-byte loads, the squares
+// summed per lane and then across the row's lanes.
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void row_norm_kernel(const T *__restrict__ x, int64_t n_rows, float *__restrict__ out) {
+    constexpr int D = LPR * 8, RPB = 256 / LPR;
+    const int tid = threadIdx.x, r = tid / LPR, o = tid % LPR;
+    for (int64_t row = (int64_t)blockIdx.x * RPB + r; row < n_rows; row += (int64_t)gridDim.x * RPB) {
+        float v[8];
+        load8<T>(x + row * D + 8 * o, v);
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = __builtin_fmaf(v[i], v[i], acc);
+#pragma unroll
+        for (int off = 1; off < LPR; off <<= 1) acc += __shfl_xor(acc, off);
+        if (o == 0) out[row] = sqrtf(acc);
+    }
+}
+
+// Routing order of one salience block: for every row of norms [BH, S] (non-negative float32; their bit patterns
+// order like the values), the positions of the S - n_hi rows outside the n_hi largest norms in ascending order,
+// then the positions of the n_hi largest in ascending order; equal norms at the threshold go to the later
+// positions first.  One block per row: a radix select over the norm bits (four passes of eight bits) finds the
+// threshold and how many rows equal to it are taken, then every thread walks a contiguous stretch of positions
+// twice (count, then write) around a block-wide scan, which keeps both parts in order.
+constexpr int ZR_THREADS = 256;
+__global__ __launch_bounds__(ZR_THREADS) void zip_route_kernel(const float *__restrict__ norms, int64_t S, int64_t n_hi,
+                                                               int32_t *__restrict__ order) {
+    __shared__ unsigned s_hist[256];
+    __shared__ unsigned s_prefix, s_pmask;
+    __shared__ long long s_want;
+    __shared__ long long s_cnt[ZR_THREADS];
+    const int tid = threadIdx.x;
+    const uint32_t *key = reinterpret_cast<const uint32_t *>(norms) + (int64_t)blockIdx.x * S;
+    int32_t *dst = order + (int64_t)blockIdx.x * S;
+    if (tid == 0) { s_prefix = 0; s_pmask = 0; s_want = n_hi; }
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        s_hist[tid] = 0;
+        __syncthreads();
+        const unsigned prefix = s_prefix, pmask = s_pmask;
+        for (int64_t i = tid; i < S; i += ZR_THREADS) {
+            const uint32_t k = key[i];
+            if ((k & pmask) == prefix) atomicAdd(&s_hist[(k >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (tid == 0) {   // the digit in which the s_want-th largest of the rows that match so far lies
+            long long above = 0;
+            int b = 255;
+            for (; b > 0; --b) {
+                if (above + s_hist[b] >= s_want) break;
+                above += s_hist[b];
+            }
+            s_want -= above;
+            s_prefix = prefix | ((unsigned)b << shift);
+            s_pmask = pmask | (255u << shift);
+        }
+        __syncthreads();
+    }
+    const uint32_t v = s_prefix;          // the threshold norm
+    const long long take_eq = s_want;     // rows equal to it that belong to the block, the latest ones
+    const int64_t C = (S + ZR_THREADS - 1) / ZR_THREADS;
+    const int64_t i0 = (int64_t)tid * C < S ? (int64_t)tid * C : S, i1 = i0 + C < S ? i0 + C : S;
+    long long eq_here = 0;
+    for (int64_t i = i0; i < i1; ++i) eq_here += key[i] == v;
+    s_cnt[tid] = eq_here;
+    __syncthreads();
+    long long eq_after = 0;               // rows equal to the threshold in later stretches
+    for (int t = tid + 1; t < ZR_THREADS; ++t) eq_after += s_cnt[t];
+    __syncthreads();
+    // a row equal to the threshold is taken when at most take_eq such rows lie at or after it
+    long long seen = 0, sel_here = 0;
+    for (int64_t i = i0; i < i1; ++i) {
+        const uint32_t k = key[i];
+        const bool eq = k == v;
+        sel_here += k > v || (eq && eq_after + eq_here - seen <= take_eq);
+        seen += eq;
+    }
+    s_cnt[tid] = sel_here;
+    __syncthreads();
+    long long sel_before = 0;
+    for (int t = 0; t < tid; ++t) sel_before += s_cnt[t];
+    int64_t out_sel = (S - n_hi) + sel_before, out_rest = i0 - sel_before;
+    seen = 0;
+    for (int64_t i = i0; i < i1; ++i) {
+        const uint32_t k = key[i];
+        const bool eq = k == v;
+        const bool sel = k > v || (eq && eq_after + eq_here - seen <= take_eq);
+        seen += eq;
+        if (sel) dst[out_sel++] = (int32_t)i;
+        else dst[out_rest++] = (int32_t)i;
+    }
+}
+
 static inline bool pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -653,7 +748,7 @@ using namespace vq;
 template <typename T, typename M, int LPR>
 static void launch_key_tile(int mode, const void *x, void *out, int64_t BH, int64_t S, int64_t xs, int group,
                             int levels, float eps, int bits, void *packed, void *scale, void *zero, int64_t cap,
-                            int64_t tok0, hipStream_t st) {
+                            int64_t tok0, hipStream_t st, const int32_t *rows = nullptr, int64_t rows_stride = 0) {
     dim3 grid((unsigned)cdiv(S, group), (unsigned)BH);
     int W = (int)cdiv(LPR * 8, 32 / (bits > 0 ? bits : 8));
     // fewer passes held in registers let more blocks share a CU
@@ -661,7 +756,7 @@ static void launch_key_tile(int mode, const void *x, void *out, int64_t BH, int6
     const bool small = group <= (KT_MAXP / 2) * RPP;
 #define VQ_LK(MODE, NP)                                                                                               \
     hipLaunchKernelGGL((kivi_key_tile_kernel<T, M, LPR, MODE, NP>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, \
-                       xs, group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W)
+                       xs, group, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W, rows, rows_stride)
     if (mode == 0) { if (small) VQ_LK(0, KT_MAXP / 2); else VQ_LK(0, KT_MAXP); }
     else { if (small) VQ_LK(1, KT_MAXP / 2); else VQ_LK(1, KT_MAXP); }
 #undef VQ_LK
@@ -756,6 +851,63 @@ int pack_kv_pair(const void *k, const void *v, int dtype, int64_t BH, int64_t S,
     return VQ_OK;
 }
 }  // namespace vq
+
+extern "C" int vq_row_norms(const void *x, int dtype, int64_t n_rows, int64_t D, float *out, void *stream) {
+    const char *fn = "vq_row_norms";
+    VQ_REQUIRE(n_rows >= 0 && D >= 0, VQ_ERR_INVALID, "%s: negative dimension", fn);
+    VQ_REQUIRE(is_float_tag(dtype), VQ_ERR_INVALID, "%s: unsupported dtype tag %d", fn, dtype);
+    if (n_rows * D == 0) return VQ_OK;
+    VQ_REQUIRE(x && out, VQ_ERR_INVALID, "%s: null pointer", fn);
+    VQ_REQUIRE((D == 64 || D == 128 || D == 256) && aligned16(x), VQ_ERR_UNSUPPORTED,
+               "%s: needs head_dim 64/128/256 and 16-byte aligned rows", fn);
+    hipStream_t st = (hipStream_t)stream;
+    int64_t blocks = cdiv(n_rows, 256 / (D / 8));
+    if (blocks > 65536) blocks = 65536;
+    VQ_DISPATCH_FLOAT(dtype, T, {
+        if (D == 64) hipLaunchKernelGGL((row_norm_kernel<T, 8>), dim3((unsigned)blocks), dim3(256), 0, st, (const T *)x, n_rows, out);
+        else if (D == 128) hipLaunchKernelGGL((row_norm_kernel<T, 16>), dim3((unsigned)blocks), dim3(256), 0, st, (const T *)x, n_rows, out);
+        else hipLaunchKernelGGL((row_norm_kernel<T, 32>), dim3((unsigned)blocks), dim3(256), 0, st, (const T *)x, n_rows, out);
+    });
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_zip_route(const float *norms, int64_t BH, int64_t S, int64_t n_hi, int32_t *order, void *stream) {
+    const char *fn = "vq_zip_route";
+    VQ_REQUIRE(BH >= 0 && S >= 0, VQ_ERR_INVALID, "%s: negative dimension", fn);
+    VQ_REQUIRE(n_hi >= 1 && n_hi < S, VQ_ERR_INVALID, "%s: n_hi=%lld must be in [1, S) (one block needs no routing)", fn,
+               (long long)n_hi);
+    VQ_REQUIRE(S < ((int64_t)1 << 31) && BH <= 0x7fffffff, VQ_ERR_INVALID, "%s: positions must fit 31 bits", fn);
+    if (BH == 0) return VQ_OK;
+    VQ_REQUIRE(norms && order, VQ_ERR_INVALID, "%s: null pointer", fn);
+    hipLaunchKernelGGL(zip_route_kernel, dim3((unsigned)BH), dim3(ZR_THREADS), 0, (hipStream_t)stream, norms, S, n_hi, order);
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_kivi_quant_dequant_rows(const void *x, void *out, int dtype, int64_t BH, int64_t n_rows, int64_t D,
+                                          int64_t stride_bh, const int32_t *rows, int64_t rows_stride, int group, int levels,
+                                          float eps, void *stream) {
+    const char *fn = "vq_kivi_quant_dequant_rows";
+    VQ_REQUIRE(group >= 1 && levels >= 1, VQ_ERR_INVALID, "%s: group_size and levels must be >= 1", fn);
+    VQ_REQUIRE(BH >= 0 && n_rows >= 0 && D >= 0, VQ_ERR_INVALID, "%s: negative dimension", fn);
+    VQ_REQUIRE(is_float_tag(dtype), VQ_ERR_INVALID, "%s: unsupported dtype tag %d", fn, dtype);
+    if (BH * n_rows * D == 0) return VQ_OK;
+    VQ_REQUIRE(x && out && rows, VQ_ERR_INVALID, "%s: null pointer", fn);
+    VQ_REQUIRE(rows_stride >= n_rows, VQ_ERR_INVALID, "%s: rows_stride %lld below n_rows %lld", fn, (long long)rows_stride,
+               (long long)n_rows);
+    VQ_REQUIRE((D == 64 || D == 128 || D == 256) && aligned16(x) && aligned16(out) && stride_bh % 8 == 0 && BH <= 65535 &&
+                   group <= KT_MAXP * (256 / (int)(D / 8)),
+               VQ_ERR_UNSUPPORTED, "%s: needs head_dim 64/128/256, 16-byte aligned slabs and a group the tile kernel holds", fn);
+    hipStream_t st = (hipStream_t)stream;
+    VQ_DISPATCH_FLOAT(dtype, T, {
+        if (D == 64) launch_key_tile<T, float, 8>(0, x, out, BH, n_rows, stride_bh, group, levels, eps, 0, nullptr, nullptr, nullptr, 0, 0, st, rows, rows_stride);
+        else if (D == 128) launch_key_tile<T, float, 16>(0, x, out, BH, n_rows, stride_bh, group, levels, eps, 0, nullptr, nullptr, nullptr, 0, 0, st, rows, rows_stride);
+        else launch_key_tile<T, float, 32>(0, x, out, BH, n_rows, stride_bh, group, levels, eps, 0, nullptr, nullptr, nullptr, 0, 0, st, rows, rows_stride);
+    });
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
 
 extern "C" int vq_kivi_quant_pack_kv(const void *k, const void *v, int dtype, int64_t BH, int64_t S, int64_t D,
                                      int64_t x_stride_bh, int group, int levels, float eps, int pack_bits, int v_layout,

@@ -157,6 +157,58 @@ def skvq_clipped_round_trip(x: torch.Tensor, bits: int, group_size: int, alphas,
     return out
 
 
+def row_norms(x: torch.Tensor) -> torch.Tensor:
+    """float32 L2 norms over the last axis of ``x [..., D]`` (D in 64 / 128 / 256), one pass over the stored rows."""
+    name = "row_norms"
+    tag = _ftag(name, x)
+    _need_gpu(name, x)
+    x = x.contiguous()
+    D = x.shape[-1]
+    out = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    _lib.check(_lib.load().vq_row_norms(x.data_ptr(), tag, x.numel() // D, D, out.data_ptr(), _stream(x)))
+    return out
+
+
+def zip_route(norms: torch.Tensor, n_hi: int) -> torch.Tensor:
+    """int32 ``[BH, S]`` routing order of a salience split of float32 ``norms [BH, S]``: the rows outside the
+    ``n_hi`` largest norms in their own order, then the ``n_hi`` largest in theirs, later rows first among equal norms
+    at the threshold (``_batched_saliency_mask`` + stable argsort of the mask,
+    veloxquant_mlx/cache/zipcache_cache.py:106-116, 186-190)."""
+    name = "zip_route"
+    if norms.ndim != 2 or norms.dtype != torch.float32:
+        raise ValueError(f"{name}: norms must be a float32 [BH, S] tensor")
+    _need_gpu(name, norms)
+    norms = norms.contiguous()
+    BH, S = norms.shape
+    order = torch.empty((BH, S), dtype=torch.int32, device=norms.device)
+    _lib.check(_lib.load().vq_zip_route(norms.data_ptr(), BH, S, int(n_hi), order.data_ptr(), _stream(norms)))
+    return order
+
+
+def kivi_group_quant_dequant_rows(x: torch.Tensor, out: torch.Tensor, rows: torch.Tensor, start: int, n_rows: int,
+                                  group_size: int, levels: int, eps: float = 1e-8) -> torch.Tensor:
+    """Token-axis round trip over routed rows, in one launch and without a gathered copy: positions
+    ``start .. start + n_rows`` of the routing order ``rows`` (int32 ``[BH, S]``) name rows of ``x [BH, S, D]``;
+    consecutive positions form the groups, every reconstruction lands in ``out`` (same shape and dtype as ``x``) at
+    its source row.  What gather -> ``_group_quant_dequant_batched`` -> scatter does for one salience block of
+    ``ZipCacheKVCache`` (veloxquant_mlx/cache/zipcache_cache.py:118-244)."""
+    name = "kivi_group_quant_dequant_rows"
+    if x.ndim != 3 or tuple(out.shape) != tuple(x.shape) or out.dtype != x.dtype or not (x.is_contiguous() and out.is_contiguous()):
+        raise ValueError(f"{name}: x and out must be contiguous [BH, S, D] tensors of one dtype")
+    BH, S, D = x.shape
+    if tuple(rows.shape) != (BH, S) or rows.dtype != torch.int32 or not rows.is_contiguous():
+        raise ValueError(f"{name}: rows must be a contiguous int32 [{BH}, {S}] tensor")
+    if not (0 <= start and start + n_rows <= S):
+        raise ValueError(f"{name}: positions [{start}, {start + n_rows}) outside [0, {S})")
+    tag = _ftag(name, x)
+    _need_gpu(name, x, out, rows)
+    rc = _lib.load().vq_kivi_quant_dequant_rows(x.data_ptr(), out.data_ptr(), tag, BH, int(n_rows), D, S * D,
+                                                rows.data_ptr() + 4 * int(start), S, int(group_size), int(levels), float(eps),
+                                                _stream(x))
+    _lib.check(rc)
+    return out
+
+
 def kivi_quant_pack(x: torch.Tensor, axis: int, group_size: int, bits: int, *, levels: int | None = None,
                     eps: float = 1e-8, meta_dtype: torch.dtype = torch.float16, v_layout: str = "channel",
                     out: tuple[torch.Tensor, torch.Tensor, torch.Tensor] | None = None,
@@ -953,7 +1005,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "kivi_group_quant_dequant", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
+    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",
