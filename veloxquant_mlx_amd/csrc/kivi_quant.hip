@@ -15,6 +15,8 @@
 //     rescans the group it needs -- slow but free of layout assumptions.
 #include "common.hpp"
 
+#include <type_traits>
+
 namespace vq {
 
 __device__ __forceinline__ float quant_code(float v, float mn, float sc, float levels) {
@@ -468,11 +470,260 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
                                           bits, packed, scale, zero, cap_tokens, dst_tok0, W);
 }
 
+// ---------------------------------------------------------------------------
+// Values, token-packed, head_dim 128: a thread owns the PER = 32 / BITS tokens of one packed word for 8
+// consecutive channels, so the eight words it writes (one per channel) are made of its own codes -- no
+// transposition through LDS -- and leave as one 32-byte piece; the scale / zero of a (token, channel group) are
+// reduced across the group's lanes with lane moves inside a row of 16 lanes, and a thread's PER values of a
+// channel group leave as whole vectors of the token-major rows.  16 lanes cover the 128 channels of PER tokens,
+// a wave four such stretches, a block sixteen.
+// ---------------------------------------------------------------------------
+template <int CTRL> __device__ __forceinline__ float lane_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+__device__ __forceinline__ float bare_min(float a, float b) { float d; asm("v_min_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b)); return d; }
+__device__ __forceinline__ float bare_max(float a, float b) { float d; asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b)); return d; }
+// minimum and maximum over the GL lanes (4, 8 or 16, aligned) that hold a channel group
+template <int GL> __device__ __forceinline__ void group_span(float &mn, float &mx) {
+    mn = bare_min(mn, lane_move<0xB1>(mn)); mx = bare_max(mx, lane_move<0xB1>(mx));     // quad_perm [1,0,3,2]
+    mn = bare_min(mn, lane_move<0x4E>(mn)); mx = bare_max(mx, lane_move<0x4E>(mx));     // quad_perm [2,3,0,1]
+    if constexpr (GL >= 8) { mn = bare_min(mn, lane_move<0x141>(mn)); mx = bare_max(mx, lane_move<0x141>(mx)); }   // row_half_mirror
+    if constexpr (GL >= 16) { mn = bare_min(mn, lane_move<0x140>(mn)); mx = bare_max(mx, lane_move<0x140>(mx)); }  // row_mirror
+}
+constexpr int VP_STRETCHES = 16;   // stretches of PER tokens per block of 256 threads
+
+// The same walk writing the reconstruction instead (the round trip): stretches of 8 tokens, the last one of a
+// sequence may be short.
+template <typename T, int GL>
+__global__ __launch_bounds__(256) void kivi_value_roundtrip_kernel(const T *__restrict__ x, T *__restrict__ out, int64_t S,
+                                                                   int64_t x_stride_bh, float levels, float eps) {
+    constexpr int D = 128, PER = 8;
+    const int tid = threadIdx.x, o = tid & 15;
+    const int64_t bh = blockIdx.y;
+    const int64_t t0 = ((int64_t)blockIdx.x * VP_STRETCHES + (tid >> 4)) * PER;
+    if (t0 >= S) return;
+    const T *xb = x + bh * x_stride_bh + t0 * D + 8 * o;
+    T *ob = out + (bh * S + t0) * D + 8 * o;
+    Raw8<T> v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i)
+        if (t0 + i < S) v[i].load(xb + (int64_t)i * D);
+        else v[i] = v[0];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        float mn, mx;
+        v[i].span(mn, mx);
+        group_span<GL>(mn, mx);
+        const float sc = group_scale(mn, mx, levels, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
+        float x8[8], q[8], y[8], mn8[8], sc8[8], rs8[8], nb8[8], tl8[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; tl8[c] = tl; }
+        v[i].floats(x8);
+        quant_codes8(x8, mn8, sc8, rs8, nb8, tl8, levels, !(rs < 1e30f), q);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) y[c] = recon(q[c], sc, mn);
+        if (t0 + i < S) store8<T>(ob + (int64_t)i * D, y);
+    }
+}
+
+template <typename T, typename M, int BITS, int GL>
+__device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T *__restrict__ x, int64_t S,
+                                                     int64_t x_stride_bh, float levels, float eps,
+                                                     uint32_t *__restrict__ packed, M *__restrict__ scale,
+                                                     M *__restrict__ zero, int64_t cap_tokens, int64_t dst_tok0) {
+    constexpr int D = 128, PER = 32 / BITS, HALF = PER / 2, GV = 16 / GL;
+    const int tid = threadIdx.x, o = tid & 15;
+    const int64_t t0 = ((int64_t)bx * VP_STRETCHES + (tid >> 4)) * PER;   // the stretch's first token
+    if (t0 >= S) return;                                                  // S is a multiple of PER: whole rows of 16 lanes leave
+    const T *xb = x + bh * x_stride_bh + t0 * D + 8 * o;
+    Raw8<T> v[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) v[i].load(xb + (int64_t)i * D);
+    float lo[8], hi[8], scv[PER], mnv[PER];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) { lo[c] = 0.f; hi[c] = 0.f; }
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        float mn, mx;
+        v[i].span(mn, mx);
+        group_span<GL>(mn, mx);
+        const float sc = group_scale(mn, mx, levels, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
+        scv[i] = sc;
+        mnv[i] = mn;
+        float x8[8], q[8], mn8[8], sc8[8], rs8[8], nb8[8], tl8[8];
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; tl8[c] = tl; }
+        v[i].floats(x8);
+        quant_codes8(x8, mn8, sc8, rs8, nb8, tl8, levels, !(rs < 1e30f), q);
+        // code of token i at bits [BITS * i, BITS * (i + 1)): two exact float sums of 16 bits each
+        const float w = (float)(1u << (BITS * (i % HALF)));
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+            if (i < HALF) lo[c] = __builtin_fmaf(q[c], w, lo[c]);
+            else hi[c] = __builtin_fmaf(q[c], w, hi[c]);
+        }
+    }
+    const int64_t tok = dst_tok0 + t0;
+    uint32_t wd[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) wd[c] = (uint32_t)lo[c] | ((uint32_t)hi[c] << 16);
+    uint4 *wp = reinterpret_cast<uint4 *>(packed + (bh * (cap_tokens / PER) + tok / PER) * D + 8 * o);
+    wp[0] = make_uint4(wd[0], wd[1], wd[2], wd[3]);
+    wp[1] = make_uint4(wd[4], wd[5], wd[6], wd[7]);
+    if ((o & (GL - 1)) == 0) {   // the first lane of a channel group writes its PER scales and zeros
+        const int64_t mi = (bh * GV + o / GL) * cap_tokens + tok;
+#pragma unroll
+        for (int i = 0; i < PER; i += 8) {
+            const float s8[8] = {scv[i], scv[i + 1], scv[i + 2], scv[i + 3], scv[i + 4], scv[i + 5], scv[i + 6], scv[i + 7]};
+            const float z8[8] = {mnv[i], mnv[i + 1], mnv[i + 2], mnv[i + 3], mnv[i + 4], mnv[i + 5], mnv[i + 6], mnv[i + 7]};
+            store_meta8<M>(scale + mi + i, s8);
+            store_meta8<M>(zero + mi + i, z8);
+        }
+    }
+}
+
+template <typename T, typename M, int BITS, int GL>
+__global__ __launch_bounds__(256) void kivi_value_pack_kernel(const T *__restrict__ x, int64_t S, int64_t x_stride_bh,
+                                                              float levels, float eps, uint32_t *__restrict__ packed,
+                                                              M *__restrict__ scale, M *__restrict__ zero,
+                                                              int64_t cap_tokens, int64_t dst_tok0) {
+    kivi_value_pack_body<T, M, BITS, GL>((int)blockIdx.x, (int64_t)blockIdx.y, x, S, x_stride_bh, levels, eps, packed, scale,
+                                         zero, cap_tokens, dst_tok0);
+}
+
+// ---------------------------------------------------------------------------
+// Keys, head_dim 128, groups of 4 * TPL tokens (32 or 64): one wave per group.  Lane 4 * o + tq owns 8
+// consecutive channels (chunk o of 16) of the TPL tokens tq * TPL .. of the group, so the per-channel minima and
+// maxima are folded in the lane and then across the four lanes of a quad with lane moves -- no block-shared
+// memory, no barrier -- and every lane ends up with the parameters of its 8 channels.  A row's 8 codes are one
+// 4-bit word (two lanes' fields make a 2-bit word).  MODE 0 writes the reconstruction, MODE 1 codes + scale/zero.
+// ---------------------------------------------------------------------------
+template <typename T> struct QuadFold {   // fold a Raw8 accumulator across the quad
+    static __device__ __forceinline__ void run(typename Raw8<T>::Acc &a) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            a.mn[i] = bare_min(a.mn[i], lane_move<0xB1>(a.mn[i])); a.mx[i] = bare_max(a.mx[i], lane_move<0xB1>(a.mx[i]));
+            a.mn[i] = bare_min(a.mn[i], lane_move<0x4E>(a.mn[i])); a.mx[i] = bare_max(a.mx[i], lane_move<0x4E>(a.mx[i]));
+        }
+    }
+};
+template <> struct QuadFold<f16> {
+    template <int CTRL> static __device__ __forceinline__ uint32_t mv(uint32_t x) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xF, 0xF, true);
+    }
+    static __device__ __forceinline__ void run(Raw8<f16>::Acc &a) {
+        typedef uint32_t w4 __attribute__((ext_vector_type(4)));
+        w4 mn = __builtin_bit_cast(w4, a.mn), mx = __builtin_bit_cast(w4, a.mx);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            mn[i] = Raw8<f16>::pk_min(mn[i], mv<0xB1>(mn[i])); mx[i] = Raw8<f16>::pk_max(mx[i], mv<0xB1>(mx[i]));
+            mn[i] = Raw8<f16>::pk_min(mn[i], mv<0x4E>(mn[i])); mx[i] = Raw8<f16>::pk_max(mx[i], mv<0x4E>(mx[i]));
+        }
+        a.mn = __builtin_bit_cast(f16x8, mn);
+        a.mx = __builtin_bit_cast(f16x8, mx);
+    }
+};
+constexpr int KQ_WAVES = 4;   // groups per block
+
+template <typename T, typename M, int MODE, int TPL>
+__device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *__restrict__ x, T *__restrict__ out, int64_t S,
+                                                   int64_t x_stride_bh, float levels, float eps, int bits,
+                                                   uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
+                                                   int64_t cap_tokens, int64_t dst_tok0, int W) {
+    constexpr int D = 128, G = 4 * TPL;
+    const int lane = threadIdx.x & 63, o = lane >> 2, tq = lane & 3;
+    const int64_t s0 = (int64_t)gk * G;
+    if (s0 >= S) return;   // the whole wave
+    const int64_t r0 = s0 + tq * TPL;   // the lane's first token
+    const T *xb = x + bh * x_stride_bh + r0 * D + 8 * o;
+    Raw8<T> v[TPL];
+    typename Raw8<T>::Acc acc;
+    Raw8<T>::init(acc);
+#pragma unroll
+    for (int i = 0; i < TPL; ++i)
+        if (r0 + i < S) {
+            v[i].load(xb + (int64_t)i * D);
+            v[i].fold(acc);
+        }
+    QuadFold<T>::run(acc);
+    float mn[8], mx[8], sc[8], rs[8], nb[8], tie_lo[8];
+    Raw8<T>::result(acc, mn, mx);
+    bool redo = false;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        sc[c] = group_scale(mn[c], mx[c], levels, eps);
+        rs[c] = fast_rcp(sc[c]);
+        nb[c] = -mn[c] * rs[c];
+        tie_lo[c] = tie_limit(levels, nb[c]);
+        redo |= !(rs[c] < 1e30f);
+    }
+    if (MODE == 1 && tq == 0) {
+        const int64_t gdst = dst_tok0 / G + gk, gcap = (cap_tokens + G - 1) / G;
+        store_meta8<M>(scale + (bh * gcap + gdst) * D + 8 * o, sc);
+        store_meta8<M>(zero + (bh * gcap + gdst) * D + 8 * o, mn);
+    }
+#pragma unroll
+    for (int i = 0; i < TPL; ++i) {
+        const int64_t srow = r0 + i;
+        const bool valid = srow < S;
+        float x8[8], q[8];
+        if (valid) v[i].floats(x8);
+        else {   // keep the arithmetic defined; the lane's results are not stored
+#pragma unroll
+            for (int c = 0; c < 8; ++c) x8[c] = mn[c];
+        }
+        quant_codes8(x8, mn, sc, rs, nb, tie_lo, levels, redo, q);
+        if (MODE == 0) {
+            if (valid) {
+                float y[8];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) y[c] = recon(q[c], sc[c], mn[c]);
+                store8<T>(out + (bh * S + srow) * D + 8 * o, y);
+            }
+        } else {
+            uint32_t *row_words = packed + (bh * cap_tokens + dst_tok0 + (valid ? srow : 0)) * W;
+            if (bits == 8) {
+                if (valid) *reinterpret_cast<uint2 *>(row_words + 2 * o) = bytes8(q);
+            } else if (bits == 4) {
+                const uint32_t w = field8(q, 4);
+                if (valid) row_words[o] = w;
+            } else {   // 2 bits: chunk o + 1 sits four lanes up
+                const uint32_t f = field8(q, 2);
+                const uint32_t up = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f, 0x104, 0xF, 0xF, true);   // row_shl:4
+                if (valid && (o & 1) == 0) row_words[o >> 1] = f | (up << 16);
+            }
+        }
+    }
+}
+
+template <typename T, typename M, int MODE, int TPL>
+__global__ __launch_bounds__(64 * KQ_WAVES) void kivi_key_quad_kernel(
+    const T *__restrict__ x, T *__restrict__ out, int64_t S, int64_t x_stride_bh, float levels, float eps, int bits,
+    uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero, int64_t cap_tokens, int64_t dst_tok0, int W) {
+    kivi_key_quad_body<T, M, MODE, TPL>((int)blockIdx.x * KQ_WAVES + (int)(threadIdx.x >> 6), (int64_t)blockIdx.y, x, out, S,
+                                        x_stride_bh, levels, eps, bits, packed, scale, zero, cap_tokens, dst_tok0, W);
+}
+
 // Keys and values of one cache flush in a single launch: blocks [0, key_blocks) of a (b, h)
 // take the key groups, the rest the value row tiles.  The two bodies are those of the kernels
 // above; a chunked prefill flushes a few hundred tokens at a time, where a second launch costs
 // as much as the work.
 struct PackDst { uint32_t *packed; void *scale, *zero; };
+// the same for head_dim 128, groups of 32 or 64, 2 or 4 bits, token-packed values: the quad-layout key body and the
+// word-owning value body, neither of which uses block-shared memory
+template <typename T, typename M, int BITS, int TPL>
+__global__ __launch_bounds__(256) void kivi_kv_pack_kernel(
+    const T *__restrict__ k, const T *__restrict__ v, int64_t S, int64_t x_stride_bh, float levels, float eps, PackDst kd,
+    PackDst vd, int64_t cap_tokens, int64_t dst_tok0, int key_blocks) {
+    const int bx = (int)blockIdx.x;
+    if (bx < key_blocks)
+        kivi_key_quad_body<T, M, 1, TPL>(bx * KQ_WAVES + (int)(threadIdx.x >> 6), (int64_t)blockIdx.y, k, nullptr, S, x_stride_bh,
+                                         levels, eps, BITS, kd.packed, (M *)kd.scale, (M *)kd.zero, cap_tokens, dst_tok0,
+                                         128 / (32 / BITS));
+    else
+        kivi_value_pack_body<T, M, BITS, TPL / 2>(bx - key_blocks, (int64_t)blockIdx.y, v, S, x_stride_bh, levels, eps, vd.packed,
+                                                  (M *)vd.scale, (M *)vd.zero, cap_tokens, dst_tok0);
+}
 template <typename T, typename M, int LPR, int NP, int VMODE>
 __global__ __launch_bounds__(256) void kivi_kv_tile_kernel(
     const T *__restrict__ k, const T *__restrict__ v, int64_t S, int64_t x_stride_bh, int group, float levels, float eps,
@@ -789,6 +1040,17 @@ static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t 
     if (mode != 0 && !(aligned16(packed) && aligned16(scale) && aligned16(zero))) return false;
     const int LPR = (int)(D / 8), RPP = 256 / LPR;
     if (axis == VQ_AXIS_TOKEN) {
+        if (D == 128 && (group == 32 || group == 64) && (mode == 0 || bits == 2 || bits == 4 || bits == 8)) {
+            const dim3 grid((unsigned)cdiv(cdiv(S, group), KQ_WAVES), (unsigned)BH);
+            const int W = (int)cdiv(D, 32 / (bits > 0 ? bits : 8));
+#define VQ_KQ(MODE, TPL)                                                                                                  \
+            hipLaunchKernelGGL((kivi_key_quad_kernel<T, M, MODE, TPL>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, \
+                               S, xs, (float)levels, eps, bits, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0, W)
+            if (mode == 0) { if (group == 32) VQ_KQ(0, 8); else VQ_KQ(0, 16); }
+            else { if (group == 32) VQ_KQ(1, 8); else VQ_KQ(1, 16); }
+#undef VQ_KQ
+            return true;
+        }
         if (group > KT_MAXP * RPP) return false;
 #define VQ_K(L) launch_key_tile<T, M, L>(mode, x, out, BH, S, xs, group, levels, eps, bits, packed, scale, zero, cap, tok0, st)
         if (LPR == 8) VQ_K(8); else if (LPR == 16) VQ_K(16); else VQ_K(32);
@@ -796,6 +1058,24 @@ static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t 
         return true;
     }
     if (group % 8 != 0 || !pow2(group / 8) || group > D || D % group != 0) return false;
+    if (mode == 0 && D == 128 && group >= 32) {
+        const dim3 grid((unsigned)cdiv(S, VP_STRETCHES * 8), (unsigned)BH);
+#define VQ_VR(GL) hipLaunchKernelGGL((kivi_value_roundtrip_kernel<T, GL>), grid, dim3(256), 0, st, (const T *)x, (T *)out, S, xs, (float)levels, eps)
+        if (group == 32) VQ_VR(4); else if (group == 64) VQ_VR(8); else VQ_VR(16);
+#undef VQ_VR
+        return true;
+    }
+    if (mode == 2 && D == 128 && (bits == 2 || bits == 4) && group >= 32 && !std::is_same<T, float>::value &&
+        S % (32 / bits) == 0 && tok0 % 8 == 0 && cap % 8 == 0) {
+        const dim3 grid((unsigned)cdiv(S, VP_STRETCHES * (32 / bits)), (unsigned)BH);
+#define VQ_VP(BITS, GL)                                                                                              \
+        hipLaunchKernelGGL((kivi_value_pack_kernel<T, M, BITS, GL>), grid, dim3(256), 0, st, (const T *)x, S, xs,       \
+                           (float)levels, eps, (uint32_t *)packed, (M *)scale, (M *)zero, cap, tok0)
+        if (bits == 4) { if (group == 32) VQ_VP(4, 4); else if (group == 64) VQ_VP(4, 8); else VQ_VP(4, 16); }
+        else { if (group == 32) VQ_VP(2, 4); else if (group == 64) VQ_VP(2, 8); else VQ_VP(2, 16); }
+#undef VQ_VP
+        return true;
+    }
     if (mode == 2 && (RPP % (32 / bits)) != 0) return false;
 #define VQ_V(L) launch_value_tile<T, M, L>(mode, x, out, BH, S, xs, group, levels, eps, bits, packed, scale, zero, cap, tok0, st)
     if (LPR == 8) VQ_V(8); else if (LPR == 16) VQ_V(16); else VQ_V(32);
@@ -826,11 +1106,30 @@ int pack_kv_pair(const void *k, const void *v, int dtype, int64_t BH, int64_t S,
         return vq_kivi_quant_pack(v, dtype, BH, S, D, xs, VQ_AXIS_CHANNEL, group, levels, eps, bits, v_layout, vp, vs, vz,
                                   meta_dtype, cap, tok0, stream);
     }
+    const PackDst kd = {(uint32_t *)kp, ks, kz}, vd = {(uint32_t *)vp, vs, vz};
+    hipStream_t st = (hipStream_t)stream;
+    if (tokpacked && (group == 32 || group == 64) && (bits == 2 || bits == 4) && tok0 % 8 == 0 && cap % 8 == 0) {
+        // group = 4 * TPL tokens for the keys = 8 * GL channels for the values: GL = TPL / 2
+        const int kb = (int)cdiv(cdiv(S, group), KQ_WAVES), vb = (int)cdiv(S, VP_STRETCHES * per);
+        const dim3 g2((unsigned)(kb + vb), (unsigned)BH);
+#define VQ_KV2(T, M, BITS, TPL)                                                                                          \
+        hipLaunchKernelGGL((kivi_kv_pack_kernel<T, M, BITS, TPL>), g2, dim3(256), 0, st, (const T *)k, (const T *)v, S, xs,  \
+                           (float)levels, eps, kd, vd, cap, tok0, kb)
+#define VQ_KV2_B(T, M)                                                                                                    \
+        do {                                                                                                             \
+            if (bits == 4) { if (group == 32) VQ_KV2(T, M, 4, 8); else VQ_KV2(T, M, 4, 16); }                            \
+            else { if (group == 32) VQ_KV2(T, M, 2, 8); else VQ_KV2(T, M, 2, 16); }                                      \
+        } while (0)
+        if (dtype == VQ_F16) { if (meta_dtype == VQ_F16) VQ_KV2_B(f16, f16); else VQ_KV2_B(f16, float); }
+        else { if (meta_dtype == VQ_F16) VQ_KV2_B(bf16_t, f16); else VQ_KV2_B(bf16_t, float); }
+#undef VQ_KV2_B
+#undef VQ_KV2
+        VQ_HIP_CHECK_LAUNCH("vq_kivi_cache_append");
+        return VQ_OK;
+    }
     const int key_blocks = (int)cdiv(S, group), value_blocks = (int)cdiv(S, ROWS);
     const dim3 grid((unsigned)(key_blocks + value_blocks), (unsigned)BH);
     const int W = (int)cdiv(LPR * 8, per);
-    const PackDst kd = {(uint32_t *)kp, ks, kz}, vd = {(uint32_t *)vp, vs, vz};
-    hipStream_t st = (hipStream_t)stream;
 #define VQ_KV(T, M, NP, VM)                                                                                              \
     hipLaunchKernelGGL((kivi_kv_tile_kernel<T, M, LPR, NP, VM>), grid, dim3(256), 0, st, (const T *)k, (const T *)v, S, xs, \
                        group, (float)levels, eps, bits, kd, vd, cap, tok0, W, key_blocks)
