@@ -649,14 +649,17 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
     float mn[8], mx[8], sc[8], rs[8], nb[8], tie_lo[8];
     Raw8<T>::result(acc, mn, mx);
     bool redo = false;
+    float tie_all = 0.5f;   // one limit for the lane's 8 channels, the tightest: a few more rows take the division
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
         sc[c] = group_scale(mn[c], mx[c], levels, eps);
         rs[c] = fast_rcp(sc[c]);
         nb[c] = -mn[c] * rs[c];
-        tie_lo[c] = tie_limit(levels, nb[c]);
+        tie_all = fminf(tie_all, tie_limit(levels, nb[c]));
         redo |= !(rs[c] < 1e30f);
     }
+#pragma unroll
+    for (int c = 0; c < 8; ++c) tie_lo[c] = tie_all;
     if (MODE == 1 && tq == 0) {
         const int64_t gdst = dst_tok0 / G + gk, gcap = (cap_tokens + G - 1) / G;
         store_meta8<M>(scale + (bh * gcap + gdst) * D + 8 * o, sc);
