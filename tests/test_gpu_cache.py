@@ -239,7 +239,7 @@ def test_sink_protected_cache_matches_model(n_sink):
 
 @pytest.mark.parametrize("mode", ["memory_bound", "stash"])
 @pytest.mark.parametrize("bits,g,v_layout", [(4, 32, "token"), (2, 32, "token"), (4, 64, "channel")])
-def test_sink_protected_cache_on_packed_storage(mode, bits, g, v_layout):
+def test_sink_protected_cache_on_packed_storage(mode, bits, g, v_layout, tmp_path):
     """``kivi_sink`` with ``fused_sdpa``: the packed store holds stand-ins at the protected positions and
     the attention call swaps the exact rows in.  The oracle is attention over the history the numpy
     model of the reference's cache returns (sink_cache.py:117-198: protected rows exact, the rest
@@ -255,10 +255,11 @@ def test_sink_protected_cache_on_packed_storage(mode, bits, g, v_layout):
     v = rng.standard_normal((B, H, n, D)).astype(np.float16)
     for b, p, f in ((0, 3, 12), (0, 40, 9), (1, 150, 12), (1, 151, 10), (1, 310, 14), (0, 333, 8)):
         k[b, :, p] *= f
-    c = KVCacheFactory.create(KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=g,
-                                            residual_length=R, n_sink_tokens=3, fused_sdpa=True,
-                                            fused_sdpa_memory_bound=(mode == "memory_bound"), kivi_meta_dtype="float32",
-                                            kivi_value_layout=v_layout))
+    cfg = KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=g,
+                        residual_length=R, n_sink_tokens=3, fused_sdpa=True,
+                        fused_sdpa_memory_bound=(mode == "memory_bound"), kivi_meta_dtype="float32",
+                        kivi_value_layout=v_layout)
+    c = KVCacheFactory.create(cfg)
     m = ok.SinkCacheModel(bits, g, R, 3)
     scale = 1 / math.sqrt(D)
 
@@ -301,6 +302,27 @@ def test_sink_protected_cache_on_packed_storage(mode, bits, g, v_layout):
     check(1, "decode after trim")
     check(16, "chunk after trim")
     assert c.sink_fp16_bytes == m.sink_fp16_bytes and c.compressed_key_bytes == m.key_bytes_compressed
+
+    # a cache rebuilt from the state (directly and through a prompt-cache file) protects the same rows:
+    # same attention output now, and after both have taken the same further tokens and flushes
+    from veloxquant_mlx_amd.cache.prompt_cache import load_prompt_cache, save_prompt_cache
+    path = str(tmp_path / "sink.safetensors")
+    save_prompt_cache(path, [c])
+    twins = [type(c).from_state(cfg, c.state, c.meta_state), load_prompt_cache(path, lambda i, name: KVCacheFactory.create(cfg))[0]]
+    q = to_dev(rng.standard_normal((B, Hq, 1, D)).astype(np.float16))
+    for t in twins:
+        assert (t.offset, t._n_quantized, t._side_pos) == (c.offset, c._n_quantized, c._side_pos)
+        assert [t.sink_positions_for(b) for b in range(B)] == [c.sink_positions_for(b) for b in range(B)]
+        assert torch.equal(t.fused_sdpa(q, scale), c.fused_sdpa(q, scale))
+    for s in range(330, 420):
+        for t in (c, *twins):
+            t.update_and_fetch(to_dev(k[:, :, s:s + 1]), to_dev(v[:, :, s:s + 1]))
+        m.update_and_fetch(k[:, :, s:s + 1], v[:, :, s:s + 1])
+    for t in twins:
+        assert t._side_pos == c._side_pos and torch.equal(t.fused_sdpa(q, scale), c.fused_sdpa(q, scale))
+    check(1, "decode after restore")
+    with pytest.raises(ValueError):
+        KVCacheFactory.create(cfg).state = c.state[:-1]
 
 
 def test_chunked_prefill_through_the_cache_matches_oracle():

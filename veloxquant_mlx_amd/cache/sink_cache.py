@@ -250,17 +250,84 @@ class SinkProtectedKVCache(KIVIKVCache):
         self._top.drop_from(self.offset)
         return trimmed
 
+    _N_SINK_ARRAYS = 5
+
     @property
     def state(self):
-        if self._fused_enabled:
-            raise NotImplementedError("SinkProtectedKVCache: saving a packed cache with protected rows is not supported")
-        return KIVIKVCache.state.fget(self)
+        """Standard mode: the fp16 history, as KIVI's.  Packed modes: KIVI's arrays followed by
+        five more, the exact rows ``[B, H, n, D]`` (keys, values) with their positions ``[B, n]``
+        (int32, -1 for an unused slot) and the running candidates (norms float32 ``[B, n_sink]``,
+        positions int64 ``[B, n_sink]``), so that a restored cache protects what this one does."""
+        base = KIVIKVCache.state.fget(self)
+        if not self._fused_enabled or not base:
+            return base
+        ref = base[0]
+        B, H, D = self._shape_bhd
+        used = max([len(ps) for ps in self._side_pos], default=0)
+        if used:
+            side_k, side_v = self._side_k[:, :, :used], self._side_v[:, :, :used]
+            table = [ps + [-1] * (used - len(ps)) for ps in self._side_pos]
+            side_pos = torch.tensor(table, dtype=torch.int32, device=ref.device)
+        else:
+            side_k = torch.zeros((B, H, 0, D), dtype=torch.float16, device=ref.device)
+            side_v, side_pos = torch.zeros_like(side_k), torch.zeros((B, 0), dtype=torch.int32, device=ref.device)
+        self._top._grow(B)
+        return (*base, side_k, side_v, side_pos, self._top.norm[:B].to(ref.device), self._top.pos[:B].to(ref.device))
 
     @state.setter
     def state(self, v) -> None:
-        if self._fused_enabled:
-            raise NotImplementedError("SinkProtectedKVCache: restoring a packed cache with protected rows is not supported")
-        KIVIKVCache.state.fset(self, v)
+        v = tuple(v)
+        self._side_k = self._side_v = self._side_pos_dev = None
+        self._side_pos = []
+        self._top = _TopNorms(self._n_sink)
+        if not self._fused_enabled or not v:
+            KIVIKVCache.state.fset(self, v)
+            return
+        if len(v) < self._N_SINK_ARRAYS:
+            raise ValueError(f"SinkProtectedKVCache.state: a packed state ends with {self._N_SINK_ARRAYS} arrays for the "
+                             f"protected rows, got {len(v)} arrays in all")
+        side_k, side_v, side_pos, top_norm, top_pos = v[-self._N_SINK_ARRAYS:]
+        KIVIKVCache.state.fset(self, v[: -self._N_SINK_ARRAYS])
+        B, H, D = self._shape_bhd
+        used = int(side_pos.shape[1]) if side_pos.dim() == 2 else -1
+        if (tuple(side_k.shape) != (B, H, used, D) or tuple(side_v.shape) != (B, H, used, D) or int(side_pos.shape[0]) != B
+                or tuple(top_norm.shape) != (B, self._n_sink) or tuple(top_pos.shape) != (B, self._n_sink)):
+            raise ValueError(f"SinkProtectedKVCache.state: protected rows {tuple(side_k.shape)}/{tuple(side_v.shape)}, positions "
+                             f"{tuple(side_pos.shape)}, candidates {tuple(top_norm.shape)}/{tuple(top_pos.shape)} do not fit "
+                             f"B={B}, H={H}, head_dim={D}, n_sink_tokens={self._n_sink}")
+        table = side_pos.cpu().tolist()
+        self._side_pos = [[p for p in row if p >= 0] for row in table]
+        for row, ps in zip(table, self._side_pos):
+            if row[: len(ps)] != ps or any(not (0 <= p < self._n_quantized) for p in ps):
+                raise ValueError("SinkProtectedKVCache.state: positions of the protected rows must fill the slots from the "
+                                 "front and lie below the quantised frontier")
+        if used:
+            cap = max(8, used)
+            self._side_k = torch.zeros((B, H, cap, D), dtype=side_k.dtype, device=side_k.device)
+            self._side_v = torch.zeros_like(self._side_k)
+            self._side_k[:, :, :used], self._side_v[:, :, :used] = side_k, side_v
+        self._top.norm = top_norm.detach().to("cpu", torch.float32).clone()
+        self._top.pos = top_pos.detach().to("cpu", torch.int64).clone()
+        self._rebuild_accounting()
+
+    def _rebuild_accounting(self) -> None:
+        """Restored rows priced as the flushes price them: protected ones (the largest count over
+        the batch) in fp16, the rest as KIVI rows."""
+        super()._rebuild_accounting()
+        n_protected = max([len(ps) for ps in self._side_pos], default=0)
+        B, H, D = self._shape_bhd
+        if n_protected and self._n_quantized:
+            k, v = self._quantized_bytes(self._n_quantized - n_protected, B, H, D)
+            self._key_bytes_compressed, self._value_bytes_compressed = k, v
+        self._sink_fp16_bytes = n_protected * D * 2 * 2 * H * B
+
+    @property
+    def nbytes(self) -> int:
+        total = KIVIKVCache.nbytes.fget(self)
+        for t in (self._side_k, self._side_v):
+            if t is not None:
+                total += t.numel() * t.element_size()
+        return total
 
     # ------------------------------------------------------------------ reporting
     @property
