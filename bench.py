@@ -47,7 +47,7 @@ def _parse():
     p.add_argument("--only-kernel", action="store_true", help="time the attention kernel loop only (profiling)")
     p.add_argument("--only", default=None, metavar="NAME",
                    help="run one side workload in a loop and print its timing (for rocprofv3): "
-                        "decode_2bit_B16, decode_2bit_B1, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache")
+                        "decode_2bit_B16, decode_2bit_B1, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
     p.add_argument("--copy-calib", action="store_true",
                    help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
@@ -334,6 +334,14 @@ def _only(a, torch, K, dev):
         kk = (torch.randn((16, 8, 8192, 128), device=dev) * torch.exp(torch.randn(128, device=dev))).to(torch.float16)
         zc = KVCacheFactory.create(KVCacheConfig(method="zipcache", head_dim=128))
         fn = lambda: zc._compress(kk, True)
+        nbytes = 2 * kk.numel() * 2
+    elif name == "skvq":
+        from veloxquant_mlx_amd.quantizers.skvq import DEFAULT_ALPHA_GRID
+        kk = (torch.randn((16, 8, 8192, 128), device=dev) * torch.exp(torch.randn(128, device=dev))).to(torch.float16)
+        perm = torch.stack([torch.randperm(128, device=dev) for _ in range(8)]).to(torch.int32)
+        inv = torch.argsort(perm.long(), dim=-1).to(torch.int32)
+        out = torch.empty_like(kk)
+        fn = lambda: K.skvq_clipped_round_trip(kk, 4, 32, DEFAULT_ALPHA_GRID, perm=perm, inv=inv, out=out)
         nbytes = 2 * kk.numel() * 2
     elif name in ("quant_pack", "quant_pack_2calls", "quant_dequant"):
         k, v = _synthetic_layer(torch, 16, 8, 8192, 128, 11, dev)

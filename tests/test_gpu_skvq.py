@@ -54,6 +54,8 @@ def _bits(a):
     (1, 1, 5, 64, 8, 1, False),      # one channel per group
     (2, 2, 33, 256, 2, 256, True),   # one group per row
     (1, 2, 700, 128, 1, 64, False),
+    (2, 2, 21, 80, 4, 32, True),     # ragged last group on the 16-byte path: the order's last channel fills it
+    (1, 3, 50, 192, 2, 64, True),    # rows of a block in several heads, groups of 64
 ])
 def test_round_trip_kernel_matches_the_oracle_bit_for_bit(dtype, B, H, r, D, bits, g, with_perm):
     require_gpu()
