@@ -742,8 +742,13 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
 
     // ---- pipeline over the work units [w0, w1) on three LDS buffers: while unit w is computed
     // from registers, unit w+1 is read from its buffer, unit w+2 is unpacked into the third and
-    // unit w+3 is requested from memory.  Half of the waves unpack before they compute and half
-    // after, so that the two waves of a SIMD are not in the same phase after every barrier.
+    // unit w+3 is requested from memory.  The producer's share comes after the unit's second product
+    // (its first instructions issue while those products run); unpacking before the products in half
+    // of the waves, to put the two waves of a SIMD out of step, measured 8 % slower.
+    // The barrier between units waits for LDS only: __syncthreads() also waits for every outstanding
+    // global load, i.e. for the unit just requested, once per unit.  For the same reason nothing
+    // requested before the loop may still be pending inside it (the compiler would wait for it at
+    // the loop head, and with it for whatever was requested since).
     Stage st;
     if (w1 > w0) {
         fetch(w0, st);
@@ -757,20 +762,16 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         load_keys(0);
         load_values(0);
     }
-    const bool early = wave < PR_THREADS / 128;
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     int cur = 0;
     for (int w = w0; w < w1; ++w) {
         const int next = cur == 2 ? 0 : cur + 1, third = next == 2 ? 0 : next + 1;
-        auto produce = [&]() {
-            if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
-            if (w + 3 < w1) fetch(w + 3, st);
-        };
-        if (early) produce();
         const bool packed = w < n_punits;
         const int base = packed ? w * 32 : (w - n_punits) * 32;
         compute(next, base, packed, packed ? full_vis : full_tvis, packed ? edge_lo : edge_tlo);
-        if (!early) produce();
-        __syncthreads();
+        if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
+        if (w + 3 < w1) fetch(w + 3, st);
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         cur = next;
     }
 
