@@ -582,16 +582,16 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     int meta_group = -1;
     auto fetch = [&](int w, Stage &st) {
         if (w >= n_punits) {   // tail unit: the thread's key and value pieces travel in the value-meta slots
+            // a block-uniform base (the unit's first token) plus a 32-bit offset of the thread's own; a token
+            // past the end of the tail reads the last one instead (masked in the softmax)
             const int64_t t0 = (int64_t)(w - n_punits) * 32;
-            int64_t tok = t0 + kt;
-            if (tok >= a.n_tail) tok = 0;   // masked in the softmax
-            st.vs.u[0] = *reinterpret_cast<const uint4 *>((const u16 *)a.k_tail + tbase + tok * MF_D + 8 * kc);
+            const int last = (int)(a.n_tail - 1 - t0);   // >= 0: the unit starts inside the tail
+            const char *kt0 = (const char *)a.k_tail + (tbase + t0 * MF_D) * 2, *vt0 = (const char *)a.v_tail + (tbase + t0 * MF_D) * 2;
+            st.vs.u[0] = *reinterpret_cast<const uint4 *>(kt0 + (unsigned)((kt < last ? kt : last) * (MF_D * 2) + 16 * kc));
             // values: four channels of a token pair, so that the transposed tile is written in whole words
-            int64_t ta = t0 + 2 * tp, tb = ta + 1;
-            if (ta >= a.n_tail) ta = 0;
-            if (tb >= a.n_tail) tb = 0;
-            const uint2 va = *reinterpret_cast<const uint2 *>((const u16 *)a.v_tail + tbase + ta * MF_D + 4 * cq);
-            const uint2 vb2 = *reinterpret_cast<const uint2 *>((const u16 *)a.v_tail + tbase + tb * MF_D + 4 * cq);
+            const int ta = 2 * tp < last ? 2 * tp : last, tb = 2 * tp + 1 < last ? 2 * tp + 1 : last;
+            const uint2 va = *reinterpret_cast<const uint2 *>(vt0 + (unsigned)(ta * (MF_D * 2) + 8 * cq));
+            const uint2 vb2 = *reinterpret_cast<const uint2 *>(vt0 + (unsigned)(tb * (MF_D * 2) + 8 * cq));
             st.vz.u[0] = make_uint4(va.x, va.y, vb2.x, vb2.y);
             return;
         }
@@ -762,7 +762,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         load_keys(0);
         load_values(0);
     }
-    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    wait_global_accesses();
     int cur = 0;
     for (int w = w0; w < w1; ++w) {
         const int next = cur == 2 ? 0 : cur + 1, third = next == 2 ? 0 : next + 1;
@@ -771,7 +771,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
         compute(next, base, packed, packed ? full_vis : full_tvis, packed ? edge_lo : edge_tlo);
         if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
         if (w + 3 < w1) fetch(w + 3, st);
-        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        lds_barrier();
         cur = next;
     }
 

@@ -35,6 +35,16 @@ typedef unsigned short u16;
 
 struct bf16_t { u16 bits; };
 
+// Barrier for data that the block exchanges through LDS.  __syncthreads() is a fence as well: it also
+// waits for every outstanding global access of the wave, so a loop that requests the next step's data
+// and then meets a __syncthreads() waits for that data once per step.  This one waits for the wave's LDS
+// accesses only; global stores that other waves of the block are to read still need __syncthreads().
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+// Waits until every global access of the wave has completed.  Before a loop that uses lds_barrier():
+// what was requested before the loop would otherwise be waited for at the loop head in every iteration,
+// and with it whatever the iteration before requested.
+__device__ __forceinline__ void wait_global_accesses() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0)
+
 __device__ __forceinline__ float bf16_to_f32(u16 b) { return __uint_as_float(((uint32_t)b) << 16); }
 __device__ __forceinline__ u16 f32_to_bf16(float f) {
     uint32_t u = __float_as_uint(f);

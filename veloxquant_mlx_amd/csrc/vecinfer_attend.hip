@@ -312,6 +312,7 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
     for (int r = 0; r < RB; ++r) m_row[r] = -INFINITY;
 
     // the indices of a step are loaded one step ahead
+    wait_global_accesses();
     for (int64_t base = t_begin; base < t_end; base += LA_SUPER) {
         // ---- phase 1: scores of the wave's tiles, and their maxima per row
         float s[LA_TILES][RB], wmax[RB];
@@ -346,9 +347,9 @@ __global__ __launch_bounds__(LA_THREADS) void lut_attend_u8_kernel(vq_lut_attend
             wmax[r] = wave_max(wmax[r]);
             if (lane == 0) s_max[wave][r] = wmax[r];
         }
-        __syncthreads();
+        lds_barrier();   // (LDS only: the indices requested above stay in flight)
         raise_references<RB>(s_max, m_row, hist, NS * LA_ROW, tid);
-        __syncthreads();   // s_max is free again; a rescaled histogram is in place
+        lds_barrier();   // s_max is free again; a rescaled histogram is in place
         // ---- phase 2: weights into the histogram
 #pragma unroll
         for (int T = 0; T < LA_TILES; ++T) {
