@@ -46,6 +46,24 @@ __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
+// The same with one limit for all eight codes: the largest distance from a whole number is compared once
+// (a NaN quotient is neither close nor far, as above).
+__device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
+                                             const float (&rs)[8], const float (&nb)[8], float tie, float levels,
+                                             bool redo, float (&q)[8]) {
+    float far = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
+        const float r = rintf(q0);
+        far = fmaxf(far, fabsf(q0 - r));
+        q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels);
+    }
+    if (__any(redo | (far >= tie))) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
+    }
+}
 __device__ __forceinline__ float tie_limit(float levels, float nb) {
     return 0.5f - (5e-7f * (levels + 1.0f) + 2e-7f * fabsf(nb));
 }
@@ -79,6 +97,30 @@ __device__ __forceinline__ float recon(float q, float sc, float mn) {
 }
 __device__ __forceinline__ float group_scale(float mn, float mx, float levels, float eps) {
     return fmaxf(__fdiv_rn(__fsub_rn(mx, mn), levels), eps);
+}
+// The same quotient in three operations where that is proved exact.  For levels = 2^b - 1, b = 1 .. 8, and
+// r = 1 / levels rounded to float, q0 = x r, e = fma(-q0, levels, x), q = fma(e, r, q0) is the correctly
+// rounded x / levels for every finite non-negative float x, subnormal quotients included: compared with the
+// division over all 2 139 095 040 of them for each of the eight level counts on a CPU
+// (tests/exact_level_division.c; the test suite runs a sample).  inf and NaN pass through as the division
+// passes them.  `inv` is r, or 0 for any other level count (then the division is used).
+struct LevelDiv { float levels, inv; };
+__device__ __forceinline__ LevelDiv level_div(float levels) {
+    const uint32_t n = (uint32_t)levels + 1u;
+    const bool proved = (float)(n - 1u) == levels && n >= 2u && n <= 256u && (n & (n - 1u)) == 0u;
+    return LevelDiv{levels, proved ? __fdiv_rn(1.0f, levels) : 0.0f};
+}
+__device__ __forceinline__ float group_scale(float mn, float mx, LevelDiv d, float eps) {
+    const float x = __fsub_rn(mx, mn);
+    float q;
+    if (d.inv != 0.0f) {   // uniform
+        const float q0 = __fmul_rn(x, d.inv);
+        q = __builtin_fmaf(__builtin_fmaf(-q0, d.levels, x), d.inv, q0);
+        q = x < INFINITY ? q : x;
+    } else {
+        q = __fdiv_rn(x, d.levels);
+    }
+    return fmaxf(q, eps);
 }
 
 template <typename T> __device__ __forceinline__ void load8(const T *p, float (&v)[8]);
@@ -504,6 +546,7 @@ __global__ __launch_bounds__(256) void kivi_value_roundtrip_kernel(const T *__re
     if (t0 >= S) return;
     const T *xb = x + bh * x_stride_bh + t0 * D + 8 * o;
     T *ob = out + (bh * S + t0) * D + 8 * o;
+    const LevelDiv ld = level_div(levels);
     Raw8<T> v[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i)
@@ -514,12 +557,12 @@ __global__ __launch_bounds__(256) void kivi_value_roundtrip_kernel(const T *__re
         float mn, mx;
         v[i].span(mn, mx);
         group_span<GL>(mn, mx);
-        const float sc = group_scale(mn, mx, levels, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
-        float x8[8], q[8], y[8], mn8[8], sc8[8], rs8[8], nb8[8], tl8[8];
+        const float sc = group_scale(mn, mx, ld, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
+        float x8[8], q[8], y[8], mn8[8], sc8[8], rs8[8], nb8[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; tl8[c] = tl; }
+        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; }
         v[i].floats(x8);
-        quant_codes8(x8, mn8, sc8, rs8, nb8, tl8, levels, !(rs < 1e30f), q);
+        quant_codes8(x8, mn8, sc8, rs8, nb8, tl, levels, !(rs < 1e30f), q);
 #pragma unroll
         for (int c = 0; c < 8; ++c) y[c] = recon(q[c], sc, mn);
         if (t0 + i < S) store8<T>(ob + (int64_t)i * D, y);
@@ -536,6 +579,7 @@ __device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T
     const int64_t t0 = ((int64_t)bx * VP_STRETCHES + (tid >> 4)) * PER;   // the stretch's first token
     if (t0 >= S) return;                                                  // S is a multiple of PER: whole rows of 16 lanes leave
     const T *xb = x + bh * x_stride_bh + t0 * D + 8 * o;
+    const LevelDiv ld = level_div(levels);
     Raw8<T> v[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) v[i].load(xb + (int64_t)i * D);
@@ -547,14 +591,14 @@ __device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T
         float mn, mx;
         v[i].span(mn, mx);
         group_span<GL>(mn, mx);
-        const float sc = group_scale(mn, mx, levels, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
+        const float sc = group_scale(mn, mx, ld, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
         scv[i] = sc;
         mnv[i] = mn;
-        float x8[8], q[8], mn8[8], sc8[8], rs8[8], nb8[8], tl8[8];
+        float x8[8], q[8], mn8[8], sc8[8], rs8[8], nb8[8];
 #pragma unroll
-        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; tl8[c] = tl; }
+        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; }
         v[i].floats(x8);
-        quant_codes8(x8, mn8, sc8, rs8, nb8, tl8, levels, !(rs < 1e30f), q);
+        quant_codes8(x8, mn8, sc8, rs8, nb8, tl, levels, !(rs < 1e30f), q);
         // code of token i at bits [BITS * i, BITS * (i + 1)): two exact float sums of 16 bits each
         const float w = (float)(1u << (BITS * (i % HALF)));
 #pragma unroll
@@ -646,20 +690,19 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
             v[i].fold(acc);
         }
     QuadFold<T>::run(acc);
-    float mn[8], mx[8], sc[8], rs[8], nb[8], tie_lo[8];
+    float mn[8], mx[8], sc[8], rs[8], nb[8];
     Raw8<T>::result(acc, mn, mx);
+    const LevelDiv ld = level_div(levels);
     bool redo = false;
     float tie_all = 0.5f;   // one limit for the lane's 8 channels, the tightest: a few more rows take the division
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-        sc[c] = group_scale(mn[c], mx[c], levels, eps);
+        sc[c] = group_scale(mn[c], mx[c], ld, eps);
         rs[c] = fast_rcp(sc[c]);
         nb[c] = -mn[c] * rs[c];
         tie_all = fminf(tie_all, tie_limit(levels, nb[c]));
         redo |= !(rs[c] < 1e30f);
     }
-#pragma unroll
-    for (int c = 0; c < 8; ++c) tie_lo[c] = tie_all;
     if (MODE == 1 && tq == 0) {
         const int64_t gdst = dst_tok0 / G + gk, gcap = (cap_tokens + G - 1) / G;
         store_meta8<M>(scale + (bh * gcap + gdst) * D + 8 * o, sc);
@@ -675,7 +718,7 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
 #pragma unroll
             for (int c = 0; c < 8; ++c) x8[c] = mn[c];
         }
-        quant_codes8(x8, mn, sc, rs, nb, tie_lo, levels, redo, q);
+        quant_codes8(x8, mn, sc, rs, nb, tie_all, levels, redo, q);
         if (MODE == 0) {
             if (valid) {
                 float y[8];
