@@ -321,7 +321,7 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
         float a = INFINITY, b = -INFINITY;
 #pragma unroll
         for (int j = 0; j < RPP; ++j) { a = fminf(a, s_mn[j][ch]); b = fmaxf(b, s_mx[j][ch]); }
-        const float scv = group_scale(a, b, levels, eps);
+        const float scv = group_scale(a, b, level_div(levels), eps);
         const float rsv = fast_rcp(scv);
         s_par[0][ch] = a;
         s_par[1][ch] = scv;
@@ -329,15 +329,16 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
         s_par[3][ch] = -a * rsv;
     }
     __syncthreads();
-    float sc[8], rs[8], nb[8], tie_lo[8];
+    float sc[8], rs[8], nb[8];
     auto row8 = [&](int k, float (&d)[8]) {
         const float4 lo = *reinterpret_cast<const float4 *>(&s_par[k][8 * o]), hi = *reinterpret_cast<const float4 *>(&s_par[k][8 * o + 4]);
         d[0] = lo.x; d[1] = lo.y; d[2] = lo.z; d[3] = lo.w; d[4] = hi.x; d[5] = hi.y; d[6] = hi.z; d[7] = hi.w;
     };
     row8(0, mn); row8(1, sc); row8(2, rs); row8(3, nb);
     bool redo = false;
+    float tie_all = 0.5f;   // the tightest of the eight channels' limits
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { tie_lo[i] = tie_limit(levels, nb[i]); redo |= !(rs[i] < 1e30f); }
+    for (int i = 0; i < 8; ++i) { tie_all = fminf(tie_all, tie_limit(levels, nb[i])); redo |= !(rs[i] < 1e30f); }
     if (MODE == 1 && r == 0) {
         int64_t gdst = dst_tok0 / group + gk;
         int64_t gcap = (cap_tokens + group - 1) / group;
@@ -358,7 +359,7 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
 #pragma unroll
             for (int i = 0; i < 8; ++i) x8[i] = mn[i];
         }
-        quant_codes8(x8, mn, sc, rs, nb, tie_lo, levels, redo, q);
+        quant_codes8(x8, mn, sc, rs, nb, tie_all, levels, redo, q);
         if (MODE == 0) {
             if (valid) {
                 float y[8];
@@ -426,7 +427,7 @@ __device__ __forceinline__ void kivi_value_tile_body(int bx, int64_t bh,
             mn = fminf(mn, __shfl_xor(mn, off));
             mx = fmaxf(mx, __shfl_xor(mx, off));
         }
-        const float sc = group_scale(mn, mx, levels, eps);
+        const float sc = group_scale(mn, mx, level_div(levels), eps);
         if (MODE != 0 && valid[j] && (o % GL) == 0) {
             int gv = o / GL;
             if (MODE == 2 && GV <= MAXGV) {
@@ -442,15 +443,15 @@ __device__ __forceinline__ void kivi_value_tile_body(int bx, int64_t bh,
         float q[8];
         {
             const float rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
-            float x8[8], mn8[8], sc8[8], rs8[8], nb8[8], tl8[8];
+            float x8[8], mn8[8], sc8[8], rs8[8], nb8[8];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) { mn8[i] = mn; sc8[i] = sc; rs8[i] = rs; nb8[i] = nb; tl8[i] = tl; }
+            for (int i = 0; i < 8; ++i) { mn8[i] = mn; sc8[i] = sc; rs8[i] = rs; nb8[i] = nb; }
             if (valid[j]) v[j].floats(x8);
             else {   // keep the arithmetic defined; the lane's results are not stored
 #pragma unroll
                 for (int i = 0; i < 8; ++i) x8[i] = 0.0f;
             }
-            quant_codes8(x8, mn8, sc8, rs8, nb8, tl8, levels, !(rs < 1e30f), q);
+            quant_codes8(x8, mn8, sc8, rs8, nb8, tl, levels, !(rs < 1e30f), q);
             if (!valid[j]) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) q[i] = 0.0f;
