@@ -64,6 +64,22 @@ int vq_device_count(void);
 int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D,
                           int axis, int group, int levels, float eps, void *stream);
 
+/* The same round trip along the token axis with a level count per channel: channel c of slab bh has
+ * levels_hi levels where hi_mask[bh * D + c] != 0 and levels_lo otherwise.  One launch for
+ * quantize_mixed_channels (veloxquant_mlx/quantizers/kitty.py:138-169), which forms the hi-bit and the
+ * lo-bit reconstruction of the whole tensor and selects per channel.  head_dim 128, groups of 32 or 64
+ * tokens; x/out [BH, S, 128] contiguous and 16-byte aligned, hi_mask [BH, 128] bytes, 8-byte aligned. */
+int vq_kivi_quant_dequant_mixed(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int group,
+                                int levels_lo, int levels_hi, const uint8_t *hi_mask, float eps, void *stream);
+
+/* Per-channel sums over the tokens of x [N, S, D] (slab stride x_stride_n elements), accumulated in double:
+ * partial[((n * chunks + k) * 2 + 0) * D + c] = sum, [... + 1 ...] = sum of squares of channel c over the
+ * k-th of `chunks` stretches of tokens; the caller adds the chunks.  The population variance Kitty ranks
+ * channels by (mx.var over the float32 copy, veloxquant_mlx/quantizers/kitty.py:44-67,
+ * veloxquant_mlx/cache/kitty_cache.py:96-104) in one pass over the stored rows.  head_dim 64 / 128 / 256. */
+int vq_channel_moments(const void *x, int dtype, int64_t N, int64_t S, int64_t D, int64_t x_stride_n, double *partial,
+                       int chunks, void *stream);
+
 /* out[r] = L2 norm of row r of x [n_rows, D], float32 arithmetic (head_dim 64 / 128 / 256).  The salience
  * signal of ZipCacheKVCache (mx.linalg.norm over the channels of the float32 copy,
  * veloxquant_mlx/cache/zipcache_cache.py:176-180) without materialising that copy. */

@@ -7,6 +7,7 @@ import torch
 
 from oracle import kitty as okt
 from tests._gpu import gpu, host, require_gpu, to_dev
+from veloxquant_mlx_amd import kernels as K
 from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
 from veloxquant_mlx_amd.cache.kitty_cache import KittyKVCache
 from veloxquant_mlx_amd.core.exceptions import QuantizerConfigError
@@ -103,3 +104,41 @@ def test_configuration():
     for bad in (1.5, -0.1):
         with pytest.raises(QuantizerConfigError, match="kitty_hi_fraction"):
             KittyKVCache(KVCacheConfig(method="kitty", head_dim=64, kitty_hi_fraction=bad))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("g,S", [(32, 200), (64, 192), (32, 31)])
+def test_one_launch_mixed_round_trip_equals_two_round_trips_and_a_select(g, S):
+    """``vq_kivi_quant_dequant_mixed`` (a level count per channel) against what it replaces: the hi-bit and the lo-bit
+    round trip of the whole tensor and a per-channel select (kitty.py:138-169), bit for bit, with ragged last groups,
+    for the bit pairs the cache uses and one whose level counts take the plain division."""
+    require_gpu()
+    rng = np.random.default_rng(g + S)
+    N, D = 5, 128
+    x = (rng.standard_normal((N, S, D)) * np.exp(rng.standard_normal(D))).astype(np.float16)
+    mask = rng.random((N, D)) < 0.3
+    mask[0] = False
+    mask[1] = True
+    xt, mt = to_dev(x), to_dev(mask)
+    for lo, hi in ((3, 15), (1, 255), (5, 10)):
+        got = K.kivi_group_quant_dequant_mixed(xt, mt, g, lo, hi)
+        want = torch.where(mt[:, None, :], K.kivi_group_quant_dequant(xt, -2, g, hi), K.kivi_group_quant_dequant(xt, -2, g, lo))
+        assert torch.equal(got, want), (lo, hi)
+    with pytest.raises(Exception):
+        K.kivi_group_quant_dequant_mixed(xt, mt, 128, 3, 15)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("N,S,D", [(3, 1000, 128), (2, 77, 64), (1, 5000, 256)])
+def test_channel_variance_in_one_pass(dtype, N, S, D):
+    """``vq_channel_moments`` against numpy's float64 variance of the same values, with a large common offset in some
+    channels (where a float32 sum of squares would lose the variance)."""
+    require_gpu()
+    rng = np.random.default_rng(N + S + D)
+    x = rng.standard_normal((N, S, D)) * np.exp(rng.standard_normal(D))
+    x[..., ::7] += 40.0
+    xt = to_dev(x.astype(np.float32)).to(dtype)
+    want = np.var(xt.double().cpu().numpy(), axis=1)
+    got = host(K.channel_variance(xt)).astype(np.float64)
+    np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-9)

@@ -16,7 +16,8 @@ import torch
 
 from .. import kernels as K
 from ..core.exceptions import QuantizerConfigError
-from ..quantizers.kitty import compute_running_variance, hi_mask_from_variance_batched, quantize_mixed_channels_batched
+from ..quantizers.kitty import (channel_variance_batched, compute_running_variance, hi_mask_from_variance_batched,
+                                quantize_mixed_channels_batched)
 from ._fp16_cache import FP16KVCache
 
 
@@ -45,7 +46,7 @@ class KittyKVCache(FP16KVCache):
         B, H, S, D = keys.shape
         flat = keys.reshape(B * H, S, D)
         if self._n_keys == 0:
-            variance = torch.var(flat.float(), dim=1, unbiased=False)
+            variance = channel_variance_batched(flat)
         else:
             var_h = compute_running_variance(self._key_sum, self._key_sq_sum, self._n_keys)
             variance = var_h[None].expand(B, H, D).reshape(B * H, D)

@@ -64,6 +64,23 @@ __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
+// The same with a level count per code (channels of different bit widths in one row).
+__device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
+                                             const float (&rs)[8], const float (&nb)[8], float tie,
+                                             const float (&levels)[8], bool redo, float (&q)[8]) {
+    float far = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
+        const float r = rintf(q0);
+        far = fmaxf(far, fabsf(q0 - r));
+        q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels[i]);
+    }
+    if (__any(redo | (far >= tie))) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels[i]);
+    }
+}
 __device__ __forceinline__ float tie_limit(float levels, float nb) {
     return 0.5f - (5e-7f * (levels + 1.0f) + 2e-7f * fabsf(nb));
 }
@@ -670,11 +687,15 @@ template <> struct QuadFold<f16> {
 };
 constexpr int KQ_WAVES = 4;   // groups per block
 
-template <typename T, typename M, int MODE, int TPL>
+// MIXED (round trip only): channel c of (sequence, head) bh has `levels_hi` levels where hi_mask[bh * 128 + c] is
+// set and `levels` otherwise (Kitty's channel-wise mixed precision, veloxquant_mlx/quantizers/kitty.py:138-169,
+// which forms both reconstructions of the whole tensor and selects per channel).
+template <typename T, typename M, int MODE, int TPL, bool MIXED = false>
 __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *__restrict__ x, T *__restrict__ out, int64_t S,
                                                    int64_t x_stride_bh, float levels, float eps, int bits,
                                                    uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
-                                                   int64_t cap_tokens, int64_t dst_tok0, int W) {
+                                                   int64_t cap_tokens, int64_t dst_tok0, int W,
+                                                   const uint8_t *__restrict__ hi_mask = nullptr, float levels_hi = 0.f) {
     constexpr int D = 128, G = 4 * TPL;
     const int lane = threadIdx.x & 63, o = lane >> 2, tq = lane & 3;
     const int64_t s0 = (int64_t)gk * G;
@@ -694,14 +715,24 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
     float mn[8], mx[8], sc[8], rs[8], nb[8];
     Raw8<T>::result(acc, mn, mx);
     const LevelDiv ld = level_div(levels);
+    LevelDiv ldh = ld;
+    uint2 hi8 = make_uint2(0u, 0u);   // MIXED: the lane's eight mask bytes
+    if constexpr (MIXED) {
+        ldh = level_div(levels_hi);
+        hi8 = *reinterpret_cast<const uint2 *>(hi_mask + bh * D + 8 * o);
+    }
+    float lv[8];
     bool redo = false;
     float tie_all = 0.5f;   // one limit for the lane's 8 channels, the tightest: a few more rows take the division
 #pragma unroll
     for (int c = 0; c < 8; ++c) {
-        sc[c] = group_scale(mn[c], mx[c], ld, eps);
+        const bool hi = MIXED && (((c < 4 ? hi8.x : hi8.y) >> (8 * (c & 3))) & 0xFFu) != 0u;
+        const LevelDiv d = hi ? ldh : ld;
+        lv[c] = d.levels;
+        sc[c] = group_scale(mn[c], mx[c], d, eps);
         rs[c] = fast_rcp(sc[c]);
         nb[c] = -mn[c] * rs[c];
-        tie_all = fminf(tie_all, tie_limit(levels, nb[c]));
+        tie_all = fminf(tie_all, tie_limit(lv[c], nb[c]));
         redo |= !(rs[c] < 1e30f);
     }
     if (MODE == 1 && tq == 0) {
@@ -719,7 +750,8 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
 #pragma unroll
             for (int c = 0; c < 8; ++c) x8[c] = mn[c];
         }
-        quant_codes8(x8, mn, sc, rs, nb, tie_all, levels, redo, q);
+        if constexpr (MIXED) quant_codes8(x8, mn, sc, rs, nb, tie_all, lv, redo, q);
+        else quant_codes8(x8, mn, sc, rs, nb, tie_all, levels, redo, q);
         if (MODE == 0) {
             if (valid) {
                 float y[8];
@@ -758,6 +790,55 @@ __global__ __launch_bounds__(64 * KQ_WAVES) void kivi_key_quad_kernel(
 struct PackDst { uint32_t *packed; void *scale, *zero; };
 // the same for head_dim 128, groups of 32 or 64, 2 or 4 bits, token-packed values: the quad-layout key body and the
 // word-owning value body, neither of which uses block-shared memory
+template <typename T, int TPL>
+__global__ __launch_bounds__(64 * KQ_WAVES) void kivi_key_quad_mixed_kernel(const T *__restrict__ x, T *__restrict__ out, int64_t S,
+                                                                           int64_t x_stride_bh, float levels_lo, float levels_hi,
+                                                                           const uint8_t *__restrict__ hi_mask, float eps) {
+    kivi_key_quad_body<T, float, 0, TPL, true>((int)blockIdx.x * KQ_WAVES + (int)(threadIdx.x >> 6), (int64_t)blockIdx.y, x, out, S,
+                                               x_stride_bh, levels_lo, eps, 0, nullptr, nullptr, nullptr, 0, 0, 0, hi_mask, levels_hi);
+}
+
+// Sum and sum of squares over the tokens of every channel of x [N, S, D] in double precision: block (chunk, n)
+// takes a stretch of tokens, a thread eight channels of every (256 / LPR)-th token of it, and writes
+// partial[((n * chunks + chunk) * 2 + which) * D + channel]; the few partials of a channel are added by the caller
+// (in a fixed order: the result does not depend on scheduling).
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void channel_moments_kernel(const T *__restrict__ x, int64_t S, int64_t x_stride_n,
+                                                              double *__restrict__ partial, int64_t tokens_per_chunk) {
+    constexpr int D = LPR * 8, RPP = 256 / LPR, RPW = 64 / LPR;   // rows per pass of the block / of a wave
+    __shared__ double s_part[4][2][D];
+    const int tid = threadIdx.x, o = tid % LPR, r = tid / LPR, wave = tid >> 6;
+    const int64_t n = blockIdx.y, t_begin = (int64_t)blockIdx.x * tokens_per_chunk;
+    const int64_t t_end = t_begin + tokens_per_chunk < S ? t_begin + tokens_per_chunk : S;
+    double sum[8], sq[8];
+#pragma unroll
+    for (int c = 0; c < 8; ++c) { sum[c] = 0.0; sq[c] = 0.0; }
+    const T *xb = x + n * x_stride_n + 8 * o;
+    for (int64_t t = t_begin + r; t < t_end; t += RPP) {
+        float v[8];
+        load8<T>(xb + t * D, v);
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { sum[c] += (double)v[c]; sq[c] += (double)v[c] * (double)v[c]; }
+    }
+    // rows of a wave sit LPR lanes apart
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+#pragma unroll
+        for (int off = LPR; off < 64; off <<= 1) { sum[c] += __shfl_xor(sum[c], off); sq[c] += __shfl_xor(sq[c], off); }
+    }
+    if ((tid & 63) < LPR) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { s_part[wave][0][8 * o + c] = sum[c]; s_part[wave][1][8 * o + c] = sq[c]; }
+    }
+    __syncthreads();
+    (void)RPW;
+    for (int e = tid; e < 2 * D; e += 256) {
+        const int which = e / D, ch = e % D;
+        const double total = ((s_part[0][which][ch] + s_part[1][which][ch]) + s_part[2][which][ch]) + s_part[3][which][ch];
+        partial[((n * gridDim.x + blockIdx.x) * 2 + which) * D + ch] = total;
+    }
+}
+
 template <typename T, typename M, int BITS, int TPL>
 __global__ __launch_bounds__(256) void kivi_kv_pack_kernel(
     const T *__restrict__ k, const T *__restrict__ v, int64_t S, int64_t x_stride_bh, float levels, float eps, PackDst kd,
@@ -1282,6 +1363,56 @@ extern "C" int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_
                                (const T *)x, (T *)out, BH, S, D, axis, group, (float)levels, eps);
     });
     VQ_HIP_CHECK_LAUNCH("vq_kivi_quant_dequant");
+    return VQ_OK;
+}
+
+extern "C" int vq_kivi_quant_dequant_mixed(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int group,
+                                           int levels_lo, int levels_hi, const uint8_t *hi_mask, float eps, void *stream) {
+    const char *fn = "vq_kivi_quant_dequant_mixed";
+    VQ_REQUIRE(D == 128 && (group == 32 || group == 64), VQ_ERR_UNSUPPORTED,
+               "%s: head_dim 128 and groups of 32 or 64 tokens only (got head_dim %lld, group %d)", fn, (long long)D, group);
+    VQ_REQUIRE(levels_lo >= 1 && levels_hi >= 1, VQ_ERR_INVALID, "%s: level counts must be >= 1, got %d and %d", fn, levels_lo, levels_hi);
+    VQ_REQUIRE(BH >= 0 && S >= 0, VQ_ERR_INVALID, "%s: negative dimension", fn);
+    VQ_REQUIRE(is_float_tag(dtype), VQ_ERR_INVALID, "%s: unsupported dtype tag %d", fn, dtype);
+    if (BH * S == 0) return VQ_OK;
+    VQ_REQUIRE(x && out && hi_mask, VQ_ERR_INVALID, "%s: null pointer", fn);
+    VQ_REQUIRE(aligned16(x) && aligned16(out) && ((uintptr_t)hi_mask % 8) == 0, VQ_ERR_UNSUPPORTED,
+               "%s: x and out must be 16-byte aligned, hi_mask 8-byte aligned", fn);
+    VQ_REQUIRE(BH <= 65535, VQ_ERR_UNSUPPORTED, "%s: at most 65535 (sequence, head) pairs, got %lld", fn, (long long)BH);
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)cdiv(cdiv(S, group), KQ_WAVES), (unsigned)BH);
+    VQ_DISPATCH_FLOAT(dtype, T, {
+        if (group == 32)
+            hipLaunchKernelGGL((kivi_key_quad_mixed_kernel<T, 8>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D,
+                               (float)levels_lo, (float)levels_hi, hi_mask, eps);
+        else
+            hipLaunchKernelGGL((kivi_key_quad_mixed_kernel<T, 16>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D,
+                               (float)levels_lo, (float)levels_hi, hi_mask, eps);
+    });
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_channel_moments(const void *x, int dtype, int64_t N, int64_t S, int64_t D, int64_t x_stride_n, double *partial,
+                                  int chunks, void *stream) {
+    const char *fn = "vq_channel_moments";
+    VQ_REQUIRE(D == 64 || D == 128 || D == 256, VQ_ERR_UNSUPPORTED, "%s: head_dim 64, 128 or 256, got %lld", fn, (long long)D);
+    VQ_REQUIRE(N >= 0 && S >= 0 && chunks >= 1 && chunks <= 65535, VQ_ERR_INVALID, "%s: bad dimensions", fn);
+    VQ_REQUIRE(is_float_tag(dtype), VQ_ERR_INVALID, "%s: unsupported dtype tag %d", fn, dtype);
+    if (N == 0) return VQ_OK;
+    VQ_REQUIRE(x && partial, VQ_ERR_INVALID, "%s: null pointer", fn);
+    VQ_REQUIRE(aligned16(x) && x_stride_n % 8 == 0 && x_stride_n >= S * D, VQ_ERR_UNSUPPORTED,
+               "%s: rows must be 16-byte aligned and x_stride_n >= S * D", fn);
+    VQ_REQUIRE(N <= 65535, VQ_ERR_UNSUPPORTED, "%s: at most 65535 slabs, got %lld", fn, (long long)N);
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t per = cdiv(S > 0 ? S : 1, chunks);
+    const dim3 grid((unsigned)chunks, (unsigned)N);
+    VQ_DISPATCH_FLOAT(dtype, T, {
+        if (D == 64) hipLaunchKernelGGL((channel_moments_kernel<T, 8>), grid, dim3(256), 0, st, (const T *)x, S, x_stride_n, partial, per);
+        else if (D == 128) hipLaunchKernelGGL((channel_moments_kernel<T, 16>), grid, dim3(256), 0, st, (const T *)x, S, x_stride_n, partial, per);
+        else hipLaunchKernelGGL((channel_moments_kernel<T, 32>), grid, dim3(256), 0, st, (const T *)x, S, x_stride_n, partial, per);
+    });
+    VQ_HIP_CHECK_LAUNCH(fn);
     return VQ_OK;
 }
 

@@ -169,6 +169,46 @@ def row_norms(x: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def channel_variance(x: torch.Tensor) -> torch.Tensor:
+    """Population variance over the tokens of every channel of ``x [N, S, D]`` (D in 64 / 128 / 256), float32
+    ``[N, D]``: one pass over the stored rows with double accumulators (``mx.var`` of the float32 copy in the
+    reference, veloxquant_mlx/quantizers/kitty.py:44-67)."""
+    name = "channel_variance"
+    tag = _ftag(name, x)
+    _need_gpu(name, x)
+    if x.ndim != 3:
+        raise ValueError(f"{name}: x must be [N, S, D], got {tuple(x.shape)}")
+    x = x.contiguous()
+    N, S, D = x.shape
+    if S == 0:
+        return torch.full((N, D), float("nan"), dtype=torch.float32, device=x.device)
+    chunks = max(1, min(64, S // 256))
+    partial = torch.empty((N, chunks, 2, D), dtype=torch.float64, device=x.device)
+    _lib.check(_lib.load().vq_channel_moments(x.data_ptr(), tag, N, S, D, S * D, partial.data_ptr(), chunks, _stream(x)))
+    total = partial.sum(dim=1)
+    mean = total[:, 0] / S
+    return torch.clamp(total[:, 1] / S - mean * mean, min=0.0).to(torch.float32)
+
+
+def kivi_group_quant_dequant_mixed(x: torch.Tensor, hi_mask: torch.Tensor, group_size: int, levels_lo: int, levels_hi: int,
+                                   eps: float = 1e-8) -> torch.Tensor:
+    """Token-axis round trip of ``x [N, S, 128]`` with ``levels_hi`` levels in the channels where ``hi_mask [N, 128]``
+    (bool) is set and ``levels_lo`` in the others, in one launch (``quantize_mixed_channels``,
+    veloxquant_mlx/quantizers/kitty.py:138-169).  Groups of 32 or 64 tokens."""
+    name = "kivi_group_quant_dequant_mixed"
+    tag = _ftag(name, x)
+    _need_gpu(name, x)
+    if x.ndim != 3 or tuple(hi_mask.shape) != (x.shape[0], x.shape[2]) or hi_mask.dtype != torch.bool:
+        raise ValueError(f"{name}: x [N, S, D] and a bool hi_mask [N, D], got {tuple(x.shape)} and {tuple(hi_mask.shape)} {hi_mask.dtype}")
+    x = x.contiguous()
+    mask = hi_mask.contiguous()
+    N, S, D = x.shape
+    out = torch.empty_like(x)
+    _lib.check(_lib.load().vq_kivi_quant_dequant_mixed(x.data_ptr(), out.data_ptr(), tag, N, S, D, int(group_size), int(levels_lo),
+                                                       int(levels_hi), mask.data_ptr(), float(eps), _stream(x)))
+    return out
+
+
 def zip_route(norms: torch.Tensor, n_hi: int) -> torch.Tensor:
     """int32 ``[BH, S]`` routing order of a salience split of float32 ``norms [BH, S]``: the rows outside the
     ``n_hi`` largest norms in their own order, then the ``n_hi`` largest in theirs, later rows first among equal norms
@@ -1005,7 +1045,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
+    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",

@@ -1,9 +1,10 @@
 """Kitty: channel-wise mixed-precision key quantisation, on the KIVI group kernel.
 
-Mirrors veloxquant_mlx/quantizers/kitty.py:44-190.  The two reconstructions (``hi_bit`` and
-``lo_bit``) are two launches of the key-axis group round trip (``vq_kivi_quant_dequant``, the
-kernel behind ``KIVIKVCache``) and the per-channel choice between them is one select; the
-ranking (a variance and two argsorts over ``D`` channels) is host-level torch on the device.
+Mirrors veloxquant_mlx/quantizers/kitty.py:44-190.  At head_dim 128 with groups of 32 or 64 tokens the mixed
+reconstruction is one launch of the key-axis group round trip with a level count per channel
+(``vq_kivi_quant_dequant_mixed``) and the variance the channels are ranked by one pass over the stored rows
+(``vq_channel_moments``); other shapes take two launches of ``vq_kivi_quant_dequant`` and a select, and
+``torch.var``.  The ranking itself (two argsorts over ``D`` channels) is host-level torch on the device.
 """
 
 from __future__ import annotations
@@ -42,9 +43,21 @@ def quantize_mixed_channels_batched(keys: torch.Tensor, hi_mask: torch.Tensor, h
                                     group_size: int = 32) -> torch.Tensor:
     """``keys [N, S, D]``, ``hi_mask [N, D]`` -> float16 reconstruction, hi-bit where the mask is set
     (kitty.py:138-169)."""
+    if keys.dtype == torch.float16 and keys.shape[-1] == 128 and group_size in (32, 64):
+        # one launch with a level count per channel: the same codes as the two whole-tensor round trips
+        # and the select below, which stay for the other shapes
+        return K.kivi_group_quant_dequant_mixed(keys, hi_mask, group_size, (1 << lo_bit) - 1, (1 << hi_bit) - 1)
     recon_hi = _group_round_trip_fp16(keys, hi_bit, group_size)
     recon_lo = _group_round_trip_fp16(keys, lo_bit, group_size)
     return torch.where(hi_mask[:, None, :], recon_hi, recon_lo)
+
+
+def channel_variance_batched(keys: torch.Tensor) -> torch.Tensor:
+    """``keys [N, S, D]`` -> float32 ``[N, D]`` population variance over the tokens (kitty_cache.py:96-104):
+    one pass over the stored rows where the kernel covers the shape, ``torch.var`` of the float32 copy otherwise."""
+    if keys.shape[-1] in (64, 128, 256) and keys.shape[1] > 0 and keys.dtype in (torch.float16, torch.bfloat16, torch.float32):
+        return K.channel_variance(keys)
+    return torch.var(keys.float(), dim=1, unbiased=False)
 
 
 def quantize_mixed_channels(keys: torch.Tensor, hi_indices, lo_indices, hi_bit: int = 4, lo_bit: int = 2,
@@ -70,4 +83,4 @@ def compute_running_variance(key_sum: torch.Tensor, key_sq_sum: torch.Tensor, n:
 
 
 __all__ = ["rank_channels_by_sensitivity", "quantize_mixed_channels", "compute_running_variance",
-           "hi_mask_from_variance_batched", "quantize_mixed_channels_batched"]
+           "hi_mask_from_variance_batched", "quantize_mixed_channels_batched", "channel_variance_batched"]
