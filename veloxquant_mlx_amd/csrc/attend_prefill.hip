@@ -499,7 +499,28 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = lane & 15, blk = lane >> 4;
-    const int64_t bh = blockIdx.y;
+    // Which (row tile, (sequence, kv head), run) this block is.  Workgroups go to the eight XCDs in turn by
+    // their linear number, and every XCD has its own L2: with the launch's own numbering the row tiles and runs
+    // of one kv head land on all eight, and each fetches that head's keys and values from HBM for itself (68 MB
+    // per launch at config 4 for 15 MB of input).  The blocks are renumbered so that a head's tiles and runs share
+    // an XCD (a multiple of eight heads) or 8 / heads of them (1, 2 or 4 heads); other counts keep the launch's
+    // numbering.
+    unsigned tile_x = blockIdx.x, bh_y = blockIdx.y, run_z = blockIdx.z;
+    if (gridDim.y % 8 == 0 || 8 % gridDim.y == 0) {
+        const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const unsigned per_head = gridDim.x * gridDim.z, xcd = lin % 8, slot = lin / 8;
+        unsigned within;
+        if (gridDim.y % 8 == 0) {
+            bh_y = xcd + 8 * (slot / per_head);
+            within = slot % per_head;
+        } else {
+            bh_y = xcd % gridDim.y;
+            within = xcd / gridDim.y + (8 / gridDim.y) * slot;
+        }
+        tile_x = within % gridDim.x;
+        run_z = within / gridDim.x;
+    }
+    const int64_t bh = bh_y;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
     take_sequence_lengths(a, b);
     const int R = (int)(a.Hq / a.Hkv);
@@ -507,7 +528,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const float c = a.scale * LOG2E;
     const u32 magic = vreg_const(Magic<BITS>::bits);
     // under a causal mask the last tiles see the most tokens: they are started first
-    const int pos0 = (int)(a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x) * qp;
+    const int pos0 = (int)(a.causal ? gridDim.x - 1 - tile_x : tile_x) * qp;
     const int64_t n_total = a.n_packed + a.n_tail;
     auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
 
@@ -549,7 +570,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int n_punits = (max_vis + 31) / 32;
     const int n_tunits = (max_tvis + 31) / 32;
     const int n_work = n_punits + n_tunits;
-    const int nsplit = (int)gridDim.z, sp = (int)blockIdx.z;
+    const int nsplit = (int)gridDim.z, sp = (int)run_z;
     // units below the window of the block's first row are seen by none of its rows
     const int64_t first_blk = window_first(a, n_total, pos0);
     const int w_lo = first_blk < a.n_packed ? (int)(first_blk / 32) : n_punits + (int)((first_blk - a.n_packed) / 32);
