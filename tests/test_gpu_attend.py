@@ -199,6 +199,32 @@ def test_flash_prefill_large_logits_bf16_and_future_keys():
     assert torch.equal(a[:, :, :-1], b[:, :, :-1]) and not torch.equal(a[:, :, -1], b[:, :, -1])
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_prefill_with_one_run_per_row_writes_the_output_itself(out_dtype):
+    """With a single run per query row the 256-row kernel normalises its own record and writes the output; no merge
+    launch follows.  Checked against the oracle for every output dtype (plain rows with a ragged last tile, and a
+    packed prefix), and against the same call cut into two runs, whose records go through the merge kernel."""
+    require_gpu()
+    rng = np.random.default_rng(5)
+    for B, Hq, Hkv, Sq, Skv in ((1, 8, 2, 128, 640), (2, 4, 4, 300, 300)):
+        q = rng.standard_normal((B, Hq, Sq, 128)).astype(np.float16)
+        k = rng.standard_normal((B, Hkv, Skv, 128)).astype(np.float16)
+        v = rng.standard_normal((B, Hkv, Skv, 128)).astype(np.float16)
+        plan = {}
+        out = K.kivi_packed_attend(to_dev(q), k_tail=to_dev(k), v_tail=to_dev(v), n_tail=Skv, scale=128 ** -0.5, causal=True,
+                                   out_dtype=out_dtype, num_splits=1, _plan_out=plan)
+        assert plan["path"] == 2 and plan["nparts"] == 1, plan
+        ref = oa.sdpa(q, k, v, 128 ** -0.5, causal=True)
+        err = float(np.max(np.abs(host(out.float()) - ref)))
+        print(f"{out_dtype}: max-abs err {err:.2e}")
+        assert err < (TOL if out_dtype == torch.float32 else 2e-2 if out_dtype == torch.bfloat16 else 4e-3)
+        # the same rows through two runs and the merge kernel
+        two = K.kivi_packed_attend(to_dev(q), k_tail=to_dev(k), v_tail=to_dev(v), n_tail=Skv, scale=128 ** -0.5, causal=True,
+                                   out_dtype=torch.float32, num_splits=2)
+        assert float((two - out.float()).abs().max()) < (1e-3 if out_dtype == torch.float32 else 2e-2)   # fp16 weights against different references
+    _packed_case(1, 8, 2, 512, 100, 128, 4, 32, "token", torch.float16, Sq=200, causal=True, seed=9, expect_path=2)
+
+
 # ------------------------------------------------------------ packed cache path
 def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, causal=False, seed=0,
                  q_dtype=torch.float16, cap_extra=0, expect_path=None, tail_dtype=torch.float16, window=0):

@@ -213,8 +213,9 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         VQ_HIP_CHECK_LAUNCH(fn);
         if (merged) return finish();
     } else if (p.path == 2) {
-        launch_attend_mfma_prefill(*a, p);
+        const bool written = launch_attend_mfma_prefill(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
+        if (written) return VQ_OK;
     } else {
         rc = launch_attend_generic(*a, p.nsplit, p.split_len);
         if (rc != VQ_OK) return rc;

@@ -109,7 +109,8 @@ int mfma_positions_per_tile(const vq_attend_args &a);
 // MFMA prefill path (attend_prefill.hip): packed prefix into partial slot 0, tail into slot 1
 bool mfma_prefill_supported(const vq_attend_args &a);
 int mfma_prefill_block_rows(const vq_attend_args &a);   // 64, or 256 when a kv head has that many query rows
-void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p);
+// returns true when the kernel wrote the output itself (one run per row: nothing to merge)
+bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p);
 // returns true when the kernel also merged the partials (sync counters were given)
 bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p);
 

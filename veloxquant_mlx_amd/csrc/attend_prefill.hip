@@ -480,6 +480,11 @@ __device__ __forceinline__ f16x8 recon8(f16x8 c, const Meta8<float> &s, const Me
     return o;
 }
 
+// one run per row, nothing to patch afterwards, 256-row blocks: the kernel writes `out`, no merge launch follows
+__host__ __device__ inline bool mfma_prefill_writes_output(const vq_attend_args &a, int nparts) {
+    return nparts == 1 && a.sink_k == nullptr && (a.Hq / a.Hkv) * a.Sq >= 256;
+}
+
 template <int BITS, typename M> struct PrStage {
     u32 kw;          // key word: the thread's 8 channels of one token (2-bit: the word holding them)
     u32 vw;          // value word: the thread's 8 tokens of one channel (2-bit: the word holding them)
@@ -797,7 +802,10 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     }
 
     // ---- every wave owns its rows: accumulator register r of lane (n, blk) is row 4 blk + r of the
-    // row block, tile nt column n is channel 16 nt + n; the row's reference sits in lane 4 blk + r
+    // row block, tile nt column n is channel 16 nt + n; the row's reference sits in lane 4 blk + r.
+    // A launch with one run per row and no protected rows to patch in writes the output itself: the merge
+    // of a single record is that record normalised (mfma_prefill_writes_output decides, for the host too).
+    const bool direct = mfma_prefill_writes_output(a, nparts);
 #pragma unroll
     for (int rb = 0; rb < PR_RB; ++rb)
 #pragma unroll
@@ -807,6 +815,19 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
             const float mr = __shfl(m_run[rb], 4 * blk + r);
             if (pr < a.Sq && jr / qp < R) {
                 const int64_t row = (b * a.Hq + hkv * R + jr / qp) * a.Sq + pr;
+                if (direct) {
+                    // the only record of its row: what the merge would make of it (0 for a row that sees nothing)
+                    const bool seen = mr != -INFINITY && L[rb][r] > 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < 8; ++nt) {
+                        const float v = seen ? __fdiv_rn(O[rb][nt][r], L[rb][r]) : 0.f;
+                        const int64_t oi = row * MF_D + 16 * nt + n;
+                        if (a.out_dtype == VQ_F16) ((f16 *)a.out)[oi] = (f16)v;
+                        else if (a.out_dtype == VQ_BF16) ((u16 *)a.out)[oi] = f32_to_bf16(v);
+                        else ((float *)a.out)[oi] = v;
+                    }
+                    continue;
+                }
                 float *o = ws + (row * nparts + sp) * MF_PART;
 #pragma unroll
                 for (int nt = 0; nt < 8; ++nt) o[2 + 16 * nt + n] = O[rb][nt][r];
@@ -851,7 +872,7 @@ int mfma_prefill_block_rows(const vq_attend_args &a) {
     return (a.Hq / a.Hkv) * a.Sq >= 256 ? 256 : 64;
 }
 
-void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
+bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     hipStream_t st = (hipStream_t)a.stream;
     float *ws = (float *)a.workspace;
     const int R = (int)(a.Hq / a.Hkv);
@@ -871,6 +892,7 @@ void launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     if (a.pack_bits == 4 || a.n_packed == 0) { if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4); }
     else { if (gv == 1) VQ_LAUNCH(2, 1); else if (gv == 2) VQ_LAUNCH(2, 2); else VQ_LAUNCH(2, 4); }
 #undef VQ_LAUNCH
+    return rows == 256 && mfma_prefill_writes_output(a, p.nparts);
 }
 
 }  // namespace vq
