@@ -275,8 +275,9 @@ typedef struct vq_attend_args {
     void *workspace;
     size_t workspace_bytes;
     void *stream;
-    /* Optional: B*Hkv int32 counters, all zero when the call is enqueued; the call leaves
-     * them zero.  With them the MFMA decode path finishes in a single launch (the last
+    /* Optional: int32 counters, one per (sequence, kv head, row tile of the decode path) -- B*Hkv for
+     * single-query calls, B*Hkv*ceil(Sq / positions per tile) for multi-query ones, at most B*Hkv*Sq --
+     * all zero when the call is enqueued; the call leaves them zero.  With them the MFMA decode path finishes in a single launch (the last
      * block of every kv head merges the split partials); without them (NULL) a separate
      * merge kernel follows.  Calls sharing counters must not overlap. */
     int32_t *sync_counters;
