@@ -72,6 +72,14 @@ int vq_kivi_quant_dequant(const void *x, void *out, int dtype, int64_t BH, int64
 int vq_kivi_quant_dequant_mixed(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int group,
                                 int levels_lo, int levels_hi, const uint8_t *hi_mask, float eps, void *stream);
 
+/* The same round trip along the token axis with a level count per token group: group_levels (device, float,
+ * ceil(S / group) entries, the same for every slab) holds 2^bits - 1 for the group's bit width, or 0 for a group
+ * that passes through unchanged.  One launch for age_tier_quantize (veloxquant_mlx/quantizers/age_tiered.py:117-174),
+ * which quantises every stretch of windows of one age tier on its own.  head_dim 128, groups of 32 or 64 tokens,
+ * fp16 or bf16 rows; x/out [BH, S, 128] contiguous, 16-byte aligned, not aliased. */
+int vq_kivi_quant_dequant_grouplevels(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int group,
+                                      const float *group_levels, float eps, void *stream);
+
 /* Per-channel sums over the tokens of x [N, S, D] (slab stride x_stride_n elements), accumulated in double:
  * partial[((n * chunks + k) * 2 + 0) * D + c] = sum, [... + 1 ...] = sum of squares of channel c over the
  * k-th of `chunks` stretches of tokens; the caller adds the chunks.  The population variance Kitty ranks

@@ -97,3 +97,26 @@ def test_bfloat16_storage_and_rejections():
         with pytest.raises(ValueError, match=pat):
             _make(**kw)
     _make(age_recent_boundary=50, age_mid_boundary=50)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("g,n", [(32, 32 * 9), (64, 64 * 5 + 17), (32, 100)])
+def test_one_launch_with_a_level_count_per_window_equals_a_launch_per_tier(g, n):
+    """``vq_kivi_quant_dequant_grouplevels`` against what it replaces: every stretch of windows of one tier round-tripped
+    on its own at that tier's bit width, 16-bit tiers copied (age_tiered.py:117-174) -- bit for bit, with a ragged last
+    window and with tiers that alternate."""
+    require_gpu()
+    from veloxquant_mlx_amd import kernels as K
+    rng = np.random.default_rng(g + n)
+    G, D = 6, 128
+    x = to_dev((rng.standard_normal((G, n, D)) * np.exp(rng.standard_normal(D))).astype(np.float16))
+    n_groups = -(-n // g)
+    for bits_of in ([16, 8, 4, 2], [4, 4, 2, 16], [2, 16, 2, 8]):
+        per_group = [bits_of[j % len(bits_of)] for j in range(n_groups)]
+        levels = torch.tensor([0.0 if b >= 16 else float((1 << b) - 1) for b in per_group], dtype=torch.float32, device=x.device)
+        got = K.kivi_group_quant_dequant_grouplevels(x, levels, g)
+        want = torch.empty_like(x)
+        for j, b in enumerate(per_group):
+            a, e = j * g, min((j + 1) * g, n)
+            want[:, a:e] = x[:, a:e] if b >= 16 else K.kivi_group_quant_dequant(x[:, a:e].contiguous(), -2, g, (1 << b) - 1)
+        assert torch.equal(got, want), bits_of

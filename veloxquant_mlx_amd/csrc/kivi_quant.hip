@@ -695,13 +695,23 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
                                                    int64_t x_stride_bh, float levels, float eps, int bits,
                                                    uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
                                                    int64_t cap_tokens, int64_t dst_tok0, int W,
-                                                   const uint8_t *__restrict__ hi_mask = nullptr, float levels_hi = 0.f) {
+                                                   const uint8_t *__restrict__ hi_mask = nullptr, float levels_hi = 0.f,
+                                                   const float *__restrict__ group_levels = nullptr) {
     constexpr int D = 128, G = 4 * TPL;
     const int lane = threadIdx.x & 63, o = lane >> 2, tq = lane & 3;
     const int64_t s0 = (int64_t)gk * G;
     if (s0 >= S) return;   // the whole wave
     const int64_t r0 = s0 + tq * TPL;   // the lane's first token
     const T *xb = x + bh * x_stride_bh + r0 * D + 8 * o;
+    if (group_levels != nullptr) {   // round trip only: a level count per token group, 0 = the group passes through
+        levels = group_levels[gk];
+        if (levels == 0.f) {
+#pragma unroll
+            for (int i = 0; i < TPL; ++i)
+                if (r0 + i < S) *reinterpret_cast<uint4 *>(out + (bh * S + r0 + i) * D + 8 * o) = *reinterpret_cast<const uint4 *>(xb + (int64_t)i * D);
+            return;
+        }
+    }
     Raw8<T> v[TPL];
     typename Raw8<T>::Acc acc;
     Raw8<T>::init(acc);
@@ -796,6 +806,16 @@ __global__ __launch_bounds__(64 * KQ_WAVES) void kivi_key_quad_mixed_kernel(cons
                                                                            const uint8_t *__restrict__ hi_mask, float eps) {
     kivi_key_quad_body<T, float, 0, TPL, true>((int)blockIdx.x * KQ_WAVES + (int)(threadIdx.x >> 6), (int64_t)blockIdx.y, x, out, S,
                                                x_stride_bh, levels_lo, eps, 0, nullptr, nullptr, nullptr, 0, 0, 0, hi_mask, levels_hi);
+}
+
+// Round trip with a level count per token group (AgeTieredKV: windows of different ages at different bit widths,
+// veloxquant_mlx/quantizers/age_tiered.py:117-174); fp16 / bf16 rows only (a passing group is copied as 16-byte pieces).
+template <typename T, int TPL>
+__global__ __launch_bounds__(64 * KQ_WAVES) void kivi_key_quad_grouplevels_kernel(const T *__restrict__ x, T *__restrict__ out, int64_t S,
+                                                                                 int64_t x_stride_bh, const float *__restrict__ group_levels,
+                                                                                 float eps) {
+    kivi_key_quad_body<T, float, 0, TPL>((int)blockIdx.x * KQ_WAVES + (int)(threadIdx.x >> 6), (int64_t)blockIdx.y, x, out, S, x_stride_bh,
+                                         1.f, eps, 0, nullptr, nullptr, nullptr, 0, 0, 0, nullptr, 0.f, group_levels);
 }
 
 // Sum and sum of squares over the tokens of every channel of x [N, S, D] in double precision: block (chunk, n)
@@ -1389,6 +1409,32 @@ extern "C" int vq_kivi_quant_dequant_mixed(const void *x, void *out, int dtype, 
             hipLaunchKernelGGL((kivi_key_quad_mixed_kernel<T, 16>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D,
                                (float)levels_lo, (float)levels_hi, hi_mask, eps);
     });
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_kivi_quant_dequant_grouplevels(const void *x, void *out, int dtype, int64_t BH, int64_t S, int64_t D, int group,
+                                                 const float *group_levels, float eps, void *stream) {
+    const char *fn = "vq_kivi_quant_dequant_grouplevels";
+    VQ_REQUIRE(D == 128 && (group == 32 || group == 64), VQ_ERR_UNSUPPORTED,
+               "%s: head_dim 128 and groups of 32 or 64 tokens only (got head_dim %lld, group %d)", fn, (long long)D, group);
+    VQ_REQUIRE(dtype == VQ_F16 || dtype == VQ_BF16, VQ_ERR_UNSUPPORTED, "%s: fp16 or bf16 rows only, got dtype tag %d", fn, dtype);
+    VQ_REQUIRE(BH >= 0 && S >= 0, VQ_ERR_INVALID, "%s: negative dimension", fn);
+    if (BH * S == 0) return VQ_OK;
+    VQ_REQUIRE(x && out && group_levels, VQ_ERR_INVALID, "%s: null pointer", fn);
+    VQ_REQUIRE(aligned16(x) && aligned16(out), VQ_ERR_UNSUPPORTED, "%s: x and out must be 16-byte aligned", fn);
+    VQ_REQUIRE(BH <= 65535, VQ_ERR_UNSUPPORTED, "%s: at most 65535 (sequence, head) pairs, got %lld", fn, (long long)BH);
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)cdiv(cdiv(S, group), KQ_WAVES), (unsigned)BH);
+    if (dtype == VQ_F16) {
+        using T = vq::f16;
+        if (group == 32) hipLaunchKernelGGL((kivi_key_quad_grouplevels_kernel<T, 8>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D, group_levels, eps);
+        else hipLaunchKernelGGL((kivi_key_quad_grouplevels_kernel<T, 16>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D, group_levels, eps);
+    } else {
+        using T = vq::bf16_t;
+        if (group == 32) hipLaunchKernelGGL((kivi_key_quad_grouplevels_kernel<T, 8>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D, group_levels, eps);
+        else hipLaunchKernelGGL((kivi_key_quad_grouplevels_kernel<T, 16>), grid, dim3(64 * KQ_WAVES), 0, st, (const T *)x, (T *)out, S, S * D, group_levels, eps);
+    }
     VQ_HIP_CHECK_LAUNCH(fn);
     return VQ_OK;
 }

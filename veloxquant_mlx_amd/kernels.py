@@ -209,6 +209,26 @@ def kivi_group_quant_dequant_mixed(x: torch.Tensor, hi_mask: torch.Tensor, group
     return out
 
 
+def kivi_group_quant_dequant_grouplevels(x: torch.Tensor, group_levels: torch.Tensor, group_size: int, eps: float = 1e-8) -> torch.Tensor:
+    """Token-axis round trip of fp16 / bf16 ``x [N, S, 128]`` with ``group_levels[j]`` levels in token group ``j`` (float32
+    on the device, ``ceil(S / group_size)`` entries; 0 = the group passes through), in one launch (``age_tier_quantize``,
+    veloxquant_mlx/quantizers/age_tiered.py:117-174).  Groups of 32 or 64 tokens."""
+    name = "kivi_group_quant_dequant_grouplevels"
+    tag = _ftag(name, x)
+    _need_gpu(name, x)
+    if x.ndim != 3:
+        raise ValueError(f"{name}: x must be [N, S, D], got {tuple(x.shape)}")
+    N, S, D = x.shape
+    n_groups = -(-S // int(group_size))
+    if group_levels.dtype != torch.float32 or group_levels.numel() != n_groups or group_levels.device != x.device:
+        raise ValueError(f"{name}: group_levels must be {n_groups} float32 values on {x.device}")
+    x = x.contiguous()
+    out = torch.empty_like(x)
+    _lib.check(_lib.load().vq_kivi_quant_dequant_grouplevels(x.data_ptr(), out.data_ptr(), tag, N, S, D, int(group_size),
+                                                             group_levels.contiguous().data_ptr(), float(eps), _stream(x)))
+    return out
+
+
 def zip_route(norms: torch.Tensor, n_hi: int) -> torch.Tensor:
     """int32 ``[BH, S]`` routing order of a salience split of float32 ``norms [BH, S]``: the rows outside the
     ``n_hi`` largest norms in their own order, then the ``n_hi`` largest in theirs, later rows first among equal norms
@@ -1045,7 +1065,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
+    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",

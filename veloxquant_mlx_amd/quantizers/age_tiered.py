@@ -52,6 +52,11 @@ def age_tier_quantize_batched(raw: torch.Tensor, group_tier, tiers_config, group
     if n == 0:
         return raw
     bits = {c.tier: c.bits for c in tiers_config}
+    if raw.dtype == torch.float16 and d == 128 and group_size in (32, 64) and len(group_tier) * group_size >= n:
+        # one launch with a level count per window (0: a tier kept in 16 bits passes through)
+        levels = torch.tensor([0.0 if bits[t] >= 16 else float((1 << bits[t]) - 1) for t in group_tier[: -(-n // group_size)]],
+                              dtype=torch.float32, device=raw.device)
+        return K.kivi_group_quant_dequant_grouplevels(raw, levels, group_size)
     out = torch.empty_like(raw)
     i, n_groups = 0, len(group_tier)
     while i < n_groups:
