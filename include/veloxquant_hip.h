@@ -343,8 +343,10 @@ typedef struct vq_attend_args {
  * runs bit for bit. */
 int vq_kivi_attend_fixed_order(int enable);
 
-/* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the
- * shapes, pack_bits, group and num_splits are ignored). */
+/* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the shapes, pack_bits,
+ * group, num_splits, sliding_window and sink_k are ignored).  0 for a launch that writes its output
+ * itself (a prefill whose row tiles fill the GPU, one run per row, no protected rows): workspace may
+ * then be NULL. */
 size_t vq_kivi_attend_workspace(const vq_attend_args *a);
 
 /* Reports what vq_kivi_attend would do for these arguments: *path = 0 for the

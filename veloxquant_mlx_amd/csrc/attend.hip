@@ -160,7 +160,9 @@ extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
     if (!a || a->B < 1 || a->Hq < 1 || a->Hkv < 1 || a->Sq < 1 || a->D < 1 || a->Hq % a->Hkv != 0 ||
         a->n_packed < 0 || a->n_tail < 0 || (a->n_packed > 0 && (a->pack_bits < 1 || a->pack_bits > 8 || a->group < 1)))
         return 0;
-    AttendPlan p = plan_attend(skip_below_window(*a));
+    const vq_attend_args w = skip_below_window(*a);
+    AttendPlan p = plan_attend(w);
+    if (p.path == 2 && mfma_prefill_direct_output(w, p.nparts)) return 0;   // the kernel writes `out` itself
     return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nparts * (size_t)(a->D + 2) * sizeof(float);
 }
 
@@ -197,7 +199,7 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         VQ_REQUIRE(p.path == 1 && a->Sq == 1, VQ_ERR_UNSUPPORTED,
                    "%s: k_new / v_new need the single-query MFMA decode path; append with vq_kv_tail_append first", fn);
     size_t need = vq_kivi_attend_workspace(a);
-    VQ_REQUIRE(a->workspace != nullptr && a->workspace_bytes >= need, VQ_ERR_WORKSPACE,
+    VQ_REQUIRE(need == 0 || (a->workspace != nullptr && a->workspace_bytes >= need), VQ_ERR_WORKSPACE,
                "%s: workspace of %zu bytes required, %zu given", fn, need, a->workspace_bytes);
     // protected rows: the patch pass reads the partials and the original (unshifted) packed store
     auto finish = [&]() -> int {

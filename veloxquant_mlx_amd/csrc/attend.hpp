@@ -111,6 +111,8 @@ bool mfma_prefill_supported(const vq_attend_args &a);
 int mfma_prefill_block_rows(const vq_attend_args &a);   // 64, or 256 when a kv head has that many query rows
 // returns true when the kernel wrote the output itself (one run per row: nothing to merge)
 bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p);
+// that case, from the shapes alone: such a launch writes no partials and needs no workspace
+bool mfma_prefill_direct_output(const vq_attend_args &a, int nparts);
 // returns true when the kernel also merged the partials (sync counters were given)
 bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p);
 

@@ -872,6 +872,10 @@ int mfma_prefill_block_rows(const vq_attend_args &a) {
     return (a.Hq / a.Hkv) * a.Sq >= 256 ? 256 : 64;
 }
 
+bool mfma_prefill_direct_output(const vq_attend_args &a, int nparts) {
+    return mfma_prefill_block_rows(a) == 256 && mfma_prefill_writes_output(a, nparts);
+}
+
 bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     hipStream_t st = (hipStream_t)a.stream;
     float *ws = (float *)a.workspace;
