@@ -332,7 +332,33 @@ typedef struct vq_attend_args {
     const int32_t *sink_pos;
     int64_t sink_cap;
     int32_t sink_dtype;
+    /* Optional: all n_packed + n_tail slots once more as ready-made fp16 tiles, written by
+     * vq_kivi_prefill_tiles: [B * Hkv, tile_cap, VQ_PREFILL_TILE_BYTES], 16-byte aligned, tile u holding
+     * slots 32 u .. 32 u + 31 (packed slots reconstructed and rounded to fp16 as the reference's cache
+     * holds them, cache/kivi_cache.py:198-201; tail slots as they are).  A multi-query call of 256 or more
+     * rows per kv head (prefill chunks) then copies tiles straight into on-chip memory instead of
+     * reconstructing the prefix in every block; the results are the same bit for bit.  Other calls ignore
+     * it, and so does a call with packed_lens (vq_kivi_attend_plan reports path 2 and 256 or more rows
+     * per kv head for the calls that read it).  The cache arrays above must still be given.  No counterpart
+     * in the reference (whose memory-bound mode dequantises the whole history to fp16 per call,
+     * cache/kivi_cache.py:262-332); a scratch of the prefill phase, 608 bytes per slot and kv head. */
+    const void *kv_tiles;
+    int64_t tile_cap;
+    /* With kv_tiles, for vq_kivi_attend: tiles from this unit on are not up to date; a call that reads the tiles
+     * writes them first (as vq_kivi_prefill_tiles would, same stream); a call that does not read them leaves them
+     * alone, so a caller learns from vq_kivi_attend_plan (path 2) whether they are up to date afterwards.  A value at or past the number of units: nothing to write. */
+    int64_t tiles_stale_from;
 } vq_attend_args;
+
+#define VQ_PREFILL_TILE_BYTES 19456
+
+/* Writes tiles first_unit .. first_unit + n_units - 1 of every (sequence, kv head) into a->kv_tiles from the
+ * cache arrays of *a (k_packed .. v_zero, n_packed, cap_tokens, k_tail, v_tail, n_tail, tail_cap, B, Hkv, D,
+ * stream; the query-side fields are ignored).  D = 128, 2- or 4-bit codes, groups of 32 / 64 / 128, values
+ * token-packed, fp16 or bf16 tail, no packed_lens; tiles past ceil((n_packed + n_tail) / 32) are refused.
+ * A caller that appends chunk by chunk rewrites only the units that changed: those that were tail slots
+ * before the last flush, and the tail.  One launch. */
+int vq_kivi_prefill_tiles(const vq_attend_args *a, int64_t first_unit, int64_t n_units);
 
 /* The decode kernel balances its waves by handing out token chunks on demand, so the order in
  * which partial sums are formed, and with it the last bits of the output, can differ from one

@@ -272,6 +272,18 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
                                out_dtype=torch.float32, _plan_out=plan, **kw)
     if expect_path is not None:
         assert plan["path"] == expect_path, plan
+    if plan["path"] == 2 and (Hq // Hkv) * Sq >= 256:
+        # the same call fed with ready-made tiles (written in two parts, into a buffer that starts out as NaNs
+        # and has spare room) runs the same arithmetic on the same numbers: identical bits
+        units = -(-(n_packed + n_tail) // 32)
+        tiles = K.prefill_tiles_empty(B, Hkv, n_packed + n_tail + 96, qt.device)
+        tiles.fill_(0xFF)
+        cache = dict(n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k, v_tail=tail_v, n_tail=n_tail, **kw)
+        K.kivi_prefill_tiles(tiles, units // 2, units - units // 2, **cache)
+        K.kivi_prefill_tiles(tiles, 0, units // 2, **cache)
+        out_t = K.kivi_packed_attend(qt, scale=scale, causal=causal, sliding_window=window, out_dtype=torch.float32,
+                                     tiles=tiles, **cache)
+        assert torch.equal(out_t, out), float((out_t - out).abs().max())
     if plan["path"] == 1:
         # the single-launch form (last block of a kv head merges the splits) and the form with a
         # separate merge kernel run the same arithmetic (compared with the token chunks dealt in

@@ -384,6 +384,50 @@ def test_config4_prefill_mfma_kernel_agrees_with_vector_kernel_at_full_size():
         assert torch.equal(c.fused_sdpa(q, scale, causal=True), o1.to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("bits,g,dtype", [(4, 32, torch.bfloat16), (2, 64, torch.float16)])
+def test_prefill_tiles_change_no_bit_and_follow_the_cache(bits, g, dtype):
+    """Chunked quantise-on-write prefill with the ready-made tiles (the default) and without them: every chunk's
+    output is identical.  The tiles follow the cache through flushes (only the units that changed are rewritten), a
+    trim below the packed frontier (rewritten from the start) and growth of the packed store; the first decode step
+    gives the scratch back."""
+    require_gpu()
+    B, Hq, Hkv, D, C = 1, 16, 4, 128, 256
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(bits + g)
+    mk = lambda n: (torch.randn((B, Hkv, n, D), generator=gen, device=dev).to(dtype) * 1.5,
+                    torch.randn((B, Hkv, n, D), generator=gen, device=dev).to(dtype))
+    caches = []
+    for on in (True, False):
+        c = _make(bit_width_inlier=bits, kivi_group_size=g, residual_length=128, fused_sdpa=True, fused_sdpa_memory_bound=True)
+        c.prefill_tiles = on
+        caches.append(c)
+    scale = 1 / math.sqrt(D)
+    written = []
+    for ci in range(7):
+        k, v = mk(C if ci != 3 else 96)          # one ragged chunk: the tail then ends inside a unit
+        q = torch.randn((B, Hq, k.shape[2], D), generator=gen, device=dev).to(dtype)
+        if ci == 5:                               # drop tokens below the packed frontier, then go on
+            for c in caches:
+                c.trim(300)
+        outs = []
+        for c in caches:
+            c.update_and_fetch(k, v)
+            outs.append(c.fused_sdpa(q, scale, causal=True))
+        if (Hq // Hkv) * k.shape[2] >= 256:
+            assert caches[0]._tiles is not None and caches[1]._tiles is None
+            written.append(caches[0]._tiles_packed)
+        assert torch.equal(outs[0], outs[1]), (ci, float((outs[0].float() - outs[1].float()).abs().max()))
+    assert written[0] < written[-1] and caches[0]._tiles_packed == caches[0]._n_quantized // 32
+    assert caches[0].nbytes > caches[1].nbytes
+    k, v = mk(1)
+    q = torch.randn((B, Hq, 1, D), generator=gen, device=dev).to(dtype)
+    outs = []
+    for c in caches:
+        c.update_and_fetch(k.clone(), v.clone())
+        outs.append(c.fused_sdpa(q, scale, fixed_order=True))
+    assert torch.equal(outs[0], outs[1]) and caches[0]._tiles is None and caches[0].nbytes == caches[1].nbytes
+
+
 def test_config4_every_chunk_against_the_oracle_on_sampled_rows():
     """Benchmark configuration 4 at full size, every one of the 8 chunks: for one kv head the host
     quantises the same bf16 keys and values with the numpy oracle (one shot over the packed prefix:

@@ -42,6 +42,7 @@ class AttendArgs(C.Structure):
         ("sliding_window", C.c_int64),
         ("sink_k", C.c_void_p), ("sink_v", C.c_void_p), ("sink_pos", C.c_void_p),
         ("sink_cap", C.c_int64), ("sink_dtype", C.c_int32),
+        ("kv_tiles", C.c_void_p), ("tile_cap", C.c_int64), ("tiles_stale_from", C.c_int64),
     ]
 
 
@@ -106,6 +107,7 @@ _SIGNATURES = {
     "vq_kivi_attend_plan": (i32, [C.POINTER(AttendArgs), C.POINTER(i32), C.POINTER(i32)]),
     "vq_kivi_attend": (i32, [C.POINTER(AttendArgs)]),
     "vq_kivi_attend_static": (i32, [C.POINTER(AttendArgs)]),
+    "vq_kivi_prefill_tiles": (i32, [C.POINTER(AttendArgs), i64, i64]),
     "vq_vecinfer_attend_workspace": (sz, [C.POINTER(LutAttendArgs)]),
     "vq_vecinfer_attend": (i32, [C.POINTER(LutAttendArgs)]),
 }

@@ -21,6 +21,7 @@ cache uses (veloxquant_mlx/cache/vecinfer_cache.py:384-411):
 from __future__ import annotations
 
 import math
+import os
 from typing import Any
 
 import torch
@@ -118,6 +119,12 @@ class KIVIKVCache(FP16KVCache):
         # tail; the next fused_sdpa stores them in the same launch that attends, anything else stores them first
         self._pending = None
         self._zero_scalar = None
+        # memory-bound prefill: the slots once more as ready-made fp16 tiles for prefill-sized attention calls
+        # (scratch of the prefill phase, given back at the first decode step); the first _tiles_packed units
+        # hold packed slots that cannot change any more
+        self.prefill_tiles = os.environ.get("VELOXQUANT_PREFILL_TILES", "1") != "0"
+        self._tiles = None
+        self._tiles_packed = 0
 
     # ------------------------------------------------------------------
     def _quant_dequant_along(self, x: torch.Tensor, axis: int) -> torch.Tensor:
@@ -329,6 +336,9 @@ class KIVIKVCache(FP16KVCache):
                   causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
                   sliding_window=int(sliding_window or 0))
         kw.update(self._extra_attend_args())
+        plan = None
+        if lengths is None and self._offer_tiles(q, kw):
+            plan = kw["_plan_out"] = {}
         if lengths is not None:
             self._store_pending()
             n = torch.as_tensor(lengths, device=q.device).to(torch.int64).reshape(-1)
@@ -342,7 +352,32 @@ class KIVIKVCache(FP16KVCache):
                 return out
             except ValueError:   # a shape that path does not take: store the token, then attend
                 self._store_pending()
-        return K.kivi_packed_attend(q, **kw)
+        out = K.kivi_packed_attend(q, **kw)
+        if plan is not None and plan.get("path") == 2:   # the launch that reads the tiles has rewritten the stale ones
+            self._tiles_packed = nq // 32
+        return out
+
+    def _offer_tiles(self, q: torch.Tensor, kw: dict) -> bool:
+        """Give a prefill-sized call the tiles it reads instead of reconstructing the prefix in every block of the
+        launch (same bits either way); the call itself first rewrites what changed since the last one: the units
+        that were tail slots then, and the tail."""
+        B, Hq, Sq, D = q.shape
+        H = self._shape_bhd[1]
+        nq, n_tail = kw["n_packed"], kw["n_tail"]
+        if not (self.prefill_tiles and self._memory_bound and self._v_layout == "token" and D == 128 and Hq % H == 0
+                and Hq // H in (1, 2, 4, 8) and (Hq // H) * Sq >= 256 and nq % 32 == 0 and "sinks" not in kw
+                and (n_tail == 0 or self._tail_k.dtype in (torch.float16, torch.bfloat16))):
+            if Sq == 1:
+                self._tiles = None   # decoding has begun
+            return False
+        units = -(-(nq + n_tail) // 32)
+        t = self._tiles
+        if t is None or t.shape[0] != B * H or t.shape[1] < units or t.device != q.device:
+            room = self._packed_cap + (self._tail_k.shape[2] if self._tail_k is not None else 0)
+            t = self._tiles = K.prefill_tiles_empty(B, H, max(room, 32 * units), q.device)
+            self._tiles_packed = 0
+        kw["tiles"], kw["tiles_stale_from"] = t, min(self._tiles_packed, nq // 32)
+        return True
 
     def _extra_attend_args(self) -> dict:
         """Further arguments of the attention call (subclasses with rows kept outside the packed store)."""
@@ -355,6 +390,7 @@ class KIVIKVCache(FP16KVCache):
         new_nq = min(self._n_quantized, (max(new_offset, 0) // gs) * gs)
         n_rolled = self._n_quantized - new_nq
         self._n_quantized = new_nq
+        self._tiles_packed = 0
         return n_rolled
 
     def _rollback_bytes(self, n_tokens: int, n_rolled: int) -> None:
@@ -473,6 +509,7 @@ class KIVIKVCache(FP16KVCache):
         self._kp = self._ks = self._kz = self._vp = self._vs = self._vz = None
         self._packed_cap = 0
         self._n_quantized = 0
+        self._tiles, self._tiles_packed = None, 0
         if not packed:
             return
         kp, ks, kz, vp, vs, vz = packed
@@ -554,7 +591,7 @@ class KIVIKVCache(FP16KVCache):
     def nbytes(self) -> int:
         total = 0 if self._memory_bound else FP16KVCache.nbytes.fget(self)
         for t in (self._kp, self._ks, self._kz, self._vp, self._vs, self._vz, self._tail_k, self._tail_v,
-                  *(self._tail_spare or ())):
+                  *(self._tail_spare or ()), self._tiles):
             if t is not None:
                 total += t.numel() * t.element_size()
         return total

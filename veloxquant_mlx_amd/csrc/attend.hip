@@ -105,6 +105,7 @@ static vq_attend_args skip_below_window(const vq_attend_args &a) {
         b.v_zero = fwd(a.v_zero, skip * GV * es);
     }
     b.n_packed = a.n_packed - skip;
+    if (a.kv_tiles != nullptr) b.kv_tiles = fwd(a.kv_tiles, skip / 32 * VQ_PREFILL_TILE_BYTES);   // tile_cap stays: it is the stride
     return b;
 }
 
@@ -121,6 +122,10 @@ static int validate(const vq_attend_args *a, const char *fn) {
     VQ_REQUIRE(a->n_packed + a->n_tail >= 1, VQ_ERR_INVALID, "%s: no key/value slots to attend to", fn);
     VQ_REQUIRE(a->fixed_order >= 0 && a->fixed_order <= 3, VQ_ERR_INVALID, "%s: fixed_order must be 0, 1, 2 or 3", fn);
     VQ_REQUIRE(a->sliding_window >= 0, VQ_ERR_INVALID, "%s: negative sliding window", fn);
+    if (a->kv_tiles != nullptr)
+        VQ_REQUIRE(((uintptr_t)a->kv_tiles & 15u) == 0 && a->tile_cap * 32 >= a->n_packed + a->n_tail, VQ_ERR_INVALID,
+                   "%s: kv_tiles must be 16-byte aligned with room for all %lld slots (tile_cap %lld)", fn,
+                   (long long)(a->n_packed + a->n_tail), (long long)a->tile_cap);
     if (a->sink_k != nullptr) {
         VQ_REQUIRE(a->sink_v != nullptr && a->sink_pos != nullptr && a->sink_cap >= 1, VQ_ERR_INVALID,
                    "%s: sink_k needs sink_v, sink_pos and sink_cap >= 1", fn);
@@ -164,6 +169,23 @@ extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
     AttendPlan p = plan_attend(w);
     if (p.path == 2 && mfma_prefill_direct_output(w, p.nparts)) return 0;   // the kernel writes `out` itself
     return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nparts * (size_t)(a->D + 2) * sizeof(float);
+}
+
+extern "C" int vq_kivi_prefill_tiles(const vq_attend_args *a, int64_t first_unit, int64_t n_units) {
+    const char *fn = "vq_kivi_prefill_tiles";
+    VQ_REQUIRE(a != nullptr, VQ_ERR_INVALID, "%s: null argument block", fn);
+    VQ_REQUIRE(a->B >= 1 && a->Hkv >= 1 && a->n_packed >= 0 && a->n_tail >= 0, VQ_ERR_INVALID, "%s: bad sizes", fn);
+    VQ_REQUIRE(a->kv_tiles != nullptr && ((uintptr_t)a->kv_tiles & 15u) == 0, VQ_ERR_INVALID, "%s: kv_tiles must be given, 16-byte aligned", fn);
+    const int64_t units = cdiv(a->n_packed + a->n_tail, 32);
+    VQ_REQUIRE(first_unit >= 0 && n_units >= 0 && first_unit + n_units <= units && units <= a->tile_cap, VQ_ERR_INVALID,
+               "%s: units [%lld, %lld) do not lie inside the %lld units of the slots (tile_cap %lld)", fn, (long long)first_unit,
+               (long long)(first_unit + n_units), (long long)units, (long long)a->tile_cap);
+    if (a->n_packed > 0)
+        VQ_REQUIRE(a->k_packed && a->v_packed && a->k_scale && a->k_zero && a->v_scale && a->v_zero, VQ_ERR_INVALID,
+                   "%s: null packed-cache pointer", fn);
+    if (a->n_tail > 0) VQ_REQUIRE(a->k_tail && a->v_tail, VQ_ERR_INVALID, "%s: null tail pointer", fn);
+    if (n_units == 0) return VQ_OK;
+    return launch_prefill_tiles(*a, first_unit, n_units);
 }
 
 extern "C" int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts) {
@@ -215,6 +237,15 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         VQ_HIP_CHECK_LAUNCH(fn);
         if (merged) return finish();
     } else if (p.path == 2) {
+        if (mfma_prefill_uses_tiles(*a)) {
+            // bring the tiles up to date first (whole-sequence unit numbers: the arguments as given, not the windowed ones)
+            const int64_t units = cdiv(a_in->n_packed + a_in->n_tail, 32);
+            const int64_t from = a_in->tiles_stale_from < 0 ? 0 : a_in->tiles_stale_from;
+            if (from < units) {
+                rc = launch_prefill_tiles(*a_in, from, units - from);
+                if (rc != VQ_OK) return rc;
+            }
+        }
         const bool written = launch_attend_mfma_prefill(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
         if (written) return VQ_OK;

@@ -113,6 +113,10 @@ int mfma_prefill_block_rows(const vq_attend_args &a);   // 64, or 256 when a kv 
 bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p);
 // that case, from the shapes alone: such a launch writes no partials and needs no workspace
 bool mfma_prefill_direct_output(const vq_attend_args &a, int nparts);
+// whether a launch of the 256-row blocks takes its units from a.kv_tiles
+bool mfma_prefill_uses_tiles(const vq_attend_args &a);
+// writes tiles [first_unit, first_unit + n_units) of every (sequence, kv head); VQ_OK or an error code
+int launch_prefill_tiles(const vq_attend_args &a, int64_t first_unit, int64_t n_units);
 // returns true when the kernel also merged the partials (sync counters were given)
 bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p);
 

@@ -41,6 +41,13 @@ __device__ __forceinline__ float vmax3(float a, float b, float c) {
 
 constexpr int PF_KSTRIDE = MF_D + 8;   // fp16 per token row of the key-code tile (272 B: conflict-free b128 reads)
 constexpr int PF_VSTRIDE = 32 + 8;     // fp16 per channel row of the value tile (80 B)
+// A unit (32 tokens of one kv head) as the 256-row blocks read it from LDS: the key tile (32 token rows of
+// PF_KSTRIDE fp16, row pf_krow(token)) followed by the value tile (128 channel rows of PF_VSTRIDE fp16, tokens
+// in order), padded to whole kilobytes.  vq_kivi_prefill_tiles writes units in this form to global memory; a
+// launch that is given them copies them into LDS as they are.
+constexpr int PF_TILE_KEYS = 32 * PF_KSTRIDE * 2;                  // bytes of the key tile
+constexpr int PF_TILE_BYTES = 19 * 1024;                           // >= PF_TILE_KEYS + 128 * PF_VSTRIDE * 2
+static_assert(PF_TILE_BYTES >= PF_TILE_KEYS + MF_D * PF_VSTRIDE * 2 && PF_TILE_BYTES == VQ_PREFILL_TILE_BYTES, "tile size");
 
 // four k-slot pair registers of one unpacked word -> the same eight values in code order
 __device__ __forceinline__ uint4 pairs_to_order(u32 r0, u32 r1, u32 r2, u32 r3) {
@@ -492,11 +499,23 @@ template <int BITS, typename M> struct PrStage {
                      // raw key and value pieces travel in the first piece of each
 };
 
-template <int BITS, int GV, typename M>
+// TILES: every unit comes ready-made from a.kv_tiles (the packed prefix and the tail alike) and is copied from
+// global memory straight into a ring of four LDS buffers, four units ahead; the block then has no producer work
+// on the vector unit and holds no staging registers.  BITS, GV and M play no part then.
+template <int BITS, int GV, typename M, bool TILES = false>
 __global__ __launch_bounds__(PR_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
 void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__restrict__ ws) {
-    __shared__ __align__(16) f16 s_k[3][32 * PF_KSTRIDE];
-    __shared__ __align__(16) f16 s_v[3][MF_D * PF_VSTRIDE];
+    __shared__ __align__(16) f16 s_k[TILES ? 1 : 3][32 * PF_KSTRIDE];
+    __shared__ __align__(16) f16 s_v[TILES ? 1 : 3][MF_D * PF_VSTRIDE];
+    __shared__ __align__(16) char s_ring[TILES ? 4 * PF_TILE_BYTES : 16];
+    auto key_tile = [&](int buf) -> const f16 * {
+        if constexpr (TILES) return reinterpret_cast<const f16 *>(s_ring + buf * PF_TILE_BYTES);
+        else return s_k[buf];
+    };
+    auto value_tile = [&](int buf) -> const f16 * {
+        if constexpr (TILES) return reinterpret_cast<const f16 *>(s_ring + buf * PF_TILE_BYTES + PF_TILE_KEYS);
+        else return s_v[buf];
+    };
 
     constexpr int PER = 32 / BITS;
     constexpr int KW = MF_D / PER;
@@ -528,6 +547,10 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     const int64_t bh = bh_y;
     const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
     take_sequence_lengths(a, b);
+    if constexpr (TILES) {   // one kind of unit: all slots count as tail slots
+        a.n_tail += a.n_packed;
+        a.n_packed = 0;
+    }
     const int R = (int)(a.Hq / a.Hkv);
     const int64_t cap = a.cap_tokens;
     const float c = a.scale * LOG2E;
@@ -704,7 +727,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     auto load_keys = [&](int buf) {
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
-            const f16 *kr = &s_k[buf][pf_krow(pf_tok(n >> 2, n & 3, T)) * PF_KSTRIDE + 8 * blk];
+            const f16 *kr = &key_tile(buf)[pf_krow(pf_tok(n >> 2, n & 3, T)) * PF_KSTRIDE + 8 * blk];
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) A[T][ks] = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
         }
@@ -712,7 +735,7 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     auto load_values = [&](int buf) {
 #pragma unroll
         for (int nt = 0; nt < 8; ++nt)
-            Bv[nt] = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+            Bv[nt] = *reinterpret_cast<const f16x8 *>(&value_tile(buf)[(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
     };
 
     // One unit: scores of the wave's row blocks (four independent accumulator chains side by
@@ -775,30 +798,73 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     // global load, i.e. for the unit just requested, once per unit.  For the same reason nothing
     // requested before the loop may still be pending inside it (the compiler would wait for it at
     // the loop head, and with it for whatever was requested since).
-    Stage st;
-    if (w1 > w0) {
-        fetch(w0, st);
-        unpack_to_lds(w0, st, 0);
-        if (w0 + 1 < w1) {
-            fetch(w0 + 1, st);
-            unpack_to_lds(w0 + 1, st, 1);
+    if constexpr (TILES) {
+        // A unit is 19 pieces of 1 KB; wave v copies pieces v, v + 8 and v + 16 (waves 3..7 copy piece v + 8 a second
+        // time instead: every wave has three copies per unit in flight, which is what the waits count).  Four
+        // buffers.  Iteration w computes unit w from registers while it reads unit w+1 from LDS into them, then waits
+        // for its copies of unit w+2 (those of unit w+3 stay in flight) and meets the other waves; after that barrier
+        // every wave has used unit w, so unit w+4 is requested into its buffer.  The barrier does not wait for the
+        // wave's own LDS reads (nothing was written through LDS instructions): they stay in flight across it, and
+        // the products that use them wait for them.  Past the end of the run the last unit is copied again.
+        // (Forming the next unit's scores between this unit's exponentials, which the spare registers of this form
+        // allow, was built and measured: no faster -- a product leaves the vector unit little room here.)
+        const char *tiles = (const char *)a.kv_tiles + bh * a.tile_cap * PF_TILE_BYTES;
+        const u32 ring = lds_addr(s_ring), lane16 = (u32)lane * 16u;
+        const int third_piece = wave < 3 ? wave + 16 : wave + 8;
+        auto request = [&](int w, int buf) __attribute__((always_inline)) {
+            const char *src = tiles + (int64_t)(w < w1 ? w : w1 - 1) * PF_TILE_BYTES;
+            const u32 dst = ring + (u32)buf * PF_TILE_BYTES;
+            lds_copy16<0>(src + 1024 * wave, lane16, dst + 1024 * wave);
+            lds_copy16<0>(src + 1024 * (wave + 8), lane16, dst + 1024 * (wave + 8));
+            lds_copy16<0>(src + 1024 * third_piece, lane16, dst + 1024 * third_piece);
+        };
+        if (w1 > w0) {
+            wait_global_accesses();
+#pragma unroll
+            for (int i = 0; i < 4; ++i) request(w0 + i, i);
+            wait_copies<9>();
+            lds_barrier();
+            load_keys(0);
+            load_values(0);
+            wait_copies<6>();
+            lds_barrier();
+            int cur = 0;
+            for (int w = w0; w < w1; ++w) {
+                const int next = (cur + 1) & 3;
+                compute(next, w * 32, false, full_tvis, edge_tlo);
+                wait_copies<3>();
+                asm volatile("s_barrier" ::: "memory");
+                request(w + 4, cur);
+                cur = next;
+            }
+            wait_copies<0>();   // nothing may land in LDS after the block has given it back
         }
-        if (w0 + 2 < w1) fetch(w0 + 2, st);
-        __syncthreads();
-        load_keys(0);
-        load_values(0);
-    }
-    wait_global_accesses();
-    int cur = 0;
-    for (int w = w0; w < w1; ++w) {
-        const int next = cur == 2 ? 0 : cur + 1, third = next == 2 ? 0 : next + 1;
-        const bool packed = w < n_punits;
-        const int base = packed ? w * 32 : (w - n_punits) * 32;
-        compute(next, base, packed, packed ? full_vis : full_tvis, packed ? edge_lo : edge_tlo);
-        if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
-        if (w + 3 < w1) fetch(w + 3, st);
-        lds_barrier();
-        cur = next;
+    } else {
+        Stage st;
+        if (w1 > w0) {
+            fetch(w0, st);
+            unpack_to_lds(w0, st, 0);
+            if (w0 + 1 < w1) {
+                fetch(w0 + 1, st);
+                unpack_to_lds(w0 + 1, st, 1);
+            }
+            if (w0 + 2 < w1) fetch(w0 + 2, st);
+            __syncthreads();
+            load_keys(0);
+            load_values(0);
+        }
+        wait_global_accesses();
+        int cur = 0;
+        for (int w = w0; w < w1; ++w) {
+            const int next = cur == 2 ? 0 : cur + 1, third = next == 2 ? 0 : next + 1;
+            const bool packed = w < n_punits;
+            const int base = packed ? w * 32 : (w - n_punits) * 32;
+            compute(next, base, packed, packed ? full_vis : full_tvis, packed ? edge_lo : edge_tlo);
+            if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
+            if (w + 3 < w1) fetch(w + 3, st);
+            lds_barrier();
+            cur = next;
+        }
     }
 
     // ---- every wave owns its rows: accumulator register r of lane (n, blk) is row 4 blk + r of the
@@ -834,6 +900,68 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
                 if (n == 0) { o[0] = mr * LN2; o[1] = L[rb][r]; }
             }
         }
+}
+
+// ---- units as ready-made tiles in global memory: grid (units, B*Hkv), block 512.  Unit first_unit + x of every
+// (sequence, kv head): packed units are reconstructed exactly as the 256-row blocks do it (c s + z rounded once
+// to fp16), tail units are the plain rows; the thread-to-piece assignment is that of the blocks' producer.
+template <int BITS, int GV, typename M>
+__global__ __launch_bounds__(PR_THREADS) void prefill_tiles_kernel(vq_attend_args a, int first_unit) {
+    constexpr int PER = 32 / BITS;
+    constexpr int KW = MF_D / PER;
+    constexpr int gshift = GV == 4 ? 5 : GV == 2 ? 6 : 7;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t bh = blockIdx.y, cap = a.cap_tokens;
+    const int w = first_unit + (int)blockIdx.x, n_punits = (int)(a.n_packed / 32);
+    char *tile = (char *)a.kv_tiles + (bh * a.tile_cap + w) * PF_TILE_BYTES;
+    f16 *kdst = reinterpret_cast<f16 *>(tile), *vdst = reinterpret_cast<f16 *>(tile + PF_TILE_KEYS);
+    const int kt = tid >> 4, kc = tid & 15;       // key tile: token, 8-channel chunk
+    const int vc = tid & 127, vq = tid >> 7;      // value tile: channel, 8-token quarter
+    if (w < n_punits) {
+        const u32 magic = vreg_const(Magic<BITS>::bits);
+        const f16x8 off8 = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair);
+        auto codes8 = [&](u32 word, int half) -> f16x8 {
+            uint4 lo;
+            if (BITS == 4) lo = word4_in_order(word, magic);
+            else {
+                uint4 hi;
+                word2_in_order(word, magic, lo, hi);
+                if (half) lo = hi;
+            }
+            return as_h8(lo) + off8;
+        };
+        const int64_t base = (int64_t)w * 32;
+        const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
+        const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
+        const M *ksb = (const M *)a.k_scale + bh * (cap >> gshift) * MF_D, *kzb = (const M *)a.k_zero + bh * (cap >> gshift) * MF_D;
+        const M *vsb = (const M *)a.v_scale + bh * GV * cap, *vzb = (const M *)a.v_zero + bh * GV * cap;
+        const u32 kw = *reinterpret_cast<const u32 *>(kb + (base + kt) * (KW * 4) + (BITS == 4 ? kc : kc >> 1) * 4);
+        const u32 vw = *reinterpret_cast<const u32 *>(vb + ((base / PER) + (BITS == 4 ? vq : vq >> 1)) * (MF_D * 4) + vc * 4);
+        Meta8<M> ks, kz, vs, vz;
+        const int64_t grp = base >> gshift;
+        ks.load(ksb + grp * MF_D + 8 * kc);
+        kz.load(kzb + grp * MF_D + 8 * kc);
+        vs.load(vsb + (int64_t)(vc >> gshift) * cap + base + 8 * vq);
+        vz.load(vzb + (int64_t)(vc >> gshift) * cap + base + 8 * vq);
+        *reinterpret_cast<f16x8 *>(&kdst[pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = recon8(codes8(kw, kc & 1), ks, kz);
+        *reinterpret_cast<f16x8 *>(&vdst[vc * PF_VSTRIDE + 8 * vq]) = recon8(codes8(vw, vq & 1), vs, vz);
+    } else {
+        // tail unit; a token past the end of the tail repeats the last one (masked in the softmax)
+        const bool tail_bf16 = a.tail_dtype == VQ_BF16;
+        const int64_t t0 = (int64_t)(w - n_punits) * 32, tbase = bh * a.tail_cap * MF_D;
+        const int last = (int)(a.n_tail - 1 - t0);
+        const int tk = kt < last ? kt : last;
+        *reinterpret_cast<f16x8 *>(&kdst[pf_krow(kt) * PF_KSTRIDE + 8 * kc]) = ld_tail8(a.k_tail, tbase + (t0 + tk) * MF_D + 8 * kc, tail_bf16);
+        const int tp = lane & 15, cq = 4 * wave + (lane >> 4);   // token pair, channel quad
+        const int ta = 2 * tp < last ? 2 * tp : last, tb = 2 * tp + 1 < last ? 2 * tp + 1 : last;
+        const char *vt0 = (const char *)a.v_tail + (tbase + t0 * MF_D) * 2;
+        const uint2 va = *reinterpret_cast<const uint2 *>(vt0 + ta * (MF_D * 2) + 8 * cq);
+        const uint2 vb2 = *reinterpret_cast<const uint2 *>(vt0 + tb * (MF_D * 2) + 8 * cq);
+        const f16x8 v0 = tail8_from_raw(make_uint4(va.x, va.y, vb2.x, vb2.y), tail_bf16);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            *reinterpret_cast<f16x2 *>(&vdst[(4 * cq + e) * PF_VSTRIDE + 2 * tp]) = f16x2{v0[e], v0[4 + e]};
+    }
 }
 
 int mfma_prefill_block_rows(const vq_attend_args &a);
@@ -876,6 +1004,44 @@ bool mfma_prefill_direct_output(const vq_attend_args &a, int nparts) {
     return mfma_prefill_block_rows(a) == 256 && mfma_prefill_writes_output(a, nparts);
 }
 
+bool mfma_prefill_uses_tiles(const vq_attend_args &a) {
+    return a.kv_tiles != nullptr && a.packed_lens == nullptr && mfma_prefill_block_rows(a) == 256 &&
+           ((uintptr_t)a.kv_tiles & 15u) == 0 && a.tile_cap * 32 >= a.n_packed + a.n_tail && a.n_packed % 32 == 0;
+}
+
+int launch_prefill_tiles(const vq_attend_args &a, int64_t first_unit, int64_t n_units) {
+    const char *fn = "vq_kivi_prefill_tiles";
+    VQ_REQUIRE(a.D == MF_D && a.packed_lens == nullptr, VQ_ERR_UNSUPPORTED, "%s: head_dim 128 and one length for the batch only", fn);
+    VQ_REQUIRE(a.B * a.Hkv <= 65535 && n_units <= 0x7fffffff, VQ_ERR_UNSUPPORTED, "%s: too many (sequence, kv head) pairs or units", fn);
+    if (a.n_packed > 0) {
+        VQ_REQUIRE((a.pack_bits == 2 || a.pack_bits == 4) && (a.group == 32 || a.group == 64 || a.group == 128) &&
+                       (a.meta_dtype == VQ_F16 || a.meta_dtype == VQ_F32) && a.v_layout == VQ_V_TOKEN_PACKED,
+                   VQ_ERR_UNSUPPORTED, "%s: 2- or 4-bit codes, groups of 32 / 64 / 128, fp16 or float32 scale / zero, token-packed values", fn);
+        VQ_REQUIRE(a.n_packed % 32 == 0 && a.cap_tokens % 32 == 0 && a.cap_tokens % a.group == 0 && a.cap_tokens <= ((int64_t)1 << 28),
+                   VQ_ERR_UNSUPPORTED, "%s: packed counts must be multiples of 32 and of the group", fn);
+        const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
+                             (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
+        VQ_REQUIRE((al & 15u) == 0, VQ_ERR_UNSUPPORTED, "%s: cache arrays must be 16-byte aligned", fn);
+    }
+    if (a.n_tail > 0)
+        VQ_REQUIRE((a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) && ((((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u) == 0) &&
+                       a.tail_cap >= a.n_tail, VQ_ERR_UNSUPPORTED, "%s: fp16 or bf16 tail, 16-byte aligned", fn);
+    hipStream_t st = (hipStream_t)a.stream;
+    const dim3 grid((unsigned)n_units, (unsigned)(a.B * a.Hkv));
+    const int gv = a.n_packed > 0 ? (int)(MF_D / a.group) : 4;
+    const bool f32 = a.n_packed > 0 && a.meta_dtype == VQ_F32;
+#define VQ_TILES(BITS, GV)                                                                                                  \
+    do {                                                                                                                   \
+        if (f32) hipLaunchKernelGGL((prefill_tiles_kernel<BITS, GV, float>), grid, dim3(PR_THREADS), 0, st, a, (int)first_unit); \
+        else hipLaunchKernelGGL((prefill_tiles_kernel<BITS, GV, f16>), grid, dim3(PR_THREADS), 0, st, a, (int)first_unit);  \
+    } while (0)
+    if (a.pack_bits == 4 || a.n_packed == 0) { if (gv == 1) VQ_TILES(4, 1); else if (gv == 2) VQ_TILES(4, 2); else VQ_TILES(4, 4); }
+    else { if (gv == 1) VQ_TILES(2, 1); else if (gv == 2) VQ_TILES(2, 2); else VQ_TILES(2, 4); }
+#undef VQ_TILES
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
 bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     hipStream_t st = (hipStream_t)a.stream;
     float *ws = (float *)a.workspace;
@@ -886,7 +1052,9 @@ bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     const dim3 grid((unsigned)tiles, (unsigned)(a.B * a.Hkv), (unsigned)p.nsplit), block(256);
 #define VQ_LAUNCH(BITS, GV)                                                                                          \
     do {                                                                                                             \
-        if (rows == 256 && a.n_packed > 0 && a.meta_dtype == VQ_F32)                                                 \
+        if (rows == 256 && mfma_prefill_uses_tiles(a))                                                               \
+            hipLaunchKernelGGL((attend_prefill_rows_kernel<4, 4, f16, true>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \
+        else if (rows == 256 && a.n_packed > 0 && a.meta_dtype == VQ_F32)                                            \
             hipLaunchKernelGGL((attend_prefill_rows_kernel<BITS, GV, float>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \
         else if (rows == 256)                                                                                        \
             hipLaunchKernelGGL((attend_prefill_rows_kernel<BITS, GV, f16>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, ws); \

@@ -800,57 +800,11 @@ def _tail_layout(t: torch.Tensor):
     return t, n
 
 
-def attend_fixed_order(enable: bool) -> bool:
-    """Deal the decode kernel's token chunks to its waves in a fixed order (bit-identical results
-    from run to run, a few percent slower) instead of on demand.  Returns the previous setting."""
-    return bool(_lib.load().vq_kivi_attend_fixed_order(1 if enable else 0))
-
-
-def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=None, v_packed=None,
-                       v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
-                       v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
-                       scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
-                       num_splits: int = 0, packed_lens: torch.Tensor | None = None,
-                       tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
-                       v_new: torch.Tensor | None = None, fixed_order: bool | None = None,
-                       out: torch.Tensor | None = None, static_scratch: bool = False, sliding_window: int = 0,
-                       sinks: tuple | None = None,
-                       _plan_out: dict | None = None, _single_launch: bool = True) -> torch.Tensor:
-    """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
-
-    q ``[B,Hq,Sq,D]``; packed buffers as :func:`kivi_quant_pack` lays them out
-    with capacity read from their shapes, of which the first ``n_packed`` tokens
-    are live; tails ``[B,Hkv,tail_cap,D]`` with ``n_tail`` live tokens.  GQA by
-    repeat-interleave.  ``causal`` aligns queries to the end of the slots.
-    ``fixed_order`` (this call only): True deals the decode kernel's token chunks to its waves
-    in a fixed order (identical bits from run to run), False on demand, None takes the process
-    default set by :func:`attend_fixed_order`.  ``out`` receives the result when given (a
-    contiguous ``[B,Hq,Sq,D]`` tensor).  ``static_scratch=True`` goes through
-    ``vq_kivi_attend_static``: the library's built-in scratch instead of a torch workspace, for
-    callers that may not allocate (give ``out`` too; calls on one GPU must not overlap).
-    ``sliding_window > 0``: a query sees only that many last slots up to its own position.
-    ``sinks=(sink_k, sink_v, sink_pos)``: exact rows ``[B,Hkv,cap,D]`` standing for the packed
-    positions ``sink_pos`` (int32 ``[B,cap]``, -1 for an unused slot) whose packed stand-ins carry
-    zero value scale / zero: the stand-ins' softmax weights are taken out and the exact rows put in."""
-    name = "kivi_packed_attend"
-    if q.ndim != 4:
-        raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
-    _need_gpu(name, q)
-    B, Hq, Sq, D = q.shape
-    q = q.contiguous()
-    if out_dtype is None:
-        out_dtype = q.dtype
-    a = AttendArgs()
-    if out is None:
-        out = torch.empty((B, Hq, Sq, D), dtype=out_dtype, device=q.device)
-    elif tuple(out.shape) != (B, Hq, Sq, D) or not out.is_contiguous() or out.device != q.device:
-        raise ValueError(f"{name}: out must be a contiguous [{B}, {Hq}, {Sq}, {D}] tensor on the device of q")
-    else:
-        out_dtype = out.dtype
-    a.q, a.out = q.data_ptr(), out.data_ptr()
-    a.q_dtype, a.out_dtype = _ftag(name, q), _FLOAT_TAG[out_dtype]
+def _cache_side(name, a, keep, k_packed, k_scale, k_zero, v_packed, v_scale, v_zero, n_packed, bits, group_size,
+                v_layout, k_tail, v_tail, n_tail):
+    """Fill the cache fields of ``a`` (packed prefix and tail); returns ``(Hkv, k_tail)`` with the tail as passed
+    to the library."""
     Hkv = None
-    keep = [q, out]
     if n_packed > 0:
         for t in (k_packed, k_scale, k_zero, v_packed, v_scale, v_zero):
             if t is None or not t.is_contiguous():
@@ -891,8 +845,102 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         keep += [k_tail, v_tail]
     if Hkv is None:
         raise ValueError(f"{name}: no key/value slots to attend to")
-    a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
     a.n_packed, a.n_tail = int(n_packed), int(n_tail)
+    return Hkv, k_tail
+
+
+PREFILL_TILE_BYTES = 19456
+
+
+def _check_tiles(name, tiles, rows, device):
+    if (tiles.dtype != torch.uint8 or tiles.ndim != 3 or tiles.shape[0] != rows or tiles.shape[2] != PREFILL_TILE_BYTES
+            or not tiles.is_contiguous() or tiles.device != device):
+        raise ValueError(f"{name}: tiles must be a contiguous uint8 [{rows}, units, {PREFILL_TILE_BYTES}] tensor on the device")
+
+
+def prefill_tiles_empty(B: int, Hkv: int, tokens: int, device) -> torch.Tensor:
+    """Room for the tiles of ``tokens`` slots per (sequence, kv head)."""
+    return torch.empty((B * Hkv, (int(tokens) + 31) // 32, PREFILL_TILE_BYTES), dtype=torch.uint8, device=device)
+
+
+def kivi_prefill_tiles(tiles: torch.Tensor, first_unit: int, n_units: int, *, k_packed=None, k_scale=None, k_zero=None,
+                       v_packed=None, v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
+                       v_layout: str = "token", k_tail=None, v_tail=None, n_tail: int = 0) -> None:
+    """Write units ``first_unit .. first_unit + n_units - 1`` (32 slots each) of ``[quantised prefix | tail]`` into
+    ``tiles`` in the form the prefill blocks of :func:`kivi_packed_attend` read from on-chip memory: packed slots
+    reconstructed and rounded to fp16 (what the reference's cache holds, cache/kivi_cache.py:198-201), tail slots
+    as they are.  One launch; a caller that appends chunk by chunk rewrites only what changed."""
+    name = "kivi_prefill_tiles"
+    a = AttendArgs()
+    keep = [tiles]
+    Hkv, _ = _cache_side(name, a, keep, k_packed, k_scale, k_zero, v_packed, v_scale, v_zero, n_packed, bits, group_size,
+                         v_layout, k_tail, v_tail, n_tail)
+    src = k_packed if n_packed > 0 else k_tail
+    B, D = src.shape[0], (k_tail.shape[3] if k_tail is not None else 128)
+    _check_tiles(name, tiles, B * Hkv, src.device)
+    a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hkv, Hkv, 1, D
+    a.kv_tiles, a.tile_cap = tiles.data_ptr(), tiles.shape[1]
+    a.stream = _stream(src)
+    _lib.check(_lib.load().vq_kivi_prefill_tiles(a, int(first_unit), int(n_units)))
+
+
+def attend_fixed_order(enable: bool) -> bool:
+    """Deal the decode kernel's token chunks to its waves in a fixed order (bit-identical results
+    from run to run, a few percent slower) instead of on demand.  Returns the previous setting."""
+    return bool(_lib.load().vq_kivi_attend_fixed_order(1 if enable else 0))
+
+
+def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=None, v_packed=None,
+                       v_scale=None, v_zero=None, n_packed: int = 0, bits: int = 4, group_size: int = 32,
+                       v_layout: str = "channel", k_tail=None, v_tail=None, n_tail: int = 0,
+                       scale: float = 1.0, causal: bool = False, out_dtype: torch.dtype | None = None,
+                       num_splits: int = 0, packed_lens: torch.Tensor | None = None,
+                       tail_lens: torch.Tensor | None = None, k_new: torch.Tensor | None = None,
+                       v_new: torch.Tensor | None = None, fixed_order: bool | None = None,
+                       out: torch.Tensor | None = None, static_scratch: bool = False, sliding_window: int = 0,
+                       sinks: tuple | None = None, tiles: torch.Tensor | None = None, tiles_stale_from: int | None = None,
+                       _plan_out: dict | None = None, _single_launch: bool = True) -> torch.Tensor:
+    """softmax(q k^T * scale) v over ``[quantised prefix | fp16 tail]``.
+
+    q ``[B,Hq,Sq,D]``; packed buffers as :func:`kivi_quant_pack` lays them out
+    with capacity read from their shapes, of which the first ``n_packed`` tokens
+    are live; tails ``[B,Hkv,tail_cap,D]`` with ``n_tail`` live tokens.  GQA by
+    repeat-interleave.  ``causal`` aligns queries to the end of the slots.
+    ``fixed_order`` (this call only): True deals the decode kernel's token chunks to its waves
+    in a fixed order (identical bits from run to run), False on demand, None takes the process
+    default set by :func:`attend_fixed_order`.  ``out`` receives the result when given (a
+    contiguous ``[B,Hq,Sq,D]`` tensor).  ``static_scratch=True`` goes through
+    ``vq_kivi_attend_static``: the library's built-in scratch instead of a torch workspace, for
+    callers that may not allocate (give ``out`` too; calls on one GPU must not overlap).
+    ``sliding_window > 0``: a query sees only that many last slots up to its own position.
+    ``sinks=(sink_k, sink_v, sink_pos)``: exact rows ``[B,Hkv,cap,D]`` standing for the packed
+    positions ``sink_pos`` (int32 ``[B,cap]``, -1 for an unused slot) whose packed stand-ins carry
+    zero value scale / zero: the stand-ins' softmax weights are taken out and the exact rows put in.
+    ``tiles``: the slots once more as ready-made tiles (:func:`kivi_prefill_tiles`); prefill-sized calls copy
+    them instead of reconstructing the prefix in every block (same bits), other calls ignore them.  With
+    ``tiles_stale_from`` a call that reads the tiles first rewrites them from that unit on (None: they are up to
+    date)."""
+    name = "kivi_packed_attend"
+    if q.ndim != 4:
+        raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
+    _need_gpu(name, q)
+    B, Hq, Sq, D = q.shape
+    q = q.contiguous()
+    if out_dtype is None:
+        out_dtype = q.dtype
+    a = AttendArgs()
+    if out is None:
+        out = torch.empty((B, Hq, Sq, D), dtype=out_dtype, device=q.device)
+    elif tuple(out.shape) != (B, Hq, Sq, D) or not out.is_contiguous() or out.device != q.device:
+        raise ValueError(f"{name}: out must be a contiguous [{B}, {Hq}, {Sq}, {D}] tensor on the device of q")
+    else:
+        out_dtype = out.dtype
+    a.q, a.out = q.data_ptr(), out.data_ptr()
+    a.q_dtype, a.out_dtype = _ftag(name, q), _FLOAT_TAG[out_dtype]
+    keep = [q, out]
+    Hkv, k_tail = _cache_side(name, a, keep, k_packed, k_scale, k_zero, v_packed, v_scale, v_zero, n_packed, bits,
+                              group_size, v_layout, k_tail, v_tail, n_tail)
+    a.B, a.Hq, a.Hkv, a.Sq, a.D = B, Hq, Hkv, Sq, D
     a.scale, a.causal, a.num_splits = float(scale), int(bool(causal)), int(num_splits)
     a.sliding_window = int(sliding_window or 0)
     if sinks is not None:
@@ -905,6 +953,11 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         a.sink_k, a.sink_v, a.sink_pos = sk.data_ptr(), sv.data_ptr(), sp.data_ptr()
         a.sink_cap, a.sink_dtype = int(cap_s), _FLOAT_TAG[sk.dtype]
         keep += [sk, sv, sp]
+    if tiles is not None:
+        _check_tiles(name, tiles, B * Hkv, q.device)
+        a.kv_tiles, a.tile_cap = tiles.data_ptr(), tiles.shape[1]
+        a.tiles_stale_from = tiles.shape[1] if tiles_stale_from is None else int(tiles_stale_from)
+        keep.append(tiles)
     a.fixed_order = 0 if fixed_order is None else (int(fixed_order) if fixed_order is not True and fixed_order is not False and int(fixed_order) > 2 else (1 if fixed_order else 2))
     if (packed_lens is None) != (tail_lens is None):
         raise ValueError(f"{name}: packed_lens and tail_lens go together")
@@ -1065,7 +1118,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant",
+    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant", "kivi_prefill_tiles", "prefill_tiles_empty",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",
