@@ -225,6 +225,28 @@ def test_prefill_with_one_run_per_row_writes_the_output_itself(out_dtype):
     _packed_case(1, 8, 2, 512, 100, 128, 4, 32, "token", torch.float16, Sq=200, causal=True, seed=9, expect_path=2)
 
 
+def test_plain_prefill_with_many_row_tiles_goes_through_a_tile_scratch():
+    """From two dozen row tiles per kv head a causal call over plain keys and values writes them once as tiles and
+    copies those: the same bits as the blocks that convert and transpose the rows themselves, and the oracle's
+    numbers.  A second, smaller call reuses the scratch."""
+    require_gpu()
+    rng = np.random.default_rng(12)
+    for Sq, Skv, dt in ((768, 800, torch.float16), (770, 770, torch.bfloat16)):
+        q = rng.standard_normal((1, 8, Sq, 128)).astype(np.float32)
+        k = rng.standard_normal((1, 1, Skv, 128)).astype(np.float32)
+        v = rng.standard_normal((1, 1, Skv, 128)).astype(np.float32)
+        qt, kt, vt = to_dev(q, dt), to_dev(k, dt), to_dev(v, dt)
+        args = dict(k_tail=kt, v_tail=vt, n_tail=Skv, scale=128 ** -0.5, causal=True, out_dtype=torch.float32)
+        plan = {}
+        out = K.kivi_packed_attend(qt, _plan_out=plan, **args)
+        assert plan["path"] == 2 and K._tile_scratches, plan
+        assert torch.equal(out, K.kivi_packed_attend(qt, tiles=False, **args))
+        ref = oa.sdpa(host(qt.float()), host(kt.float()), host(vt.float()), 128 ** -0.5, causal=True)
+        err = float(np.max(np.abs(host(out) - ref)))
+        print(f"{dt}: max-abs err {err:.2e}")
+        assert err < TOL
+
+
 # ------------------------------------------------------------ packed cache path
 def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, causal=False, seed=0,
                  q_dtype=torch.float16, cap_extra=0, expect_path=None, tail_dtype=torch.float16, window=0):

@@ -773,6 +773,17 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+_tile_scratches: dict[tuple, torch.Tensor] = {}
+
+
+def _tile_scratch(device: torch.device, rows: int, units: int) -> torch.Tensor:
+    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    t = _tile_scratches.get(key)
+    if t is None or t.numel() < rows * units * PREFILL_TILE_BYTES:
+        t = _tile_scratches[key] = torch.empty(rows * units * PREFILL_TILE_BYTES, dtype=torch.uint8, device=device)
+    return t[: rows * units * PREFILL_TILE_BYTES].view(rows, units, PREFILL_TILE_BYTES)
+
+
 _sync_counters: dict[tuple, torch.Tensor] = {}
 
 
@@ -919,7 +930,8 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
     ``tiles``: the slots once more as ready-made tiles (:func:`kivi_prefill_tiles`); prefill-sized calls copy
     them instead of reconstructing the prefix in every block (same bits), other calls ignore them.  With
     ``tiles_stale_from`` a call that reads the tiles first rewrites them from that unit on (None: they are up to
-    date)."""
+    date).  A causal call over plain keys and values with two dozen row tiles or more per kv head makes such tiles
+    itself, in a scratch kept per device and stream (``tiles=False``: not even then)."""
     name = "kivi_packed_attend"
     if q.ndim != 4:
         raise ValueError(f"{name}: q must be 4D, got {tuple(q.shape)}")
@@ -953,6 +965,15 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         a.sink_k, a.sink_v, a.sink_pos = sk.data_ptr(), sv.data_ptr(), sp.data_ptr()
         a.sink_cap, a.sink_dtype = int(cap_s), _FLOAT_TAG[sk.dtype]
         keep += [sk, sv, sp]
+    if (tiles is None and n_packed == 0 and causal and D == 128 and Hq % Hkv == 0 and Hq // Hkv in (1, 2, 4, 8)
+            and (Hq // Hkv) * Sq >= 24 * 256 and k_tail.dtype in (torch.float16, torch.bfloat16)
+            and packed_lens is None and sinks is None and k_new is None):
+        # Plain keys and values under so many row tiles that every unit is read two dozen times or more: written
+        # once as tiles (a scratch kept per device and stream, 608 B per slot and kv head) they are copied into
+        # on-chip memory instead of being converted and transposed by every block that reads them; same bits.
+        tiles, tiles_stale_from = _tile_scratch(q.device, B * Hkv, -(-int(n_tail) // 32)), 0
+    if tiles is False:   # no tiles, not even the scratch above
+        tiles = None
     if tiles is not None:
         _check_tiles(name, tiles, B * Hkv, q.device)
         a.kv_tiles, a.tile_cap = tiles.data_ptr(), tiles.shape[1]
