@@ -561,15 +561,16 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
 
     // ---- this lane's query rows (score columns): row j = 32 wave + 16 rb + n of the block
+    const int qshift = 31 - __builtin_clz((unsigned)qp);   // the block covers a power of two of positions (256 / R)
     int lane_vis[PR_RB], lane_tvis[PR_RB];
     int lane_lo[PR_RB], lane_tlo[PR_RB];   // sliding window: first packed / tail token the row sees
     f16x8 qn[PR_RB][4];   // B operands: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of its row
 #pragma unroll
     for (int rb = 0; rb < PR_RB; ++rb) {
         const int j = 16 * PR_RB * wave + 16 * rb + n;
-        const int64_t pos = pos0 + j % qp;
-        const bool row_ok = pos < a.Sq && j / qp < R;
-        const int64_t qrow = (b * a.Hq + hkv * R + (j / qp < R ? j / qp : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
+        const int64_t pos = pos0 + (j & (qp - 1));
+        const bool row_ok = pos < a.Sq && (j >> qshift) < R;
+        const int64_t qrow = (b * a.Hq + hkv * R + ((j >> qshift) < R ? (j >> qshift) : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
         const int64_t vis = visible(row_ok ? pos : a.Sq - 1);
         lane_vis[rb] = (int)(vis < a.n_packed ? vis : a.n_packed);
         const int64_t tv = vis - a.n_packed;
@@ -877,10 +878,10 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int jr = 16 * PR_RB * wave + 16 * rb + 4 * blk + r;
-            const int64_t pr = pos0 + jr % qp;
+            const int64_t pr = pos0 + (jr & (qp - 1));
             const float mr = __shfl(m_run[rb], 4 * blk + r);
-            if (pr < a.Sq && jr / qp < R) {
-                const int64_t row = (b * a.Hq + hkv * R + jr / qp) * a.Sq + pr;
+            if (pr < a.Sq && (jr >> qshift) < R) {
+                const int64_t row = (b * a.Hq + hkv * R + (jr >> qshift)) * a.Sq + pr;
                 if (direct) {
                     // the only record of its row: what the merge would make of it (0 for a row that sees nothing)
                     const bool seen = mr != -INFINITY && L[rb][r] > 0.f;
