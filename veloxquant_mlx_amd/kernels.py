@@ -774,6 +774,7 @@ def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
 
 
 _tile_scratches: dict[tuple, torch.Tensor] = {}
+_TILE_SCRATCH_MAX = 2 << 30   # bytes; larger inputs are attended without tiles
 
 
 def _tile_scratch(device: torch.device, rows: int, units: int) -> torch.Tensor:
@@ -967,7 +968,8 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         keep += [sk, sv, sp]
     if (tiles is None and n_packed == 0 and causal and D == 128 and Hq % Hkv == 0 and Hq // Hkv in (1, 2, 4, 8)
             and (Hq // Hkv) * Sq >= 24 * 256 and k_tail.dtype in (torch.float16, torch.bfloat16)
-            and packed_lens is None and sinks is None and k_new is None):
+            and packed_lens is None and sinks is None and k_new is None
+            and B * Hkv * -(-int(n_tail) // 32) * PREFILL_TILE_BYTES <= _TILE_SCRATCH_MAX):
         # Plain keys and values under so many row tiles that every unit is read two dozen times or more: written
         # once as tiles (a scratch kept per device and stream, 608 B per slot and kv head) they are copied into
         # on-chip memory instead of being converted and transposed by every block that reads them; same bits.
