@@ -58,3 +58,15 @@ def test_argument_errors_surface_without_a_gpu():
     a.n_tail = 4
     assert lib.vq_kivi_attend(a) == _lib.VQ_ERR_INVALID
     assert "multiple of H_kv" in _lib.last_error()
+    # ready-made tiles: a missing or short buffer is refused by the writer and by the attention call
+    t = _lib.AttendArgs()
+    t.B, t.Hq, t.Hkv, t.Sq, t.D = 1, 4, 4, 1, 128
+    t.n_tail = 64
+    assert lib.vq_kivi_prefill_tiles(t, 0, 2) == _lib.VQ_ERR_INVALID
+    assert "kv_tiles must be given" in _lib.last_error()
+    t.kv_tiles, t.tile_cap = 4096, 1
+    assert lib.vq_kivi_prefill_tiles(t, 0, 2) == _lib.VQ_ERR_INVALID
+    assert "do not lie inside" in _lib.last_error()
+    assert lib.vq_kivi_attend(t) == _lib.VQ_ERR_INVALID
+    assert "room for all 64 slots" in _lib.last_error()
+
