@@ -247,6 +247,41 @@ def test_plain_prefill_with_many_row_tiles_goes_through_a_tile_scratch():
         assert err < TOL
 
 
+@pytest.mark.parametrize("Hq,Hkv,Sq,n_packed,n_tail,b,g,meta,causal,window", [
+    (8, 1, 40, 384, 77, 2, 128, torch.float32, True, 0),      # eight heads per kv head, float32 scale / zero
+    (3, 3, 300, 256, 45, 4, 64, torch.float16, False, 0),     # one head per kv head, no mask, ragged row tile
+    (4, 2, 200, 1024, 200, 4, 32, torch.float16, True, 300),  # window that skips packed units
+    (4, 1, 100, 0, 333, 4, 32, torch.float16, True, 0),       # no packed prefix
+])
+def test_tiles_and_producer_blocks_agree_bit_for_bit(Hq, Hkv, Sq, n_packed, n_tail, b, g, meta, causal, window):
+    """The 256-row blocks fed with ready-made tiles against the same blocks reconstructing the units themselves, over
+    shapes the oracle-checked cases above do not all reach: the outputs are identical."""
+    require_gpu()
+    B, D, per = 2, 128, 32 // b
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(Hq * 100 + Sq)
+    k = torch.randn((B, Hkv, n_packed + n_tail, D), generator=gen, device=dev).to(torch.float16)
+    v = torch.randn((B, Hkv, n_packed + n_tail, D), generator=gen, device=dev).to(torch.float16)
+    q = torch.randn((B, Hq, Sq, D), generator=gen, device=dev).to(torch.bfloat16)
+    cache = dict(n_packed=n_packed, bits=b, group_size=g, v_layout="token", n_tail=n_tail,
+                 k_tail=k[:, :, n_packed:].to(torch.bfloat16).contiguous(), v_tail=v[:, :, n_packed:].to(torch.bfloat16).contiguous())
+    if n_packed:
+        kp, ks, kz = K.kivi_quant_pack(k[:, :, :n_packed].contiguous(), -2, g, b, meta_dtype=meta)
+        vp, vs, vz = K.kivi_quant_pack(v[:, :, :n_packed].contiguous(), -1, g, b, meta_dtype=meta, v_layout="token")
+        cache.update(k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz)
+    args = dict(scale=D ** -0.5, causal=causal, sliding_window=window, out_dtype=torch.float32, **cache)
+    plan = {}
+    plain = K.kivi_packed_attend(q, tiles=False, _plan_out=plan, **args)
+    assert plan["path"] == 2, plan
+    tiles = K.prefill_tiles_empty(B, Hkv, n_packed + n_tail, dev)
+    tiles.fill_(0xFF)
+    fed = K.kivi_packed_attend(q, tiles=tiles, tiles_stale_from=0, **args)   # the call writes the tiles itself
+    assert torch.equal(fed, plain), float((fed - plain).abs().max())
+    assert torch.isfinite(fed).all()
+    again = K.kivi_packed_attend(q, tiles=tiles, **args)                     # and finds them up to date afterwards
+    assert torch.equal(again, plain)
+
+
 # ------------------------------------------------------------ packed cache path
 def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, causal=False, seed=0,
                  q_dtype=torch.float16, cap_extra=0, expect_path=None, tail_dtype=torch.float16, window=0):
