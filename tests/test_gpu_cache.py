@@ -426,6 +426,15 @@ def test_prefill_tiles_change_no_bit_and_follow_the_cache(bits, g, dtype):
         c.update_and_fetch(k.clone(), v.clone())
         outs.append(c.fused_sdpa(q, scale, fixed_order=True))
     assert torch.equal(outs[0], outs[1]) and caches[0]._tiles is None and caches[0].nbytes == caches[1].nbytes
+    # a prefill that would need more tile memory than the cache allows goes on without tiles, same bits
+    k, v = mk(C)
+    q = torch.randn((B, Hq, C, D), generator=gen, device=dev).to(dtype)
+    caches[0].prefill_tiles_max_bytes = 1 << 20
+    outs = []
+    for c in caches:
+        c.update_and_fetch(k, v)
+        outs.append(c.fused_sdpa(q, scale, causal=True))
+    assert torch.equal(outs[0], outs[1]) and caches[0]._tiles is None
 
 
 def test_config4_every_chunk_against_the_oracle_on_sampled_rows():

@@ -123,6 +123,7 @@ class KIVIKVCache(FP16KVCache):
         # (scratch of the prefill phase, given back at the first decode step); the first _tiles_packed units
         # hold packed slots that cannot change any more
         self.prefill_tiles = os.environ.get("VELOXQUANT_PREFILL_TILES", "1") != "0"
+        self.prefill_tiles_max_bytes = 256 << 20   # per cache (layer); a longer prefill goes on without tiles
         self._tiles = None
         self._tiles_packed = 0
 
@@ -371,9 +372,13 @@ class KIVIKVCache(FP16KVCache):
                 self._tiles = None   # decoding has begun
             return False
         units = -(-(nq + n_tail) // 32)
+        if B * H * units * K.PREFILL_TILE_BYTES > self.prefill_tiles_max_bytes:
+            self._tiles = None
+            return False
         t = self._tiles
         if t is None or t.shape[0] != B * H or t.shape[1] < units or t.device != q.device:
             room = self._packed_cap + (self._tail_k.shape[2] if self._tail_k is not None else 0)
+            room = min(room, self.prefill_tiles_max_bytes // (B * H * K.PREFILL_TILE_BYTES) * 32)
             t = self._tiles = K.prefill_tiles_empty(B, H, max(room, 32 * units), q.device)
             self._tiles_packed = 0
         kw["tiles"], kw["tiles_stale_from"] = t, min(self._tiles_packed, nq // 32)
