@@ -260,6 +260,24 @@ def _decode_2bit_case(torch, dev, B):
     return c, (lambda: c.fused_sdpa(q, 1 / math.sqrt(D))), _algorithmic_bytes_per_layer(B, Hkv, 32768, D, 2, 32)
 
 
+def _decode_cfg1_case(torch, dev):
+    """Config 1: 32 query / 8 kv heads, D=128, B=1, 8192 tokens as 2-bit group-32 packed codes plus the
+    most recent 128 tokens in fp16, one fp16 query token.  Bytes: codes 2 x 2,097,152 + fp16 scale / zero
+    2 x 1,048,576 + tail 524,288 + query and output 16,384 = 6,832,128."""
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+    D, Hq, Hkv, S, R = 128, 32, 8, 8192, 128
+    cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=2, kivi_group_size=32, residual_length=R,
+                        fused_sdpa=True, fused_sdpa_memory_bound=True)
+    c = KVCacheFactory.create(cfg)
+    k, v = _synthetic_layer(torch, 1, Hkv, S + R, D, 3, dev)
+    c.update_and_fetch(k, v)
+    assert c._n_quantized == S, c._n_quantized
+    q = torch.randn((1, Hq, 1, D), device=dev).to(torch.float16)
+    nbytes = _algorithmic_bytes_per_layer(1, Hkv, S, D, 2, 32) + 2 * Hkv * R * D * 2 + 2 * Hq * D * 2
+    assert nbytes == 6832128, nbytes
+    return c, (lambda: c.fused_sdpa(q, 1 / math.sqrt(D))), nbytes
+
+
 def _prefill_case(torch, dev):
     """Config 4: 8 chunks of 512 bf16 queries over a 4-bit packed prefix of 4096 tokens plus their own,
     quantise-on-write (group 32, residual 128).  Returns a function that runs one whole pass and
@@ -403,6 +421,17 @@ def _extras(torch, K, dev):
                                         "ms_graph": round(ms_g, 5), "frac_hbm_graph": round(nbytes / ms_g / 1e6 / HBM_PEAK_GBS, 4),
                                         "note": "ms: one Python call per launch; ms_graph: the same launches replayed from a HIP graph"}
         del c
+    # config 1: Llama-3-8B layer, one sequence, 8192 tokens as 2-bit group-32 codes plus a 128-token fp16 tail
+    c1, fn1, nbytes1 = _decode_cfg1_case(torch, dev)
+    for _ in range(3):
+        fn1()
+    ms1, ms1_g = _side_ms(fn1, 30, torch), _graph_ms(fn1, torch)
+    ex["decode_cfg1"] = {"ms": round(ms1, 5), "GBps": round(nbytes1 / ms1 / 1e6, 1), "bytes": nbytes1,
+                         "frac_hbm": round(nbytes1 / ms1 / 1e6 / HBM_PEAK_GBS, 4),
+                         "ms_graph": round(ms1_g, 5), "frac_hbm_graph": round(nbytes1 / ms1_g / 1e6 / HBM_PEAK_GBS, 4),
+                         "note": "32 query / 8 kv heads, B=1, 8192 packed tokens + 128 fp16 tail tokens, one launch; "
+                                 "ms: one Python call per launch, ms_graph: replayed from a HIP graph"}
+    del c1
     # config 0: quantise + pack of one layer's K and V [1,8,2048,128], 4-bit, group 32; and a large flush
     for name, shape in (("cfg0_[1,8,2048,128]", (1, 8, 2048, 128)), ("large_[16,8,8192,128]", (16, 8, 8192, 128))):
         k, v = _synthetic_layer(torch, shape[0], shape[1], shape[2], shape[3], 11, dev)
@@ -425,6 +454,25 @@ def _extras(torch, K, dev):
         ms_qp2 = _side_ms(qp2, 30, torch)
         ex[f"quant_pack_two_calls_{name}"] = {"ms": round(ms_qp2, 5), "GBps": round(b_qp / ms_qp2 / 1e6, 1), "bytes": b_qp}
         ex[f"quant_dequant_{name}"] = {"ms": round(ms_rt, 5), "GBps": round(b_rt / ms_rt / 1e6, 1), "bytes": b_rt}
+        if shape[0] == 1:
+            # config 0's second half: the standalone dequantise of the packed layer back to fp16
+            # (scalar_decode_once, metal/_scalar_attend.py:650-699): packed codes + fp16 scale / zero in,
+            # fp16 K and V out -- the quantise+pack traffic in reverse
+            S_, D_ = shape[2], shape[3]
+            kp, ks, kz = K.kivi_quant_pack(k, -2, 32, 4)
+            vp, vs, vz = K.kivi_quant_pack(v, -1, 32, 4, v_layout="token")
+            def dq():
+                K.kivi_dequant(kp, ks, kz, -2, 32, 4, S_, D_)
+                K.kivi_dequant(vp, vs, vz, -1, 32, 4, S_, D_, v_layout="token")
+            for _ in range(3):
+                dq()
+            ms_dq, ms_dq_g = _side_ms(dq, 30, torch), _graph_ms(dq, torch)
+            ex["dequant_cfg0"] = {"ms": round(ms_dq, 5), "GBps": round(b_qp / ms_dq / 1e6, 1), "bytes": b_qp,
+                                  "ms_graph": round(ms_dq_g, 5), "GBps_graph": round(b_qp / ms_dq_g / 1e6, 1),
+                                  "note": "K.kivi_dequant of K and V (two launches); ms: Python call per launch, "
+                                          "ms_graph: replayed from a HIP graph"}
+            ms_qp_g = _graph_ms(qp, torch)
+            ex[f"quant_pack_{name}"].update({"ms_graph": round(ms_qp_g, 5), "GBps_graph": round(b_qp / ms_qp_g / 1e6, 1)})
     # config 4: causal prefill of 4096 bf16 queries in chunks of 512 over a 4-bit packed prefix of 4096
     # tokens plus their own tokens, quantise-on-write (group 32, residual 128)
     prefill_pass = _prefill_case(torch, dev)
@@ -494,8 +542,8 @@ def _extras(torch, K, dev):
         fn()
     ms = _side_ms(fn, 5, torch)
     ex["zipcache_keys_[16,8,8192,128]"] = {"ms": round(ms, 5), "GBps": round(nb / ms / 1e6, 1), "bytes": nb,
-                                           "note": "fp16 keys in, fp16 mixed-precision reconstruction out; the routing "
-                                                   "(norms, ranks, gather, scatter) is torch around two kernel launches"}
+                                           "note": "fp16 keys in, fp16 mixed-precision reconstruction out: four launches "
+                                                   "(row norms, routing order, one routed round trip per bit width)"}
     del zc
     del kk, kc
     # config 2 with the key transform in front: (keys / smooth) @ Hadamard -> indices, one launch,

@@ -437,6 +437,48 @@ def test_prefill_tiles_change_no_bit_and_follow_the_cache(bits, g, dtype):
     assert torch.equal(outs[0], outs[1]) and caches[0]._tiles is None
 
 
+def test_prefill_tile_scratch_is_given_back_by_every_kind_of_decode_step():
+    """The tile scratch of a memory-bound prefill lives only until decoding begins: a single-token append, a
+    single-query attend with per-sequence ``lengths`` and the layer-stacked launch all return ``nbytes`` to the
+    packed size."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    B, Hq, Hkv, D, C = 2, 16, 4, 128, 256
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(9)
+    scale = 1 / math.sqrt(D)
+
+    def prefilled(tiles=True):
+        c = _make(bit_width_inlier=4, kivi_group_size=32, residual_length=128, fused_sdpa=True, fused_sdpa_memory_bound=True)
+        c.prefill_tiles = tiles
+        for _ in range(3):
+            k = torch.randn((B, Hkv, C, D), generator=gen, device=dev).to(torch.float16)
+            v = torch.randn((B, Hkv, C, D), generator=gen, device=dev).to(torch.float16)
+            q = torch.randn((B, Hq, C, D), generator=gen, device=dev).to(torch.float16)
+            c.update_and_fetch(k, v)
+            c.fused_sdpa(q, scale, causal=True)
+        return c
+
+    plain = prefilled(tiles=False).nbytes
+    q1 = torch.randn((B, Hq, 1, D), generator=gen, device=dev).to(torch.float16)
+    # (a) decode with per-sequence lengths, no append in between
+    c = prefilled()
+    assert c._tiles is not None and c.nbytes > plain
+    c.fused_sdpa(q1, scale, lengths=torch.tensor([c.offset, c.offset - 5]))
+    assert c._tiles is None and c.nbytes == plain
+    # (b) the single-token append alone
+    c = prefilled()
+    c.update_and_fetch(torch.randn((B, Hkv, 1, D), generator=gen, device=dev).to(torch.float16),
+                       torch.randn((B, Hkv, 1, D), generator=gen, device=dev).to(torch.float16))
+    assert c._tiles is None
+    # (c) the layer-stacked launch
+    layers = [prefilled(), prefilled()]
+    assert all(l._tiles is not None for l in layers)
+    stack = LayerStackedKIVICache.from_layers(layers)
+    stack.fused_sdpa_all(torch.stack([q1, q1]), scale)
+    assert all(l._tiles is None for l in layers)
+
+
 def test_config4_every_chunk_against_the_oracle_on_sampled_rows():
     """Benchmark configuration 4 at full size, every one of the 8 chunks: for one kv head the host
     quantises the same bf16 keys and values with the numpy oracle (one shot over the packed prefix:

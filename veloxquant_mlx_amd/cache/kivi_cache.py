@@ -227,6 +227,8 @@ class KIVIKVCache(FP16KVCache):
     def _update_memory_bound(self, keys: torch.Tensor, values: torch.Tensor):
         B, H, S, D = keys.shape
         self._store_pending()
+        if S == 1:
+            self._drop_tiles()   # decoding has begun: the prefill scratch goes back
         n_tail = self.offset - self._n_quantized
         need = n_tail + S
         if (S == 1 and self._n_quantized > 0 and self._tail_k is not None and need <= self._tail_k.shape[2]
@@ -325,6 +327,8 @@ class KIVIKVCache(FP16KVCache):
             raise RuntimeError("KIVIKVCache.fused_sdpa called before any tokens were cached via update_and_fetch.")
         nq = self._n_quantized
         n_tail = self.offset - nq
+        if q.shape[2] == 1:
+            self._drop_tiles()   # a decode step, with or without per-sequence lengths
         if self._pending is not None and q.shape[2] != 1:
             self._store_pending()
         if self._memory_bound:
@@ -368,8 +372,6 @@ class KIVIKVCache(FP16KVCache):
         if not (self.prefill_tiles and self._memory_bound and self._v_layout == "token" and D == 128 and Hq % H == 0
                 and Hq // H in (1, 2, 4, 8) and (Hq // H) * Sq >= 256 and nq % 32 == 0 and "sinks" not in kw
                 and (n_tail == 0 or self._tail_k.dtype in (torch.float16, torch.bfloat16))):
-            if Sq == 1:
-                self._tiles = None   # decoding has begun
             return False
         units = -(-(nq + n_tail) // 32)
         if B * H * units * K.PREFILL_TILE_BYTES > self.prefill_tiles_max_bytes:
@@ -383,6 +385,11 @@ class KIVIKVCache(FP16KVCache):
             self._tiles_packed = 0
         kw["tiles"], kw["tiles_stale_from"] = t, min(self._tiles_packed, nq // 32)
         return True
+
+    def _drop_tiles(self) -> None:
+        """Give the prefill tile scratch back (it is worth ~1.2x an fp16 copy of K and V while it lives; the
+        reference's memory-bound mode never holds more than one transient reconstruction)."""
+        self._tiles, self._tiles_packed = None, 0
 
     def _extra_attend_args(self) -> dict:
         """Further arguments of the attention call (subclasses with rows kept outside the packed store)."""

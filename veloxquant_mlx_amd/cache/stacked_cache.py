@@ -158,6 +158,7 @@ class LayerStackedKIVICache:
                 raise RuntimeError(f"LayerStackedKIVICache.fused_sdpa_all: layer {l} has no packed tokens yet")
             if c._shape_bhd[0] != B:
                 raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: layer {l} holds batch {c._shape_bhd[0]}, q has {B}")
+            c._drop_tiles()   # the stacked launch never reads a layer's prefill tile scratch
         if not self._packed_in_place(B):
             self._restack_packed(B)
         ti = self._which_tail(B)

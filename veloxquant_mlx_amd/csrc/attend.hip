@@ -64,10 +64,10 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     p.split_len = len;
     // MFMA decode path: the tail is run by up to eight waves of split 0, every wave into a partial of
     // its own.  A launch with many blocks is bound by throughput: one wave takes eight units of 32
-    // tokens (the other waves stream meanwhile); a launch with few is bound by latency: two units a wave.
+    // tokens (the other waves stream meanwhile); a launch with few is bound by latency: one unit a wave.
     p.nparts = p.nsplit;
     if (p.path == 1 && a.n_tail > 0) {
-        int64_t tw = cdiv(cdiv(a.n_tail, 32), units >= 64 ? 8 : 2);
+        int64_t tw = cdiv(cdiv(a.n_tail, 32), units >= 64 ? 8 : 1);
         p.nparts += (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw);
     }
     return p;

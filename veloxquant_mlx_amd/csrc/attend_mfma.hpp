@@ -115,6 +115,66 @@ __device__ __forceinline__ void unpack8_pair_upper2(u32 w0, u32 w1, u32 magic, f
     unpack8_pair_at<2, 0, -2, -4, -6>(pack64(w0, w1), magic, a0, a1);
 }
 
+// ---- codes as fp16 SUBNORMALS (the packed decode kernel).
+// A half whose exponent field is zero reads mantissa * 2^-24, and the matrix unit takes such
+// operands exactly.  A code left where a shifted packed word holds it, at mantissa bit POS,
+// therefore reads code * 2^(POS - 24): one AND per two codes (one per register of the
+// operand) and no constant to subtract afterwards.  The other operand of the same k-slot
+// carries 2^(E - POS), an exact scaling, so every product is code * value * 2^(E - 24).
+// The unit aligns the products of an instruction to the largest NOMINAL exponent among them
+// (-14 for every subnormal, whatever its leading zeros) and keeps about 25 bits below it: a
+// code at bit POS is good to 2^-(15 + POS) of the instruction's largest other-operand value,
+// which is why the fields sit at bits 2, 4, 6, 8 (2-bit) and 2, 6 (4-bit) and not lower.
+template <int BITS> struct Sub {
+    // mantissa bit of k-slot pair p (p = 0..3) of an operand
+    static constexpr int pos(int p) { return BITS == 2 ? 2 + 2 * p : 2 + 4 * (p & 1); }
+    static constexpr u32 mask(int p) { return (BITS == 2 ? 0x00030003u : 0x000F000Fu) << pos(p); }
+    // exponents carried by the other operand: keys 2^(EK - pos), values 2^(EV - pos) >= 1
+    static constexpr int EK = BITS == 2 ? 5 : 4;
+    static constexpr int EV = BITS == 2 ? 8 : 6;
+    // probabilities may reach 2^SLACK before the softmax reference moves; times 2^(EV - 2) and
+    // the value scale they must stay inside fp16 (2^SLACK * 2^(EV - 2) = 2^8 either way)
+    static constexpr float SLACK = BITS == 2 ? 2.f : 4.f;
+    static constexpr float KSCALE = (float)(1 << (24 - EK));       // scores: accumulator * KSCALE
+    static constexpr float KSCALE_INV = 1.f / (float)(1 << (24 - EK));
+    static constexpr float VSCALE = (float)(1 << (24 - EV));       // outputs: accumulator * VSCALE
+    static constexpr float wk(int p) { return EK >= pos(p) ? (float)(1 << (EK >= pos(p) ? EK - pos(p) : 0))
+                                                           : 1.f / (float)(1 << (pos(p) > EK ? pos(p) - EK : 0)); }
+    static constexpr float wv(int p) { return (float)(1 << (EV - pos(p))); }
+    static constexpr float wv_inv(int p) { return 1.f / (float)(1 << (EV - pos(p))); }
+};
+template <int BITS> __device__ __forceinline__ f16x8 sub4(u32 w) {
+    return as_h8(w & Sub<BITS>::mask(0), w & Sub<BITS>::mask(1), w & Sub<BITS>::mask(2), w & Sub<BITS>::mask(3));
+}
+// 4-bit: the eight codes of w0 (and of w1) as one operand each, pair p = (code p, code p + 4);
+// codes 0, 1 come from the word moved up by two bits, codes 2, 3 from the word moved down by six
+__device__ __forceinline__ void sub_unpack4(u32 w0, u32 w1, f16x8 &a0, f16x8 &a1) {
+    const u64 x = pack64(w0, w1), l = shift64<2>(x), r = shift64<-6>(x);
+    constexpr u32 m0 = Sub<4>::mask(0), m1 = Sub<4>::mask(1);
+    a0 = as_h8((u32)l & m0, (u32)l & m1, (u32)r & m0, (u32)r & m1);
+    a1 = as_h8((u32)(l >> 32) & m0, (u32)(l >> 32) & m1, (u32)(r >> 32) & m0, (u32)(r >> 32) & m1);
+}
+// 2-bit: the sixteen codes of w0 (and of w1) as two operands each: `lo*` codes 0-3 | 8-11, `up*`
+// codes 4-7 | 12-15, pair p = (code p, code p + 8) of that set
+__device__ __forceinline__ void sub_unpack2(u32 w0, u32 w1, f16x8 &lo0, f16x8 &up0, f16x8 &lo1, f16x8 &up1) {
+    const u64 x = pack64(w0, w1), l = shift64<2>(x), r = shift64<-6>(x);
+    lo0 = sub4<2>((u32)l);
+    lo1 = sub4<2>((u32)(l >> 32));
+    up0 = sub4<2>((u32)r);
+    up1 = sub4<2>((u32)(r >> 32));
+}
+// largest of three / two without the quieting of signalling NaNs that fmaxf asks for (scores are never NaN)
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float max_raw(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+
 // channel (0..31 inside a lane's 32-channel slice) of k-slot pair p of k-step ks
 template <int BITS> __device__ __forceinline__ constexpr int kchan_lo(int ks, int p) {
     return BITS == 4 ? 8 * ks + p : 16 * (ks / 2) + 4 * (ks % 2) + p;
@@ -302,12 +362,6 @@ __device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, c
 
     const bool bf16 = a.tail_dtype == VQ_BF16;
     const int64_t tbase = bh * a.tail_cap * MF_D;
-    f16x8 qT[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        qT[ks] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (i < R) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * q_stride + 32 * blk + 8 * ks);
-    }
     const f16x8 ones = ones8();
     const int n_tu = (int)((a.n_tail + 31) / 32);
 
@@ -340,6 +394,13 @@ __device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, c
     };
     auto compute = [&](int u, const TUnit &d) {
         const int64_t base = (int64_t)u * 32;
+        // the query operand is read again for every unit: sixteen registers that need not live across the loads
+        f16x8 qT[4];
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            qT[ks] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (i < R) qT[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + i * q_stride + 32 * blk + 8 * ks);
+        }
         f32x4 S[2];
 #pragma unroll
         for (int Tt = 0; Tt < 2; ++Tt) {
@@ -362,13 +423,11 @@ __device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, c
         }
         acc.O[8] = __builtin_amdgcn_mfma_f32_16x16x32_f16(P, ones, acc.O[8], 0, 0, 0);
     };
-    // two units of the wave in flight at a time
-    for (int u = w; u < n_tu; u += 2 * T) {
-        TUnit d0, d1;
-        load(u, d0);
-        if (u + T < n_tu) load(u + T, d1);
-        compute(u, d0);
-        if (u + T < n_tu) compute(u + T, d1);
+    // one unit in registers at a time (64 of them): the kernel runs three waves to a SIMD
+    for (int u = w; u < n_tu; u += T) {
+        TUnit d;
+        load(u, d);
+        compute(u, d);
     }
     // the partial: accumulator register r of lane (i, blk) is row 4*blk + r, channels 8*i .. 8*i + 7;
     // the maximum of row i sits in lane i of every lane group

@@ -2,16 +2,16 @@
 //
 // One block of eight waves per (kv head, token split), one block per CU.  Every wave streams
 // units of 32 tokens and never reconstructs a key or a value: both products run on the raw
-// codes, which are dropped from the packed word into the mantissa of an fp16
-// constant by one and-or per two codes (value = offset + code, exact), and every
-// affine term is pushed onto the matrix unit:
+// codes.  A code stays where the (shifted) packed word holds it, inside the mantissa of an fp16
+// SUBNORMAL -- one AND per two codes, value code * 2^(bit - 24), exact, no offset -- and the
+// other operand of that k-slot carries the matching power of two (see Sub<BITS>):
 //
-//   scores   S^T[token, col]  = sum_d (off + c_td) (q s)_d           A = codes, B = folded query
-//                             + sum_d z_d q_d - off * sum_d s_d q_d    the accumulator the product starts from
-//   output   O^T[chan, col]   = sum_t (off + c_t,chan) (P s_g)[t, col]   A = codes, B = P scaled by the column's
-//                                                                      channel group (hi + remainder)
-//   sums     Z[i, col]        = sum_t A_z[i, t] P[t, col]             rows i: value zeros of group i, value
-//                                                                      scales of group i, ones (the denominator)
+//   scores   S^T[token, col]  = sum_d c_td (q s)_d 2^(EK - 24)     A = codes, B = folded query
+//                             + 2^(EK - 24) sum_d z_d q_d            the accumulator the product starts from
+//   output   O^T[chan, col]   = sum_t c_t,chan (P s_g)[t, col] 2^(EV - 24)   A = codes, B = P scaled by the
+//                                                                    column's channel group (hi + remainder)
+//   sums     Z[i, col]        = sum_t A_z[i, t] P[t, col]             rows i: value zeros of group i, ones
+//                                                                    (the denominator)
 //
 // The 16 columns of a tile carry the RTP (4 or 8) query rows of the block several times over:
 //   * first product: column n is query row n % RTP; columns with (n / RTP) even hold the fp16
@@ -28,8 +28,9 @@
 //
 // Opening a token group (keys: per-channel scale s_d, zero z_d per group of tokens) is shared
 // work of the wave: every lane forms q*s (high part and remainder) for eight channels of one
-// row, the pieces go through a small LDS image and come back in operand order; the row bias is
-// one MFMA chain with the group's zeros in operand rows 0-7 and its scales in rows 8-15.
+// row, the pieces go through a small LDS image and come back in operand order; the row bias
+// sum_d z_d q_d is one MFMA chain with the group's zeros in every operand row, so that each
+// accumulator register of a lane holds the bias of the lane's column.
 //
 // Keys are packed along channels, so a lane's eight k-slots of the first product are eight
 // channels of one token; values are packed along tokens (VQ_V_TOKEN_PACKED), so a lane's eight
@@ -42,17 +43,17 @@
 // wave are set by the ring, not by the register file.  The softmax keeps a lazily updated
 // reference maximum, so the common path has no cross-lane traffic at all.
 #pragma once
+#include <atomic>
+
 #include "attend_mfma.hpp"
 
 namespace vq {
 
 
-// One block of PK_WAVES waves per CU (two waves per SIMD, the register file split in two).
-#ifndef VQ_PK_WAVES
-#define VQ_PK_WAVES 8
-#endif
-constexpr int PK_WAVES = VQ_PK_WAVES;
-constexpr int PK_THREADS = 64 * PK_WAVES;
+// One block per CU, of twelve waves (three per SIMD, 168 registers each) where twelve rings of at least
+// two units fit the CU's LDS, of eight waves otherwise: Ring<...>::WAVES.  The unit loop is a chain of
+// LDS round trips and dependent matrix products; the third wave of a SIMD fills what two leave idle.
+constexpr int PK_MAX_WAVES = 12;
 // Every lambda below must be inlined at every call: a closure left in memory would be read back
 // with vector loads, whose completion the ring's copy counter cannot tell from its own.
 #define VQ_INLINE_LAMBDA __attribute__((always_inline))
@@ -92,13 +93,13 @@ template <int GV, int RTP> struct Cols {
 };
 
 // Per-wave state of the packed kernel.
-template <int NP, bool OFF_TILES> struct PackedAcc {
-    f32x4 O[8];     // tile nt, register r: channel 16*nt + 4*blk + r of the lane's column, still carrying
-                    // off * sum_t (P s_g)[t]
-    f32x4 Z;        // register r = operand row 4*blk + r: sum_t P z_g (rows g < GV), sum_t P s_g (rows GV + g),
-                    // sum_t P (rows >= 8)
-    f32x4 Off[OFF_TILES ? NP : 1];   // float32 scale / zero only: sum_t (P s_g)[t] from the very operands of O
+struct PackedAcc {
+    f32x4 O[8];     // tile nt, register r: channel 16*nt + 4*blk + r of the lane's column, times 2^(EV - 24)
+    f32x4 Z;        // register r = operand row 4*blk + r: sum_t P z_g (rows g < GV), sum_t P (rows >= 8)
     float m_run;    // softmax reference, log2 domain, of the lane's column (query row)
+    float thr;      // m_run + SLACK: a score above it moves the reference
+    float nm[4];    // what register r of a score tile adds before exp2: -m_run + (EV - pos(r)), the weight of
+                    // its k-slot pair in the second product
 };
 
 template <int BITS, typename M, int NP> struct PackedUnit {
@@ -121,10 +122,12 @@ constexpr int PK_QIMG_ROW = 272;              // bytes between rows of a wave's 
 // that opens a group brings them along.  Blocks start on a group boundary, so units open a
 // group every UPG units.
 // The exchange arrays of the waves (cross-wave merge) share the rings' bytes:
-// accumulators [PK_WAVES][MF_ROWS][MF_D], zero-point sums [PK_WAVES][MF_ROWS][8], maxima and
-// sums [PK_WAVES][MF_ROWS]
-constexpr int EX_O = PK_WAVES * MF_ROWS * MF_D * 4, EX_Z = PK_WAVES * MF_ROWS * 8 * 4, EX_M = PK_WAVES * MF_ROWS * 4;
-constexpr int EX_BYTES = EX_O + EX_Z + 2 * EX_M;
+// accumulators [WAVES][MF_ROWS][MF_D], zero-point sums [WAVES][MF_ROWS][8], maxima and
+// sums [WAVES][MF_ROWS]
+constexpr int ex_o(int waves) { return waves * MF_ROWS * MF_D * 4; }
+constexpr int ex_z(int waves) { return waves * MF_ROWS * 8 * 4; }
+constexpr int ex_m(int waves) { return waves * MF_ROWS * 4; }
+constexpr int ex_bytes(int waves) { return ex_o(waves) + ex_z(waves) + 2 * ex_m(waves); }
 constexpr int PK_ALIGN = 128;                 // tokens: blocks start on a multiple of the largest token group
 constexpr int PK_STATIC_LDS = 4096;           // query rows, constant rows, counters (static block-shared memory)
 
@@ -140,13 +143,18 @@ template <int BITS, typename M, int GV, int RTP> struct Ring {
     static constexpr int UNIT_COPIES = (BITS == 4 ? 4 : 2) + 2 * VM_COPIES, GROUP_COPIES = 2 * KM_COPIES;
     static constexpr int UPG = 4 / GV;             // units per token group
     static constexpr int QIMG = 2 * RTP * PK_QIMG_ROW;
-    // the block has the CU's 160 KB to itself
-    static constexpr int BUDGET = (160 * 1024 - PK_STATIC_LDS) / PK_WAVES - QIMG;
     // a group slot is read only while its group is opened, and refilled by the opener issued
     // ceil(DEPTH / UPG) openers later -- at the earliest in the same pass, after that read
     static constexpr int group_slots(int depth) { return (depth + UPG - 1) / UPG; }
     static constexpr int bytes_at(int depth) { return depth * SLOT + group_slots(depth) * GROUP_SLOT; }
+    // the block has the CU's 160 KB to itself
+    static constexpr int budget(int waves) { return (160 * 1024 - PK_STATIC_LDS) / waves - QIMG; }
+    // (float32 scale / zero: the unit loop holds more than a third of the register file, eight waves)
+    static constexpr int WAVES = MSZ == 2 && bytes_at(2) <= budget(PK_MAX_WAVES) ? PK_MAX_WAVES : 8;
+    static constexpr int THREADS = 64 * WAVES;
+    static constexpr int BUDGET = budget(WAVES);
     static constexpr int DEPTH = bytes_at(5) <= BUDGET ? 5 : bytes_at(4) <= BUDGET ? 4 : bytes_at(3) <= BUDGET ? 3 : 2;
+    static_assert(bytes_at(DEPTH) <= BUDGET, "the rings do not fit the CU's LDS");
     static constexpr int GROUP_SLOTS = group_slots(DEPTH);
     static constexpr int GROUP_OFF = DEPTH * SLOT;
     static constexpr int QIMG_OFF = GROUP_OFF + GROUP_SLOTS * GROUP_SLOT;
@@ -154,7 +162,7 @@ template <int BITS, typename M, int GV, int RTP> struct Ring {
     // least (DEPTH - 1) / UPG open a group
     static constexpr int LATER = (DEPTH - 1) * UNIT_COPIES + ((DEPTH - 1) / UPG) * GROUP_COPIES;
     static constexpr int WAVE_BYTES = QIMG_OFF + QIMG;
-    static constexpr int BYTES = PK_WAVES * WAVE_BYTES > EX_BYTES ? PK_WAVES * WAVE_BYTES : EX_BYTES;
+    static constexpr int BYTES = WAVES * WAVE_BYTES > ex_bytes(WAVES) ? WAVES * WAVE_BYTES : ex_bytes(WAVES);
     // Units are handed out to the waves in chunks of CHUNK consecutive units: whole token groups,
     // and at least DEPTH units, so that the copies never run more than one chunk ahead of
     // the arithmetic.
@@ -163,9 +171,9 @@ template <int BITS, typename M, int GV, int RTP> struct Ring {
 };
 
 // The query rows of the block as fp16 in LDS, PK_QROW halves apart; rows the tile does not have are zero.
-template <int RTP>
+template <int RTP, int THREADS>
 __device__ __forceinline__ void stage_query(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw) {
-    for (int e = tid; e < RTP * MF_D / 8; e += PK_THREADS) {
+    for (int e = tid; e < RTP * MF_D / 8; e += THREADS) {
         const int row = e / (MF_D / 8), d = 8 * (e % (MF_D / 8));
         f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (tile.valid(row)) {
@@ -190,7 +198,7 @@ template <int N> __device__ __forceinline__ float row_ror(float x) {
 template <int BITS, typename M, int GV, int RTP>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, float c, int64_t t_begin,
                                              int n_units, int lane_vis, int full_vis, int lane_lo, int lo_edge, int lane, int wave,
-                                             PackedAcc<Cols<GV, RTP>::NP, sizeof(M) != 2> &acc, const f16 *s_qraw,
+                                             PackedAcc &acc, const f16 *s_qraw,
                                              const char *s_const, char *ring, int *s_next, int order) {
     using CL = Cols<GV, RTP>;
     constexpr int PER = 32 / BITS;           // codes per word
@@ -200,8 +208,9 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     constexpr int G = MF_D / GV;             // tokens per key group = channels per value group
     constexpr u32 MSZ = sizeof(M);
     constexpr bool F32META = sizeof(M) != 2;
+    using SB = Sub<BITS>;
     const int n = lane & 15, blk = lane >> 4;
-    const u32 magic = vreg_const(Magic<BITS>::bits);
+    const float cs = c * SB::KSCALE;   // accumulated scores carry 2^(EK - 24)
     const int64_t cap = a.cap_tokens;
     const bool fixed_order = (order & 1) != 0, wait_all = (order & 2) != 0;
 
@@ -271,16 +280,17 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 
     // ---- what a lane reads back (ordinary LDS loads)
     const int vrow = BITS == 4 ? blk : blk >> 1;          // word row of the lane's eight tokens
-    const u32 vshift = BITS == 2 ? 8u * (blk & 1) : 0u;
+    // 2-bit: the lane's byte of each half of a 16-token word goes to mantissa bits 2..9: a rotation to
+    // the right by 30 (up by two bits) for the lower byte, by 6 for the upper one
+    const u32 vrot = (blk & 1) ? 6u : 30u;
     const int tok_a = vtok_lo<BITS>(blk, 0);
     // column n of the second product: channel group vgrp of every probability operand, query row n % RTP
     const int col_row = n % RTP, col_lo = (n / RTP) & 1, vgrp = (n / RTP) % CL::GPP;
-    // operand row n of the sums product: zeros of group n, scales of group n - GV, ones from row 8 on
-    // (rows 2 GV .. 7 are not used: they read scales).  Byte offset inside a slot, or inside the
-    // block's constants when the row is ones.
+    // operand row n of the sums product: zeros of group n, ones from row 8 on (rows GV .. 7 are not
+    // used: they read the zeros of group 0).  Byte offset inside a slot, or inside the block's
+    // constants when the row is ones.
     const bool zs_ones = n >= 8;
-    const int zs_off = (zs_ones ? 0 : (n < GV ? RG::VZ_OFF + n * VROW : RG::VS_OFF + (n < 2 * GV ? n - GV : 0) * VROW)) +
-                       tok_a * (int)MSZ;
+    const int zs_off = (zs_ones ? 0 : RG::VZ_OFF + (n < GV ? n : 0) * VROW) + tok_a * (int)MSZ;
     auto read_unit = [&](int slot, Unit &d) VQ_INLINE_LAMBDA {
         const char *sl = wring + slot * RG::SLOT;
         if constexpr (BITS == 4) {
@@ -321,13 +331,14 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
             const f16 *qr = s_qraw + (w_row + 4 * u) * PK_QROW + w_ch0 + p;
-            qpair[u][p] = as_u(f16x2{qr[0], qr[PAIR_GAP]});
+            // k-slot pair p of an operand sits at mantissa bit pos(p): its query side carries 2^(EK - pos(p))
+            qpair[u][p] = as_u(f16x2{qr[0], qr[PAIR_GAP]} * h2(SB::wk(p)));
         }
     char *qimg = wring + RG::QIMG_OFF;
     const int w_off = w_row * PK_QIMG_ROW + w_blk * 64 + w_ks * 16;
     const int r_off = (col_lo * RTP + col_row) * PK_QIMG_ROW + blk * 64;
-    // bias chain: operand rows 0-7 carry the group's zeros, rows 8-15 its scales (fp16 scale / zero);
-    // the query rows (high columns only; remainder columns read zeros) are the other operand
+    // bias chain: every operand row carries the group's zeros; the query rows (high columns only;
+    // remainder columns read zeros) are the other operand
     f16x8 q0[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
@@ -367,8 +378,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                 *reinterpret_cast<uint4 *>(qimg + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
                 *reinterpret_cast<uint4 *>(qimg + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
             }
-            // ---- bias chain
-            const char *zs = gs + (n < 8 ? RG::KMR : 0) + 64 * blk;
+            // ---- bias chain: the zeros of the lane's 32 channels in every operand row
+            const char *zs = gs + RG::KMR + 64 * blk;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks)
                 bt = VQ_MFMA(as_h8(*reinterpret_cast<const uint4 *>(zs + 16 * ks)), q0[ks], bt);
@@ -389,31 +400,27 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                 *reinterpret_cast<uint4 *>(qimg + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
                 *reinterpret_cast<uint4 *>(qimg + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
             }
-            // bias chain: operand rows 0-3 high parts of the zeros, 4-7 their remainders, 8-11 and 12-15
-            // the same of the scales
-            const char *zs = gs + (n < 8 ? RG::KMR : 0) + 128 * blk;
-            const bool rem = (n & 4) != 0;
+            // bias chain: the zeros as fp16 high parts, then their remainders, in every operand row
+            const char *zs = gs + RG::KMR + 128 * blk;
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
                 const float4 x0 = *reinterpret_cast<const float4 *>(zs + 32 * ks);
                 const float4 x1 = *reinterpret_cast<const float4 *>(zs + 32 * ks + 16);
                 const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                f16x8 o;
+                f16x8 oh, ol;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     const f16 h = (f16)x[j];
-                    const f16 l = (f16)(x[j] - (float)h);
-                    o[j] = rem ? l : h;
+                    oh[j] = h;
+                    ol[j] = (f16)(x[j] - (float)h);
                 }
-                bt = VQ_MFMA(o, q0[ks], bt);
+                bt = VQ_MFMA(oh, q0[ks], bt);
+                bt = VQ_MFMA(ol, q0[ks], bt);
             }
-            bt[0] += __shfl_xor(bt[0], 16);   // high part + remainder
         }
-        // lanes 0-31 hold sum z q of their column, lanes 32-63 sum s q
-        const float other = __shfl_xor(bt[0], 32);
-        const float zq = blk < 2 ? bt[0] : other, sq = blk < 2 ? other : bt[0];
-        const float b = zq - Magic<BITS>::off * sq;
-        bias = f32x4{b, b, b, b};
+        // every register of a lane holds sum z q of the lane's column; the score accumulators carry 2^(EK - 24)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) bias[r] = bt[r] * SB::KSCALE_INV;
         // ---- folded query, reader role (the image is this wave's own: its LDS accesses run in order)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -428,11 +435,10 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         for (int T = 0; T < 2; ++T) {
             f16x8 A[4];   // per k-step
             if constexpr (BITS == 4) {
-                unpack8_pair<4>(cur.kw[T][0], cur.kw[T][1], magic, A[0], A[1]);
-                unpack8_pair<4>(cur.kw[T][2], cur.kw[T][3], magic, A[2], A[3]);
-            } else {   // word j holds k-steps 2j (low bytes) and 2j + 1 (high bytes)
-                unpack8_pair<2>(cur.kw[T][0], cur.kw[T][1], magic, A[0], A[2]);
-                unpack8_pair_upper2(cur.kw[T][0], cur.kw[T][1], magic, A[1], A[3]);
+                sub_unpack4(cur.kw[T][0], cur.kw[T][1], A[0], A[1]);
+                sub_unpack4(cur.kw[T][2], cur.kw[T][3], A[2], A[3]);
+            } else {   // word j holds k-steps 2j (codes 0-3 | 8-11) and 2j + 1 (codes 4-7 | 12-15)
+                sub_unpack2(cur.kw[T][0], cur.kw[T][1], A[0], A[1], A[2], A[3]);
             }
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) S[T] = VQ_MFMA(A[ks], qB[ks], ks == 0 ? bias : S[T]);
@@ -464,10 +470,10 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         }
 
         // softmax against a lazily updated reference: the fast path touches no other lane
-        const float mx = fmaxf(fmaxf(fmaxf(S[0][0], S[0][1]), fmaxf(S[0][2], S[0][3])),
-                               fmaxf(fmaxf(S[1][0], S[1][1]), fmaxf(S[1][2], S[1][3])));
-        if (__any(mx * c > acc.m_run + RESCALE_SLACK)) {
-            float m_seen = mx * c;
+        const float mx = max3_raw(max3_raw(S[0][0], S[0][1], S[0][2]), max3_raw(S[0][3], S[1][0], S[1][1]),
+                                  max_raw(S[1][2], S[1][3]));
+        if (__any(mx * cs > acc.thr)) {
+            float m_seen = mx * cs;
             m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 16));
             m_seen = fmaxf(m_seen, __shfl_xor(m_seen, 32));
             const float m_new = fmaxf(acc.m_run, m_seen);
@@ -479,20 +485,19 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
                 for (int r = 0; r < 4; ++r) acc.O[nt][r] *= alpha;
 #pragma unroll
             for (int r = 0; r < 4; ++r) acc.Z[r] *= alpha;
-            if constexpr (F32META) {
-#pragma unroll
-                for (int p = 0; p < CL::NP; ++p)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r) acc.Off[p][r] *= alpha;
-            }
             acc.m_run = m_new;
+            acc.thr = m_new + SB::SLACK;
+            const float nm = m_new == -INFINITY ? 0.f : -m_new;   // a row with no visible token yet
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc.nm[r] = nm + (float)(SB::EV - SB::pos(r));
         }
-        const float nm = acc.m_run == -INFINITY ? 0.f : -acc.m_run;   // a row with no visible token yet
+        // register r of either tile is k-slot pair r of the second product, whose codes sit at mantissa
+        // bit pos(r): its probabilities carry 2^(EV - pos(r)), added in the exponent
         u32 P[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], c, nm));
-            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], c, nm));
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[0][r], cs, acc.nm[r]));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(S[1][r], cs, acc.nm[r]));
             P[r] = as_u(f16x2{(f16)p0, (f16)p1});
         }
         const f16x8 P8 = as_h8(P[0], P[1], P[2], P[3]);
@@ -521,31 +526,32 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             for (int j = 0; j < CL::TPP; j += 2) {
                 const int nt = p * CL::TPP + j;
                 f16x8 Av0, Av1;
-                if constexpr (BITS == 4) unpack8_pair<4>(cur.vw[nt], cur.vw[nt + 1], magic, Av0, Av1);
+                if constexpr (BITS == 4) sub_unpack4(cur.vw[nt], cur.vw[nt + 1], Av0, Av1);
                 else {
-                    const u64 x = pack64(cur.vw[nt], cur.vw[nt + 1]) >> vshift;   // the lane's byte of each 16-token word
-                    unpack8_pair<2>((u32)x, (u32)(x >> 32), magic, Av0, Av1);
+                    Av0 = sub4<2>(__builtin_amdgcn_alignbit(cur.vw[nt], cur.vw[nt], vrot));
+                    Av1 = sub4<2>(__builtin_amdgcn_alignbit(cur.vw[nt + 1], cur.vw[nt + 1], vrot));
                 }
                 acc.O[nt] = VQ_MFMA(Av0, Bh, acc.O[nt]);
                 acc.O[nt + 1] = VQ_MFMA(Av1, Bh, acc.O[nt + 1]);
                 acc.O[nt] = VQ_MFMA(Av0, Bl, acc.O[nt]);
                 acc.O[nt + 1] = VQ_MFMA(Av1, Bl, acc.O[nt + 1]);
             }
-            if constexpr (F32META) {
-                acc.Off[p] = VQ_MFMA(ones, Bh, acc.Off[p]);
-                acc.Off[p] = VQ_MFMA(ones, Bl, acc.Off[p]);
-            }
         }
-        // sums: operand rows = zeros of each group, scales of each group, ones
+        // sums: operand rows = zeros of each group, ones; the weights of the probabilities are undone per
+        // k-slot pair (exact powers of two)
         if constexpr (!F32META) {
-            acc.Z = VQ_MFMA(as_h8(cur.z.pair(0), cur.z.pair(1), cur.z.pair(2), cur.z.pair(3)), P8, acc.Z);
+            u32 zw[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) zw[j] = as_u(as_h2(cur.z.pair(j)) * h2(SB::wv_inv(j)));
+            acc.Z = VQ_MFMA(as_h8(zw[0], zw[1], zw[2], zw[3]), P8, acc.Z);
         } else {
             u32 zh[4], zl[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const f16x2 h = {(f16)cur.z.lo(j), (f16)cur.z.hi(j)};
+                const float z0 = cur.z.lo(j) * SB::wv_inv(j), z1 = cur.z.hi(j) * SB::wv_inv(j);
+                const f16x2 h = {(f16)z0, (f16)z1};
                 zh[j] = as_u(h);
-                zl[j] = as_u(f16x2{(f16)(cur.z.lo(j) - (float)h[0]), (f16)(cur.z.hi(j) - (float)h[1])});
+                zl[j] = as_u(f16x2{(f16)(z0 - (float)h[0]), (f16)(z1 - (float)h[1])});
             }
             acc.Z = VQ_MFMA(as_h8(zh[0], zh[1], zh[2], zh[3]), P8, acc.Z);
             acc.Z = VQ_MFMA(as_h8(zl[0], zl[1], zl[2], zl[3]), P8, acc.Z);
@@ -562,15 +568,15 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     // nothing queued, END = the block has no more).
     constexpr int CH = RG::CHUNK;
     const int n_chunks = (n_units + CH - 1) / CH;
-    int dealt = wave;   // fixed order: wave w takes chunks w, w + PK_WAVES, ...
+    int dealt = wave;   // fixed order: wave w takes chunks w, w + WAVES, ...
     auto draw = [&]() VQ_INLINE_LAMBDA {   // the next chunk of the block; the value is used a chunk later
         int id = 0;
-        if (fixed_order) id = (dealt += PK_WAVES);
+        if (fixed_order) id = (dealt += RG::WAVES);
         else if (lane == 0) id = __hip_atomic_fetch_add(s_next, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
         return id;
     };
     auto chunk_len = [&](int chunk) VQ_INLINE_LAMBDA { return n_units - chunk * CH < CH ? n_units - chunk * CH : CH; };
-    if (wave >= n_chunks) return;   // the first PK_WAVES chunks are dealt out, the counter starts behind them
+    if (wave >= n_chunks) return;   // the first WAVES chunks are dealt out, the counter starts behind them
     constexpr int END = -1, NONE = -2;
     int i_chunk = wave, i_pos = 0, i_slot = 0, i_gslot = 0;
     int c_chunk = wave, c_pos = 0, c_next = NONE, c_after = NONE, c_slot = 0, c_gslot = 0;
@@ -625,17 +631,20 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     }
 }
 
-// grid (nsplit, B*Hkv*tiles), PK_THREADS threads.  A block works on one tile of query rows (the GQA
+// grid (nsplit, B*Hkv*tiles), Ring<...>::THREADS threads.  A block works on one tile of query rows (the GQA
 // group at pq consecutive positions) and on packed tokens
 // [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)), cut to what the
 // tile sees; in the block of split 0 the last nparts - nsplit waves first run the fp16 tail, each
 // into a partial slot of its own.  With sync counters the block that finishes last for its tile
 // merges the nparts partials into the output.
-template <int BITS, typename M, int GV, int RTP>
-__global__ __launch_bounds__(PK_THREADS) __attribute__((amdgpu_waves_per_eu(VQ_PK_WAVES / 4, VQ_PK_WAVES / 4)))
+template <int BITS, typename M, int GV, int RTP, int WAVES = Ring<BITS, M, GV, RTP>::WAVES>
+__global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4)))
 void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
                                int order, float *__restrict__ ws) {
     using CL = Cols<GV, RTP>;
+    using RG = Ring<BITS, M, GV, RTP>;
+    constexpr int PK_WAVES = RG::WAVES, PK_THREADS = RG::THREADS;
+    constexpr int EX_O = ex_o(PK_WAVES), EX_Z = ex_z(PK_WAVES), EX_M = ex_m(PK_WAVES);
     // query rows of the block; constants: [0, 128) ones for 32 tokens in the scale / zero type, then zeros
     __shared__ __align__(16) f16 s_qraw[8 * PK_QROW];
     __shared__ __align__(16) char s_const[512];
@@ -655,7 +664,6 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         if (sizeof(M) == 2) reinterpret_cast<u32 *>(s_const)[tid] = tid < 16 ? 0x3C003C00u : 0u;
         else reinterpret_cast<u32 *>(s_const)[tid] = tid < 32 ? __float_as_uint(1.f) : 0u;
     }
-    const int n = lane & 15, blk = lane >> 4;
     const int by = blockIdx.y;
     const int sp = (int)blockIdx.x, nsplit = (int)gridDim.x;
     const int64_t bh = by / tiles;
@@ -675,7 +683,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int RT = tile.RT;
 
     const bool single_launch = a.sync_counters != nullptr;
-    stage_query<RTP>(a, tile, tid, s_qraw);
+    stage_query<RTP, PK_THREADS>(a, tile, tid, s_qraw);
     if (sp == 0 && a.k_new != nullptr && a.n_tail >= 1 && tid < 32) {
         // the newest token's key and value rows become the last tail row: 16 pieces of 16 bytes each
         const int piece = tid & 15;
@@ -692,16 +700,21 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (sp == 0 && wave >= PK_WAVES - tail_waves)
         tail_wave(a, bh, tile, c, nsplit + wave - (PK_WAVES - tail_waves), nparts, ws, s_qraw, PK_QROW, lane,
                   wave - (PK_WAVES - tail_waves), tail_waves, single_launch);
+    // what the unit loop derives from the lane number is formed from here on, not ahead of the tail: the tail
+    // needs its 168 registers to itself
+    int lane_u = lane;
+    asm volatile("" : "+v"(lane_u));
+    const int n = lane_u & 15, blk = lane_u >> 4;
 
-    PackedAcc<CL::NP, sizeof(M) != 2> acc;
+    using SB = Sub<BITS>;
+    PackedAcc acc;
 #pragma unroll
     for (int nt = 0; nt < 8; ++nt) acc.O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.Z = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
-    if constexpr (sizeof(M) != 2) {
+    acc.thr = -INFINITY;
 #pragma unroll
-        for (int p = 0; p < CL::NP; ++p) acc.Off[p] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
+    for (int r = 0; r < 4; ++r) acc.nm[r] = (float)(SB::EV - SB::pos(r));
 
     // packed tokens the rows of the tile see: all of them up to full_vis, none from max_vis on
     int64_t full_vis = tile.visible(0), max_vis = tile.visible(RT - 1);
@@ -723,7 +736,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int64_t lane_first = tile.first(n % RTP < RT ? n % RTP : 0) - t_begin, edge_first = tile.first(RT - 1) - t_begin;
     const int lo_rel = (int)(lane_first < 0 ? 0 : lane_first > rel_cap ? rel_cap : lane_first);
     const int edge_rel = (int)(edge_first < 0 ? 0 : edge_first > rel_cap ? rel_cap : edge_first);
-    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lo_rel, edge_rel, lane, wave, acc, s_qraw, s_const,
+    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lo_rel, edge_rel, lane_u, wave, acc, s_qraw, s_const,
                                    s_ring, &s_next, order);
     __syncthreads();   // every wave has read its last slot
 
@@ -737,18 +750,14 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
             const int g = nt / CL::TPG;
             if (col_set == g % CL::GPP) {
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float v = acc.O[nt][r];
-                    if constexpr (sizeof(M) != 2) v -= Magic<BITS>::off * acc.Off[g / CL::GPP][r];
-                    s_o[wave][col_row][16 * nt + 4 * blk + r] = v;
-                }
+                for (int r = 0; r < 4; ++r) s_o[wave][col_row][16 * nt + 4 * blk + r] = acc.O[nt][r] * SB::VSCALE;
             }
         }
         if (col_set == 0) {
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int i = 4 * blk + r;
-                if (i < 2 * GV) s_z[wave][col_row][i] = acc.Z[r];
+                if (i < GV) s_z[wave][col_row][i] = acc.Z[r];
                 if (i == 8) s_l[wave][col_row] = acc.Z[r];
             }
         }
@@ -766,8 +775,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
             if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit, or saw nothing
             const float f = exp2f(s_m[w][row] - gm);
             const int g = d / (MF_D / GV);
-            const float off_sum = sizeof(M) == 2 ? Magic<BITS>::off * s_z[w][row][GV + g] : 0.f;
-            num += ((s_o[w][row][d] - off_sum) + s_z[w][row][g]) * f;
+            num += (s_o[w][row][d] + s_z[w][row][g]) * f;
             den += s_l[w][row] * f;
         }
         float *o = ws + (tile.row(row) * nparts + sp) * MF_PART;
@@ -776,17 +784,18 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     }
 
     // ---- last block of this tile merges the splits (no block ever waits for another).
-    // Partials travel as device-scope (write-through) stores and device-scope loads, so no
-    // cache-wide write-back or invalidate is needed.  What orders them against the ticket:
-    // every thread waits until its own stores (these and the tail's) have been acknowledged
-    // -- stores count in vmcnt on this target, and a barrier alone does not wait for them --
-    // then the barrier collects the block, then one thread takes a ticket.  The merging
-    // block's loads depend on the ticket's value, so they are issued after it returned.
+    // Partials travel as device-scope (write-through) stores and device-scope loads.  What
+    // orders them against the ticket: every thread waits until its own stores (these and the
+    // tail's) have been acknowledged -- stores count in vmcnt on this target, and a barrier
+    // alone does not wait for them -- then the barrier collects the block, then one thread takes
+    // a ticket with release-acquire ordering at device scope: the release publishes the block's
+    // partials before the count moves, the acquire orders the merging block's loads after it
+    // (the block barrier behind it extends that to the other threads).
     if (!single_launch) return;
     wait_copies<0>();
     __syncthreads();
     if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != nsplit - 1) return;
     merge_rows(a, tile, nparts, ws, tid, PK_THREADS);
@@ -795,21 +804,22 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
 
 template <typename M, int RTP>
 static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
-    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles)), block(PK_THREADS);
+    const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles));
     const int gv = (int)(MF_D / a.group);
     // more than 64 KB of block-shared memory has to be allowed per kernel and device, once
 #define VQ_LAUNCH(BITS, GV)                                                                                            \
     do {                                                                                                               \
         constexpr int ring_bytes = Ring<BITS, M, GV, RTP>::BYTES;                                                      \
-        static bool allowed[64] = {};                                                                                  \
+        static std::atomic<bool> allowed[64] = {};   /* set once per device; a second setter repeats the same call */ \
         int dev = 0;                                                                                                   \
         (void)hipGetDevice(&dev);                                                                                      \
-        if (dev < 0 || dev >= 64 || !allowed[dev]) {                                                                   \
+        if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {                                   \
             (void)hipFuncSetAttribute((const void *)attend_mfma_packed_kernel<BITS, M, GV, RTP>,                       \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);                         \
-            if (dev >= 0 && dev < 64) allowed[dev] = true;                                                             \
+            if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);                             \
         }                                                                                                              \
-        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV, RTP>), grid, block, ring_bytes, st, a, p.split_len, \
+        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV, RTP>), grid, dim3(Ring<BITS, M, GV, RTP>::THREADS),  \
+                           ring_bytes, st, a, p.split_len,                                                             \
                            p.tail_equiv, p.nparts, p.pq, p.tiles, p.fixed_order, ws);                                  \
     } while (0)
     if (a.pack_bits == 4) {
