@@ -326,6 +326,35 @@ def _vq_assign_case(torch, K, dev):
     return x, cb, (lambda: K.vecinfer_quantize_metal(x, cb, 8, index_dtype=torch.uint8))
 
 
+def _vq_census(torch, x, cb, idx):
+    """Brute force on the device in the reference's arithmetic (float32 differences, squares rounded separately,
+    dimensions added left to right, allocators/vecinfer.py:301-315): whether every index is the lowest-index
+    argmin, and how many sub-vectors have their two nearest centroids within 4 ulp of the best distance -- the
+    cases where a different (unpinned) summation order in the reference's own backend could pick the other one."""
+    sub = cb.shape[1]
+    xs = x.reshape(-1, sub).float()
+    c = cb.float()
+    got = idx.reshape(-1).long()
+    near = 0
+    equal = True
+    for lo in range(0, xs.shape[0], 32768):
+        xv = xs[lo: lo + 32768]
+        d = torch.zeros((xv.shape[0], c.shape[0]), dtype=torch.float32, device=xs.device)
+        for i in range(sub):
+            diff = xv[:, i: i + 1] - c[None, :, i]
+            d = d + diff * diff
+        best2, arg2 = torch.topk(d, 2, dim=1, largest=False)
+        amin = torch.argmin(d, dim=1)   # (ties: checked through the distance of the chosen index below)
+        chosen = d.gather(1, got[lo: lo + 32768, None])[:, 0]
+        equal = equal and bool((chosen == best2[:, 0]).all()) and bool((got[lo: lo + 32768] <= amin).all() | True)
+        # lowest index among the exact minima
+        first_min = (d == best2[:, :1]).float().argmax(dim=1)
+        equal = equal and bool((got[lo: lo + 32768] == first_min).all())
+        ulp = torch.nextafter(best2[:, 0], torch.full_like(best2[:, 0], float("inf"))) - best2[:, 0]
+        near += int(((best2[:, 1] - best2[:, 0]) <= 4 * ulp).sum())
+    return {"indices_match_bruteforce": equal, "near_ties_le_4ulp": near, "sub_vectors_checked": int(xs.shape[0])}
+
+
 def _only(a, torch, K, dev):
     """One side workload in a loop, for profilers: prints its average milliseconds."""
     name = a.only
@@ -500,6 +529,21 @@ def _extras(torch, K, dev):
     flops = 2 * 524288 * 256 * 8
     ex["vq_assign_cfg2"] = {"ms": round(ms, 5), "TFLOPs_gemm_form": round(flops / ms / 1e9, 2),
                             "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 5)}
+    ex["vq_assign_cfg2"].update(_vq_census(torch, x, cb, fn()))
+    # the reference's default key codebook: 4096 centroids of 4 dims (key_codebook_bits 12, key_sub_dim 4,
+    # cache/options.py:36-43), Llama-shaped keys [4, 4096, 128] -> 524 288 sub-vectors, int32 indices
+    x4d = (torch.randn((4, 4096, 128), device=dev) * torch.exp(torch.randn(128, device=dev))).to(torch.float16)
+    cb4 = torch.randn((4096, 4), device=dev).to(torch.float16)
+    fn4 = lambda: K.vecinfer_quantize_metal(x4d, cb4, 4)
+    for _ in range(3):
+        fn4()
+    ms4 = _side_ms(fn4, 10, torch)
+    flops4 = 2 * 524288 * 4096 * 4
+    ex["vq_assign_4096_centroids_sub4"] = {"ms": round(ms4, 5), "TFLOPs_gemm_form": round(flops4 / ms4 / 1e9, 2),
+                                           "frac_mfma_f16_peak": round(flops4 / ms4 / 1e9 / MFMA_F16_PEAK_TFLOPS, 5),
+                                           "note": "codebook tiles streamed from LDS, 16 chunks of 256 centroids"}
+    ex["vq_assign_4096_centroids_sub4"].update(_vq_census(torch, x4d[:1, :1024], cb4, fn4()[:1, :1024]))
+    del x4d, cb4
     # Kitty keys (mixed 4/2-bit by channel variance): two launches of the key-axis round trip plus the ranking
     kc = KVCacheFactory.create(KVCacheConfig(method="kitty", head_dim=D))
     kk = (torch.randn((16, Hkv, 8192, D), device=dev) * torch.exp(torch.randn(D, device=dev))).to(torch.float16)
