@@ -343,10 +343,7 @@ def _vq_census(torch, x, cb, idx):
         for i in range(sub):
             diff = xv[:, i: i + 1] - c[None, :, i]
             d = d + diff * diff
-        best2, arg2 = torch.topk(d, 2, dim=1, largest=False)
-        amin = torch.argmin(d, dim=1)   # (ties: checked through the distance of the chosen index below)
-        chosen = d.gather(1, got[lo: lo + 32768, None])[:, 0]
-        equal = equal and bool((chosen == best2[:, 0]).all()) and bool((got[lo: lo + 32768] <= amin).all() | True)
+        best2 = torch.topk(d, 2, dim=1, largest=False).values
         # lowest index among the exact minima
         first_min = (d == best2[:, :1]).float().argmax(dim=1)
         equal = equal and bool((got[lo: lo + 32768] == first_min).all())

@@ -684,6 +684,65 @@ def test_config3_decode_at_full_size_against_the_oracle_and_the_vector_kernel():
     assert err < 2e-3
 
 
+def test_config3_all_36_layers_in_one_launch_equal_the_per_layer_calls_bit_for_bit():
+    """Benchmark configuration 3 at full size through ``LayerStackedKIVICache``: 36 layers x 16 sequences x
+    32768 tokens of 4-bit group-64 packed context plus the fp16 residual, the newest token appended by the
+    launch itself.  With chunks dealt in a fixed order the one launch over all layers equals the 36
+    per-layer launches bit for bit (the layer-batched call of veloxquant_mlx/metal/_scalar_attend.py:496-647
+    against its per-layer loop, tests/metal/test_scalar_attend.py:660-707); one layer's last sequence is
+    checked against the scalar C oracle."""
+    require_gpu()
+    from oracle import cref
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    NL, B, Hq, Hkv, D, ctx, g, bits = 36, 16, 32, 8, 128, 32768, 64, 4
+    dev = "cuda:0"
+    gen = torch.Generator(device=dev).manual_seed(3)
+    f = torch.exp(torch.randn(D, generator=gen, device=dev))
+    n_total = ctx + 128 + 37
+    layers = []
+    for l in range(NL):
+        c = _make(bit_width_inlier=bits, kivi_group_size=g, residual_length=128, fused_sdpa=True,
+                  fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=ctx + 4096)
+        for s0 in range(0, n_total, 8192):
+            n = min(8192, n_total - s0)
+            c.update_and_fetch((torch.randn((B, Hkv, n, D), generator=gen, device=dev) * f).half(),
+                               torch.randn((B, Hkv, n, D), generator=gen, device=dev).half())
+        assert c._n_quantized == ctx
+        layers.append(c)
+    stack = LayerStackedKIVICache.from_layers(layers)
+    q = torch.randn((NL, B, Hq, 1, D), generator=gen, device=dev).half()
+    scale = 1 / math.sqrt(D)
+    # (the same cut of the context on both sides: left to themselves 576 sequences take one run, 16 take two)
+    all_at_once = stack.fused_sdpa_all(q, scale, fixed_order=True, num_splits=2)
+    assert all_at_once.shape == (NL, B, Hq, 1, D)
+    for l, c in enumerate(layers):
+        one = c.fused_sdpa(q[l], scale, fixed_order=True, num_splits=2)
+        assert torch.equal(one, all_at_once[l]), (l, float((one.float() - all_at_once[l].float()).abs().max()))
+    # the default order (chunks handed out on demand) agrees to rounding
+    assert float((stack.fused_sdpa_all(q, scale).float() - all_at_once.float()).abs().max()) < 2e-3
+    # a decode step of all layers: 36 appends that launch nothing, one launch that stores and attends
+    k_new, v_new = (torch.randn((NL, B, Hkv, 1, D), generator=gen, device=dev).half() for _ in range(2))
+    for l, c in enumerate(layers):
+        c.update_and_fetch(k_new[l], v_new[l])
+    stepped = stack.fused_sdpa_all(q, scale)
+    l, b, per = NL - 1, B - 1, 32 // bits
+    c = layers[l]
+    assert c._pending is None and c.offset == n_total + 1 and torch.equal(c._tail_k[:, :, n_total - ctx, :], k_new[l][:, :, 0, :])
+    nq, n_tail = c._n_quantized, c.offset - c._n_quantized
+    kp = c._kp[b:b + 1, :, :nq].cpu().numpy().view(np.uint32)
+    codes_k = ok.unpack_indices(kp, bits, D)
+    vp = c._vp[b:b + 1, :, : nq // per].cpu().numpy().view(np.uint32)
+    codes_v = np.ascontiguousarray(ok.unpack_indices(np.ascontiguousarray(vp.swapaxes(-1, -2)), bits, nq).swapaxes(-1, -2))
+    ks, kz = (t[b:b + 1, :, : nq // g].float().cpu().numpy() for t in (c._ks, c._kz))
+    vs, vz = (np.ascontiguousarray(t[b:b + 1, :, :, :nq].float().cpu().numpy().swapaxes(-1, -2)) for t in (c._vs, c._vz))
+    ref = cref.attend(q[l, b:b + 1].float().cpu().numpy(), codes_k, ks, kz, codes_v, vs, vz, g, scale,
+                      k_tail=c._tail_k[b:b + 1, :, :n_tail].float().cpu().numpy(),
+                      v_tail=c._tail_v[b:b + 1, :, :n_tail].float().cpu().numpy())
+    err = float(np.max(np.abs(stepped[l, b:b + 1].float().cpu().numpy() - ref)))
+    print(f"layer {l}, last sequence: max |one launch - oracle| = {err:.2e}")
+    assert err < 2e-3
+
+
 def test_kivi_quantizer_encode_decode():
     require_gpu()
     rng = np.random.default_rng(0)

@@ -310,7 +310,7 @@ class KIVIKVCache(FP16KVCache):
         return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
 
     def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0,
-                   fixed_order: bool | None = None, lengths: torch.Tensor | None = None):
+                   fixed_order: bool | None = None, lengths: torch.Tensor | None = None, num_splits: int = 0):
         """Attention of ``q [B,H_q,S_q,D]`` over the packed prefix and the fp16 tail,
         queries aligned to the end of the cache (the contract of
         ``VecInferKVCache.fused_sdpa``, veloxquant_mlx/cache/vecinfer_cache.py:670-731), under an
@@ -319,7 +319,8 @@ class KIVIKVCache(FP16KVCache):
         :func:`veloxquant_mlx_amd.kernels.kivi_packed_attend`).  ``lengths`` (int ``[B]``, on the
         device or the host) gives every sequence of a right-padded batch its own number of live
         tokens: sequence ``b`` attends over its first ``lengths[b]`` slots, its queries aligned to
-        the end of those."""
+        the end of those.  ``num_splits`` > 0 fixes into how many runs the context is cut (0: chosen from the
+        shapes; two calls that are to agree bit for bit need the same cut as well as ``fixed_order``)."""
         if not self._fused_enabled:
             raise RuntimeError("KIVIKVCache.fused_sdpa called but fused_sdpa was not enabled via "
                                "KVCacheConfig.fused_sdpa=True.")
@@ -339,7 +340,7 @@ class KIVIKVCache(FP16KVCache):
                   v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
                   k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
                   causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
-                  sliding_window=int(sliding_window or 0))
+                  sliding_window=int(sliding_window or 0), num_splits=max(0, int(num_splits)))
         kw.update(self._extra_attend_args())
         plan = None
         if lengths is None and self._offer_tiles(q, kw):

@@ -145,9 +145,9 @@ class LayerStackedKIVICache:
 
     # ------------------------------------------------------------------ attention
     def fused_sdpa_all(self, q: torch.Tensor, scale: float, *, causal: bool = True,
-                       fixed_order: bool | None = None) -> torch.Tensor:
+                       fixed_order: bool | None = None, num_splits: int = 0) -> torch.Tensor:
         """Attention of ``q [NL, B, H_q, S_q, D]`` over every layer's cache in one launch; layer
-        ``l``'s queries align to the end of layer ``l``'s tokens.  ``fixed_order`` as in
+        ``l``'s queries align to the end of layer ``l``'s tokens.  ``fixed_order`` and ``num_splits`` as in
         ``KIVIKVCache.fused_sdpa``."""
         NL = len(self.layers)
         if q.ndim != 5 or q.shape[0] != NL:
@@ -189,7 +189,8 @@ class LayerStackedKIVICache:
         kw = dict(k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz, n_packed=max(nq), bits=c0._b,
                   group_size=c0._group_size, v_layout=c0._v_layout, k_tail=tk if max(nt) else None,
                   v_tail=tv if max(nt) else None, n_tail=max(nt), scale=float(scale),
-                  causal=bool(causal) and q.shape[3] > 1, out_dtype=q.dtype, fixed_order=fixed_order, **lens)
+                  causal=bool(causal) and q.shape[3] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
+                  num_splits=max(0, int(num_splits)), **lens)
         qf = q.reshape((NL * B,) + tuple(q.shape[2:]))
         if k_new is not None:
             try:
