@@ -400,7 +400,10 @@ int vq_kivi_attend(const vq_attend_args *a);
  * with more than 16384 (sequence, kv head, row tile) triples return VQ_ERR_WORKSPACE.  The call
  * itself allocates and frees nothing.  All calls on one GPU share that GPU's array: calls that
  * overlap on one GPU (two streams, two threads) race -- serialise them, or use vq_kivi_attend
- * with a workspace per stream. */
+ * with a workspace per stream.  The first call on a device looks the array's address up, and the
+ * first launch of each kernel instantiation raises its block-shared-memory limit: make one call
+ * per device and shape class (bit width, group size, scale type, rows per kv head) outside any
+ * stream capture before capturing.  A call that fails clears the shared counters behind itself. */
 int vq_kivi_attend_static(const vq_attend_args *a);
 
 /* ---- attention over VecInfer indices ----------------------------------------- */

@@ -437,6 +437,45 @@ def test_prefill_tiles_change_no_bit_and_follow_the_cache(bits, g, dtype):
     assert torch.equal(outs[0], outs[1]) and caches[0]._tiles is None
 
 
+@pytest.mark.parametrize("bits,g", [(4, 32), (2, 32)])
+def test_sink_protected_cache_with_prefill_sized_query_blocks(bits, g):
+    """Protected rows under a prefill-sized call (64 positions x 4 query heads = 256 rows a kv head, the
+    256-row attention blocks): the stand-ins' weights are taken out of sums the matrix unit formed from
+    fp16-rounded reconstructions, so the queries here are aimed at the stand-ins themselves and at the
+    rows next to them, where those weights carry most of a row's mass."""
+    require_gpu()
+    rng = np.random.default_rng(23)
+    B, Hq, H, D, R, n = 1, 8, 2, 128, 64, 448
+    k = rng.standard_normal((B, H, n, D)).astype(np.float16)
+    v = rng.standard_normal((B, H, n, D)).astype(np.float16)
+    for p, f in ((5, 12), (77, 10), (200, 14), (201, 9)):
+        k[0, :, p] *= f
+    cfg = KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=g, residual_length=R,
+                        n_sink_tokens=3, fused_sdpa=True, fused_sdpa_memory_bound=True, kivi_meta_dtype="float32")
+    c = KVCacheFactory.create(cfg)
+    m = ok.SinkCacheModel(bits, g, R, 3)
+    for s0, s1 in ((0, 256), (256, 384), (384, 448)):
+        c.update_and_fetch(to_dev(k[:, :, s0:s1]), to_dev(v[:, :, s0:s1]))
+        m.update_and_fetch(k[:, :, s0:s1], v[:, :, s0:s1])
+    assert c._n_quantized == m.n_quantized and any(c._side_pos[b] for b in range(B))
+    km, vm = m.keys[:, :, : m.offset], m.values[:, :, : m.offset]
+    Sq = 64
+    q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float16)
+    sinks = m.sink_positions_for(0)
+    for i, p in enumerate(sinks):
+        for dp in (0, 1):                              # the protected row, and its neighbour
+            row = km[0, 0, min(p + dp, m.offset - 1)].astype(np.float32)
+            q[0, i % Hq, -(1 + 2 * i + dp) % Sq] += (row / np.linalg.norm(row) * 6).astype(np.float16)
+    scale = 1 / math.sqrt(D)
+    for w in (0, 130):
+        plan = {}
+        got = host(c.fused_sdpa(to_dev(q), scale, causal=True, sliding_window=w)).astype(np.float32)
+        ref = oa.sdpa(q, km, vm, scale, causal=True, sliding_window=w)
+        err = float(np.max(np.abs(got - ref)))
+        print(f"bits {bits}: window {w}: protected rows {sinks}, max err {err:.2e}")
+        assert err < 2e-3, (w, err)
+
+
 def test_prefill_tile_scratch_is_given_back_by_every_kind_of_decode_step():
     """The tile scratch of a memory-bound prefill lives only until decoding begins: a single-token append, a
     single-query attend with per-sequence ``lengths`` and the layer-stacked launch all return ``nbytes`` to the

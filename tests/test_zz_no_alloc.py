@@ -58,3 +58,26 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point():
     q512 = to_dev(np.random.default_rng(4).standard_normal((2, 32, 512, 128)).astype(np.float16))
     with pytest.raises(RuntimeError, match="built-in scratch"):   # 32768 query rows: 17 MB of partials
         K.kivi_packed_attend(q512, static_scratch=True, **{**big[1], "causal": True})
+
+
+def test_static_scratch_makes_no_tile_scratch_for_long_plain_prefill():
+    """A causal call over plain keys and values with thousands of query rows per kv head: the ordinary call
+    writes the input once as tiles into a scratch it keeps; with ``static_scratch=True`` nothing may be
+    allocated, the blocks convert the rows themselves, and the bits are the same."""
+    require_gpu()
+    B, Hq, Hkv, S, D = 1, 8, 2, 1536, 128                  # 4 query heads x 1536 positions = 6144 rows per kv head
+    rng = np.random.default_rng(12)
+    q, k, v = (to_dev(rng.standard_normal((B, h, S, D)).astype(np.float16)) for h in (Hq, Hkv, Hkv))
+    # one part per block: the blocks write ``out`` themselves and no split partials are needed
+    kw = dict(k_tail=k, v_tail=v, n_tail=S, scale=1 / math.sqrt(D), causal=True, num_splits=1)
+    out = torch.empty_like(q)
+    K.release_tile_scratch()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    K.kivi_packed_attend(q, out=out, static_scratch=True, **kw)
+    torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before
+    ref = K.kivi_packed_attend(q, **kw)                   # makes and uses the tile scratch
+    assert torch.cuda.memory_allocated() > before + out.numel() * 2
+    assert torch.equal(out, ref)
+    assert K.release_tile_scratch() > 0

@@ -6,14 +6,14 @@ three storage modes (dequantise-only, dequantise + index stash, memory-bound
 indices only), geometric growth of the ``[B, H, cap, n_sub]`` index buffers,
 ``state`` / ``trim`` / ``nbytes`` per mode and :meth:`fused_sdpa` over the stored
 indices.  Assignment and gather run in the HIP kernels; the transform is a dense
-``D x D`` product.  :meth:`fused_sdpa` gathers the transformed keys and the values
-from their indices and runs the attention kernel over them (the score/gather
-fusion of veloxquant_mlx/metal/fused_sdpa.py:200-299 is not built yet).
+``D x D`` product (or, with 16-byte aligned keys, part of the fused key-encode kernel).
+:meth:`fused_sdpa` attends straight from the stored indices through
+``kernels.metal_fused_sdpa`` (the look-up-table attention of
+veloxquant_mlx/metal/fused_sdpa.py:200-299).
 """
 
 from __future__ import annotations
 
-import math
 import warnings
 from typing import Any
 
@@ -27,6 +27,34 @@ from ._fp16_cache import FP16KVCache
 
 _SMOOTH_FLOOR = 1e-12
 
+# KVCacheConfig fields the cache reads, with the defaults of veloxquant_mlx/cache/options.py:36-43
+_FIELDS = {"key_sub_dim": 4, "value_sub_dim": 8, "key_codebook_bits": 12, "value_codebook_bits": 8,
+           "residual_length": 128, "seed": 42}
+
+
+class _Tally:
+    """Byte and token counters of the cache, kept together so that an append adds to all of them and a trim
+    scales all of them (the accounting of vecinfer_cache.py:617-664: tracked per call, so a trim is an
+    estimate in proportion to the tokens kept)."""
+
+    NAMES = ("key_compressed", "value_compressed", "key_fp16", "value_fp16", "tokens_seen", "tokens_quantized")
+
+    def __init__(self) -> None:
+        self.n = dict.fromkeys(self.NAMES, 0)
+
+    def append(self, rows: int, tokens: int, head_dim: int, key_index_bits: int, value_index_bits: int) -> None:
+        """``rows`` = batch x heads x tokens appended; index bits per row of ``head_dim`` channels."""
+        self.n["key_compressed"] += -(-key_index_bits // 8) * rows
+        self.n["value_compressed"] += -(-value_index_bits // 8) * rows
+        self.n["key_fp16"] += rows * head_dim * 2
+        self.n["value_fp16"] += rows * head_dim * 2
+        self.n["tokens_seen"] += tokens
+        self.n["tokens_quantized"] += tokens
+
+    def keep_fraction(self, kept: float) -> None:
+        for name in self.NAMES:
+            self.n[name] = int(self.n[name] * kept)
+
 
 class VecInferKVCache(FP16KVCache):
     """KV cache implementing VecInfer's dual-transform product VQ.
@@ -35,13 +63,11 @@ class VecInferKVCache(FP16KVCache):
 
     def __init__(self, config: Any) -> None:
         super().__init__()
-        self._head_dim = int(config.head_dim)
-        self._key_sub_dim = int(getattr(config, "key_sub_dim", 4))
-        self._value_sub_dim = int(getattr(config, "value_sub_dim", 8))
-        self._key_bits = int(getattr(config, "key_codebook_bits", 12))
-        self._value_bits = int(getattr(config, "value_codebook_bits", 8))
-        self._residual_length = int(getattr(config, "residual_length", 128))
-        D = self._head_dim
+        opt = {name: int(getattr(config, name, default)) for name, default in _FIELDS.items()}
+        D = self._head_dim = int(config.head_dim)
+        self._key_sub_dim, self._value_sub_dim = opt["key_sub_dim"], opt["value_sub_dim"]
+        self._key_bits, self._value_bits = opt["key_codebook_bits"], opt["value_codebook_bits"]
+        self._residual_length = opt["residual_length"]
         if D < 1 or (D & (D - 1)) != 0:
             raise QuantizerConfigError(
                 f"VecInferKVCache requires a power-of-2 head_dim (the Walsh-Hadamard transform needs it); "
@@ -58,7 +84,7 @@ class VecInferKVCache(FP16KVCache):
         self._H = walsh_hadamard_matrix(D, dtype=torch.float32)
 
         n_kc, n_vc = 2 ** self._key_bits, 2 ** self._value_bits
-        seed = int(getattr(config, "seed", 42))
+        seed = opt["seed"]
         missing = [n for n in ("key_codebook", "value_codebook") if getattr(config, n, None) is None]
         if missing:
             warnings.warn(
@@ -75,12 +101,7 @@ class VecInferKVCache(FP16KVCache):
             val_cb = torch.randn((n_vc, self._value_sub_dim), generator=torch.Generator().manual_seed(seed + 1))
         self._value_codebook = torch.as_tensor(val_cb).float()
 
-        self._key_bytes_compressed = 0
-        self._key_bytes_fp16 = 0
-        self._value_bytes_compressed = 0
-        self._value_bytes_fp16 = 0
-        self._tokens_seen = 0
-        self._tokens_quantized = 0
+        self._tally = _Tally()
 
         requested = getattr(config, "use_metal_kernels", None)
         if not K._lib.library_present():
@@ -308,14 +329,9 @@ class VecInferKVCache(FP16KVCache):
         trimmed = super().trim(n)
         if not trimmed:
             return trimmed
+        # the index buffers advance by _stored_S_kv, not by offset: left alone they would keep the dropped tokens
         self._stored_S_kv = min(self._stored_S_kv, self.offset)
-        keep = self.offset / old_offset
-        self._key_bytes_compressed = int(self._key_bytes_compressed * keep)
-        self._value_bytes_compressed = int(self._value_bytes_compressed * keep)
-        self._key_bytes_fp16 = int(self._key_bytes_fp16 * keep)
-        self._value_bytes_fp16 = int(self._value_bytes_fp16 * keep)
-        self._tokens_seen = int(self._tokens_seen * keep)
-        self._tokens_quantized = int(self._tokens_quantized * keep)
+        self._tally.keep_fraction(self.offset / old_offset)
         return trimmed
 
     def size(self) -> int:
@@ -331,14 +347,8 @@ class VecInferKVCache(FP16KVCache):
 
     def _account_bytes(self, B: int, H: int, S: int, D: int) -> None:
         """vecinfer_cache.py:654-664."""
-        k_bits = (D // self._key_sub_dim) * self._key_bits
-        v_bits = (D // self._value_sub_dim) * self._value_bits
-        self._key_bytes_compressed += math.ceil(k_bits / 8) * H * B * S
-        self._value_bytes_compressed += math.ceil(v_bits / 8) * H * B * S
-        self._key_bytes_fp16 += H * B * S * D * 2
-        self._value_bytes_fp16 += H * B * S * D * 2
-        self._tokens_seen += S
-        self._tokens_quantized += S
+        self._tally.append(B * H * S, S, D, (D // self._key_sub_dim) * self._key_bits,
+                           (D // self._value_sub_dim) * self._value_bits)
 
     # ------------------------------------------------------------------ attention
     def fused_sdpa(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0):
@@ -375,21 +385,13 @@ class VecInferKVCache(FP16KVCache):
                                     causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype)
 
     # ------------------------------------------------------------------ reporting
-    @property
-    def compressed_key_bytes(self) -> int:
-        return self._key_bytes_compressed
-
-    @property
-    def fp16_key_bytes(self) -> int:
-        return self._key_bytes_fp16
-
-    @property
-    def compressed_value_bytes(self) -> int:
-        return self._value_bytes_compressed
-
-    @property
-    def fp16_value_bytes(self) -> int:
-        return self._value_bytes_fp16
+    compressed_key_bytes = property(lambda self: self._tally.n["key_compressed"])
+    fp16_key_bytes = property(lambda self: self._tally.n["key_fp16"])
+    compressed_value_bytes = property(lambda self: self._tally.n["value_compressed"])
+    fp16_value_bytes = property(lambda self: self._tally.n["value_fp16"])
+    # (the names the other caches keep their counters under)
+    _tokens_seen = property(lambda self: self._tally.n["tokens_seen"])
+    _tokens_quantized = property(lambda self: self._tally.n["tokens_quantized"])
 
     @property
     def codebook_bytes(self) -> int:

@@ -273,6 +273,11 @@ constexpr size_t STATIC_COUNTERS = 16384;             // int32 sync counters, on
 static __device__ __align__(256) unsigned char scratch[STATIC_WS_BYTES + STATIC_COUNTERS * sizeof(int32_t)];
 std::mutex g_scratch_mutex;
 unsigned char *g_scratch_ptr[64] = {};
+
+// a fill kernel, not hipMemsetAsync: the call may sit inside a stream capture
+__global__ void zero_counters_kernel(int32_t *c, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) c[i] = 0;
+}
 }  // namespace
 
 extern "C" int vq_kivi_attend_static(const vq_attend_args *a) {
@@ -305,7 +310,15 @@ extern "C" int vq_kivi_attend_static(const vq_attend_args *a) {
     vq_attend_args b = *a;
     b.workspace = ptr;
     b.workspace_bytes = STATIC_WS_BYTES;
-    // the counters start at zero (static storage) and every finished call leaves them at zero
+    // the counters start at zero (static storage) and every finished call leaves them at zero; a call that
+    // failed half-way (a launch error) may not have, and a later call would then never reach its last ticket
+    // and leave `out` unwritten: the counters are cleared again behind a failed call
     b.sync_counters = reinterpret_cast<int32_t *>(ptr + STATIC_WS_BYTES);
-    return vq_kivi_attend(&b);
+    rc = vq_kivi_attend(&b);
+    if (rc != VQ_OK) {
+        hipLaunchKernelGGL(zero_counters_kernel, dim3(16), dim3(256), 0, (hipStream_t)a->stream, b.sync_counters,
+                           (int)STATIC_COUNTERS);
+        (void)hipGetLastError();   // the error reported is the call's own (already recorded)
+    }
+    return rc;
 }

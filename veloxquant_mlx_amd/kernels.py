@@ -785,6 +785,15 @@ def _tile_scratch(device: torch.device, rows: int, units: int) -> torch.Tensor:
     return t[: rows * units * PREFILL_TILE_BYTES].view(rows, units, PREFILL_TILE_BYTES)
 
 
+def release_tile_scratch() -> int:
+    """Give back the tile scratches :func:`kivi_packed_attend` keeps per device and stream for long causal calls
+    over plain keys and values; returns the bytes released.  (A call with ``static_scratch=True`` never makes
+    one: it allocates nothing, so it takes tiles only when the caller passes them.)"""
+    n = sum(t.numel() for t in _tile_scratches.values())
+    _tile_scratches.clear()
+    return n
+
+
 _sync_counters: dict[tuple, torch.Tensor] = {}
 
 
@@ -968,7 +977,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         keep += [sk, sv, sp]
     if (tiles is None and n_packed == 0 and causal and D == 128 and Hq % Hkv == 0 and Hq // Hkv in (1, 2, 4, 8)
             and (Hq // Hkv) * Sq >= 24 * 256 and k_tail.dtype in (torch.float16, torch.bfloat16)
-            and packed_lens is None and sinks is None and k_new is None
+            and packed_lens is None and sinks is None and k_new is None and not static_scratch
             and B * Hkv * -(-int(n_tail) // 32) * PREFILL_TILE_BYTES <= _TILE_SCRATCH_MAX):
         # Plain keys and values under so many row tiles that every unit is read two dozen times or more: written
         # once as tiles (a scratch kept per device and stream, 608 B per slot and kv head) they are copied into
@@ -1141,7 +1150,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant", "kivi_prefill_tiles", "prefill_tiles_empty",
+    "hip_available", "release_tile_scratch", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant", "kivi_prefill_tiles", "prefill_tiles_empty",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",
