@@ -142,3 +142,31 @@ def test_channel_variance_in_one_pass(dtype, N, S, D):
     want = np.var(xt.double().cpu().numpy(), axis=1)
     got = host(K.channel_variance(xt)).astype(np.float64)
     np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-9)
+
+
+@pytest.mark.parametrize("D", [64, 48])       # 64: one-pass variance kernel; 48: torch.var of the float32 copy
+def test_near_tie_and_tied_variances_rank_alike_on_both_paths(D):
+    """Channels that hold +a and -a on alternate tokens: mean 0 and variance a^2 in every arithmetic (sums of
+    equal powers of two times a 22-bit square stay exact), so the ranking cannot depend on how a path forms
+    the variance.  The amplitudes are neighbouring fp16 numbers with exact repeats; equal variances go to
+    the lower channel (kitty.py:61-64, 112-135)."""
+    require_gpu()
+    rng = np.random.default_rng(D)
+    S, N = 64, 3
+    ladder = [np.float16(1.25)]
+    for _ in range(5):
+        ladder.append(np.nextafter(ladder[-1], np.float16(2)))
+    ladder = np.array(ladder, np.float16)
+    amp = ladder[rng.integers(0, 6, (N, D))]
+    sign = np.where(np.arange(S) % 2 == 0, 1, -1).astype(np.float16)
+    keys = (amp[:, None, :] * sign[None, :, None]).astype(np.float16)
+    var = host(qk.channel_variance_batched(to_dev(keys)))
+    assert np.array_equal(var, amp.astype(np.float32) ** 2)
+    for frac in (0.125, 0.25, 0.5):
+        got = host(qk.hi_mask_from_variance_batched(qk.channel_variance_batched(to_dev(keys)), frac))
+        want = okt.hi_mask_from_variance(var, frac)
+        assert np.array_equal(got, want)
+        n_hi = max(1, int(D * frac))
+        for n in range(N):
+            beat = (var[n][None, :] > var[n][:, None]) | ((var[n][None, :] == var[n][:, None]) & (np.arange(D)[None, :] < np.arange(D)[:, None]))
+            assert np.array_equal(want[n], beat.sum(1) < n_hi)

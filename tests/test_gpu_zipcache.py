@@ -119,3 +119,37 @@ def test_routing_kernel_equals_the_stable_sorts():
             want = torch.argsort((rank >= S - n_hi).to(torch.int32), dim=-1, stable=True)
             got = K.zip_route(norms.to("cuda:0"), n_hi).cpu().long()
             assert torch.equal(got, want), (S, n_hi)
+
+
+@pytest.mark.parametrize("D", [128, 96])      # 128: norms and routing in the kernels; 96: the torch path
+def test_near_tie_and_tied_norms_route_alike_on_both_paths(D):
+    """Rows with one non-zero element: its square has 22 significant bits, so every summation order and
+    float width gives the norm |x| exactly and the routing cannot depend on how a path rounds.  The values
+    are neighbouring fp16 numbers (near ties, one unit in the last place apart) with exact repeats among
+    them; on equal norms the later row goes to the high block (zipcache_cache.py:106-116), and both
+    paths must reproduce the model's reconstruction bit for bit and its norms exactly."""
+    require_gpu()
+    B, H, S = 1, 3, 96
+    rng = np.random.default_rng(D)
+    base = np.float16(1.5)
+    ladder = np.array([base] * 8, np.float16)
+    for i in range(1, 8):
+        ladder[i] = np.nextafter(ladder[i - 1], np.float16(2))
+    k = np.zeros((B, H, S, D), np.float16)
+    for h in range(H):
+        vals = ladder[rng.integers(0, 8, S)]                       # many exact ties, neighbours everywhere
+        cols = rng.integers(0, D, S)
+        k[0, h, np.arange(S), cols] = vals * rng.choice(np.array([-1, 1], np.float16), S)
+    c = _make(head_dim=D, zipcache_hi_fraction=0.3)
+    got, norms, _ = c._compress(to_dev(k), True)
+    want, wnorms, _ = oz.compress(k, True, 4, 2, 0.3, 32)
+    assert np.array_equal(host(norms), wnorms)
+    assert np.array_equal(host(norms).reshape(H, S), np.abs(k.astype(np.float32)).max(-1)[0])
+    assert np.array_equal(host(got).view(np.uint16), want.view(np.uint16))
+    # the tie rule itself, stated without a sort: a row is in the high block iff fewer than n_hi rows
+    # beat it, where a later row with the same norm beats an earlier one
+    n_hi = int(np.ceil(S * 0.3))
+    nm = wnorms.reshape(H, S)
+    for h in range(H):
+        beat = (nm[h][None, :] > nm[h][:, None]) | ((nm[h][None, :] == nm[h][:, None]) & (np.arange(S)[None, :] > np.arange(S)[:, None]))
+        assert np.array_equal(oz.saliency_mask(nm[h:h + 1], n_hi)[0], beat.sum(1) < n_hi)
