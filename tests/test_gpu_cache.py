@@ -1059,6 +1059,95 @@ def test_layer_stacked_cache_attends_for_all_layers_at_once():
         stacked.fused_sdpa_all(rnd(2, B, Hq, 1, D), scale)
 
 
+@pytest.mark.parametrize("bits,meta", [(4, "float16"), (2, "float32")])
+def test_layer_stacked_cache_with_protected_rows_and_a_sliding_window(bits, meta):
+    """``LayerStackedKIVICache`` over ``method="kivi_sink"`` layers: every layer protects its own rows (different
+    positions and different counts per layer and sequence), the one launch patches all of them, with and without
+    a sliding window; against separate ``SinkProtectedKVCache`` objects fed the same tokens, bit for bit under
+    ``fixed_order`` with the same cut, and against the oracle's model of layer 0."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    from veloxquant_mlx_amd.cache.sink_cache import SinkProtectedKVCache
+    NL, B, Hq, Hkv, D, R = 3, 2, 8, 2, 128, 64
+    cfg = KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=32, residual_length=R,
+                        n_sink_tokens=3, fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=1024,
+                        kivi_meta_dtype=meta)
+    stacked = LayerStackedKIVICache(cfg, NL)
+    assert all(isinstance(c, SinkProtectedKVCache) for c in stacked.layers)
+    solo = [KVCacheFactory.create(cfg) for _ in range(NL)]
+    model = ok.SinkCacheModel(bits, 32, R, 3)
+    rng = np.random.default_rng(101 + bits)
+    scale = 1 / math.sqrt(D)
+    pos = [0] * NL
+
+    def feed(layer, n):
+        k = rng.standard_normal((B, Hkv, n, D)).astype(np.float16)
+        v = rng.standard_normal((B, Hkv, n, D)).astype(np.float16)
+        for b in range(B):                     # loud rows at places that differ by layer and sequence
+            for p in range(pos[layer], pos[layer] + n):
+                if p % (37 + 11 * layer + 5 * b) == 3 + layer:
+                    k[b, :, p - pos[layer]] *= 9 + (p % 5)
+        pos[layer] += n
+        stacked[layer].update_and_fetch(to_dev(k), to_dev(v))
+        solo[layer].update_and_fetch(to_dev(k), to_dev(v))
+        if layer == 0:
+            model.update_and_fetch(k, v)
+
+    def check(Sq=1, window=0):
+        q = rng.standard_normal((NL, B, Hq, Sq, D)).astype(np.float16)
+        # aim one head of every layer at one of its protected rows
+        for layer in range(NL):
+            ps = solo[layer]._side_pos[0] if solo[layer]._side_pos else []
+            if ps:
+                slot = len(ps) - 1
+                row = host(solo[layer]._side_k[0, 0, slot]).astype(np.float32)
+                q[layer, 0, 1, -1] += (row / np.linalg.norm(row) * 5).astype(np.float16)
+        qd = to_dev(q)
+        kw = dict(sliding_window=window, fixed_order=True, num_splits=2)
+        out = stacked.fused_sdpa_all(qd, scale, **kw)
+        for layer in range(NL):
+            ref = solo[layer].fused_sdpa(qd[layer], scale, **kw)
+            assert torch.equal(out[layer], ref), (layer, Sq, window)
+        km, vm = model.keys[:, :, : model.offset], model.values[:, :, : model.offset]
+        want = oa.sdpa(q[0], km, vm, scale, causal=Sq > 1, sliding_window=window)
+        err = float(np.max(np.abs(host(out[0]).astype(np.float32) - want)))
+        # the model keeps float32 group parameters; a store with fp16 ones adds their rounding (2^-11 of a
+        # scale of ~0.5 on codes up to 15) to every reconstructed element
+        assert err < (2e-3 if meta == "float32" else 6e-3), (Sq, window, err)
+
+    for layer in range(NL):
+        feed(layer, 300)
+    assert any(any(c._side_pos[b] for b in range(B)) for c in stacked.layers)
+    check()
+    check(window=100)
+    side = stacked._sinks[1][0]
+    check()
+    assert stacked._sinks[1][0] is side                      # nothing changed: the stacked side store is reused
+    for step in range(70):                                   # crosses two flushes; protected rows age out on the way
+        for layer in range(NL):
+            feed(layer, 1)
+        if step % 7 == 0 or step > 60:
+            check(window=0 if step % 2 else 150)
+    assert stacked._sinks[1][0] is not side
+    for layer in range(NL):
+        a, b = stacked[layer], solo[layer]
+        assert a._side_pos == b._side_pos and a._n_quantized == b._n_quantized and a.sink_positions == b.sink_positions
+    check(Sq=4)
+    check(Sq=4, window=90)
+    feed(0, 1)                                               # a forward pass in flight: ragged lengths
+    check()
+    # trimming a layer below a protected row takes the row out of the stacked side store as well
+    n_side = [sum(len(ps) for ps in c._side_pos) for c in stacked.layers]
+    stacked[2].trim(pos[2] - 150)
+    solo[2].trim(pos[2] - 150)
+    pos[2] = 150
+    assert sum(len(ps) for ps in stacked[2]._side_pos) <= n_side[2] and stacked[2]._side_pos == solo[2]._side_pos
+    q = to_dev(rng.standard_normal((NL, B, Hq, 1, D)).astype(np.float16))
+    out = stacked.fused_sdpa_all(q, scale, fixed_order=True, num_splits=2)
+    for layer in range(NL):
+        assert torch.equal(out[layer], solo[layer].fused_sdpa(q[layer], scale, fixed_order=True, num_splits=2)), layer
+
+
 def test_context_limit_error_leaves_the_cache_as_it_was():
     """An append whose flush would pass ``fused_sdpa_max_ctx`` raises before offset, rows or packed
     store change: the cache answers the same query with the same bits afterwards."""

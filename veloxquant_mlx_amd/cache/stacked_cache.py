@@ -9,6 +9,11 @@ cache object works on its slice of them through the ordinary cache API, and
 ``fused_sdpa_all`` hands the whole buffers to one attention launch with the layer axis folded
 into the batch axis.  Layers whose lengths differ by a step (a forward pass in flight) go
 through the per-sequence lengths of the attention entry point.
+
+With ``method="kivi_sink"`` the layers are ``SinkProtectedKVCache`` objects: their exact rows
+are gathered into one ``[NL * B, H, cap, D]`` side store (rebuilt only after a flush, a trim
+or a restored state changed some layer's rows) and the one launch patches every layer's
+protected positions.  ``sliding_window`` is the attention call's.
 """
 
 from __future__ import annotations
@@ -19,6 +24,7 @@ import torch
 
 from .. import kernels as K
 from .kivi_cache import KIVIKVCache
+from .sink_cache import SinkProtectedKVCache
 
 _PACKED = ("_kp", "_ks", "_kz", "_vp", "_vs", "_vz")
 
@@ -39,10 +45,12 @@ class LayerStackedKIVICache:
         if not (getattr(config, "fused_sdpa", False) and getattr(config, "fused_sdpa_memory_bound", False)):
             raise RuntimeError("LayerStackedKIVICache needs KVCacheConfig(fused_sdpa=True, fused_sdpa_memory_bound=True): "
                                "the stack holds packed codes and the fp16 tail, nothing else.")
-        self.layers = [KIVIKVCache(config) for _ in range(n_layers)]
+        kind = SinkProtectedKVCache if getattr(config, "method", "kivi") == "kivi_sink" else KIVIKVCache
+        self.layers = [kind(config) for _ in range(n_layers)]
         self._packed: tuple[torch.Tensor, ...] | None = None      # six [NL*B, ...] stacks
         self._tails: list[tuple[torch.Tensor, torch.Tensor]] = []  # two pairs of [NL*B, H, cap, D] stacks
         self._lens = None   # (key, packed_lens, tail_lens) of the last ragged call
+        self._sinks = None  # (key, (side_k, side_v, side_pos)) of the last call with protected rows
 
     @classmethod
     def from_layers(cls, layers) -> "LayerStackedKIVICache":
@@ -58,7 +66,7 @@ class LayerStackedKIVICache:
             raise ValueError("LayerStackedKIVICache.from_layers: the layers differ in bit width, group size or layout")
         self = cls.__new__(cls)
         self.layers = layers
-        self._packed, self._tails, self._lens = None, [], None
+        self._packed, self._tails, self._lens, self._sinks = None, [], None, None
         return self
 
     def __len__(self) -> int:
@@ -143,12 +151,38 @@ class LayerStackedKIVICache:
             c._tail_spare = (sk[sl], sv[sl])
         return 0
 
+    def _stacked_sinks(self, B: int) -> dict:
+        """The exact rows of every layer's protected positions as one side store ``[NL*B, H, cap, D]`` with
+        positions ``[NL*B, cap]`` (-1: unused slot).  A layer's rows change only where its ``_side_pos_dev`` is
+        dropped (flush, trim, restored state), so the table objects of the layers identify a stack."""
+        per_layer = [c._extra_attend_args().get("sinks") if isinstance(c, SinkProtectedKVCache) else None
+                     for c in self.layers]
+        if not any(s is not None for s in per_layer):
+            self._sinks = None
+            return {}
+        key = tuple(None if s is None else id(s[2]) for s in per_layer)
+        if self._sinks is None or self._sinks[0] != key:
+            first = next(s for s in per_layer if s is not None)
+            H, D = first[0].shape[1], first[0].shape[3]
+            cap = max(s[0].shape[2] for s in per_layer if s is not None)
+            NL = len(self.layers)
+            sk = torch.zeros((NL * B, H, cap, D), dtype=first[0].dtype, device=first[0].device)
+            sv = torch.zeros_like(sk)
+            sp = torch.full((NL * B, cap), -1, dtype=torch.int32, device=first[0].device)
+            for l, s in enumerate(per_layer):
+                if s is None:
+                    continue
+                n = s[0].shape[2]
+                sk[l * B:(l + 1) * B, :, :n], sv[l * B:(l + 1) * B, :, :n], sp[l * B:(l + 1) * B, :n] = s
+            self._sinks = (key, (sk, sv, sp), [s[2] for s in per_layer if s is not None])   # the tables stay alive: their ids are the key
+        return {"sinks": self._sinks[1]}
+
     # ------------------------------------------------------------------ attention
-    def fused_sdpa_all(self, q: torch.Tensor, scale: float, *, causal: bool = True,
+    def fused_sdpa_all(self, q: torch.Tensor, scale: float, *, causal: bool = True, sliding_window: int = 0,
                        fixed_order: bool | None = None, num_splits: int = 0) -> torch.Tensor:
         """Attention of ``q [NL, B, H_q, S_q, D]`` over every layer's cache in one launch; layer
-        ``l``'s queries align to the end of layer ``l``'s tokens.  ``fixed_order`` and ``num_splits`` as in
-        ``KIVIKVCache.fused_sdpa``."""
+        ``l``'s queries align to the end of layer ``l``'s tokens.  ``sliding_window``, ``fixed_order`` and
+        ``num_splits`` as in ``KIVIKVCache.fused_sdpa``."""
         NL = len(self.layers)
         if q.ndim != 5 or q.shape[0] != NL:
             raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: q must be [NL={NL},B,H_q,S_q,D], got {tuple(q.shape)}")
@@ -190,7 +224,8 @@ class LayerStackedKIVICache:
                   group_size=c0._group_size, v_layout=c0._v_layout, k_tail=tk if max(nt) else None,
                   v_tail=tv if max(nt) else None, n_tail=max(nt), scale=float(scale),
                   causal=bool(causal) and q.shape[3] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
-                  num_splits=max(0, int(num_splits)), **lens)
+                  sliding_window=int(sliding_window or 0), num_splits=max(0, int(num_splits)), **lens,
+                  **self._stacked_sinks(B))
         qf = q.reshape((NL * B,) + tuple(q.shape[2:]))
         if k_new is not None:
             try:
