@@ -419,14 +419,27 @@ def test_attend_errors():
 @pytest.mark.parametrize("b,g", [(2, 32), (4, 64), (4, 128), (2, 128)])
 @pytest.mark.parametrize("Hq,Hkv", [(8, 8), (16, 2), (32, 8), (12, 4)])
 def test_mfma_decode_head_ratios_and_groups(b, g, Hq, Hkv):
-    """GQA ratios 1, 8, 4, 3 through the MFMA kernel (ratios above 8 take the vector kernel)."""
+    """GQA ratios 1, 8, 4, 3 through the MFMA kernel."""
     _packed_case(2, Hq, Hkv, 1024, 0, 128, b, g, "token", torch.float16, seed=Hq + g + b, expect_path=1)
+
+
+@pytest.mark.parametrize("b,g,meta", [(2, 32, torch.float16), (4, 64, torch.float32), (4, 32, torch.float16), (2, 128, torch.float32)])
+@pytest.mark.parametrize("Hq,Hkv,Sq,n_tail", [(32, 2, 1, 37), (16, 1, 1, 0), (24, 2, 1, 5), (18, 2, 1, 64), (32, 2, 3, 20), (40, 1, 5, 0)])
+def test_mfma_decode_groups_of_more_than_eight_heads(b, g, meta, Hq, Hkv, Sq, n_tail):
+    """GQA ratios 16, 12, 9 and 40 (multi-query attention): tiles of eight heads, the last one short, every tile
+    a block column of its own over the same keys and values; with a tail, several query positions and a
+    window."""
+    _packed_case(2, Hq, Hkv, 1024, n_tail, 128, b, g, "token", meta, Sq=Sq, causal=Sq > 1, seed=Hq + g + b + Sq,
+                 expect_path=1)
+    if Sq == 3:
+        _packed_case(1, Hq, Hkv, 640, n_tail, 128, b, g, "token", meta, Sq=Sq, causal=True, seed=Hq + g, expect_path=1,
+                     window=200)
 
 
 def test_mfma_decode_many_splits_and_single_unit():
     _packed_case(1, 4, 1, 32, 3, 128, 4, 32, "token", torch.float16, seed=2, expect_path=1)
     _packed_case(1, 4, 1, 4096, 200, 128, 2, 64, "token", torch.float32, seed=3, expect_path=1)
-    _packed_case(1, 32, 2, 256, 0, 128, 4, 64, "token", torch.float16, seed=4, expect_path=0)   # ratio 16
+    _packed_case(1, 32, 2, 256, 0, 128, 4, 64, "token", torch.float16, seed=4, expect_path=1)   # ratio 16: two tiles of eight heads
 
 
 def test_mfma_decode_peaked_attention():

@@ -41,7 +41,7 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     int64_t n_split = a.n_packed + a.n_tail;
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
-        p.tiles = (int)cdiv(a.Sq, p.pq);
+        p.tiles = mfma_row_tiles(a);
         p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * TAIL_EQUIV, 128) * 128 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }

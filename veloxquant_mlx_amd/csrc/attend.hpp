@@ -30,7 +30,7 @@ struct AttendPlan {
     // [max(0, s*split_len - tail_equiv), min(n_packed, (s+1)*split_len - tail_equiv))
     int64_t tail_equiv;
     // MFMA path: a block works on the GQA group of one kv head at pq consecutive query
-    // positions; tiles = ceil(Sq / pq) such blocks per (batch, kv head)
+    // positions (eight heads of a group of more than eight, pq = 1); tiles such blocks per (batch, kv head)
     int pq, tiles;
     // MFMA decode path: deal token chunks to the waves round robin instead of on demand, so that
     // results are identical from run to run
@@ -104,6 +104,7 @@ void launch_merge_rows(const float *ws, int64_t rows, int nparts, int64_t D, voi
 
 // MFMA decode path (attend_mfma.hip)
 bool mfma_decode_supported(const vq_attend_args &a);
+int mfma_row_tiles(const vq_attend_args &a);
 int mfma_positions_per_tile(const vq_attend_args &a);
 
 // MFMA prefill path (attend_prefill.hip): packed prefix into partial slot 0, tail into slot 1

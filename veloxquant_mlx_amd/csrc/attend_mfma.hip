@@ -8,16 +8,25 @@ namespace vq {
 // (a high and a remainder column each in the 16-wide tile).
 int mfma_positions_per_tile(const vq_attend_args &a) {
     const int64_t R = a.Hq / a.Hkv;
-    if (a.Sq == 1) return 1;
+    if (a.Sq == 1 || R > 8) return 1;
     return (int)(8 / R);
+}
+
+// Row tiles per (sequence, kv head): positions in steps of mfma_positions_per_tile, times the tiles of
+// eight heads a GQA group of more than eight falls into.
+int mfma_row_tiles(const vq_attend_args &a) {
+    const int64_t R = a.Hq / a.Hkv;
+    return (int)(cdiv(a.Sq, mfma_positions_per_tile(a)) * (R > 8 ? cdiv(R, 8) : 1));
 }
 
 bool mfma_decode_supported(const vq_attend_args &a) {
     if (a.D != MF_D || a.n_packed <= 0) return false;
-    if (a.Hq % a.Hkv != 0 || 2 * (a.Hq / a.Hkv) > MF_ROWS) return false;  // high + remainder columns
+    if (a.Hq % a.Hkv != 0) return false;
     const int64_t R = a.Hq / a.Hkv;
-    if (a.Sq > 1 && !(R == 1 || R == 2 || R == 4 || R == 8)) return false;
-    if (a.B * a.Hkv * cdiv(a.Sq, mfma_positions_per_tile(a)) > 65535) return false;   // grid y, sync counters
+    // a tile has eight rows (a high and a remainder column each): the whole group at one position, a
+    // power-of-two group at 8 / R positions, or eight heads of a larger group
+    if (a.Sq > 1 && !(R == 1 || R == 2 || R == 4 || R >= 8)) return false;
+    if (a.B * a.Hkv * (int64_t)mfma_row_tiles(a) > 65535) return false;   // grid y, sync counters
     if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
     if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
     if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
@@ -35,7 +44,8 @@ bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p) {
     hipStream_t st = (hipStream_t)a.stream;
     float *ws = (float *)a.workspace;
     // rows a block carries: the GQA group at p.pq positions, padded to 4 or 8
-    const bool wide = (a.Hq / a.Hkv) * p.pq > 4;
+    const int64_t R = a.Hq / a.Hkv;
+    const bool wide = (R > 8 ? 8 : R) * p.pq > 4;
     if (a.meta_dtype == VQ_F16) {
         if (wide) launch_mfma_packed_f16meta_r8(a, p, ws, st);
         else launch_mfma_packed_f16meta_r4(a, p, ws, st);

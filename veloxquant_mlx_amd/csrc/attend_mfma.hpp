@@ -246,7 +246,9 @@ __device__ __forceinline__ u32 lds_addr(const void *p) {
 struct RowTile {
     int64_t base_row;   // flattened [B, Hq, Sq] row of (b, first head of the group, position 0)
     int64_t Sq, n_total;
-    int R, RT, pos0, causal;
+    // R heads of the GQA group from head h0 on (all of them unless the group has more than eight: then tiles
+    // of eight heads at one position), RT = R * positions rows in all
+    int R, RT, pos0, causal, h0;
     int64_t window;     // sliding window (0: none)
     __device__ __forceinline__ bool valid(int j) const { return j < RT && pos0 + j / R < Sq; }
     // first visible slot of tile row j
@@ -256,7 +258,7 @@ struct RowTile {
         const int64_t lo = n_total - Sq + pos + 1 - window;
         return window > 0 && lo > 0 ? lo : 0;
     }
-    __device__ __forceinline__ int64_t row(int j) const { return base_row + (int64_t)(j % R) * Sq + pos0 + j / R; }
+    __device__ __forceinline__ int64_t row(int j) const { return base_row + (int64_t)(h0 + j % R) * Sq + pos0 + j / R; }
     // number of visible slots of tile row j (queries align to the end of the slots)
     __device__ __forceinline__ int64_t visible(int j) const {
         int64_t pos = pos0 + j / R;

@@ -632,7 +632,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 }
 
 // grid (nsplit, B*Hkv*tiles), Ring<...>::THREADS threads.  A block works on one tile of query rows (the GQA
-// group at pq consecutive positions) and on packed tokens
+// group at pq consecutive positions; of a group of more than eight heads, eight at one position) and on packed tokens
 // [max(0, x*split_len - tail_equiv), min(n_packed, (x+1)*split_len - tail_equiv)), cut to what the
 // tile sees; in the block of split 0 the last nparts - nsplit waves first run the fp16 tail, each
 // into a partial slot of its own.  With sync counters the block that finishes last for its tile
@@ -672,14 +672,18 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const float c = a.scale * LOG2E;
 
     RowTile tile;
-    tile.R = (int)(a.Hq / a.Hkv);
+    const int group = (int)(a.Hq / a.Hkv);                 // query heads per kv head
+    const int htiles = group > 8 ? (group + 7) / 8 : 1;   // more than eight: tiles of eight heads (pq is 1 then)
+    const int t_in_bh = by % tiles;
+    tile.h0 = (t_in_bh % htiles) * 8;
+    tile.R = htiles > 1 ? (group - tile.h0 < 8 ? group - tile.h0 : 8) : group;
     tile.RT = tile.R * pq;
-    tile.pos0 = (int)(by % tiles) * pq;
+    tile.pos0 = (t_in_bh / htiles) * pq;
     tile.Sq = a.Sq;
     tile.n_total = a.n_packed + a.n_tail;
     tile.causal = a.causal;
     tile.window = a.sliding_window;
-    tile.base_row = (b * a.Hq + hkv * tile.R) * a.Sq;
+    tile.base_row = (b * a.Hq + hkv * group) * a.Sq;
     const int RT = tile.RT;
 
     const bool single_launch = a.sync_counters != nullptr;
