@@ -6,11 +6,14 @@ quoted on): Qwen3-8B shape, 36 layers, 32 query / 8 kv heads, D=128, batch 16,
 32768 tokens of context per sequence stored as 4-bit packed KIVI codes (keys per
 channel, values per token, group 64) plus an fp16 tail.  One step = one decode
 token for every sequence through all 36 layers: append K/V to the fp16 tail,
-flush a 64-token block into the packed store when one is due, attend.
+flush a 64-token block into the packed store when one is due, attend -- in the
+reference's layer-batched form (one attention launch over a leading layer axis,
+veloxquant_mlx/metal/_scalar_attend.py:496-647); ``per_layer_launches`` holds the same
+step issued as one launch per layer.
 
 Prints ONE JSON line.  ``value`` is algorithmic HBM bytes per step divided by
 the step time, inputs resident in HBM.  ``roofline`` prices the attention
-kernel alone (HIP events on the launch stream); ``cpu_baseline`` times the reference's
+launch alone (HIP events on the launch stream); ``cpu_baseline`` times the reference's
 CPU path (its operations restated on torch CPU, all host threads torch is given) on a
 bounded sample of the same workload; ``extras.cpu_baselines`` holds the same for the
 other workloads and the one-thread scalar C port.
@@ -44,7 +47,10 @@ def _parse():
     p.add_argument("--group", type=int, default=64)
     p.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     p.add_argument("--no-extras", action="store_true", help="skip the per-kernel side measurements")
-    p.add_argument("--only-kernel", action="store_true", help="time the attention kernel loop only (profiling)")
+    p.add_argument("--only-kernel", action="store_true",
+                   help="time the attention launch only (profiling): the layer-batched launch, or with --per-layer "
+                        "the loop of one launch per layer")
+    p.add_argument("--per-layer", action="store_true", help="with --only-kernel: one launch per layer")
     p.add_argument("--only", default=None, metavar="NAME",
                    help="run one side workload in a loop and print its timing (for rocprofv3): "
                         "decode_2bit_B16, decode_2bit_B1, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
@@ -146,8 +152,11 @@ def main() -> int:
                         fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=ctx + 4096)
     caches = []
     chunk = 4096
-    # stop ten tokens short of the next 64-token flush so that one falls inside the timed steps
-    prefill = ctx + R + g - 10
+    # stop short of the next 64-token flush so that it falls inside the timed steps of the headline form
+    # (the per-layer form before it appends 2 + n_pl tokens, the warm-up a.warmup)
+    n_pl = max(3, a.steps // 4)
+    short = 2 + n_pl + a.warmup + max(1, a.steps // 2)
+    prefill = ctx + R + g - (short if short < g else 10)
     for l in range(NL):
         c = KVCacheFactory.create(cfg)
         for s0 in range(0, prefill, chunk):
@@ -164,21 +173,64 @@ def main() -> int:
     k_new = torch.randn((NL, B, Hkv, 1, D), generator=gen, device=dev).to(torch.float16)
     v_new = torch.randn((NL, B, Hkv, 1, D), generator=gen, device=dev).to(torch.float16)
 
-    def step():
+    # Two forms of the same step.  The headline is the reference's layer-batched form (the kernel with a leading
+    # NL axis, metal/_scalar_attend.py:496-647, which the 36-layer configuration is quoted on): every layer's
+    # cache takes its token through the ordinary cache API (nothing is launched: the token is pending), then ONE
+    # launch stores the 36 x 16 new tokens and attends for all layers.  The per-layer form (one launch per layer,
+    # what a model's forward pass issues) is timed beside it.
+    def step_per_layer():
         for l, c in enumerate(caches):
             c.update_and_fetch(k_new[l], v_new[l])
             c.fused_sdpa(q[l], scale)
 
-    def attend_only():
+    def attend_per_layer():
         for l, c in enumerate(caches):
             c.fused_sdpa(q[l], scale)
 
     layer_bytes = _algorithmic_bytes_per_layer(B, Hkv, ctx, D, bits, g)
+    step_bytes = layer_bytes * NL
+    per_layer = None
+    if not a.only_kernel or a.per_layer:
+        n = n_pl if not a.only_kernel else a.steps
+        for _ in range(2 if not a.only_kernel else a.warmup):
+            (attend_per_layer if a.only_kernel else step_per_layer)()
+        if a.only_kernel:
+            ms = _event_ms(attend_per_layer, n, torch) / NL
+            print(json.dumps({"form": "one launch per layer", "attend_ms_per_layer": ms, "GBps": layer_bytes / ms / 1e6}))
+            return 0
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            step_per_layer()
+        torch.cuda.synchronize()
+        dt_pl = (time.perf_counter() - t0) / n
+        kern_pl = _event_ms(attend_per_layer, n, torch) / NL
+        per_layer = {
+            "ms_per_step": round(dt_pl * 1e3, 4), "GBps": round(step_bytes / dt_pl / 1e9, 1),
+            "frac_hbm": round(step_bytes / dt_pl / 1e9 / HBM_PEAK_GBS, 4), "steps": n,
+            "attend_ms_per_launch": round(kern_pl, 5), "attend_GBps": round(layer_bytes / kern_pl / 1e6, 1),
+            "attend_frac_hbm": round(layer_bytes / kern_pl / 1e6 / HBM_PEAK_GBS, 4), "bytes_per_launch": layer_bytes,
+            "note": "the same step as one append + one attention launch per layer (what a model's forward pass issues)"}
+
+    # the layers' caches adopted by a layer-stacked cache: their buffers become slices of [NL*B, ...] stacks
+    # (copied once, here), every layer's cache object keeps working on its slice
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    stack = LayerStackedKIVICache.from_layers(caches)
+
+    def step():
+        for l, c in enumerate(caches):
+            c.update_and_fetch(k_new[l], v_new[l])
+        stack.fused_sdpa_all(q, scale)
+
+    def attend_only():
+        stack.fused_sdpa_all(q, scale)
+
     if a.only_kernel:
         for _ in range(a.warmup):
             attend_only()
-        ms = _event_ms(attend_only, a.steps, torch) / NL
-        print(json.dumps({"attend_ms_per_layer": ms, "GBps": layer_bytes / ms / 1e6}))
+        ms = _event_ms(attend_only, a.steps, torch)
+        print(json.dumps({"form": f"one launch for {NL} layers", "attend_ms_per_launch": ms, "attend_ms_per_layer": ms / NL,
+                          "GBps": step_bytes / ms / 1e6}))
         return 0
 
     for _ in range(a.warmup):
@@ -189,21 +241,22 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / a.steps
-    step_bytes = layer_bytes * NL
     value = step_bytes / dt / 1e9
 
-    # ---- roofline of the dominant kernel (attention), events on the launch stream
-    kern_ms = _event_ms(attend_only, max(3, a.steps // 2), torch) / NL
-    achieved = layer_bytes / (kern_ms * 1e-3) / 1e9
+    # ---- roofline of the dominant kernel (the attention launch), events on the launch stream
+    kern_ms = _event_ms(attend_only, max(3, a.steps // 2), torch)
+    achieved = step_bytes / (kern_ms * 1e-3) / 1e9
     # HBM bytes one attention launch moved under rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (calibrated
     # against a 1 GiB device copy): read from profiles/hbm_traffic.json, which records the hash of the
     # attention sources it was measured on -- a kernel changed since then reports null
-    default_workload = (B, ctx, bits, g) == (16, 32768, 4, 64)
+    default_workload = (NL, B, ctx, bits, g) == (36, 16, 32768, 4, 64)
     roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": _recorded_traffic("decode_cfg3_4bit_g64_B16") if default_workload else None,
-                "kernel": "attend_mfma_packed_kernel<4, f16, 2, 4>: one launch per layer does the fp16 tail, "
-                          "the packed prefix and the split merge (vq_kivi_attend with sync counters)",
-                "bytes_per_launch": layer_bytes, "ms_per_launch": round(kern_ms, 5)}
+                "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": _recorded_traffic("decode_cfg3_4bit_g64_B16_36_layers") if default_workload else None,
+                "kernel": f"attend_mfma_packed_kernel<4, f16, 2, 4>: one launch stores the new token of {NL} layers x {B} "
+                          "sequences, runs their fp16 tails and packed prefixes and merges the splits "
+                          "(vq_kivi_attend with k_new / v_new and sync counters, the layer axis folded into the batch axis)",
+                "bytes_per_launch": step_bytes, "ms_per_launch": round(kern_ms, 5)}
 
     out = {
         "metric": "dequant-SDPA decode HBM GB/s @32k ctx", "value": round(value, 1), "unit": "GB/s",
@@ -211,32 +264,18 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8/f16 (f32 accumulate)",
         "data": "synthetic",
         "config": {"workload": f"configs[3]: batched decode, {NL} layers, 32q/8kv heads, D=128, batch {B}, "
-                               f"context {ctx}, {bits}-bit packed KV group {g}, append+flush+attend per step",
+                               f"context {ctx}, {bits}-bit packed KV group {g}; per step every layer's cache appends its "
+                               "token (flushing a 64-token block when one is due), then one layer-batched launch attends",
                    "layers": NL, "batch": B, "context": ctx, "bits": bits, "group": g,
                    "algorithmic_bytes_per_step": step_bytes},
         "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
         "roofline": roofline,
     }
+    if per_layer is not None:
+        out["per_layer_launches"] = per_layer
 
     if not a.no_extras:
         out["extras"] = _extras(torch, K, dev)
-        # the same step with the layers' caches adopted by a layer-stacked cache (their buffers become
-        # slices of [NL*B, ...] stacks, copied once): 36 appends that launch nothing and ONE launch that
-        # stores every layer's new token and attends for all layers
-        from veloxquant_mlx_amd.cache import LayerStackedKIVICache
-        stack = LayerStackedKIVICache.from_layers(caches)
-
-        def step_all():
-            for l, c in enumerate(caches):
-                c.update_and_fetch(k_new[l], v_new[l])
-            stack.fused_sdpa_all(q, scale)
-        for _ in range(2):
-            step_all()
-        ms = _side_ms(step_all, 5, torch)
-        out["extras"]["decode_cfg3_36_layers_one_launch"] = {
-            "ms": round(ms, 4), "ms_per_layer": round(ms / NL, 5), "GBps": round(step_bytes / ms / 1e6, 1),
-            "frac_hbm": round(step_bytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": step_bytes,
-            "note": "LayerStackedKIVICache over the resident caches: append + attend of all layers per step"}
     if not a.no_cpu:
         head, others = _cpu_baselines(np, torch, caches[0], q[0], ctx, Hkv, D, bits, g, scale)
         out["cpu_baseline"] = head
