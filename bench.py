@@ -486,6 +486,22 @@ def _extras(torch, K, dev):
                                         "ms_graph": round(ms_g, 5), "frac_hbm_graph": round(nbytes / ms_g / 1e6 / HBM_PEAK_GBS, 4),
                                         "note": "ms: one Python call per launch; ms_graph: the same launches replayed from a HIP graph"}
         del c
+    # the same 2-bit cache for eight layers in the layer-batched form: the launch ramp and the uneven finish of
+    # the compute units are paid once for eight layers' bytes
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    NL2 = 8
+    layers2 = [_decode_2bit_case(torch, dev, 16)[0] for _ in range(NL2)]
+    stack2 = LayerStackedKIVICache.from_layers(layers2)
+    q2 = torch.randn((NL2, 16, Hq, 1, D), device=dev).to(torch.float16)
+    fn2 = lambda: stack2.fused_sdpa_all(q2, 1 / math.sqrt(D))
+    for _ in range(3):
+        fn2()
+    ms2 = _side_ms(fn2, 10, torch)
+    nbytes2 = NL2 * _algorithmic_bytes_per_layer(16, Hkv, 32768, D, 2, 32)
+    ex["decode_2bit_32k_B16_8_layers_one_launch"] = {
+        "ms": round(ms2, 5), "ms_per_layer": round(ms2 / NL2, 5), "GBps": round(nbytes2 / ms2 / 1e6, 1),
+        "frac_hbm": round(nbytes2 / ms2 / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes2}
+    del layers2, stack2, q2
     # config 1: Llama-3-8B layer, one sequence, 8192 tokens as 2-bit group-32 codes plus a 128-token fp16 tail
     c1, fn1, nbytes1 = _decode_cfg1_case(torch, dev)
     for _ in range(3):
