@@ -341,6 +341,15 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
         out_t = K.kivi_packed_attend(qt, scale=scale, causal=causal, sliding_window=window, out_dtype=torch.float32,
                                      tiles=tiles, **cache)
         assert torch.equal(out_t, out), float((out_t - out).abs().max())
+    if plan["path"] == 3:
+        # the four-rows-a-block vector kernel against the one-wave-a-row one: both rebuild code * scale + zero in
+        # float32, so they differ by the order of their sums only
+        gen_plan = {}
+        out_g = K.kivi_packed_attend(qt, n_packed=n_packed, bits=b, group_size=g, v_layout=v_layout, k_tail=tail_k,
+                                     v_tail=tail_v, n_tail=n_tail, scale=scale, causal=causal, sliding_window=window,
+                                     out_dtype=torch.float32, num_splits=-1, _plan_out=gen_plan, **kw)
+        assert gen_plan["path"] == 0
+        assert float((out - out_g).abs().max()) < 5e-5, float((out - out_g).abs().max())
     if plan["path"] == 1:
         # the single-launch form (last block of a kv head merges the splits) and the form with a
         # separate merge kernel run the same arithmetic (compared with the token chunks dealt in
@@ -377,14 +386,14 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
 @pytest.mark.parametrize("meta", [torch.float16, torch.float32])
 def test_packed_decode_with_tail(v_layout, b, g, meta):
     _packed_case(2, 8, 2, 512, 37, 128, b, g, v_layout, meta, seed=b + g,
-                 expect_path=1 if v_layout == "token" else 0)
+                 expect_path=1 if v_layout == "token" else 3)
 
 
 @pytest.mark.parametrize("v_layout", ["channel", "token"])
 def test_packed_decode_config1_llama_shape(v_layout):
     """32 query heads / 8 kv heads, 8192 tokens 2-bit group 32 + 128-token fp16 tail."""
     _packed_case(1, 32, 8, 8192, 128, 128, 2, 32, v_layout, torch.float16, seed=1,
-                 expect_path=1 if v_layout == "token" else 0)
+                 expect_path=1 if v_layout == "token" else 3)
 
 
 def test_packed_decode_no_tail_and_spare_capacity():
@@ -434,6 +443,41 @@ def test_mfma_decode_groups_of_more_than_eight_heads(b, g, meta, Hq, Hkv, Sq, n_
     if Sq == 3:
         _packed_case(1, Hq, Hkv, 640, n_tail, 128, b, g, "token", meta, Sq=Sq, causal=True, seed=Hq + g, expect_path=1,
                      window=200)
+
+
+@pytest.mark.parametrize("D,b,g,Hq,Hkv,v_layout,meta", [
+    (256, 2, 32, 12, 4, "token", torch.float16),     # the head size of config 2's model, 3 query heads a kv head
+    (256, 4, 64, 8, 2, "token", torch.float16),
+    (256, 4, 32, 16, 2, "channel", torch.float32),   # eight query heads a kv head: two tiles of four
+    (128, 3, 32, 32, 8, "token", torch.float16),     # words of ten codes: a lane's channels straddle value groups
+    (128, 3, 64, 6, 2, "channel", torch.float32),
+    (64, 4, 32, 8, 8, "token", torch.float16),
+    (64, 2, 32, 4, 1, "channel", torch.float16),
+    (96, 8, 32, 6, 2, "token", torch.float16),
+    (128, 1, 32, 8, 2, "token", torch.float16),      # 32 codes a word, eight channels a lane
+    (128, 4, 32, 20, 4, "channel", torch.float16),   # channel-packed values at the MFMA kernel's head size; ratio 5
+    (160, 5, 32, 4, 2, "token", torch.float32),      # six codes a word
+])
+def test_rows_kernel_head_sizes_bit_widths_and_layouts(D, b, g, Hq, Hkv, v_layout, meta):
+    """The shapes the matrix-unit kernels do not take (head sizes other than 128, bit widths other than 2 and 4,
+    channel-packed values, float32 tails) run on the vector kernel that shares a kv head's bytes among its query
+    heads (the reference's kernel covers D up to 256 and 2 / 3 / 4 bits,
+    veloxquant_mlx/tests/metal/test_scalar_attend.py:165-235): single-query decode with a tail, a few query positions
+    under the causal mask and a window, and against the one-wave-a-row kernel."""
+    n_packed = 960 if b != 3 and b != 5 else 960 - 960 % (32 // b * g // math.gcd(32 // b, g))
+    _packed_case(2, Hq, Hkv, n_packed, 37, D, b, g, v_layout, meta, seed=D + b, expect_path=3)
+    _packed_case(1, Hq, Hkv, n_packed, 0, D, b, g, v_layout, meta, Sq=5, causal=True, seed=D + b + 1, expect_path=3)
+    _packed_case(1, Hq, Hkv, n_packed, 21, D, b, g, v_layout, meta, Sq=3, causal=True, seed=D + b + 2, expect_path=3,
+                 window=300, tail_dtype=torch.bfloat16)
+
+
+def test_rows_kernel_plain_rows_and_many_splits():
+    """No packed prefix at a head size of 256 (plain fp16 / float32 keys and values, decode and a short causal
+    prefill), and a long context that is cut into many runs."""
+    _packed_case(2, 8, 2, 0, 700, 256, 4, 32, "token", torch.float16, seed=91, expect_path=3)
+    _packed_case(1, 8, 2, 0, 300, 256, 4, 32, "token", torch.float16, Sq=40, causal=True, seed=92, expect_path=3,
+                 tail_dtype=torch.float32)
+    _packed_case(1, 3, 1, 16384, 100, 256, 2, 32, "token", torch.float16, seed=93, expect_path=3)
 
 
 def test_mfma_decode_many_splits_and_single_unit():
@@ -494,7 +538,7 @@ def test_mfma_prefill_not_causal_and_split_tokens():
 
 
 def test_mfma_prefill_odd_head_ratio_takes_vector_kernel():
-    _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=4, causal=True, seed=23, expect_path=0)
+    _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=4, causal=True, seed=23, expect_path=3)
     _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=1, seed=24, expect_path=1)
 
 
@@ -506,7 +550,7 @@ def test_mfma_path_takes_bf16_tails():
     _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=12, causal=True, seed=34,
                  q_dtype=torch.bfloat16, tail_dtype=torch.bfloat16, expect_path=1)
     _packed_case(1, 8, 2, 256, 77, 128, 4, 32, "token", torch.float16, Sq=1, seed=33, tail_dtype=torch.float32,
-                 expect_path=0)
+                 expect_path=3)
 
 
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 2)])
@@ -620,7 +664,7 @@ def test_counted_copy_waits_equal_waiting_for_every_copy(bits, g, meta, Hq, Hkv)
     (3, 1, 8, 1, 2, 32, torch.float32),      # decode kernel, row tiles of several positions
     (64, 2, 8, 2, 4, 32, torch.float16),     # 64-row prefill blocks
     (80, 2, 16, 4, 2, 64, torch.float16),    # 256-row prefill blocks, last tile ragged
-    (5, 0, 6, 2, 3, 32, torch.float32),      # vector kernel (3-bit codes)
+    (5, 3, 6, 2, 3, 32, torch.float32),      # vector kernel (3-bit codes)
 ])
 def test_sliding_window(window, Sq, path, Hq, Hkv, b, g, meta):
     """A query at position p sees the slots (p - window, p] only (the window of
@@ -628,7 +672,7 @@ def test_sliding_window(window, Sq, path, Hq, Hkv, b, g, meta):
     windows that end inside the fp16 rows, straddle the packed / fp16 edge, cover a stretch of the
     packed prefix that is dropped whole, and exceed the sequence."""
     causal = Sq > 1
-    layout = "channel" if path == 0 else "token"
+    layout = "channel" if path == 3 else "token"
     # a window that ends inside the fp16 rows leaves no packed token: such a call takes whichever
     # kernel serves plain rows
     _packed_case(2, Hq, Hkv, 1024 + 128, 77, 128, b, g, layout, meta, Sq=Sq, causal=causal, seed=window + Sq,

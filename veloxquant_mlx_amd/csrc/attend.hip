@@ -36,6 +36,24 @@ AttendPlan plan_attend(const vq_attend_args &a) {
         p.nparts = p.nsplit;
         return p;
     }
+    if (p.path == 0 && a.num_splits >= 0 && rows_kernel_supported(a)) {
+        // four query rows of a kv head per block; splits until the grid holds four blocks per compute unit,
+        // of at least 256 tokens each
+        p.path = 3;
+        rows_tiling(a, p.pq, p.tiles);
+        const int64_t n_total = a.n_packed + a.n_tail;
+        const int64_t units = a.B * a.Hkv * p.tiles;
+        int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(1024, units > 0 ? units : 1);
+        const int64_t most = n_total > 256 ? n_total / 256 : 1;
+        if (ns > most) ns = most;
+        if (ns > 512) ns = 512;
+        if (ns < 1) ns = 1;
+        const int64_t len = cdiv(cdiv(n_total > 0 ? n_total : 1, ns), 64) * 64;
+        p.nsplit = (int)cdiv(n_total > 0 ? n_total : 1, len);
+        p.split_len = len;
+        p.nparts = p.nsplit;
+        return p;
+    }
     // tokens the kernel splits: the MFMA path hands the tail to a few waves of the block of split 0
     // and prices a tail token at TAIL_EQUIV packed tokens when it balances the splits
     int64_t n_split = a.n_packed + a.n_tail;
@@ -249,6 +267,10 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         const bool written = launch_attend_mfma_prefill(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
         if (written) return VQ_OK;
+    } else if (p.path == 3) {
+        rc = launch_attend_rows(*a, p);
+        if (rc != VQ_OK) return rc;
+        VQ_HIP_CHECK_LAUNCH(fn);
     } else {
         rc = launch_attend_generic(*a, p.nsplit, p.split_len);
         if (rc != VQ_OK) return rc;

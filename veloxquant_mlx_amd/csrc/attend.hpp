@@ -21,7 +21,8 @@ __device__ __host__ __forceinline__ int64_t window_first(const vq_attend_args &a
 }
 
 struct AttendPlan {
-    int path;           // 0 generic waves, 1 MFMA decode (row tiles of <= 8), 2 MFMA prefill (LDS-staged, 64-row blocks)
+    int path;           // 0 generic waves, 1 MFMA decode (row tiles of <= 8), 2 MFMA prefill (LDS-staged, 64-row blocks),
+                        // 3 vector-unit rows kernel (any head_dim / bit width, four query rows a block)
     int nsplit;         // splits along the tokens the main kernel covers
     int nparts;         // partials per query row handed to the merge kernel
     int64_t split_len;  // tokens per split (multiple of 64)
@@ -95,6 +96,11 @@ __device__ __forceinline__ float merge_records(const float *p, int nparts, int64
 AttendPlan plan_attend(const vq_attend_args &a);
 
 int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len);
+// vector-unit kernel with the kv head's bytes shared by its query heads (attend_rows.hip): whether it takes the
+// shapes, its row tiling (positions per tile, tiles per (sequence, kv head)), the launch
+bool rows_kernel_supported(const vq_attend_args &a);
+void rows_tiling(const vq_attend_args &a, int &pq, int &tiles);
+int launch_attend_rows(const vq_attend_args &a, const AttendPlan &p);
 int launch_attend_merge(const vq_attend_args &a, int nparts);
 // protected rows (vq_attend_args.sink_k): rewrites every output row from the partials in the
 // workspace, with the stand-ins' weights taken out and the exact rows put in
