@@ -53,7 +53,7 @@ def _parse():
     p.add_argument("--per-layer", action="store_true", help="with --only-kernel: one launch per layer")
     p.add_argument("--only", default=None, metavar="NAME",
                    help="run one side workload in a loop and print its timing (for rocprofv3): "
-                        "decode_2bit_B16, decode_2bit_B1, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
+                        "decode_2bit_B16, decode_2bit_B1, decode_d256_2bit_32k_B16, decode_3bit_32k_B16, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
     p.add_argument("--copy-calib", action="store_true",
                    help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
@@ -284,6 +284,28 @@ def main() -> int:
     return 0
 
 
+_ROWS_CASES = {"decode_d256_2bit_32k_B16": (12, 4, 256, 2, 32), "decode_3bit_32k_B16": (32, 8, 128, 3, 32)}
+
+
+def _decode_rows_case(torch, dev, name):
+    """Shapes the matrix-unit decode kernel does not take (they run on ``attend_rows_kernel``): the head size of config
+    2's model (Falcon3-7B: 12 query / 4 kv heads, D = 256) at 2 bits, and 3-bit codes (ten to a word) at the headline's
+    head shape; batch 16, 32768 packed tokens plus the fp16 residual."""
+    from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
+    hq, hkv, d, bits, g = _ROWS_CASES[name]
+    cfg = KVCacheConfig(method="kivi", head_dim=d, bit_width_inlier=bits, kivi_group_size=g, residual_length=128,
+                        fused_sdpa=True, fused_sdpa_memory_bound=True)
+    c = KVCacheFactory.create(cfg)
+    for s0 in range(0, 32768 + 128, 8192):
+        n = min(8192, 32768 + 128 - s0)
+        k, v = _synthetic_layer(torch, 16, hkv, n, d, 5 + s0, dev)
+        c.update_and_fetch(k, v)
+    q = torch.randn((16, hq, 1, d), device=dev).to(torch.float16)
+    words = -(-d // (32 // bits))     # 32-bit words a token row of codes takes
+    nbytes = 2 * 16 * hkv * 32768 * words * 4 + 2 * 16 * hkv * (32768 // g) * d * 2 * 2
+    return c, (lambda: c.fused_sdpa(q, 1 / math.sqrt(d))), nbytes
+
+
 def _decode_2bit_case(torch, dev, B):
     """2-bit group-32 packed cache of 32768 tokens plus the fp16 residual, one query token (the "@32k" target)."""
     from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
@@ -396,6 +418,8 @@ def _only(a, torch, K, dev):
     name = a.only
     if name in ("decode_2bit_B16", "decode_2bit_B1"):
         c, fn, nbytes = _decode_2bit_case(torch, dev, 16 if name.endswith("16") else 1)
+    elif name in _ROWS_CASES:
+        c, fn, nbytes = _decode_rows_case(torch, dev, name)
     elif name == "vq_assign":
         x, cb, fn = _vq_assign_case(torch, K, dev)
         nbytes = None
@@ -502,28 +526,15 @@ def _extras(torch, K, dev):
         "ms": round(ms2, 5), "ms_per_layer": round(ms2 / NL2, 5), "GBps": round(nbytes2 / ms2 / 1e6, 1),
         "frac_hbm": round(nbytes2 / ms2 / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes2}
     del layers2, stack2, q2
-    # shapes the matrix-unit decode kernel does not take run on the vector kernel that shares a kv head's bytes among
-    # its query heads: the head size of config 2's model (Falcon3-7B: 12 query / 4 kv heads, D = 256) at 2 bits,
-    # and 3-bit codes (ten to a word) at the headline's head shape
-    for name, (hq, hkv, d, bits, g) in (("decode_d256_2bit_32k_B16", (12, 4, 256, 2, 32)),
-                                        ("decode_3bit_32k_B16", (32, 8, 128, 3, 32))):
-        cfg = KVCacheConfig(method="kivi", head_dim=d, bit_width_inlier=bits, kivi_group_size=g, residual_length=128,
-                            fused_sdpa=True, fused_sdpa_memory_bound=True)
-        cv = KVCacheFactory.create(cfg)
-        for s0 in range(0, 32768 + 128, 8192):
-            n = min(8192, 32768 + 128 - s0)
-            kk, vv = _synthetic_layer(torch, 16, hkv, n, d, 5 + s0, dev)
-            cv.update_and_fetch(kk, vv)
-        qv = torch.randn((16, hq, 1, d), device=dev).to(torch.float16)
-        fnv = lambda: cv.fused_sdpa(qv, 1 / math.sqrt(d))
+    # shapes the matrix-unit decode kernel does not take: the vector kernel that shares a kv head's bytes among its query heads
+    for name in _ROWS_CASES:
+        cv, fnv, nb = _decode_rows_case(torch, dev, name)
         for _ in range(2):
             fnv()
         msv = _side_ms(fnv, 5, torch)
-        nb = _algorithmic_bytes_per_layer(16, hkv, 32768, d, bits, g) if bits != 3 else (
-            2 * 16 * hkv * 32768 * (-(-d // 10)) * 4 + 2 * 16 * hkv * (32768 // g) * d * 2 * 2)
         ex[name] = {"ms": round(msv, 4), "GBps": round(nb / msv / 1e6, 1), "frac_hbm": round(nb / msv / 1e6 / HBM_PEAK_GBS, 4),
                     "bytes": nb, "note": "vector-unit kernel (attend_rows_kernel), four query rows of a kv head per block"}
-        del cv, kk, vv, qv
+        del cv, fnv
     # config 1: Llama-3-8B layer, one sequence, 8192 tokens as 2-bit group-32 codes plus a 128-token fp16 tail
     c1, fn1, nbytes1 = _decode_cfg1_case(torch, dev)
     for _ in range(3):
