@@ -446,8 +446,8 @@ def test_mfma_decode_groups_of_more_than_eight_heads(b, g, meta, Hq, Hkv, Sq, n_
 
 
 @pytest.mark.parametrize("D,b,g,Hq,Hkv,v_layout,meta", [
-    (256, 2, 32, 12, 4, "token", torch.float16),     # the head size of config 2's model, 3 query heads a kv head
-    (256, 4, 64, 8, 2, "token", torch.float16),
+    (256, 2, 32, 12, 4, "channel", torch.float16),   # the head size of config 2's model, 3 query heads a kv head
+    (256, 8, 64, 8, 2, "token", torch.float16),
     (256, 4, 32, 16, 2, "channel", torch.float32),   # eight query heads a kv head: two tiles of four
     (128, 3, 32, 32, 8, "token", torch.float16),     # words of ten codes: a lane's channels straddle value groups
     (128, 3, 64, 6, 2, "channel", torch.float32),
@@ -477,7 +477,28 @@ def test_rows_kernel_plain_rows_and_many_splits():
     _packed_case(2, 8, 2, 0, 700, 256, 4, 32, "token", torch.float16, seed=91, expect_path=3)
     _packed_case(1, 8, 2, 0, 300, 256, 4, 32, "token", torch.float16, Sq=40, causal=True, seed=92, expect_path=3,
                  tail_dtype=torch.float32)
-    _packed_case(1, 3, 1, 16384, 100, 256, 2, 32, "token", torch.float16, seed=93, expect_path=3)
+    _packed_case(1, 3, 1, 16320, 100, 256, 3, 32, "token", torch.float16, seed=93, expect_path=3)
+
+
+@pytest.mark.parametrize("b,g,meta", [(2, 32, torch.float16), (4, 64, torch.float16), (4, 32, torch.float32),
+                                      (2, 128, torch.float32), (4, 128, torch.float16), (2, 64, torch.float16)])
+@pytest.mark.parametrize("Hq,Hkv", [(12, 4), (8, 2), (8, 1), (4, 4), (32, 2)])
+def test_mfma_decode_head_size_256(b, g, meta, Hq, Hkv):
+    """A head of 256 channels on the matrix-unit decode kernel (the head size of config 2's model, and of the
+    reference's own decode test, veloxquant_mlx/tests/metal/test_scalar_attend.py:202-218): two halves of 128 channels
+    in the first product, sixteen value tiles in the second, the fp16 tail as a partial of the vector kernel.  GQA
+    ratios 3, 4, 8, 1 and 16; with and without a tail; several query positions under the causal mask."""
+    _packed_case(2, Hq, Hkv, 1024, 37, 256, b, g, "token", meta, seed=Hq + g + b, expect_path=1)
+    _packed_case(1, Hq, Hkv, 2048 + 128, 0, 256, b, g, "token", meta, seed=Hq + g + b + 1, expect_path=1, cap_extra=128)
+    # several positions a tile: groups of 1, 2, 4 heads (8 / R positions), or eight heads of a larger group; a group of
+    # three heads at several positions is the vector kernel's
+    _packed_case(1, Hq, Hkv, 640, 70, 256, b, g, "token", meta, Sq=3, causal=True, seed=Hq + g + b + 2,
+                 expect_path=3 if Hq // Hkv == 3 else 1, tail_dtype=torch.bfloat16, window=500)
+
+
+def test_mfma_decode_head_size_256_long_context_and_float32_tail():
+    _packed_case(1, 12, 4, 16384, 100, 256, 2, 32, "token", torch.float16, seed=93, expect_path=1)
+    _packed_case(2, 12, 4, 4096, 64, 256, 4, 64, "token", torch.float16, seed=94, expect_path=1, tail_dtype=torch.float32)
 
 
 def test_mfma_decode_many_splits_and_single_unit():

@@ -60,7 +60,8 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     if (p.path == 1) {
         p.pq = mfma_positions_per_tile(a);
         p.tiles = mfma_row_tiles(a);
-        p.tail_equiv = a.n_tail > 0 ? cdiv(a.n_tail * TAIL_EQUIV, 128) * 128 : 0;
+        // (a head of 256 channels: the tail is a partial of the vector kernel, none of the block's work)
+        p.tail_equiv = a.n_tail > 0 && a.D == 128 ? cdiv(a.n_tail * TAIL_EQUIV, 128) * 128 : 0;
         n_split = a.n_packed + p.tail_equiv;
     }
     // the MFMA kernel wants every block to start on a boundary of the largest token group (128)
@@ -86,7 +87,7 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     p.nparts = p.nsplit;
     if (p.path == 1 && a.n_tail > 0) {
         int64_t tw = cdiv(cdiv(a.n_tail, 32), units >= 64 ? 8 : 1);
-        p.nparts += (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw);
+        p.nparts += a.D == 128 ? (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw) : 1;
     }
     return p;
 }
@@ -251,6 +252,11 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         return VQ_OK;
     };
     if (p.path == 1) {
+        if (a->D != 128 && a->n_tail > 0) {   // the tail as partial p.nsplit of every row, from the vector kernel
+            rc = launch_attend_rows_tail(*a, p.nsplit, p.nparts);
+            if (rc != VQ_OK) return rc;
+            VQ_HIP_CHECK_LAUNCH(fn);
+        }
         const bool merged = launch_attend_mfma_decode(*a, p);
         VQ_HIP_CHECK_LAUNCH(fn);
         if (merged) return finish();

@@ -36,6 +36,8 @@ struct AttendPlan {
     // MFMA decode path: deal token chunks to the waves round robin instead of on demand, so that
     // results are identical from run to run
     int fixed_order;
+    // rows kernel over the tail only: first partial it writes (-1: the whole context, partials 0 .. nsplit - 1)
+    int part0 = -1;
 };
 
 // One output element from the split partials of its query row: p points at nparts records
@@ -101,6 +103,8 @@ int launch_attend_generic(const vq_attend_args &a, int nsplit, int64_t split_len
 bool rows_kernel_supported(const vq_attend_args &a);
 void rows_tiling(const vq_attend_args &a, int &pq, int &tiles);
 int launch_attend_rows(const vq_attend_args &a, const AttendPlan &p);
+// the same kernel over the tail tokens only, into partial `part0` of `nparts` per query row
+int launch_attend_rows_tail(const vq_attend_args &a, int part0, int nparts);
 int launch_attend_merge(const vq_attend_args &a, int nparts);
 // protected rows (vq_attend_args.sink_k): rewrites every output row from the partials in the
 // workspace, with the stand-ins' weights taken out and the exact rows put in

@@ -20,7 +20,10 @@ int mfma_row_tiles(const vq_attend_args &a) {
 }
 
 bool mfma_decode_supported(const vq_attend_args &a) {
-    if (a.D != MF_D || a.n_packed <= 0) return false;
+    if ((a.D != MF_D && a.D != 2 * MF_D) || a.n_packed <= 0) return false;
+    // a head of 256 channels: packed prefix only (its tail goes through the vector kernel, one more launch), no
+    // token brought along by the call
+    if (a.D == 2 * MF_D && (a.k_new != nullptr || !rows_kernel_supported(a))) return false;
     if (a.Hq % a.Hkv != 0) return false;
     const int64_t R = a.Hq / a.Hkv;
     // a tile has eight rows (a high and a remainder column each): the whole group at one position, a
@@ -33,7 +36,9 @@ bool mfma_decode_supported(const vq_attend_args &a) {
     if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
     if (a.cap_tokens > (1 << 24)) return false;   // per-lane byte offsets are 32-bit
     if (!(a.scale > 0.f)) return false;
-    if (a.n_tail > 0 && (!(a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
+    if (a.D == MF_D && a.n_tail > 0 &&
+        (!(a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u)))
+        return false;
     const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
                          (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
     if (al & 15u) return false;
@@ -46,7 +51,15 @@ bool launch_attend_mfma_decode(const vq_attend_args &a, const AttendPlan &p) {
     // rows a block carries: the GQA group at p.pq positions, padded to 4 or 8
     const int64_t R = a.Hq / a.Hkv;
     const bool wide = (R > 8 ? 8 : R) * p.pq > 4;
-    if (a.meta_dtype == VQ_F16) {
+    if (a.D == 2 * MF_D) {
+        if (a.meta_dtype == VQ_F16) {
+            if (wide) launch_mfma_packed_d256_f16meta_r8(a, p, ws, st);
+            else launch_mfma_packed_d256_f16meta_r4(a, p, ws, st);
+        } else {
+            if (wide) launch_mfma_packed_d256_f32meta_r8(a, p, ws, st);
+            else launch_mfma_packed_d256_f32meta_r4(a, p, ws, st);
+        }
+    } else if (a.meta_dtype == VQ_F16) {
         if (wide) launch_mfma_packed_f16meta_r8(a, p, ws, st);
         else launch_mfma_packed_f16meta_r4(a, p, ws, st);
     } else {

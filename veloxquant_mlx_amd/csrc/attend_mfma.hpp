@@ -448,15 +448,17 @@ __device__ __forceinline__ void tail_wave(const vq_attend_args &a, int64_t bh, c
 // Combine the nparts partials of the tile's query rows into the output (the
 // arithmetic of attend_merge_kernel, which shares merge_partials).  Partials written by
 // other blocks of this launch are read with device-scope loads.
+template <int DH = 1>
 __device__ __forceinline__ void merge_rows(const vq_attend_args &a, const RowTile &tile, int nparts, const float *ws,
                                            int tid, int nthreads) {
-    for (int e = tid; e < tile.RT * MF_D; e += nthreads) {
-        const int j = e / MF_D, d = e % MF_D;
+    constexpr int DD = MF_D * DH, PART = DD + 2;
+    for (int e = tid; e < tile.RT * DD; e += nthreads) {
+        const int j = e / DD, d = e % DD;
         if (!tile.valid(j)) continue;
         const int64_t row = tile.row(j);
         // partials of other blocks come from beyond this XCD's L2: as few rounds of loads as possible
-        const float v = merge_records<true>(ws + row * nparts * MF_PART, nparts, MF_PART, d);
-        const int64_t oi = row * MF_D + d;
+        const float v = merge_records<true>(ws + row * nparts * PART, nparts, PART, d);
+        const int64_t oi = row * DD + d;
         if (a.out_dtype == VQ_F16) ((f16 *)a.out)[oi] = (f16)v;
         else if (a.out_dtype == VQ_BF16) ((u16 *)a.out)[oi] = f32_to_bf16(v);
         else ((float *)a.out)[oi] = v;
@@ -470,5 +472,10 @@ void launch_mfma_packed_f16meta_r4(const vq_attend_args &a, const AttendPlan &p,
 void launch_mfma_packed_f16meta_r8(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
 void launch_mfma_packed_f32meta_r4(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
 void launch_mfma_packed_f32meta_r8(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+// the same for a head of 256 channels (packed prefix only)
+void launch_mfma_packed_d256_f16meta_r4(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_d256_f16meta_r8(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_d256_f32meta_r4(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
+void launch_mfma_packed_d256_f32meta_r8(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st);
 
 }  // namespace vq

@@ -85,16 +85,18 @@ template <> struct TokMeta<float> {
 
 // How the 16 columns of the second product map to channel groups: GPP groups per probability
 // operand, NP operands per unit, TPP value tiles (of 16 channels) per operand.
-template <int GV, int RTP> struct Cols {
+// GV counts the groups of the whole head (DH * 128 channels, NT = 8 * DH value tiles).
+template <int GV, int RTP, int DH = 1> struct Cols {
+    static constexpr int NT = 8 * DH;
     static constexpr int GPP = GV < 16 / RTP ? GV : 16 / RTP;
     static constexpr int NP = GV / GPP;
-    static constexpr int TPG = 8 / GV;
-    static constexpr int TPP = 8 / NP;
+    static constexpr int TPG = NT / GV;
+    static constexpr int TPP = NT / NP;
 };
 
 // Per-wave state of the packed kernel.
-struct PackedAcc {
-    f32x4 O[8];     // tile nt, register r: channel 16*nt + 4*blk + r of the lane's column, times 2^(EV - 24)
+template <int NT = 8> struct PackedAcc {
+    f32x4 O[NT];    // tile nt, register r: channel 16*nt + 4*blk + r of the lane's column, times 2^(EV - 24)
     f32x4 Z;        // register r = operand row 4*blk + r: sum_t P z_g (rows g < GV), sum_t P (rows >= 8)
     float m_run;    // softmax reference, log2 domain, of the lane's column (query row)
     float thr;      // m_run + SLACK: a score above it moves the reference
@@ -102,14 +104,14 @@ struct PackedAcc {
                     // its k-slot pair in the second product
 };
 
-template <int BITS, typename M, int NP> struct PackedUnit {
-    u32 kw[2][(MF_D * BITS / 32) / 4];   // key words of the lane's 32 channels, two token rows
-    u32 vw[8];                           // value words, one per 16-channel tile
+template <int BITS, typename M, int NP, int DH = 1> struct PackedUnit {
+    u32 kw[DH][2][(MF_D * BITS / 32) / 4];   // key words of the lane's 32 channels of every 128-channel half, two token rows
+    u32 vw[8 * DH];                      // value words, one per 16-channel tile
     TokMeta<M> s[NP];                    // value scales of the lane's eight tokens, the lane's group of each operand
     TokMeta<M> z;                        // operand row of the sums product (see PackedAcc::Z)
 };
 
-constexpr int PK_QROW = 136;                  // halves between query rows in LDS (128 + 8: rows on different banks)
+constexpr int PK_QROW = 136;                  // halves between query rows in LDS (128 + 8: rows on different banks; a head of 256 channels: 264)
 constexpr int PK_QIMG_ROW = 272;              // bytes between rows of a wave's folded-query image
 
 // A wave's ring: DEPTH unit slots, then GROUP_SLOTS group slots, then the folded-query image.
@@ -131,26 +133,28 @@ constexpr int ex_bytes(int waves) { return ex_o(waves) + ex_z(waves) + 2 * ex_m(
 constexpr int PK_ALIGN = 128;                 // tokens: blocks start on a multiple of the largest token group
 constexpr int PK_STATIC_LDS = 4096;           // query rows, constant rows, counters (static block-shared memory)
 
-template <int BITS, typename M, int GV, int RTP> struct Ring {
+template <int BITS, typename M, int GV, int RTP, int DH = 1> struct Ring {
     static constexpr int MSZ = sizeof(M);
-    static constexpr int KB = 512 * BITS, VB = 512 * BITS;
+    static constexpr int KB = 512 * BITS * DH, VB = 512 * BITS * DH;
     static constexpr int VMR = GV * 32 * MSZ;      // bytes of the scale rows (and of the zero rows)
-    static constexpr int KMR = MF_D * MSZ;         // bytes of a key scale (zero) row
+    static constexpr int KMR = MF_D * DH * MSZ;    // bytes of a key scale (zero) row
     static constexpr int K_OFF = 0, V_OFF = KB, VS_OFF = KB + VB, VZ_OFF = VS_OFF + VMR;
     static constexpr int SLOT = VZ_OFF + VMR, GROUP_SLOT = 2 * KMR;
     // copies per unit, and per unit that opens a token group
     static constexpr int VM_COPIES = VMR > 256 ? VMR / 256 : 1, KM_COPIES = KMR / 256;
-    static constexpr int UNIT_COPIES = (BITS == 4 ? 4 : 2) + 2 * VM_COPIES, GROUP_COPIES = 2 * KM_COPIES;
-    static constexpr int UPG = 4 / GV;             // units per token group
-    static constexpr int QIMG = 2 * RTP * PK_QIMG_ROW;
+    static constexpr int UNIT_COPIES = (BITS == 4 ? 4 : 2) * DH + 2 * VM_COPIES, GROUP_COPIES = 2 * KM_COPIES;
+    static constexpr int UPG = (MF_D * DH / GV) / 32;   // units per token group
+    static constexpr int QIMG = 2 * RTP * PK_QIMG_ROW * DH;
     // a group slot is read only while its group is opened, and refilled by the opener issued
     // ceil(DEPTH / UPG) openers later -- at the earliest in the same pass, after that read
     static constexpr int group_slots(int depth) { return (depth + UPG - 1) / UPG; }
     static constexpr int bytes_at(int depth) { return depth * SLOT + group_slots(depth) * GROUP_SLOT; }
     // the block has the CU's 160 KB to itself
-    static constexpr int budget(int waves) { return (160 * 1024 - PK_STATIC_LDS) / waves - QIMG; }
-    // (float32 scale / zero: the unit loop holds more than a third of the register file, eight waves)
-    static constexpr int WAVES = MSZ == 2 && bytes_at(2) <= budget(PK_MAX_WAVES) ? PK_MAX_WAVES : 8;
+    static constexpr int budget(int waves) { return (160 * 1024 - PK_STATIC_LDS * DH) / waves - QIMG; }
+    // (float32 scale / zero: the unit loop holds more than a third of the register file, eight waves; a head of
+    // 256 channels: 64 accumulator registers, eight waves, or four where eight rings of two units do not fit)
+    static constexpr int WAVES = DH == 1 ? (MSZ == 2 && bytes_at(2) <= budget(PK_MAX_WAVES) ? PK_MAX_WAVES : 8)
+                                         : (bytes_at(2) <= budget(8) ? 8 : 4);
     static constexpr int THREADS = 64 * WAVES;
     static constexpr int BUDGET = budget(WAVES);
     static constexpr int DEPTH = bytes_at(5) <= BUDGET ? 5 : bytes_at(4) <= BUDGET ? 4 : bytes_at(3) <= BUDGET ? 3 : 2;
@@ -162,7 +166,8 @@ template <int BITS, typename M, int GV, int RTP> struct Ring {
     // least (DEPTH - 1) / UPG open a group
     static constexpr int LATER = (DEPTH - 1) * UNIT_COPIES + ((DEPTH - 1) / UPG) * GROUP_COPIES;
     static constexpr int WAVE_BYTES = QIMG_OFF + QIMG;
-    static constexpr int BYTES = WAVES * WAVE_BYTES > ex_bytes(WAVES) ? WAVES * WAVE_BYTES : ex_bytes(WAVES);
+    static constexpr int EX_BYTES = ex_o(WAVES) * DH + ex_z(WAVES) + 2 * ex_m(WAVES);
+    static constexpr int BYTES = WAVES * WAVE_BYTES > EX_BYTES ? WAVES * WAVE_BYTES : EX_BYTES;
     // Units are handed out to the waves in chunks of CHUNK consecutive units: whole token groups,
     // and at least DEPTH units, so that the copies never run more than one chunk ahead of
     // the arithmetic.
@@ -171,13 +176,14 @@ template <int BITS, typename M, int GV, int RTP> struct Ring {
 };
 
 // The query rows of the block as fp16 in LDS, PK_QROW halves apart; rows the tile does not have are zero.
-template <int RTP, int THREADS>
+template <int RTP, int THREADS, int DH = 1>
 __device__ __forceinline__ void stage_query(const vq_attend_args &a, const RowTile &tile, int tid, f16 *s_qraw) {
-    for (int e = tid; e < RTP * MF_D / 8; e += THREADS) {
-        const int row = e / (MF_D / 8), d = 8 * (e % (MF_D / 8));
+    constexpr int DD = MF_D * DH, PK_QROW = DD + 8;
+    for (int e = tid; e < RTP * DD / 8; e += THREADS) {
+        const int row = e / (DD / 8), d = 8 * (e % (DD / 8));
         f16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
         if (tile.valid(row)) {
-            const int64_t i = tile.row(row) * MF_D + d;
+            const int64_t i = tile.row(row) * DD + d;
             if (a.q_dtype == VQ_F16) v = *reinterpret_cast<const f16x8 *>((const f16 *)a.q + i);
             else {
 #pragma unroll
@@ -195,17 +201,20 @@ template <int N> __device__ __forceinline__ float row_ror(float x) {
 
 // order: bit 0 = deal the chunks round robin, bit 1 = wait for every copy in flight instead of the
 // counted ones (a slower, count-free cross-check of the ring's accounting)
-template <int BITS, typename M, int GV, int RTP>
+template <int BITS, typename M, int GV, int RTP, int DH = 1>
 __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh, float c, int64_t t_begin,
                                              int n_units, int lane_vis, int full_vis, int lane_lo, int lo_edge, int lane, int wave,
-                                             PackedAcc &acc, const f16 *s_qraw,
+                                             PackedAcc<8 * DH> &acc, const f16 *s_qraw,
                                              const char *s_const, char *ring, int *s_next, int order) {
-    using CL = Cols<GV, RTP>;
+    using CL = Cols<GV, RTP, DH>;
+    constexpr int DD = MF_D * DH;            // head size: DH halves of 128 channels, each worked like a head of 128
+    constexpr int QROW = DD + 8;             // halves between query rows in LDS
     constexpr int PER = 32 / BITS;           // codes per word
-    constexpr int KW = MF_D / PER;           // key words per token row
-    constexpr int KWL = KW / 4;              // key words one lane loads per token (its 32 channels)
+    constexpr int KW = DD / PER;             // key words per token row
+    constexpr int KWL = (MF_D / PER) / 4;    // key words one lane loads per token and half (its 32 channels)
+    constexpr int HB = 16 * BITS;            // bytes of a half inside a token row of key codes
     constexpr int GAP = vtok_gap<BITS>();
-    constexpr int G = MF_D / GV;             // tokens per key group = channels per value group
+    constexpr int G = DD / GV;               // tokens per key group = channels per value group
     constexpr u32 MSZ = sizeof(M);
     constexpr bool F32META = sizeof(M) != 2;
     using SB = Sub<BITS>;
@@ -216,14 +225,14 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 
     // block-uniform bases, 32-bit per-lane byte offsets
     const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
-    const char *vb = (const char *)a.v_packed + bh * (cap / PER) * MF_D * 4;
-    const char *ksb = (const char *)a.k_scale + bh * (cap / G) * MF_D * MSZ;
-    const char *kzb = (const char *)a.k_zero + bh * (cap / G) * MF_D * MSZ;
+    const char *vb = (const char *)a.v_packed + bh * (cap / PER) * DD * 4;
+    const char *ksb = (const char *)a.k_scale + bh * (cap / G) * DD * MSZ;
+    const char *kzb = (const char *)a.k_zero + bh * (cap / G) * DD * MSZ;
     const char *vsb = (const char *)a.v_scale + bh * GV * cap * MSZ;
     const char *vzb = (const char *)a.v_zero + bh * GV * cap * MSZ;
 
-    using RG = Ring<BITS, M, GV, RTP>;
-    using Unit = PackedUnit<BITS, M, CL::NP>;
+    using RG = Ring<BITS, M, GV, RTP, DH>;
+    using Unit = PackedUnit<BITS, M, CL::NP, DH>;
     char *wring = ring + wave * RG::WAVE_BYTES;
     const u32 wring_lds = lds_addr(wring);
     // ---- what a lane copies.  Key codes: token of S^T row n in tile T is vtok_lo(n / 4, n % 4) + T * GAP.
@@ -235,8 +244,10 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const u32 l16 = 16u * lane, l4 = 4u * lane;
     // value scale (zero) rows: byte 4*lane (+256 for a second copy) of the [GV][32] image, row g at g*cap
     constexpr int VROW = 32 * (int)MSZ;
-    const u32 vmoff0 = (u32)((int64_t)(l4 / VROW) * cap * MSZ + l4 % VROW);
-    const u32 vmoff1 = (u32)((int64_t)((256 + l4) / VROW) * cap * MSZ + (256 + l4) % VROW);
+    u32 vmoff[RG::VM_COPIES];   // copy c: byte 256 c + 4 lane of the image
+#pragma unroll
+    for (int cc = 0; cc < RG::VM_COPIES; ++cc)
+        vmoff[cc] = (u32)((int64_t)((256 * cc + l4) / VROW) * cap * MSZ + (256 * cc + l4) % VROW);
     constexpr u32 VM_ACTIVE = RG::VMR / 4 < 64 ? RG::VMR / 4 : 64;
 
     // a unit that opens a token group brings the group's key scale / zero along, into group slot `gslot`
@@ -247,22 +258,27 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         const u32 ug = unit0 + (u32)u;   // unit number counted from token 0
         const u32 sl = wring_lds + (u32)slot * RG::SLOT;
         const char *kp = kb + ug * (u32)RG::KB;
-        if constexpr (BITS == 4) {
-            lds_copy16<0>(kp, koff, sl + RG::K_OFF);
-            lds_copy16<GAP * KW * 4>(kp, koff, sl + RG::K_OFF + 1024 - GAP * KW * 4);
-        } else {
-            lds_copy16<0>(kp, koff, sl + RG::K_OFF);
+        // key codes: every half of the head lands as a head of 128 channels does, KB / DH bytes apart
+#pragma unroll
+        for (int h = 0; h < DH; ++h) {
+            const u32 kh_lds = sl + RG::K_OFF + h * (RG::KB / DH);
+            lds_copy16<0>(kp, koff + h * HB, kh_lds);
+            if constexpr (BITS == 4) lds_copy16<GAP * KW * 4>(kp, koff + h * HB, kh_lds + 1024 - GAP * KW * 4);
         }
+        // value codes: the unit's word rows as they lie in memory, a kilobyte a copy
         const char *vp = vb + ug * (u32)RG::VB;
         lds_copy16<0>(vp, l16, sl + RG::V_OFF);
-        if constexpr (BITS == 4) lds_copy16<1024>(vp, l16, sl + RG::V_OFF);
+        if constexpr (RG::VB >= 2048) lds_copy16<1024>(vp, l16, sl + RG::V_OFF);
+        if constexpr (RG::VB >= 4096) {
+            lds_copy16<2048>(vp, l16, sl + RG::V_OFF);
+            lds_copy16<3072>(vp, l16, sl + RG::V_OFF);
+        }
         const char *vsp = vsb + ug * (32 * MSZ), *vzp = vzb + ug * (32 * MSZ);
         if (VM_ACTIVE == 64 || lane < (int)VM_ACTIVE) {
-            lds_copy4<0>(vsp, vmoff0, sl + RG::VS_OFF);
-            lds_copy4<0>(vzp, vmoff0, sl + RG::VZ_OFF);
-            if constexpr (RG::VM_COPIES == 2) {
-                lds_copy4<0>(vsp, vmoff1, sl + RG::VS_OFF + 256);
-                lds_copy4<0>(vzp, vmoff1, sl + RG::VZ_OFF + 256);
+#pragma unroll
+            for (int cc = 0; cc < RG::VM_COPIES; ++cc) {
+                lds_copy4<0>(vsp, vmoff[cc], sl + RG::VS_OFF + 256 * cc);
+                lds_copy4<0>(vzp, vmoff[cc], sl + RG::VZ_OFF + 256 * cc);
             }
         }
         if (opener) {
@@ -271,9 +287,15 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             const u32 gs = wring_lds + RG::GROUP_OFF + (u32)gslot * RG::GROUP_SLOT;
             lds_copy4<0>(ksp, l4, gs);
             lds_copy4<0>(kzp, l4, gs + RG::KMR);
-            if constexpr (RG::KM_COPIES == 2) {
+            if constexpr (RG::KM_COPIES >= 2) {
                 lds_copy4<256>(ksp, l4, gs);
                 lds_copy4<256>(kzp, l4, gs + RG::KMR);
+            }
+            if constexpr (RG::KM_COPIES >= 4) {
+                lds_copy4<512>(ksp, l4, gs);
+                lds_copy4<512>(kzp, l4, gs + RG::KMR);
+                lds_copy4<768>(ksp, l4, gs);
+                lds_copy4<768>(kzp, l4, gs + RG::KMR);
             }
         }
     };
@@ -293,22 +315,26 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     const int zs_off = (zs_ones ? 0 : RG::VZ_OFF + (n < GV ? n : 0) * VROW) + tok_a * (int)MSZ;
     auto read_unit = [&](int slot, Unit &d) VQ_INLINE_LAMBDA {
         const char *sl = wring + slot * RG::SLOT;
-        if constexpr (BITS == 4) {
 #pragma unroll
-            for (int T = 0; T < 2; ++T) {
-                const uint4 x = *reinterpret_cast<const uint4 *>(sl + RG::K_OFF + 1024 * T + 16 * lane);
-                d.kw[T][0] = x.x; d.kw[T][1] = x.y; d.kw[T][2] = x.z; d.kw[T][3] = x.w;
-            }
-        } else {
+        for (int h = 0; h < DH; ++h) {
+            const char *kh = sl + RG::K_OFF + h * (RG::KB / DH);
+            if constexpr (BITS == 4) {
 #pragma unroll
-            for (int T = 0; T < 2; ++T) {
-                const uint2 x = *reinterpret_cast<const uint2 *>(sl + RG::K_OFF + (16 * (2 * (blk >> 1) + T) + n) * 16 + 8 * (blk & 1));
-                d.kw[T][0] = x.x; d.kw[T][1] = x.y;
+                for (int T = 0; T < 2; ++T) {
+                    const uint4 x = *reinterpret_cast<const uint4 *>(kh + 1024 * T + 16 * lane);
+                    d.kw[h][T][0] = x.x; d.kw[h][T][1] = x.y; d.kw[h][T][2] = x.z; d.kw[h][T][3] = x.w;
+                }
+            } else {
+#pragma unroll
+                for (int T = 0; T < 2; ++T) {
+                    const uint2 x = *reinterpret_cast<const uint2 *>(kh + (16 * (2 * (blk >> 1) + T) + n) * 16 + 8 * (blk & 1));
+                    d.kw[h][T][0] = x.x; d.kw[h][T][1] = x.y;
+                }
             }
         }
 #pragma unroll
-        for (int nt = 0; nt < 8; ++nt)
-            d.vw[nt] = *reinterpret_cast<const u32 *>(sl + RG::V_OFF + vrow * 512 + (16 * nt + n) * 4);
+        for (int nt = 0; nt < CL::NT; ++nt)
+            d.vw[nt] = *reinterpret_cast<const u32 *>(sl + RG::V_OFF + vrow * (4 * DD) + (16 * nt + n) * 4);
 #pragma unroll
         for (int p = 0; p < CL::NP; ++p)
             d.s[p].read(sl + RG::VS_OFF + (p * CL::GPP + vgrp) * VROW + tok_a * (int)MSZ, GAP * (int)MSZ);
@@ -325,97 +351,110 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     // first channel of the piece in k-slot pair order: pair p = (ch0 + p, ch0 + p + PAIR_GAP)
     constexpr int PAIR_GAP = BITS == 4 ? 4 : 8;
     const int w_ch0 = 32 * w_blk + (BITS == 4 ? 8 * w_ks : 16 * (w_ks >> 1) + 4 * (w_ks & 1));
-    u32 qpair[WR][4];
+    u32 qpair[DH][WR][4];
 #pragma unroll
-    for (int u = 0; u < WR; ++u)
+    for (int h = 0; h < DH; ++h)
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const f16 *qr = s_qraw + (w_row + 4 * u) * PK_QROW + w_ch0 + p;
-            // k-slot pair p of an operand sits at mantissa bit pos(p): its query side carries 2^(EK - pos(p))
-            qpair[u][p] = as_u(f16x2{qr[0], qr[PAIR_GAP]} * h2(SB::wk(p)));
-        }
+        for (int u = 0; u < WR; ++u)
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const f16 *qr = s_qraw + (w_row + 4 * u) * QROW + MF_D * h + w_ch0 + p;
+                // k-slot pair p of an operand sits at mantissa bit pos(p): its query side carries 2^(EK - pos(p))
+                qpair[h][u][p] = as_u(f16x2{qr[0], qr[PAIR_GAP]} * h2(SB::wk(p)));
+            }
     char *qimg = wring + RG::QIMG_OFF;
+    constexpr int IMG = 2 * RTP * PK_QIMG_ROW;   // bytes of the folded-query image of one half
     const int w_off = w_row * PK_QIMG_ROW + w_blk * 64 + w_ks * 16;
     const int r_off = (col_lo * RTP + col_row) * PK_QIMG_ROW + blk * 64;
     // bias chain: every operand row carries the group's zeros; the query rows (high columns only;
-    // remainder columns read zeros) are the other operand
-    f16x8 q0[4];
+    // remainder columns read zeros) are the other operand.  A head of 128 channels keeps them in registers;
+    // a wider one, whose accumulators need the room, reads them again for every group.
+    auto q_rows = [&](int h, int ks) VQ_INLINE_LAMBDA {
+        f16x8 v = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
+        if (!col_lo) v = *reinterpret_cast<const f16x8 *>(s_qraw + col_row * QROW + MF_D * h + 32 * blk + 8 * ks);
+        return v;
+    };
+    f16x8 q0[DH == 1 ? 4 : 1];
+    if constexpr (DH == 1) {
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-        q0[ks] = f16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        if (!col_lo) q0[ks] = *reinterpret_cast<const f16x8 *>(s_qraw + col_row * PK_QROW + 32 * blk + 8 * ks);
+        for (int ks = 0; ks < 4; ++ks) q0[ks] = q_rows(0, ks);
     }
 
-    f16x8 qB[4];   // folded query of the open token group (high columns | remainder columns)
+    f16x8 qB[DH][4];   // folded query of the open token group (high columns | remainder columns)
     f32x4 bias;    // what the score accumulators start from; every register alike
-    const f16x8 ones = ones8();
 
     auto open_group = [&](int gslot) VQ_INLINE_LAMBDA {
         const char *gs = wring + RG::GROUP_OFF + gslot * RG::GROUP_SLOT;
         f32x4 bt = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (!F32META) {
-            // ---- folded query, writer role
-            u32 sp[4];
-            if constexpr (BITS == 4) {
-                const uint4 x = *reinterpret_cast<const uint4 *>(gs + w_ch0 * 2);
-                sp[0] = pair_lo(x.x, x.z); sp[1] = pair_hi(x.x, x.z); sp[2] = pair_lo(x.y, x.w); sp[3] = pair_hi(x.y, x.w);
+#pragma unroll
+        for (int h = 0; h < DH; ++h) {
+            char *img = qimg + h * IMG;
+            if constexpr (!F32META) {
+                // ---- folded query, writer role
+                u32 sp[4];
+                const char *sh = gs + (MF_D * h + w_ch0) * 2;
+                if constexpr (BITS == 4) {
+                    const uint4 x = *reinterpret_cast<const uint4 *>(sh);
+                    sp[0] = pair_lo(x.x, x.z); sp[1] = pair_hi(x.x, x.z); sp[2] = pair_lo(x.y, x.w); sp[3] = pair_hi(x.y, x.w);
+                } else {
+                    const uint2 x = *reinterpret_cast<const uint2 *>(sh);
+                    const uint2 y = *reinterpret_cast<const uint2 *>(sh + 16);
+                    sp[0] = pair_lo(x.x, y.x); sp[1] = pair_hi(x.x, y.x); sp[2] = pair_lo(x.y, y.y); sp[3] = pair_hi(x.y, y.y);
+                }
+#pragma unroll
+                for (int u = 0; u < WR; ++u) {
+                    u32 hi[4], lo[4];
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const f16x2 t = as_h2(qpair[h][u][p]) * as_h2(sp[p]);   // round(q s)
+                        // q*s has at most 22 significant bits: the remainder after the fp16
+                        // high part is itself an fp16 number, so this fma is exact
+                        hi[p] = as_u(t);
+                        lo[p] = as_u(__builtin_elementwise_fma(as_h2(qpair[h][u][p]), as_h2(sp[p]), -t));
+                    }
+                    *reinterpret_cast<uint4 *>(img + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
+                    *reinterpret_cast<uint4 *>(img + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
+                }
+                // ---- bias chain: the zeros of the lane's 32 channels in every operand row
+                const char *zs = gs + RG::KMR + MF_D * h * 2 + 64 * blk;
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+                    bt = VQ_MFMA(as_h8(*reinterpret_cast<const uint4 *>(zs + 16 * ks)), DH == 1 ? q0[DH == 1 ? ks : 0] : q_rows(h, ks), bt);
             } else {
-                const uint2 x = *reinterpret_cast<const uint2 *>(gs + w_ch0 * 2);
-                const uint2 y = *reinterpret_cast<const uint2 *>(gs + (w_ch0 + 8) * 2);
-                sp[0] = pair_lo(x.x, y.x); sp[1] = pair_hi(x.x, y.x); sp[2] = pair_lo(x.y, y.y); sp[3] = pair_hi(x.y, y.y);
-            }
+                // float32 scale / zero: q * s formed in float32 and split into an fp16 pair
 #pragma unroll
-            for (int u = 0; u < WR; ++u) {
-                u32 hi[4], lo[4];
+                for (int u = 0; u < WR; ++u) {
+                    u32 hi[4], lo[4];
 #pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const f16x2 t = as_h2(qpair[u][p]) * as_h2(sp[p]);   // round(q s)
-                    // q*s has at most 22 significant bits: the remainder after the fp16
-                    // high part is itself an fp16 number, so this fma is exact
-                    hi[p] = as_u(t);
-                    lo[p] = as_u(__builtin_elementwise_fma(as_h2(qpair[u][p]), as_h2(sp[p]), -t));
+                    for (int p = 0; p < 4; ++p) {
+                        const float s0 = *reinterpret_cast<const float *>(gs + (MF_D * h + w_ch0 + p) * 4);
+                        const float s1 = *reinterpret_cast<const float *>(gs + (MF_D * h + w_ch0 + p + PAIR_GAP) * 4);
+                        const float t0 = (float)as_h2(qpair[h][u][p])[0] * s0, t1 = (float)as_h2(qpair[h][u][p])[1] * s1;
+                        const f16x2 hp = pinned_h2(f16x2{(f16)t0, (f16)t1});
+                        hi[p] = as_u(hp);
+                        lo[p] = as_u(f16x2{(f16)(t0 - (float)hp[0]), (f16)(t1 - (float)hp[1])});
+                    }
+                    *reinterpret_cast<uint4 *>(img + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
+                    *reinterpret_cast<uint4 *>(img + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
                 }
-                *reinterpret_cast<uint4 *>(qimg + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
-                *reinterpret_cast<uint4 *>(qimg + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
-            }
-            // ---- bias chain: the zeros of the lane's 32 channels in every operand row
-            const char *zs = gs + RG::KMR + 64 * blk;
+                // bias chain: the zeros as fp16 high parts, then their remainders, in every operand row
+                const char *zs = gs + RG::KMR + MF_D * h * 4 + 128 * blk;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-                bt = VQ_MFMA(as_h8(*reinterpret_cast<const uint4 *>(zs + 16 * ks)), q0[ks], bt);
-        } else {
-            // float32 scale / zero: q * s formed in float32 and split into an fp16 pair
+                for (int ks = 0; ks < 4; ++ks) {
+                    const float4 x0 = *reinterpret_cast<const float4 *>(zs + 32 * ks);
+                    const float4 x1 = *reinterpret_cast<const float4 *>(zs + 32 * ks + 16);
+                    const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+                    f16x8 oh, ol;
 #pragma unroll
-            for (int u = 0; u < WR; ++u) {
-                u32 hi[4], lo[4];
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const float s0 = *reinterpret_cast<const float *>(gs + (w_ch0 + p) * 4);
-                    const float s1 = *reinterpret_cast<const float *>(gs + (w_ch0 + p + PAIR_GAP) * 4);
-                    const float t0 = (float)as_h2(qpair[u][p])[0] * s0, t1 = (float)as_h2(qpair[u][p])[1] * s1;
-                    const f16x2 h = pinned_h2(f16x2{(f16)t0, (f16)t1});
-                    hi[p] = as_u(h);
-                    lo[p] = as_u(f16x2{(f16)(t0 - (float)h[0]), (f16)(t1 - (float)h[1])});
+                    for (int j = 0; j < 8; ++j) {
+                        const f16 hv = (f16)x[j];
+                        oh[j] = hv;
+                        ol[j] = (f16)(x[j] - (float)hv);
+                    }
+                    const f16x8 qr = DH == 1 ? q0[DH == 1 ? ks : 0] : q_rows(h, ks);
+                    bt = VQ_MFMA(oh, qr, bt);
+                    bt = VQ_MFMA(ol, qr, bt);
                 }
-                *reinterpret_cast<uint4 *>(qimg + w_off + 4 * u * PK_QIMG_ROW) = uint4{hi[0], hi[1], hi[2], hi[3]};
-                *reinterpret_cast<uint4 *>(qimg + w_off + (RTP + 4 * u) * PK_QIMG_ROW) = uint4{lo[0], lo[1], lo[2], lo[3]};
-            }
-            // bias chain: the zeros as fp16 high parts, then their remainders, in every operand row
-            const char *zs = gs + RG::KMR + 128 * blk;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                const float4 x0 = *reinterpret_cast<const float4 *>(zs + 32 * ks);
-                const float4 x1 = *reinterpret_cast<const float4 *>(zs + 32 * ks + 16);
-                const float x[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
-                f16x8 oh, ol;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const f16 h = (f16)x[j];
-                    oh[j] = h;
-                    ol[j] = (f16)(x[j] - (float)h);
-                }
-                bt = VQ_MFMA(oh, q0[ks], bt);
-                bt = VQ_MFMA(ol, q0[ks], bt);
             }
         }
         // every register of a lane holds sum z q of the lane's column; the score accumulators carry 2^(EK - 24)
@@ -426,22 +465,27 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qB[ks] = as_h8(*reinterpret_cast<const uint4 *>(qimg + r_off + 16 * ks));
+        for (int h = 0; h < DH; ++h)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) qB[h][ks] = as_h8(*reinterpret_cast<const uint4 *>(qimg + h * IMG + r_off + 16 * ks));
     };
 
     // ---- one unit, first half: scores
     auto scores = [&](const Unit &cur, f32x4 (&S)[2]) VQ_INLINE_LAMBDA {
 #pragma unroll
         for (int T = 0; T < 2; ++T) {
-            f16x8 A[4];   // per k-step
-            if constexpr (BITS == 4) {
-                sub_unpack4(cur.kw[T][0], cur.kw[T][1], A[0], A[1]);
-                sub_unpack4(cur.kw[T][2], cur.kw[T][3], A[2], A[3]);
-            } else {   // word j holds k-steps 2j (codes 0-3 | 8-11) and 2j + 1 (codes 4-7 | 12-15)
-                sub_unpack2(cur.kw[T][0], cur.kw[T][1], A[0], A[1], A[2], A[3]);
-            }
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) S[T] = VQ_MFMA(A[ks], qB[ks], ks == 0 ? bias : S[T]);
+            for (int h = 0; h < DH; ++h) {
+                f16x8 A[4];   // per k-step
+                if constexpr (BITS == 4) {
+                    sub_unpack4(cur.kw[h][T][0], cur.kw[h][T][1], A[0], A[1]);
+                    sub_unpack4(cur.kw[h][T][2], cur.kw[h][T][3], A[2], A[3]);
+                } else {   // word j holds k-steps 2j (codes 0-3 | 8-11) and 2j + 1 (codes 4-7 | 12-15)
+                    sub_unpack2(cur.kw[h][T][0], cur.kw[h][T][1], A[0], A[1], A[2], A[3]);
+                }
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) S[T] = VQ_MFMA(A[ks], qB[h][ks], (h == 0 && ks == 0) ? bias : S[T]);
+            }
         }
     };
 
@@ -480,7 +524,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
             const float alpha = m_new == -INFINITY ? 1.f : exp2f(acc.m_run - m_new);   // 0 on the first unit
             // accumulators are [channel][column]: the factor is the lane's own
 #pragma unroll
-            for (int nt = 0; nt < 8; ++nt)
+            for (int nt = 0; nt < CL::NT; ++nt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) acc.O[nt][r] *= alpha;
 #pragma unroll
@@ -637,21 +681,25 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
 // tile sees; in the block of split 0 the last nparts - nsplit waves first run the fp16 tail, each
 // into a partial slot of its own.  With sync counters the block that finishes last for its tile
 // merges the nparts partials into the output.
-template <int BITS, typename M, int GV, int RTP, int WAVES = Ring<BITS, M, GV, RTP>::WAVES>
+// DH = 2: a head of 256 channels, worked as two halves of 128 in the first product (eight k-steps into the same
+// scores) and as sixteen value tiles in the second; GV counts the groups of the whole head.  Such a launch runs no
+// tail waves (the fp16 tail comes as a partial of its own from the vector kernel) and takes no k_new / v_new.
+template <int BITS, typename M, int GV, int RTP, int DH = 1, int WAVES = Ring<BITS, M, GV, RTP, DH>::WAVES>
 __global__ __launch_bounds__(64 * WAVES) __attribute__((amdgpu_waves_per_eu(WAVES / 4, WAVES / 4)))
 void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail_equiv, int nparts, int pq, int tiles,
                                int order, float *__restrict__ ws) {
-    using CL = Cols<GV, RTP>;
-    using RG = Ring<BITS, M, GV, RTP>;
+    using CL = Cols<GV, RTP, DH>;
+    using RG = Ring<BITS, M, GV, RTP, DH>;
+    constexpr int DD = MF_D * DH, QROW = DD + 8, PART = DD + 2;
     constexpr int PK_WAVES = RG::WAVES, PK_THREADS = RG::THREADS;
-    constexpr int EX_O = ex_o(PK_WAVES), EX_Z = ex_z(PK_WAVES), EX_M = ex_m(PK_WAVES);
+    constexpr int EX_O = ex_o(PK_WAVES) * DH, EX_Z = ex_z(PK_WAVES), EX_M = ex_m(PK_WAVES);
     // query rows of the block; constants: [0, 128) ones for 32 tokens in the scale / zero type, then zeros
-    __shared__ __align__(16) f16 s_qraw[8 * PK_QROW];
+    __shared__ __align__(16) f16 s_qraw[8 * QROW];
     __shared__ __align__(16) char s_const[512];
     // the waves' rings; after the units the same bytes are the exchange buffer
     // s_o[PK_WAVES][MF_ROWS][MF_D] of the cross-wave merge
     extern __shared__ __align__(16) char s_ring[];
-    float (*s_o)[MF_ROWS][MF_D] = reinterpret_cast<float (*)[MF_ROWS][MF_D]>(s_ring);
+    float (*s_o)[MF_ROWS][DD] = reinterpret_cast<float (*)[MF_ROWS][DD]>(s_ring);
     float (*s_z)[MF_ROWS][8] = reinterpret_cast<float (*)[MF_ROWS][8]>(s_ring + EX_O);
     float (*s_m)[MF_ROWS] = reinterpret_cast<float (*)[MF_ROWS]>(s_ring + EX_O + EX_Z);
     float (*s_l)[MF_ROWS] = reinterpret_cast<float (*)[MF_ROWS]>(s_ring + EX_O + EX_Z + EX_M);
@@ -687,8 +735,8 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int RT = tile.RT;
 
     const bool single_launch = a.sync_counters != nullptr;
-    stage_query<RTP, PK_THREADS>(a, tile, tid, s_qraw);
-    if (sp == 0 && a.k_new != nullptr && a.n_tail >= 1 && tid < 32) {
+    stage_query<RTP, PK_THREADS, DH>(a, tile, tid, s_qraw);
+    if (DH == 1 && sp == 0 && a.k_new != nullptr && a.n_tail >= 1 && tid < 32) {
         // the newest token's key and value rows become the last tail row: 16 pieces of 16 bytes each
         const int piece = tid & 15;
         const bool val = tid >= 16;
@@ -700,10 +748,12 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     __syncthreads();
     // the launch has nparts - nsplit tail slots (filled even when this sequence's tail is empty): the
     // last waves of split 0 run the tail first, each into a slot of its own, while the others stream
-    const int tail_waves = nparts - nsplit;
-    if (sp == 0 && wave >= PK_WAVES - tail_waves)
-        tail_wave(a, bh, tile, c, nsplit + wave - (PK_WAVES - tail_waves), nparts, ws, s_qraw, PK_QROW, lane,
-                  wave - (PK_WAVES - tail_waves), tail_waves, single_launch);
+    if constexpr (DH == 1) {
+        const int tail_waves = nparts - nsplit;
+        if (sp == 0 && wave >= PK_WAVES - tail_waves)
+            tail_wave(a, bh, tile, c, nsplit + wave - (PK_WAVES - tail_waves), nparts, ws, s_qraw, PK_QROW, lane,
+                      wave - (PK_WAVES - tail_waves), tail_waves, single_launch);
+    }
     // what the unit loop derives from the lane number is formed from here on, not ahead of the tail: the tail
     // needs its 168 registers to itself
     int lane_u = lane;
@@ -711,9 +761,9 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int n = lane_u & 15, blk = lane_u >> 4;
 
     using SB = Sub<BITS>;
-    PackedAcc acc;
+    PackedAcc<CL::NT> acc;
 #pragma unroll
-    for (int nt = 0; nt < 8; ++nt) acc.O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < CL::NT; ++nt) acc.O[nt] = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.Z = f32x4{0.f, 0.f, 0.f, 0.f};
     acc.m_run = -INFINITY;
     acc.thr = -INFINITY;
@@ -740,7 +790,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     const int64_t lane_first = tile.first(n % RTP < RT ? n % RTP : 0) - t_begin, edge_first = tile.first(RT - 1) - t_begin;
     const int lo_rel = (int)(lane_first < 0 ? 0 : lane_first > rel_cap ? rel_cap : lane_first);
     const int edge_rel = (int)(edge_first < 0 ? 0 : edge_first > rel_cap ? rel_cap : edge_first);
-    packed_units<BITS, M, GV, RTP>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lo_rel, edge_rel, lane_u, wave, acc, s_qraw, s_const,
+    packed_units<BITS, M, GV, RTP, DH>(a, bh, c, t_begin, n_units, lane_rel, full_rel, lo_rel, edge_rel, lane_u, wave, acc, s_qraw, s_const,
                                    s_ring, &s_next, order);
     __syncthreads();   // every wave has read its last slot
 
@@ -750,7 +800,7 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     if (n < RTP && blk == 0) s_m[wave][n] = acc.m_run;
     if (col_row < RT) {
 #pragma unroll
-        for (int nt = 0; nt < 8; ++nt) {
+        for (int nt = 0; nt < CL::NT; ++nt) {
             const int g = nt / CL::TPG;
             if (col_set == g % CL::GPP) {
 #pragma unroll
@@ -767,8 +817,8 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         }
     }
     __syncthreads();
-    for (int e = tid; e < RT * MF_D; e += PK_THREADS) {
-        const int row = e / MF_D, d = e % MF_D;
+    for (int e = tid; e < RT * DD; e += PK_THREADS) {
+        const int row = e / DD, d = e % DD;
         if (!tile.valid(row)) continue;
         float gm = -INFINITY;
 #pragma unroll
@@ -778,11 +828,11 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         for (int w = 0; w < PK_WAVES; ++w) {
             if (s_m[w][row] == -INFINITY) continue;   // a wave that had no unit, or saw nothing
             const float f = exp2f(s_m[w][row] - gm);
-            const int g = d / (MF_D / GV);
+            const int g = d / (DD / GV);
             num += (s_o[w][row][d] + s_z[w][row][g]) * f;
             den += s_l[w][row] * f;
         }
-        float *o = ws + (tile.row(row) * nparts + sp) * MF_PART;
+        float *o = ws + (tile.row(row) * nparts + sp) * PART;
         st_partial(o + 2 + d, num, single_launch);
         if (d == 0) { st_partial(o, gm * LN2, single_launch); st_partial(o + 1, den, single_launch); }
     }
@@ -802,34 +852,35 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
         s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     __syncthreads();
     if (s_ticket != nsplit - 1) return;
-    merge_rows(a, tile, nparts, ws, tid, PK_THREADS);
+    merge_rows<DH>(a, tile, nparts, ws, tid, PK_THREADS);
     if (tid == 0) __hip_atomic_store(a.sync_counters + by, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-template <typename M, int RTP>
+template <typename M, int RTP, int DH = 1>
 static void launch_mfma_packed(const vq_attend_args &a, const AttendPlan &p, float *ws, hipStream_t st) {
     const dim3 grid((unsigned)p.nsplit, (unsigned)(a.B * a.Hkv * p.tiles));
-    const int gv = (int)(MF_D / a.group);
+    const int gv = (int)(MF_D * DH / a.group);   // groups of the whole head
     // more than 64 KB of block-shared memory has to be allowed per kernel and device, once
 #define VQ_LAUNCH(BITS, GV)                                                                                            \
     do {                                                                                                               \
-        constexpr int ring_bytes = Ring<BITS, M, GV, RTP>::BYTES;                                                      \
+        using RGL = Ring<BITS, M, GV, RTP, DH>;                                                                        \
+        constexpr int ring_bytes = RGL::BYTES;                                                                         \
         static std::atomic<bool> allowed[64] = {};   /* set once per device; a second setter repeats the same call */ \
         int dev = 0;                                                                                                   \
         (void)hipGetDevice(&dev);                                                                                      \
         if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {                                   \
-            (void)hipFuncSetAttribute((const void *)attend_mfma_packed_kernel<BITS, M, GV, RTP>,                       \
+            (void)hipFuncSetAttribute((const void *)attend_mfma_packed_kernel<BITS, M, GV, RTP, DH>,                   \
                                       hipFuncAttributeMaxDynamicSharedMemorySize, ring_bytes);                         \
             if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);                             \
         }                                                                                                              \
-        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV, RTP>), grid, dim3(Ring<BITS, M, GV, RTP>::THREADS),  \
+        hipLaunchKernelGGL((attend_mfma_packed_kernel<BITS, M, GV, RTP, DH>), grid, dim3(RGL::THREADS),                \
                            ring_bytes, st, a, p.split_len,                                                             \
                            p.tail_equiv, p.nparts, p.pq, p.tiles, p.fixed_order, ws);                                  \
     } while (0)
     if (a.pack_bits == 4) {
-        if (gv == 1) VQ_LAUNCH(4, 1); else if (gv == 2) VQ_LAUNCH(4, 2); else VQ_LAUNCH(4, 4);
+        if (gv == DH) VQ_LAUNCH(4, DH); else if (gv == 2 * DH) VQ_LAUNCH(4, 2 * DH); else VQ_LAUNCH(4, 4 * DH);
     } else {
-        if (gv == 1) VQ_LAUNCH(2, 1); else if (gv == 2) VQ_LAUNCH(2, 2); else VQ_LAUNCH(2, 4);
+        if (gv == DH) VQ_LAUNCH(2, DH); else if (gv == 2 * DH) VQ_LAUNCH(2, 2 * DH); else VQ_LAUNCH(2, 4 * DH);
     }
 #undef VQ_LAUNCH
 }

@@ -82,7 +82,7 @@ bool rows_kernel_supported(const vq_attend_args &a) {
 // NR: the rows a tile can hold (1 .. AR_NR): the per-row loops of a launch whose tiles are smaller shrink with it
 template <int BITS, int NR>
 __global__ __launch_bounds__(256) void attend_rows_kernel(vq_attend_args a, int64_t split_len, int pq, int tiles,
-                                                          float *__restrict__ ws) {
+                                                          float *__restrict__ ws, int part0, int nparts) {
     constexpr int PER = 32 / BITS, CPL = ar_cpl(PER), SUBW = PER / CPL;   // SUBW lanes share a word
     constexpr uint32_t MASK = (1u << BITS) - 1u;
     __shared__ float s_q[NR][256];
@@ -133,7 +133,8 @@ __global__ __launch_bounds__(256) void attend_rows_kernel(vq_attend_args a, int6
             t_hi = vis[r] > t_hi ? vis[r] : t_hi;
         }
     }
-    int64_t t0 = (int64_t)sp * split_len, t1 = t0 + split_len;
+    // part0 >= 0: this launch covers the tail tokens only and writes partial part0 + sp of nparts
+    int64_t t0 = (part0 >= 0 ? a.n_packed : 0) + (int64_t)sp * split_len, t1 = t0 + split_len;
     if (t0 < t_lo) t0 = t_lo;
     if (t1 > t_hi) t1 = t_hi;
     // rows that see every token of [t0, t1) need no mask
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(256) void attend_rows_kernel(vq_attend_args a, int6
             for (int v = 0; v < 4; ++v)
                 if (s_part[v][r][0] != -INFINITY) x += s_part[v][r][c] * __expf(s_part[v][r][0] - gm);
         }
-        ws[(tile.row(r) * nsplit + sp) * (D + 2) + c] = x;
+        ws[(tile.row(r) * (part0 >= 0 ? nparts : nsplit) + (part0 >= 0 ? part0 : 0) + sp) * (D + 2) + c] = x;
     }
 }
 
@@ -354,11 +355,22 @@ static void launch_rows_bits(const vq_attend_args &a, const AttendPlan &p, dim3 
     const int64_t R = a.Hq / a.Hkv;
     const int rows = (int)((R > AR_NR ? AR_NR : R) * p.pq);   // rows of the largest tile
     switch (rows) {
-        case 1: hipLaunchKernelGGL((attend_rows_kernel<BITS, 1>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws); break;
-        case 2: hipLaunchKernelGGL((attend_rows_kernel<BITS, 2>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws); break;
-        case 3: hipLaunchKernelGGL((attend_rows_kernel<BITS, 3>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws); break;
-        default: hipLaunchKernelGGL((attend_rows_kernel<BITS, 4>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws); break;
+        case 1: hipLaunchKernelGGL((attend_rows_kernel<BITS, 1>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws, p.part0, p.nparts); break;
+        case 2: hipLaunchKernelGGL((attend_rows_kernel<BITS, 2>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws, p.part0, p.nparts); break;
+        case 3: hipLaunchKernelGGL((attend_rows_kernel<BITS, 3>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws, p.part0, p.nparts); break;
+        default: hipLaunchKernelGGL((attend_rows_kernel<BITS, 4>), grid, dim3(256), 0, st, a, p.split_len, p.pq, p.tiles, ws, p.part0, p.nparts); break;
     }
+}
+
+int launch_attend_rows_tail(const vq_attend_args &a, int part0, int nparts) {
+    AttendPlan p = {};
+    p.path = 3;
+    rows_tiling(a, p.pq, p.tiles);
+    p.nsplit = 1;
+    p.split_len = a.n_tail > 0 ? a.n_tail : 1;
+    p.nparts = nparts;
+    p.part0 = part0;
+    return launch_attend_rows(a, p);
 }
 
 int launch_attend_rows(const vq_attend_args &a, const AttendPlan &p) {
