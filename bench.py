@@ -53,7 +53,7 @@ def _parse():
     p.add_argument("--per-layer", action="store_true", help="with --only-kernel: one launch per layer")
     p.add_argument("--only", default=None, metavar="NAME",
                    help="run one side workload in a loop and print its timing (for rocprofv3): "
-                        "decode_2bit_B16, decode_2bit_B1, decode_d256_2bit_32k_B16, decode_3bit_32k_B16, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
+                        "decode_2bit_B16, decode_2bit_B1, decode_d256_2bit_32k_B16, decode_d256_4bit_32k_B16, decode_3bit_32k_B16, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
     p.add_argument("--copy-calib", action="store_true",
                    help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
@@ -284,13 +284,17 @@ def main() -> int:
     return 0
 
 
-_ROWS_CASES = {"decode_d256_2bit_32k_B16": (12, 4, 256, 2, 32), "decode_3bit_32k_B16": (32, 8, 128, 3, 32)}
+_ROWS_CASES = {"decode_d256_2bit_32k_B16": (12, 4, 256, 2, 32), "decode_d256_4bit_32k_B16": (12, 4, 256, 4, 64),
+               "decode_3bit_32k_B16": (32, 8, 128, 3, 32)}
+_ROWS_NOTES = {"decode_d256_2bit_32k_B16": "matrix-unit decode kernel, head of 256 channels (two launches: the fp16 tail comes from the vector kernel)",
+               "decode_d256_4bit_32k_B16": "matrix-unit decode kernel, head of 256 channels, four waves per CU",
+               "decode_3bit_32k_B16": "vector-unit kernel (attend_rows_kernel), four query rows of a kv head per block"}
 
 
 def _decode_rows_case(torch, dev, name):
-    """Shapes the matrix-unit decode kernel does not take (they run on ``attend_rows_kernel``): the head size of config
-    2's model (Falcon3-7B: 12 query / 4 kv heads, D = 256) at 2 bits, and 3-bit codes (ten to a word) at the headline's
-    head shape; batch 16, 32768 packed tokens plus the fp16 residual."""
+    """Decode outside the headline's head shape: the head size of config 2's model (Falcon3-7B: 12 query / 4 kv heads,
+    D = 256) at 2 and 4 bits, on the matrix-unit kernel's 256-channel form, and 3-bit codes (ten to a word) at the
+    headline's head shape, on the vector kernel; batch 16, 32768 packed tokens plus the fp16 residual."""
     from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
     hq, hkv, d, bits, g = _ROWS_CASES[name]
     cfg = KVCacheConfig(method="kivi", head_dim=d, bit_width_inlier=bits, kivi_group_size=g, residual_length=128,
@@ -526,14 +530,14 @@ def _extras(torch, K, dev):
         "ms": round(ms2, 5), "ms_per_layer": round(ms2 / NL2, 5), "GBps": round(nbytes2 / ms2 / 1e6, 1),
         "frac_hbm": round(nbytes2 / ms2 / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes2}
     del layers2, stack2, q2
-    # shapes the matrix-unit decode kernel does not take: the vector kernel that shares a kv head's bytes among its query heads
+    # decode outside the headline's head shape: heads of 256 channels, 3-bit codes
     for name in _ROWS_CASES:
         cv, fnv, nb = _decode_rows_case(torch, dev, name)
         for _ in range(2):
             fnv()
         msv = _side_ms(fnv, 5, torch)
         ex[name] = {"ms": round(msv, 4), "GBps": round(nb / msv / 1e6, 1), "frac_hbm": round(nb / msv / 1e6 / HBM_PEAK_GBS, 4),
-                    "bytes": nb, "note": "vector-unit kernel (attend_rows_kernel), four query rows of a kv head per block"}
+                    "bytes": nb, "note": _ROWS_NOTES[name]}
         del cv, fnv
     # config 1: Llama-3-8B layer, one sequence, 8192 tokens as 2-bit group-32 codes plus a 128-token fp16 tail
     c1, fn1, nbytes1 = _decode_cfg1_case(torch, dev)
