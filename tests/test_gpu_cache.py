@@ -90,6 +90,49 @@ def test_trim_equals_model_and_requantises():
     assert np.array_equal(host(ko), mk) and np.array_equal(host(vo), mv)
 
 
+@pytest.mark.parametrize("bits,g", [(2, 32), (4, 64), (3, 32)])
+def test_decode_at_head_size_256_through_the_cache_and_the_layer_stack(bits, g):
+    """Head size 256 (configuration 2's own model: 12 query / 4 kv heads): a memory-bound cache decodes through the
+    matrix-unit kernel's 256-channel form (2 and 4 bits) or the vector kernel (3 bits) over steps that cross a flush,
+    against the oracle; the layer-stacked cache gives the per-layer results under ``fixed_order``."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    B, Hq, Hkv, D, R, NL = 2, 12, 4, 256, 64, 2
+    cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=bits, kivi_group_size=g, residual_length=R,
+                        fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=1280)
+    solo = [KVCacheFactory.create(cfg) for _ in range(NL)]
+    stack = LayerStackedKIVICache(cfg, NL)
+    n0 = 960 if bits == 3 else 1000
+    ks = [outlier_kv((B, Hkv, n0 + 80, D), seed=31 * l + bits) for l in range(NL)]
+    rng = np.random.default_rng(5)
+    scale = 1 / math.sqrt(D)
+    for l in range(NL):
+        for c in (solo[l], stack[l]):
+            c.update_and_fetch(to_dev(ks[l][0][:, :, :n0]), to_dev(ks[l][1][:, :, :n0]))
+    levels = (1 << bits) - 1
+    for t in range(n0, n0 + 80):
+        q = rng.standard_normal((NL, B, Hq, 1, D)).astype(np.float16)
+        for l in range(NL):
+            for c in (solo[l], stack[l]):
+                c.update_and_fetch(to_dev(ks[l][0][:, :, t:t + 1]), to_dev(ks[l][1][:, :, t:t + 1]))
+        if t % 9 and t < n0 + 76:
+            continue
+        outs = [solo[l].fused_sdpa(to_dev(q[l]), scale, fixed_order=True) for l in range(NL)]
+        all_out = stack.fused_sdpa_all(to_dev(q), scale, fixed_order=True)
+        for l in range(NL):
+            nq = solo[l]._n_quantized
+            assert nq == ok.quantization_boundary(t + 1, R, g) and stack[l]._n_quantized == nq
+            k, v = ks[l]
+            kq = ok.group_quant_codes(k[:, :, :nq], -2, g, levels)
+            vq = ok.group_quant_codes(v[:, :, :nq], -1, g, levels)
+            ref = oa.kivi_attend(q[l], kq[0], kq[1].astype(np.float16), kq[2].astype(np.float16), vq[0], vq[1].astype(np.float16),
+                                 vq[2].astype(np.float16), g, k[:, :, nq:t + 1], v[:, :, nq:t + 1], scale)
+            err = float(np.max(np.abs(host(outs[l]).astype(np.float32) - ref)))
+            assert err < 2e-3, (t, l, err)
+            # the stacked launch may cut the context differently (its batch axis is NL times as long): values, not bits
+            assert float((all_out[l].float() - outs[l].float()).abs().max()) < 1e-3, (t, l)
+
+
 @pytest.mark.parametrize("memory_bound", [False, True])
 @pytest.mark.parametrize("bits,g,meta", [(2, 32, "float16"), (4, 64, "float16"), (4, 32, "float32")])
 def test_fused_sdpa_over_packed_prefix(memory_bound, bits, g, meta):
