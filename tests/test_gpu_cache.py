@@ -519,6 +519,39 @@ def test_sink_protected_cache_with_prefill_sized_query_blocks(bits, g):
         assert err < 2e-3, (w, err)
 
 
+@pytest.mark.parametrize("D,bits", [(64, 4), (256, 2), (128, 3)])
+def test_sink_protected_cache_on_the_other_decode_kernels(D, bits):
+    """Protected rows where the attention kernel is the vector one (head size 64, 3-bit codes) or the 256-channel form of
+    the matrix-unit one: the patch pass works from the partials, whichever kernel wrote them."""
+    require_gpu()
+    rng = np.random.default_rng(D + bits)
+    B, Hq, H, R, n = 2, 8, 2, 64, 420 if bits != 3 else 480
+    k = rng.standard_normal((B, H, n, D)).astype(np.float16)
+    v = rng.standard_normal((B, H, n, D)).astype(np.float16)
+    for p, f in ((7, 11), (130, 9), (131, 13)):
+        k[:, :, p] *= f
+    cfg = KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=32, residual_length=R,
+                        n_sink_tokens=3, fused_sdpa=True, fused_sdpa_memory_bound=True, kivi_meta_dtype="float32")
+    c = KVCacheFactory.create(cfg)
+    m = ok.SinkCacheModel(bits, 32, R, 3)
+    c.update_and_fetch(to_dev(k[:, :, :320]), to_dev(v[:, :, :320]))
+    m.update_and_fetch(k[:, :, :320], v[:, :, :320])
+    for t in range(320, n):
+        c.update_and_fetch(to_dev(k[:, :, t:t + 1]), to_dev(v[:, :, t:t + 1]))
+        m.update_and_fetch(k[:, :, t:t + 1], v[:, :, t:t + 1])
+    assert c._n_quantized == m.n_quantized and any(c._side_pos[b] for b in range(B))
+    km, vm = m.keys[:, :, : m.offset], m.values[:, :, : m.offset]
+    scale = 1 / math.sqrt(D)
+    for Sq in (1, 3):
+        q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float16)
+        row = km[0, 0, m.sink_positions_for(0)[0]].astype(np.float32)
+        q[0, 0, -1] += (row / np.linalg.norm(row) * 5).astype(np.float16)
+        got = host(c.fused_sdpa(to_dev(q), scale, causal=True)).astype(np.float32)
+        ref = oa.sdpa(q, km, vm, scale, causal=True)
+        err = float(np.max(np.abs(got - ref)))
+        assert err < 2e-3, (Sq, err)
+
+
 def test_prefill_tile_scratch_is_given_back_by_every_kind_of_decode_step():
     """The tile scratch of a memory-bound prefill lives only until decoding begins: a single-token append, a
     single-query attend with per-sequence ``lengths`` and the layer-stacked launch all return ``nbytes`` to the
