@@ -64,6 +64,26 @@ __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&
         for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
+// The same when the parameters of the exact division are not at hand: `slow_params(mn, sc)` fetches them, and only
+// a wave that redoes its codes calls it (every lane of the wave does: it may move data between lanes).
+template <typename F>
+__device__ __forceinline__ void quant_codes8_lazy(const float (&v)[8], const float (&rs)[8], const float (&nb)[8], float tie,
+                                                  float levels, bool redo, float (&q)[8], F &&slow_params) {
+    float far = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
+        const float r = rintf(q0);
+        far = fmaxf(far, fabsf(q0 - r));
+        q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels);
+    }
+    if (__any(redo | (far >= tie))) {
+        float mn[8], sc[8];
+        slow_params(mn, sc);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
+    }
+}
 // The same with a level count per code (channels of different bit widths in one row).
 __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
                                              const float (&rs)[8], const float (&nb)[8], float tie,
@@ -317,14 +337,17 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
     Raw8<T> v[NP];   // NP passes of RPP rows cover the group
     typename Raw8<T>::Acc acc;
     Raw8<T>::init(acc);
+    // every row is requested before the first is used
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
-        if (rl < group && s < S) {
-            v[p].load(xb + routed(s) * D + 8 * o);
-            v[p].fold(acc);
-        }
+        if (rl < group && s < S) v[p].load(xb + routed(s) * D + 8 * o);
+    }
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        int rl = p * RPP + r;
+        if (rl < group && s0 + rl < S) v[p].fold(acc);
     }
     float mn[8], mx[8];
     Raw8<T>::result(acc, mn, mx);
@@ -541,6 +564,14 @@ __global__ __launch_bounds__(256) void kivi_value_tile_kernel(
 template <int CTRL> __device__ __forceinline__ float lane_move(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
 }
+// lane k's value in every lane of its quad
+template <int K> __device__ __forceinline__ float quad_bcast(float x) { return lane_move<K * 0x55>(x); }
+__device__ __forceinline__ float pick4(int i, float a, float b, float c, float d) { return (i & 2) ? ((i & 1) ? d : c) : ((i & 1) ? b : a); }
+template <typename M> __device__ __forceinline__ void store_meta2(M *p, float a, float b);
+template <> __device__ __forceinline__ void store_meta2<float>(float *p, float a, float b) { *reinterpret_cast<float2 *>(p) = make_float2(a, b); }
+template <> __device__ __forceinline__ void store_meta2<f16>(f16 *p, float a, float b) {
+    *reinterpret_cast<uint32_t *>(p) = __builtin_bit_cast(uint32_t, f16x2{(f16)a, (f16)b});
+}
 __device__ __forceinline__ float bare_min(float a, float b) { float d; asm("v_min_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b)); return d; }
 __device__ __forceinline__ float bare_max(float a, float b) { float d; asm("v_max_f32 %0, %1, %2" : "=v"(d) : "v"(a), "v"(b)); return d; }
 // minimum and maximum over the GL lanes (4, 8 or 16, aligned) that hold a channel group
@@ -567,9 +598,7 @@ __global__ __launch_bounds__(256) void kivi_value_roundtrip_kernel(const T *__re
     const LevelDiv ld = level_div(levels);
     Raw8<T> v[PER];
 #pragma unroll
-    for (int i = 0; i < PER; ++i)
-        if (t0 + i < S) v[i].load(xb + (int64_t)i * D);
-        else v[i] = v[0];
+    for (int i = 0; i < PER; ++i) v[i].load(xb + (t0 + i < S ? (int64_t)i * D : 0));   // past the end: the first row again
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
         float mn, mx;
@@ -587,12 +616,40 @@ __global__ __launch_bounds__(256) void kivi_value_roundtrip_kernel(const T *__re
     }
 }
 
+// The GL lanes of a channel group hold the same (token, group) extrema after the fold: with GL = 4 or 8 each of them
+// works out the scale, reciprocal and offset of 8 / GL of every eight tokens and the group passes them round.
+// value of the lane four lanes up (lanes 0-3, 8-11 of a row of 16) or down (lanes 4-7, 12-15)
+__device__ __forceinline__ float other_quad(float x) {
+    int t = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x104, 0xF, 0x5, false);   // row_shl:4 into quads 0, 2
+    t = __builtin_amdgcn_update_dpp(t, __builtin_bit_cast(int, x), 0x114, 0xF, 0xA, false);       // row_shr:4 into quads 1, 3
+    return __builtin_bit_cast(float, t);
+}
+// all[t], t = 0..7: element t % TP of lane t / TP of the group (TP = 8 / GL)
+template <int GL> __device__ __forceinline__ void group_gather8(const float (&own)[8 / GL], bool upper_quad, float (&all)[8]) {
+    if constexpr (GL == 4) {
+        all[0] = quad_bcast<0>(own[0]); all[1] = quad_bcast<0>(own[1]); all[2] = quad_bcast<1>(own[0]); all[3] = quad_bcast<1>(own[1]);
+        all[4] = quad_bcast<2>(own[0]); all[5] = quad_bcast<2>(own[1]); all[6] = quad_bcast<3>(own[0]); all[7] = quad_bcast<3>(own[1]);
+    } else {
+        const float other = other_quad(own[0]);
+        const float lo = upper_quad ? other : own[0], hi = upper_quad ? own[0] : other;   // lanes 0-3 / 4-7 of the group
+        all[0] = quad_bcast<0>(lo); all[1] = quad_bcast<1>(lo); all[2] = quad_bcast<2>(lo); all[3] = quad_bcast<3>(lo);
+        all[4] = quad_bcast<0>(hi); all[5] = quad_bcast<1>(hi); all[6] = quad_bcast<2>(hi); all[7] = quad_bcast<3>(hi);
+    }
+}
+// element TP * j + e of eight values, j the lane's place in its group
+template <int GL> __device__ __forceinline__ float group_pick8(int j, int e, const float (&v)[8]) {
+    if constexpr (GL == 4) return pick4(j, v[e], v[2 + e], v[4 + e], v[6 + e]);
+    else return (j & 4) ? pick4(j, v[4], v[5], v[6], v[7]) : pick4(j, v[0], v[1], v[2], v[3]);
+}
+
 template <typename T, typename M, int BITS, int GL>
 __device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T *__restrict__ x, int64_t S,
                                                      int64_t x_stride_bh, float levels, float eps,
                                                      uint32_t *__restrict__ packed, M *__restrict__ scale,
                                                      M *__restrict__ zero, int64_t cap_tokens, int64_t dst_tok0) {
     constexpr int D = 128, PER = 32 / BITS, HALF = PER / 2, GV = 16 / GL;
+    constexpr bool SHARE = GL <= 8;
+    constexpr int TP = SHARE ? 8 / GL : 1;
     const int tid = threadIdx.x, o = tid & 15;
     const int64_t t0 = ((int64_t)bx * VP_STRETCHES + (tid >> 4)) * PER;   // the stretch's first token
     if (t0 >= S) return;                                                  // S is a multiple of PER: whole rows of 16 lanes leave
@@ -601,22 +658,12 @@ __device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T
     Raw8<T> v[PER];
 #pragma unroll
     for (int i = 0; i < PER; ++i) v[i].load(xb + (int64_t)i * D);
-    float lo[8], hi[8], scv[PER], mnv[PER];
+    float lo[8], hi[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) { lo[c] = 0.f; hi[c] = 0.f; }
-#pragma unroll
-    for (int i = 0; i < PER; ++i) {
-        float mn, mx;
-        v[i].span(mn, mx);
-        group_span<GL>(mn, mx);
-        const float sc = group_scale(mn, mx, ld, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
-        scv[i] = sc;
-        mnv[i] = mn;
-        float x8[8], q[8], mn8[8], sc8[8], rs8[8], nb8[8];
-#pragma unroll
-        for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; }
-        v[i].floats(x8);
-        quant_codes8(x8, mn8, sc8, rs8, nb8, tl, levels, !(rs < 1e30f), q);
+    const int64_t tok = dst_tok0 + t0;
+    const int64_t mi = (bh * GV + o / GL) * cap_tokens + tok;
+    auto code_fields = [&](int i, const float (&q)[8]) __attribute__((always_inline)) {
         // code of token i at bits [BITS * i, BITS * (i + 1)): two exact float sums of 16 bits each
         const float w = (float)(1u << (BITS * (i % HALF)));
 #pragma unroll
@@ -624,24 +671,92 @@ __device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T
             if (i < HALF) lo[c] = __builtin_fmaf(q[c], w, lo[c]);
             else hi[c] = __builtin_fmaf(q[c], w, hi[c]);
         }
+    };
+    if constexpr (SHARE) {
+        const int j = o & (GL - 1);
+        const bool upper_quad = (o & 4) != 0;
+#pragma unroll
+        for (int i0 = 0; i0 < PER; i0 += 8) {
+            float mnb[8], mxb[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                v[i0 + i].span(mnb[i], mxb[i]);
+                group_span<GL>(mnb[i], mxb[i]);
+            }
+            float own_sc[TP], own_rs[TP], own_nb[TP], own_mn[TP], tie = 0.5f;
+            bool redo = false;   // the lane's own tokens: any lane's flag redoes the whole wave
+#pragma unroll
+            for (int e = 0; e < TP; ++e) {
+                own_mn[e] = group_pick8<GL>(j, e, mnb);
+                own_sc[e] = group_scale(own_mn[e], group_pick8<GL>(j, e, mxb), ld, eps);
+                own_rs[e] = fast_rcp(own_sc[e]);
+                own_nb[e] = -own_mn[e] * own_rs[e];
+                tie = fminf(tie, tie_limit(levels, own_nb[e]));
+                redo |= !(own_rs[e] < 1e30f);
+            }
+            // one limit for the eight tokens, the tightest: a few more rows take the division
+            tie = fminf(tie, lane_move<0xB1>(tie));
+            tie = fminf(tie, lane_move<0x4E>(tie));
+            if constexpr (GL == 8) tie = fminf(tie, lane_move<0x141>(tie));
+            float rsb[8], nbb[8];
+            group_gather8<GL>(own_rs, upper_quad, rsb);
+            group_gather8<GL>(own_nb, upper_quad, nbb);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                float x8[8], q[8], rs8[8], nb8[8];
+#pragma unroll
+                for (int c = 0; c < 8; ++c) { rs8[c] = rsb[i]; nb8[c] = nbb[i]; }
+                v[i0 + i].floats(x8);
+                quant_codes8_lazy(x8, rs8, nb8, tie, levels, redo, q, [&](float (&m8)[8], float (&s8)[8]) {
+                    float scb[8];
+                    group_gather8<GL>(own_sc, upper_quad, scb);
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) { m8[c] = mnb[i]; s8[c] = scb[i]; }
+                });
+                code_fields(i0 + i, q);
+            }
+            // every lane its own tokens' scale and zero
+            if constexpr (TP == 2) {
+                store_meta2<M>(scale + mi + i0 + 2 * j, own_sc[0], own_sc[1]);
+                store_meta2<M>(zero + mi + i0 + 2 * j, own_mn[0], own_mn[1]);
+            } else {
+                store_meta<M>(scale + mi + i0 + j, own_sc[0]);
+                store_meta<M>(zero + mi + i0 + j, own_mn[0]);
+            }
+        }
+    } else {
+        float scv[PER], mnv[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            float mn, mx;
+            v[i].span(mn, mx);
+            group_span<GL>(mn, mx);
+            const float sc = group_scale(mn, mx, ld, eps), rs = fast_rcp(sc), nb = -mn * rs, tl = tie_limit(levels, nb);
+            scv[i] = sc;
+            mnv[i] = mn;
+            float x8[8], q[8], mn8[8], sc8[8], rs8[8], nb8[8];
+#pragma unroll
+            for (int c = 0; c < 8; ++c) { mn8[c] = mn; sc8[c] = sc; rs8[c] = rs; nb8[c] = nb; }
+            v[i].floats(x8);
+            quant_codes8(x8, mn8, sc8, rs8, nb8, tl, levels, !(rs < 1e30f), q);
+            code_fields(i, q);
+        }
+        if ((o & (GL - 1)) == 0) {   // the first lane of a channel group writes its PER scales and zeros
+#pragma unroll
+            for (int i = 0; i < PER; i += 8) {
+                const float s8[8] = {scv[i], scv[i + 1], scv[i + 2], scv[i + 3], scv[i + 4], scv[i + 5], scv[i + 6], scv[i + 7]};
+                const float z8[8] = {mnv[i], mnv[i + 1], mnv[i + 2], mnv[i + 3], mnv[i + 4], mnv[i + 5], mnv[i + 6], mnv[i + 7]};
+                store_meta8<M>(scale + mi + i, s8);
+                store_meta8<M>(zero + mi + i, z8);
+            }
+        }
     }
-    const int64_t tok = dst_tok0 + t0;
     uint32_t wd[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) wd[c] = (uint32_t)lo[c] | ((uint32_t)hi[c] << 16);
     uint4 *wp = reinterpret_cast<uint4 *>(packed + (bh * (cap_tokens / PER) + tok / PER) * D + 8 * o);
     wp[0] = make_uint4(wd[0], wd[1], wd[2], wd[3]);
     wp[1] = make_uint4(wd[4], wd[5], wd[6], wd[7]);
-    if ((o & (GL - 1)) == 0) {   // the first lane of a channel group writes its PER scales and zeros
-        const int64_t mi = (bh * GV + o / GL) * cap_tokens + tok;
-#pragma unroll
-        for (int i = 0; i < PER; i += 8) {
-            const float s8[8] = {scv[i], scv[i + 1], scv[i + 2], scv[i + 3], scv[i + 4], scv[i + 5], scv[i + 6], scv[i + 7]};
-            const float z8[8] = {mnv[i], mnv[i + 1], mnv[i + 2], mnv[i + 3], mnv[i + 4], mnv[i + 5], mnv[i + 6], mnv[i + 7]};
-            store_meta8<M>(scale + mi + i, s8);
-            store_meta8<M>(zero + mi + i, z8);
-        }
-    }
 }
 
 template <typename T, typename M, int BITS, int GL>
@@ -715,12 +830,20 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
     Raw8<T> v[TPL];
     typename Raw8<T>::Acc acc;
     Raw8<T>::init(acc);
+    // a whole group (all but the last of a ragged sequence): every row is requested before the first is used
+    const bool whole = s0 + G <= S;   // the same for the wave
+    if (whole) {
 #pragma unroll
-    for (int i = 0; i < TPL; ++i)
-        if (r0 + i < S) {
-            v[i].load(xb + (int64_t)i * D);
-            v[i].fold(acc);
-        }
+        for (int i = 0; i < TPL; ++i) v[i].load(xb + (int64_t)i * D);
+#pragma unroll
+        for (int i = 0; i < TPL; ++i) v[i].fold(acc);
+    } else {   // a row past the end stands in as the group's first row, which changes no minimum or maximum
+        const T *x0 = x + bh * x_stride_bh + s0 * D + 8 * o;
+#pragma unroll
+        for (int i = 0; i < TPL; ++i) v[i].load(r0 + i < S ? xb + (int64_t)i * D : x0);
+#pragma unroll
+        for (int i = 0; i < TPL; ++i) v[i].fold(acc);
+    }
     QuadFold<T>::run(acc);
     float mn[8], mx[8], sc[8], rs[8], nb[8];
     Raw8<T>::result(acc, mn, mx);
@@ -734,56 +857,98 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
     float lv[8];
     bool redo = false;
     float tie_all = 0.5f;   // one limit for the lane's 8 channels, the tightest: a few more rows take the division
+    float own_sc[2] = {0.f, 0.f};
+    if constexpr (MIXED) {
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        const bool hi = MIXED && (((c < 4 ? hi8.x : hi8.y) >> (8 * (c & 3))) & 0xFFu) != 0u;
-        const LevelDiv d = hi ? ldh : ld;
-        lv[c] = d.levels;
-        sc[c] = group_scale(mn[c], mx[c], d, eps);
-        rs[c] = fast_rcp(sc[c]);
-        nb[c] = -mn[c] * rs[c];
-        tie_all = fminf(tie_all, tie_limit(lv[c], nb[c]));
-        redo |= !(rs[c] < 1e30f);
+        for (int c = 0; c < 8; ++c) {
+            const bool hi = (((c < 4 ? hi8.x : hi8.y) >> (8 * (c & 3))) & 0xFFu) != 0u;
+            const LevelDiv d = hi ? ldh : ld;
+            lv[c] = d.levels;
+            sc[c] = group_scale(mn[c], mx[c], d, eps);
+            rs[c] = fast_rcp(sc[c]);
+            nb[c] = -mn[c] * rs[c];
+            tie_all = fminf(tie_all, tie_limit(lv[c], nb[c]));
+            redo |= !(rs[c] < 1e30f);
+        }
+    } else {
+        // The four lanes of a quad hold the same eight minima and maxima: lane tq works out the parameters of
+        // channels 2 tq and 2 tq + 1 only and the quad passes them round (a quarter of the divisions; the same
+        // values, so the same codes).  `redo` stays the lane's own: any lane's flag redoes the whole wave.
+        float own_rs[2], own_nb[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const float m = pick4(tq, mn[e], mn[2 + e], mn[4 + e], mn[6 + e]), x = pick4(tq, mx[e], mx[2 + e], mx[4 + e], mx[6 + e]);
+            own_sc[e] = group_scale(m, x, ld, eps);
+            own_rs[e] = fast_rcp(own_sc[e]);
+            own_nb[e] = -m * own_rs[e];
+            tie_all = fminf(tie_all, tie_limit(levels, own_nb[e]));
+            redo |= !(own_rs[e] < 1e30f);
+        }
+        tie_all = fminf(tie_all, lane_move<0xB1>(tie_all));
+        tie_all = fminf(tie_all, lane_move<0x4E>(tie_all));
+#define VQ_QUAD_GATHER(DST, SRC) \
+        DST[0] = quad_bcast<0>(SRC[0]); DST[1] = quad_bcast<0>(SRC[1]); DST[2] = quad_bcast<1>(SRC[0]); DST[3] = quad_bcast<1>(SRC[1]); \
+        DST[4] = quad_bcast<2>(SRC[0]); DST[5] = quad_bcast<2>(SRC[1]); DST[6] = quad_bcast<3>(SRC[0]); DST[7] = quad_bcast<3>(SRC[1])
+        VQ_QUAD_GATHER(rs, own_rs);
+        VQ_QUAD_GATHER(nb, own_nb);
+        if (MODE == 0) { VQ_QUAD_GATHER(sc, own_sc); }
     }
-    if (MODE == 1 && tq == 0) {
+    if (MODE == 1) {
         const int64_t gdst = dst_tok0 / G + gk, gcap = (cap_tokens + G - 1) / G;
-        store_meta8<M>(scale + (bh * gcap + gdst) * D + 8 * o, sc);
-        store_meta8<M>(zero + (bh * gcap + gdst) * D + 8 * o, mn);
-    }
-#pragma unroll
-    for (int i = 0; i < TPL; ++i) {
-        const int64_t srow = r0 + i;
-        const bool valid = srow < S;
-        float x8[8], q[8];
-        if (valid) v[i].floats(x8);
-        else {   // keep the arithmetic defined; the lane's results are not stored
-#pragma unroll
-            for (int c = 0; c < 8; ++c) x8[c] = mn[c];
-        }
-        if constexpr (MIXED) quant_codes8(x8, mn, sc, rs, nb, tie_all, lv, redo, q);
-        else quant_codes8(x8, mn, sc, rs, nb, tie_all, levels, redo, q);
-        if (MODE == 0) {
-            if (valid) {
-                float y[8];
-#pragma unroll
-                for (int c = 0; c < 8; ++c) y[c] = recon(q[c], sc[c], mn[c]);
-                store8<T>(out + (bh * S + srow) * D + 8 * o, y);
+        if constexpr (MIXED) {
+            if (tq == 0) {
+                store_meta8<M>(scale + (bh * gcap + gdst) * D + 8 * o, sc);
+                store_meta8<M>(zero + (bh * gcap + gdst) * D + 8 * o, mn);
             }
-        } else {
-            uint32_t *row_words = packed + (bh * cap_tokens + dst_tok0 + (valid ? srow : 0)) * W;
-            if (bits == 8) {
-                if (valid) *reinterpret_cast<uint2 *>(row_words + 2 * o) = bytes8(q);
-            } else if (bits == 4) {
-                const uint32_t w = field8(q, 4);
-                if (valid) row_words[o] = w;
-            } else {   // 2 bits: chunk o + 1 sits four lanes up
-                const uint32_t f = field8(q, 2);
-                const uint32_t up = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f, 0x104, 0xF, 0xF, true);   // row_shl:4
-                if (valid && (o & 1) == 0) row_words[o >> 1] = f | (up << 16);
-            }
+        } else {   // every lane its own two channels
+            store_meta2<M>(scale + (bh * gcap + gdst) * D + 8 * o + 2 * tq, own_sc[0], own_sc[1]);
+            store_meta2<M>(zero + (bh * gcap + gdst) * D + 8 * o + 2 * tq, pick4(tq, mn[0], mn[2], mn[4], mn[6]),
+                           pick4(tq, mn[1], mn[3], mn[5], mn[7]));
         }
     }
+    auto rows = [&](auto whole_group) __attribute__((always_inline)) {
+        constexpr bool WHOLE = decltype(whole_group)::value;
+#pragma unroll
+        for (int i = 0; i < TPL; ++i) {
+            const int64_t srow = r0 + i;
+            const bool valid = WHOLE || srow < S;
+            float x8[8], q[8];
+            v[i].floats(x8);   // a row past the end holds the group's first row; its results are not stored
+            if constexpr (MIXED) quant_codes8(x8, mn, sc, rs, nb, tie_all, lv, redo, q);
+            else if (MODE == 0) quant_codes8(x8, mn, sc, rs, nb, tie_all, levels, redo, q);
+            else
+                quant_codes8_lazy(x8, rs, nb, tie_all, levels, redo, q, [&](float (&m8)[8], float (&s8)[8]) {
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) m8[c] = mn[c];
+                    VQ_QUAD_GATHER(s8, own_sc);
+                });
+            if (MODE == 0) {
+                if (valid) {
+                    float y[8];
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) y[c] = recon(q[c], sc[c], mn[c]);
+                    store8<T>(out + (bh * S + srow) * D + 8 * o, y);
+                }
+            } else {
+                uint32_t *row_words = packed + (bh * cap_tokens + dst_tok0 + (valid ? srow : 0)) * W;
+                if (bits == 8) {
+                    if (valid) *reinterpret_cast<uint2 *>(row_words + 2 * o) = bytes8(q);
+                } else if (bits == 4) {
+                    const uint32_t w = field8(q, 4);
+                    if (valid) row_words[o] = w;
+                } else {   // 2 bits: chunk o + 1 sits four lanes up
+                    const uint32_t f = field8(q, 2);
+                    const uint32_t up = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)f, 0x104, 0xF, 0xF, true);   // row_shl:4
+                    if (valid && (o & 1) == 0) row_words[o >> 1] = f | (up << 16);
+                }
+            }
+        }
+    };
+    if (whole) rows(std::true_type{});
+    else rows(std::false_type{});
 }
+
+#undef VQ_QUAD_GATHER
 
 template <typename T, typename M, int MODE, int TPL>
 __global__ __launch_bounds__(64 * KQ_WAVES) void kivi_key_quad_kernel(
