@@ -27,23 +27,26 @@ __device__ __forceinline__ float quant_code(float v, float mn, float sc, float l
 // q0 = fma(v, rs, nb) lies within 3e-7 * q + 6e-8 * |nb| of the correctly rounded quotient
 // q = (v - mn) / sc, so rint(q0) == rint(q) unless q0 is that close to a tie k + 0.5:
 // `tie_lo` = 0.5 - (5e-7 * (levels + 1) + 2e-7 * |nb|) is the distance from rint(q0) beyond
-// which a lane counts as undecided.  A wave in which any lane is undecided (or `redo`: a scale
-// too small for rcp) redoes its eight codes with the true division.  Bit-identical to quant_code;
+// which a lane counts as undecided.  A wave in which any lane is undecided about its code i (or `redo`:
+// a scale too small for rcp) redoes code i with the true division -- with 16-bit inputs exact ties are
+// common enough that one wave in eight has one among its 512 quotients.  Bit-identical to quant_code;
 // the codes come back as floats.
 __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
                                              const float (&rs)[8], const float (&nb)[8], const float (&tie_lo)[8],
                                              float levels, bool redo, float (&q)[8]) {
-    bool close = redo;
+    bool close = redo, near[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
         const float r = rintf(q0);
-        close |= fabsf(q0 - r) >= tie_lo[i];
+        near[i] = fabsf(q0 - r) >= tie_lo[i];
+        close |= near[i];
         q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels);   // clamp; a NaN becomes 0 as with fmaxf / fminf
     }
     if (__any(close)) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
+        for (int i = 0; i < 8; ++i)
+            if (__any(redo | near[i])) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
 // The same with one limit for all eight codes: the largest distance from a whole number is compared once
@@ -51,17 +54,19 @@ __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&
 __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
                                              const float (&rs)[8], const float (&nb)[8], float tie, float levels,
                                              bool redo, float (&q)[8]) {
-    float far = 0.f;
+    float far = 0.f, dist[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
         const float r = rintf(q0);
-        far = fmaxf(far, fabsf(q0 - r));
+        dist[i] = fabsf(q0 - r);
+        far = fmaxf(far, dist[i]);
         q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels);
     }
-    if (__any(redo | (far >= tie))) {
+    if (__any(redo | (far >= tie))) {   // common with 16-bit inputs (exact ties): only the codes some lane is unsure of
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
+        for (int i = 0; i < 8; ++i)
+            if (__any(redo | (dist[i] >= tie))) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
 // The same when the parameters of the exact division are not at hand: `slow_params(mn, sc)` fetches them, and only
@@ -69,36 +74,40 @@ __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&
 template <typename F>
 __device__ __forceinline__ void quant_codes8_lazy(const float (&v)[8], const float (&rs)[8], const float (&nb)[8], float tie,
                                                   float levels, bool redo, float (&q)[8], F &&slow_params) {
-    float far = 0.f;
+    float far = 0.f, dist[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
         const float r = rintf(q0);
-        far = fmaxf(far, fabsf(q0 - r));
+        dist[i] = fabsf(q0 - r);
+        far = fmaxf(far, dist[i]);
         q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels);
     }
     if (__any(redo | (far >= tie))) {
         float mn[8], sc[8];
         slow_params(mn, sc);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels);
+        for (int i = 0; i < 8; ++i)
+            if (__any(redo | (dist[i] >= tie))) q[i] = quant_code(v[i], mn[i], sc[i], levels);
     }
 }
 // The same with a level count per code (channels of different bit widths in one row).
 __device__ __forceinline__ void quant_codes8(const float (&v)[8], const float (&mn)[8], const float (&sc)[8],
                                              const float (&rs)[8], const float (&nb)[8], float tie,
                                              const float (&levels)[8], bool redo, float (&q)[8]) {
-    float far = 0.f;
+    float far = 0.f, dist[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
         const float q0 = __builtin_fmaf(v[i], rs[i], nb[i]);
         const float r = rintf(q0);
-        far = fmaxf(far, fabsf(q0 - r));
+        dist[i] = fabsf(q0 - r);
+        far = fmaxf(far, dist[i]);
         q[i] = __builtin_amdgcn_fmed3f(r, 0.0f, levels[i]);
     }
     if (__any(redo | (far >= tie))) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) q[i] = quant_code(v[i], mn[i], sc[i], levels[i]);
+        for (int i = 0; i < 8; ++i)
+            if (__any(redo | (dist[i] >= tie))) q[i] = quant_code(v[i], mn[i], sc[i], levels[i]);
     }
 }
 __device__ __forceinline__ float tie_limit(float levels, float nb) {
@@ -337,13 +346,17 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
     Raw8<T> v[NP];   // NP passes of RPP rows cover the group
     typename Raw8<T>::Acc acc;
     Raw8<T>::init(acc);
-    // every row is requested before the first is used
+    // every row is requested before the first is used (and, under a routing, every row number before the first row)
+    int64_t src[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
         int64_t s = s0 + rl;
-        if (rl < group && s < S) v[p].load(xb + routed(s) * D + 8 * o);
+        src[p] = rl < group && s < S ? routed(s) : -1;
     }
+#pragma unroll
+    for (int p = 0; p < NP; ++p)
+        if (src[p] >= 0) v[p].load(xb + src[p] * D + 8 * o);
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
         int rl = p * RPP + r;
@@ -405,7 +418,7 @@ __device__ __forceinline__ void kivi_key_tile_body(int bx, int64_t bh,
                 float y[8];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) y[i] = recon(q[i], sc[i], mn[i]);
-                store8<T>(rows != nullptr ? out + bh * x_stride_bh + routed(s) * D + 8 * o : out + (bh * S + s) * D + 8 * o, y);
+                store8<T>(rows != nullptr ? out + bh * x_stride_bh + src[p] * D + 8 * o : out + (bh * S + s) * D + 8 * o, y);
             }
         } else {
             uint32_t *row = packed + (bh * cap_tokens + dst_tok0 + (valid ? s : 0)) * W;

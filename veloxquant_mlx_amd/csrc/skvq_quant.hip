@@ -43,16 +43,18 @@ __device__ __forceinline__ float sk_code(float x, float lo, float sc, float rs, 
 // rounding does; inside it q0 is within 1.5e-7 * (levels + 1) of the true quotient, less than the
 // 1e-6 * (levels + 2) by which `tie` stays below one half.
 __device__ __forceinline__ void sk_codes8(const float *x, float (&q)[8], float lo, float sc, float rs, float levels, float tie) {
-    bool close = false;
+    float far = 0.f, dist[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const float q0 = __fmul_rn(__fsub_rn(x[j], lo), rs);
         q[j] = rintf(q0);
-        close |= fabsf(q0 - q[j]) >= tie;
+        dist[j] = fabsf(q0 - q[j]);
+        far = fmaxf(far, dist[j]);
     }
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(close) != 0, 0)) {
+    if (__builtin_amdgcn_ballot_w64(far >= tie) != 0) {   // exact ties are common with 16-bit inputs: only the codes some lane is unsure of
 #pragma unroll
-        for (int j = 0; j < 8; ++j) q[j] = rintf(__fdiv_rn(__fsub_rn(x[j], lo), sc));
+        for (int j = 0; j < 8; ++j)
+            if (__builtin_amdgcn_ballot_w64(dist[j] >= tie) != 0) q[j] = rintf(__fdiv_rn(__fsub_rn(x[j], lo), sc));
     }
 #pragma unroll
     for (int j = 0; j < 8; ++j) q[j] = __builtin_amdgcn_fmed3f(q[j], 0.f, levels);   // a NaN becomes 0, as with fmaxf / fminf
