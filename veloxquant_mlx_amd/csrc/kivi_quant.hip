@@ -1313,6 +1313,112 @@ __global__ __launch_bounds__(ZR_THREADS) void zip_route_kernel(const float *__re
     }
 }
 
+// The same order for rows of at most ZR_THREADS * KPT norms, with every norm of the row in a register (position
+// j * ZR_THREADS + tid): one read of the norms, the histogram's digit found by all threads at once (a suffix sum over
+// the 256 bins instead of one thread walking them), and the two ordered parts written from per-wave ballots -- chunk j
+// of 256 positions, wave w, lane l is the order of the positions, so "rows before" and "equal rows at or after" are
+// sums over whole (chunk, wave) cells plus bits of the lane's own ballot.
+template <int KPT>
+__global__ __launch_bounds__(ZR_THREADS) void zip_route_regs_kernel(const float *__restrict__ norms, int S, int n_hi,
+                                                                    int32_t *__restrict__ order) {
+    constexpr int NW = ZR_THREADS / 64, CELLS = KPT * NW;
+    static_assert(CELLS <= ZR_THREADS, "one thread per (chunk, wave) cell");
+    __shared__ unsigned s_hist[256];
+    __shared__ unsigned s_wsum[NW];
+    __shared__ unsigned s_prefix, s_pmask;
+    __shared__ int s_want;
+    __shared__ int s_cell[CELLS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t *key = reinterpret_cast<const uint32_t *>(norms) + (int64_t)blockIdx.x * S;
+    int32_t *dst = order + (int64_t)blockIdx.x * S;
+    uint32_t k[KPT];
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) k[j] = j * ZR_THREADS + tid < S ? key[j * ZR_THREADS + tid] : 0u;
+    if (tid == 0) { s_prefix = 0; s_pmask = 0; s_want = n_hi; }
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        s_hist[tid] = 0;
+        __syncthreads();
+        const unsigned prefix = s_prefix, pmask = s_pmask;
+        const int want = s_want;
+#pragma unroll
+        for (int j = 0; j < KPT; ++j)
+            if (j * ZR_THREADS + tid < S && (k[j] & pmask) == prefix) atomicAdd(&s_hist[(k[j] >> shift) & 255u], 1u);
+        __syncthreads();
+        // rows in bins above bin `tid`: a suffix sum over the 256 bins
+        const unsigned h = s_hist[tid];
+        unsigned suf = h;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const unsigned up = __shfl_down(suf, off);
+            if (lane + off < 64) suf += up;
+        }
+        if (lane == 0) s_wsum[wave] = suf;
+        __syncthreads();
+        unsigned above = suf - h;
+        for (int w = wave + 1; w < NW; ++w) above += s_wsum[w];
+        // the digit in which the want-th largest of the rows that match so far lies (bin 0 if none above holds it)
+        if ((int)above < want && (tid == 0 || (int)(above + h) >= want)) {
+            s_want = want - (int)above;
+            s_prefix = prefix | ((unsigned)tid << shift);
+            s_pmask = pmask | (255u << shift);
+        }
+        __syncthreads();
+    }
+    const uint32_t v = s_prefix;     // the threshold norm
+    const int take_eq = s_want;      // rows equal to it that belong to the block, the latest ones
+    const unsigned long long lt = (1ull << lane) - 1ull;   // the lanes before this one
+    // exclusive prefix sum of s_cell over the cells in (chunk, wave) order, in place; returns the total
+    auto scan_cells = [&]() __attribute__((always_inline)) {
+        int x = tid < CELLS ? s_cell[tid] : 0;
+        const int own = x;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int dn = __shfl_up(x, off);
+            if (lane >= off) x += dn;
+        }
+        if (lane == 63) s_wsum[wave] = (unsigned)x;
+        __syncthreads();
+        int base = 0, total = 0;
+        for (int w = 0; w < NW; ++w) { if (w < wave) base += (int)s_wsum[w]; total += (int)s_wsum[w]; }
+        if (tid < CELLS) s_cell[tid] = base + x - own;
+        __syncthreads();
+        return total;
+    };
+    // rows equal to the threshold, per cell
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const unsigned long long b = __ballot(j * ZR_THREADS + tid < S && k[j] == v);
+        if (lane == 0) s_cell[j * NW + wave] = __popcll(b);
+    }
+    __syncthreads();
+    const int eq_total = scan_cells();
+    // a row equal to the threshold is taken when at most take_eq such rows lie at or after it
+    unsigned sel_bits = 0;   // bit j: the lane's row of chunk j belongs to the high block
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const bool in = j * ZR_THREADS + tid < S, eq = in && k[j] == v;
+        const unsigned long long b = __ballot(eq);
+        const int at_or_after = eq_total - s_cell[j * NW + wave] - __popcll(b & lt);
+        if (in && (k[j] > v || (eq && at_or_after <= take_eq))) sel_bits |= 1u << j;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const unsigned long long b = __ballot((sel_bits >> j) & 1u);
+        if (lane == 0) s_cell[j * NW + wave] = __popcll(b);
+    }
+    __syncthreads();
+    scan_cells();
+#pragma unroll
+    for (int j = 0; j < KPT; ++j) {
+        const int i = j * ZR_THREADS + tid;
+        const bool sel = (sel_bits >> j) & 1u;
+        const unsigned long long b = __ballot(sel);
+        const int before = s_cell[j * NW + wave] + __popcll(b & lt);   // rows of the high block at earlier positions
+        if (i < S) dst[sel ? (S - n_hi) + before : i - before] = i;
+    }
+}
+
 static inline bool pow2(int64_t v) { return v > 0 && (v & (v - 1)) == 0; }
 static inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
@@ -1505,7 +1611,14 @@ extern "C" int vq_zip_route(const float *norms, int64_t BH, int64_t S, int64_t n
     VQ_REQUIRE(S < ((int64_t)1 << 31) && BH <= 0x7fffffff, VQ_ERR_INVALID, "%s: positions must fit 31 bits", fn);
     if (BH == 0) return VQ_OK;
     VQ_REQUIRE(norms && order, VQ_ERR_INVALID, "%s: null pointer", fn);
-    hipLaunchKernelGGL(zip_route_kernel, dim3((unsigned)BH), dim3(ZR_THREADS), 0, (hipStream_t)stream, norms, S, n_hi, order);
+    if (S <= 8 * ZR_THREADS)
+        hipLaunchKernelGGL(zip_route_regs_kernel<8>, dim3((unsigned)BH), dim3(ZR_THREADS), 0, (hipStream_t)stream, norms, (int)S,
+                           (int)n_hi, order);
+    else if (S <= 32 * ZR_THREADS)
+        hipLaunchKernelGGL(zip_route_regs_kernel<32>, dim3((unsigned)BH), dim3(ZR_THREADS), 0, (hipStream_t)stream, norms, (int)S,
+                           (int)n_hi, order);
+    else
+        hipLaunchKernelGGL(zip_route_kernel, dim3((unsigned)BH), dim3(ZR_THREADS), 0, (hipStream_t)stream, norms, S, n_hi, order);
     VQ_HIP_CHECK_LAUNCH(fn);
     return VQ_OK;
 }
