@@ -88,6 +88,16 @@ int vq_kivi_quant_dequant_grouplevels(const void *x, void *out, int dtype, int64
 int vq_channel_moments(const void *x, int dtype, int64_t N, int64_t S, int64_t D, int64_t x_stride_n, double *partial,
                        int chunks, void *stream);
 
+/* variance[n * D + c] = max(sq / S - (sum / S)^2, 0), float32, from the partial sums vq_channel_moments wrote
+ * (chunks added in order, double arithmetic): the rest of the same mx.var (veloxquant_mlx/quantizers/kitty.py:44-67,
+ * veloxquant_mlx/cache/kitty_cache.py:96-104) in one launch. */
+int vq_channel_variance(const double *partial, int64_t N, int chunks, int64_t D, int64_t S, float *variance, void *stream);
+
+/* mask[n * D + c] = 1 where channel c is among the n_hi channels of largest variance[n][:], 0 elsewhere: the rank of
+ * a channel is its place in a stable ascending sort of -variance (equal variances: the lower channel first, a NaN
+ * after every number), which is the double argsort of veloxquant_mlx/quantizers/kitty.py:112-135.  D <= 1024. */
+int vq_channel_hi_mask(const float *variance, int64_t N, int64_t D, int64_t n_hi, uint8_t *mask, void *stream);
+
 /* out[r] = L2 norm of row r of x [n_rows, D], float32 arithmetic (head_dim 64 / 128 / 256).  The salience
  * signal of ZipCacheKVCache (mx.linalg.norm over the channels of the float32 copy,
  * veloxquant_mlx/cache/zipcache_cache.py:176-180) without materialising that copy. */

@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     for name in _declared():
         assert hasattr(lib, name), name
-    assert lib.vq_abi_version() == 15
+    assert lib.vq_abi_version() == 16
 
 
 def test_attend_args_struct_matches_header_field_order():

@@ -144,6 +144,32 @@ def test_channel_variance_in_one_pass(dtype, N, S, D):
     np.testing.assert_allclose(got, want, rtol=2e-6, atol=1e-9)
 
 
+@pytest.mark.gpu
+def test_hi_mask_kernel_equals_the_double_stable_argsort():
+    """``vq_channel_hi_mask`` against the definition it replaces (argsort of -variance, stable, then the rank of
+    every channel, kitty.py:112-135) on rows with many exact ties, zeros of both signs, infinities and NaNs, for
+    every n_hi at a small width and a few at the others; and the oracle's mask on the rows without NaN."""
+    require_gpu()
+    g = torch.Generator().manual_seed(9)
+    for D in (1, 7, 64, 128, 200, 1024):
+        v = torch.randint(0, 6, (6, D), generator=g).float() * 0.25
+        v[1] = torch.rand(D, generator=g)
+        v[2, ::3] = -0.0
+        if D > 4:
+            v[3, 1] = float("nan"); v[3, D - 2] = float("nan"); v[4, 2] = float("inf"); v[4, 0] = float("inf")
+        for n_hi in (range(0, D + 1) if D <= 7 else (1, 2, D // 4, D // 2, D - 1, D)):
+            order = torch.argsort(-v, dim=-1, stable=True)
+            want = torch.argsort(order, dim=-1, stable=True) < n_hi
+            got = K.channel_hi_mask(v.to("cuda:0"), n_hi).cpu()
+            assert torch.equal(got, want), (D, n_hi)
+    v = torch.rand((5, 128), generator=g)
+    v[:, 10:20] = v[:, 30:40]
+    for frac in (0.125, 0.25, 0.5):
+        assert np.array_equal(host(qk.hi_mask_from_variance_batched(v.to("cuda:0"), frac)), okt.hi_mask_from_variance(v.numpy(), frac))
+    with pytest.raises(ValueError):
+        K.channel_hi_mask(torch.zeros((2, 2048), device="cuda:0"), 3)
+
+
 @pytest.mark.parametrize("D", [64, 48])       # 64: one-pass variance kernel; 48: torch.var of the float32 copy
 def test_near_tie_and_tied_variances_rank_alike_on_both_paths(D):
     """Channels that hold +a and -a on alternate tokens: mean 0 and variance a^2 in every arithmetic (sums of

@@ -89,6 +89,8 @@ _SIGNATURES = {
     "vq_row_norms": (i32, [vp, i32, i64, i64, vp, vp]),
     "vq_kivi_quant_dequant_mixed": (i32, [vp, vp, i32, i64, i64, i64, i32, i32, i32, vp, f32, vp]),
     "vq_channel_moments": (i32, [vp, i32, i64, i64, i64, i64, vp, i32, vp]),
+    "vq_channel_variance": (i32, [vp, i64, i32, i64, i64, vp, vp]),
+    "vq_channel_hi_mask": (i32, [vp, i64, i64, i64, vp, vp]),
     "vq_kivi_quant_dequant_grouplevels": (i32, [vp, vp, i32, i64, i64, i64, i32, vp, f32, vp]),
     "vq_kivi_quant_dequant_rows": (i32, [vp, vp, i32, i64, i64, i64, i64, vp, i64, i32, i32, f32, vp]),
     "vq_kivi_quant_pack_kv": (i32, [vp, vp, i32, i64, i64, i64, i64, i32, i32, f32, i32, i32, vp, vp, vp, vp, vp, vp, i32, i64, i64, vp]),

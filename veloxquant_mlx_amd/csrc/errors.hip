@@ -25,7 +25,7 @@ int fail(int code, const char *fmt, ...) {
 
 }  // namespace vq
 
-extern "C" int vq_abi_version(void) { return 15; }
+extern "C" int vq_abi_version(void) { return 16; }
 
 extern "C" int vq_last_error(char *buf, size_t n) {
     size_t len = strlen(vq::g_err);

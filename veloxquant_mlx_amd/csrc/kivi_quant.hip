@@ -1012,7 +1012,19 @@ __global__ __launch_bounds__(256) void channel_moments_kernel(const T *__restric
 #pragma unroll
     for (int c = 0; c < 8; ++c) { sum[c] = 0.0; sq[c] = 0.0; }
     const T *xb = x + n * x_stride_n + 8 * o;
-    for (int64_t t = t_begin + r; t < t_end; t += RPP) {
+    // four rows are requested before the first is added (the sums keep their order: row by row)
+    int64_t t = t_begin + r;
+    for (; t + 3 * RPP < t_end; t += 4 * RPP) {
+        float v[4][8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load8<T>(xb + (t + i * RPP) * D, v[i]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int c = 0; c < 8; ++c) { sum[c] += (double)v[i][c]; sq[c] += (double)v[i][c] * (double)v[i][c]; }
+        }
+    }
+    for (; t < t_end; t += RPP) {
         float v[8];
         load8<T>(xb + t * D, v);
 #pragma unroll
@@ -1035,6 +1047,45 @@ __global__ __launch_bounds__(256) void channel_moments_kernel(const T *__restric
         const double total = ((s_part[0][which][ch] + s_part[1][which][ch]) + s_part[2][which][ch]) + s_part[3][which][ch];
         partial[((n * gridDim.x + blockIdx.x) * 2 + which) * D + ch] = total;
     }
+}
+
+// variance[n][c] = max(sq / S - (sum / S)^2, 0) from the partial sums of channel_moments_kernel, the chunks added
+// in order, double arithmetic with one rounding per operation, the result rounded to float32.
+__global__ __launch_bounds__(256) void channel_variance_kernel(const double *__restrict__ partial, int64_t N, int chunks, int D,
+                                                               double n_tokens, float *__restrict__ variance) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= N * D) return;
+    const int64_t n = e / D;
+    const int c = (int)(e - n * D);
+    double sum = 0.0, sq = 0.0;
+    for (int k = 0; k < chunks; ++k) {
+        sum += partial[((n * chunks + k) * 2 + 0) * D + c];
+        sq += partial[((n * chunks + k) * 2 + 1) * D + c];
+    }
+    const double mean = sum / n_tokens;
+    const double var = sq / n_tokens - mean * mean;
+    variance[e] = (float)(var > 0.0 ? var : (var == var ? 0.0 : var));   // clamp at zero; a NaN stays a NaN
+}
+
+// mask[n][c] = 1 where channel c is among the n_hi largest of variance[n][:]: the rank of a channel is the number
+// of channels that come before it in a stable ascending sort of -variance (equal values: the lower channel first;
+// a NaN after every number), one block of D threads per row.
+__global__ void channel_hi_mask_kernel(const float *__restrict__ variance, int D, int n_hi, uint8_t *__restrict__ mask) {
+    extern __shared__ uint32_t s_key[];
+    const int c = threadIdx.x;
+    const int64_t n = blockIdx.x;
+    // -variance as an unsigned key that orders like the sort: -0 and +0 alike, NaN last
+    const float t = -variance[n * D + c] + 0.0f;
+    const uint32_t b = __float_as_uint(t);
+    const uint32_t key = t != t ? 0xFFFFFFFFu : ((b & 0x80000000u) ? ~b : (b | 0x80000000u));
+    s_key[c] = key;
+    __syncthreads();
+    int before = 0;
+    for (int j = 0; j < D; ++j) {
+        const uint32_t kj = s_key[j];
+        before += (kj < key) || (kj == key && j < c);
+    }
+    mask[n * D + c] = before < n_hi ? 1 : 0;
 }
 
 template <typename T, typename M, int BITS, int TPL>
@@ -1749,6 +1800,31 @@ extern "C" int vq_channel_moments(const void *x, int dtype, int64_t N, int64_t S
         else if (D == 128) hipLaunchKernelGGL((channel_moments_kernel<T, 16>), grid, dim3(256), 0, st, (const T *)x, S, x_stride_n, partial, per);
         else hipLaunchKernelGGL((channel_moments_kernel<T, 32>), grid, dim3(256), 0, st, (const T *)x, S, x_stride_n, partial, per);
     });
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_channel_variance(const double *partial, int64_t N, int chunks, int64_t D, int64_t S, float *variance,
+                                   void *stream) {
+    const char *fn = "vq_channel_variance";
+    VQ_REQUIRE(N >= 0 && D >= 1 && D <= 65536 && chunks >= 1 && S >= 1, VQ_ERR_INVALID, "%s: bad dimensions", fn);
+    if (N == 0) return VQ_OK;
+    VQ_REQUIRE(partial && variance, VQ_ERR_INVALID, "%s: null pointer", fn);
+    hipLaunchKernelGGL(channel_variance_kernel, dim3((unsigned)cdiv(N * D, 256)), dim3(256), 0, (hipStream_t)stream, partial, N, chunks,
+                       (int)D, (double)S, variance);
+    VQ_HIP_CHECK_LAUNCH(fn);
+    return VQ_OK;
+}
+
+extern "C" int vq_channel_hi_mask(const float *variance, int64_t N, int64_t D, int64_t n_hi, uint8_t *mask, void *stream) {
+    const char *fn = "vq_channel_hi_mask";
+    VQ_REQUIRE(N >= 0 && N <= 0x7fffffff && D >= 1, VQ_ERR_INVALID, "%s: bad dimensions", fn);
+    VQ_REQUIRE(D <= 1024, VQ_ERR_UNSUPPORTED, "%s: at most 1024 channels, got %lld", fn, (long long)D);
+    VQ_REQUIRE(n_hi >= 0 && n_hi <= D, VQ_ERR_INVALID, "%s: n_hi=%lld outside [0, %lld]", fn, (long long)n_hi, (long long)D);
+    if (N == 0) return VQ_OK;
+    VQ_REQUIRE(variance && mask, VQ_ERR_INVALID, "%s: null pointer", fn);
+    hipLaunchKernelGGL(channel_hi_mask_kernel, dim3((unsigned)N), dim3((unsigned)D), (size_t)D * sizeof(uint32_t), (hipStream_t)stream,
+                       variance, (int)D, (int)n_hi, mask);
     VQ_HIP_CHECK_LAUNCH(fn);
     return VQ_OK;
 }

@@ -184,10 +184,26 @@ def channel_variance(x: torch.Tensor) -> torch.Tensor:
         return torch.full((N, D), float("nan"), dtype=torch.float32, device=x.device)
     chunks = max(1, min(64, S // 256))
     partial = torch.empty((N, chunks, 2, D), dtype=torch.float64, device=x.device)
-    _lib.check(_lib.load().vq_channel_moments(x.data_ptr(), tag, N, S, D, S * D, partial.data_ptr(), chunks, _stream(x)))
-    total = partial.sum(dim=1)
-    mean = total[:, 0] / S
-    return torch.clamp(total[:, 1] / S - mean * mean, min=0.0).to(torch.float32)
+    var = torch.empty((N, D), dtype=torch.float32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.vq_channel_moments(x.data_ptr(), tag, N, S, D, S * D, partial.data_ptr(), chunks, _stream(x)))
+    _lib.check(lib.vq_channel_variance(partial.data_ptr(), N, chunks, D, S, var.data_ptr(), _stream(x)))
+    return var
+
+
+def channel_hi_mask(variance: torch.Tensor, n_hi: int) -> torch.Tensor:
+    """``[N, D]`` float32 variances -> bool mask of every row's ``n_hi`` channels of largest variance, equal variances
+    to the lower channel, a NaN after every number (the double stable argsort of
+    veloxquant_mlx/quantizers/kitty.py:112-135), one launch.  D <= 1024."""
+    name = "channel_hi_mask"
+    _need_gpu(name, variance)
+    if variance.ndim != 2 or variance.dtype != torch.float32:
+        raise ValueError(f"{name}: variance must be float32 [N, D], got {tuple(variance.shape)} {variance.dtype}")
+    variance = variance.contiguous()
+    N, D = variance.shape
+    mask = torch.empty((N, D), dtype=torch.bool, device=variance.device)
+    _lib.check(_lib.load().vq_channel_hi_mask(variance.data_ptr(), N, D, int(n_hi), mask.data_ptr(), _stream(variance)))
+    return mask
 
 
 def kivi_group_quant_dequant_mixed(x: torch.Tensor, hi_mask: torch.Tensor, group_size: int, levels_lo: int, levels_hi: int,
@@ -1150,7 +1166,7 @@ def flash_prefill_attend(q, k, v, scale) -> torch.Tensor:
 
 
 __all__ = [
-    "hip_available", "release_tile_scratch", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant", "kivi_prefill_tiles", "prefill_tiles_empty",
+    "hip_available", "release_tile_scratch", "kivi_group_quant_dequant", "kivi_group_quant_dequant_rows", "kivi_group_quant_dequant_mixed", "kivi_group_quant_dequant_grouplevels", "channel_variance", "channel_hi_mask", "row_norms", "zip_route", "kivi_quant_pack", "kivi_quant_pack_kv", "kivi_quant_codes", "kivi_dequant", "kivi_prefill_tiles", "prefill_tiles_empty",
     "scalar_decode_once", "pack_indices", "unpack_indices", "turboquant_bit_pack", "turboquant_bit_unpack",
     "vecinfer_quantize_metal", "vecinfer_dequant_metal", "vecinfer_quantize_hip", "vecinfer_dequant_hip",
     "vecinfer_encode_decode_metal", "vecinfer_encode_decode_simple_metal", "metal_fused_sdpa", "vecinfer_fused_sdpa",

@@ -27,6 +27,8 @@ def hi_mask_from_variance_batched(variance: torch.Tensor, hi_fraction: float) ->
     ties to the lower channel index (kitty.py:112-135)."""
     d = variance.shape[-1]
     n_hi = max(1, int(d * hi_fraction))
+    if variance.is_cuda and variance.ndim == 2 and variance.dtype == torch.float32 and d <= 1024:
+        return K.channel_hi_mask(variance, n_hi)
     order = torch.argsort(-variance, dim=-1, stable=True)
     rank = torch.argsort(order, dim=-1, stable=True)
     return rank < n_hi
