@@ -175,6 +175,9 @@ def _pack_exact(x_np, axis, b, g, meta_dtype, v_layout="channel"):
     if axis == -1 and v_layout == "token":
         sm, zm = sm.swapaxes(-1, -2), zm.swapaxes(-1, -2)
     np.testing.assert_array_equal(host(back), ok.group_dequant(codes, sm, zm, axis, g))
+    for dt in (torch.float16, torch.bfloat16):   # the same values rounded once to the output type
+        low = K.kivi_dequant(p, s, z, axis, g, b, S, D, v_layout=v_layout, out_dtype=dt)
+        assert torch.equal(low, back.to(dt))
 
 
 @pytest.mark.parametrize("axis", [-2, -1])

@@ -1226,6 +1226,61 @@ __global__ void kivi_dequant_kernel(const uint32_t *__restrict__ packed, const M
     }
 }
 
+// The same reconstruction, eight consecutive channels of a token per thread, for D % 8 == 0, group % 8 == 0 and
+// 2, 4 or 8 bits: a thread's codes are one piece of one or two words (channel-packed) or the same field of eight
+// consecutive words (token-packed), its scale / zero eight consecutive values (keys) or one (values), and the eight
+// results leave as one store.  PB = log2(bits).
+template <typename O, typename M, int PB>
+__global__ __launch_bounds__(256) void kivi_dequant8_kernel(const uint32_t *__restrict__ packed, const M *__restrict__ scale,
+                                                            const M *__restrict__ zero, int64_t n_rows, int64_t S, int D, int axis,
+                                                            int group, int layout, int64_t cap_tokens, int64_t src_tok0,
+                                                            O *__restrict__ out) {
+    constexpr int BITS = 1 << PB, PER = 32 / BITS;
+    constexpr uint32_t MASK = (1u << BITS) - 1u;
+    const int pieces = D / 8;
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= n_rows * pieces) return;
+    const int64_t row = e / pieces;                 // bh * S + s
+    const int d0 = 8 * (int)(e - row * pieces);
+    const int64_t bh = row / S, t = src_tok0 + (row - bh * S);
+    float c[8];
+    if (layout == 0) {
+        const uint32_t *w = packed + (bh * cap_tokens + t) * ((D + PER - 1) / PER);
+        if constexpr (PER >= 8) {
+            const uint32_t x = w[d0 / PER] >> ((d0 % PER) * BITS);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) c[i] = (float)((x >> (i * BITS)) & MASK);
+        } else {   // 8 bits: two words
+            const uint2 x = *reinterpret_cast<const uint2 *>(w + d0 / PER);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { c[i] = (float)((x.x >> (8 * i)) & 255u); c[4 + i] = (float)((x.y >> (8 * i)) & 255u); }
+        }
+    } else {
+        const uint32_t *w = packed + (bh * (cap_tokens / PER) + t / PER) * D + d0;
+        const uint4 a = *reinterpret_cast<const uint4 *>(w), b = *reinterpret_cast<const uint4 *>(w + 4);
+        const int sh = (int)(t % PER) * BITS;
+        const uint32_t x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int i = 0; i < 8; ++i) c[i] = (float)((x[i] >> sh) & MASK);
+    }
+    float y[8];
+    if (axis == VQ_AXIS_TOKEN) {
+        const int64_t mi = (bh * ((cap_tokens + group - 1) / group) + t / group) * D + d0;
+        float sc[8], zr[8];
+        load8<M>(scale + mi, sc);
+        load8<M>(zero + mi, zr);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = recon(c[i], sc[i], zr[i]);
+    } else {
+        const int64_t GV = D / group;
+        const int64_t mi = layout == 0 ? (bh * cap_tokens + t) * GV + d0 / group : (bh * GV + d0 / group) * cap_tokens + t;
+        const float sc = load_meta<M>(scale + mi), zr = load_meta<M>(zero + mi);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) y[i] = recon(c[i], sc, zr);
+    }
+    store8<O>(out + row * D + d0, y);
+}
+
 __global__ void pack_words_kernel(const uint8_t *__restrict__ idx, int64_t rows, int64_t D, int bits,
                                   uint32_t *__restrict__ words) {
     const int per = 32 / bits;
@@ -1888,6 +1943,23 @@ extern "C" int vq_kivi_dequant(const void *packed, const void *scale, const void
     if (BH * S * D == 0) return VQ_OK;
     VQ_REQUIRE(packed && scale && zero && out, VQ_ERR_INVALID, "%s: null pointer", fn);
     hipStream_t st = (hipStream_t)stream;
+    const int pb = pack_bits == 2 ? 1 : pack_bits == 4 ? 2 : pack_bits == 8 ? 3 : -1;
+    if (pb > 0 && D % 8 == 0 && D % group == 0 && group % 8 == 0 && D <= (1 << 20) && aligned16(packed) && aligned16(scale) &&
+        aligned16(zero) && aligned16(out) && BH * S * (D / 8) < ((int64_t)1 << 40)) {
+        // eight channels a thread (channel-packed words hold 4, 8 or 16 codes: D % 8 == 0 keeps a thread inside its words)
+        const int64_t n_rows = BH * S;
+        const dim3 g8((unsigned)cdiv(n_rows * (D / 8), 256));
+#define VQ_DQ8(O, M, PB) hipLaunchKernelGGL((kivi_dequant8_kernel<O, M, PB>), g8, dim3(256), 0, st, (const uint32_t *)packed,        \
+                                            (const M *)scale, (const M *)zero, n_rows, S, (int)D, axis, group, tokpacked ? 1 : 0,   \
+                                            cap_tokens, src_tok0, (O *)out)
+        VQ_DISPATCH_FLOAT(out_dtype, O, {
+            if (meta_dtype == VQ_F32) { if (pb == 1) VQ_DQ8(O, float, 1); else if (pb == 2) VQ_DQ8(O, float, 2); else VQ_DQ8(O, float, 3); }
+            else { if (pb == 1) VQ_DQ8(O, f16, 1); else if (pb == 2) VQ_DQ8(O, f16, 2); else VQ_DQ8(O, f16, 3); }
+        });
+#undef VQ_DQ8
+        VQ_HIP_CHECK_LAUNCH(fn);
+        return VQ_OK;
+    }
     dim3 grid(grid_for(BH * S * D, 256));
     VQ_DISPATCH_FLOAT(out_dtype, O, {
         if (meta_dtype == VQ_F32)
