@@ -108,7 +108,7 @@ def test_routing_kernel_equals_the_stable_sorts():
     block, every block size from 1 to S - 1 at the small lengths."""
     require_gpu()
     g = torch.Generator().manual_seed(4)
-    for S in (2, 7, 255, 256, 257, 1000, 8192):
+    for S in (2, 7, 255, 256, 257, 1000, 2048, 2049, 5000, 8192, 8193):   # 8 and 32 norms a thread in registers, then the walk over memory
         norms = torch.randint(0, 9, (5, S), generator=g).float() * 0.37
         norms[1] = torch.rand(S, generator=g)
         if S > 10:
