@@ -26,6 +26,8 @@
 // packed-cache attention combines them.  Two kernels: lut_attend_u8_kernel for byte indices
 // with the same, compile-time number of sub-vectors on both sides (tables laid out so that one
 // LDS read returns the entries of all RB rows), and lut_attend_any_kernel for everything else.
+#include <atomic>
+
 #include "attend.hpp"
 #include "vecinfer.hpp"
 
@@ -591,12 +593,12 @@ extern "C" int vq_vecinfer_attend(const vq_lut_attend_args *a) {
     // dynamic LDS above 64 KB has to be allowed once per kernel and device
 #define VQ_LUT_LAUNCH(KERNEL, ...)                                                                                  \
     do {                                                                                                            \
-        static bool allowed[64] = {};                                                                               \
+        static std::atomic<bool> allowed[64] = {};   /* a second thread that gets here first repeats the same call */ \
         int dev = 0;                                                                                                \
         (void)hipGetDevice(&dev);                                                                                   \
-        if (dev < 0 || dev >= 64 || !allowed[dev]) {                                                                \
+        if (dev < 0 || dev >= 64 || !allowed[dev].load(std::memory_order_acquire)) {                                \
             (void)hipFuncSetAttribute((const void *)KERNEL, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LA_MAX_LDS); \
-            if (dev >= 0 && dev < 64) allowed[dev] = true;                                                          \
+            if (dev >= 0 && dev < 64) allowed[dev].store(true, std::memory_order_release);                          \
         }                                                                                                           \
         hipLaunchKernelGGL(KERNEL, grid, dim3(LA_THREADS), p.lds, st, *a, p.tiles, p.split_len, p.nsplit, __VA_ARGS__); \
     } while (0)
