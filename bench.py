@@ -707,6 +707,15 @@ def _extras(torch, K, dev):
         lds_ops = B * Hq * 32768 * 16 * 2 / 64    # one look-up and one histogram addition per row, token and sub-vector, 64 lanes an instruction
         ex[f"index_attend_32k_B{B}"] = {"ms": round(ms, 5), "GBps": round(nbytes / ms / 1e6, 1), "bytes": nbytes,
                                         "lds_cycles_per_wave_op_per_cu": round(ms * 1e-3 * 2.1e9 * 256 / lds_ops, 2)}
+    # the same at the head shape of config 2's model (12 query / 4 kv heads, D 256 in 32 sub-vectors): one query row a block
+    ki = torch.randint(0, 256, (16, 4, 32768, 32), device=dev).to(torch.uint8)
+    vi = torch.randint(0, 256, (16, 4, 32768, 32), device=dev).to(torch.uint8)
+    q = torch.randn((16, 12, 1, 256), device=dev).to(torch.float16)
+    fn = lambda: K.metal_fused_sdpa(q, ki, kcb, vi, vcb, 1 / math.sqrt(256))
+    for _ in range(3):
+        fn()
+    ms = _side_ms(fn, 30, torch)
+    ex["index_attend_d256_32k_B16"] = {"ms": round(ms, 5), "GBps": round(2 * ki.numel() / ms / 1e6, 1), "bytes": 2 * ki.numel()}
     return ex
 
 
