@@ -31,8 +31,21 @@ def hip_available() -> bool:
     return _lib.library_present() and torch.cuda.is_available()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(t: torch.Tensor) -> int:
+    """Handle of torch's current stream on the tensor's device (the raw getter skips the Stream object)."""
+    if _raw_stream is not None:
+        i = t.device.index
+        return _raw_stream(torch.cuda.current_device() if i is None else i)
     return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _stream_of(device: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device() if device.index is None else device.index)
+    return torch.cuda.current_stream(device).cuda_stream
 
 
 def _need_gpu(name: str, *tensors: torch.Tensor) -> None:
@@ -781,7 +794,7 @@ _workspaces: dict[tuple, torch.Tensor] = {}
 
 
 def _workspace(device: torch.device, nbytes: int) -> torch.Tensor:
-    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.type, device.index, _stream_of(device))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
@@ -794,7 +807,7 @@ _TILE_SCRATCH_MAX = 2 << 30   # bytes; larger inputs are attended without tiles
 
 
 def _tile_scratch(device: torch.device, rows: int, units: int) -> torch.Tensor:
-    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.type, device.index, _stream_of(device))
     t = _tile_scratches.get(key)
     if t is None or t.numel() < rows * units * PREFILL_TILE_BYTES:
         t = _tile_scratches[key] = torch.empty(rows * units * PREFILL_TILE_BYTES, dtype=torch.uint8, device=device)
@@ -816,7 +829,7 @@ _sync_counters: dict[tuple, torch.Tensor] = {}
 def _counters(device: torch.device) -> torch.Tensor:
     """Per-(device, stream) int32 counters the single-launch decode path needs: zero when a
     call is enqueued, left zero by it (65536 = the largest B*H_kv the MFMA path takes)."""
-    key = (device.type, device.index, torch.cuda.current_stream(device).cuda_stream)
+    key = (device.type, device.index, _stream_of(device))
     c = _sync_counters.get(key)
     if c is None:
         c = torch.zeros(65536, dtype=torch.int32, device=device)
