@@ -655,22 +655,27 @@ template <int GL> __device__ __forceinline__ float group_pick8(int j, int e, con
     else return (j & 4) ? pick4(j, v[4], v[5], v[6], v[7]) : pick4(j, v[0], v[1], v[2], v[3]);
 }
 
-template <typename T, typename M, int BITS, int GL>
+template <typename T, typename M, int BITS, int GL, bool TWO = false>
 __device__ __forceinline__ void kivi_value_pack_body(int bx, int64_t bh, const T *__restrict__ x, int64_t S,
                                                      int64_t x_stride_bh, float levels, float eps,
                                                      uint32_t *__restrict__ packed, M *__restrict__ scale,
-                                                     M *__restrict__ zero, int64_t cap_tokens, int64_t dst_tok0) {
+                                                     M *__restrict__ zero, int64_t cap_tokens, int64_t dst_tok0,
+                                                     const T *__restrict__ alt = nullptr, int64_t alt_first = 0,
+                                                     int64_t alt_rs = 128) {
     constexpr int D = 128, PER = 32 / BITS, HALF = PER / 2, GV = 16 / GL;
     constexpr bool SHARE = GL <= 8;
     constexpr int TP = SHARE ? 8 / GL : 1;
     const int tid = threadIdx.x, o = tid & 15;
     const int64_t t0 = ((int64_t)bx * VP_STRETCHES + (tid >> 4)) * PER;   // the stretch's first token
     if (t0 >= S) return;                                                  // S is a multiple of PER: whole rows of 16 lanes leave
-    const T *xb = x + bh * x_stride_bh + t0 * D + 8 * o;
+    // TWO: tokens from alt_first (a multiple of PER) on are rows of a second tensor, as in the key body
+    const bool from_alt = TWO && t0 >= alt_first;
+    const int64_t rs = from_alt ? alt_rs : (int64_t)D;
+    const T *xb = (from_alt ? alt + (t0 - alt_first) * rs : x + bh * x_stride_bh + t0 * D) + 8 * o;
     const LevelDiv ld = level_div(levels);
     Raw8<T> v[PER];
 #pragma unroll
-    for (int i = 0; i < PER; ++i) v[i].load(xb + (int64_t)i * D);
+    for (int i = 0; i < PER; ++i) v[i].load(xb + (int64_t)i * rs);
     float lo[8], hi[8];
 #pragma unroll
     for (int c = 0; c < 8; ++c) { lo[c] = 0.f; hi[c] = 0.f; }
@@ -818,25 +823,32 @@ constexpr int KQ_WAVES = 4;   // groups per block
 // MIXED (round trip only): channel c of (sequence, head) bh has `levels_hi` levels where hi_mask[bh * 128 + c] is
 // set and `levels` otherwise (Kitty's channel-wise mixed precision, veloxquant_mlx/quantizers/kitty.py:138-169,
 // which forms both reconstructions of the whole tensor and selects per channel).
-template <typename T, typename M, int MODE, int TPL, bool MIXED = false>
+// TWO (the cache's append): tokens from `alt_first` on are rows of a second tensor, `alt` being the row of token
+// alt_first for this (sequence, head) and `alt_rs` its row stride in elements; alt_first is a multiple of the group
+// (or lies at or past S), so a group reads one source.
+template <typename T, typename M, int MODE, int TPL, bool MIXED = false, bool TWO = false>
 __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *__restrict__ x, T *__restrict__ out, int64_t S,
                                                    int64_t x_stride_bh, float levels, float eps, int bits,
                                                    uint32_t *__restrict__ packed, M *__restrict__ scale, M *__restrict__ zero,
                                                    int64_t cap_tokens, int64_t dst_tok0, int W,
                                                    const uint8_t *__restrict__ hi_mask = nullptr, float levels_hi = 0.f,
-                                                   const float *__restrict__ group_levels = nullptr) {
+                                                   const float *__restrict__ group_levels = nullptr,
+                                                   const T *__restrict__ alt = nullptr, int64_t alt_first = 0, int64_t alt_rs = 128) {
     constexpr int D = 128, G = 4 * TPL;
     const int lane = threadIdx.x & 63, o = lane >> 2, tq = lane & 3;
     const int64_t s0 = (int64_t)gk * G;
     if (s0 >= S) return;   // the whole wave
     const int64_t r0 = s0 + tq * TPL;   // the lane's first token
-    const T *xb = x + bh * x_stride_bh + r0 * D + 8 * o;
+    const bool from_alt = TWO && s0 >= alt_first;   // the same for the wave
+    const int64_t row_gap = from_alt ? alt_rs : (int64_t)D;   // elements between rows (a constant without TWO)
+    const T *xg = (from_alt ? alt + (s0 - alt_first) * row_gap : x + bh * x_stride_bh + s0 * D) + 8 * o;   // the group's first row
+    const T *xb = xg + (int64_t)(tq * TPL) * row_gap;
     if (group_levels != nullptr) {   // round trip only: a level count per token group, 0 = the group passes through
         levels = group_levels[gk];
         if (levels == 0.f) {
 #pragma unroll
             for (int i = 0; i < TPL; ++i)
-                if (r0 + i < S) *reinterpret_cast<uint4 *>(out + (bh * S + r0 + i) * D + 8 * o) = *reinterpret_cast<const uint4 *>(xb + (int64_t)i * D);
+                if (r0 + i < S) *reinterpret_cast<uint4 *>(out + (bh * S + r0 + i) * D + 8 * o) = *reinterpret_cast<const uint4 *>(xb + (int64_t)i * row_gap);
             return;
         }
     }
@@ -847,13 +859,12 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
     const bool whole = s0 + G <= S;   // the same for the wave
     if (whole) {
 #pragma unroll
-        for (int i = 0; i < TPL; ++i) v[i].load(xb + (int64_t)i * D);
+        for (int i = 0; i < TPL; ++i) v[i].load(xb + (int64_t)i * row_gap);
 #pragma unroll
         for (int i = 0; i < TPL; ++i) v[i].fold(acc);
     } else {   // a row past the end stands in as the group's first row, which changes no minimum or maximum
-        const T *x0 = x + bh * x_stride_bh + s0 * D + 8 * o;
 #pragma unroll
-        for (int i = 0; i < TPL; ++i) v[i].load(r0 + i < S ? xb + (int64_t)i * D : x0);
+        for (int i = 0; i < TPL; ++i) v[i].load(r0 + i < S ? xb + (int64_t)i * row_gap : xg);
 #pragma unroll
         for (int i = 0; i < TPL; ++i) v[i].fold(acc);
     }
@@ -1101,6 +1112,41 @@ __global__ __launch_bounds__(256) void kivi_kv_pack_kernel(
         kivi_value_pack_body<T, M, BITS, TPL / 2>(bx - key_blocks, (int64_t)blockIdx.y, v, S, x_stride_bh, levels, eps, vd.packed,
                                                   (M *)vd.scale, (M *)vd.zero, cap_tokens, dst_tok0);
 }
+// A whole append of the packed cache in one launch: the keys and values of tokens [0, n_flush) of [tail ; new rows]
+// are quantised and packed straight from where they lie (new rows are not copied into the tail first), and the rows
+// from n_flush on, old or new, go to the front of the spare tail.  Blocks [0, key_blocks) take key groups, the next
+// value_blocks the value stretches, the rest the kept rows (one 16-byte piece a thread).
+struct NewRows { const void *k, *v; int64_t k_sb, k_sh, k_ss, v_sb, v_sh, v_ss; };   // strides in elements
+template <typename T, typename M, int BITS, int TPL>
+__global__ __launch_bounds__(256) void kivi_kv_append_kernel(
+    const T *__restrict__ k_tail, const T *__restrict__ v_tail, int64_t tail_cap, NewRows nw, int H, int64_t n_tail, int64_t n_flush,
+    int64_t need, float levels, float eps, PackDst kd, PackDst vd, int64_t cap_tokens, int64_t dst_tok0, int key_blocks,
+    int value_blocks, T *__restrict__ k_spare, T *__restrict__ v_spare, int64_t spare_cap) {
+    constexpr int D = 128;
+    const int bx = (int)blockIdx.x;
+    const int64_t bh = blockIdx.y, b = bh / H, h = bh - b * H;
+    const T *kn = (const T *)nw.k + b * nw.k_sb + h * nw.k_sh, *vn = (const T *)nw.v + b * nw.v_sb + h * nw.v_sh;
+    if (bx < key_blocks) {
+        kivi_key_quad_body<T, M, 1, TPL, false, true>(bx * KQ_WAVES + (int)(threadIdx.x >> 6), bh, k_tail, nullptr, n_flush, tail_cap * D,
+                                                      levels, eps, BITS, kd.packed, (M *)kd.scale, (M *)kd.zero, cap_tokens, dst_tok0,
+                                                      128 / (32 / BITS), nullptr, 0.f, nullptr, kn, n_tail, nw.k_ss);
+    } else if (bx < key_blocks + value_blocks) {
+        kivi_value_pack_body<T, M, BITS, TPL / 2, true>(bx - key_blocks, bh, v_tail, n_flush, tail_cap * D, levels, eps, vd.packed,
+                                                        (M *)vd.scale, (M *)vd.zero, cap_tokens, dst_tok0, vn, n_tail, nw.v_ss);
+    } else {
+        constexpr int RV = D * (int)sizeof(T) / 16;   // 16-byte pieces of a row
+        const int64_t keep = need - n_flush, i = (int64_t)(bx - key_blocks - value_blocks) * 256 + threadIdx.x;
+        if (i >= 2 * keep * RV) return;
+        const bool values = i >= keep * RV;
+        const int64_t j = values ? i - keep * RV : i, r = n_flush + j / RV, c = j % RV;
+        const T *tail = values ? v_tail : k_tail, *fresh = values ? vn : kn;
+        const int64_t fs = values ? nw.v_ss : nw.k_ss;
+        const uint4 x = r < n_tail ? reinterpret_cast<const uint4 *>(tail + (bh * tail_cap + r) * D)[c]
+                                   : reinterpret_cast<const uint4 *>(fresh + (r - n_tail) * fs)[c];
+        reinterpret_cast<uint4 *>((values ? v_spare : k_spare) + (bh * spare_cap + (r - n_flush)) * D)[c] = x;
+    }
+}
+
 template <typename T, typename M, int LPR, int NP, int VMODE>
 __global__ __launch_bounds__(256) void kivi_kv_tile_kernel(
     const T *__restrict__ k, const T *__restrict__ v, int64_t S, int64_t x_stride_bh, int group, float levels, float eps,
@@ -1624,6 +1670,47 @@ static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t 
 namespace vq {
 // Keys (groups along tokens) and values (groups along channels, v_layout) of the same S tokens in
 // one launch where the tile kernels take the shape, else as two single calls.
+// The whole append as one launch where the fused key / value kernel takes the shape (head size 128, 16-bit rows,
+// token-packed values, groups of 32 / 64, 2 or 4 bits) and no group of flushed tokens mixes old and new rows.
+bool append_one_launch(const void *k_new, const void *v_new, const int64_t ks[3], const int64_t vs[3], const void *k_tail,
+                       const void *v_tail, void *k_spare, void *v_spare, int dtype, int64_t B, int64_t H, int64_t D, int64_t tail_cap,
+                       int64_t spare_cap, int64_t n_tail, int64_t n_flush, int64_t need, int group, int levels, float eps, int bits,
+                       int v_layout, void *kp, void *ksc, void *kz, void *vp, void *vsc, void *vz, int meta_dtype, int64_t cap,
+                       int64_t tok0, void *stream) {
+    const int per = bits >= 1 && bits <= 8 ? 32 / bits : 1;
+    const int64_t BH = B * H;
+    const bool ok = D == 128 && (dtype == VQ_F16 || dtype == VQ_BF16) && (meta_dtype == VQ_F16 || meta_dtype == VQ_F32) && BH >= 1 &&
+                    BH <= 65535 && H <= 0x7fffffff && n_flush >= 1 && v_layout == VQ_V_TOKEN_PACKED && (group == 32 || group == 64) &&
+                    (bits == 2 || bits == 4) && levels >= 1 && levels <= (1 << bits) - 1 && tok0 >= 0 && tok0 + n_flush <= cap &&
+                    tok0 % group == 0 && tok0 % per == 0 && n_flush % per == 0 && cap % per == 0 && tok0 % 8 == 0 && cap % 8 == 0 &&
+                    (n_tail >= n_flush || n_tail % group == 0) && aligned16(k_tail) && aligned16(v_tail) && aligned16(k_new) &&
+                    aligned16(v_new) && aligned16(k_spare) && aligned16(v_spare) && aligned16(kp) && aligned16(ksc) && aligned16(kz) &&
+                    aligned16(vp) && aligned16(vsc) && aligned16(vz) && ks[0] % 8 == 0 && ks[1] % 8 == 0 && ks[2] % 8 == 0 &&
+                    vs[0] % 8 == 0 && vs[1] % 8 == 0 && vs[2] % 8 == 0;
+    if (!ok) return false;
+    const int kb = (int)cdiv(cdiv(n_flush, group), KQ_WAVES), vb = (int)cdiv(n_flush, VP_STRETCHES * per);
+    const int64_t keep = need - n_flush;
+    const int rb = (int)cdiv(2 * keep * (D * 2 / 16), 256);
+    const dim3 grid((unsigned)(kb + vb + rb), (unsigned)BH);
+    const PackDst kd = {(uint32_t *)kp, ksc, kz}, vd = {(uint32_t *)vp, vsc, vz};
+    const NewRows nw = {k_new, v_new, ks[0], ks[1], ks[2], vs[0], vs[1], vs[2]};
+    hipStream_t st = (hipStream_t)stream;
+#define VQ_AP(T, M, BITS, TPL)                                                                                                  \
+    hipLaunchKernelGGL((kivi_kv_append_kernel<T, M, BITS, TPL>), grid, dim3(256), 0, st, (const T *)k_tail, (const T *)v_tail, tail_cap, \
+                       nw, (int)H, n_tail, n_flush, need, (float)levels, eps, kd, vd, cap, tok0, kb, vb, (T *)k_spare, (T *)v_spare,    \
+                       spare_cap)
+#define VQ_AP_B(T, M)                                                                                  \
+    do {                                                                                               \
+        if (bits == 4) { if (group == 32) VQ_AP(T, M, 4, 8); else VQ_AP(T, M, 4, 16); }                \
+        else { if (group == 32) VQ_AP(T, M, 2, 8); else VQ_AP(T, M, 2, 16); }                          \
+    } while (0)
+    if (dtype == VQ_F16) { if (meta_dtype == VQ_F16) VQ_AP_B(f16, f16); else VQ_AP_B(f16, float); }
+    else { if (meta_dtype == VQ_F16) VQ_AP_B(bf16_t, f16); else VQ_AP_B(bf16_t, float); }
+#undef VQ_AP_B
+#undef VQ_AP
+    return true;
+}
+
 int pack_kv_pair(const void *k, const void *v, int dtype, int64_t BH, int64_t S, int64_t D, int64_t xs, int group,
                  int levels, float eps, int bits, int v_layout, void *kp, void *ks, void *kz, void *vp, void *vs, void *vz,
                  int meta_dtype, int64_t cap, int64_t tok0, void *stream) {

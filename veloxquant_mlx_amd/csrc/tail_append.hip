@@ -45,6 +45,11 @@ __global__ __launch_bounds__(256) void kv_chunk_route_kernel(TailSrc k, TailSrc 
 int pack_kv_pair(const void *k, const void *v, int dtype, int64_t BH, int64_t S, int64_t D, int64_t xs, int group,
                  int levels, float eps, int bits, int v_layout, void *kp, void *ks, void *kz, void *vp, void *vs, void *vz,
                  int meta_dtype, int64_t cap, int64_t tok0, void *stream);
+bool append_one_launch(const void *k_new, const void *v_new, const int64_t ks[3], const int64_t vs[3], const void *k_tail,
+                       const void *v_tail, void *k_spare, void *v_spare, int dtype, int64_t B, int64_t H, int64_t D, int64_t tail_cap,
+                       int64_t spare_cap, int64_t n_tail, int64_t n_flush, int64_t need, int group, int levels, float eps, int bits,
+                       int v_layout, void *kp, void *ksc, void *kz, void *vp, void *vsc, void *vz, int meta_dtype, int64_t cap,
+                       int64_t tok0, void *stream);
 
 }  // namespace vq
 
@@ -118,6 +123,14 @@ extern "C" int vq_kivi_cache_append(const vq_kivi_append_args *pa, void *stream)
                VQ_ERR_UNSUPPORTED, "%s: pointers must be 16-byte aligned", fn);
     VQ_REQUIRE(a.k_packed && a.k_scale && a.k_zero && a.v_packed && a.v_scale && a.v_zero, VQ_ERR_INVALID,
                "%s: null packed store", fn);
+    // one launch where the fused kernel takes the shape: new rows are quantised from where they lie
+    if (a.S > 0 && append_one_launch(a.k_new, a.v_new, a.k_strides, a.v_strides, a.k_tail, a.v_tail, a.k_spare, a.v_spare, a.dtype,
+                                     a.B, a.H, a.D, a.tail_cap, a.spare_cap, a.n_tail, a.n_flush, need, a.group, a.levels, a.eps,
+                                     a.pack_bits, a.v_layout, a.k_packed, a.k_scale, a.k_zero, a.v_packed, a.v_scale, a.v_zero,
+                                     a.meta_dtype, a.cap_tokens, a.dst_tok0, stream)) {
+        VQ_HIP_CHECK_LAUNCH(fn);
+        return VQ_OK;
+    }
     const int64_t vec = 16 / es, row_vecs = a.D / vec;
     const int64_t r0 = a.n_tail < a.n_flush ? a.n_tail : a.n_flush, total = a.B * a.H * (need - r0) * row_vecs;
     if (total > 0) {
