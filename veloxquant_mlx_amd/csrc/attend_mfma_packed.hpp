@@ -613,6 +613,13 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     constexpr int CH = RG::CHUNK;
     const int n_chunks = (n_units + CH - 1) / CH;
     int dealt = wave;   // fixed order: wave w takes chunks w, w + WAVES, ...
+    // 2-bit codes: every block starts its walk at a chunk of its own.  The blocks of a launch otherwise walk
+    // identically laid-out heads in lockstep and their 256-byte scale / zero copies meet in the same memory
+    // channels (3 % at 2 bits, where those copies are a third of the bytes; nothing at 4 bits).  Not under
+    // `fixed_order`, whose results must not depend on a block's place in the grid (a layer-batched launch equals the
+    // per-layer ones bit for bit there).
+    const int rot = BITS == 2 && !fixed_order && n_chunks > 1 ? (int)((((unsigned)blockIdx.x * 2654435761u + (unsigned)blockIdx.y * 40503u) >> 12) % (unsigned)n_chunks) : 0;
+    auto phys = [&](int id) VQ_INLINE_LAMBDA { const int q = id + rot; return q >= n_chunks ? q - n_chunks : q; };
     auto draw = [&]() VQ_INLINE_LAMBDA {   // the next chunk of the block; the value is used a chunk later
         int id = 0;
         if (fixed_order) id = (dealt += RG::WAVES);
@@ -622,8 +629,8 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
     auto chunk_len = [&](int chunk) VQ_INLINE_LAMBDA { return n_units - chunk * CH < CH ? n_units - chunk * CH : CH; };
     if (wave >= n_chunks) return;   // the first WAVES chunks are dealt out, the counter starts behind them
     constexpr int END = -1, NONE = -2;
-    int i_chunk = wave, i_pos = 0, i_slot = 0, i_gslot = 0;
-    int c_chunk = wave, c_pos = 0, c_next = NONE, c_after = NONE, c_slot = 0, c_gslot = 0;
+    int i_chunk = phys(wave), i_pos = 0, i_slot = 0, i_gslot = 0;
+    int c_chunk = i_chunk, c_pos = 0, c_next = NONE, c_after = NONE, c_slot = 0, c_gslot = 0;
     int in_flight = 0;
     int drawn = draw();
     auto issue_next = [&]() VQ_INLINE_LAMBDA {
@@ -635,7 +642,7 @@ __device__ __forceinline__ void packed_units(const vq_attend_args &a, int64_t bh
         ++in_flight;
         if (++i_pos == chunk_len(i_chunk)) {
             const int got = __builtin_amdgcn_readfirstlane(drawn);
-            i_chunk = got < n_chunks ? got : END;
+            i_chunk = got < n_chunks ? phys(got) : END;
             i_pos = 0;
             if (c_next == NONE) c_next = i_chunk;
             else c_after = i_chunk;
