@@ -930,6 +930,7 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
                            pick4(tq, mn[1], mn[3], mn[5], mn[7]));
         }
     }
+    uint32_t *const words0 = MODE == 1 ? packed + (bh * cap_tokens + dst_tok0 + r0) * W : nullptr;   // the lane's first row of words
     auto rows = [&](auto whole_group) __attribute__((always_inline)) {
         constexpr bool WHOLE = decltype(whole_group)::value;
 #pragma unroll
@@ -954,7 +955,8 @@ __device__ __forceinline__ void kivi_key_quad_body(int gk, int64_t bh, const T *
                     store8<T>(out + (bh * S + srow) * D + 8 * o, y);
                 }
             } else {
-                uint32_t *row_words = packed + (bh * cap_tokens + dst_tok0 + (valid ? srow : 0)) * W;
+                // (a whole group: one base for the lane's rows, the rows a constant apart)
+                uint32_t *row_words = WHOLE ? words0 + (int64_t)i * W : packed + (bh * cap_tokens + dst_tok0 + (valid ? srow : 0)) * W;
                 if (bits == 8) {
                     if (valid) *reinterpret_cast<uint2 *>(row_words + 2 * o) = bytes8(q);
                 } else if (bits == 4) {
