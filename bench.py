@@ -286,7 +286,7 @@ def main() -> int:
 
 _ROWS_CASES = {"decode_d256_2bit_32k_B16": (12, 4, 256, 2, 32), "decode_d256_4bit_32k_B16": (12, 4, 256, 4, 64),
                "decode_3bit_32k_B16": (32, 8, 128, 3, 32)}
-_ROWS_NOTES = {"decode_d256_2bit_32k_B16": "matrix-unit decode kernel, head of 256 channels (two launches: the fp16 tail comes from the vector kernel)",
+_ROWS_NOTES = {"decode_d256_2bit_32k_B16": "matrix-unit decode kernel, head of 256 channels (two launches: the fp16 tail comes from the vector kernel, four runs)",
                "decode_d256_4bit_32k_B16": "matrix-unit decode kernel, head of 256 channels, four waves per CU",
                "decode_3bit_32k_B16": "vector-unit kernel (attend_rows_kernel), four query rows of a kv head per block"}
 

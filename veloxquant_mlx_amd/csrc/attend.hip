@@ -87,7 +87,9 @@ AttendPlan plan_attend(const vq_attend_args &a) {
     p.nparts = p.nsplit;
     if (p.path == 1 && a.n_tail > 0) {
         int64_t tw = cdiv(cdiv(a.n_tail, 32), units >= 64 ? 8 : 1);
-        p.nparts += a.D == 128 ? (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw) : 1;
+        // (a head of 256 channels: the tail launch of the vector kernel, up to four runs of at least 16 tokens)
+        const int64_t tr = cdiv(a.n_tail, 16);
+        p.nparts += a.D == 128 ? (int)(tw < 1 ? 1 : tw > 8 ? 8 : tw) : (int)(tr > 4 ? 4 : tr);
     }
     return p;
 }

@@ -36,6 +36,19 @@ __device__ __forceinline__ float ar_ld(const void *p, int tag, int64_t i) {
     if (tag == VQ_BF16) return bf16_to_f32(((const u16 *)p)[i]);
     return ((const float *)p)[i];
 }
+// Eight 16-bit channels of a plain row (one 16-byte piece) as floats.
+__device__ __forceinline__ void ar_piece8(const uint4 &v, int tag, float (&o)[8]) {
+    const u32 w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        if (tag == VQ_F16) {
+            const f16x2 h = __builtin_bit_cast(f16x2, w[j]);
+            o[2 * j] = (float)h[0]; o[2 * j + 1] = (float)h[1];
+        } else {
+            o[2 * j] = __uint_as_float(w[j] << 16); o[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+        }
+    }
+}
 template <int CTRL> __device__ __forceinline__ float ar_dpp(float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
 }
@@ -285,15 +298,47 @@ __global__ __launch_bounds__(256) void attend_rows_kernel(vq_attend_args a, int6
     const int64_t q0 = t0 > a.n_packed ? t0 : a.n_packed;
     if (q0 < t1) {
         if (cur_kg != -2) fold(-2);
-        for (int64_t t = q0 + gslot; t < t1; t += nslots) {
-            float kc[CPL], vc[CPL];
-            const int64_t ti = (bh * a.tail_cap + (t - a.n_packed)) * D + d0;
-#pragma unroll
-            for (int j = 0; j < CPL; ++j) {
-                kc[j] = j < nch ? ar_ld(a.k_tail, a.tail_dtype, ti + j) : 0.f;
-                vc[j] = j < nch ? ar_ld(a.v_tail, a.tail_dtype, ti + j) : 0.f;
+        // Lanes that own eight whole 16-bit channels (the head sizes that are multiples of 8) take their piece of a row
+        // as one 16-byte load, and two tokens of a slot are requested before the first is used.
+        const bool vec = CPL == 8 && a.tail_dtype != VQ_F32 && D % 8 == 0 && ((((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u) == 0);
+        if constexpr (CPL == 8) {
+            if (vec) {
+                const u16 *kt = (const u16 *)a.k_tail, *vt = (const u16 *)a.v_tail;
+                for (int64_t t = q0 + gslot; t < t1; t += 2 * nslots) {
+                    const bool two = t + nslots < t1;   // the same for the lanes of a slot
+                    const int64_t ti = (bh * a.tail_cap + (t - a.n_packed)) * D + d0;
+                    uint4 k0 = make_uint4(0, 0, 0, 0), v0 = k0, k1 = k0, v1 = k0;
+                    if (live) {
+                        k0 = *reinterpret_cast<const uint4 *>(kt + ti);
+                        v0 = *reinterpret_cast<const uint4 *>(vt + ti);
+                        if (two) {
+                            k1 = *reinterpret_cast<const uint4 *>(kt + ti + (int64_t)nslots * D);
+                            v1 = *reinterpret_cast<const uint4 *>(vt + ti + (int64_t)nslots * D);
+                        }
+                    }
+                    float kc[8], vc[8];
+                    ar_piece8(k0, a.tail_dtype, kc);
+                    ar_piece8(v0, a.tail_dtype, vc);
+                    token(t, kc, vc, 1.f, 0.f, 1.f, 0.f);
+                    if (two) {
+                        ar_piece8(k1, a.tail_dtype, kc);
+                        ar_piece8(v1, a.tail_dtype, vc);
+                        token(t + nslots, kc, vc, 1.f, 0.f, 1.f, 0.f);
+                    }
+                }
             }
-            token(t, kc, vc, 1.f, 0.f, 1.f, 0.f);
+        }
+        if (!vec) {
+            for (int64_t t = q0 + gslot; t < t1; t += nslots) {
+                float kc[CPL], vc[CPL];
+                const int64_t ti = (bh * a.tail_cap + (t - a.n_packed)) * D + d0;
+#pragma unroll
+                for (int j = 0; j < CPL; ++j) {
+                    kc[j] = j < nch ? ar_ld(a.k_tail, a.tail_dtype, ti + j) : 0.f;
+                    vc[j] = j < nch ? ar_ld(a.v_tail, a.tail_dtype, ti + j) : 0.f;
+                }
+                token(t, kc, vc, 1.f, 0.f, 1.f, 0.f);
+            }
         }
     }
 
@@ -366,8 +411,8 @@ int launch_attend_rows_tail(const vq_attend_args &a, int part0, int nparts) {
     AttendPlan p = {};
     p.path = 3;
     rows_tiling(a, p.pq, p.tiles);
-    p.nsplit = 1;
-    p.split_len = a.n_tail > 0 ? a.n_tail : 1;
+    p.nsplit = nparts - part0 > 1 ? nparts - part0 : 1;   // the partials past part0 are this launch's runs
+    p.split_len = a.n_tail > 0 ? cdiv(a.n_tail, p.nsplit) : 1;
     p.nparts = nparts;
     p.part0 = part0;
     return launch_attend_rows(a, p);
