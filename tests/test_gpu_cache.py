@@ -99,7 +99,7 @@ def test_decode_at_head_size_256_through_the_cache_and_the_layer_stack(bits, g):
     from veloxquant_mlx_amd.cache import LayerStackedKIVICache
     B, Hq, Hkv, D, R, NL = 2, 12, 4, 256, 64, 2
     cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=bits, kivi_group_size=g, residual_length=R,
-                        fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=1280)
+                        fused_sdpa=True, fused_sdpa_memory_bound=True, fused_sdpa_max_ctx=1280, kivi_code_field="tight")
     solo = [KVCacheFactory.create(cfg) for _ in range(NL)]
     stack = LayerStackedKIVICache(cfg, NL)
     n0 = 960 if bits == 3 else 1000
@@ -519,6 +519,70 @@ def test_sink_protected_cache_with_prefill_sized_query_blocks(bits, g):
         assert err < 2e-3, (w, err)
 
 
+@pytest.mark.parametrize("bits,D,g,Hq,meta", [(3, 128, 32, 8, "float16"), (1, 128, 32, 8, "float32"), (3, 128, 64, 4, "float32"),
+                                              (3, 256, 32, 6, "float16"), (1, 256, 64, 2, "float16")])
+def test_odd_code_widths_in_the_next_even_field(bits, D, g, Hq, meta, tmp_path):
+    """3-bit codes in 4-bit fields and 1-bit codes in 2-bit fields (``kivi_code_field="auto"``, the default): the same
+    levels, hence the same codes, scale and zero as the tight packing, on the kernels of the even widths -- a prefill in
+    chunks, decode steps across flushes, a trim, the saved state -- against the oracle and against a tight-packed cache."""
+    require_gpu()
+    B, H, R = 2, 2, 64
+    kw = dict(head_dim=D, bit_width_inlier=bits, kivi_group_size=g, residual_length=R, fused_sdpa=True,
+              fused_sdpa_memory_bound=True, kivi_meta_dtype=meta)
+    c, tight = _make(**kw), _make(**kw, kivi_code_field="tight")
+    assert c._field == {3: 4, 1: 2}[bits] and tight._field == bits and c._v_layout == "token"
+    n0, n1 = 700, 790
+    k, v = outlier_kv((B, H, n1, D), seed=bits * 100 + D + g)
+    rng = np.random.default_rng(bits + D)
+    scale, levels = 1 / math.sqrt(D), (1 << bits) - 1
+    for x in (c, tight):
+        for lo in range(0, n0, 256):
+            hi = min(lo + 256, n0)
+            x.update_and_fetch(to_dev(k[:, :, lo:hi]), to_dev(v[:, :, lo:hi]))
+
+    def check(t_end, Sq=1, oracle=True):
+        nq = c._n_quantized
+        assert nq == tight._n_quantized and c.offset == tight.offset == t_end
+        q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float16)
+        got = host(c.fused_sdpa(to_dev(q), scale, causal=True)).astype(np.float32)
+        ref_t = host(tight.fused_sdpa(to_dev(q), scale, causal=True)).astype(np.float32)
+        assert float(np.max(np.abs(got - ref_t))) < 2e-3, (t_end, Sq)
+        if not oracle:
+            return
+        md = np.float16 if meta == "float16" else np.float32
+        kq = ok.group_quant_codes(k[:, :, :nq], -2, g, levels)
+        vq = ok.group_quant_codes(v[:, :, :nq], -1, g, levels)
+        ref = oa.kivi_attend(q, kq[0], kq[1].astype(md), kq[2].astype(md), vq[0], vq[1].astype(md), vq[2].astype(md), g,
+                             k[:, :, nq:t_end], v[:, :, nq:t_end], scale, causal=True)
+        assert float(np.max(np.abs(got - ref))) < 2e-3, (t_end, Sq)
+        # the codes themselves: what the wide fields hold is what the tight words hold
+        kd = K.kivi_dequant(c._kp, c._ks, c._kz, -2, g, c._field, nq, D)
+        kt = K.kivi_dequant(tight._kp, tight._ks, tight._kz, -2, g, bits, nq, D)
+        vd = K.kivi_dequant(c._vp, c._vs, c._vz, -1, g, c._field, nq, D, v_layout=c._v_layout)
+        vt = K.kivi_dequant(tight._vp, tight._vs, tight._vz, -1, g, bits, nq, D, v_layout=tight._v_layout)
+        assert torch.equal(kd, kt) and torch.equal(vd, vt)
+
+    check(n0)
+    check(n0, Sq=3)
+    for t in range(n0, n1):
+        for x in (c, tight):
+            x.update_and_fetch(to_dev(k[:, :, t:t + 1]), to_dev(v[:, :, t:t + 1]))
+        if t % 13 == 0 or t == n1 - 1:
+            check(t + 1)
+    # saved and restored: the width of the field travels in meta_state, and a cache of the other packing refuses the file
+    assert c.meta_state[2] == f"{bits}/{c._field}" and tight.meta_state[2] == str(bits)
+    r = type(c).from_state(KVCacheConfig(method="kivi", **kw), c.state, c.meta_state)
+    q = rng.standard_normal((B, Hq, 1, D)).astype(np.float16)
+    assert torch.equal(r.fused_sdpa(to_dev(q), scale, fixed_order=True), c.fused_sdpa(to_dev(q), scale, fixed_order=True))
+    with pytest.raises(ValueError):
+        _make(**kw, kivi_code_field="tight").meta_state = c.meta_state
+    # a trim into the packed rows brings them back as their reconstruction, the same one from either packing
+    for x in (c, tight):
+        assert x.trim(120) == 120
+    check(n1 - 120, oracle=False)
+    assert torch.equal(c._tail_k[:, :, : c.offset - c._n_quantized], tight._tail_k[:, :, : c.offset - c._n_quantized])
+
+
 @pytest.mark.parametrize("D,bits", [(64, 4), (256, 2), (128, 3)])
 def test_sink_protected_cache_on_the_other_decode_kernels(D, bits):
     """Protected rows where the attention kernel is the vector one (head size 64, 3-bit codes) or the 256-channel form of
@@ -531,7 +595,8 @@ def test_sink_protected_cache_on_the_other_decode_kernels(D, bits):
     for p, f in ((7, 11), (130, 9), (131, 13)):
         k[:, :, p] *= f
     cfg = KVCacheConfig(method="kivi_sink", head_dim=D, bit_width_inlier=bits, kivi_group_size=32, residual_length=R,
-                        n_sink_tokens=3, fused_sdpa=True, fused_sdpa_memory_bound=True, kivi_meta_dtype="float32")
+                        n_sink_tokens=3, fused_sdpa=True, fused_sdpa_memory_bound=True, kivi_meta_dtype="float32",
+                        kivi_code_field="tight")
     c = KVCacheFactory.create(cfg)
     m = ok.SinkCacheModel(bits, 32, R, 3)
     c.update_and_fetch(to_dev(k[:, :, :320]), to_dev(v[:, :, :320]))

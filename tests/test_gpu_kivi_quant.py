@@ -197,7 +197,8 @@ def test_quant_pack_odd_shapes(shape, g, b, axis):
     _pack_exact(k if axis == -2 else v, axis, b, g, torch.float32)
 
 
-@pytest.mark.parametrize("b,g,D", [(4, 32, 128), (2, 32, 128), (4, 64, 128), (2, 64, 128), (8, 32, 64), (3, 32, 96), (2, 64, 256)])
+@pytest.mark.parametrize("b,g,D", [(4, 32, 128), (2, 32, 128), (4, 64, 128), (2, 64, 128), (8, 32, 64), (3, 32, 96), (2, 64, 256),
+                                   (2, 32, 256), (4, 32, 256), (2, 128, 256), (2, 32, 64), (1, 32, 128)])
 def test_value_token_packed_layout(b, g, D):
     per = 32 // b
     S = per * 12

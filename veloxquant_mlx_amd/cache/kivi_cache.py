@@ -85,7 +85,13 @@ class KIVIKVCache(FP16KVCache):
         if meta not in _META:
             raise QuantizerConfigError(f"KIVIKVCache: kivi_meta_dtype={meta!r} must be 'float16' or 'float32'.")
         self._meta_dtype = _META[meta]
-        per = 32 // self._b
+        # bits a code takes in the packed words: the quantiser's own width, or the next width the matrix-unit
+        # kernels read (2 for 1-bit codes, 4 for 3-bit codes); the levels, hence every value, are the same
+        field = getattr(config, "kivi_code_field", "auto")
+        if field not in ("auto", "tight"):
+            raise QuantizerConfigError(f"KIVIKVCache: kivi_code_field={field!r} must be 'auto' or 'tight'.")
+        self._field = {1: 2, 3: 4}.get(self._b, self._b) if field == "auto" else self._b
+        per = 32 // self._field
         layout = getattr(config, "kivi_value_layout", "auto")
         if layout == "auto":
             layout = "token" if self._group_size % per == 0 else "channel"
@@ -93,7 +99,7 @@ class KIVIKVCache(FP16KVCache):
             raise QuantizerConfigError(f"KIVIKVCache: kivi_value_layout={layout!r} must be token/channel/auto.")
         if layout == "token" and self._group_size % per != 0:
             raise QuantizerConfigError(
-                f"KIVIKVCache: token-packed values need kivi_group_size % {per} == 0 at {self._b} bits.")
+                f"KIVIKVCache: token-packed values need kivi_group_size % {per} == 0 at {self._field} bits a code.")
         self._v_layout = layout
         self._per = per
 
@@ -188,10 +194,10 @@ class KIVIKVCache(FP16KVCache):
         """Quantise + pack fp16 tokens (a group-aligned block) at packed position ``lo``."""
         B, H, n, D = k_blk.shape
         self._ensure_packed_capacity(B, H, D, lo + n, k_blk.device)
-        K.kivi_quant_pack(k_blk, -2, self._group_size, self._b, eps=self._eps, meta_dtype=self._meta_dtype,
-                          out=(self._kp, self._ks, self._kz), dst_tok0=lo)
-        K.kivi_quant_pack(v_blk, -1, self._group_size, self._b, eps=self._eps, meta_dtype=self._meta_dtype,
-                          v_layout=self._v_layout, out=(self._vp, self._vs, self._vz), dst_tok0=lo)
+        K.kivi_quant_pack(k_blk, -2, self._group_size, self._field, levels=self._levels, eps=self._eps,
+                          meta_dtype=self._meta_dtype, out=(self._kp, self._ks, self._kz), dst_tok0=lo)
+        K.kivi_quant_pack(v_blk, -1, self._group_size, self._field, levels=self._levels, eps=self._eps,
+                          meta_dtype=self._meta_dtype, v_layout=self._v_layout, out=(self._vp, self._vs, self._vz), dst_tok0=lo)
 
     # ------------------------------------------------------------------ protocol
     def update_and_fetch(self, keys: torch.Tensor, values: torch.Tensor):
@@ -291,7 +297,7 @@ class KIVIKVCache(FP16KVCache):
             self._append_args = K.kivi_cache_append(
                 keys, values, self._tail_k, self._tail_v, n_tail, max(n_quant_now, 0),
                 (self._kp, self._ks, self._kz, self._vp, self._vs, self._vz), self._n_quantized, spare,
-                bits=self._b, group_size=self._group_size, levels=self._levels, eps=self._eps,
+                bits=self._field, group_size=self._group_size, levels=self._levels, eps=self._eps,
                 v_layout=self._v_layout, args=self._append_args)
         elif n_quant_now > 0:
             self._pack_block(self._tail_k[:, :, :n_quant_now], self._tail_v[:, :, :n_quant_now], self._n_quantized)
@@ -337,7 +343,7 @@ class KIVIKVCache(FP16KVCache):
         else:
             tk, tv = self.keys[:, :, nq:], self.values[:, :, nq:]
         kw = dict(k_packed=self._kp, k_scale=self._ks, k_zero=self._kz, v_packed=self._vp, v_scale=self._vs,
-                  v_zero=self._vz, n_packed=nq, bits=self._b, group_size=self._group_size, v_layout=self._v_layout,
+                  v_zero=self._vz, n_packed=nq, bits=self._field, group_size=self._group_size, v_layout=self._v_layout,
                   k_tail=tk if n_tail else None, v_tail=tv if n_tail else None, n_tail=n_tail, scale=float(scale),
                   causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype, fixed_order=fixed_order,
                   sliding_window=int(sliding_window or 0), num_splits=max(0, int(num_splits)))
@@ -436,10 +442,10 @@ class KIVIKVCache(FP16KVCache):
                         self._tail_v = torch.zeros_like(self._tail_k)
                     lo = self._n_quantized
                     self._tail_k[:, :, :live] = K.kivi_dequant(
-                        self._kp, self._ks, self._kz, -2, self._group_size, self._b, live, D,
+                        self._kp, self._ks, self._kz, -2, self._group_size, self._field, live, D,
                         out_dtype=self._tail_k.dtype, src_tok0=lo)
                     self._tail_v[:, :, :live] = K.kivi_dequant(
-                        self._vp, self._vs, self._vz, -1, self._group_size, self._b, live, D,
+                        self._vp, self._vs, self._vz, -1, self._group_size, self._field, live, D,
                         v_layout=self._v_layout, out_dtype=self._tail_v.dtype, src_tok0=lo)
             self._rollback_bytes(trimmed, n_rolled)
         del old_nq
@@ -537,7 +543,7 @@ class KIVIKVCache(FP16KVCache):
         want = ((B, H, n, W), (B, H, n // g, D), (B, H, n // g, D), *want_v)
         got = tuple(tuple(t.shape) for t in packed)
         if n % g or (self._v_layout == "token" and n % per) or got != want:
-            raise ValueError(f"KIVIKVCache.state: packed rows {got} do not fit bits={self._b}, group={g}, "
+            raise ValueError(f"KIVIKVCache.state: packed rows {got} do not fit {self._field} bits a code, group={g}, "
                              f"value layout {self._v_layout!r}, head_dim={D} (expected {want})")
         if any(t.dtype != self._meta_dtype for t in (ks, kz, vs, vz)):
             raise ValueError(f"KIVIKVCache.state: scale/zero must be {self._meta_dtype}")
@@ -569,7 +575,8 @@ class KIVIKVCache(FP16KVCache):
         """Strings, as prompt-cache files store them: what a restored cache must agree with
         (offset, frontier, bit width, group, value layout, scale/zero dtype, mode)."""
         mode = "memory_bound" if self._memory_bound else ("stash" if self._fused_enabled else "standard")
-        return tuple(map(str, (self.offset, self._n_quantized, self._b, self._group_size, self._v_layout,
+        bits = self._b if self._field == self._b else f"{self._b}/{self._field}"   # code width / width of its field
+        return tuple(map(str, (self.offset, self._n_quantized, bits, self._group_size, self._v_layout,
                                str(self._meta_dtype).replace("torch.", ""), mode)))
 
     @meta_state.setter

@@ -61,7 +61,7 @@ class LayerStackedKIVICache:
         if not layers or not all(isinstance(c, KIVIKVCache) and c._memory_bound for c in layers):
             raise ValueError("LayerStackedKIVICache.from_layers: needs memory-bound packed KIVIKVCache objects")
         c0 = layers[0]
-        if any((c._b, c._group_size, c._v_layout, c._meta_dtype) != (c0._b, c0._group_size, c0._v_layout, c0._meta_dtype)
+        if any((c._b, c._field, c._group_size, c._v_layout, c._meta_dtype) != (c0._b, c0._field, c0._group_size, c0._v_layout, c0._meta_dtype)
                for c in layers):
             raise ValueError("LayerStackedKIVICache.from_layers: the layers differ in bit width, group size or layout")
         self = cls.__new__(cls)
@@ -220,7 +220,7 @@ class LayerStackedKIVICache:
                 self._lens = (key, rep(nq), rep(nt))
             lens = dict(packed_lens=self._lens[1], tail_lens=self._lens[2])
         kp, ks, kz, vp, vs, vz = self._packed
-        kw = dict(k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz, n_packed=max(nq), bits=c0._b,
+        kw = dict(k_packed=kp, k_scale=ks, k_zero=kz, v_packed=vp, v_scale=vs, v_zero=vz, n_packed=max(nq), bits=c0._field,
                   group_size=c0._group_size, v_layout=c0._v_layout, k_tail=tk if max(nt) else None,
                   v_tail=tv if max(nt) else None, n_tail=max(nt), scale=float(scale),
                   causal=bool(causal) and q.shape[3] > 1, out_dtype=q.dtype, fixed_order=fixed_order,

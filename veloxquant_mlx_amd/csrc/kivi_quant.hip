@@ -1662,7 +1662,7 @@ static bool try_tile_path(int mode, int axis, const void *x, void *out, int64_t 
 #undef VQ_VP
         return true;
     }
-    if (mode == 2 && (RPP % (32 / bits)) != 0) return false;
+    if (mode == 2 && ((RPP * VT_TILES) % (32 / bits)) != 0) return false;   // a block's rows hold whole words
 #define VQ_V(L) launch_value_tile<T, M, L>(mode, x, out, BH, S, xs, group, levels, eps, bits, packed, scale, zero, cap, tok0, st)
     if (LPR == 8) VQ_V(8); else if (LPR == 16) VQ_V(16); else VQ_V(32);
 #undef VQ_V
