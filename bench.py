@@ -53,7 +53,7 @@ def _parse():
     p.add_argument("--per-layer", action="store_true", help="with --only-kernel: one launch per layer")
     p.add_argument("--only", default=None, metavar="NAME",
                    help="run one side workload in a loop and print its timing (for rocprofv3): "
-                        "decode_2bit_B16, decode_2bit_B1, decode_d256_2bit_32k_B16, decode_d256_4bit_32k_B16, decode_3bit_32k_B16, decode_3bit_tight_32k_B16, decode_1bit_32k_B16, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
+                        "decode_2bit_B16, decode_2bit_B1, decode_d256_2bit_32k_B16, decode_d256_4bit_32k_B16, decode_3bit_32k_B16, decode_3bit_tight_32k_B16, decode_1bit_32k_B16, decode_d64_4bit_32k_B16, decode_d64_unpaired_4bit_32k_B16, vq_assign, flash_prefill_<S>, prefill, quant_pack, quant_dequant, zipcache, skvq")
     p.add_argument("--copy-calib", action="store_true",
                    help="run a plain 1 GiB device copy a few times and exit (calibrates HBM byte counters)")
     return p.parse_args()
@@ -286,23 +286,28 @@ def main() -> int:
 
 _ROWS_CASES = {"decode_d256_2bit_32k_B16": (12, 4, 256, 2, 32), "decode_d256_4bit_32k_B16": (12, 4, 256, 4, 64),
                "decode_3bit_32k_B16": (32, 8, 128, 3, 32), "decode_3bit_tight_32k_B16": (32, 8, 128, 3, 32),
-               "decode_1bit_32k_B16": (32, 8, 128, 1, 32)}
+               "decode_1bit_32k_B16": (32, 8, 128, 1, 32), "decode_d64_4bit_32k_B16": (32, 8, 64, 4, 32),
+               "decode_d64_unpaired_4bit_32k_B16": (32, 8, 64, 4, 32)}
 _ROWS_NOTES = {"decode_d256_2bit_32k_B16": "matrix-unit decode kernel, head of 256 channels (two launches: the fp16 tail comes from the vector kernel, four runs)",
                "decode_d256_4bit_32k_B16": "matrix-unit decode kernel, head of 256 channels, four waves per CU",
                "decode_3bit_32k_B16": "3-bit codes in 4-bit fields (the cache's default): matrix-unit decode kernel",
                "decode_3bit_tight_32k_B16": "3-bit codes ten to a word (kivi_code_field='tight'): vector-unit kernel (attend_rows_kernel), four query rows of a kv head per block",
-               "decode_1bit_32k_B16": "1-bit codes in 2-bit fields (the cache's default): matrix-unit decode kernel"}
+               "decode_1bit_32k_B16": "1-bit codes in 2-bit fields (the cache's default): matrix-unit decode kernel",
+               "decode_d64_4bit_32k_B16": "heads of 64 channels (Llama-3.2-1B: 32 query / 8 kv heads), kv heads kept in pairs as heads of 128 channels (the cache's default): matrix-unit decode kernel, queries zero-padded into their half",
+               "decode_d64_unpaired_4bit_32k_B16": "heads of 64 channels, kivi_pair_heads=False: vector-unit kernel (attend_rows_kernel)"}
 
 
 def _decode_rows_case(torch, dev, name):
     """Decode outside the headline's head shape: the head size of config 2's model (Falcon3-7B: 12 query / 4 kv heads,
     D = 256) at 2 and 4 bits, on the matrix-unit kernel's 256-channel form, and 3-bit / 1-bit codes at the headline's
     head shape: in 4-bit / 2-bit fields on the matrix-unit kernel (the cache's default) and ten 3-bit codes to a word on
-    the vector kernel; batch 16, 32768 packed tokens plus the fp16 residual."""
+    the vector kernel; heads of 64 channels kept in pairs (the default) and singly; batch 16, 32768 packed tokens plus
+    the fp16 residual."""
     from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
     hq, hkv, d, bits, g = _ROWS_CASES[name]
     cfg = KVCacheConfig(method="kivi", head_dim=d, bit_width_inlier=bits, kivi_group_size=g, residual_length=128,
-                        fused_sdpa=True, fused_sdpa_memory_bound=True, kivi_code_field="tight" if "tight" in name else "auto")
+                        fused_sdpa=True, fused_sdpa_memory_bound=True, kivi_code_field="tight" if "tight" in name else "auto",
+                        kivi_pair_heads="unpaired" not in name)
     c = KVCacheFactory.create(cfg)
     for s0 in range(0, 32768 + 128, 8192):
         n = min(8192, 32768 + 128 - s0)

@@ -583,6 +583,92 @@ def test_odd_code_widths_in_the_next_even_field(bits, D, g, Hq, meta, tmp_path):
     assert torch.equal(c._tail_k[:, :, : c.offset - c._n_quantized], tight._tail_k[:, :, : c.offset - c._n_quantized])
 
 
+@pytest.mark.parametrize("bits,g,Hq,H,meta", [(4, 32, 32, 8, "float16"), (2, 64, 8, 2, "float32"), (2, 32, 14, 2, "float16"),
+                                              (4, 64, 12, 4, "float16"), (3, 32, 4, 4, "float32")])
+def test_heads_of_64_channels_are_kept_in_pairs(bits, g, Hq, H, meta):
+    """A memory-bound cache of 64-channel heads keeps kv heads 2m and 2m+1 as one head of 128 channels (the head size of
+    the matrix-unit kernels; queries zero-padded into their half): the stored codes are those of the unpaired cache, and
+    chunked prefill, decode across flushes, per-sequence lengths, a window, the saved state, a trim and the layer stack
+    agree with the oracle and with an unpaired cache (the vector kernel)."""
+    require_gpu()
+    from veloxquant_mlx_amd.cache import LayerStackedKIVICache
+    B, D, R = 2, 64, 64
+    kw = dict(head_dim=D, bit_width_inlier=bits, kivi_group_size=g, residual_length=R, fused_sdpa=True,
+              fused_sdpa_memory_bound=True, kivi_meta_dtype=meta)
+    c, plain = _make(**kw), _make(**kw, kivi_pair_heads=False)
+    stack = LayerStackedKIVICache(KVCacheConfig(method="kivi", **kw), 2)
+    n0, n1 = 600, 680
+    k, v = outlier_kv((B, H, n1, D), seed=bits * 10 + g + Hq)
+    rng = np.random.default_rng(Hq + g)
+    scale, levels = 1 / math.sqrt(D), (1 << bits) - 1
+    md = np.float16 if meta == "float16" else np.float32
+
+    def oracle(q, t_end, nq, **okw):
+        kq = ok.group_quant_codes(k[:, :, :nq], -2, g, levels)
+        vq = ok.group_quant_codes(v[:, :, :nq], -1, g, levels)
+        return oa.kivi_attend(q, kq[0], kq[1].astype(md), kq[2].astype(md), vq[0], vq[1].astype(md), vq[2].astype(md), g,
+                              k[:, :, nq:t_end], v[:, :, nq:t_end], scale, **okw)
+
+    # chunked prefill: every chunk attends causally over what is cached, itself included
+    for lo in range(0, n0, 200):
+        hi = min(lo + 200, n0)
+        for x in (c, plain, stack[0], stack[1]):
+            ret = x.update_and_fetch(to_dev(k[:, :, lo:hi]), to_dev(v[:, :, lo:hi]))
+        assert tuple(ret[0].shape) == (B, H, hi, D)
+        q = rng.standard_normal((B, Hq, hi - lo, D)).astype(np.float16)
+        got = host(c.fused_sdpa(to_dev(q), scale, causal=True)).astype(np.float32)
+        # (blocks of 256 query rows attend over the reconstruction rounded to fp16, as the reference's cache holds it)
+        ref = oracle(q, hi, c._n_quantized, causal=True)
+        assert float(np.max(np.abs(got - ref))) < 1e-2, (lo, float(np.max(np.abs(got - ref))))
+    assert c._pair and not plain._pair and c._shape_bhd == (B, H // 2, 128) and c._n_quantized == plain._n_quantized
+    assert c._kp.shape[1] == H // 2 and c._tail_k.shape[-1] == 128
+    # the stored codes: the paired head holds its two heads' channels side by side
+    nq = c._n_quantized
+    f = c._field
+    kd = K.kivi_dequant(c._kp, c._ks, c._kz, -2, g, f, nq, 128)
+    vd = K.kivi_dequant(c._vp, c._vs, c._vz, -1, g, f, nq, 128, v_layout=c._v_layout)
+    kp_ = K.kivi_dequant(plain._kp, plain._ks, plain._kz, -2, g, f, nq, D)
+    vp_ = K.kivi_dequant(plain._vp, plain._vs, plain._vz, -1, g, f, nq, D, v_layout=plain._v_layout)
+    unpair = lambda x: x.view(B, H // 2, nq, 2, D).transpose(2, 3).reshape(B, H, nq, D)
+    assert torch.equal(unpair(kd), kp_) and torch.equal(unpair(vd), vp_)
+
+    def step_checks(t_end):
+        q = rng.standard_normal((2, B, Hq, 1, D)).astype(np.float16)
+        got = host(c.fused_sdpa(to_dev(q[0]), scale)).astype(np.float32)
+        other = host(plain.fused_sdpa(to_dev(q[0]), scale)).astype(np.float32)
+        ref = oracle(q[0], t_end, c._n_quantized)
+        assert got.shape == (B, Hq, 1, D)
+        assert float(np.max(np.abs(got - ref))) < 2e-3 and float(np.max(np.abs(got - other))) < 2e-3, t_end
+        both = stack.fused_sdpa_all(to_dev(q), scale)
+        assert tuple(both.shape) == (2, B, Hq, 1, D)
+        assert float((both[0].float().cpu() - torch.from_numpy(got)).abs().max()) < 1e-3
+        assert float(np.max(np.abs(host(both[1]).astype(np.float32) - oracle(q[1], t_end, c._n_quantized)))) < 2e-3
+
+    for t in range(n0, n1):
+        for x in (c, plain, stack[0], stack[1]):
+            x.update_and_fetch(to_dev(k[:, :, t:t + 1]), to_dev(v[:, :, t:t + 1]))
+        if t % 11 == 0 or t == n1 - 1:
+            step_checks(t + 1)
+    # per-sequence lengths and a sliding window
+    q = rng.standard_normal((B, Hq, 1, D)).astype(np.float16)
+    lens = torch.tensor([n1 - 37, n1], dtype=torch.int32)
+    got = host(c.fused_sdpa(to_dev(q), scale, lengths=lens)).astype(np.float32)
+    other = host(plain.fused_sdpa(to_dev(q), scale, lengths=lens)).astype(np.float32)
+    assert float(np.max(np.abs(got - other))) < 2e-3
+    got = host(c.fused_sdpa(to_dev(q), scale, sliding_window=100)).astype(np.float32)
+    ref = oracle(q, n1, c._n_quantized, sliding_window=100)
+    assert float(np.max(np.abs(got - ref))) < 2e-3
+    # saved and restored (the rows of the state are the paired ones), then trimmed
+    r = type(c).from_state(KVCacheConfig(method="kivi", **kw), c.state, c.meta_state)
+    assert r._pair and r._shape_bhd == c._shape_bhd and r.offset == c.offset
+    assert torch.equal(r.fused_sdpa(to_dev(q), scale, fixed_order=True), c.fused_sdpa(to_dev(q), scale, fixed_order=True))
+    for x in (c, plain):
+        assert x.trim(100) == 100
+    got = host(c.fused_sdpa(to_dev(q), scale)).astype(np.float32)
+    other = host(plain.fused_sdpa(to_dev(q), scale)).astype(np.float32)
+    assert c.offset == plain.offset == n1 - 100 and float(np.max(np.abs(got - other))) < 2e-3
+
+
 @pytest.mark.parametrize("D,bits", [(64, 4), (256, 2), (128, 3)])
 def test_sink_protected_cache_on_the_other_decode_kernels(D, bits):
     """Protected rows where the attention kernel is the vector one (head size 64, 3-bit codes) or the 256-channel form of

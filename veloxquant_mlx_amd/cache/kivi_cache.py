@@ -33,6 +33,35 @@ from ._fp16_cache import FP16KVCache
 _META = {"float16": torch.float16, "float32": torch.float32}
 
 
+def pair_heads(x: torch.Tensor) -> torch.Tensor:
+    """``[..., H, S, D]`` -> ``[..., H/2, S, 2D]``: kv heads 2m and 2m+1 side by side in one head of twice the channels.
+    Group quantisation along tokens is per channel and along channels per group of ``g`` (``g`` divides ``D``), so the
+    codes, scale and zero of the paired head are those of the two heads."""
+    *lead, H, S, D = x.shape
+    return x.reshape(*lead, H // 2, 2, S, D).transpose(-3, -2).reshape(*lead, H // 2, S, 2 * D)
+
+
+def pad_queries_for_paired_heads(q: torch.Tensor, n_kv_heads: int, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``q [..., H_q, S_q, D]`` -> ``[..., H_q, S_q, 2D]`` for a cache of paired kv heads: a query head's channels in the
+    half of its own kv head, zeros in the other (``q . [k_a, k_b] = q . k_a``).  ``out``: a buffer of the result's
+    shape whose other halves are already zero."""
+    *lead, Hq, Sq, D = q.shape
+    R = Hq // n_kv_heads
+    if out is None:
+        out = q.new_zeros((*lead, Hq, Sq, 2 * D))
+    wide = out.view(*lead, n_kv_heads // 2, 2, R, Sq, 2, D).diagonal(dim1=-5, dim2=-2)      # [..., P, R, Sq, D, 2]
+    wide.copy_(q.reshape(*lead, n_kv_heads // 2, 2, R, Sq, D).movedim(-4, -1))
+    return out
+
+
+def own_half_of_paired_output(o: torch.Tensor, n_kv_heads: int) -> torch.Tensor:
+    """``o [..., H_q, S_q, 2D]`` (attention over paired kv heads) -> ``[..., H_q, S_q, D]``: every query head's own half."""
+    *lead, Hq, Sq, D2 = o.shape
+    R, D = Hq // n_kv_heads, D2 // 2
+    own = o.view(*lead, n_kv_heads // 2, 2, R, Sq, 2, D).diagonal(dim1=-5, dim2=-2)          # [..., P, R, Sq, D, 2]
+    return own.movedim(-1, -4).reshape(*lead, Hq, Sq, D)
+
+
 class KIVIKVCache(FP16KVCache):
     """KV cache with KIVI asymmetric group quantisation.
 
@@ -102,6 +131,13 @@ class KIVIKVCache(FP16KVCache):
                 f"KIVIKVCache: token-packed values need kivi_group_size % {per} == 0 at {self._field} bits a code.")
         self._v_layout = layout
         self._per = per
+        # heads of 64 channels, memory-bound mode: kv heads 2m and 2m+1 are kept side by side as one head of 128
+        # channels (same codes, scale and zero; queries zero-padded into their own half), the head size the
+        # matrix-unit kernels and the one-launch append take; decided at the first tokens (an even head count)
+        self._pair_wanted = (bool(getattr(config, "kivi_pair_heads", True)) and self._memory_bound and self._head_dim == 64
+                             and type(self) is KIVIKVCache and 64 % self._group_size == 0)
+        self._pair = False
+        self._q_pad = None
 
         # byte accounting (kivi_cache.py:132-146)
         self._key_bytes_compressed = 0
@@ -205,9 +241,19 @@ class KIVIKVCache(FP16KVCache):
         fp16 residual window, in ``kivi_group_size``-aligned blocks
         (kivi_cache.py:230-262)."""
         B, H, S, D = keys.shape
-        self._shape_bhd = (B, H, D)
         if self._memory_bound:
+            if self.offset == 0 and self._n_quantized == 0:
+                self._pair = self._pair_wanted and D == 64 and H % 2 == 0
+            if self._pair:
+                if D != 64 or H != 2 * self._shape_bhd[1] and self.offset > 0:
+                    raise ValueError(f"KIVIKVCache.update_and_fetch: this cache pairs kv heads of 64 channels, got {tuple(keys.shape)}")
+                self._shape_bhd = (B, H // 2, 2 * D)
+                self._update_memory_bound(pair_heads(keys), pair_heads(values))
+                z = self._zero_scalar
+                return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
+            self._shape_bhd = (B, H, D)
             return self._update_memory_bound(keys, values)
+        self._shape_bhd = (B, H, D)
         k_all, v_all = super().update_and_fetch(keys, values)
         new_boundary = self._quantization_boundary()
         n_quant_now = new_boundary - self._n_quantized
@@ -332,6 +378,16 @@ class KIVIKVCache(FP16KVCache):
                                "KVCacheConfig.fused_sdpa=True.")
         if self.offset == 0:
             raise RuntimeError("KIVIKVCache.fused_sdpa called before any tokens were cached via update_and_fetch.")
+        if self._pair and q.shape[-1] == 64:
+            H = 2 * self._shape_bhd[1]
+            if q.shape[1] % H:
+                raise ValueError(f"KIVIKVCache.fused_sdpa: {q.shape[1]} query heads over {H} kv heads")
+            key = (tuple(q.shape), q.dtype, q.device, K._stream_of(q.device))
+            if self._q_pad is None or self._q_pad[0] != key:   # the zero halves are written once
+                self._q_pad = (key, q.new_zeros((*q.shape[:-1], 128)))
+            wide = self.fused_sdpa(pad_queries_for_paired_heads(q, H, self._q_pad[1]), scale, causal=causal,
+                                   sliding_window=sliding_window, fixed_order=fixed_order, lengths=lengths, num_splits=num_splits)
+            return own_half_of_paired_output(wide, H)
         nq = self._n_quantized
         n_tail = self.offset - nq
         if q.shape[2] == 1:
@@ -504,7 +560,10 @@ class KIVIKVCache(FP16KVCache):
             packed, tail = v[2:], ()
         ref = packed[0] if packed else (tail[0] if tail else (v[0] if v else None))
         if ref is not None:
-            self._shape_bhd = (int(ref.shape[0]), int(ref.shape[1]), self._head_dim)
+            # rows of twice the head size: a state saved with paired heads
+            d = int((packed[1] if packed else ref).shape[-1])
+            self._pair = self._memory_bound and self._pair_wanted and d == 2 * self._head_dim
+            self._shape_bhd = (int(ref.shape[0]), int(ref.shape[1]), d if self._pair else self._head_dim)
         self._restore_packed(packed)
         if self._memory_bound:
             n_tail = int(tail[0].shape[2]) if tail else 0

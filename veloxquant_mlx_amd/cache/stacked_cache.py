@@ -23,7 +23,7 @@ from typing import Any
 import torch
 
 from .. import kernels as K
-from .kivi_cache import KIVIKVCache
+from .kivi_cache import KIVIKVCache, own_half_of_paired_output, pad_queries_for_paired_heads
 from .sink_cache import SinkProtectedKVCache
 
 _PACKED = ("_kp", "_ks", "_kz", "_vp", "_vs", "_vz")
@@ -51,6 +51,7 @@ class LayerStackedKIVICache:
         self._tails: list[tuple[torch.Tensor, torch.Tensor]] = []  # two pairs of [NL*B, H, cap, D] stacks
         self._lens = None   # (key, packed_lens, tail_lens) of the last ragged call
         self._sinks = None  # (key, (side_k, side_v, side_pos)) of the last call with protected rows
+        self._q_pad = None  # zero-padded queries of a stack of paired 64-channel heads
 
     @classmethod
     def from_layers(cls, layers) -> "LayerStackedKIVICache":
@@ -67,6 +68,7 @@ class LayerStackedKIVICache:
         self = cls.__new__(cls)
         self.layers = layers
         self._packed, self._tails, self._lens, self._sinks = None, [], None, None
+        self._q_pad = None
         return self
 
     def __len__(self) -> int:
@@ -187,6 +189,16 @@ class LayerStackedKIVICache:
         if q.ndim != 5 or q.shape[0] != NL:
             raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: q must be [NL={NL},B,H_q,S_q,D], got {tuple(q.shape)}")
         B = q.shape[1]
+        if self.layers[0]._pair and q.shape[-1] == 64:   # kv heads of 64 channels kept in pairs: see KIVIKVCache
+            H = 2 * self.layers[0]._shape_bhd[1]
+            if q.shape[2] % H:
+                raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: {q.shape[2]} query heads over {H} kv heads")
+            key = (tuple(q.shape), q.dtype, q.device, K._stream_of(q.device))
+            if self._q_pad is None or self._q_pad[0] != key:
+                self._q_pad = (key, q.new_zeros((*q.shape[:-1], 128)))
+            wide = self.fused_sdpa_all(pad_queries_for_paired_heads(q, H, self._q_pad[1]), scale, causal=causal,
+                                       sliding_window=sliding_window, fixed_order=fixed_order, num_splits=num_splits)
+            return own_half_of_paired_output(wide, H)
         for l, c in enumerate(self.layers):
             if c.offset == 0 or c._n_quantized == 0:
                 raise RuntimeError(f"LayerStackedKIVICache.fused_sdpa_all: layer {l} has no packed tokens yet")
