@@ -382,7 +382,10 @@ int vq_kivi_attend_fixed_order(int enable);
 /* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the shapes, pack_bits,
  * group, num_splits, sliding_window and sink_k are ignored).  0 for a launch that writes its output
  * itself (a prefill whose row tiles fill the GPU, one run per row, no protected rows): workspace may
- * then be NULL. */
+ * then be NULL.  A call with several query positions and a GQA group of 3, 5, 6 or 7 heads runs as
+ * the next group size the matrix-unit kernels tile (4 or 8: every group filled up with heads of
+ * zeros, whose rows are computed and dropped); its queries and outputs in that form are part of
+ * this figure, and the workspace must then be 256-byte aligned, q and out 16-byte aligned. */
 size_t vq_kivi_attend_workspace(const vq_attend_args *a);
 
 /* Reports what vq_kivi_attend would do for these arguments: *path = 0 for the

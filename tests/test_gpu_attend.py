@@ -329,7 +329,10 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
                                out_dtype=torch.float32, _plan_out=plan, **kw)
     if expect_path is not None:
         assert plan["path"] == expect_path, plan
-    if plan["path"] == 2 and (Hq // Hkv) * Sq >= 256:
+    # several positions of a GQA group of 3, 5, 6 or 7 heads run as the next group size the matrix unit tiles
+    R = Hq // Hkv
+    Rp = R if Sq == 1 or R in (1, 2, 4) or R >= 8 or plan["path"] not in (1, 2) else (4 if R == 3 else 8)
+    if plan["path"] == 2 and Rp * Sq >= 256:
         # the same call fed with ready-made tiles (written in two parts, into a buffer that starts out as NaNs
         # and has spare room) runs the same arithmetic on the same numbers: identical bits
         units = -(-(n_packed + n_tail) // 32)
@@ -367,7 +370,7 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
                          sliding_window=window)
     err = float(np.max(np.abs(host(out) - ref)))
     print(f"max-abs err {err:.2e} (path {plan['path']}, {plan['nparts']} partials)")
-    if plan["path"] == 2 and (Hq // Hkv) * Sq >= 256:
+    if plan["path"] == 2 and Rp * Sq >= 256:
         # The 256-row prefill blocks attend over the reconstruction rounded to fp16, which is
         # what the reference's cache holds (kivi_cache.py:198-201): that is the oracle at the
         # usual tolerance; against the float32 reconstruction the rounding of keys and values
@@ -491,9 +494,9 @@ def test_mfma_decode_head_size_256(b, g, meta, Hq, Hkv):
     _packed_case(2, Hq, Hkv, 1024, 37, 256, b, g, "token", meta, seed=Hq + g + b, expect_path=1)
     _packed_case(1, Hq, Hkv, 2048 + 128, 0, 256, b, g, "token", meta, seed=Hq + g + b + 1, expect_path=1, cap_extra=128)
     # several positions a tile: groups of 1, 2, 4 heads (8 / R positions), or eight heads of a larger group; a group of
-    # three heads at several positions is the vector kernel's
+    # three heads at several positions runs as a group of four
     _packed_case(1, Hq, Hkv, 640, 70, 256, b, g, "token", meta, Sq=3, causal=True, seed=Hq + g + b + 2,
-                 expect_path=3 if Hq // Hkv == 3 else 1, tail_dtype=torch.bfloat16, window=500)
+                 expect_path=1, tail_dtype=torch.bfloat16, window=500)
 
 
 def test_mfma_decode_head_size_256_long_context_and_float32_tail():
@@ -558,9 +561,24 @@ def test_mfma_prefill_not_causal_and_split_tokens():
     _packed_case(1, 8, 2, 2048, 100, 128, 4, 64, "token", torch.float16, Sq=6, causal=True, seed=22, expect_path=1)
 
 
-def test_mfma_prefill_odd_head_ratio_takes_vector_kernel():
-    _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=4, causal=True, seed=23, expect_path=3)
+def test_odd_head_ratios_run_as_the_next_group_size_the_matrix_unit_tiles():
+    """Several query positions of a GQA group of 3, 5, 6 or 7 heads (Llama-3.2-3B: 24 / 8, Qwen2.5-7B: 28 / 4): the
+    library fills every group up to 4 or 8 heads with rows of zeros in its workspace, runs the matrix-unit kernel of that
+    group size and drops those rows; a single position takes the decode kernel as it is."""
+    _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=4, causal=True, seed=23, expect_path=1)
     _packed_case(1, 6, 2, 128, 10, 128, 4, 32, "token", torch.float16, Sq=1, seed=24, expect_path=1)
+    _packed_case(2, 24, 8, 512, 70, 128, 4, 32, "token", torch.float16, Sq=100, causal=True, seed=25, expect_path=2)   # 256-row blocks
+    _packed_case(2, 6, 2, 512, 70, 128, 2, 64, "token", torch.float16, Sq=20, causal=True, seed=26, expect_path=2)     # 64-row blocks
+    _packed_case(1, 6, 2, 512, 40, 128, 4, 32, "token", torch.float32, Sq=30, causal=True, seed=27, expect_path=1)     # float32 scale / zero
+    _packed_case(1, 28, 4, 1024, 150, 128, 2, 32, "token", torch.float16, Sq=64, causal=True, seed=28, expect_path=2,
+                 q_dtype=torch.bfloat16)
+    _packed_case(1, 10, 2, 384, 33, 128, 4, 64, "token", torch.float16, Sq=40, causal=True, seed=29, expect_path=2, window=100)
+    _packed_case(2, 12, 2, 256, 0, 128, 4, 32, "token", torch.float16, Sq=17, causal=False, seed=30, expect_path=2)
+    _packed_case(1, 12, 4, 0, 400, 128, 4, 32, "token", torch.float16, Sq=400, causal=True, seed=31, expect_path=2)    # plain keys and values
+    _packed_case(1, 12, 4, 640, 70, 256, 2, 32, "token", torch.float16, Sq=3, causal=True, seed=32, expect_path=1)     # heads of 256 channels
+    _packed_case(1, 5, 1, 256, 12, 128, 4, 32, "token", torch.float16, Sq=2, causal=True, seed=33, expect_path=1)
+    # what the matrix-unit kernels refuse at any group size stays on the vector kernel
+    _packed_case(1, 6, 2, 128, 10, 128, 3, 32, "channel", torch.float16, Sq=4, causal=True, seed=34, expect_path=3)
 
 
 def test_mfma_path_takes_bf16_tails():

@@ -433,7 +433,7 @@ class KIVIKVCache(FP16KVCache):
         H = self._shape_bhd[1]
         nq, n_tail = kw["n_packed"], kw["n_tail"]
         if not (self.prefill_tiles and self._memory_bound and self._v_layout == "token" and D == 128 and Hq % H == 0
-                and Hq // H in (1, 2, 4, 8) and (Hq // H) * Sq >= 256 and nq % 32 == 0 and "sinks" not in kw
+                and 1 <= Hq // H <= 8 and (Hq // H) * Sq >= 256 and nq % 32 == 0 and "sinks" not in kw
                 and (n_tail == 0 or self._tail_k.dtype in (torch.float16, torch.bfloat16))):
             return False
         units = -(-(nq + n_tail) // 32)

@@ -173,6 +173,46 @@ static int validate(const vq_attend_args *a, const char *fn) {
     return VQ_OK;
 }
 
+// Several query positions of a GQA group of 3, 5, 6 or 7 heads: the matrix-unit kernels tile groups of 1, 2, 4
+// and 8 (or more) heads.  Such a call runs as the next of those sizes -- every kv head's group filled up with
+// heads of zeros, whose rows are computed and dropped -- when that takes a matrix-unit path and the call as given
+// does not.  Returns the padded group size, 0 when the call runs as it is.
+static int64_t padded_group(const vq_attend_args &a) {
+    if (a.Sq < 2 || a.Hkv < 1 || a.Hq % a.Hkv != 0 || a.k_new != nullptr || a.num_splits < 0) return 0;
+    const int64_t R = a.Hq / a.Hkv;
+    if (R == 1 || R == 2 || R == 4 || R >= 8) return 0;
+    if ((a.Sq * a.D * (a.q_dtype == VQ_F32 ? 4 : 2)) % 16 != 0 || (a.Sq * a.D * (a.out_dtype == VQ_F32 ? 4 : 2)) % 16 != 0) return 0;
+    if ((((uintptr_t)a.q | (uintptr_t)a.out) & 15u) != 0) return 0;
+    const int path = plan_attend(a).path;
+    if (path == 1 || path == 2) return 0;
+    vq_attend_args b = a;
+    b.Hq = a.Hkv * (R == 3 ? 4 : 8);
+    b.q = nullptr;   // stands for a 256-byte aligned buffer
+    const int padded = plan_attend(b).path;
+    return padded == 1 || padded == 2 ? b.Hq / a.Hkv : 0;
+}
+
+static size_t round256(size_t n) { return (n + 255) / 256 * 256; }
+
+// rows of `row16` 16-byte pieces: group g of R_to rows takes its first R_from rows from group g of R_from rows of
+// `src` and zeros after them (R_from < R_to: queries), or keeps the first R_to of R_from rows (outputs)
+__global__ void regroup_rows_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t groups, int R_from,
+                                    int R_to, int64_t row16) {
+    const int64_t n = groups * R_to * row16;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t c = e % row16, r = (e / row16) % R_to, g = e / (row16 * R_to);
+        dst[e] = r < R_from ? src[(g * R_from + r) * row16 + c] : make_uint4(0u, 0u, 0u, 0u);
+    }
+}
+
+static void launch_regroup(const void *src, void *dst, int64_t groups, int64_t R_from, int64_t R_to, int64_t row_bytes,
+                           hipStream_t st) {
+    const int64_t n = groups * R_to * (row_bytes / 16);
+    const int64_t blocks = cdiv(n, 256);
+    hipLaunchKernelGGL(regroup_rows_kernel, dim3((unsigned)(blocks < 65535 * 16 ? blocks : 65535 * 16)), dim3(256), 0, st,
+                       (const uint4 *)src, (uint4 *)dst, groups, (int)R_from, (int)R_to, row_bytes / 16);
+}
+
 }  // namespace vq
 
 using namespace vq;
@@ -187,6 +227,15 @@ extern "C" size_t vq_kivi_attend_workspace(const vq_attend_args *a) {
         a->n_packed < 0 || a->n_tail < 0 || (a->n_packed > 0 && (a->pack_bits < 1 || a->pack_bits > 8 || a->group < 1)))
         return 0;
     const vq_attend_args w = skip_below_window(*a);
+    if (const int64_t Rp = padded_group(w)) {
+        // the padded call's own workspace, then its queries and its outputs
+        vq_attend_args b = *a;
+        b.Hq = a->Hkv * Rp;
+        b.q = nullptr;
+        const size_t rows = (size_t)(b.B * b.Hq * b.Sq) * (size_t)b.D;
+        return round256(vq_kivi_attend_workspace(&b)) + round256(rows * (a->q_dtype == VQ_F32 ? 4 : 2)) +
+               round256(rows * (a->out_dtype == VQ_F32 ? 4 : 2));
+    }
     AttendPlan p = plan_attend(w);
     if (p.path == 2 && mfma_prefill_direct_output(w, p.nparts)) return 0;   // the kernel writes `out` itself
     return (size_t)(a->B * a->Hq * a->Sq) * (size_t)p.nparts * (size_t)(a->D + 2) * sizeof(float);
@@ -212,7 +261,12 @@ extern "C" int vq_kivi_prefill_tiles(const vq_attend_args *a, int64_t first_unit
 extern "C" int vq_kivi_attend_plan(const vq_attend_args *a, int *path, int *nparts) {
     int rc = validate(a, "vq_kivi_attend_plan");
     if (rc != VQ_OK) return rc;
-    AttendPlan p = plan_attend(skip_below_window(*a));
+    vq_attend_args w = skip_below_window(*a);
+    if (const int64_t Rp = padded_group(w)) {   // the plan of the call that runs
+        w.Hq = w.Hkv * Rp;
+        w.q = nullptr;
+    }
+    AttendPlan p = plan_attend(w);
     if (path) *path = p.path;
     if (nparts) *nparts = p.nparts;
     return VQ_OK;
@@ -236,6 +290,32 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         VQ_REQUIRE(a->n_tail >= 1, VQ_ERR_INVALID, "%s: k_new / v_new fill the last tail row, so n_tail must be >= 1", fn);
         VQ_REQUIRE((((uintptr_t)a->k_new | (uintptr_t)a->v_new) & 15u) == 0, VQ_ERR_UNSUPPORTED,
                    "%s: k_new / v_new must be 16-byte aligned", fn);
+    }
+    if (const int64_t Rp = padded_group(*a)) {
+        const size_t need = vq_kivi_attend_workspace(a_in);
+        VQ_REQUIRE(a_in->workspace != nullptr && a_in->workspace_bytes >= need, VQ_ERR_WORKSPACE,
+                   "%s: workspace of %zu bytes required, %zu given", fn, need, a_in->workspace_bytes);
+        VQ_REQUIRE(((uintptr_t)a_in->workspace & 255u) == 0, VQ_ERR_INVALID, "%s: the workspace must be 256-byte aligned", fn);
+        const int64_t R = a_in->Hq / a_in->Hkv;
+        vq_attend_args b = *a_in;   // the arguments as given: the inner call cuts the window itself
+        b.Hq = a_in->Hkv * Rp;
+        b.q = nullptr;
+        const size_t inner = round256(vq_kivi_attend_workspace(&b));
+        const size_t rows = (size_t)(b.B * b.Hq * b.Sq) * (size_t)b.D;
+        char *base = static_cast<char *>(a_in->workspace);
+        void *q_wide = base + inner;
+        void *out_wide = base + inner + round256(rows * (a_in->q_dtype == VQ_F32 ? 4 : 2));
+        b.q = q_wide;
+        b.out = out_wide;
+        b.workspace_bytes = inner;
+        hipStream_t st = (hipStream_t)a_in->stream;
+        launch_regroup(a_in->q, q_wide, a_in->B * a_in->Hkv, R, Rp, a_in->Sq * a_in->D * (a_in->q_dtype == VQ_F32 ? 4 : 2), st);
+        VQ_HIP_CHECK_LAUNCH(fn);
+        rc = vq_kivi_attend(&b);
+        if (rc != VQ_OK) return rc;
+        launch_regroup(out_wide, a_in->out, a_in->B * a_in->Hkv, Rp, R, a_in->Sq * a_in->D * (a_in->out_dtype == VQ_F32 ? 4 : 2), st);
+        VQ_HIP_CHECK_LAUNCH(fn);
+        return VQ_OK;
     }
     AttendPlan p = plan_attend(*a);
     if (a->k_new != nullptr)
@@ -318,7 +398,12 @@ extern "C" int vq_kivi_attend_static(const vq_attend_args *a) {
     VQ_REQUIRE(need <= STATIC_WS_BYTES, VQ_ERR_WORKSPACE,
                "%s: these shapes need %zu bytes of split partials, the built-in scratch holds %zu; use vq_kivi_attend "
                "with a workspace of its own", fn, need, STATIC_WS_BYTES);
-    const AttendPlan p = plan_attend(skip_below_window(*a));
+    vq_attend_args w = skip_below_window(*a);
+    if (const int64_t Rp = padded_group(w)) {   // the call that runs: its GQA groups filled up
+        w.Hq = w.Hkv * Rp;
+        w.q = nullptr;
+    }
+    const AttendPlan p = plan_attend(w);
     VQ_REQUIRE((size_t)(a->B * a->Hkv * p.tiles) <= STATIC_COUNTERS, VQ_ERR_WORKSPACE,
                "%s: B * H_kv * row tiles = %lld exceeds the %zu built-in sync counters", fn,
                (long long)(a->B * a->Hkv * p.tiles), STATIC_COUNTERS);

@@ -1004,7 +1004,7 @@ def kivi_packed_attend(q: torch.Tensor, *, k_packed=None, k_scale=None, k_zero=N
         a.sink_k, a.sink_v, a.sink_pos = sk.data_ptr(), sv.data_ptr(), sp.data_ptr()
         a.sink_cap, a.sink_dtype = int(cap_s), _FLOAT_TAG[sk.dtype]
         keep += [sk, sv, sp]
-    if (tiles is None and n_packed == 0 and causal and D == 128 and Hq % Hkv == 0 and Hq // Hkv in (1, 2, 4, 8)
+    if (tiles is None and n_packed == 0 and causal and D == 128 and Hq % Hkv == 0 and 1 <= Hq // Hkv <= 8
             and (Hq // Hkv) * Sq >= 24 * 256 and k_tail.dtype in (torch.float16, torch.bfloat16)
             and packed_lens is None and sinks is None and k_new is None and not static_scratch
             and B * Hkv * -(-int(n_tail) // 32) * PREFILL_TILE_BYTES <= _TILE_SCRATCH_MAX):
