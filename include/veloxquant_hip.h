@@ -384,7 +384,8 @@ int vq_kivi_attend_fixed_order(int enable);
  * itself (a prefill whose row tiles fill the GPU, one run per row, no protected rows): workspace may
  * then be NULL.  A call with several query positions and a GQA group of 3, 5, 6 or 7 heads runs as
  * the next group size the matrix-unit kernels tile (4 or 8: every group filled up with heads of
- * zeros, whose rows are computed and dropped); its queries and outputs in that form are part of
+ * zeros, whose rows are computed and dropped), a prefill-sized one with more than eight heads a
+ * group as passes of eight heads; its queries and outputs in that form are part of
  * this figure, and the workspace must then be 256-byte aligned, q and out 16-byte aligned. */
 size_t vq_kivi_attend_workspace(const vq_attend_args *a);
 

@@ -331,7 +331,8 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
         assert plan["path"] == expect_path, plan
     # several positions of a GQA group of 3, 5, 6 or 7 heads run as the next group size the matrix unit tiles
     R = Hq // Hkv
-    Rp = R if Sq == 1 or R in (1, 2, 4) or R >= 8 or plan["path"] not in (1, 2) else (4 if R == 3 else 8)
+    # (and prefill-sized calls with more than eight heads a group as passes of eight heads)
+    Rp = R if Sq == 1 or R in (1, 2, 4, 8) or plan["path"] not in (1, 2) else (4 if R == 3 else 8)
     if plan["path"] == 2 and Rp * Sq >= 256:
         # the same call fed with ready-made tiles (written in two parts, into a buffer that starts out as NaNs
         # and has spare room) runs the same arithmetic on the same numbers: identical bits
@@ -579,6 +580,12 @@ def test_odd_head_ratios_run_as_the_next_group_size_the_matrix_unit_tiles():
     _packed_case(1, 5, 1, 256, 12, 128, 4, 32, "token", torch.float16, Sq=2, causal=True, seed=33, expect_path=1)
     # what the matrix-unit kernels refuse at any group size stays on the vector kernel
     _packed_case(1, 6, 2, 128, 10, 128, 3, 32, "channel", torch.float16, Sq=4, causal=True, seed=34, expect_path=3)
+    # more than eight heads a group at prefill size: eight at a time through the prefill blocks, the last pass filled up
+    _packed_case(1, 32, 2, 512, 70, 128, 4, 32, "token", torch.float16, Sq=100, causal=True, seed=35, expect_path=2)
+    _packed_case(2, 14, 1, 384, 33, 128, 2, 64, "token", torch.float32, Sq=40, causal=True, seed=36, expect_path=2, window=200)
+    _packed_case(1, 18, 2, 256, 0, 128, 4, 64, "token", torch.float16, Sq=16, causal=False, seed=37, expect_path=2)
+    _packed_case(1, 24, 2, 0, 300, 128, 4, 32, "token", torch.float16, Sq=300, causal=True, seed=38, expect_path=2)
+    _packed_case(1, 32, 2, 512, 70, 128, 4, 32, "token", torch.float16, Sq=6, causal=True, seed=39, expect_path=1)   # a few positions: the decode tiles
 
 
 def test_mfma_path_takes_bf16_tails():

@@ -432,8 +432,10 @@ class KIVIKVCache(FP16KVCache):
         B, Hq, Sq, D = q.shape
         H = self._shape_bhd[1]
         nq, n_tail = kw["n_packed"], kw["n_tail"]
+        R = Hq // max(H, 1)
+        rows = (R if R in (1, 2, 4) else 4 if R == 3 else 8) * Sq   # a block's rows: the library runs groups of 1, 2, 4, 8 heads
         if not (self.prefill_tiles and self._memory_bound and self._v_layout == "token" and D == 128 and Hq % H == 0
-                and 1 <= Hq // H <= 8 and (Hq // H) * Sq >= 256 and nq % 32 == 0 and "sinks" not in kw
+                and rows >= 256 and nq % 32 == 0 and "sinks" not in kw
                 and (n_tail == 0 or self._tail_k.dtype in (torch.float16, torch.bfloat16))):
             return False
         units = -(-(nq + n_tail) // 32)

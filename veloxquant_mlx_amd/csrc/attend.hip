@@ -176,41 +176,50 @@ static int validate(const vq_attend_args *a, const char *fn) {
 // Several query positions of a GQA group of 3, 5, 6 or 7 heads: the matrix-unit kernels tile groups of 1, 2, 4
 // and 8 (or more) heads.  Such a call runs as the next of those sizes -- every kv head's group filled up with
 // heads of zeros, whose rows are computed and dropped -- when that takes a matrix-unit path and the call as given
-// does not.  Returns the padded group size, 0 when the call runs as it is.
+// does not.  A prefill-sized call with more than eight heads a group runs eight of them at a time through the prefill
+// blocks (one pass per eight heads, the last filled up) instead of one position a tile through the decode kernel.
+// Returns the group size of the calls that run, 0 when the call runs as it is.
 static int64_t padded_group(const vq_attend_args &a) {
     if (a.Sq < 2 || a.Hkv < 1 || a.Hq % a.Hkv != 0 || a.k_new != nullptr || a.num_splits < 0) return 0;
     const int64_t R = a.Hq / a.Hkv;
-    if (R == 1 || R == 2 || R == 4 || R >= 8) return 0;
+    if (R == 1 || R == 2 || R == 4 || R == 8) return 0;
     if ((a.Sq * a.D * (a.q_dtype == VQ_F32 ? 4 : 2)) % 16 != 0 || (a.Sq * a.D * (a.out_dtype == VQ_F32 ? 4 : 2)) % 16 != 0) return 0;
     if ((((uintptr_t)a.q | (uintptr_t)a.out) & 15u) != 0) return 0;
     const int path = plan_attend(a).path;
-    if (path == 1 || path == 2) return 0;
     vq_attend_args b = a;
-    b.Hq = a.Hkv * (R == 3 ? 4 : 8);
     b.q = nullptr;   // stands for a 256-byte aligned buffer
+    if (R > 8) {
+        if (a.Sq < 16 || path == 2) return 0;
+        b.Hq = a.Hkv * 8;
+        return plan_attend(b).path == 2 ? 8 : 0;
+    }
+    if (path == 1 || path == 2) return 0;
+    b.Hq = a.Hkv * (R == 3 ? 4 : 8);
     const int padded = plan_attend(b).path;
     return padded == 1 || padded == 2 ? b.Hq / a.Hkv : 0;
 }
 
 static size_t round256(size_t n) { return (n + 255) / 256 * 256; }
 
-// rows of `row16` 16-byte pieces: group g of R_to rows takes its first R_from rows from group g of R_from rows of
-// `src` and zeros after them (R_from < R_to: queries), or keeps the first R_to of R_from rows (outputs)
-__global__ void regroup_rows_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t groups, int R_from,
-                                    int R_to, int64_t row16) {
-    const int64_t n = groups * R_to * row16;
+// rows of `row16` 16-byte pieces, in groups of R_src (src) and R_dst (dst) rows: rows [dst_off, dst_off + n_write) of
+// every dst group become rows [src_off, src_off + n_write) of the same src group, zeros from the n_valid-th on
+__global__ void regroup_rows_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t groups, int R_src,
+                                    int src_off, int R_dst, int dst_off, int n_write, int n_valid, int64_t row16) {
+    const int64_t n = groups * n_write * row16;
     for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (int64_t)gridDim.x * blockDim.x) {
-        const int64_t c = e % row16, r = (e / row16) % R_to, g = e / (row16 * R_to);
-        dst[e] = r < R_from ? src[(g * R_from + r) * row16 + c] : make_uint4(0u, 0u, 0u, 0u);
+        const int64_t c = e % row16, r = (e / row16) % n_write, g = e / (row16 * n_write);
+        dst[(g * R_dst + dst_off + r) * row16 + c] =
+            r < n_valid ? src[(g * R_src + src_off + r) * row16 + c] : make_uint4(0u, 0u, 0u, 0u);
     }
 }
 
-static void launch_regroup(const void *src, void *dst, int64_t groups, int64_t R_from, int64_t R_to, int64_t row_bytes,
-                           hipStream_t st) {
-    const int64_t n = groups * R_to * (row_bytes / 16);
+static void launch_regroup(const void *src, void *dst, int64_t groups, int64_t R_src, int64_t src_off, int64_t R_dst,
+                           int64_t dst_off, int64_t n_write, int64_t n_valid, int64_t row_bytes, hipStream_t st) {
+    const int64_t n = groups * n_write * (row_bytes / 16);
     const int64_t blocks = cdiv(n, 256);
     hipLaunchKernelGGL(regroup_rows_kernel, dim3((unsigned)(blocks < 65535 * 16 ? blocks : 65535 * 16)), dim3(256), 0, st,
-                       (const uint4 *)src, (uint4 *)dst, groups, (int)R_from, (int)R_to, row_bytes / 16);
+                       (const uint4 *)src, (uint4 *)dst, groups, (int)R_src, (int)src_off, (int)R_dst, (int)dst_off,
+                       (int)n_write, (int)n_valid, row_bytes / 16);
 }
 
 }  // namespace vq
@@ -309,12 +318,19 @@ extern "C" int vq_kivi_attend(const vq_attend_args *a_in) {
         b.out = out_wide;
         b.workspace_bytes = inner;
         hipStream_t st = (hipStream_t)a_in->stream;
-        launch_regroup(a_in->q, q_wide, a_in->B * a_in->Hkv, R, Rp, a_in->Sq * a_in->D * (a_in->q_dtype == VQ_F32 ? 4 : 2), st);
-        VQ_HIP_CHECK_LAUNCH(fn);
-        rc = vq_kivi_attend(&b);
-        if (rc != VQ_OK) return rc;
-        launch_regroup(out_wide, a_in->out, a_in->B * a_in->Hkv, Rp, R, a_in->Sq * a_in->D * (a_in->out_dtype == VQ_F32 ? 4 : 2), st);
-        VQ_HIP_CHECK_LAUNCH(fn);
+        const int64_t groups = a_in->B * a_in->Hkv;
+        const int64_t q_row = a_in->Sq * a_in->D * (a_in->q_dtype == VQ_F32 ? 4 : 2);
+        const int64_t out_row = a_in->Sq * a_in->D * (a_in->out_dtype == VQ_F32 ? 4 : 2);
+        for (int64_t first = 0; first < R; first += Rp) {   // one pass for groups of up to eight heads
+            const int64_t n_valid = R - first < Rp ? R - first : Rp;
+            launch_regroup(a_in->q, q_wide, groups, R, first, Rp, 0, Rp, n_valid, q_row, st);
+            VQ_HIP_CHECK_LAUNCH(fn);
+            rc = vq_kivi_attend(&b);
+            if (rc != VQ_OK) return rc;
+            launch_regroup(out_wide, a_in->out, groups, Rp, 0, R, first, n_valid, n_valid, out_row, st);
+            VQ_HIP_CHECK_LAUNCH(fn);
+            b.tiles_stale_from = b.tile_cap;   // the first pass has brought the tiles up to date
+        }
         return VQ_OK;
     }
     AttendPlan p = plan_attend(*a);
