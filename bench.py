@@ -352,12 +352,11 @@ def _decode_cfg1_case(torch, dev):
     return c, (lambda: c.fused_sdpa(q, 1 / math.sqrt(D))), nbytes
 
 
-def _prefill_case(torch, dev):
+def _prefill_case(torch, dev, Hq=32, Hkv=8, D=128):
     """Config 4: 8 chunks of 512 bf16 queries over a 4-bit packed prefix of 4096 tokens plus their own,
     quantise-on-write (group 32, residual 128).  Returns a function that runs one whole pass and
     gives its milliseconds."""
     from veloxquant_mlx_amd.cache import KVCacheConfig, KVCacheFactory
-    D, Hq, Hkv = 128, 32, 8
 
     def prefill_pass():
         cfg = KVCacheConfig(method="kivi", head_dim=D, bit_width_inlier=4, kivi_group_size=32, residual_length=128,
@@ -610,6 +609,18 @@ def _extras(torch, K, dev):
                           "frac_mfma_f16_peak": round(flops / ms / 1e9 / MFMA_F16_PEAK_TFLOPS, 4), "flops": flops,
                           "note": "8 chunks of 512 queries: quantise-on-write append + attention per chunk; "
                                   "the packed store is sized once by fused_sdpa_max_ctx=8192"}
+    # config 4's pass at the head counts of other models of the reference's scripts: GQA groups the matrix-unit kernels do
+    # not tile run filled up to the next size that they do, 64-channel heads in pairs, 256-channel heads in 128-row blocks
+    for tag, hq, hkv, d, note in (
+            ("24q_8kv", 24, 8, 128, "Llama-3.2-3B: groups of 3 run as groups of 4"),
+            ("28q_4kv", 28, 4, 128, "Qwen2.5-7B: groups of 7 run as groups of 8"),
+            ("32q_8kv_d64", 32, 8, 64, "Llama-3.2-1B: kv heads of 64 channels in pairs, groups of 8"),
+            ("12q_4kv_d256", 12, 4, 256, "Falcon3-7B: heads of 256 channels, 128-row blocks, one launch per half of the output's channels; groups of 3 run as groups of 4")):
+        run_ = _prefill_case(torch, dev, hq, hkv, d)
+        run_()
+        ms_ = min(run_() for _ in range(3))
+        fl_ = flops * hq * d // (32 * 128)
+        ex[f"prefill_cfg4_{tag}"] = {"ms": round(ms_, 4), "TFLOPs": round(fl_ / ms_ / 1e9, 1), "flops": fl_, "note": note}
     # causal attention over plain fp16 K/V (the reference's flash-prefill shape: 32 heads, D 128, S_q = S_kv)
     for S in (2048, 8192):
         fn, flops = _flash_prefill_case(torch, K, dev, S)

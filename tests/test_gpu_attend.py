@@ -333,7 +333,8 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
     R = Hq // Hkv
     # (and prefill-sized calls with more than eight heads a group as passes of eight heads)
     Rp = R if Sq == 1 or R in (1, 2, 4, 8) or plan["path"] not in (1, 2) else (4 if R == 3 else 8)
-    if plan["path"] == 2 and Rp * Sq >= 256:
+    row_blocks = plan["path"] == 2 and Rp * Sq >= (128 if D == 256 else 256)   # the blocks of eight waves
+    if row_blocks and D == 128:
         # the same call fed with ready-made tiles (written in two parts, into a buffer that starts out as NaNs
         # and has spare room) runs the same arithmetic on the same numbers: identical bits
         units = -(-(n_packed + n_tail) // 32)
@@ -371,7 +372,7 @@ def _packed_case(B, Hq, Hkv, n_packed, n_tail, D, b, g, v_layout, meta, Sq=1, ca
                          sliding_window=window)
     err = float(np.max(np.abs(host(out) - ref)))
     print(f"max-abs err {err:.2e} (path {plan['path']}, {plan['nparts']} partials)")
-    if plan["path"] == 2 and Rp * Sq >= 256:
+    if row_blocks:
         # The 256-row prefill blocks attend over the reconstruction rounded to fp16, which is
         # what the reference's cache holds (kivi_cache.py:198-201): that is the oracle at the
         # usual tolerance; against the float32 reconstruction the rounding of keys and values
@@ -498,6 +499,24 @@ def test_mfma_decode_head_size_256(b, g, meta, Hq, Hkv):
     # three heads at several positions runs as a group of four
     _packed_case(1, Hq, Hkv, 640, 70, 256, b, g, "token", meta, Sq=3, causal=True, seed=Hq + g + b + 2,
                  expect_path=1, tail_dtype=torch.bfloat16, window=500)
+
+
+def test_mfma_prefill_head_size_256():
+    """Prefill-sized calls at a head size of 256 (Falcon3-7B 12 / 4, gemma-3 8 / 4): blocks of 128 rows, eight k-steps of
+    scores, one launch per half of the output's channels; against the oracle over the reconstruction rounded to fp16."""
+    _packed_case(1, 12, 4, 640, 70, 256, 2, 32, "token", torch.float16, Sq=100, causal=True, seed=51, expect_path=2)    # groups of 3 as 4
+    _packed_case(2, 8, 4, 512, 100, 256, 4, 64, "token", torch.float16, Sq=64, causal=True, seed=52, expect_path=2)
+    _packed_case(1, 8, 1, 1024, 37, 256, 4, 128, "token", torch.float16, Sq=200, causal=True, seed=53, expect_path=2, window=300)
+    _packed_case(1, 4, 4, 256, 0, 256, 2, 64, "token", torch.float16, Sq=130, causal=False, seed=54, expect_path=2)
+    _packed_case(1, 8, 2, 0, 300, 256, 4, 32, "token", torch.float16, Sq=300, causal=True, seed=55, expect_path=2)      # plain keys and values
+    _packed_case(1, 8, 2, 384, 90, 256, 2, 32, "token", torch.float16, Sq=80, causal=True, seed=56, expect_path=2,
+                 q_dtype=torch.bfloat16, tail_dtype=torch.bfloat16)
+    _packed_case(1, 4, 1, 4096, 0, 256, 4, 32, "token", torch.float16, Sq=32, causal=True, seed=57, expect_path=2)      # one tile, eight runs
+    _packed_case(1, 8, 2, 512, 33, 256, 4, 32, "token", torch.float16, Sq=50, causal=True, seed=58, expect_path=2,
+                 q_dtype=torch.float32)
+    # float32 scale / zero and fewer than 128 rows a kv head stay on the decode kernel's tiles
+    _packed_case(1, 8, 2, 512, 33, 256, 4, 32, "token", torch.float32, Sq=50, causal=True, seed=59, expect_path=1)
+    _packed_case(1, 8, 4, 512, 33, 256, 4, 32, "token", torch.float16, Sq=20, causal=True, seed=60, expect_path=1)
 
 
 def test_mfma_decode_head_size_256_long_context_and_float32_tail():

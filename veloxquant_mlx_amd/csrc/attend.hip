@@ -27,7 +27,7 @@ AttendPlan plan_attend(const vq_attend_args &a) {
         const int rows = mfma_prefill_block_rows(a);
         const int64_t blocks = a.B * a.Hkv * cdiv(a.Sq, rows / (a.Hq / a.Hkv));
         const int64_t work = cdiv(a.n_packed + a.n_tail, 32);
-        int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(rows == 256 ? 256 : 512, blocks);
+        int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(rows != 64 ? 256 : 512, blocks);
         if (ns > 8) ns = 8;
         if (ns > work) ns = work;
         if (ns < 1) ns = 1;

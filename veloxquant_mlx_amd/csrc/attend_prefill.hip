@@ -489,7 +489,7 @@ __device__ __forceinline__ f16x8 recon8(f16x8 c, const Meta8<float> &s, const Me
 
 // one run per row, nothing to patch afterwards, 256-row blocks: the kernel writes `out`, no merge launch follows
 __host__ __device__ inline bool mfma_prefill_writes_output(const vq_attend_args &a, int nparts) {
-    return nparts == 1 && a.sink_k == nullptr && (a.Hq / a.Hkv) * a.Sq >= 256;
+    return nparts == 1 && a.sink_k == nullptr && (a.Hq / a.Hkv) * a.Sq >= (a.D == 2 * MF_D ? 128 : 256);
 }
 
 template <int BITS, typename M> struct PrStage {
@@ -965,19 +965,400 @@ __global__ __launch_bounds__(PR_THREADS) void prefill_tiles_kernel(vq_attend_arg
     }
 }
 
+// ---------------------------------------------------------------------------
+// Heads of 256 channels on the same blocks: the scores run over eight k-steps instead of four, so a wave holds one
+// 16-row block (a block of eight waves = 128 rows = the GQA group at 128 / R positions) where the kernel above holds
+// two -- queries 32 registers, key operands 64, accumulators 32, value operands 32, as there -- and a launch forms
+// the output's channels [128 v_half, 128 v_half + 128): the call is two launches that compute the same scores and
+// probabilities and each take one half of the value tile.  Tiles, token order, softmax and partial format are the
+// kernel's above; a record has 258 floats and the launch of the first half writes its maximum and sum.
+// ---------------------------------------------------------------------------
+constexpr int P2_RB = 1;
+
+template <typename M> struct PrStage2 {
+    uint4 k2;        // packed unit: the two key words (8 channels of a token in either half of the channels) and the
+                     // value word; tail unit: the raw key piece of the second half
+    Meta8<M> vs, vz; // value scale / zero of the thread's 8 tokens; a tail unit's raw key (first half) and value pieces
+                     // travel in the first piece of each
+};
+
+template <int BITS, int GV, typename M>
+__global__ __launch_bounds__(PR_THREADS) __attribute__((amdgpu_waves_per_eu(2, 2)))
+void attend_prefill_rows_d256_kernel(vq_attend_args a, int qp, int nparts, int v_half, float *__restrict__ ws) {
+    constexpr int DH = 2 * MF_D;          // channels of a head
+    constexpr int KST = DH + 8;           // fp16 per token row of the key tile (528 B: conflict-free b128 reads)
+    __shared__ __align__(16) f16 s_k[3][32 * KST];
+    __shared__ __align__(16) f16 s_v[3][MF_D * PF_VSTRIDE];
+
+    constexpr int PER = 32 / BITS;
+    constexpr int KW = DH / PER;
+    constexpr int gshift = GV == 8 ? 5 : GV == 4 ? 6 : 7;   // log2 of the group size
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = lane & 15, blk = lane >> 4;
+    // Which (row tile, (sequence, kv head), run) this block is.  Workgroups go to the eight XCDs in turn by
+    // their linear number, and every XCD has its own L2: with the launch's own numbering the row tiles and runs
+    // of one kv head land on all eight, and each fetches that head's keys and values from HBM for itself (68 MB
+    // per launch at config 4 for 15 MB of input).  The blocks are renumbered so that a head's tiles and runs share
+    // an XCD (a multiple of eight heads) or 8 / heads of them (1, 2 or 4 heads); other counts keep the launch's
+    // numbering.
+    unsigned tile_x = blockIdx.x, bh_y = blockIdx.y, run_z = blockIdx.z;
+    if (gridDim.y % 8 == 0 || 8 % gridDim.y == 0) {
+        const unsigned lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+        const unsigned per_head = gridDim.x * gridDim.z, xcd = lin % 8, slot = lin / 8;
+        unsigned within;
+        if (gridDim.y % 8 == 0) {
+            bh_y = xcd + 8 * (slot / per_head);
+            within = slot % per_head;
+        } else {
+            bh_y = xcd % gridDim.y;
+            within = xcd / gridDim.y + (8 / gridDim.y) * slot;
+        }
+        tile_x = within % gridDim.x;
+        run_z = within / gridDim.x;
+    }
+    const int64_t bh = bh_y;
+    const int64_t hkv = bh % a.Hkv, b = bh / a.Hkv;
+    take_sequence_lengths(a, b);
+    const int R = (int)(a.Hq / a.Hkv);
+    const int64_t cap = a.cap_tokens;
+    const float c = a.scale * LOG2E;
+    const u32 magic = vreg_const(Magic<BITS>::bits);
+    // under a causal mask the last tiles see the most tokens: they are started first
+    const int pos0 = (int)(a.causal ? gridDim.x - 1 - tile_x : tile_x) * qp;
+    const int64_t n_total = a.n_packed + a.n_tail;
+    auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
+
+    // ---- this lane's query row (score column): row j = 16 wave + n of the block
+    const int qshift = 31 - __builtin_clz((unsigned)qp);   // the block covers a power of two of positions (128 / R)
+    int lane_vis[P2_RB], lane_tvis[P2_RB];
+    int lane_lo[P2_RB], lane_tlo[P2_RB];   // sliding window: first packed / tail token the row sees
+    f16x8 qn[P2_RB][8];   // B operands: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of its row
+#pragma unroll
+    for (int rb = 0; rb < P2_RB; ++rb) {
+        const int j = 16 * P2_RB * wave + 16 * rb + n;
+        const int64_t pos = pos0 + (j & (qp - 1));
+        const bool row_ok = pos < a.Sq && (j >> qshift) < R;
+        const int64_t qrow = (b * a.Hq + hkv * R + ((j >> qshift) < R ? (j >> qshift) : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
+        const int64_t vis = visible(row_ok ? pos : a.Sq - 1);
+        lane_vis[rb] = (int)(vis < a.n_packed ? vis : a.n_packed);
+        const int64_t tv = vis - a.n_packed;
+        lane_tvis[rb] = (int)(tv < 0 ? 0 : tv < a.n_tail ? tv : a.n_tail);
+        const int64_t first = window_first(a, n_total, row_ok ? pos : a.Sq - 1);
+        lane_lo[rb] = (int)(first < a.n_packed ? first : a.n_packed);
+        lane_tlo[rb] = (int)(first > a.n_packed ? first - a.n_packed : 0);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            const int64_t e0 = qrow * DH + 32 * ks + 8 * blk;
+            if (a.q_dtype == VQ_F32) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) qn[rb][ks][e] = (f16)((const float *)a.q)[e0 + e];
+            } else {
+                qn[rb][ks] = ld_tail8(a.q, e0, a.q_dtype == VQ_BF16);
+            }
+        }
+    }
+    const int64_t last_pos = pos0 + qp - 1 < a.Sq - 1 ? pos0 + qp - 1 : a.Sq - 1;
+    const int64_t vis_min = visible(pos0), vis_max = visible(last_pos);
+    const int full_vis = (int)(vis_min < a.n_packed ? vis_min : a.n_packed);
+    const int max_vis = (int)(vis_max < a.n_packed ? vis_max : a.n_packed);
+    const int64_t tv_min = vis_min - a.n_packed, tv_max = vis_max - a.n_packed;
+    const int full_tvis = (int)(tv_min < 0 ? 0 : tv_min < a.n_tail ? tv_min : a.n_tail);
+    const int max_tvis = (int)(tv_max < 0 ? 0 : tv_max < a.n_tail ? tv_max : a.n_tail);
+    const int n_punits = (max_vis + 31) / 32;
+    const int n_tunits = (max_tvis + 31) / 32;
+    const int n_work = n_punits + n_tunits;
+    const int nsplit = (int)gridDim.z, sp = (int)run_z;
+    // units below the window of the block's first row are seen by none of its rows
+    const int64_t first_blk = window_first(a, n_total, pos0);
+    const int w_lo = first_blk < a.n_packed ? (int)(first_blk / 32) : n_punits + (int)((first_blk - a.n_packed) / 32);
+    const int w_n = n_work > w_lo ? n_work - w_lo : 0;
+    const int w0 = w_lo + (int)((int64_t)w_n * sp / nsplit), w1 = w_lo + (int)((int64_t)w_n * (sp + 1) / nsplit);
+    const int64_t first_all = window_first(a, n_total, last_pos);   // below it some row of the block sees nothing
+    const int edge_lo = (int)(first_all < a.n_packed ? first_all : a.n_packed);
+    const int edge_tlo = (int)(first_all > a.n_packed ? first_all - a.n_packed : 0);
+
+    // ---- producer side
+    const char *kb = (const char *)a.k_packed + bh * cap * KW * 4;
+    const char *vb = (const char *)a.v_packed + bh * (cap / PER) * DH * 4;
+    const M *ksb = (const M *)a.k_scale + bh * (cap >> gshift) * DH;
+    const M *kzb = (const M *)a.k_zero + bh * (cap >> gshift) * DH;
+    const M *vsb = (const M *)a.v_scale + bh * GV * cap;
+    const M *vzb = (const M *)a.v_zero + bh * GV * cap;
+    const int kt = tid >> 4, kc = tid & 15;       // key tile: token, 8-channel chunk of either half of the channels
+    const int vc = tid & 127, vq = tid >> 7;      // value tile: channel of this launch's half, 8-token quarter
+    const int vch = MF_D * v_half + vc;           // the thread's value channel in the head
+    const int vg = vch >> gshift;                 // its channel group
+    // byte offsets of the thread's key words (chunks kc and kc + 16), value word and value scale / zero piece inside a unit
+    const unsigned k_off = (unsigned)((kt * KW + (BITS == 4 ? kc : kc >> 1)) * 4);
+    constexpr unsigned k_off2 = (BITS == 4 ? 16 : 8) * 4;
+    const unsigned v_off = (unsigned)(((BITS == 4 ? vq : vq >> 1) * DH + vch) * 4);
+    const unsigned m_off = (unsigned)(((int64_t)vg * cap + 8 * vq) * sizeof(M));
+    const int tp = lane & 15, cq = 4 * wave + (lane >> 4);   // tail values: token pair, channel quad
+    const bool tail_bf16 = a.tail_dtype == VQ_BF16;
+    const int64_t tbase = bh * a.tail_cap * DH;
+    const f16x8 off8 = as_h8(Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair, Magic<BITS>::neg_off_pair);
+    using Stage = PrStage2<M>;
+    Meta8<M> ksr[2], kzr[2];   // key scale / zero of the thread's 2 x 8 channels in the token group last fetched
+    int meta_group = -1;
+    auto fetch = [&](int w, Stage &st) {
+        if (w >= n_punits) {   // tail unit: the thread's key and value pieces travel in the value-meta slots
+            // a block-uniform base (the unit's first token) plus a 32-bit offset of the thread's own; a token
+            // past the end of the tail reads the last one instead (masked in the softmax)
+            const int64_t t0 = (int64_t)(w - n_punits) * 32;
+            const int last = (int)(a.n_tail - 1 - t0);   // >= 0: the unit starts inside the tail
+            const char *kt0 = (const char *)a.k_tail + (tbase + t0 * DH) * 2, *vt0 = (const char *)a.v_tail + (tbase + t0 * DH) * 2 + 2 * MF_D * v_half;
+            st.vs.u[0] = *reinterpret_cast<const uint4 *>(kt0 + (unsigned)((kt < last ? kt : last) * (DH * 2) + 16 * kc));
+            st.k2 = *reinterpret_cast<const uint4 *>(kt0 + (unsigned)((kt < last ? kt : last) * (DH * 2) + 2 * MF_D + 16 * kc));
+            // values: four channels of a token pair, so that the transposed tile is written in whole words
+            const int ta = 2 * tp < last ? 2 * tp : last, tb = 2 * tp + 1 < last ? 2 * tp + 1 : last;
+            const uint2 va = *reinterpret_cast<const uint2 *>(vt0 + (unsigned)(ta * (DH * 2) + 8 * cq));
+            const uint2 vb2 = *reinterpret_cast<const uint2 *>(vt0 + (unsigned)(tb * (DH * 2) + 8 * cq));
+            st.vz.u[0] = make_uint4(va.x, va.y, vb2.x, vb2.y);
+            return;
+        }
+        // a block-uniform base that moves with the unit plus a 32-bit offset of the thread's own: the
+        // per-unit address arithmetic stays on the scalar unit
+        const int64_t base = (int64_t)w * 32;
+        st.k2.x = *reinterpret_cast<const u32 *>(kb + base * (KW * 4) + k_off);
+        st.k2.y = *reinterpret_cast<const u32 *>(kb + base * (KW * 4) + k_off + k_off2);
+        st.k2.z = *reinterpret_cast<const u32 *>(vb + (base / PER) * (DH * 4) + v_off);
+        st.vs.load((const char *)vsb + base * sizeof(M) + m_off);
+        st.vz.load((const char *)vzb + base * sizeof(M) + m_off);
+        const int grp = (int)(base >> gshift);
+        if (grp != meta_group) {   // block-uniform
+            meta_group = grp;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                ksr[i].load((const char *)ksb + (int64_t)grp * (DH * sizeof(M)) + 8u * (unsigned)sizeof(M) * (unsigned)(kc + 16 * i));
+                kzr[i].load((const char *)kzb + (int64_t)grp * (DH * sizeof(M)) + 8u * (unsigned)sizeof(M) * (unsigned)(kc + 16 * i));
+            }
+        }
+    };
+    // the thread's eight codes of a word, in order, as exact fp16 numbers
+    auto codes8 = [&](u32 w, int half) -> f16x8 {
+        uint4 lo;
+        if (BITS == 4) lo = word4_in_order(w, magic);
+        else {
+            uint4 hi;
+            word2_in_order(w, magic, lo, hi);
+            if (half) lo = hi;
+        }
+        return as_h8(lo) + off8;
+    };
+    auto unpack_to_lds = [&](int w, const Stage &st, int buf) {
+        if (w < n_punits) {
+            // keys: 2 x 8 channels of token kt; c s + z is formed exactly and rounded once
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * KST + 8 * kc]) = recon8(codes8(st.k2.x, kc & 1), ksr[0], kzr[0]);
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * KST + MF_D + 8 * kc]) = recon8(codes8(st.k2.y, kc & 1), ksr[1], kzr[1]);
+            // values: 8 tokens of channel vch
+            *reinterpret_cast<f16x8 *>(&s_v[buf][vc * PF_VSTRIDE + 8 * vq]) = recon8(codes8(st.k2.z, vq & 1), st.vs, st.vz);
+        } else {
+            // tail unit: plain key row chunk; values transposed, one word (a token pair of one channel)
+            // at a time: the lanes of a wave cover 16 token pairs x 4 channel quads = 64 different banks
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * KST + 8 * kc]) = tail8_from_raw(st.vs.u[0], tail_bf16);
+            *reinterpret_cast<f16x8 *>(&s_k[buf][pf_krow(kt) * KST + MF_D + 8 * kc]) = tail8_from_raw(st.k2, tail_bf16);
+            const f16x8 v0 = tail8_from_raw(st.vz.u[0], tail_bf16);   // channels 0..3 of the first token, then of the second
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                *reinterpret_cast<f16x2 *>(&s_v[buf][(4 * cq + e) * PF_VSTRIDE + 2 * tp]) = f16x2{v0[e], v0[4 + e]};
+        }
+    };
+
+    // ---- consumer state: O[rb][nt] rows 16 rb + 4 blk + r of the wave, channels 16 nt + n; L the row sums
+    f32x4 O[P2_RB][8], L[P2_RB];
+    float m_run[P2_RB], m_seen[P2_RB];
+#pragma unroll
+    for (int rb = 0; rb < P2_RB; ++rb) {
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) O[rb][nt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        L[rb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        m_run[rb] = -INFINITY;
+        m_seen[rb] = -INFINITY;
+    }
+    const f16x8 ones = ones8();
+
+    // move the reference of every row up to what it has seen and rescale the accumulators
+    auto rescale = [&]() {
+#pragma unroll
+        for (int rb = 0; rb < P2_RB; ++rb) {
+            float ms = m_seen[rb];
+            ms = fmaxf(ms, __shfl_xor(ms, 16));
+            ms = fmaxf(ms, __shfl_xor(ms, 32));
+            const float m_new = fmaxf(m_run[rb], ms);
+            const float alpha = m_new == -INFINITY ? 1.f : exp2f(m_run[rb] - m_new);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float al = __shfl(alpha, 4 * blk + r);
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) O[rb][nt][r] *= al;
+                L[rb][r] *= al;
+            }
+            m_run[rb] = m_new;
+        }
+    };
+
+    // The operands of a unit live in registers from one iteration to the next: the key tile's
+    // rows (A) and the value tile's rows (Bv) of unit w+1 are read from LDS while unit w is
+    // still being computed, so that the LDS traffic of the eight waves runs beside the products
+    // and the softmax instead of in front of them.
+    f16x8 A[2][8], Bv[8];
+    auto load_keys = [&](int buf) {
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+            const f16 *kr = &s_k[buf][pf_krow(pf_tok(n >> 2, n & 3, T)) * KST + 8 * blk];
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks) A[T][ks] = *reinterpret_cast<const f16x8 *>(kr + 32 * ks);
+        }
+    };
+    auto load_values = [&](int buf) {
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt)
+            Bv[nt] = *reinterpret_cast<const f16x8 *>(&s_v[buf][(16 * nt + n) * PF_VSTRIDE + 8 * blk]);
+    };
+
+    // One unit: scores of the wave's row blocks (four independent accumulator chains side by
+    // side), softmax against the lazily updated references (raised in place, with the
+    // accumulators rescaled, when some row's scores outgrow its reference), second product.
+    // `next` is the buffer of the following unit (stale but harmless after the last one).
+    auto compute = [&](int next, int base, bool packed, int full, int lo_edge) {
+        f32x4 S[P2_RB][2];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+                for (int rb = 0; rb < P2_RB; ++rb)
+                    S[rb][T] = VQ_MFMA(A[T][ks], qn[rb][ks], ks == 0 ? (f32x4{0.f, 0.f, 0.f, 0.f}) : S[rb][T]);
+        load_keys(next);
+        bool grow = false;
+#pragma unroll
+        for (int rb = 0; rb < P2_RB; ++rb) {
+            if (base + 32 > full || base < lo_edge) {
+                const int lim = packed ? lane_vis[rb] : lane_tvis[rb], lo = packed ? lane_lo[rb] : lane_tlo[rb];
+#pragma unroll
+                for (int T = 0; T < 2; ++T)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (base + pf_tok(blk, r, T) >= lim || base + pf_tok(blk, r, T) < lo) S[rb][T][r] = -INFINITY;
+            }
+            const float mx = vmax3(vmax3(S[rb][0][0], S[rb][0][1], S[rb][0][2]), vmax3(S[rb][0][3], S[rb][1][0], S[rb][1][1]),
+                                   vmax3(S[rb][1][2], S[rb][1][3], S[rb][1][3]));
+            m_seen[rb] = mx * c;
+            grow |= mx * c > m_run[rb] + RESCALE_SLACK;
+        }
+        if (__any(grow)) rescale();
+        f16x8 P8[P2_RB];
+#pragma unroll
+        for (int rb = 0; rb < P2_RB; ++rb) {
+            const float nm = m_run[rb] == -INFINITY ? 0.f : -m_run[rb];
+            u32 P[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                P[r] = as_u(f16x2{(f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[rb][0][r], c, nm)),
+                                  (f16)__builtin_amdgcn_exp2f(__builtin_fmaf(S[rb][1][r], c, nm))});
+            P8[rb] = as_h8(P[0], P[1], P[2], P[3]);
+        }
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt)
+#pragma unroll
+            for (int rb = 0; rb < P2_RB; ++rb) O[rb][nt] = VQ_MFMA(P8[rb], Bv[nt], O[rb][nt]);
+#pragma unroll
+        for (int rb = 0; rb < P2_RB; ++rb) L[rb] = VQ_MFMA(P8[rb], ones, L[rb]);
+        load_values(next);
+    };
+
+    // ---- pipeline over the work units [w0, w1) on three LDS buffers: while unit w is computed
+    // from registers, unit w+1 is read from its buffer, unit w+2 is unpacked into the third and
+    // unit w+3 is requested from memory.  The producer's share comes after the unit's second product
+    // (its first instructions issue while those products run); unpacking before the products in half
+    // of the waves, to put the two waves of a SIMD out of step, measured 8 % slower.
+    // The barrier between units waits for LDS only: __syncthreads() also waits for every outstanding
+    // global load, i.e. for the unit just requested, once per unit.  For the same reason nothing
+    // requested before the loop may still be pending inside it (the compiler would wait for it at
+    // the loop head, and with it for whatever was requested since).
+    Stage st;
+    if (w1 > w0) {
+        fetch(w0, st);
+        unpack_to_lds(w0, st, 0);
+        if (w0 + 1 < w1) {
+            fetch(w0 + 1, st);
+            unpack_to_lds(w0 + 1, st, 1);
+        }
+        if (w0 + 2 < w1) fetch(w0 + 2, st);
+        __syncthreads();
+        load_keys(0);
+        load_values(0);
+    }
+    wait_global_accesses();
+    int cur = 0;
+    for (int w = w0; w < w1; ++w) {
+        const int next = cur == 2 ? 0 : cur + 1, third = next == 2 ? 0 : next + 1;
+        const bool packed = w < n_punits;
+        const int base = packed ? w * 32 : (w - n_punits) * 32;
+        compute(next, base, packed, packed ? full_vis : full_tvis, packed ? edge_lo : edge_tlo);
+        if (w + 2 < w1) unpack_to_lds(w + 2, st, third);
+        if (w + 3 < w1) fetch(w + 3, st);
+        lds_barrier();
+        cur = next;
+    }
+
+    // ---- every wave owns its rows: accumulator register r of lane (n, blk) is row 4 blk + r of the
+    // row block, tile nt column n is channel 16 nt + n; the row's reference sits in lane 4 blk + r.
+    // A launch with one run per row and no protected rows to patch in writes the output itself: the merge
+    // of a single record is that record normalised (mfma_prefill_writes_output decides, for the host too).
+    const bool direct = mfma_prefill_writes_output(a, nparts);
+#pragma unroll
+    for (int rb = 0; rb < P2_RB; ++rb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int jr = 16 * P2_RB * wave + 16 * rb + 4 * blk + r;
+            const int64_t pr = pos0 + (jr & (qp - 1));
+            const float mr = __shfl(m_run[rb], 4 * blk + r);
+            if (pr < a.Sq && (jr >> qshift) < R) {
+                const int64_t row = (b * a.Hq + hkv * R + (jr >> qshift)) * a.Sq + pr;
+                if (direct) {
+                    // the only record of its row: what the merge would make of it (0 for a row that sees nothing)
+                    const bool seen = mr != -INFINITY && L[rb][r] > 0.f;
+#pragma unroll
+                    for (int nt = 0; nt < 8; ++nt) {
+                        const float v = seen ? __fdiv_rn(O[rb][nt][r], L[rb][r]) : 0.f;
+                        const int64_t oi = row * DH + MF_D * v_half + 16 * nt + n;
+                        if (a.out_dtype == VQ_F16) ((f16 *)a.out)[oi] = (f16)v;
+                        else if (a.out_dtype == VQ_BF16) ((u16 *)a.out)[oi] = f32_to_bf16(v);
+                        else ((float *)a.out)[oi] = v;
+                    }
+                    continue;
+                }
+                float *o = ws + (row * nparts + sp) * (DH + 2);
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) o[2 + MF_D * v_half + 16 * nt + n] = O[rb][nt][r];
+                if (n == 0 && v_half == 0) { o[0] = mr * LN2; o[1] = L[rb][r]; }   // both launches form the same two
+            }
+        }
+}
+
 int mfma_prefill_block_rows(const vq_attend_args &a);
 
+// the blocks of eight waves: 256 rows of 128-channel heads, 128 rows of 256-channel heads (which have no other blocks)
+static bool prefill_row_blocks(const vq_attend_args &a) {
+    return (a.Hq / a.Hkv) * a.Sq >= (a.D == 2 * MF_D ? 128 : 256);
+}
+
 bool mfma_prefill_supported(const vq_attend_args &a) {
-    if (a.D != MF_D || a.n_packed < 0 || a.Sq < 16) return false;
+    if ((a.D != MF_D && a.D != 2 * MF_D) || a.n_packed < 0 || a.Sq < 16) return false;
     if (a.Hq % a.Hkv != 0) return false;
     const int64_t R = a.Hq / a.Hkv;
     if (!(R == 1 || R == 2 || R == 4 || R == 8)) return false;
+    // (256-channel heads: 128-row blocks only, fp16 scale / zero -- float32 ones do not fit the registers beside
+    // twice the key operands)
+    if (a.D == 2 * MF_D && (!prefill_row_blocks(a) || (a.n_packed > 0 && a.meta_dtype != VQ_F16))) return false;
     if (a.n_packed > 0) {
         if (!(a.pack_bits == 2 || a.pack_bits == 4)) return false;
         if (!(a.group == 32 || a.group == 64 || a.group == 128)) return false;
         // float32 scale / zero: the 256-row blocks take it (they reconstruct in the producer); fewer rows stay on
         // the 8-row tiles of the decode kernel
-        if (a.meta_dtype != VQ_F16 && !(a.meta_dtype == VQ_F32 && (a.Hq / a.Hkv) * a.Sq >= 256)) return false;
+        if (a.meta_dtype != VQ_F16 && !(a.meta_dtype == VQ_F32 && prefill_row_blocks(a))) return false;
         if (a.v_layout != VQ_V_TOKEN_PACKED) return false;
         if (a.n_packed % 32 != 0 || a.cap_tokens % 32 != 0 || a.cap_tokens % a.group != 0) return false;
         if (a.cap_tokens > ((int64_t)1 << 28)) return false;   // 32-bit byte offsets inside one (sequence, kv head) slab
@@ -989,24 +1370,24 @@ bool mfma_prefill_supported(const vq_attend_args &a) {
     if (!(a.scale > 0.f)) return false;
     if (a.n_tail > 0 && (!(a.tail_dtype == VQ_F16 || a.tail_dtype == VQ_BF16) || (((uintptr_t)a.k_tail | (uintptr_t)a.v_tail) & 15u))) return false;
     if (a.B * a.Hkv > 65535) return false;
-    if (a.n_tail > 0 && a.tail_cap * MF_D % 8 != 0) return false;
+    if (a.n_tail > 0 && a.tail_cap * a.D % 8 != 0) return false;
     const uintptr_t al = (uintptr_t)a.k_packed | (uintptr_t)a.v_packed | (uintptr_t)a.k_scale | (uintptr_t)a.k_zero |
                          (uintptr_t)a.v_scale | (uintptr_t)a.v_zero;
     if (a.n_packed > 0 && (al & 15u)) return false;
-    if (mfma_prefill_block_rows(a) == 256 && a.q_dtype != VQ_F32 && ((uintptr_t)a.q & 15u)) return false;
+    if (prefill_row_blocks(a) && a.q_dtype != VQ_F32 && ((uintptr_t)a.q & 15u)) return false;
     return true;
 }
 
 int mfma_prefill_block_rows(const vq_attend_args &a) {
-    return (a.Hq / a.Hkv) * a.Sq >= 256 ? 256 : 64;
+    return a.D == 2 * MF_D ? 128 : prefill_row_blocks(a) ? 256 : 64;
 }
 
 bool mfma_prefill_direct_output(const vq_attend_args &a, int nparts) {
-    return mfma_prefill_block_rows(a) == 256 && mfma_prefill_writes_output(a, nparts);
+    return prefill_row_blocks(a) && mfma_prefill_writes_output(a, nparts);
 }
 
 bool mfma_prefill_uses_tiles(const vq_attend_args &a) {
-    return a.kv_tiles != nullptr && a.packed_lens == nullptr && mfma_prefill_block_rows(a) == 256 &&
+    return a.kv_tiles != nullptr && a.packed_lens == nullptr && a.D == MF_D && mfma_prefill_block_rows(a) == 256 &&
            ((uintptr_t)a.kv_tiles & 15u) == 0 && a.tile_cap * 32 >= a.n_packed + a.n_tail && a.n_packed % 32 == 0;
 }
 
@@ -1049,8 +1430,19 @@ bool launch_attend_mfma_prefill(const vq_attend_args &a, const AttendPlan &p) {
     const int R = (int)(a.Hq / a.Hkv);
     const int rows = mfma_prefill_block_rows(a);
     const int qp = rows / R, tiles = (int)cdiv(a.Sq, qp);
-    const int gv = a.n_packed > 0 ? (int)(MF_D / a.group) : 4;   // without packed units any instantiation serves
     const dim3 grid((unsigned)tiles, (unsigned)(a.B * a.Hkv), (unsigned)p.nsplit), block(256);
+    if (a.D == 2 * MF_D) {
+        // heads of 256 channels: one launch per half of the output's channels
+        const int gv2 = a.n_packed > 0 ? (int)(2 * MF_D / a.group) : 8;
+#define VQ_LAUNCH2(BITS, GV)                                                                                            \
+        for (int half = 0; half < 2; ++half)                                                                            \
+            hipLaunchKernelGGL((attend_prefill_rows_d256_kernel<BITS, GV, f16>), grid, dim3(PR_THREADS), 0, st, a, qp, p.nparts, half, ws);
+        if (a.pack_bits == 4 || a.n_packed == 0) { if (gv2 == 2) VQ_LAUNCH2(4, 2) else if (gv2 == 4) VQ_LAUNCH2(4, 4) else VQ_LAUNCH2(4, 8) }
+        else { if (gv2 == 2) VQ_LAUNCH2(2, 2) else if (gv2 == 4) VQ_LAUNCH2(2, 4) else VQ_LAUNCH2(2, 8) }
+#undef VQ_LAUNCH2
+        return mfma_prefill_writes_output(a, p.nparts);
+    }
+    const int gv = a.n_packed > 0 ? (int)(MF_D / a.group) : 4;   // without packed units any instantiation serves
 #define VQ_LAUNCH(BITS, GV)                                                                                          \
     do {                                                                                                             \
         if (rows == 256 && mfma_prefill_uses_tiles(a))                                                               \
