@@ -1100,6 +1100,35 @@ def test_vecinfer_fused_modes_and_state_round_trip(memory_bound):
     assert np.max(np.abs(host(out_w).astype(np.float32) - ref_w)) < 2e-3
 
 
+@pytest.mark.parametrize("D,Hq,H,Sq,window", [(128, 8, 2, 100, 0), (128, 6, 2, 120, 64), (256, 12, 4, 100, 0), (128, 8, 2, 40, 0)])
+def test_vecinfer_prefill_sized_queries_attend_over_gathered_rows(D, Hq, H, Sq, window):
+    """256 query rows or more per kv head: the cache gathers the centroids once into 16-bit rows and runs the
+    matrix-unit prefill blocks over them instead of building a look-up table per query row; fewer rows (the last case)
+    stay on the table kernel.  Both against the oracle over the stored indices."""
+    require_gpu()
+    rng = np.random.default_rng(D + Sq)
+    cfg = _vi_cfg(head_dim=D, fused_sdpa=True, fused_sdpa_memory_bound=True)
+    c = KVCacheFactory.create(cfg)
+    n = 700
+    k, v = _kv(2, H, n, D, 5)
+    c.update_and_fetch(to_dev(k[:, :, :400]), to_dev(v[:, :, :400]))
+    c.update_and_fetch(to_dev(k[:, :, 400:]), to_dev(v[:, :, 400:]))
+    q = rng.standard_normal((2, Hq, Sq, D)).astype(np.float16)
+    out = host(c.fused_sdpa(to_dev(q), 0.09, causal=True, sliding_window=window)).astype(np.float32)
+    Hm = ov.walsh_hadamard_matrix(D)
+    k_t_hat = ov.dequantize_vq(host(c._stored_k_indices[:, :, :n]), cfg.key_codebook)
+    v_hat = ov.dequantize_vq(host(c._stored_v_indices[:, :, :n]), cfg.value_codebook)
+    gathered = (Hq // H) * Sq >= 256
+    if gathered:   # the rows are rounded to the queries' type, as the reconstruction the cache hands out is
+        k_t_hat, v_hat = k_t_hat.astype(np.float16).astype(np.float32), v_hat.astype(np.float16).astype(np.float32)
+    ref = oa.sdpa(q.astype(np.float32) @ Hm, k_t_hat, v_hat, 0.09, causal=True, sliding_window=window)
+    assert np.max(np.abs(out - ref)) < 2e-3, float(np.max(np.abs(out - ref)))
+    # and against the table kernel on the same indices
+    tab = K.metal_fused_sdpa(to_dev(q).float() @ to_dev(Hm), c._stored_k_indices, c._key_codebook, c._stored_v_indices,
+                             c._value_codebook, 0.09, causal=True, sliding_window=window, out_dtype=torch.float16, n_tokens=n)
+    assert float(np.max(np.abs(out - host(tab).astype(np.float32)))) < (4e-3 if gathered else 1e-6)
+
+
 def test_vecinfer_max_ctx_cap():
     require_gpu()
     c = KVCacheFactory.create(_vi_cfg(fused_sdpa=True, fused_sdpa_max_ctx=100))

@@ -369,20 +369,27 @@ class VecInferKVCache(FP16KVCache):
         table_kernel = (kcb.shape[0] == vcb.shape[0] <= 256 and max(n_sub_k, n_sub_v) <= 32
                         and (n_sub_k + n_sub_v) * kcb.shape[0] * 4 <= 65536
                         and (self._stored_k_indices.dtype != torch.uint8 or (n_sub_k % 4 == 0 and n_sub_v % 4 == 0)))
-        if table_kernel:
+        # A prefill-sized call (256 query rows or more per kv head at a head size the matrix-unit prefill blocks take)
+        # gathers the centroids once into a transient copy in the queries' 16-bit type -- what update_and_fetch hands
+        # a host that attends by itself (vecinfer_cache.py:336-379: the reconstruction cast to the input dtype) -- and
+        # attends over it with those blocks: the table kernel builds a table per query row, which pays for a few rows
+        # per kv head only (512 queries over 4.6k tokens, 32 / 8 heads: 0.64 ms from the tables, 0.09 ms this way).
+        H_kv = self._stored_k_indices.shape[1]
+        prefill_sized = (self._head_dim in (128, 256) and q.shape[1] % H_kv == 0 and (q.shape[1] // H_kv) * q.shape[2] >= 256
+                         and q.dtype in (torch.float16, torch.bfloat16))
+        if table_kernel and not prefill_sized:
             # look-up table + centroid histogram straight from the indices
             return K.metal_fused_sdpa(q_tilde, self._stored_k_indices, kcb, self._stored_v_indices, vcb, float(scale),
                                       causal=bool(causal) and q.shape[2] > 1, sliding_window=int(sliding_window or 0),
                                       out_dtype=q.dtype, n_tokens=n)
-        if sliding_window:
-            raise ValueError("VecInferKVCache.fused_sdpa: sliding_window attention needs the table kernel "
-                             "(n_centroids <= 256, at most 32 sub-vectors per head)")
+        rows_dtype = q.dtype if prefill_sized else torch.float32
         k_tilde_hat = K.vecinfer_dequant_metal(self._stored_k_indices[:, :, :n].contiguous(), self._key_codebook,
-                                               out_dtype=torch.float32)
+                                               out_dtype=rows_dtype)
         v_hat = K.vecinfer_dequant_metal(self._stored_v_indices[:, :, :n].contiguous(), self._value_codebook,
-                                         out_dtype=torch.float32)
+                                         out_dtype=rows_dtype)
         return K.kivi_packed_attend(q_tilde, k_tail=k_tilde_hat, v_tail=v_hat, n_tail=n, scale=float(scale),
-                                    causal=bool(causal) and q.shape[2] > 1, out_dtype=q.dtype)
+                                    causal=bool(causal) and q.shape[2] > 1, sliding_window=int(sliding_window or 0),
+                                    out_dtype=q.dtype)
 
     # ------------------------------------------------------------------ reporting
     compressed_key_bytes = property(lambda self: self._tally.n["key_compressed"])
