@@ -480,15 +480,15 @@ def test_prefill_tiles_change_no_bit_and_follow_the_cache(bits, g, dtype):
     assert torch.equal(outs[0], outs[1]) and caches[0]._tiles is None
 
 
-@pytest.mark.parametrize("bits,g", [(4, 32), (2, 32)])
-def test_sink_protected_cache_with_prefill_sized_query_blocks(bits, g):
+@pytest.mark.parametrize("bits,g,Hq,Sq", [(4, 32, 8, 64), (2, 32, 8, 64), (4, 32, 6, 96), (2, 32, 14, 40)])
+def test_sink_protected_cache_with_prefill_sized_query_blocks(bits, g, Hq, Sq):
     """Protected rows under a prefill-sized call (64 positions x 4 query heads = 256 rows a kv head, the
-    256-row attention blocks): the stand-ins' weights are taken out of sums the matrix unit formed from
-    fp16-rounded reconstructions, so the queries here are aimed at the stand-ins themselves and at the
-    rows next to them, where those weights carry most of a row's mass."""
+    256-row attention blocks; groups of 3 and 7 heads, which run as groups of 4 and 8): the stand-ins' weights are
+    taken out of sums the matrix unit formed from fp16-rounded reconstructions, so the queries here are aimed at the
+    stand-ins themselves and at the rows next to them, where those weights carry most of a row's mass."""
     require_gpu()
     rng = np.random.default_rng(23)
-    B, Hq, H, D, R, n = 1, 8, 2, 128, 64, 448
+    B, H, D, R, n = 1, 2, 128, 64, 448
     k = rng.standard_normal((B, H, n, D)).astype(np.float16)
     v = rng.standard_normal((B, H, n, D)).astype(np.float16)
     for p, f in ((5, 12), (77, 10), (200, 14), (201, 9)):
@@ -502,7 +502,6 @@ def test_sink_protected_cache_with_prefill_sized_query_blocks(bits, g):
         m.update_and_fetch(k[:, :, s0:s1], v[:, :, s0:s1])
     assert c._n_quantized == m.n_quantized and any(c._side_pos[b] for b in range(B))
     km, vm = m.keys[:, :, : m.offset], m.values[:, :, : m.offset]
-    Sq = 64
     q = rng.standard_normal((B, Hq, Sq, D)).astype(np.float16)
     sinks = m.sink_positions_for(0)
     for i, p in enumerate(sinks):
