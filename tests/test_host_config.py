@@ -160,3 +160,39 @@ def test_core_types():
     with pytest.raises(QuantizerConfigError, match="'channel' or 'token'"):
         QuantizerRegistry.create("kivi", d=16, axis="rows")
     assert issubclass(QuantizerConfigError, ValueError)
+
+
+def test_paired_heads_are_the_same_attention():
+    """Two kv heads of 64 channels side by side as one head of 128, every query head zero-padded into the half of its own
+    kv head and reading that half of the output: the attention of the single heads (the form a memory-bound KIVI cache
+    keeps 64-channel heads in), here in plain float64 arithmetic."""
+    import torch
+    from veloxquant_mlx_amd.cache.kivi_cache import own_half_of_paired_output, pad_queries_for_paired_heads, pair_heads
+    g = torch.Generator().manual_seed(0)
+    B, H, S, D, Hq, Sq = 2, 4, 9, 64, 12, 3
+    R = Hq // H
+    k, v = (torch.randn((B, H, S, D), generator=g, dtype=torch.float64) for _ in range(2))
+    q = torch.randn((B, Hq, Sq, D), generator=g, dtype=torch.float64)
+    kp = pair_heads(k)
+    assert kp.shape == (B, H // 2, S, 2 * D)
+    for m in range(H // 2):
+        assert torch.equal(kp[:, m, :, :D], k[:, 2 * m]) and torch.equal(kp[:, m, :, D:], k[:, 2 * m + 1])
+    wide = pad_queries_for_paired_heads(q, H)
+    for h in range(Hq):
+        half = (h // R) % 2
+        assert torch.equal(wide[:, h, :, half * D:(half + 1) * D], q[:, h])
+        assert float(wide[:, h, :, (1 - half) * D:(2 - half) * D].abs().sum()) == 0.0
+    assert torch.equal(own_half_of_paired_output(wide, H), q)
+    # a buffer whose other halves are already zero is filled in place
+    buf = torch.zeros_like(wide)
+    assert pad_queries_for_paired_heads(q, H, buf) is buf and torch.equal(buf, wide)
+
+    def attend(q_, k_, v_, ratio):
+        k_, v_ = k_.repeat_interleave(ratio, 1), v_.repeat_interleave(ratio, 1)
+        return torch.softmax(q_ @ k_.transpose(-1, -2) * 0.125, -1) @ v_
+
+    got = own_half_of_paired_output(attend(wide, kp, pair_heads(v), 2 * R), H)
+    assert float((got - attend(q, k, v, R)).abs().max()) < 1e-12
+    # a leading layer axis (the layer stack) goes through unchanged
+    q5 = torch.randn((3, B, Hq, 1, D), generator=g, dtype=torch.float64)
+    assert torch.equal(own_half_of_paired_output(pad_queries_for_paired_heads(q5, H), H), q5)
