@@ -612,10 +612,10 @@ def _extras(torch, K, dev):
     # config 4's pass at the head counts of other models of the reference's scripts: GQA groups the matrix-unit kernels do
     # not tile run filled up to the next size that they do, 64-channel heads in pairs, 256-channel heads in 128-row blocks
     for tag, hq, hkv, d, note in (
-            ("24q_8kv", 24, 8, 128, "Llama-3.2-3B: groups of 3 run as groups of 4"),
-            ("28q_4kv", 28, 4, 128, "Qwen2.5-7B: groups of 7 run as groups of 8"),
+            ("24q_8kv", 24, 8, 128, "Llama-3.2-3B: groups of 3 heads, 85 positions a block"),
+            ("28q_4kv", 28, 4, 128, "Qwen2.5-7B: groups of 7 heads, 36 positions a block"),
             ("32q_8kv_d64", 32, 8, 64, "Llama-3.2-1B: kv heads of 64 channels in pairs, groups of 8"),
-            ("12q_4kv_d256", 12, 4, 256, "Falcon3-7B: heads of 256 channels, 128-row blocks, one launch per half of the output's channels; groups of 3 run as groups of 4")):
+            ("12q_4kv_d256", 12, 4, 256, "Falcon3-7B: heads of 256 channels, 128-row blocks, one launch per half of the output's channels; groups of 3 heads, 42 positions a block")):
         run_ = _prefill_case(torch, dev, hq, hkv, d)
         run_()
         ms_ = min(run_() for _ in range(3))

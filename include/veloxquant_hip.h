@@ -382,7 +382,7 @@ int vq_kivi_attend_fixed_order(int enable);
 /* Bytes of scratch vq_kivi_attend needs for these shapes (fields other than the shapes, pack_bits,
  * group, num_splits, sliding_window and sink_k are ignored).  0 for a launch that writes its output
  * itself (a prefill whose row tiles fill the GPU, one run per row, no protected rows): workspace may
- * then be NULL.  A call with several query positions and a GQA group of 3, 5, 6 or 7 heads runs as
+ * then be NULL.  A call with several query positions (fewer than 256 rows a kv head) and a GQA group of 3, 5, 6 or 7 heads runs as
  * the next group size the matrix-unit kernels tile (4 or 8: every group filled up with heads of
  * zeros, whose rows are computed and dropped), a prefill-sized one with more than eight heads a
  * group as passes of eight heads; its queries and outputs in that form are part of

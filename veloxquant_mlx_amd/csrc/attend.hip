@@ -27,7 +27,8 @@ AttendPlan plan_attend(const vq_attend_args &a) {
         const int rows = mfma_prefill_block_rows(a);
         const int64_t blocks = a.B * a.Hkv * cdiv(a.Sq, rows / (a.Hq / a.Hkv));
         const int64_t work = cdiv(a.n_packed + a.n_tail, 32);
-        int64_t ns = a.num_splits > 0 ? a.num_splits : cdiv(rows != 64 ? 256 : 512, blocks);
+        // (as many runs as still fit the chip in one round: a few blocks more than that would run as a second round)
+        int64_t ns = a.num_splits > 0 ? a.num_splits : (rows != 64 ? 256 : 512) / (blocks > 0 ? blocks : 1);
         if (ns > 8) ns = 8;
         if (ns > work) ns = work;
         if (ns < 1) ns = 1;
@@ -173,8 +174,8 @@ static int validate(const vq_attend_args *a, const char *fn) {
     return VQ_OK;
 }
 
-// Several query positions of a GQA group of 3, 5, 6 or 7 heads: the matrix-unit kernels tile groups of 1, 2, 4
-// and 8 (or more) heads.  Such a call runs as the next of those sizes -- every kv head's group filled up with
+// Several query positions of a GQA group of 3, 5, 6 or 7 heads, fewer than 256 rows a kv head: the decode kernel's
+// tiles and the 64-row prefill blocks hold groups of 1, 2, 4 and 8 (or more) heads.  Such a call runs as the next of those sizes -- every kv head's group filled up with
 // heads of zeros, whose rows are computed and dropped -- when that takes a matrix-unit path and the call as given
 // does not.  A prefill-sized call with more than eight heads a group runs eight of them at a time through the prefill
 // blocks (one pass per eight heads, the last filled up) instead of one position a tile through the decode kernel.

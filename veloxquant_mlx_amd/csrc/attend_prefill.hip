@@ -561,16 +561,17 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
     auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
 
     // ---- this lane's query rows (score columns): row j = 32 wave + 16 rb + n of the block
-    const int qshift = 31 - __builtin_clz((unsigned)qp);   // the block covers a power of two of positions (256 / R)
+    // the block covers qp = 256 / R positions (rounded down: a group of 3 heads 85, and the last row of the block idles)
     int lane_vis[PR_RB], lane_tvis[PR_RB];
     int lane_lo[PR_RB], lane_tlo[PR_RB];   // sliding window: first packed / tail token the row sees
     f16x8 qn[PR_RB][4];   // B operands: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of its row
 #pragma unroll
     for (int rb = 0; rb < PR_RB; ++rb) {
         const int j = 16 * PR_RB * wave + 16 * rb + n;
-        const int64_t pos = pos0 + (j & (qp - 1));
-        const bool row_ok = pos < a.Sq && (j >> qshift) < R;
-        const int64_t qrow = (b * a.Hq + hkv * R + ((j >> qshift) < R ? (j >> qshift) : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
+        const int jh = (int)((unsigned)j / (unsigned)qp);   // head of the group, position in the block
+        const int64_t pos = pos0 + (j - jh * qp);
+        const bool row_ok = pos < a.Sq && jh < R;
+        const int64_t qrow = (b * a.Hq + hkv * R + (jh < R ? jh : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
         const int64_t vis = visible(row_ok ? pos : a.Sq - 1);
         lane_vis[rb] = (int)(vis < a.n_packed ? vis : a.n_packed);
         const int64_t tv = vis - a.n_packed;
@@ -878,10 +879,11 @@ void attend_prefill_rows_kernel(vq_attend_args a, int qp, int nparts, float *__r
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int jr = 16 * PR_RB * wave + 16 * rb + 4 * blk + r;
-            const int64_t pr = pos0 + (jr & (qp - 1));
+            const int jrh = (int)((unsigned)jr / (unsigned)qp);
+            const int64_t pr = pos0 + (jr - jrh * qp);
             const float mr = __shfl(m_run[rb], 4 * blk + r);
-            if (pr < a.Sq && (jr >> qshift) < R) {
-                const int64_t row = (b * a.Hq + hkv * R + (jr >> qshift)) * a.Sq + pr;
+            if (pr < a.Sq && jrh < R) {
+                const int64_t row = (b * a.Hq + hkv * R + jrh) * a.Sq + pr;
                 if (direct) {
                     // the only record of its row: what the merge would make of it (0 for a row that sees nothing)
                     const bool seen = mr != -INFINITY && L[rb][r] > 0.f;
@@ -1030,16 +1032,17 @@ void attend_prefill_rows_d256_kernel(vq_attend_args a, int qp, int nparts, int v
     auto visible = [&](int64_t p) { return a.causal ? n_total - a.Sq + p + 1 : n_total; };   // slots row p sees
 
     // ---- this lane's query row (score column): row j = 16 wave + n of the block
-    const int qshift = 31 - __builtin_clz((unsigned)qp);   // the block covers a power of two of positions (128 / R)
+    // the block covers qp = 128 / R positions (rounded down)
     int lane_vis[P2_RB], lane_tvis[P2_RB];
     int lane_lo[P2_RB], lane_tlo[P2_RB];   // sliding window: first packed / tail token the row sees
     f16x8 qn[P2_RB][8];   // B operands: lane (n, blk) holds channels 32 ks + 8 blk + 0..7 of its row
 #pragma unroll
     for (int rb = 0; rb < P2_RB; ++rb) {
         const int j = 16 * P2_RB * wave + 16 * rb + n;
-        const int64_t pos = pos0 + (j & (qp - 1));
-        const bool row_ok = pos < a.Sq && (j >> qshift) < R;
-        const int64_t qrow = (b * a.Hq + hkv * R + ((j >> qshift) < R ? (j >> qshift) : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
+        const int jh = (int)((unsigned)j / (unsigned)qp);   // head of the group, position in the block
+        const int64_t pos = pos0 + (j - jh * qp);
+        const bool row_ok = pos < a.Sq && jh < R;
+        const int64_t qrow = (b * a.Hq + hkv * R + (jh < R ? jh : R - 1)) * a.Sq + (pos < a.Sq ? pos : a.Sq - 1);
         const int64_t vis = visible(row_ok ? pos : a.Sq - 1);
         lane_vis[rb] = (int)(vis < a.n_packed ? vis : a.n_packed);
         const int64_t tv = vis - a.n_packed;
@@ -1313,10 +1316,11 @@ void attend_prefill_rows_d256_kernel(vq_attend_args a, int qp, int nparts, int v
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int jr = 16 * P2_RB * wave + 16 * rb + 4 * blk + r;
-            const int64_t pr = pos0 + (jr & (qp - 1));
+            const int jrh = (int)((unsigned)jr / (unsigned)qp);
+            const int64_t pr = pos0 + (jr - jrh * qp);
             const float mr = __shfl(m_run[rb], 4 * blk + r);
-            if (pr < a.Sq && (jr >> qshift) < R) {
-                const int64_t row = (b * a.Hq + hkv * R + (jr >> qshift)) * a.Sq + pr;
+            if (pr < a.Sq && jrh < R) {
+                const int64_t row = (b * a.Hq + hkv * R + jrh) * a.Sq + pr;
                 if (direct) {
                     // the only record of its row: what the merge would make of it (0 for a row that sees nothing)
                     const bool seen = mr != -INFINITY && L[rb][r] > 0.f;
@@ -1349,7 +1353,9 @@ bool mfma_prefill_supported(const vq_attend_args &a) {
     if ((a.D != MF_D && a.D != 2 * MF_D) || a.n_packed < 0 || a.Sq < 16) return false;
     if (a.Hq % a.Hkv != 0) return false;
     const int64_t R = a.Hq / a.Hkv;
-    if (!(R == 1 || R == 2 || R == 4 || R == 8)) return false;
+    // the blocks of eight waves take any group of up to eight heads (256 / R or 128 / R positions a block, rounded
+    // down); the 64-row blocks the powers of two
+    if (!(R == 1 || R == 2 || R == 4 || R == 8) && !(R >= 1 && R <= 8 && prefill_row_blocks(a))) return false;
     // (256-channel heads: 128-row blocks only, fp16 scale / zero -- float32 ones do not fit the registers beside
     // twice the key operands)
     if (a.D == 2 * MF_D && (!prefill_row_blocks(a) || (a.n_packed > 0 && a.meta_dtype != VQ_F16))) return false;
