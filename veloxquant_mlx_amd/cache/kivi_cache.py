@@ -433,7 +433,8 @@ class KIVIKVCache(FP16KVCache):
         H = self._shape_bhd[1]
         nq, n_tail = kw["n_packed"], kw["n_tail"]
         R = Hq // max(H, 1)
-        rows = (R if R in (1, 2, 4) else 4 if R == 3 else 8) * Sq   # a block's rows: the library runs groups of 1, 2, 4, 8 heads
+        # the rows a kv head's blocks hold: below 256 the library fills a group up to the next of 1, 2, 4, 8 heads
+        rows = (R if R in (1, 2, 4, 8) or (R <= 64 and R * Sq >= 256) else 4 if R == 3 else 8) * Sq
         if not (self.prefill_tiles and self._memory_bound and self._v_layout == "token" and D == 128 and Hq % H == 0
                 and rows >= 256 and nq % 32 == 0 and "sinks" not in kw
                 and (n_tail == 0 or self._tail_k.dtype in (torch.float16, torch.bfloat16))):

@@ -1353,9 +1353,9 @@ bool mfma_prefill_supported(const vq_attend_args &a) {
     if ((a.D != MF_D && a.D != 2 * MF_D) || a.n_packed < 0 || a.Sq < 16) return false;
     if (a.Hq % a.Hkv != 0) return false;
     const int64_t R = a.Hq / a.Hkv;
-    // the blocks of eight waves take any group of up to eight heads (256 / R or 128 / R positions a block, rounded
-    // down); the 64-row blocks the powers of two
-    if (!(R == 1 || R == 2 || R == 4 || R == 8) && !(R >= 1 && R <= 8 && prefill_row_blocks(a))) return false;
+    // the blocks of eight waves take any group of up to 64 heads (256 / R or 128 / R positions a block, rounded
+    // down); the 64-row blocks the powers of two up to eight
+    if (!(R == 1 || R == 2 || R == 4 || R == 8) && !(R >= 1 && R <= 64 && prefill_row_blocks(a))) return false;
     // (256-channel heads: 128-row blocks only, fp16 scale / zero -- float32 ones do not fit the registers beside
     // twice the key operands)
     if (a.D == 2 * MF_D && (!prefill_row_blocks(a) || (a.n_packed > 0 && a.meta_dtype != VQ_F16))) return false;
