@@ -54,6 +54,12 @@ def test_static_scratch_entry_point_equals_the_workspace_entry_point():
         a = K.kivi_packed_attend(q4, static_scratch=True, **{**kw, **extra})
         b = K.kivi_packed_attend(q4, **{**kw, **extra})
         assert torch.equal(a, b)
+    # a GQA group of three heads at a few positions runs filled up to four heads: queries and outputs in that form
+    # sit in the scratch as well
+    q3 = to_dev(np.random.default_rng(6).standard_normal((1, 6, 4, 128)).astype(np.float16))
+    plan = {}
+    a = K.kivi_packed_attend(q3, static_scratch=True, causal=True, _plan_out=plan, **kw)
+    assert plan["path"] == 1 and torch.equal(a, K.kivi_packed_attend(q3, causal=True, **kw))
     # beyond the built-in scratch: refused with a clear error, nothing launched
     q512 = to_dev(np.random.default_rng(4).standard_normal((2, 32, 512, 128)).astype(np.float16))
     with pytest.raises(RuntimeError, match="built-in scratch"):   # 32768 query rows: 17 MB of partials
