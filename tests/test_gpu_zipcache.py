@@ -55,7 +55,7 @@ def test_cache_matches_the_model_bit_for_bit(B, H, S, D, kw):
         k1, v1 = _kv(B, H, 1, D, seed=100 + t)
         ko, vo = c.update_and_fetch(to_dev(k1), to_dev(v1))
         assert np.array_equal(host(ko)[:, :, -1:].view(np.uint16), oz.compress(k1, True, hb, lb, fr, gs)[0].view(np.uint16))
-    assert ko.shape[2] == S + 3 and len(c._ledger) == 2 and c._ledger[-1][1] == 3
+    assert ko.shape[2] == S + 3 and len(c._runs) == 2 and (c._runs[-1].unit, c._runs[-1].end - c._runs[-1].start) == (1, 3)
 
 
 def test_trim_takes_charges_back_and_nan_chunk_is_reported_by_the_next_call():

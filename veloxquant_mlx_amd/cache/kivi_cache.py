@@ -472,15 +472,16 @@ class KIVIKVCache(FP16KVCache):
         return n_rolled
 
     def _rollback_bytes(self, n_tokens: int, n_rolled: int) -> None:
+        """Take ``n_tokens`` trimmed tokens, ``n_rolled`` of them packed, back out of the counters (none goes below
+        zero), kivi_cache.py:280-291."""
         B, H, D = self._shape_bhd
-        if n_rolled > 0:
-            k, v = self._quantized_bytes(n_rolled, B, H, D)
-            self._key_bytes_compressed = max(0, self._key_bytes_compressed - k)
-            self._value_bytes_compressed = max(0, self._value_bytes_compressed - v)
-        self._key_bytes_fp16 = max(0, self._key_bytes_fp16 - H * B * n_tokens * D * 2)
-        self._value_bytes_fp16 = max(0, self._value_bytes_fp16 - H * B * n_tokens * D * 2)
-        self._tokens_seen = max(0, self._tokens_seen - n_tokens)
-        self._residual_fp16_bytes = (self.offset - self._n_quantized) * D * 2 * 2 * H * B
+        row16 = B * H * D * 2                                     # one token of keys (or values) in fp16
+        packed_k, packed_v = self._quantized_bytes(n_rolled, B, H, D) if n_rolled > 0 else (0, 0)
+        for name, less in (("_key_bytes_compressed", packed_k), ("_value_bytes_compressed", packed_v),
+                           ("_key_bytes_fp16", row16 * n_tokens), ("_value_bytes_fp16", row16 * n_tokens),
+                           ("_tokens_seen", n_tokens)):
+            setattr(self, name, max(0, getattr(self, name) - less))
+        self._residual_fp16_bytes = 2 * row16 * (self.offset - self._n_quantized)
 
     def trim(self, n: int) -> int:
         """Drop the last ``n`` tokens and roll frontier and accounting back (kivi_cache.py:293-299)."""

@@ -22,26 +22,28 @@ from ..quantizers.skvq import DEFAULT_ALPHA_GRID, skvq_compressed_bytes, skvq_fp
 from ._fp16_cache import FP16KVCache
 
 
+# (attribute, configuration field, type, default)
+_SKVQ_FIELDS = (("_bits_k", "skvq_bits_key", int, 4), ("_bits_v", "skvq_bits_value", int, 4), ("_group_size", "skvq_group_size", int, 32),
+                ("_window", "skvq_window", int, 128), ("_n_sink", "skvq_n_sink", int, 5), ("_reorder", "skvq_reorder", bool, True),
+                ("_clip_search", "skvq_clip_search", bool, True), ("_clip_alpha", "skvq_clip_alpha", float, 1.0))
+
+
 class SKVQKVCache(FP16KVCache):
     def __init__(self, config: Any) -> None:
         super().__init__()
         if not K._lib.library_present():
             raise RuntimeError("SKVQKVCache: the HIP kernel library is not available on this build; there is no fallback path.")
         self._D = int(config.head_dim)
-        self._bits_k = int(getattr(config, "skvq_bits_key", 4))
-        self._bits_v = int(getattr(config, "skvq_bits_value", 4))
-        self._group_size = int(getattr(config, "skvq_group_size", 32))
-        self._window = int(getattr(config, "skvq_window", 128))
-        self._n_sink = int(getattr(config, "skvq_n_sink", 5))
-        self._reorder = bool(getattr(config, "skvq_reorder", True))
-        self._clip_search = bool(getattr(config, "skvq_clip_search", True))
-        self._clip_alpha = float(getattr(config, "skvq_clip_alpha", 1.0))
-        max_ctx = getattr(config, "skvq_max_ctx", None)
-        self._max_ctx: int | None = None if max_ctx is None else int(max_ctx)
+        # the skvq_* fields of the configuration with the reference's defaults (skvq_cache.py:88-101)
+        for attr, field, kind, default in _SKVQ_FIELDS:
+            setattr(self, attr, kind(getattr(config, field, default)))
+        cap = getattr(config, "skvq_max_ctx", None)
+        self._max_ctx: int | None = int(cap) if cap is not None else None
         # same checks and key phrases as skvq_cache.py:103-127
-        for name, b in (("skvq_bits_key", self._bits_k), ("skvq_bits_value", self._bits_v)):
-            if not 1 <= b <= 8:
-                raise QuantizerConfigError(f"SKVQKVCache: {name}={b} must be in [1, 8] (uint8 codes)")
+        for field in ("skvq_bits_key", "skvq_bits_value"):
+            width = self._bits_k if field.endswith("key") else self._bits_v
+            if width < 1 or width > 8:
+                raise QuantizerConfigError(f"SKVQKVCache: {field}={width} must be in [1, 8] (uint8 codes)")
         if self._group_size < 1:
             raise QuantizerConfigError(f"SKVQKVCache: skvq_group_size={self._group_size} must be >= 1")
         if self._window < 2:
@@ -58,13 +60,10 @@ class SKVQKVCache(FP16KVCache):
         self._perm_v: torch.Tensor | None = None
         self._inv_v: torch.Tensor | None = None
         self._q_end = 0                            # tokens [0, _q_end) are flushed; a multiple of the window
-        self._compressed_key_bytes = 0
-        self._compressed_value_bytes = 0
-        self._fp16_key_bytes = 0
-        self._fp16_value_bytes = 0
+        self._compressed_key_bytes = self._compressed_value_bytes = 0
+        self._fp16_key_bytes = self._fp16_value_bytes = 0
         self._tokens_seen = 0
-        self._B = 1
-        self._H = 1
+        self._B = self._H = 1
 
     # ------------------------------------------------------------------ permutations
     def _round_trip(self, x: torch.Tensor, perm, inv, bits: int, out: torch.Tensor | None = None) -> torch.Tensor:

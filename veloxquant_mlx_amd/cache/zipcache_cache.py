@@ -55,6 +55,14 @@ def base_only_bytes(S: int, D: int, bits: int, group_size: int = 32) -> int:
     return math.ceil(S * D * bits / 8) + math.ceil(S / group_size) * D * 2 * 2
 
 
+class _Run:
+    """Tokens [start, end) of the cache: updates of ``unit`` tokens each, every one at ``cost``."""
+    __slots__ = ("start", "end", "unit", "cost")
+
+    def __init__(self, start: int, end: int, unit: int, cost: tuple) -> None:
+        self.start, self.end, self.unit, self.cost = start, end, unit, cost
+
+
 class ZipCacheKVCache(FP16KVCache):
     def __init__(self, config: Any) -> None:
         super().__init__()
@@ -63,8 +71,9 @@ class ZipCacheKVCache(FP16KVCache):
         cfg = validate_zipcache_config(config)
         self._hi_bits, self._lo_bits = cfg["hi_bits"], cfg["lo_bits"]
         self._hi_fraction, self._gs, self._quant_values = cfg["hi_fraction"], cfg["group_size"], cfg["quantize_values"]
-        # one entry per update: [tokens, repeat count, (key stored, key baseline, key fp16, value stored, baseline, fp16)]
-        self._ledger: list[list] = []
+        # what every stretch of tokens cost, in token order: a stretch is one multi-token update, or a run of
+        # single-token updates of the same cost (a long generation stays a handful of entries)
+        self._runs: list[_Run] = []
         self._pending = None   # (finite flag on the device, tokens, offset after the chunk)
 
     @staticmethod
@@ -138,34 +147,35 @@ class ZipCacheKVCache(FP16KVCache):
         bytes_ = (per_slab * BH, base_only_bytes(S, D, self._lo_bits, gs) * BH, B * H * S * D * 2)
         return out.reshape(B, H, S, D).to(out_dtype), norms, bytes_
 
-    def _charge(self, tokens: int, charges: tuple) -> None:
-        led = self._ledger
-        if tokens == 1 and led and led[-1][0] == 1 and led[-1][2] == charges:
-            led[-1][1] += 1   # a run of identical decode steps is one entry
+    def _charge(self, tokens: int, cost: tuple) -> None:
+        """``tokens`` new tokens at ``cost`` = bytes (key stored, key baseline, key fp16, value stored, baseline, fp16)."""
+        runs = self._runs
+        at = runs[-1].end if runs else 0
+        if tokens == 1 and runs and runs[-1].unit == 1 and runs[-1].cost == cost:
+            runs[-1].end += 1
         else:
-            led.append([tokens, 1, charges])
+            runs.append(_Run(at, at + tokens, tokens, cost))
 
     def trim(self, n: int) -> int:
-        """Drop the last ``n`` tokens and their charges; an update cut in the middle is pro-rated (zipcache_cache.py:263-287)."""
+        """Drop the last ``n`` tokens and what they cost; a multi-token update cut in the middle keeps the share of
+        its cost that its remaining tokens are of it (the contract of zipcache_cache.py:263-287)."""
         self._pending = None
         n = super().trim(n)
-        left, led = n, self._ledger
-        while left > 0 and led:
-            tokens, count, charges = led[-1]
-            if left >= tokens * count:
-                led.pop()
-                left -= tokens * count
-            elif tokens == 1:
-                led[-1][1] -= left
-                left = 0
-            else:
-                keep = tokens - left
-                led[-1] = [keep, 1, tuple(round(c * keep / tokens) for c in charges)]
-                left = 0
+        runs = self._runs
+        end = (runs[-1].end if runs else 0) - n
+        while runs and runs[-1].start >= end:
+            runs.pop()
+        if runs and runs[-1].end > end:
+            last = runs[-1]
+            if last.unit > 1:
+                kept = end - last.start
+                last.cost = tuple(round(c * kept / last.unit) for c in last.cost)
+                last.unit = kept
+            last.end = end
         return n
 
     def _total(self, i: int) -> int:
-        return sum(count * charges[i] for _, count, charges in self._ledger)
+        return sum((r.end - r.start) // r.unit * r.cost[i] for r in self._runs)
 
     def _resolve_pending(self, pending) -> None:
         """Report a previous prefill chunk that held NaN/Inf, after taking it back out (zipcache_cache.py:294-306)."""
@@ -183,15 +193,12 @@ class ZipCacheKVCache(FP16KVCache):
         on the device and is read by the next call, so no call waits for its own kernels."""
         if self._pending is not None:
             self._resolve_pending(self._pending)
-        k_out, k_norms, (kc, kb, kf) = self._compress(keys, True, keys.dtype)
-        if self._quant_values:
-            v_out, v_norms, (vc, vb, vf) = self._compress(values, False, values.dtype)
-        else:
-            v_out, v_norms = values, None
-            B, H, S, D = values.shape
-            vc, vb, vf = 0, 0, B * H * S * D * 2
         S = keys.shape[2]
-        self._charge(S, (kc, kb, kf, vc, vb, vf))
+        k_out, k_norms, k_cost = self._compress(keys, True, keys.dtype)
+        # values left alone cost their fp16 bytes and nothing else
+        v_out, v_norms, v_cost = (self._compress(values, False, values.dtype) if self._quant_values
+                                  else (values, None, (0, 0, values.numel() * 2)))
+        self._charge(S, (*k_cost, *v_cost))
         out = super().update_and_fetch(k_out, v_out)
         if S > 1:
             ok = torch.isfinite(k_norms).all()
