@@ -140,13 +140,9 @@ class KIVIKVCache(FP16KVCache):
         self._q_pad = None
 
         # byte accounting (kivi_cache.py:132-146)
-        self._key_bytes_compressed = 0
-        self._key_bytes_fp16 = 0
-        self._value_bytes_compressed = 0
-        self._value_bytes_fp16 = 0
-        self._residual_fp16_bytes = 0
-        self._tokens_seen = 0
-        self._n_quantized = 0
+        for counter in ("_key_bytes_compressed", "_key_bytes_fp16", "_value_bytes_compressed", "_value_bytes_fp16",
+                        "_residual_fp16_bytes", "_tokens_seen", "_n_quantized"):
+            setattr(self, counter, 0)
         self._shape_bhd: tuple[int, int, int] = (1, 1, int(config.head_dim))
 
         # packed store (fused modes)
