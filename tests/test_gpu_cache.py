@@ -583,7 +583,8 @@ def test_odd_code_widths_in_the_next_even_field(bits, D, g, Hq, meta, tmp_path):
 
 
 @pytest.mark.parametrize("bits,g,Hq,H,meta", [(4, 32, 32, 8, "float16"), (2, 64, 8, 2, "float32"), (2, 32, 14, 2, "float16"),
-                                              (4, 64, 12, 4, "float16"), (3, 32, 4, 4, "float32")])
+                                              (4, 64, 12, 4, "float16"), (3, 32, 4, 4, "float32"), (4, 32, 9, 3, "float16"),
+                                              (2, 32, 5, 5, "float32")])
 def test_heads_of_64_channels_are_kept_in_pairs(bits, g, Hq, H, meta):
     """A memory-bound cache of 64-channel heads keeps kv heads 2m and 2m+1 as one head of 128 channels (the head size of
     the matrix-unit kernels; queries zero-padded into their half): the stored codes are those of the unpaired cache, and
@@ -619,8 +620,9 @@ def test_heads_of_64_channels_are_kept_in_pairs(bits, g, Hq, H, meta):
         # (blocks of 256 query rows attend over the reconstruction rounded to fp16, as the reference's cache holds it)
         ref = oracle(q, hi, c._n_quantized, causal=True)
         assert float(np.max(np.abs(got - ref))) < 1e-2, (lo, float(np.max(np.abs(got - ref))))
-    assert c._pair and not plain._pair and c._shape_bhd == (B, H // 2, 128) and c._n_quantized == plain._n_quantized
-    assert c._kp.shape[1] == H // 2 and c._tail_k.shape[-1] == 128
+    P = (H + 1) // 2   # an odd count: the last head's partner is a head of zeros
+    assert c._pair and not plain._pair and c._shape_bhd == (B, P, 128) and c._n_quantized == plain._n_quantized
+    assert c._kp.shape[1] == P and c._tail_k.shape[-1] == 128
     # the stored codes: the paired head holds its two heads' channels side by side
     nq = c._n_quantized
     f = c._field
@@ -628,7 +630,7 @@ def test_heads_of_64_channels_are_kept_in_pairs(bits, g, Hq, H, meta):
     vd = K.kivi_dequant(c._vp, c._vs, c._vz, -1, g, f, nq, 128, v_layout=c._v_layout)
     kp_ = K.kivi_dequant(plain._kp, plain._ks, plain._kz, -2, g, f, nq, D)
     vp_ = K.kivi_dequant(plain._vp, plain._vs, plain._vz, -1, g, f, nq, D, v_layout=plain._v_layout)
-    unpair = lambda x: x.view(B, H // 2, nq, 2, D).transpose(2, 3).reshape(B, H, nq, D)
+    unpair = lambda x: x.view(B, P, nq, 2, D).transpose(2, 3).reshape(B, 2 * P, nq, D)[:, :H]
     assert torch.equal(unpair(kd), kp_) and torch.equal(unpair(vd), vp_)
 
     def step_checks(t_end):

@@ -196,3 +196,15 @@ def test_paired_heads_are_the_same_attention():
     # a leading layer axis (the layer stack) goes through unchanged
     q5 = torch.randn((3, B, Hq, 1, D), generator=g, dtype=torch.float64)
     assert torch.equal(own_half_of_paired_output(pad_queries_for_paired_heads(q5, H), H), q5)
+    # an odd number of kv heads: the last one is paired with a head of zeros, whose query heads are zeros too
+    for H3, Hq3 in ((3, 9), (5, 5)):
+        k3, v3 = (torch.randn((B, H3, S, D), generator=g, dtype=torch.float64) for _ in range(2))
+        q3 = torch.randn((B, Hq3, Sq, D), generator=g, dtype=torch.float64)
+        R3 = Hq3 // H3
+        assert pair_heads(k3).shape == (B, (H3 + 1) // 2, S, 2 * D) and float(pair_heads(k3)[:, -1, :, D:].abs().sum()) == 0.0
+        w3 = pad_queries_for_paired_heads(q3, H3)
+        assert w3.shape == (B, (H3 + 1) * R3, Sq, 2 * D) and torch.equal(own_half_of_paired_output(w3, H3), q3)
+        got3 = own_half_of_paired_output(attend(w3, pair_heads(k3), pair_heads(v3), 2 * R3), H3)
+        assert float((got3 - attend(q3, k3, v3, R3)).abs().max()) < 1e-12
+        q35 = torch.randn((2, B, Hq3, 1, D), generator=g, dtype=torch.float64)
+        assert torch.equal(own_half_of_paired_output(pad_queries_for_paired_heads(q35, H3), H3), q35)

@@ -34,32 +34,51 @@ _META = {"float16": torch.float16, "float32": torch.float32}
 
 
 def pair_heads(x: torch.Tensor) -> torch.Tensor:
-    """``[..., H, S, D]`` -> ``[..., H/2, S, 2D]``: kv heads 2m and 2m+1 side by side in one head of twice the channels.
-    Group quantisation along tokens is per channel and along channels per group of ``g`` (``g`` divides ``D``), so the
-    codes, scale and zero of the paired head are those of the two heads."""
+    """``[..., H, S, D]`` -> ``[..., ceil(H/2), S, 2D]``: kv heads 2m and 2m+1 side by side in one head of twice the
+    channels (an odd count gets a head of zeros for the last one's partner).  Group quantisation along tokens is per
+    channel and along channels per group of ``g`` (``g`` divides ``D``), so the codes, scale and zero of the paired head
+    are those of the two heads."""
     *lead, H, S, D = x.shape
+    if H % 2:
+        x = torch.cat([x, x.new_zeros((*lead, 1, S, D))], dim=-3)
+        H += 1
     return x.reshape(*lead, H // 2, 2, S, D).transpose(-3, -2).reshape(*lead, H // 2, S, 2 * D)
 
 
 def pad_queries_for_paired_heads(q: torch.Tensor, n_kv_heads: int, out: torch.Tensor | None = None) -> torch.Tensor:
-    """``q [..., H_q, S_q, D]`` -> ``[..., H_q, S_q, 2D]`` for a cache of paired kv heads: a query head's channels in the
-    half of its own kv head, zeros in the other (``q . [k_a, k_b] = q . k_a``).  ``out``: a buffer of the result's
-    shape whose other halves are already zero."""
+    """``q [..., H_q, S_q, D]`` -> ``[..., 2 * ceil(H/2) * R, S_q, 2D]`` for a cache of paired kv heads (``H`` kv heads,
+    ``R = H_q / H``): a query head's channels in the half of its own kv head, zeros in the other
+    (``q . [k_a, k_b] = q . k_a``); with an odd ``H`` the partner of the last kv head brings ``R`` query heads of zeros
+    along.  ``out``: a buffer of the result's shape whose other halves are already zero."""
     *lead, Hq, Sq, D = q.shape
-    R = Hq // n_kv_heads
+    H, R, P = n_kv_heads, Hq // n_kv_heads, (n_kv_heads + 1) // 2
     if out is None:
-        out = q.new_zeros((*lead, Hq, Sq, 2 * D))
-    wide = out.view(*lead, n_kv_heads // 2, 2, R, Sq, 2, D).diagonal(dim1=-5, dim2=-2)      # [..., P, R, Sq, D, 2]
-    wide.copy_(q.reshape(*lead, n_kv_heads // 2, 2, R, Sq, D).movedim(-4, -1))
+        out = q.new_zeros((*lead, 2 * P * R, Sq, 2 * D))
+    wide = out.view(*lead, P, 2, R, Sq, 2, D).diagonal(dim1=-5, dim2=-2)      # [..., P, R, Sq, D, 2]
+    if H % 2 == 0:
+        wide.copy_(q.reshape(*lead, P, 2, R, Sq, D).movedim(-4, -1))
+    else:
+        heads = q.reshape(*lead, H, R, Sq, D)
+        wide[..., 0].copy_(heads[..., 0::2, :, :, :])
+        if H > 1:
+            wide[..., : H // 2, :, :, :, 1].copy_(heads[..., 1::2, :, :, :])
     return out
 
 
 def own_half_of_paired_output(o: torch.Tensor, n_kv_heads: int) -> torch.Tensor:
-    """``o [..., H_q, S_q, 2D]`` (attention over paired kv heads) -> ``[..., H_q, S_q, D]``: every query head's own half."""
-    *lead, Hq, Sq, D2 = o.shape
-    R, D = Hq // n_kv_heads, D2 // 2
-    own = o.view(*lead, n_kv_heads // 2, 2, R, Sq, 2, D).diagonal(dim1=-5, dim2=-2)          # [..., P, R, Sq, D, 2]
-    return own.movedim(-1, -4).reshape(*lead, Hq, Sq, D)
+    """``o [..., 2 * ceil(H/2) * R, S_q, 2D]`` (attention over paired kv heads) -> ``[..., H * R, S_q, D]``: every
+    query head's own half."""
+    *lead, Hq2, Sq, D2 = o.shape
+    H, P, D = n_kv_heads, (n_kv_heads + 1) // 2, D2 // 2
+    R = Hq2 // (2 * P)
+    own = o.view(*lead, P, 2, R, Sq, 2, D).diagonal(dim1=-5, dim2=-2)          # [..., P, R, Sq, D, 2]
+    if H % 2 == 0:
+        return own.movedim(-1, -4).reshape(*lead, H * R, Sq, D)
+    res = o.new_empty((*lead, H, R, Sq, D))
+    res[..., 0::2, :, :, :] = own[..., 0]
+    if H > 1:
+        res[..., 1::2, :, :, :] = own[..., : H // 2, :, :, :, 1]
+    return res.view(*lead, H * R, Sq, D)
 
 
 class KIVIKVCache(FP16KVCache):
@@ -137,6 +156,7 @@ class KIVIKVCache(FP16KVCache):
         self._pair_wanted = (bool(getattr(config, "kivi_pair_heads", True)) and self._memory_bound and self._head_dim == 64
                              and type(self) is KIVIKVCache and 64 % self._group_size == 0)
         self._pair = False
+        self._kv_heads = 0     # the caller's kv head count while heads are kept in pairs
         self._q_pad = None
 
         # byte accounting (kivi_cache.py:132-146)
@@ -239,11 +259,17 @@ class KIVIKVCache(FP16KVCache):
         B, H, S, D = keys.shape
         if self._memory_bound:
             if self.offset == 0 and self._n_quantized == 0:
-                self._pair = self._pair_wanted and D == 64 and H % 2 == 0
+                # (an odd head count pairs its last head with a head of zeros: not worth it for a single head)
+                self._pair = self._pair_wanted and D == 64 and H >= 2
+                self._kv_heads = H
             if self._pair:
-                if D != 64 or H != 2 * self._shape_bhd[1] and self.offset > 0:
-                    raise ValueError(f"KIVIKVCache.update_and_fetch: this cache pairs kv heads of 64 channels, got {tuple(keys.shape)}")
-                self._shape_bhd = (B, H // 2, 2 * D)
+                # (a restored state shows the pairs, not whether the last one is whole: the first keys say)
+                same = H == self._kv_heads or (self._kv_heads < 0 and (H + 1) // 2 == self._shape_bhd[1])
+                if D != 64 or not same:
+                    raise ValueError(f"KIVIKVCache.update_and_fetch: this cache pairs {abs(self._kv_heads)} kv heads of 64 channels, "
+                                     f"got {tuple(keys.shape)}")
+                self._kv_heads = H
+                self._shape_bhd = (B, (H + 1) // 2, 2 * D)
                 self._update_memory_bound(pair_heads(keys), pair_heads(values))
                 z = self._zero_scalar
                 return z.expand(B, H, self.offset, D), z.expand(B, H, self.offset, D)
@@ -375,12 +401,15 @@ class KIVIKVCache(FP16KVCache):
         if self.offset == 0:
             raise RuntimeError("KIVIKVCache.fused_sdpa called before any tokens were cached via update_and_fetch.")
         if self._pair and q.shape[-1] == 64:
-            H = 2 * self._shape_bhd[1]
+            H = abs(self._kv_heads)
+            if self._kv_heads < 0 and q.shape[1] % H and q.shape[1] % (H - 1) == 0:
+                H -= 1   # a state restored without its meta_state: the query heads do not divide over an even count
             if q.shape[1] % H:
                 raise ValueError(f"KIVIKVCache.fused_sdpa: {q.shape[1]} query heads over {H} kv heads")
             key = (tuple(q.shape), q.dtype, q.device, K._stream_of(q.device))
             if self._q_pad is None or self._q_pad[0] != key:   # the zero halves are written once
-                self._q_pad = (key, q.new_zeros((*q.shape[:-1], 128)))
+                wide_heads = 2 * self._shape_bhd[1] * (q.shape[1] // H)
+                self._q_pad = (key, q.new_zeros((q.shape[0], wide_heads, q.shape[2], 128)))
             wide = self.fused_sdpa(pad_queries_for_paired_heads(q, H, self._q_pad[1]), scale, causal=causal,
                                    sliding_window=sliding_window, fixed_order=fixed_order, lengths=lengths, num_splits=num_splits)
             return own_half_of_paired_output(wide, H)
@@ -563,6 +592,8 @@ class KIVIKVCache(FP16KVCache):
             # rows of twice the head size: a state saved with paired heads
             d = int((packed[1] if packed else ref).shape[-1])
             self._pair = self._memory_bound and self._pair_wanted and d == 2 * self._head_dim
+            if self._pair:
+                self._kv_heads = -2 * int(ref.shape[1])   # negative: taken from the pairs, an odd count is one less
             self._shape_bhd = (int(ref.shape[0]), int(ref.shape[1]), d if self._pair else self._head_dim)
         self._restore_packed(packed)
         if self._memory_bound:
@@ -634,6 +665,8 @@ class KIVIKVCache(FP16KVCache):
         """Strings, as prompt-cache files store them: what a restored cache must agree with
         (offset, frontier, bit width, group, value layout, scale/zero dtype, mode)."""
         mode = "memory_bound" if self._memory_bound else ("stash" if self._fused_enabled else "standard")
+        if self._pair and self._kv_heads > 0 and self._kv_heads % 2:
+            mode += f"/{self._kv_heads}"   # an odd number of kv heads kept in pairs: the pairs do not show it
         bits = self._b if self._field == self._b else f"{self._b}/{self._field}"   # code width / width of its field
         return tuple(map(str, (self.offset, self._n_quantized, bits, self._group_size, self._v_layout,
                                str(self._meta_dtype).replace("torch.", ""), mode)))
@@ -643,7 +676,12 @@ class KIVIKVCache(FP16KVCache):
         v = tuple(v)
         if len(v) != 7:
             raise ValueError(f"KIVIKVCache.meta_state: expected 7 fields, got {len(v)}")
+        mode, _, heads = str(v[6]).partition("/")
+        v = (*v[:6], mode)
+        if heads and self._pair and (int(heads) + 1) // 2 == self._shape_bhd[1]:
+            self._kv_heads = int(heads)
         mine = self.meta_state
+        mine = (*mine[:6], mine[6].partition("/")[0])
         if tuple(v[2:]) != mine[2:]:
             raise ValueError(f"KIVIKVCache.meta_state: saved with (bits, group, value layout, meta dtype, mode) = {tuple(v[2:])}, "
                              f"this cache is configured as {mine[2:]}")

@@ -190,12 +190,13 @@ class LayerStackedKIVICache:
             raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: q must be [NL={NL},B,H_q,S_q,D], got {tuple(q.shape)}")
         B = q.shape[1]
         if self.layers[0]._pair and q.shape[-1] == 64:   # kv heads of 64 channels kept in pairs: see KIVIKVCache
-            H = 2 * self.layers[0]._shape_bhd[1]
+            H = abs(self.layers[0]._kv_heads)
             if q.shape[2] % H:
                 raise ValueError(f"LayerStackedKIVICache.fused_sdpa_all: {q.shape[2]} query heads over {H} kv heads")
             key = (tuple(q.shape), q.dtype, q.device, K._stream_of(q.device))
             if self._q_pad is None or self._q_pad[0] != key:
-                self._q_pad = (key, q.new_zeros((*q.shape[:-1], 128)))
+                wide_heads = 2 * self.layers[0]._shape_bhd[1] * (q.shape[2] // H)
+                self._q_pad = (key, q.new_zeros((q.shape[0], q.shape[1], wide_heads, q.shape[3], 128)))
             wide = self.fused_sdpa_all(pad_queries_for_paired_heads(q, H, self._q_pad[1]), scale, causal=causal,
                                        sliding_window=sliding_window, fixed_order=fixed_order, num_splits=num_splits)
             return own_half_of_paired_output(wide, H)
