@@ -208,3 +208,19 @@ def test_paired_heads_are_the_same_attention():
         assert float((got3 - attend(q3, k3, v3, R3)).abs().max()) < 1e-12
         q35 = torch.randn((2, B, Hq3, 1, D), generator=g, dtype=torch.float64)
         assert torch.equal(own_half_of_paired_output(pad_queries_for_paired_heads(q35, H3), H3), q35)
+
+
+def test_kivi_storage_options():
+    """The additions that pick how a packed KIVI cache stores its codes: the width of a code's field and the pairing of
+    64-channel heads (host-side decisions; the kernels are the same ones)."""
+    def make(**kw):
+        return KVCacheFactory.create(KVCacheConfig(method="kivi", fused_sdpa=True, fused_sdpa_memory_bound=True, **kw))
+    assert [make(bit_width_inlier=b)._field for b in (1, 2, 3, 4, 8)] == [2, 2, 4, 4, 8]
+    assert [make(bit_width_inlier=b, kivi_code_field="tight")._field for b in (1, 2, 3, 4)] == [1, 2, 3, 4]
+    assert [make(bit_width_inlier=b)._levels for b in (1, 3)] == [1, 7]          # the levels stay the quantiser's
+    assert make(bit_width_inlier=3)._v_layout == "token" and make(bit_width_inlier=3, kivi_code_field="tight")._v_layout == "channel"
+    with pytest.raises(QuantizerConfigError, match="kivi_code_field"):
+        make(kivi_code_field="wide")
+    assert make(head_dim=64)._pair_wanted and not make(head_dim=64, kivi_pair_heads=False)._pair_wanted
+    assert not make(head_dim=128)._pair_wanted
+    assert not KVCacheFactory.create(KVCacheConfig(method="kivi", head_dim=64))._pair_wanted   # the fp16-history modes keep single heads
