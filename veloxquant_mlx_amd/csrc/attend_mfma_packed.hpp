@@ -852,15 +852,19 @@ void attend_mfma_packed_kernel(vq_attend_args a, int64_t split_len, int64_t tail
     // a ticket with release-acquire ordering at device scope: the release publishes the block's
     // partials before the count moves, the acquire orders the merging block's loads after it
     // (the block barrier behind it extends that to the other threads).
+    // A tile with a single run has no other block to count: the barrier has collected its own partials (the
+    // packed one and the tail waves'; the tail launch of a 256-channel head ended before this one began).
     if (!single_launch) return;
     wait_copies<0>();
     __syncthreads();
-    if (tid == 0)
-        s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    __syncthreads();
-    if (s_ticket != nsplit - 1) return;
+    if (nsplit > 1) {
+        if (tid == 0)
+            s_ticket = __hip_atomic_fetch_add(a.sync_counters + by, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (s_ticket != nsplit - 1) return;
+    }
     merge_rows<DH>(a, tile, nparts, ws, tid, PK_THREADS);
-    if (tid == 0) __hip_atomic_store(a.sync_counters + by, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (nsplit > 1 && tid == 0) __hip_atomic_store(a.sync_counters + by, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 template <typename M, int RTP, int DH = 1>
